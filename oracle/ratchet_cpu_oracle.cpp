@@ -1,0 +1,54 @@
+// TEST INFRASTRUCTURE ONLY (see ratchet_cpu_oracle.h): C entry points; picks the F16C build of the kernels when the
+// host CPU has the instructions, the portable build otherwise.
+#include "ratchet_cpu_oracle.h"
+#include "orc_table.h"
+
+int g_orc_f16_sum_sequential = 0;
+int g_orc_reference_copies = 1;
+
+static int g_use_hw = -1;
+static const OrcTable& table() {
+    if (g_use_hw < 0) g_use_hw = __builtin_cpu_supports("f16c") ? 1 : 0;
+    return g_use_hw ? orc_hw::kTable : orc_soft::kTable;
+}
+
+extern "C" {
+int orc_binary(int op, int dt, const void* a, const void* b, void* y, size_t n) { return table().binary(op, dt, a, b, y, n); }
+int orc_unary(int op, int dt, const void* x, void* y, size_t n) { return table().unary(op, dt, x, y, n); }
+int orc_cast(int s, int d, const void* x, void* y, size_t n) { return table().cast(s, d, x, y, n); }
+int orc_permute(int eb, const void* x, void* y, int rank, const uint64_t* shape, const uint32_t* dims) {
+    return table().permute(eb, x, y, rank, shape, dims);
+}
+int orc_slice(int eb, const void* x, void* y, int rank, const uint64_t* shape, const uint64_t* start, const uint64_t* stop) {
+    return table().slice(eb, x, y, rank, shape, start, stop);
+}
+int orc_broadcast(int eb, const void* x, void* y, int sr, const uint64_t* ss, int dr, const uint64_t* ds, int np) {
+    return table().broadcast(eb, x, y, sr, ss, dr, ds, np);
+}
+int orc_concat(int eb, int n, const void* const* xs, int rank, const uint64_t* shapes, int dim, void* y) {
+    return table().concat(eb, n, xs, rank, shapes, dim, y);
+}
+int orc_softmax(int dt, const void* x, void* y, size_t rows, size_t cols) { return table().softmax(dt, x, y, rows, cols); }
+int orc_layer_norm(int dt, const void* x, const void* s, const void* b, void* y, size_t rows, size_t cols, float eps,
+                   size_t shape0) {
+    return table().layer_norm(dt, x, s, b, y, rows, cols, eps, shape0);
+}
+int orc_rms_norm(int dt, const void* x, const void* s, void* y, size_t rows, size_t cols, float eps, size_t shape0) {
+    return table().rms_norm(dt, x, s, y, rows, cols, eps, shape0);
+}
+int orc_group_norm(int dt, const void* x, const void* s, const void* b, void* y, size_t B, size_t C, size_t L, size_t G,
+                   float eps) {
+    return table().group_norm(dt, x, s, b, y, B, C, L, G, eps);
+}
+void orc_set_reference_copies(int on) { g_orc_reference_copies = on ? 1 : 0; }
+void orc_set_f16_sum_mode(int seq) { g_orc_f16_sum_sequential = seq ? 1 : 0; }
+void orc_set_hw_f16(int on) { g_use_hw = (on && __builtin_cpu_supports("f16c")) ? 1 : 0; }
+int orc_has_hw_f16(void) { return __builtin_cpu_supports("f16c") ? 1 : 0; }
+uint16_t orc_f32_to_f16(float f) { return table().f32_to_f16(f); }
+float orc_f16_to_f32(uint16_t h) { return table().f16_to_f32(h); }
+uint16_t orc_f32_to_bf16(float f) { return table().f32_to_bf16(f); }
+float orc_bf16_to_f32(uint16_t h) { return table().bf16_to_f32(h); }
+size_t orc_count_not_close(int dt, const void* a, const void* b, size_t n, double atol, double rtol, double* mx) {
+    return table().count_not_close(dt, a, b, n, atol, rtol, mx);
+}
+}

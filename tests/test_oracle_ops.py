@@ -1,0 +1,353 @@
+"""CPU-only checks that pin the oracle's op-level functions.
+
+Referees: torch CPU (the referee the reference's own tests use, at the reference's own tolerances), float64
+evaluation, numpy index operations, brute-force Python models on tiny inputs, and invariants.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+ALL_F16 = np.arange(65536, dtype=np.uint32).astype(np.uint16).view(np.float16)
+
+
+def _bits(a):
+    return a.view({2: np.uint16, 4: np.uint32}[a.dtype.itemsize])
+
+
+def _ulp_diff_f32(a, b):
+    """distance in units in the last place between two float32 arrays (finite entries)"""
+    def key(x):
+        i = x.view(np.int32).astype(np.int64)
+        return np.where(i < 0, -(i & 0x7fffffff), i)
+    return np.abs(key(a) - key(b))
+
+
+def _ulp_diff_f16(a, b):
+    def key(x):
+        i = x.view(np.int16).astype(np.int64)
+        return np.where(i < 0, -(i & 0x7fff), i)
+    return np.abs(key(a) - key(b))
+
+
+TORCH_UNARY = {
+    "gelu": lambda t: F.gelu(t, approximate="tanh"), "tanh": torch.tanh, "exp": torch.exp, "log": torch.log,
+    "sin": torch.sin, "cos": torch.cos, "abs": torch.abs, "sqrt": torch.sqrt, "relu": torch.relu,
+    "floor": torch.floor, "ceil": torch.ceil, "neg": torch.neg, "silu": F.silu, "sigmoid": torch.sigmoid,
+}
+
+
+@pytest.mark.parametrize("op", list(TORCH_UNARY))
+def test_unary_f32_vs_torch_reference_tolerance(oracle, op):
+    # crates/ratchet-core/src/ops/unary.rs:365-461: randn [1..2, 1..128], tol 5e-2 for gelu/tanh, 1e-4 otherwise
+    rng = np.random.default_rng(10)
+    x = rng.standard_normal((2, 128)).astype(np.float32)
+    with np.errstate(all="ignore"):
+        want = TORCH_UNARY[op](torch.from_numpy(x)).numpy()
+    got = oracle.unary(op, x)
+    tol = 5e-2 if op in ("gelu", "tanh") else 1e-4
+    bad, mx = oracle.count_not_close(got, want, tol, tol)
+    assert bad == 0, (op, mx)
+
+
+def _f64_model(op, x64):
+    with np.errstate(all="ignore"):
+        if op == "gelu":
+            return 0.5 * x64 * (1 + np.tanh(np.float64(np.float32(0.7978846)) * x64 *
+                                            (1 + np.float64(np.float32(0.044715)) * x64 * x64)))
+        if op == "silu":
+            return x64 / (1 + np.exp(-x64))
+        if op == "sigmoid":
+            return 1 / (1 + np.exp(-x64))
+        return {"tanh": np.tanh, "exp": np.exp, "log": np.log, "sin": np.sin, "cos": np.cos, "abs": np.abs,
+                "sqrt": np.sqrt, "relu": lambda v: np.maximum(v, 0), "floor": np.floor, "ceil": np.ceil,
+                "neg": np.negative}[op](x64)
+
+
+@pytest.mark.parametrize("op", ["tanh", "exp", "log", "sin", "cos", "sqrt", "silu", "sigmoid", "abs", "floor", "ceil",
+                                "neg", "relu"])
+def test_unary_f32_close_to_float64(oracle, op):
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal(200_000) * 4).astype(np.float32)
+    if op in ("log", "sqrt"):
+        x = np.abs(x) + np.float32(1e-3)
+    got = oracle.unary(op, x)
+    want = _f64_model(op, x.astype(np.float64)).astype(np.float32)
+    limit = {"silu": 3, "sigmoid": 3, "tanh": 2}.get(op, 1)   # glibc tanhf is a 2-ulp routine; compositions add rounding
+    assert _ulp_diff_f32(got, want).max() <= limit
+
+
+def test_gelu_f32_formula_association(oracle):
+    # step-by-step float32 replay of crates/ratchet-core/src/cpu/unary.rs:46-51 with libm tanh from numpy's float64
+    # (rounded): a dropped term, a swapped constant or a different association changes many results by far more
+    # than the ~1e-6 relative slack allowed here
+    rng = np.random.default_rng(12)
+    x = (rng.standard_normal(100_000) * 3).astype(np.float32)
+    f = np.float32
+    inner = f(1.0) + (f(0.044715) * x) * x
+    arg = (f(0.7978846) * x) * inner
+    t = np.tanh(arg.astype(np.float64)).astype(np.float32)
+    want = (f(0.5) * x) * (f(1.0) + t)
+    got = oracle.unary("gelu", x)
+    assert np.allclose(got, want, rtol=2e-6, atol=2e-7)
+    # exact zero and sign behaviour
+    z = oracle.unary("gelu", np.array([0.0, -0.0, 30.0, -30.0], dtype=np.float32))
+    assert z[0] == 0 and z[1] == 0 and z[2] == 30.0 and z[3] == 0.0
+
+
+EXACT_F16 = {"abs": np.abs, "neg": np.negative, "floor": np.floor, "ceil": np.ceil, "sqrt": np.sqrt}
+
+
+@pytest.mark.parametrize("op", list(EXACT_F16))
+def test_unary_f16_exhaustive_exact_ops(oracle, op):
+    with np.errstate(all="ignore"):
+        want = EXACT_F16[op](ALL_F16)
+    got = oracle.unary(op, ALL_F16)
+    both_nan = np.isnan(got) & np.isnan(want)
+    assert np.all((_bits(got) == _bits(want)) | both_nan)
+
+
+def test_unary_f16_relu_exhaustive(oracle):
+    got = oracle.unary("relu", ALL_F16)
+    x = ALL_F16
+    want = np.where(x < 0, np.float16(0), x)            # NaN stays NaN, -0.0 stays -0.0 (half's max)
+    both_nan = np.isnan(got) & np.isnan(want)
+    assert np.all((_bits(got) == _bits(want)) | both_nan)
+
+
+def _f16_steps_model(op, x):
+    """independent model: numpy float16 arithmetic rounds after every operation, transcendental calls are
+    evaluated in float64 and rounded through float32 to float16"""
+    h = np.float16
+    def libm(fn, v):
+        with np.errstate(all="ignore"):
+            return fn(v.astype(np.float64)).astype(np.float32).astype(np.float16)
+    with np.errstate(all="ignore"):
+        if op == "gelu":
+            inner = h(1.0) + (h(0.044715) * x) * x
+            arg = (h(0.7978846) * x) * inner
+            return (h(0.5) * x) * (h(1.0) + libm(np.tanh, arg))
+        if op == "silu":
+            return x / (h(1.0) + libm(np.exp, -x))
+        if op == "sigmoid":
+            return h(1.0) / (h(1.0) + libm(np.exp, -x))
+        return libm({"tanh": np.tanh, "exp": np.exp, "log": np.log, "sin": np.sin, "cos": np.cos}[op], x)
+
+
+@pytest.mark.parametrize("op", ["gelu", "silu", "sigmoid", "tanh", "exp", "log", "sin", "cos"])
+def test_unary_f16_exhaustive_vs_stepwise_model(oracle, op):
+    got = oracle.unary(op, ALL_F16)
+    want = _f16_steps_model(op, ALL_F16)
+    ok = (_bits(got) == _bits(want)) | (np.isnan(got) & np.isnan(want))
+    # host libm's float32 result is not always the correctly rounded one, so a handful of the 65536 inputs may land on
+    # the other side of a float16 rounding boundary; anything structural (a missing rounding step, a different
+    # association) shows up as thousands of mismatches
+    mism = np.count_nonzero(~ok)
+    assert mism <= 40, mism
+    if op not in ("gelu",):                              # gelu's 1 + tanh cancellation can amplify a 1-ulp tanh flip
+        fin = ~ok & np.isfinite(got) & np.isfinite(want)
+        assert np.all(_ulp_diff_f16(got[fin], want[fin]) <= 1)
+
+
+def test_softmax_f32_vs_torch_reference_tolerance(oracle):
+    # crates/ratchet-core/src/ops/softmax.rs:308-365: randn [1..3, 1..256, 1..256], dim 2, tol 1e-6
+    rng = np.random.default_rng(13)
+    for shape in [(3, 256, 256), (1, 7, 33), (2, 1, 1), (1, 5, 255)]:
+        x = rng.standard_normal(shape).astype(np.float32)
+        want = F.softmax(torch.from_numpy(x), dim=-1).numpy()
+        got = oracle.softmax(x)
+        bad, mx = oracle.count_not_close(got, want, 1e-6, 1e-6)
+        assert bad == 0, (shape, mx)
+        assert np.allclose(got.sum(-1), 1.0, atol=1e-5)
+
+
+def test_softmax_masks_overflow_and_order(oracle):
+    ninf = -np.inf
+    x = np.array([[0.0, ninf, ninf, ninf], [1.0, 1.0, ninf, ninf], [100.0, 0.0, 0.0, 0.0]], dtype=np.float32)
+    y = oracle.softmax(x)
+    assert np.array_equal(y[0], np.array([1, 0, 0, 0], dtype=np.float32))      # single unmasked entry -> exactly 1
+    assert np.array_equal(y[1], np.array([0.5, 0.5, 0, 0], dtype=np.float32))
+    # exp(100) overflows float32: no max subtraction in the reference -> inf/inf = NaN there, 0 elsewhere
+    assert np.isnan(y[2, 0]) and np.all(y[2, 1:] == 0)
+    # float16: sequential accumulation in float16, order dependent.  2048 + 1 + 1 ... never grows in f16.
+    big = np.float16(math.log(2048.0))
+    row = np.full(64, 0.0, dtype=np.float16)
+    row[0] = big
+    e0 = np.exp(np.float64(big)).astype(np.float32).astype(np.float16)
+    y16 = oracle.softmax(row[None, :])
+    s = e0
+    for _ in range(63):
+        s = np.float16(np.float32(s) + np.float32(1.0))
+    assert y16[0, 1] == np.float16(np.float32(1.0) / np.float32(s))
+    rev = oracle.softmax(row[::-1].copy()[None, :])
+    assert rev[0, 0] != y16[0, 1]                        # same row reversed gives a different denominator
+
+
+def test_softmax_f16_bruteforce(oracle):
+    rng = np.random.default_rng(14)
+    x = (rng.standard_normal((6, 97)) * 2).astype(np.float16)
+    got = oracle.softmax(x)
+    for r in range(x.shape[0]):
+        e = np.exp(x[r].astype(np.float64)).astype(np.float32).astype(np.float16)
+        s = np.float16(0)
+        for j in range(x.shape[1]):
+            s = np.float16(np.float32(s) + np.float32(e[j]))
+        want = (e.astype(np.float32) / np.float32(s)).astype(np.float16)
+        mism = np.count_nonzero(_bits(want) != _bits(got[r]))
+        assert mism <= 1                                  # libm float32 exp vs float64 exp double rounding
+
+
+@pytest.mark.parametrize("shape", [(3, 256, 256), (2, 57, 1001), (1, 1, 1), (1, 13, 7)])
+def test_layer_norm_f32_vs_torch(oracle, shape):
+    # crates/ratchet-core/src/ops/norm/mod.rs:400-512: scale, bias ~ N(0,1), eps 1e-5, tol 1e-4
+    rng = np.random.default_rng(15)
+    x = rng.standard_normal(shape).astype(np.float32)
+    n = shape[-1]
+    w = rng.standard_normal(n).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32)
+    want = F.layer_norm(torch.from_numpy(x), (n,), torch.from_numpy(w), torch.from_numpy(b), eps=1e-5).numpy()
+    got = oracle.layer_norm(x, w, b, 1e-5)
+    bad, mx = oracle.count_not_close(got, want, 1e-4, 1e-4)
+    assert bad == 0, mx
+    want_nb = F.layer_norm(torch.from_numpy(x), (n,), torch.from_numpy(w), None, eps=1e-5).numpy()
+    bad, mx = oracle.count_not_close(oracle.layer_norm(x, w, None, 1e-5), want_nb, 1e-4, 1e-4)
+    assert bad == 0, mx
+
+
+def test_rms_norm_f32_vs_manual_torch(oracle):
+    rng = np.random.default_rng(16)
+    x = rng.standard_normal((2, 64, 200)).astype(np.float32)
+    w = rng.standard_normal(200).astype(np.float32)
+    t = torch.from_numpy(x)
+    want = (t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + 1e-5) * torch.from_numpy(w)).numpy()
+    got = oracle.rms_norm(x, w, 1e-5)
+    bad, mx = oracle.count_not_close(got, want, 1e-4, 1e-4)
+    assert bad == 0, mx
+
+
+def test_norm_invariants_and_variance_form(oracle):
+    rng = np.random.default_rng(17)
+    x = (rng.standard_normal((32, 384)) * 3 + 1).astype(np.float32)
+    one, zero = np.ones(384, np.float32), np.zeros(384, np.float32)
+    y = oracle.layer_norm(x, one, zero, 1e-5)
+    assert np.allclose(y.mean(-1), 0, atol=1e-5) and np.allclose(y.var(-1), 1, atol=1e-3)
+    # the reference's variance is E[x^2] - mu^2 (crates/ratchet-core/src/cpu/norm.rs:117-123): with a large common
+    # offset that form loses digits, a two-pass variance would not
+    xo = (rng.standard_normal((4, 64)) * 1e-2 + 100).astype(np.float32)
+    y_ref = oracle.layer_norm(xo, np.ones(64, np.float32), None, 1e-5)
+    two_pass = F.layer_norm(torch.from_numpy(xo), (64,), eps=1e-5).numpy()
+    diff = np.abs(y_ref - two_pass)
+    assert np.isnan(diff).any() or diff.max() > 1e-2     # a negative variance (NaN) is the extreme case of the loss
+
+
+def test_layer_norm_f16_stepwise_model(oracle):
+    rng = np.random.default_rng(18)
+    h = np.float16
+    x = rng.standard_normal((5, 96)).astype(h)
+    w = (1 + 0.02 * rng.standard_normal(96)).astype(h)
+    b = (0.02 * rng.standard_normal(96)).astype(h)
+    got = oracle.layer_norm(x, w, b, 1e-5)
+    n = h(np.float32(96))
+    for r in range(5):
+        xr = x[r]
+        mu = h(np.float32(xr.astype(np.float32).sum(dtype=np.float32))) / n      # f32 accumulate, round, f16 divide
+        mu2 = mu * mu
+        sq = xr * xr
+        x2 = h(np.float32(sq.astype(np.float32).sum(dtype=np.float32))) / n
+        var = x2 - mu2
+        xc = xr - mu
+        r_ = h(1.0) / np.sqrt(var + h(np.float32(1e-5)))
+        want = ((xc * r_) * w) + b
+        # numpy's pairwise float32 summation may differ from the sequential sum in the last float32 bit, which
+        # can move a float16 rounding on rare rows; everything else is exact
+        assert np.count_nonzero(_ulp_diff_f16(got[r], want.astype(h)) > 1) == 0
+        assert np.count_nonzero(_bits(got[r]) != _bits(want.astype(h))) <= 96 // 2
+
+
+def test_layer_norm_scale_vector_special_case(oracle):
+    # crates/ratchet-core/src/cpu/reindex.rs:165-173 through norm.rs:136-142: when the input's first dimension equals
+    # N, scale is repeated element-wise over numel/N outputs instead of tiled along rows
+    x = np.arange(16, dtype=np.float32).reshape(4, 4) ** 2
+    w = np.array([1, 2, 3, 4], dtype=np.float32)
+    quirk = oracle.layer_norm(x, w, None, 1e-5)
+    intended = oracle.layer_norm(x, w, None, 1e-5, intended=True)
+    base = oracle.layer_norm(x, np.ones(4, np.float32), None, 1e-5)
+    assert np.allclose(intended, base * w[None, :])
+    assert np.allclose(quirk, base * w[:, None])
+
+
+@pytest.mark.parametrize("B,C,L,G", [(1, 3, 1, 1), (2, 8, 5, 4), (1, 6, 7, 6), (3, 4, 9, 1)])
+def test_group_norm_vs_torch(oracle, B, C, L, G):
+    # crates/ratchet-core/src/ops/norm/groupnorm.rs:24-31 (F.group_norm is the only contract), tol 1e-4
+    rng = np.random.default_rng(19)
+    x = rng.standard_normal((B, C, L)).astype(np.float32)
+    w = rng.standard_normal(C).astype(np.float32)
+    b = rng.standard_normal(C).astype(np.float32)
+    want = F.group_norm(torch.from_numpy(x), G, torch.from_numpy(w), torch.from_numpy(b), eps=1e-5).numpy()
+    got = oracle.group_norm(x, G, w, b, 1e-5)
+    bad, mx = oracle.count_not_close(got, want, 1e-5, 1e-5)
+    assert bad == 0, mx
+
+
+def test_group_norm_reduces_to_layer_norm(oracle):
+    rng = np.random.default_rng(20)
+    x = rng.standard_normal((4, 32, 1)).astype(np.float32)         # G = 1, L = 1: LayerNorm over C
+    w = rng.standard_normal(32).astype(np.float32)
+    b = rng.standard_normal(32).astype(np.float32)
+    gn = oracle.group_norm(x, 1, w, b, 1e-5)[:, :, 0]
+    ln = F.layer_norm(torch.from_numpy(x[:, :, 0]), (32,), torch.from_numpy(w), torch.from_numpy(b), 1e-5).numpy()
+    assert np.allclose(gn, ln, atol=1e-5)
+
+
+# ------------------------------------------------------------------------------------------- reindex / concat
+def test_permute_vs_numpy(oracle):
+    rng = np.random.default_rng(21)
+    import itertools
+    x = rng.standard_normal((2, 3, 5, 7)).astype(np.float32)
+    for perm in itertools.permutations(range(4)):
+        assert np.array_equal(oracle.permute(x, perm), np.ascontiguousarray(x.transpose(perm)))
+    x3 = rng.standard_normal((4, 6, 10)).astype(np.float16)
+    for perm in itertools.permutations(range(3)):
+        assert np.array_equal(oracle.permute(x3, perm), np.ascontiguousarray(x3.transpose(perm)))
+    with pytest.raises(ValueError):
+        oracle.permute(x, (0, 1, 1, 3))
+
+
+def test_slice_vs_numpy(oracle):
+    rng = np.random.default_rng(22)
+    x = rng.standard_normal((6, 5, 9, 33)).astype(np.float32)
+    got = oracle.slice_(x, [(1, 4), (0, 5), (3, 8), (7, 30)])
+    assert np.array_equal(got, x[1:4, 0:5, 3:8, 7:30])
+    x2 = rng.standard_normal((10, 20)).astype(np.float16)
+    assert np.array_equal(oracle.slice_(x2, [(2, 3), (0, 20)]), x2[2:3, :])
+    with pytest.raises(ValueError):
+        oracle.slice_(x2, [(3, 3), (0, 20)])              # start < end is asserted (cpu/reindex.rs:103-105)
+
+
+def test_broadcast_vs_numpy_and_vector_special_case(oracle):
+    rng = np.random.default_rng(23)
+    for src, dst in [((1, 5, 1, 16), (3, 5, 4, 16)), ((1,), (4, 32, 8, 8)), ((2, 1, 1, 1), (2, 3, 4, 5)),
+                     ((7,), (2, 7)), ((3, 1), (3, 4)), ((1, 1, 6), (2, 5, 6))]:
+        x = rng.standard_normal(src).astype(np.float32)
+        assert np.array_equal(oracle.broadcast(x, dst), np.broadcast_to(x, dst)), (src, dst)
+    # the special case: a lower-rank vector whose length equals the destination's first dimension
+    v = np.array([1, 2, 3], dtype=np.float32)
+    assert np.array_equal(oracle.broadcast(v, (3, 3)), np.repeat(v, 3).reshape(3, 3))
+    assert np.array_equal(oracle.broadcast(v, (3, 3), numpy_semantics=True), np.broadcast_to(v, (3, 3)))
+    with pytest.raises(ValueError):
+        oracle.broadcast(np.zeros((2, 3), np.float32), (2, 4))
+
+
+def test_concat_reference_case(oracle):
+    # crates/ratchet-core/src/ops/concat.rs:273-359: five [4,2,{50,13,77,55,11},128] tensors along dim 2
+    rng = np.random.default_rng(24)
+    xs = [rng.standard_normal((4, 2, k, 128)).astype(np.float32) for k in (50, 13, 77, 55, 11)]
+    assert np.array_equal(oracle.concat(xs, 2), np.concatenate(xs, axis=2))
+    ys = [rng.standard_normal((3, k)).astype(np.float16) for k in (1, 4)]
+    assert np.array_equal(oracle.concat(ys, 1), np.concatenate(ys, axis=1))
+    zs = [rng.standard_normal((k, 3)).astype(np.float16) for k in (2, 5, 1)]
+    assert np.array_equal(oracle.concat(zs, 0), np.concatenate(zs, axis=0))
+    with pytest.raises(ValueError):
+        oracle.concat([np.zeros((2, 3), np.float32), np.zeros((3, 4), np.float32)], 0)
