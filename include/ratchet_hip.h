@@ -1,0 +1,141 @@
+/*
+ * ratchet_hip.h - C ABI of the MI355X (gfx950) device backend for ratchet-core's memory-bound tensor ops.
+ *
+ * This is the seam a Rust `-sys` crate binds: it takes the place of ratchet-core's wgpu storage layer, of its
+ * run-time WGSL kernel generation + dispatch, and of its command-encoder execution.  All citations are paths in
+ * huggingface/ratchet (crates/ratchet-core/src/...).
+ *
+ * Conventions
+ *   - status: 0 = ok; > 0 = rt error (enum below), detected before any HIP call; < 0 = -(hipError_t).
+ *   - every launch function enqueues on the device's single in-order stream and returns immediately; only
+ *     rt_sync, rt_h2d, rt_d2h, rt_event_elapsed_ms block.  Steps therefore run in call order, each seeing the
+ *     previous one's writes, as the reference's single compute pass does (executable.rs:33-59).
+ *   - shapes are rank-4, left-padded with 1s, exactly what Shape::promote(_, 4) produces (shape.rs:92-96).
+ *   - dtype codes: F32 = 0, F16 = 1 as DType::to_u32 (dtype/mod.rs:32-38); BF16 = 2, I32 = 3, U32 = 4 added.
+ *   - the caller owns every device pointer; the library allocates nothing inside launch functions except scratch
+ *     owned by rt_device (GroupNorm partial statistics, the f16 lookup tables).
+ *   - calls on one rt_device must be serialised by the caller (the reference keeps its device behind a RwLock,
+ *     gpu/device.rs:20-29).  rt_last_error() is thread-local.
+ *   - results follow ratchet's CPU executor (the cpu/ directory), including its f16 rounding points.
+ */
+#ifndef RATCHET_HIP_H
+#define RATCHET_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum rt_status {
+    RT_OK = 0,
+    RT_ERR_NULL_POINTER = 1,   /* a required pointer argument is NULL */
+    RT_ERR_DTYPE = 2,          /* dtype code not supported by this op */
+    RT_ERR_OP = 3,             /* op code out of range */
+    RT_ERR_SHAPE = 4,          /* shapes inconsistent (broadcast rule, concat rule, slice bounds, zero extent) */
+    RT_ERR_PERM = 5,           /* permutation is not a permutation of 0..3 (InvariantError::DuplicateDims) */
+    RT_ERR_SIZE = 6,           /* element count overflows what the kernels index (2^40 elements) */
+    RT_ERR_ARG = 7,            /* other bad argument (n_inputs, dim, groups, mode, elem_bytes, eps) */
+    RT_ERR_NULL_DEVICE = 8,    /* rt_device* is NULL */
+    RT_ERR_ALIGN = 9           /* pointer not aligned to its element size */
+};
+
+enum rt_dtype { RT_F32 = 0, RT_F16 = 1, RT_BF16 = 2, RT_I32 = 3, RT_U32 = 4 };
+/* BinaryOp, ops/binary.rs:19-24 */
+enum rt_binary_op { RT_ADD = 0, RT_SUB = 1, RT_MUL = 2, RT_DIV = 3 };
+/* UnaryOp, ops/unary.rs:23-38 */
+enum rt_unary_op {
+    RT_GELU = 0, RT_TANH, RT_EXP, RT_LOG, RT_SIN, RT_COS, RT_ABS, RT_SQRT,
+    RT_RELU, RT_FLOOR, RT_CEIL, RT_NEG, RT_SILU, RT_SIGMOID, RT_UNARY_COUNT
+};
+/* softmax arithmetic: REFERENCE reproduces cpu/softmax.rs (no max subtraction; for 16-bit types the row sum is
+ * accumulated sequentially in the element type); STABLE subtracts the row maximum and accumulates in f32. */
+enum rt_softmax_mode { RT_SOFTMAX_REFERENCE = 0, RT_SOFTMAX_STABLE = 1 };
+
+typedef struct rt_device rt_device;   /* opaque: HIP device ordinal + one stream + scratch */
+typedef struct rt_event rt_event;     /* opaque: a HIP event on a device's stream */
+
+/* ---- device / storage: replaces WgpuDevice (gpu/device.rs:18-30,53-119) and GPUBuffer
+ *      (storage/gpu_buffer.rs:20-94,153-158,199-218) ------------------------------------------------------- */
+int rt_device_count(int* out);
+int rt_device_create(int ordinal, rt_device** out);          /* Device::request_device (device.rs:61-77) */
+int rt_device_destroy(rt_device* dev);
+int rt_sync(rt_device* dev);                                 /* device.poll(Wait) (tensor.rs:855-856) */
+const char* rt_last_error(void);                             /* message for the last non-zero status, thread-local */
+const char* rt_status_name(int status);
+int rt_malloc(rt_device* dev, size_t bytes, void** dptr);    /* BufferPool::get_or_create (buffer_pool.rs:68-116): sizes
+                                                                are rounded up to 4 B, minimum 16 B (:82-93) */
+int rt_free(rt_device* dev, void* dptr);                     /* last drop of a PooledGPUBuffer */
+int rt_memset0(rt_device* dev, void* dptr, size_t bytes);    /* GPUBuffer::zeros (gpu_buffer.rs:29-37) */
+int rt_h2d(rt_device* dev, void* dptr, const void* host, size_t bytes);   /* GPUBuffer::from_bytes (:49-59), blocking */
+int rt_d2h(rt_device* dev, void* host, const void* dptr, size_t bytes);   /* GPUBuffer::to_cpu (:199-218), blocking */
+int rt_d2d(rt_device* dev, void* dst, const void* src, size_t bytes);     /* GPUBuffer::deep_clone (:61-94), async */
+
+/* timing helpers for benchmarks; take the place of the wgpu timestamp-query profiler (gpu/profiler.rs:95-238) */
+int rt_event_create(rt_device* dev, rt_event** out);
+int rt_event_destroy(rt_event* ev);
+int rt_event_record(rt_device* dev, rt_event* ev);
+int rt_event_elapsed_ms(rt_event* start, rt_event* stop, float* ms);      /* waits for `stop` */
+
+/* ---- ops: each replaces GPUOperation::compile_gpu (op.rs:280-362) + one dispatch of Executable::dispatch
+ *      (executable.rs:33-59) for the op named -------------------------------------------------------------- */
+
+/* Binary (ops/binary.rs:135-182; arithmetic cpu/binary.rs:27-32,85-88): y[i] = a[i] op b[i], equal lengths.
+ * y may alias a (the reference's in-place rule, tensor.rs:823-824) or b.  dt: F32, F16, BF16. */
+int rt_binary(rt_device* dev, int op, int dt, const void* a, const void* b, void* y, uint64_t numel);
+
+/* Binary with numpy broadcasting resolved at launch instead of a materialised broadcast_to operand
+ * (tensor.rs:249-280 inserts Broadcast; this fuses it).  a_shape/b_shape must each broadcast to y_shape
+ * (Shape::multi_broadcast, shape.rs:118-136).  Both sides may broadcast.  y must not alias a or b unless that
+ * operand already has y_shape. */
+int rt_binary_bcast(rt_device* dev, int op, int dt, const void* a, const uint32_t a_shape[4], const void* b,
+                    const uint32_t b_shape[4], void* y, const uint32_t y_shape[4]);
+
+/* Unary (ops/unary.rs:234-271; formulas cpu/unary.rs:43-66).  y may alias x.  dt: F32, F16, BF16. */
+int rt_unary(rt_device* dev, int op, int dt, const void* x, void* y, uint64_t numel);
+
+/* Cast (ops/cast.rs:113-132; cpu/mod.rs:116-156).  f32<->f16, f32<->bf16 numeric (round to nearest even);
+ * f32<->i32/u32 is a bit reinterpretation as in the reference; equal dtypes copy.  Never in place. */
+int rt_cast(rt_device* dev, int src_dt, int dst_dt, const void* x, void* y, uint64_t numel);
+
+/* Permute (ops/reindex/permute.rs:22-73; cpu/reindex.rs:43-72): dst_shape[i] = src_shape[perm[i]],
+ * dst[idx] = src[idx scattered through perm].  elem_bytes: 2 or 4. */
+int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uint32_t src_shape[4],
+               const uint32_t perm[4]);
+
+/* Slice (ops/reindex/slice.rs:22-69; cpu/reindex.rs:92-129): y = x[start : start + dst_shape] in every dim. */
+int rt_slice(rt_device* dev, int elem_bytes, const void* x, void* y, const uint32_t src_shape[4],
+             const uint32_t start[4], const uint32_t dst_shape[4]);
+
+/* Broadcast (ops/reindex/broadcast.rs:17-82; cpu/reindex.rs:181-222 generic_broadcast): numpy broadcast_to. */
+int rt_broadcast(rt_device* dev, int elem_bytes, const void* x, void* y, const uint32_t src_shape[4],
+                 const uint32_t dst_shape[4]);
+
+/* Concat (ops/concat.rs:13-158; cpu/mod.rs:158-182): 2..8 inputs, equal shapes except along dim. */
+int rt_concat(rt_device* dev, int elem_bytes, int n_inputs, const void* const* xs, const uint32_t (*shapes)[4],
+              int dim, void* y);
+
+/* Softmax over the last dimension (ops/softmax.rs:14-39,183-199; cpu/softmax.rs:22-42): rows x cols, contiguous.
+ * y may alias x (the reference kernel is in-place only, ops/softmax.rs:47-49).  dt: F32, F16, BF16. */
+int rt_softmax(rt_device* dev, int dt, const void* x, void* y, uint64_t rows, uint32_t cols, int mode);
+
+/* LayerNorm over the last dimension (ops/norm/mod.rs:17-91; cpu/norm.rs:91-147); bias may be NULL.
+ * eps is converted to the element type inside (T::from(eps), cpu/norm.rs:128). */
+int rt_layer_norm(rt_device* dev, int dt, const void* x, const void* scale, const void* bias, void* y,
+                  uint64_t rows, uint32_t cols, float eps);
+
+/* RMSNorm over the last dimension (cpu/norm.rs:185-213). */
+int rt_rms_norm(rt_device* dev, int dt, const void* x, const void* scale, void* y, uint64_t rows, uint32_t cols,
+                float eps);
+
+/* GroupNorm on [B, C, L] with per-channel scale/bias (either may be NULL): the semantics of
+ * torch.nn.functional.group_norm, which is the reference test's ground truth (ops/norm/groupnorm.rs:24-31);
+ * the reference's own CPU implementation is a no-op (cpu/norm.rs:215-219). */
+int rt_group_norm(rt_device* dev, int dt, const void* x, const void* scale, const void* bias, void* y, uint32_t B,
+                  uint32_t C, uint32_t L, uint32_t groups, float eps);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,244 @@
+// Device, storage and timing entry points of the C ABI: hipMalloc'd storage and one in-order stream take the place
+// of ratchet-core's wgpu device, buffer pool and queue (gpu/device.rs, gpu/pools/buffer_pool.rs,
+// storage/gpu_buffer.rs in crates/ratchet-core/src).
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "rt_internal.h"
+
+static thread_local char g_err[512] = "";
+
+int rt_fail(int status, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+int rt_fail_hip(hipError_t e, const char* what) {
+    snprintf(g_err, sizeof(g_err), "%s: %s (%s)", what, hipGetErrorString(e), hipGetErrorName(e));
+    (void)hipGetLastError();   // clear the sticky error so the next call reports its own
+    return -(int)e;
+}
+
+int rt_enter(rt_device* dev) {
+    if (!dev) return rt_fail(RT_ERR_NULL_DEVICE, "rt_device is NULL");
+    hipError_t e = hipSetDevice(dev->ordinal);
+    if (e != hipSuccess) return rt_fail_hip(e, "hipSetDevice");
+    return RT_OK;
+}
+
+// bytes [0, head) and the tail after the last whole 16-byte vector are cleared bytewise by block 0
+__global__ void __launch_bounds__(256) zero_bytes_kernel(unsigned char* p, size_t head, size_t nvec, size_t bytes) {
+    uint4* v = reinterpret_cast<uint4*>(p + head);
+    const size_t base = (size_t)blockIdx.x * (256 * 4) + threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const size_t i = base + (size_t)k * 256;
+        if (i < nvec) v[i] = make_uint4(0, 0, 0, 0);
+    }
+    if (blockIdx.x == 0) {
+        const size_t tail_start = head + nvec * 16;
+        for (size_t i = threadIdx.x; i < head; i += 256) p[i] = 0;
+        for (size_t i = tail_start + threadIdx.x; i < bytes; i += 256) p[i] = 0;
+    }
+}
+
+extern "C" {
+
+const char* rt_last_error(void) { return g_err; }
+
+const char* rt_status_name(int status) {
+    switch (status) {
+        case RT_OK: return "RT_OK";
+        case RT_ERR_NULL_POINTER: return "RT_ERR_NULL_POINTER";
+        case RT_ERR_DTYPE: return "RT_ERR_DTYPE";
+        case RT_ERR_OP: return "RT_ERR_OP";
+        case RT_ERR_SHAPE: return "RT_ERR_SHAPE";
+        case RT_ERR_PERM: return "RT_ERR_PERM";
+        case RT_ERR_SIZE: return "RT_ERR_SIZE";
+        case RT_ERR_ARG: return "RT_ERR_ARG";
+        case RT_ERR_NULL_DEVICE: return "RT_ERR_NULL_DEVICE";
+        case RT_ERR_ALIGN: return "RT_ERR_ALIGN";
+        default: return status < 0 ? "HIP_ERROR" : "RT_ERR_UNKNOWN";
+    }
+}
+
+int rt_device_count(int* out) {
+    RT_REQUIRE(out, RT_ERR_NULL_POINTER, "rt_device_count: out is NULL");
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) {
+        *out = 0;
+        return rt_fail_hip(e, "hipGetDeviceCount");
+    }
+    *out = n;
+    return RT_OK;
+}
+
+int rt_device_create(int ordinal, rt_device** out) {
+    RT_REQUIRE(out, RT_ERR_NULL_POINTER, "rt_device_create: out is NULL");
+    *out = nullptr;
+    RT_REQUIRE(ordinal >= 0, RT_ERR_ARG, "rt_device_create: negative ordinal %d", ordinal);
+    int n = 0;
+    RT_HIP(hipGetDeviceCount(&n));
+    RT_REQUIRE(ordinal < n, RT_ERR_ARG, "rt_device_create: ordinal %d but %d device(s) visible", ordinal, n);
+    RT_HIP(hipSetDevice(ordinal));
+    hipDeviceProp_t prop;
+    RT_HIP(hipGetDeviceProperties(&prop, ordinal));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return rt_fail(RT_ERR_ARG, "rt_device_create: device %d is %s; this library is built for gfx950 only", ordinal,
+                       prop.gcnArchName);
+    rt_device* dev = new rt_device();
+    memset(dev, 0, sizeof(*dev));
+    dev->ordinal = ordinal;
+    dev->num_cus = prop.multiProcessorCount;
+    hipError_t e = hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking);   // default priority
+    if (e != hipSuccess) {
+        delete dev;
+        return rt_fail_hip(e, "hipStreamCreateWithFlags");
+    }
+    dev->gn_scratch_bytes = 1u << 20;
+    e = hipMalloc((void**)&dev->gn_scratch, dev->gn_scratch_bytes);
+    if (e != hipSuccess) {
+        (void)hipStreamDestroy(dev->stream);
+        delete dev;
+        return rt_fail_hip(e, "hipMalloc(scratch)");
+    }
+    *out = dev;
+    return RT_OK;
+}
+
+int rt_device_destroy(rt_device* dev) {
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    (void)hipStreamSynchronize(dev->stream);
+    for (int i = 0; i < RT_UNARY_COUNT; i++)
+        if (dev->unary_lut[i]) (void)hipFree(dev->unary_lut[i]);
+    if (dev->gn_scratch) (void)hipFree(dev->gn_scratch);
+    hipError_t e = hipStreamDestroy(dev->stream);
+    delete dev;
+    if (e != hipSuccess) return rt_fail_hip(e, "hipStreamDestroy");
+    return RT_OK;
+}
+
+int rt_sync(rt_device* dev) {
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    RT_HIP(hipStreamSynchronize(dev->stream));
+    return RT_OK;
+}
+
+int rt_malloc(rt_device* dev, size_t bytes, void** dptr) {
+    RT_REQUIRE(dptr, RT_ERR_NULL_POINTER, "rt_malloc: dptr is NULL");
+    *dptr = nullptr;
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    // the reference rounds sizes up to 4 bytes and never allocates less than 16 (buffer_pool.rs:82-93)
+    size_t sz = (bytes + 3) & ~(size_t)3;
+    if (sz < 16) sz = 16;
+    RT_HIP(hipMalloc(dptr, sz));
+    return RT_OK;
+}
+
+int rt_free(rt_device* dev, void* dptr) {
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    if (!dptr) return RT_OK;
+    // work queued on the stream may still use the buffer
+    RT_HIP(hipStreamSynchronize(dev->stream));
+    RT_HIP(hipFree(dptr));
+    return RT_OK;
+}
+
+int rt_memset0(rt_device* dev, void* dptr, size_t bytes) {
+    RT_REQUIRE(dptr || bytes == 0, RT_ERR_NULL_POINTER, "rt_memset0: dptr is NULL");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    if (bytes == 0) return RT_OK;
+    // a fill kernel rather than hipMemsetAsync, so that a caller may capture this call in a HIP graph
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(dptr);
+    const size_t head = (size_t)((16 - (addr & 15)) & 15) < bytes ? (size_t)((16 - (addr & 15)) & 15) : bytes;
+    const size_t nvec = (bytes - head) / 16;
+    const size_t per_block = 256 * 4;
+    const size_t blocks = nvec ? (nvec + per_block - 1) / per_block : 1;
+    RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_memset0: %zu bytes is too large", bytes);
+    hipLaunchKernelGGL(zero_bytes_kernel, dim3((unsigned)blocks), dim3(256), 0, dev->stream, (unsigned char*)dptr, head,
+                       nvec, bytes);
+    RT_CHECK_LAUNCH("zero_bytes_kernel");
+    return RT_OK;
+}
+
+int rt_h2d(rt_device* dev, void* dptr, const void* host, size_t bytes) {
+    RT_REQUIRE((dptr && host) || bytes == 0, RT_ERR_NULL_POINTER, "rt_h2d: NULL pointer");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    if (bytes == 0) return RT_OK;
+    RT_HIP(hipMemcpyAsync(dptr, host, bytes, hipMemcpyHostToDevice, dev->stream));
+    RT_HIP(hipStreamSynchronize(dev->stream));
+    return RT_OK;
+}
+
+int rt_d2h(rt_device* dev, void* host, const void* dptr, size_t bytes) {
+    RT_REQUIRE((dptr && host) || bytes == 0, RT_ERR_NULL_POINTER, "rt_d2h: NULL pointer");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    if (bytes == 0) return RT_OK;
+    RT_HIP(hipMemcpyAsync(host, dptr, bytes, hipMemcpyDeviceToHost, dev->stream));
+    RT_HIP(hipStreamSynchronize(dev->stream));
+    return RT_OK;
+}
+
+int rt_d2d(rt_device* dev, void* dst, const void* src, size_t bytes) {
+    RT_REQUIRE((dst && src) || bytes == 0, RT_ERR_NULL_POINTER, "rt_d2d: NULL pointer");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    if (bytes == 0) return RT_OK;
+    RT_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, dev->stream));
+    return RT_OK;
+}
+
+int rt_event_create(rt_device* dev, rt_event** out) {
+    RT_REQUIRE(out, RT_ERR_NULL_POINTER, "rt_event_create: out is NULL");
+    *out = nullptr;
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    rt_event* ev = new rt_event();
+    ev->ordinal = dev->ordinal;
+    hipError_t e = hipEventCreate(&ev->ev);
+    if (e != hipSuccess) {
+        delete ev;
+        return rt_fail_hip(e, "hipEventCreate");
+    }
+    *out = ev;
+    return RT_OK;
+}
+
+int rt_event_destroy(rt_event* ev) {
+    RT_REQUIRE(ev, RT_ERR_NULL_POINTER, "rt_event_destroy: event is NULL");
+    (void)hipSetDevice(ev->ordinal);
+    hipError_t e = hipEventDestroy(ev->ev);
+    delete ev;
+    if (e != hipSuccess) return rt_fail_hip(e, "hipEventDestroy");
+    return RT_OK;
+}
+
+int rt_event_record(rt_device* dev, rt_event* ev) {
+    RT_REQUIRE(ev, RT_ERR_NULL_POINTER, "rt_event_record: event is NULL");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    RT_HIP(hipEventRecord(ev->ev, dev->stream));
+    return RT_OK;
+}
+
+int rt_event_elapsed_ms(rt_event* start, rt_event* stop, float* ms) {
+    RT_REQUIRE(start && stop && ms, RT_ERR_NULL_POINTER, "rt_event_elapsed_ms: NULL argument");
+    (void)hipSetDevice(stop->ordinal);
+    RT_HIP(hipEventSynchronize(stop->ev));
+    RT_HIP(hipEventElapsedTime(ms, start->ev, stop->ev));
+    return RT_OK;
+}
+
+}  // extern "C"

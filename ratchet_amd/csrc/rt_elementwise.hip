@@ -1,0 +1,525 @@
+// Elementwise kernels: binary (contiguous and broadcast-fused), unary, cast.
+//
+// All of them are streaming kernels bounded by HBM bandwidth: every lane moves 16 bytes per access (dwordx4), a
+// 256-thread block covers UNROLL consecutive 4 KiB slabs per operand so that a wave always touches one contiguous
+// 1 KiB span, and loads of a whole tile are issued before the first store.  Arithmetic follows rt_arith.h.
+#include "rt_arith.h"
+#include "rt_internal.h"
+
+namespace {
+
+constexpr int BLOCK = 256;
+constexpr int UNROLL = 4;
+
+// ------------------------------------------------------------------------------------------------ binary, contiguous
+template <typename T, int OP>
+__global__ void __launch_bounds__(BLOCK) binary_vec_kernel(const T* __restrict__ a, const T* __restrict__ b, T* y,
+                                                           uint64_t numel) {
+    constexpr int VE = 16 / sizeof(T);
+    const uint64_t nvec = numel / VE;
+    const uint4* av = reinterpret_cast<const uint4*>(a);
+    const uint4* bv = reinterpret_cast<const uint4*>(b);
+    uint4* yv = reinterpret_cast<uint4*>(y);
+    const uint64_t base = (uint64_t)blockIdx.x * (BLOCK * UNROLL) + threadIdx.x;
+    Vec16<T> ra[UNROLL], rb[UNROLL];
+#pragma unroll
+    for (int k = 0; k < UNROLL; k++) {
+        const uint64_t i = base + (uint64_t)k * BLOCK;
+        if (i < nvec) {
+            ra[k].u = av[i];
+            rb[k].u = bv[i];
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < UNROLL; k++) {
+        const uint64_t i = base + (uint64_t)k * BLOCK;
+        if (i < nvec) {
+            Vec16<T> r;
+#pragma unroll
+            for (int e = 0; e < VE; e++) r.e[e] = ar_binary<OP, T>(ra[k].e[e], rb[k].e[e]);
+            yv[i] = r.u;
+        }
+    }
+    if (blockIdx.x == 0) {                              // the numel % VE trailing elements
+        const uint64_t i = nvec * VE + threadIdx.x;
+        if (i < numel) y[i] = ar_binary<OP, T>(a[i], b[i]);
+    }
+}
+
+// fallback for pointers that are not 16-byte aligned
+template <typename T, int OP>
+__global__ void __launch_bounds__(BLOCK) binary_scalar_kernel(const T* a, const T* b, T* y, uint64_t numel) {
+    const uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+    if (i < numel) y[i] = ar_binary<OP, T>(a[i], b[i]);
+}
+
+// ------------------------------------------------------------------------------------------------ binary, broadcast
+// y_shape = [d0, d1, d2, d3]; a/b strides in elements, 0 on broadcast dims.  One thread per VE consecutive outputs of
+// the last dimension; an operand whose last-dim stride is 0 is loaded once and splatted.
+struct BcastArgs {
+    FastDiv cv;        // column vectors per row = d3 / VE
+    FastDiv d2, d1;
+    uint32_t as[4], bs[4];
+    uint32_t nvec;     // total vectors
+};
+
+template <typename T, int OP, int VE>
+__global__ void __launch_bounds__(BLOCK) binary_bcast_kernel(const T* __restrict__ a, const T* __restrict__ b,
+                                                             T* __restrict__ y, BcastArgs p) {
+    const uint32_t base = blockIdx.x * (BLOCK * UNROLL) + threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < UNROLL; k++) {
+        const uint32_t v = base + k * BLOCK;
+        if (v >= p.nvec) break;
+        uint32_t row, col, i0, i1, i2, t;
+        fd_divmod(v, p.cv, row, col);
+        fd_divmod(row, p.d2, t, i2);
+        fd_divmod(t, p.d1, i0, i1);
+        const uint64_t ao = (uint64_t)i0 * p.as[0] + (uint64_t)i1 * p.as[1] + (uint64_t)i2 * p.as[2] +
+                            (uint64_t)col * VE * p.as[3];
+        const uint64_t bo = (uint64_t)i0 * p.bs[0] + (uint64_t)i1 * p.bs[1] + (uint64_t)i2 * p.bs[2] +
+                            (uint64_t)col * VE * p.bs[3];
+        T ra[VE], rb[VE], r[VE];
+        if (VE > 1 && p.as[3] == 1) {
+            Vec16<T> t16;
+            t16.u = *reinterpret_cast<const uint4*>(a + ao);
+#pragma unroll
+            for (int e = 0; e < VE; e++) ra[e] = t16.e[e];
+        } else {
+#pragma unroll
+            for (int e = 0; e < VE; e++) ra[e] = a[ao + (uint64_t)e * p.as[3]];
+        }
+        if (VE > 1 && p.bs[3] == 1) {
+            Vec16<T> t16;
+            t16.u = *reinterpret_cast<const uint4*>(b + bo);
+#pragma unroll
+            for (int e = 0; e < VE; e++) rb[e] = t16.e[e];
+        } else {
+#pragma unroll
+            for (int e = 0; e < VE; e++) rb[e] = b[bo + (uint64_t)e * p.bs[3]];
+        }
+#pragma unroll
+        for (int e = 0; e < VE; e++) r[e] = ar_binary<OP, T>(ra[e], rb[e]);
+        const uint64_t yo = (uint64_t)v * VE;
+        if (VE > 1) {
+            Vec16<T> t16;
+#pragma unroll
+            for (int e = 0; e < VE; e++) t16.e[e] = r[e];
+            *reinterpret_cast<uint4*>(y + yo) = t16.u;
+        } else {
+            y[yo] = r[0];
+        }
+    }
+}
+
+// "suffix" broadcast: b spans the trailing dims of y entirely (bias over rows, an [S,S] mask over heads) and a has
+// y's shape: y[o, i] = a[o, i] op b[i].  A thread keeps its 16 bytes of b in registers and walks `orows` outer rows,
+// so b is read from memory once per outer chunk instead of once per output row.
+template <typename T, int OP>
+__global__ void __launch_bounds__(BLOCK) binary_suffix_kernel(const T* __restrict__ a, const T* __restrict__ b,
+                                                              T* __restrict__ y, uint32_t inner_vec, uint32_t outer,
+                                                              uint32_t orows, int b_is_lhs) {
+    constexpr int VE = 16 / sizeof(T);
+    const uint32_t iv = blockIdx.x * BLOCK + threadIdx.x;
+    if (iv >= inner_vec) return;
+    Vec16<T> rb;
+    rb.u = reinterpret_cast<const uint4*>(b)[iv];
+    const uint32_t o0 = blockIdx.y * orows;
+    const uint32_t o1 = (o0 + orows < outer) ? o0 + orows : outer;
+    const uint4* av = reinterpret_cast<const uint4*>(a);
+    uint4* yv = reinterpret_cast<uint4*>(y);
+    for (uint32_t o = o0; o < o1; o += UNROLL) {
+        Vec16<T> ra[UNROLL];
+#pragma unroll
+        for (int k = 0; k < UNROLL; k++)
+            if (o + k < o1) ra[k].u = av[(uint64_t)(o + k) * inner_vec + iv];
+#pragma unroll
+        for (int k = 0; k < UNROLL; k++) {
+            if (o + k < o1) {
+                Vec16<T> r;
+#pragma unroll
+                for (int e = 0; e < VE; e++)
+                    r.e[e] = b_is_lhs ? ar_binary<OP, T>(rb.e[e], ra[k].e[e]) : ar_binary<OP, T>(ra[k].e[e], rb.e[e]);
+                yv[(uint64_t)(o + k) * inner_vec + iv] = r.u;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ unary
+template <typename T, int OP>
+__global__ void __launch_bounds__(BLOCK) unary_vec_kernel(const T* __restrict__ x, T* y, uint64_t numel) {
+    constexpr int VE = 16 / sizeof(T);
+    const uint64_t nvec = numel / VE;
+    const uint4* xv = reinterpret_cast<const uint4*>(x);
+    uint4* yv = reinterpret_cast<uint4*>(y);
+    const uint64_t base = (uint64_t)blockIdx.x * (BLOCK * UNROLL) + threadIdx.x;
+    Vec16<T> rx[UNROLL];
+#pragma unroll
+    for (int k = 0; k < UNROLL; k++) {
+        const uint64_t i = base + (uint64_t)k * BLOCK;
+        if (i < nvec) rx[k].u = xv[i];
+    }
+#pragma unroll
+    for (int k = 0; k < UNROLL; k++) {
+        const uint64_t i = base + (uint64_t)k * BLOCK;
+        if (i < nvec) {
+            Vec16<T> r;
+#pragma unroll
+            for (int e = 0; e < VE; e++) r.e[e] = ar_unary<OP, T>(rx[k].e[e]);
+            yv[i] = r.u;
+        }
+    }
+    if (blockIdx.x == 0) {
+        const uint64_t i = nvec * VE + threadIdx.x;
+        if (i < numel) y[i] = ar_unary<OP, T>(x[i]);
+    }
+}
+
+template <typename T, int OP>
+__global__ void __launch_bounds__(BLOCK) unary_scalar_kernel(const T* x, T* y, uint64_t numel) {
+    const uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+    if (i < numel) y[i] = ar_unary<OP, T>(x[i]);
+}
+
+// ------------------------------------------------------------------------------------------------ cast
+template <typename S, typename D> __device__ __forceinline__ D cast_one(S v);
+template <> __device__ __forceinline__ half_t cast_one<float, half_t>(float v) { return (half_t)v; }
+template <> __device__ __forceinline__ float cast_one<half_t, float>(half_t v) { return (float)v; }
+template <> __device__ __forceinline__ bf16_t cast_one<float, bf16_t>(float v) { return Ar<bf16_t>::conv(v); }
+template <> __device__ __forceinline__ float cast_one<bf16_t, float>(bf16_t v) { return Ar<bf16_t>::widen(v); }
+
+// 8 elements per thread: 16 bytes on the 2-byte side, 2 x 16 bytes on the 4-byte side
+template <typename S, typename D>
+__global__ void __launch_bounds__(BLOCK) cast_vec_kernel(const S* __restrict__ x, D* __restrict__ y, uint64_t numel) {
+    constexpr int PER = 8;
+    const uint64_t ngrp = numel / PER;
+    const uint64_t base = (uint64_t)blockIdx.x * (BLOCK * 2) + threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        const uint64_t g = base + (uint64_t)k * BLOCK;
+        if (g < ngrp) {
+            S in[PER];
+            D out[PER];
+            const uint4* src = reinterpret_cast<const uint4*>(x + g * PER);
+            constexpr int NS = PER * sizeof(S) / 16, ND = PER * sizeof(D) / 16;
+            uint4 raw[NS];
+#pragma unroll
+            for (int q = 0; q < NS; q++) raw[q] = src[q];
+            __builtin_memcpy(in, raw, sizeof(in));
+#pragma unroll
+            for (int e = 0; e < PER; e++) out[e] = cast_one<S, D>(in[e]);
+            uint4 o[ND];
+            __builtin_memcpy(o, out, sizeof(out));
+            uint4* dst = reinterpret_cast<uint4*>(y + g * PER);
+#pragma unroll
+            for (int q = 0; q < ND; q++) dst[q] = o[q];
+        }
+    }
+    if (blockIdx.x == 0) {
+        const uint64_t i = ngrp * PER + threadIdx.x;
+        if (i < numel) y[i] = cast_one<S, D>(x[i]);
+    }
+}
+
+template <typename S, typename D>
+__global__ void __launch_bounds__(BLOCK) cast_scalar_kernel(const S* x, D* y, uint64_t numel) {
+    const uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+    if (i < numel) y[i] = cast_one<S, D>(x[i]);
+}
+
+// plain copy (same-dtype cast, f32 <-> i32/u32 reinterpretation)
+__global__ void __launch_bounds__(BLOCK) copy_vec_kernel(const unsigned char* __restrict__ x, unsigned char* __restrict__ y,
+                                                         uint64_t bytes) {
+    const uint64_t nvec = bytes / 16;
+    const uint4* xv = reinterpret_cast<const uint4*>(x);
+    uint4* yv = reinterpret_cast<uint4*>(y);
+    const uint64_t base = (uint64_t)blockIdx.x * (BLOCK * UNROLL) + threadIdx.x;
+    uint4 r[UNROLL];
+#pragma unroll
+    for (int k = 0; k < UNROLL; k++) {
+        const uint64_t i = base + (uint64_t)k * BLOCK;
+        if (i < nvec) r[k] = xv[i];
+    }
+#pragma unroll
+    for (int k = 0; k < UNROLL; k++) {
+        const uint64_t i = base + (uint64_t)k * BLOCK;
+        if (i < nvec) yv[i] = r[k];
+    }
+    if (blockIdx.x == 0) {
+        const uint64_t i = nvec * 16 + threadIdx.x;
+        if (i < bytes) y[i] = x[i];
+    }
+}
+__global__ void __launch_bounds__(BLOCK) copy_bytes_kernel(const unsigned char* x, unsigned char* y, uint64_t bytes) {
+    const uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+    if (i < bytes) y[i] = x[i];
+}
+
+// ------------------------------------------------------------------------------------------------ launch helpers
+inline unsigned blocks_for(uint64_t items, uint64_t per_block) {
+    const uint64_t b = (items + per_block - 1) / per_block;
+    return (unsigned)(b ? b : 1);
+}
+
+template <typename T, int OP>
+int launch_binary(rt_device* dev, const void* a, const void* b, void* y, uint64_t numel) {
+    const bool vec = rt_aligned(a, 16) && rt_aligned(b, 16) && rt_aligned(y, 16);
+    if (vec) {
+        constexpr int VE = 16 / sizeof(T);
+        hipLaunchKernelGGL((binary_vec_kernel<T, OP>), dim3(blocks_for(numel / VE, BLOCK * UNROLL)), dim3(BLOCK), 0,
+                           dev->stream, (const T*)a, (const T*)b, (T*)y, numel);
+    } else {
+        hipLaunchKernelGGL((binary_scalar_kernel<T, OP>), dim3(blocks_for(numel, BLOCK)), dim3(BLOCK), 0, dev->stream,
+                           (const T*)a, (const T*)b, (T*)y, numel);
+    }
+    RT_CHECK_LAUNCH("binary kernel");
+    return RT_OK;
+}
+
+template <typename T>
+int dispatch_binary(rt_device* dev, int op, const void* a, const void* b, void* y, uint64_t numel) {
+    switch (op) {
+        case RT_ADD: return launch_binary<T, RT_ADD>(dev, a, b, y, numel);
+        case RT_SUB: return launch_binary<T, RT_SUB>(dev, a, b, y, numel);
+        case RT_MUL: return launch_binary<T, RT_MUL>(dev, a, b, y, numel);
+        default: return launch_binary<T, RT_DIV>(dev, a, b, y, numel);
+    }
+}
+
+template <typename T, int OP>
+int launch_unary(rt_device* dev, const void* x, void* y, uint64_t numel) {
+    const bool vec = rt_aligned(x, 16) && rt_aligned(y, 16);
+    if (vec) {
+        constexpr int VE = 16 / sizeof(T);
+        hipLaunchKernelGGL((unary_vec_kernel<T, OP>), dim3(blocks_for(numel / VE, BLOCK * UNROLL)), dim3(BLOCK), 0,
+                           dev->stream, (const T*)x, (T*)y, numel);
+    } else {
+        hipLaunchKernelGGL((unary_scalar_kernel<T, OP>), dim3(blocks_for(numel, BLOCK)), dim3(BLOCK), 0, dev->stream,
+                           (const T*)x, (T*)y, numel);
+    }
+    RT_CHECK_LAUNCH("unary kernel");
+    return RT_OK;
+}
+
+template <typename T> int dispatch_unary(rt_device* dev, int op, const void* x, void* y, uint64_t numel) {
+    switch (op) {
+#define RT_CASE(OPC) case OPC: return launch_unary<T, OPC>(dev, x, y, numel);
+        RT_CASE(RT_GELU) RT_CASE(RT_TANH) RT_CASE(RT_EXP) RT_CASE(RT_LOG) RT_CASE(RT_SIN) RT_CASE(RT_COS)
+        RT_CASE(RT_ABS) RT_CASE(RT_SQRT) RT_CASE(RT_RELU) RT_CASE(RT_FLOOR) RT_CASE(RT_CEIL) RT_CASE(RT_NEG)
+        RT_CASE(RT_SILU) RT_CASE(RT_SIGMOID)
+#undef RT_CASE
+        default: return rt_fail(RT_ERR_OP, "rt_unary: op %d out of range", op);
+    }
+}
+
+template <typename S, typename D> int launch_cast(rt_device* dev, const void* x, void* y, uint64_t numel) {
+    if (rt_aligned(x, 16) && rt_aligned(y, 16)) {
+        hipLaunchKernelGGL((cast_vec_kernel<S, D>), dim3(blocks_for(numel / 8, BLOCK * 2)), dim3(BLOCK), 0, dev->stream,
+                           (const S*)x, (D*)y, numel);
+    } else {
+        hipLaunchKernelGGL((cast_scalar_kernel<S, D>), dim3(blocks_for(numel, BLOCK)), dim3(BLOCK), 0, dev->stream,
+                           (const S*)x, (D*)y, numel);
+    }
+    RT_CHECK_LAUNCH("cast kernel");
+    return RT_OK;
+}
+
+int launch_copy(rt_device* dev, const void* x, void* y, uint64_t bytes) {
+    if (rt_aligned(x, 16) && rt_aligned(y, 16)) {
+        hipLaunchKernelGGL(copy_vec_kernel, dim3(blocks_for(bytes / 16, BLOCK * UNROLL)), dim3(BLOCK), 0, dev->stream,
+                           (const unsigned char*)x, (unsigned char*)y, bytes);
+    } else {
+        hipLaunchKernelGGL(copy_bytes_kernel, dim3(blocks_for(bytes, BLOCK)), dim3(BLOCK), 0, dev->stream,
+                           (const unsigned char*)x, (unsigned char*)y, bytes);
+    }
+    RT_CHECK_LAUNCH("copy kernel");
+    return RT_OK;
+}
+
+// strides (in elements) of an operand of shape s broadcast against y: 0 where the operand's extent is 1
+inline void bcast_strides(const uint32_t s[4], uint32_t out[4]) {
+    uint64_t st = 1;
+    for (int i = 3; i >= 0; i--) {
+        out[i] = (s[i] == 1) ? 0u : (uint32_t)st;
+        st *= s[i];
+    }
+}
+
+template <typename T, int OP>
+int launch_bcast(rt_device* dev, const void* a, const uint32_t a_shape[4], const void* b, const uint32_t b_shape[4], void* y,
+                 const uint32_t y_shape[4], uint64_t y_numel) {
+    constexpr int VEMAX = 16 / sizeof(T);
+    uint64_t a_numel = 1, b_numel = 1;
+    for (int i = 0; i < 4; i++) { a_numel *= a_shape[i]; b_numel *= b_shape[i]; }
+
+    // suffix fast path: one operand has y's shape, the other equals y's trailing dims with leading 1s
+    for (int which = 0; which < 2; which++) {
+        const uint32_t* part = which == 0 ? b_shape : a_shape;
+        const void* fullp = which == 0 ? a : b;
+        const void* partp = which == 0 ? b : a;
+        const uint64_t part_numel = which == 0 ? b_numel : a_numel;
+        const uint64_t full_numel = which == 0 ? a_numel : b_numel;
+        if (full_numel != y_numel || part_numel == y_numel || part_numel < (uint64_t)VEMAX) continue;
+        bool suffix = true, seen_non1 = false;
+        for (int i = 0; i < 4; i++) {
+            if (part[i] != 1) seen_non1 = true;
+            if (seen_non1 && part[i] != y_shape[i]) suffix = false;
+        }
+        if (!suffix || part_numel % VEMAX != 0) continue;
+        if (!(rt_aligned(fullp, 16) && rt_aligned(partp, 16) && rt_aligned(y, 16))) continue;
+        const uint64_t inner_vec = part_numel / VEMAX;
+        const uint64_t outer = y_numel / part_numel;
+        if (inner_vec > 0xffffffffull || outer > 0xffffffffull) continue;
+        // enough blocks to fill the chip, while each thread reuses its slice of b over as many rows as possible
+        const uint64_t bx = (inner_vec + BLOCK - 1) / BLOCK;
+        uint64_t by = (4096 + bx - 1) / bx;
+        if (by > outer) by = outer;
+        if (by > 65535) by = 65535;
+        if (by < 1) by = 1;
+        const uint32_t orows = (uint32_t)((outer + by - 1) / by);
+        by = (outer + orows - 1) / orows;
+        if (bx > 0x7fffffffull) continue;
+        hipLaunchKernelGGL((binary_suffix_kernel<T, OP>), dim3((unsigned)bx, (unsigned)by), dim3(BLOCK), 0, dev->stream,
+                           (const T*)fullp, (const T*)partp, (T*)y, (uint32_t)inner_vec, (uint32_t)outer, orows, which == 1);
+        RT_CHECK_LAUNCH("binary_suffix_kernel");
+        return RT_OK;
+    }
+
+    BcastArgs p;
+    bcast_strides(a_shape, p.as);
+    bcast_strides(b_shape, p.bs);
+    // vector width: the last dim must split into whole vectors, every vector-loaded operand must keep 16-byte alignment
+    int ve = VEMAX;
+    auto operand_ok = [&](const void* ptr, const uint32_t st[4]) {
+        if (st[3] == 0) return true;                               // splat: scalar loads
+        if (!rt_aligned(ptr, 16)) return false;
+        for (int i = 0; i < 3; i++)
+            if (st[i] % VEMAX != 0) return false;
+        return true;
+    };
+    if (y_shape[3] % VEMAX != 0 || !rt_aligned(y, 16) || !operand_ok(a, p.as) || !operand_ok(b, p.bs)) ve = 1;
+    const uint64_t nvec = y_numel / ve;
+    RT_REQUIRE(nvec <= 0xffffffffull - (uint64_t)BLOCK * UNROLL, RT_ERR_SIZE,
+               "rt_binary_bcast: %llu output vectors exceed the 32-bit index space", (unsigned long long)nvec);
+    p.cv = make_fastdiv(y_shape[3] / ve);
+    p.d2 = make_fastdiv(y_shape[2]);
+    p.d1 = make_fastdiv(y_shape[1]);
+    p.nvec = (uint32_t)nvec;
+    const unsigned blocks = blocks_for(nvec, BLOCK * UNROLL);
+    if (ve == VEMAX) {
+        hipLaunchKernelGGL((binary_bcast_kernel<T, OP, VEMAX>), dim3(blocks), dim3(BLOCK), 0, dev->stream, (const T*)a,
+                           (const T*)b, (T*)y, p);
+    } else {
+        hipLaunchKernelGGL((binary_bcast_kernel<T, OP, 1>), dim3(blocks), dim3(BLOCK), 0, dev->stream, (const T*)a,
+                           (const T*)b, (T*)y, p);
+    }
+    RT_CHECK_LAUNCH("binary_bcast_kernel");
+    return RT_OK;
+}
+
+template <typename T>
+int dispatch_bcast(rt_device* dev, int op, const void* a, const uint32_t as[4], const void* b, const uint32_t bs[4], void* y,
+                   const uint32_t ys[4], uint64_t n) {
+    switch (op) {
+        case RT_ADD: return launch_bcast<T, RT_ADD>(dev, a, as, b, bs, y, ys, n);
+        case RT_SUB: return launch_bcast<T, RT_SUB>(dev, a, as, b, bs, y, ys, n);
+        case RT_MUL: return launch_bcast<T, RT_MUL>(dev, a, as, b, bs, y, ys, n);
+        default: return launch_bcast<T, RT_DIV>(dev, a, as, b, bs, y, ys, n);
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int rt_binary(rt_device* dev, int op, int dt, const void* a, const void* b, void* y, uint64_t numel) {
+    RT_REQUIRE(op >= RT_ADD && op <= RT_DIV, RT_ERR_OP, "rt_binary: op %d out of range", op);
+    RT_REQUIRE(rt_is_float_dt(dt), RT_ERR_DTYPE, "rt_binary: dtype %d is not F32/F16/BF16", dt);
+    RT_REQUIRE(numel <= RT_MAX_NUMEL, RT_ERR_SIZE, "rt_binary: numel %llu too large", (unsigned long long)numel);
+    if (numel == 0) return dev ? RT_OK : rt_fail(RT_ERR_NULL_DEVICE, "rt_device is NULL");
+    RT_REQUIRE(a && b && y, RT_ERR_NULL_POINTER, "rt_binary: NULL operand");
+    const size_t eb = (size_t)rt_dt_bytes(dt);
+    RT_REQUIRE(rt_aligned(a, eb) && rt_aligned(b, eb) && rt_aligned(y, eb), RT_ERR_ALIGN, "rt_binary: misaligned pointer");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    switch (dt) {
+        case RT_F32: return dispatch_binary<float>(dev, op, a, b, y, numel);
+        case RT_F16: return dispatch_binary<half_t>(dev, op, a, b, y, numel);
+        default: return dispatch_binary<bf16_t>(dev, op, a, b, y, numel);
+    }
+}
+
+int rt_binary_bcast(rt_device* dev, int op, int dt, const void* a, const uint32_t a_shape[4], const void* b,
+                    const uint32_t b_shape[4], void* y, const uint32_t y_shape[4]) {
+    RT_REQUIRE(op >= RT_ADD && op <= RT_DIV, RT_ERR_OP, "rt_binary_bcast: op %d out of range", op);
+    RT_REQUIRE(rt_is_float_dt(dt), RT_ERR_DTYPE, "rt_binary_bcast: dtype %d is not F32/F16/BF16", dt);
+    RT_REQUIRE(a_shape && b_shape && y_shape, RT_ERR_NULL_POINTER, "rt_binary_bcast: NULL shape");
+    uint64_t n = 1;
+    for (int i = 0; i < 4; i++) {
+        RT_REQUIRE(a_shape[i] > 0 && b_shape[i] > 0 && y_shape[i] > 0, RT_ERR_SHAPE, "rt_binary_bcast: zero extent in dim %d", i);
+        // Shape::multi_broadcast (shape.rs:118-136): each operand extent is 1 or the output extent
+        RT_REQUIRE((a_shape[i] == 1 || a_shape[i] == y_shape[i]) && (b_shape[i] == 1 || b_shape[i] == y_shape[i]) &&
+                       (y_shape[i] == (a_shape[i] > b_shape[i] ? a_shape[i] : b_shape[i])),
+                   RT_ERR_SHAPE, "rt_binary_bcast: dim %d: %u and %u do not broadcast to %u", i, a_shape[i], b_shape[i],
+                   y_shape[i]);
+        n *= y_shape[i];
+        RT_REQUIRE(n <= RT_MAX_NUMEL, RT_ERR_SIZE, "rt_binary_bcast: output too large");
+    }
+    RT_REQUIRE(a && b && y, RT_ERR_NULL_POINTER, "rt_binary_bcast: NULL operand");
+    const size_t eb = (size_t)rt_dt_bytes(dt);
+    RT_REQUIRE(rt_aligned(a, eb) && rt_aligned(b, eb) && rt_aligned(y, eb), RT_ERR_ALIGN,
+               "rt_binary_bcast: misaligned pointer");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    bool same = true;
+    for (int i = 0; i < 4; i++) same = same && a_shape[i] == y_shape[i] && b_shape[i] == y_shape[i];
+    if (same) return rt_binary(dev, op, dt, a, b, y, n);
+    switch (dt) {
+        case RT_F32: return dispatch_bcast<float>(dev, op, a, a_shape, b, b_shape, y, y_shape, n);
+        case RT_F16: return dispatch_bcast<half_t>(dev, op, a, a_shape, b, b_shape, y, y_shape, n);
+        default: return dispatch_bcast<bf16_t>(dev, op, a, a_shape, b, b_shape, y, y_shape, n);
+    }
+}
+
+int rt_unary(rt_device* dev, int op, int dt, const void* x, void* y, uint64_t numel) {
+    RT_REQUIRE(op >= 0 && op < RT_UNARY_COUNT, RT_ERR_OP, "rt_unary: op %d out of range", op);
+    RT_REQUIRE(rt_is_float_dt(dt), RT_ERR_DTYPE, "rt_unary: dtype %d is not F32/F16/BF16", dt);
+    RT_REQUIRE(numel <= RT_MAX_NUMEL, RT_ERR_SIZE, "rt_unary: numel %llu too large", (unsigned long long)numel);
+    if (numel == 0) return dev ? RT_OK : rt_fail(RT_ERR_NULL_DEVICE, "rt_device is NULL");
+    RT_REQUIRE(x && y, RT_ERR_NULL_POINTER, "rt_unary: NULL operand");
+    const size_t eb = (size_t)rt_dt_bytes(dt);
+    RT_REQUIRE(rt_aligned(x, eb) && rt_aligned(y, eb), RT_ERR_ALIGN, "rt_unary: misaligned pointer");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    switch (dt) {
+        case RT_F32: return dispatch_unary<float>(dev, op, x, y, numel);
+        case RT_F16: return dispatch_unary<half_t>(dev, op, x, y, numel);
+        default: return dispatch_unary<bf16_t>(dev, op, x, y, numel);
+    }
+}
+
+int rt_cast(rt_device* dev, int src_dt, int dst_dt, const void* x, void* y, uint64_t numel) {
+    const int sb = rt_dt_bytes(src_dt), db = rt_dt_bytes(dst_dt);
+    RT_REQUIRE(sb && db, RT_ERR_DTYPE, "rt_cast: unknown dtype %d -> %d", src_dt, dst_dt);
+    // the conversions cpu_cast implements (cpu/mod.rs:131-153); anything else is unimplemented!() there
+    const bool numeric = (src_dt == RT_F32 && (dst_dt == RT_F16 || dst_dt == RT_BF16)) ||
+                         ((src_dt == RT_F16 || src_dt == RT_BF16) && dst_dt == RT_F32);
+    const bool reinterpret = (src_dt == RT_F32 && (dst_dt == RT_I32 || dst_dt == RT_U32)) ||
+                             ((src_dt == RT_I32 || src_dt == RT_U32) && dst_dt == RT_F32);
+    RT_REQUIRE(numeric || reinterpret || src_dt == dst_dt, RT_ERR_DTYPE, "rt_cast: %d -> %d is not a supported cast", src_dt,
+               dst_dt);
+    RT_REQUIRE(numel <= RT_MAX_NUMEL, RT_ERR_SIZE, "rt_cast: numel %llu too large", (unsigned long long)numel);
+    if (numel == 0) return dev ? RT_OK : rt_fail(RT_ERR_NULL_DEVICE, "rt_device is NULL");
+    RT_REQUIRE(x && y, RT_ERR_NULL_POINTER, "rt_cast: NULL operand");
+    RT_REQUIRE(rt_aligned(x, (size_t)sb) && rt_aligned(y, (size_t)db), RT_ERR_ALIGN, "rt_cast: misaligned pointer");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    if (!numeric) return (x == y) ? RT_OK : launch_copy(dev, x, y, numel * (uint64_t)sb);
+    if (src_dt == RT_F32 && dst_dt == RT_F16) return launch_cast<float, half_t>(dev, x, y, numel);
+    if (src_dt == RT_F32 && dst_dt == RT_BF16) return launch_cast<float, bf16_t>(dev, x, y, numel);
+    if (src_dt == RT_F16) return launch_cast<half_t, float>(dev, x, y, numel);
+    return launch_cast<bf16_t, float>(dev, x, y, numel);
+}
+
+}  // extern "C"

@@ -1,0 +1,98 @@
+// Internal definitions shared by the HIP translation units of libratchet_hip.so (gfx950 only).
+#ifndef RT_INTERNAL_H
+#define RT_INTERNAL_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+#include "../../include/ratchet_hip.h"
+
+struct rt_device {
+    int ordinal;
+    hipStream_t stream;
+    int num_cus;
+    // GroupNorm partial statistics: {mean, m2, count} triples, one per (group, split)
+    float* gn_scratch;
+    size_t gn_scratch_bytes;
+    // 65536-entry f16 -> f16 lookup tables, built on first use by the exact kernels (index = rt_unary_op)
+    uint16_t* unary_lut[RT_UNARY_COUNT];
+};
+
+struct rt_event {
+    hipEvent_t ev;
+    int ordinal;
+};
+
+// error reporting (thread-local message)
+int rt_fail(int status, const char* fmt, ...);
+int rt_fail_hip(hipError_t e, const char* what);
+
+#define RT_HIP(call)                                         \
+    do {                                                     \
+        hipError_t _e = (call);                              \
+        if (_e != hipSuccess) return rt_fail_hip(_e, #call); \
+    } while (0)
+
+#define RT_REQUIRE(cond, status, ...)                          \
+    do {                                                       \
+        if (!(cond)) return rt_fail((status), __VA_ARGS__);    \
+    } while (0)
+
+// Returns rt_fail_hip(...) if the launch that was just enqueued was rejected.
+#define RT_CHECK_LAUNCH(name)                                   \
+    do {                                                        \
+        hipError_t _e = hipGetLastError();                      \
+        if (_e != hipSuccess) return rt_fail_hip(_e, name);     \
+    } while (0)
+
+static inline bool rt_is_float_dt(int dt) { return dt == RT_F32 || dt == RT_F16 || dt == RT_BF16; }
+static inline int rt_dt_bytes(int dt) {
+    switch (dt) {
+        case RT_F32: case RT_I32: case RT_U32: return 4;
+        case RT_F16: case RT_BF16: return 2;
+        default: return 0;
+    }
+}
+static inline bool rt_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// the kernels index elements with 64-bit integers but grid sizes are 32-bit; 2^40 elements is far beyond 288 GB
+static const uint64_t RT_MAX_NUMEL = 1ull << 40;
+
+// Makes dev's ordinal current.  Every entry point calls it first.
+int rt_enter(rt_device* dev);
+
+// ---------------------------------------------------------------------------------------------------------
+// u32 division by a launch-time constant: q = (n * m) >> (32 + s), exact for all n < 2^32 (round-up method)
+// ---------------------------------------------------------------------------------------------------------
+struct FastDiv {
+    uint32_t d;   // divisor
+    uint32_t m;   // magic multiplier
+    uint32_t s;   // post shift
+    uint32_t add; // 1: use the (n + hi) / 2 correction path
+};
+static inline FastDiv make_fastdiv(uint32_t d) {
+    FastDiv f;
+    f.d = d;
+    if (d == 1) { f.m = 0; f.s = 0; f.add = 2; return f; }   // add == 2: identity
+    uint32_t l = 0;
+    while ((1ull << l) < d) l++;                              // l = ceil(log2 d)
+    const uint64_t m = ((1ull << 32) * ((1ull << l) - d)) / d + 1;
+    f.m = (uint32_t)m;
+    f.s = l - 1;
+    f.add = 1;
+    return f;
+}
+#ifdef __HIPCC__
+__device__ __forceinline__ uint32_t fd_div(uint32_t n, const FastDiv& f) {
+    if (f.add == 2) return n;
+    const uint32_t t = __umulhi(n, f.m);
+    return (t + ((n - t) >> 1)) >> f.s;
+}
+__device__ __forceinline__ void fd_divmod(uint32_t n, const FastDiv& f, uint32_t& q, uint32_t& r) {
+    q = fd_div(n, f);
+    r = n - q * f.d;
+}
+#endif
+
+#endif

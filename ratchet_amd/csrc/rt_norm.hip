@@ -1,0 +1,469 @@
+// LayerNorm, RMSNorm (one wave64 per row, row held in registers, 16-byte loads, butterfly reductions) and GroupNorm
+// (split statistics + apply, two launches).
+//
+// Arithmetic contract for LayerNorm / RMSNorm = crates/ratchet-core/src/cpu/norm.rs:91-147,185-213, in the element type T
+// with one rounding per operation:
+//     mu   = sum(x) / T(N)                 (sum::<T>: f32 accumulation; for 16-bit T rounded to T once)
+//     x2   = sum(x*x) / T(N)               (each square rounded to T first)
+//     var  = x2 - mu*mu                    (E[x^2] - mu^2, not a two-pass variance)
+//     r    = T(1) / sqrt(var + T(eps))
+//     y    = ((x - mu) * r) * scale + bias
+// f32 rows: one wave64 per row, the row stays in registers, the additions form a butterfly tree instead of the
+//   reference's sequential fold; that changes the sums by float rounding only (far inside the 1e-5 bar).
+// 16-bit rows: the two sums are rounded to the 16-bit type before they are used (sum(x*x) ~ N has an ulp of 1-2 there),
+//   so a different f32 summation order can flip that rounding and move a whole row by an ulp of r, more than 1e-3
+//   allows.  These kernels therefore replay the reference's order exactly: tiles of x and T(x*x) are staged through LDS
+//   as f32 and one lane per (row, sum) walks its row left to right with v_add_f32.  The walk is latency bound
+//   (one dependent add per element), so many small row groups run side by side.
+// GroupNorm follows torch.nn.functional.group_norm, the ground truth of the reference's own test
+// (ops/norm/groupnorm.rs:24-31): statistics in f32 (Chan-combined partial mean/M2), f32 arithmetic, one final rounding.
+#include "rt_arith.h"
+#include "rt_internal.h"
+
+namespace {
+
+constexpr int WAVE = 64;
+constexpr int BLOCK = 256;
+constexpr int WAVES = BLOCK / WAVE;
+
+enum { NORM_LAYER = 0, NORM_RMS = 1 };
+
+// per-row statistics in T arithmetic, given f32 sums
+template <typename T> struct RowStats {
+    T mu, r;
+};
+template <typename T, int KIND> __device__ __forceinline__ RowStats<T> finish_stats(float sum_x, float sum_sq, uint32_t cols, float eps) {
+    typedef Ar<T> A;
+    RowStats<T> st;
+    const T n = A::conv((float)cols);                       // T::from(step as f32)
+    const T x2 = A::div(A::conv(sum_sq), n);
+    T var;
+    if (KIND == NORM_LAYER) {
+        st.mu = A::div(A::conv(sum_x), n);
+        var = A::sub(x2, A::mul(st.mu, st.mu));
+    } else {
+        st.mu = A::conv(0.0f);
+        var = x2;
+    }
+    const T t = A::add(var, A::conv(eps));
+    st.r = A::div(A::conv(1.0f), ar_sqrt<T>(t));
+    return st;
+}
+
+template <typename T, int KIND> __device__ __forceinline__ T norm_one(T x, const RowStats<T>& st, T scale, T bias, bool has_bias) {
+    typedef Ar<T> A;
+    T v = (KIND == NORM_LAYER) ? A::sub(x, st.mu) : x;
+    v = A::mul(v, st.r);
+    v = A::mul(v, scale);
+    if (KIND == NORM_LAYER && has_bias) v = A::add(v, bias);
+    return v;
+}
+
+// cols % VE == 0, rows 16-byte aligned, cols / VE <= 64 * NV
+template <typename T, int NV, int KIND>
+__global__ void __launch_bounds__(BLOCK) norm_wave_kernel(const T* __restrict__ x, const T* __restrict__ scale,
+                                                          const T* __restrict__ bias, T* __restrict__ y, uint64_t rows, uint32_t cols,
+                                                          float eps) {
+    constexpr int VE = 16 / sizeof(T);
+    const uint64_t row = (uint64_t)blockIdx.x * WAVES + (threadIdx.x / WAVE);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & (WAVE - 1);
+    const uint32_t nvec = cols / VE;
+    const uint4* xr = reinterpret_cast<const uint4*>(x + row * cols);
+    uint4* yr = reinterpret_cast<uint4*>(y + row * cols);
+    Vec16<T> v[NV];
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        const uint32_t i = lane + k * WAVE;
+        if (i < nvec) v[k].u = xr[i];
+    }
+    float sx = 0.0f, sq = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NV; k++)
+        if (lane + k * WAVE < nvec)
+#pragma unroll
+            for (int q = 0; q < VE; q++) {
+                const T e = v[k].e[q];
+                if (KIND == NORM_LAYER) sx += Ar<T>::widen(e);
+                sq += Ar<T>::widen(Ar<T>::mul(e, e));
+            }
+    if (KIND == NORM_LAYER) sx = wave_sum(sx);
+    sq = wave_sum(sq);
+    const RowStats<T> st = finish_stats<T, KIND>(sx, sq, cols, eps);
+    const uint4* sv = reinterpret_cast<const uint4*>(scale);
+    const uint4* bv = reinterpret_cast<const uint4*>(bias);
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        const uint32_t i = lane + k * WAVE;
+        if (i < nvec) {
+            Vec16<T> s, b, o;
+            s.u = sv[i];
+            if (KIND == NORM_LAYER && bias) b.u = bv[i];
+#pragma unroll
+            for (int q = 0; q < VE; q++) o.e[q] = norm_one<T, KIND>(v[k].e[q], st, s.e[q], b.e[q], bias != nullptr);
+            yr[i] = o.u;
+        }
+    }
+}
+
+// any cols / alignment: one block per row, scalar accesses, the row is re-read from cache for the second pass
+template <typename T, int KIND>
+__global__ void __launch_bounds__(BLOCK) norm_generic_kernel(const T* __restrict__ x, const T* __restrict__ scale,
+                                                             const T* __restrict__ bias, T* __restrict__ y, uint64_t rows, uint32_t cols,
+                                                             float eps) {
+    __shared__ float red[2][WAVES];
+    const uint64_t row = blockIdx.x;
+    const T* xr = x + row * cols;
+    T* yr = y + row * cols;
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    float sx = 0.0f, sq = 0.0f;
+    for (uint32_t j = threadIdx.x; j < cols; j += BLOCK) {
+        const T e = xr[j];
+        sx += Ar<T>::widen(e);
+        sq += Ar<T>::widen(Ar<T>::mul(e, e));
+    }
+    sx = wave_sum(sx);
+    sq = wave_sum(sq);
+    if (lane == 0) { red[0][wave] = sx; red[1][wave] = sq; }
+    __syncthreads();
+    sx = red[0][0]; sq = red[1][0];
+    for (int w = 1; w < WAVES; w++) { sx += red[0][w]; sq += red[1][w]; }
+    const RowStats<T> st = finish_stats<T, KIND>(sx, sq, cols, eps);
+    for (uint32_t j = threadIdx.x; j < cols; j += BLOCK) {
+        const T b = (KIND == NORM_LAYER && bias) ? bias[j] : Ar<T>::conv(0.0f);
+        yr[j] = norm_one<T, KIND>(xr[j], st, scale[j], b, bias != nullptr);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// 16-bit LayerNorm / RMSNorm with the reference's sequential f32 accumulation.
+// A block owns RB consecutive rows.  Pass A: per column tile, all threads load 16-byte vectors, widen x and T(x*x) to
+// f32 and park them in LDS; lanes [0, RB) then add the squares of "their" row left to right, lanes [RB, 2RB) the values
+// (LayerNorm only).  Pass B re-reads x (from cache: the block touched it moments ago), normalises and stores.
+// ------------------------------------------------------------------------------------------------------------------
+template <typename T, int RB, int KIND, bool VEC>
+__global__ void __launch_bounds__(BLOCK) norm_seq16_kernel(const T* __restrict__ x, const T* __restrict__ scale,
+                                                           const T* __restrict__ bias, T* __restrict__ y, uint64_t rows, uint32_t cols,
+                                                           float eps) {
+    constexpr int TC = 128;
+    constexpr int PAD = 4;
+    constexpr int VE = VEC ? 8 : 1;
+    constexpr int TV = TC / VE;
+    constexpr int NSUM = (KIND == NORM_LAYER) ? 2 : 1;
+    __shared__ __attribute__((aligned(16))) float tile[NSUM][RB][TC + PAD];      // [0] = squares, [1] = values
+    __shared__ float sums[NSUM][RB];
+    __shared__ T s_mu[RB], s_r[RB];
+    const uint64_t row0 = (uint64_t)blockIdx.x * RB;
+    const uint32_t nrows = (rows - row0 < (uint64_t)RB) ? (uint32_t)(rows - row0) : (uint32_t)RB;
+    const uint32_t wrow = threadIdx.x % RB, wsum = threadIdx.x / RB;                // walker role of this thread
+    const bool walker = (threadIdx.x < NSUM * RB) && (wrow < nrows);
+    float run = 0.0f;
+
+    for (uint32_t c0 = 0; c0 < cols; c0 += TC) {
+        const uint32_t ncol = (cols - c0 < (uint32_t)TC) ? cols - c0 : (uint32_t)TC;
+        for (uint32_t idx = threadIdx.x; idx < (uint32_t)RB * TV; idx += BLOCK) {
+            const uint32_t r = idx / TV, col = (idx % TV) * VE;
+            if (r < nrows && col < ncol) {
+                const T* src = x + (row0 + r) * cols + c0 + col;
+                if (VEC) {
+                    Vec16<T> in;
+                    in.u = *reinterpret_cast<const uint4*>(src);
+                    float sq[8], xv[8];
+#pragma unroll
+                    for (int q = 0; q < 8; q++) {
+                        sq[q] = Ar<T>::widen(Ar<T>::mul(in.e[q], in.e[q]));
+                        xv[q] = Ar<T>::widen(in.e[q]);
+                    }
+                    float4* d0 = reinterpret_cast<float4*>(&tile[0][r][col]);
+                    d0[0] = make_float4(sq[0], sq[1], sq[2], sq[3]);
+                    d0[1] = make_float4(sq[4], sq[5], sq[6], sq[7]);
+                    if (KIND == NORM_LAYER) {
+                        float4* d1 = reinterpret_cast<float4*>(&tile[NSUM - 1][r][col]);
+                        d1[0] = make_float4(xv[0], xv[1], xv[2], xv[3]);
+                        d1[1] = make_float4(xv[4], xv[5], xv[6], xv[7]);
+                    }
+                } else {
+                    const T e = *src;
+                    tile[0][r][col] = Ar<T>::widen(Ar<T>::mul(e, e));
+                    if (KIND == NORM_LAYER) tile[NSUM - 1][r][col] = Ar<T>::widen(e);
+                }
+            }
+        }
+        __syncthreads();
+        if (walker) {
+            const float* trow = tile[wsum][wrow];
+            uint32_t j = 0;
+            for (; j + 4 <= ncol; j += 4) {
+                const float4 t = *reinterpret_cast<const float4*>(trow + j);
+                run += t.x;
+                run += t.y;
+                run += t.z;
+                run += t.w;
+            }
+            for (; j < ncol; j++) run += trow[j];
+        }
+        __syncthreads();
+    }
+    if (walker) sums[wsum][wrow] = run;
+    __syncthreads();
+    if (threadIdx.x < nrows) {
+        const RowStats<T> st = finish_stats<T, KIND>(KIND == NORM_LAYER ? sums[NSUM - 1][threadIdx.x] : 0.0f, sums[0][threadIdx.x],
+                                                     cols, eps);
+        s_mu[threadIdx.x] = st.mu;
+        s_r[threadIdx.x] = st.r;
+    }
+    __syncthreads();
+
+    const uint32_t cvec = cols / VE;
+    for (uint32_t r = 0; r < nrows; r++) {
+        RowStats<T> st;
+        st.mu = s_mu[r];
+        st.r = s_r[r];
+        const T* src = x + (row0 + r) * cols;
+        T* dst = y + (row0 + r) * cols;
+        for (uint32_t cv = threadIdx.x; cv < cvec; cv += BLOCK) {
+            if (VEC) {
+                Vec16<T> in, sc, bi, out;
+                in.u = reinterpret_cast<const uint4*>(src)[cv];
+                sc.u = reinterpret_cast<const uint4*>(scale)[cv];
+                if (KIND == NORM_LAYER && bias) bi.u = reinterpret_cast<const uint4*>(bias)[cv];
+#pragma unroll
+                for (int q = 0; q < 8; q++) out.e[q] = norm_one<T, KIND>(in.e[q], st, sc.e[q], bi.e[q], bias != nullptr);
+                reinterpret_cast<uint4*>(dst)[cv] = out.u;
+            } else {
+                const T b = (KIND == NORM_LAYER && bias) ? bias[cv] : Ar<T>::conv(0.0f);
+                dst[cv] = norm_one<T, KIND>(src[cv], st, scale[cv], b, bias != nullptr);
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// GroupNorm.  x is [B, C, L] contiguous, so group (b, g) is one contiguous run of glen = (C/G)*L elements.
+// stats kernel: grid (B*G, splits); block s of a group reduces elements [s*chunk, min((s+1)*chunk, glen)) to
+//               (mean, M2, count) with a two-pass local variance (second pass re-reads the slice from cache).
+// apply kernel: same grid; every block combines the group's partials (Chan et al.), then normalises its slice:
+//               y = (x - mean) * rstd * w[c] + b[c], f32 arithmetic, rounded to T once.
+// ------------------------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(BLOCK) gn_stats_kernel(const T* __restrict__ x, float* __restrict__ part, uint32_t glen,
+                                                         uint32_t chunk, uint32_t splits) {
+    __shared__ float red[WAVES];
+    __shared__ float bc;
+    const uint32_t s = blockIdx.y, grp = blockIdx.x;
+    const T* xs = x + (uint64_t)grp * glen;
+    const uint32_t c0 = s * chunk;
+    const uint32_t c1 = (c0 + chunk < glen) ? c0 + chunk : glen;
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    float acc = 0.0f;
+    for (uint32_t i = c0 + threadIdx.x; i < c1; i += BLOCK) acc += Ar<T>::widen(xs[i]);
+    acc = wave_sum(acc);
+    if (lane == 0) red[wave] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = 0.0f;
+        for (int w = 0; w < WAVES; w++) t += red[w];
+        bc = t / (float)(c1 - c0);
+    }
+    __syncthreads();
+    const float mean = bc;
+    float m2 = 0.0f;
+    for (uint32_t i = c0 + threadIdx.x; i < c1; i += BLOCK) {
+        const float d = Ar<T>::widen(xs[i]) - mean;
+        m2 += d * d;
+    }
+    m2 = wave_sum(m2);
+    __syncthreads();
+    if (lane == 0) red[wave] = m2;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = 0.0f;
+        for (int w = 0; w < WAVES; w++) t += red[w];
+        float* o = part + ((uint64_t)grp * splits + s) * 3;
+        o[0] = mean;
+        o[1] = t;
+        o[2] = (float)(c1 - c0);
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(BLOCK) gn_apply_kernel(const T* __restrict__ x, const T* __restrict__ scale,
+                                                         const T* __restrict__ bias, T* __restrict__ y,
+                                                         const float* __restrict__ part, uint32_t glen, uint32_t chunk, uint32_t splits,
+                                                         uint32_t cpg, uint32_t groups, FastDiv L, float eps) {
+    const uint32_t s = blockIdx.y, grp = blockIdx.x;
+    // every thread combines the (few) partials itself: no shared memory, no barrier
+    double n = 0.0, mean = 0.0, m2 = 0.0;
+    const float* p = part + (uint64_t)grp * splits * 3;
+    for (uint32_t k = 0; k < splits; k++) {
+        const double nb = (double)p[3 * k + 2], mb = (double)p[3 * k], m2b = (double)p[3 * k + 1];
+        const double nt = n + nb;
+        const double delta = mb - mean;
+        mean += delta * (nb / nt);
+        m2 += m2b + delta * delta * (n * nb / nt);
+        n = nt;
+    }
+    const float meanf = (float)mean;
+    const float rstd = (float)(1.0 / sqrt(m2 / n + (double)eps));
+    const uint32_t g = grp % groups;
+    const T* xs = x + (uint64_t)grp * glen;
+    T* ys = y + (uint64_t)grp * glen;
+    const uint32_t c0 = s * chunk;
+    const uint32_t c1 = (c0 + chunk < glen) ? c0 + chunk : glen;
+    for (uint32_t i = c0 + threadIdx.x; i < c1; i += BLOCK) {
+        const uint32_t c = g * cpg + fd_div(i, L);
+        const float w = scale ? Ar<T>::widen(scale[c]) : 1.0f;
+        const float b = bias ? Ar<T>::widen(bias[c]) : 0.0f;
+        const float v = (Ar<T>::widen(xs[i]) - meanf) * rstd;
+        ys[i] = Ar<T>::conv(v * w + b);
+    }
+}
+
+template <typename T, int KIND>
+int launch_norm(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint64_t rows, uint32_t cols, float eps) {
+    constexpr int VE = 16 / sizeof(T);
+    const bool vec_ok = (cols % VE == 0) && rt_aligned(x, 16) && rt_aligned(y, 16) && rt_aligned(scale, 16) &&
+                        (!bias || rt_aligned(bias, 16)) && (cols / VE) <= (uint32_t)(WAVE * 8);
+    if (vec_ok) {
+        const uint32_t nv = (cols / VE + WAVE - 1) / WAVE;
+        const uint64_t blocks = (rows + WAVES - 1) / WAVES;
+        RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
+        const dim3 grid((unsigned)blocks), block(BLOCK);
+#define RT_NORM(NVC)                                                                                                           \
+    hipLaunchKernelGGL((norm_wave_kernel<T, NVC, KIND>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, \
+                       (T*)y, rows, cols, eps)
+        if (nv <= 1) RT_NORM(1);
+        else if (nv <= 2) RT_NORM(2);
+        else if (nv <= 3) RT_NORM(3);
+        else if (nv <= 4) RT_NORM(4);
+        else if (nv <= 5) RT_NORM(5);
+        else if (nv <= 6) RT_NORM(6);
+        else RT_NORM(8);
+#undef RT_NORM
+        RT_CHECK_LAUNCH("norm_wave_kernel");
+        return RT_OK;
+    }
+    RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
+    hipLaunchKernelGGL((norm_generic_kernel<T, KIND>), dim3((unsigned)rows), dim3(BLOCK), 0, dev->stream, (const T*)x, (const T*)scale,
+                       (const T*)bias, (T*)y, rows, cols, eps);
+    RT_CHECK_LAUNCH("norm_generic_kernel");
+    return RT_OK;
+}
+
+template <typename T, int KIND, int RB>
+int launch_norm16_rb(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint64_t rows, uint32_t cols, float eps) {
+    const uint64_t blocks = (rows + RB - 1) / RB;
+    RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
+    const bool vec_ok = (cols % 8 == 0) && rt_aligned(x, 16) && rt_aligned(y, 16) && rt_aligned(scale, 16) && (!bias || rt_aligned(bias, 16));
+    if (vec_ok) {
+        hipLaunchKernelGGL((norm_seq16_kernel<T, RB, KIND, true>), dim3((unsigned)blocks), dim3(BLOCK), 0, dev->stream, (const T*)x,
+                           (const T*)scale, (const T*)bias, (T*)y, rows, cols, eps);
+    } else {
+        hipLaunchKernelGGL((norm_seq16_kernel<T, RB, KIND, false>), dim3((unsigned)blocks), dim3(BLOCK), 0, dev->stream, (const T*)x,
+                           (const T*)scale, (const T*)bias, (T*)y, rows, cols, eps);
+    }
+    RT_CHECK_LAUNCH("norm_seq16_kernel");
+    return RT_OK;
+}
+
+// the row walk is latency bound, so prefer many small row groups until the chip is covered a few times over
+template <typename T, int KIND>
+int launch_norm16(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint64_t rows, uint32_t cols, float eps) {
+    const uint64_t want_blocks = (uint64_t)dev->num_cus * 4;
+    if (rows / 32 >= want_blocks) return launch_norm16_rb<T, KIND, 32>(dev, x, scale, bias, y, rows, cols, eps);
+    if (rows / 16 >= want_blocks) return launch_norm16_rb<T, KIND, 16>(dev, x, scale, bias, y, rows, cols, eps);
+    return launch_norm16_rb<T, KIND, 8>(dev, x, scale, bias, y, rows, cols, eps);
+}
+
+int norm_entry(rt_device* dev, int kind, int dt, const void* x, const void* scale, const void* bias, void* y, uint64_t rows,
+               uint32_t cols, float eps, const char* who) {
+    RT_REQUIRE(rt_is_float_dt(dt), RT_ERR_DTYPE, "%s: dtype %d is not F32/F16/BF16", who, dt);
+    RT_REQUIRE(cols > 0, RT_ERR_SHAPE, "%s: cols is 0", who);
+    RT_REQUIRE(rows <= RT_MAX_NUMEL / cols, RT_ERR_SIZE, "%s: tensor too large", who);
+    RT_REQUIRE(eps == eps, RT_ERR_ARG, "%s: eps is NaN", who);
+    if (rows == 0) return dev ? RT_OK : rt_fail(RT_ERR_NULL_DEVICE, "rt_device is NULL");
+    RT_REQUIRE(x && scale && y, RT_ERR_NULL_POINTER, "%s: NULL operand", who);
+    const size_t eb = (size_t)rt_dt_bytes(dt);
+    RT_REQUIRE(rt_aligned(x, eb) && rt_aligned(y, eb) && rt_aligned(scale, eb) && (!bias || rt_aligned(bias, eb)), RT_ERR_ALIGN,
+               "%s: misaligned pointer", who);
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    if (kind == NORM_LAYER) {
+        switch (dt) {
+            case RT_F32: return launch_norm<float, NORM_LAYER>(dev, x, scale, bias, y, rows, cols, eps);
+            case RT_F16: return launch_norm16<half_t, NORM_LAYER>(dev, x, scale, bias, y, rows, cols, eps);
+            default: return launch_norm16<bf16_t, NORM_LAYER>(dev, x, scale, bias, y, rows, cols, eps);
+        }
+    }
+    switch (dt) {
+        case RT_F32: return launch_norm<float, NORM_RMS>(dev, x, scale, nullptr, y, rows, cols, eps);
+        case RT_F16: return launch_norm16<half_t, NORM_RMS>(dev, x, scale, nullptr, y, rows, cols, eps);
+        default: return launch_norm16<bf16_t, NORM_RMS>(dev, x, scale, nullptr, y, rows, cols, eps);
+    }
+}
+
+template <typename T>
+int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint32_t bg, uint32_t glen, uint32_t cpg,
+              uint32_t groups, uint32_t L, float eps) {
+    // enough blocks to cover the chip, slices of at least 2048 elements
+    uint32_t splits = (2048 + bg - 1) / bg;
+    const uint32_t max_splits = (glen + 2047) / 2048;
+    if (splits > max_splits) splits = max_splits;
+    if (splits > 64) splits = 64;
+    if (splits < 1) splits = 1;
+    const uint32_t chunk = (glen + splits - 1) / splits;
+    splits = (glen + chunk - 1) / chunk;
+    const size_t need = (size_t)bg * splits * 3 * sizeof(float);
+    if (need > dev->gn_scratch_bytes) {
+        RT_HIP(hipStreamSynchronize(dev->stream));
+        RT_HIP(hipFree(dev->gn_scratch));
+        dev->gn_scratch = nullptr;
+        dev->gn_scratch_bytes = 0;
+        RT_HIP(hipMalloc((void**)&dev->gn_scratch, need));
+        dev->gn_scratch_bytes = need;
+    }
+    const dim3 grid(bg, splits), block(BLOCK);
+    hipLaunchKernelGGL((gn_stats_kernel<T>), grid, block, 0, dev->stream, (const T*)x, dev->gn_scratch, glen, chunk, splits);
+    RT_CHECK_LAUNCH("gn_stats_kernel");
+    hipLaunchKernelGGL((gn_apply_kernel<T>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, (T*)y,
+                       (const float*)dev->gn_scratch, glen, chunk, splits, cpg, groups, make_fastdiv(L), eps);
+    RT_CHECK_LAUNCH("gn_apply_kernel");
+    return RT_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rt_layer_norm(rt_device* dev, int dt, const void* x, const void* scale, const void* bias, void* y, uint64_t rows, uint32_t cols,
+                  float eps) {
+    return norm_entry(dev, NORM_LAYER, dt, x, scale, bias, y, rows, cols, eps, "rt_layer_norm");
+}
+
+int rt_rms_norm(rt_device* dev, int dt, const void* x, const void* scale, void* y, uint64_t rows, uint32_t cols, float eps) {
+    return norm_entry(dev, NORM_RMS, dt, x, scale, nullptr, y, rows, cols, eps, "rt_rms_norm");
+}
+
+int rt_group_norm(rt_device* dev, int dt, const void* x, const void* scale, const void* bias, void* y, uint32_t B, uint32_t C, uint32_t L,
+                  uint32_t groups, float eps) {
+    RT_REQUIRE(rt_is_float_dt(dt), RT_ERR_DTYPE, "rt_group_norm: dtype %d is not F32/F16/BF16", dt);
+    RT_REQUIRE(B > 0 && C > 0 && L > 0, RT_ERR_SHAPE, "rt_group_norm: zero extent");
+    RT_REQUIRE(groups > 0 && C % groups == 0, RT_ERR_ARG, "rt_group_norm: %u channels do not split into %u groups", C, groups);
+    RT_REQUIRE(eps == eps, RT_ERR_ARG, "rt_group_norm: eps is NaN");
+    const uint64_t glen = (uint64_t)(C / groups) * L;
+    RT_REQUIRE(glen <= 0x7fffffffull && (uint64_t)B * groups <= 0x7fffffffull, RT_ERR_SIZE, "rt_group_norm: group too large");
+    RT_REQUIRE(x && y, RT_ERR_NULL_POINTER, "rt_group_norm: NULL operand");
+    const size_t eb = (size_t)rt_dt_bytes(dt);
+    RT_REQUIRE(rt_aligned(x, eb) && rt_aligned(y, eb) && (!scale || rt_aligned(scale, eb)) && (!bias || rt_aligned(bias, eb)),
+               RT_ERR_ALIGN, "rt_group_norm: misaligned pointer");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    const uint32_t bg = B * groups;
+    switch (dt) {
+        case RT_F32: return launch_gn<float>(dev, x, scale, bias, y, bg, (uint32_t)glen, C / groups, groups, L, eps);
+        case RT_F16: return launch_gn<half_t>(dev, x, scale, bias, y, bg, (uint32_t)glen, C / groups, groups, L, eps);
+        default: return launch_gn<bf16_t>(dev, x, scale, bias, y, bg, (uint32_t)glen, C / groups, groups, L, eps);
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,436 @@
+// Reindex kernels: permute, slice, broadcast (one gather formulation) and concat.
+//
+// ratchet's kernels for these ops move one scalar per thread and pay three integer divisions per element
+// (ops/reindex/mod.rs:48-124, gpu/wgsl/kernel_builder.rs:198-221 in crates/ratchet-core/src).  Here the host folds the
+// op into "dst[i0,i1,i2,i3] = src[base + i0*S0 + i1*S1 + i2*S2 + i3*S3]" with strides resolved at launch, picks the
+// widest vector (16/8/4/2 bytes) that keeps every source and destination access aligned, and each thread moves whole
+// vectors along the destination's last dimension with multiply-shift index math.  A permutation that moves the
+// source's contiguous dimension goes through an LDS tile so both the read and the write side stay coalesced.
+#include "rt_internal.h"
+
+namespace {
+
+constexpr int BLOCK = 256;
+constexpr int UNROLL = 4;
+
+struct GatherArgs {
+    FastDiv d3, d2, d1;      // destination extents, d3 in vectors
+    uint64_t base;           // source offset of dst[0,0,0,0], in vectors (elements for the splat kernel)
+    uint64_t s[4];           // source strides per destination dim, in vectors (elements for the splat kernel)
+    uint32_t nvec;           // destination vectors
+};
+
+// one VecT per thread-iteration; source contiguous along the destination's last dim (s[3] == 1)
+template <typename VecT>
+__global__ void __launch_bounds__(BLOCK) gather_vec_kernel(const VecT* __restrict__ x, VecT* __restrict__ y, GatherArgs p) {
+    const uint32_t base = blockIdx.x * (BLOCK * UNROLL) + threadIdx.x;
+    VecT r[UNROLL];
+#pragma unroll
+    for (int k = 0; k < UNROLL; k++) {
+        const uint32_t v = base + k * BLOCK;
+        if (v < p.nvec) {
+            uint32_t row, i3, t, i2, i1, i0;
+            fd_divmod(v, p.d3, row, i3);
+            fd_divmod(row, p.d2, t, i2);
+            fd_divmod(t, p.d1, i0, i1);
+            r[k] = x[p.base + i0 * p.s[0] + i1 * p.s[1] + i2 * p.s[2] + i3 * p.s[3]];
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < UNROLL; k++) {
+        const uint32_t v = base + k * BLOCK;
+        if (v < p.nvec) y[v] = r[k];
+    }
+}
+
+// source broadcast along the destination's last dim (s[3] == 0): load one element, replicate it through a VecT.
+// Strides and base are in elements here; PER = elements per VecT.
+template <typename ElemT, typename VecT>
+__global__ void __launch_bounds__(BLOCK) gather_splat_kernel(const ElemT* __restrict__ x, VecT* __restrict__ y, GatherArgs p) {
+    constexpr int PER = sizeof(VecT) / sizeof(ElemT);
+    const uint32_t base = blockIdx.x * (BLOCK * UNROLL) + threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < UNROLL; k++) {
+        const uint32_t v = base + k * BLOCK;
+        if (v < p.nvec) {
+            uint32_t row, i3, t, i2, i1, i0;
+            fd_divmod(v, p.d3, row, i3);
+            fd_divmod(row, p.d2, t, i2);
+            fd_divmod(t, p.d1, i0, i1);
+            const ElemT e = x[p.base + i0 * p.s[0] + i1 * p.s[1] + i2 * p.s[2]];
+            union { VecT v; ElemT e[PER]; } u;
+#pragma unroll
+            for (int q = 0; q < PER; q++) u.e[q] = e;
+            y[v] = u.v;
+        }
+    }
+}
+
+// Tiled transpose for permutations that move the source's contiguous dimension.
+// Destination dims: `q` is the one fed by the source's last dim; 3 is fed by source dim with stride sj.
+// A block owns a TILE x TILE patch over (dst dim q, dst dim 3); the two remaining dims are flattened in blockIdx.z.
+constexpr int TILE = 64;
+struct TransposeArgs {
+    uint32_t nq, n3;         // extents of dst dim q and dst dim 3
+    uint64_t s3;             // source stride (elements) of the dim that becomes dst dim 3
+    uint64_t dq;             // destination stride (elements) of dim q
+    FastDiv gx, gy;          // tile counts along dst dim q and dst dim 3 (blockIdx.x = (z * gy + ty) * gx + tx)
+    FastDiv ob;              // extent of the second "other" dim (other dims = (oa, ob), ob fastest)
+    uint64_t sa, sb;         // source strides of the other dims
+    uint64_t da, db;         // destination strides of the other dims
+};
+
+template <typename ElemT>
+__global__ void __launch_bounds__(BLOCK) transpose_kernel(const ElemT* __restrict__ x, ElemT* __restrict__ y, TransposeArgs p) {
+    __shared__ ElemT tile[TILE][TILE + (sizeof(ElemT) == 4 ? 1 : 2)];
+    uint32_t oa, obi, bz, byx, by, bx;
+    fd_divmod(blockIdx.x, p.gx, byx, bx);
+    fd_divmod(byx, p.gy, bz, by);
+    fd_divmod(bz, p.ob, oa, obi);
+    const uint64_t src0 = oa * p.sa + obi * p.sb;
+    const uint64_t dst0 = oa * p.da + obi * p.db;
+    const uint32_t q0 = bx * TILE, j0 = by * TILE;                     // origin in (dst dim q, dst dim 3)
+    const uint32_t tx = threadIdx.x & (TILE - 1), ty = threadIdx.x / TILE;   // 64 x 4
+    // read: rows = dst-dim-3 index (source stride s3), columns = source's contiguous dim (dst dim q)
+#pragma unroll 4
+    for (uint32_t r = ty; r < TILE; r += BLOCK / TILE) {
+        const uint32_t j = j0 + r, q = q0 + tx;
+        if (j < p.n3 && q < p.nq) tile[r][tx] = x[src0 + (uint64_t)j * p.s3 + q];
+    }
+    __syncthreads();
+    // write: rows = dst dim q, columns = dst dim 3 (contiguous in the destination)
+#pragma unroll 4
+    for (uint32_t r = ty; r < TILE; r += BLOCK / TILE) {
+        const uint32_t q = q0 + r, j = j0 + tx;
+        if (q < p.nq && j < p.n3) y[dst0 + (uint64_t)q * p.dq + j] = tile[tx][r];
+    }
+}
+
+// concat: input k is [a_dim, bv[k]] vectors, copied into dst rows of dst_sv vectors at column dst_ov[k]
+struct ConcatArgs {
+    const void* src[8];
+    FastDiv bv[8];
+    uint32_t dst_ov[8];
+    uint32_t nvec[8];
+    uint32_t dst_sv;
+};
+
+template <typename VecT>
+__global__ void __launch_bounds__(BLOCK) concat_kernel(VecT* __restrict__ y, ConcatArgs p) {
+    const int k = blockIdx.y;
+    const VecT* __restrict__ x = reinterpret_cast<const VecT*>(p.src[k]);
+    const uint32_t nvec = p.nvec[k];
+    const uint32_t base = blockIdx.x * (BLOCK * UNROLL) + threadIdx.x;
+    if (blockIdx.x * (BLOCK * UNROLL) >= nvec) return;
+    VecT r[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const uint32_t v = base + u * BLOCK;
+        if (v < nvec) r[u] = x[v];
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const uint32_t v = base + u * BLOCK;
+        if (v < nvec) {
+            uint32_t row, col;
+            fd_divmod(v, p.bv[k], row, col);
+            y[(uint64_t)row * p.dst_sv + p.dst_ov[k] + col] = r[u];
+        }
+    }
+}
+
+inline unsigned blocks_for(uint64_t items, uint64_t per_block) {
+    const uint64_t b = (items + per_block - 1) / per_block;
+    return (unsigned)(b ? b : 1);
+}
+
+inline void contiguous_strides(const uint32_t shape[4], uint64_t out[4]) {
+    uint64_t s = 1;
+    for (int i = 3; i >= 0; i--) { out[i] = s; s *= shape[i]; }
+}
+
+// Launches the gather dst[i] = src[base + sum i_k * S_k] (all in elements) choosing the widest usable vector.
+int launch_gather(rt_device* dev, int eb, const void* x, void* y, const uint32_t dst_shape_in[4], const uint64_t S_in[4],
+                  uint64_t base_elems, const char* who) {
+    // Drop size-1 dims and merge neighbours that are contiguous on both sides (the destination always is): a slice of
+    // the leading dim only, or a broadcast of whole rows, becomes one long row and gets the widest vectors.
+    uint32_t dst_shape[4] = {1, 1, 1, 1};
+    uint64_t S[4] = {0, 0, 0, 0};
+    {
+        uint64_t ext[4], st[4];
+        int m = 0;
+        for (int i = 0; i < 4; i++) {
+            if (dst_shape_in[i] == 1) continue;
+            if (m > 0 && st[m - 1] == S_in[i] * dst_shape_in[i] && ext[m - 1] * dst_shape_in[i] <= 0xffffffffull &&
+                (S_in[i] != 0 || st[m - 1] == 0)) {
+                ext[m - 1] *= dst_shape_in[i];
+                st[m - 1] = S_in[i];
+            } else {
+                ext[m] = dst_shape_in[i];
+                st[m] = S_in[i];
+                m++;
+            }
+        }
+        for (int i = 0; i < m; i++) {
+            dst_shape[4 - m + i] = (uint32_t)ext[i];
+            S[4 - m + i] = st[i];
+        }
+    }
+    uint64_t n = 1;
+    for (int i = 0; i < 4; i++) n *= dst_shape[i];
+    const uint64_t row_bytes = (uint64_t)dst_shape[3] * eb;
+    const bool splat = (S[3] == 0 && dst_shape[3] > 1);
+    // widest vector width (bytes) that divides the row, the strides and the base, with both pointers aligned
+    int vb = 16;
+    for (; vb > eb; vb >>= 1) {
+        if (row_bytes % vb) continue;
+        if (!rt_aligned(y, (size_t)vb)) continue;
+        if (!splat) {
+            if (!rt_aligned(x, (size_t)vb)) continue;
+            if ((base_elems * eb) % vb) continue;
+            bool ok = true;
+            for (int i = 0; i < 3; i++)
+                if (dst_shape[i] > 1 && (S[i] * eb) % vb) ok = false;
+            if (!ok) continue;
+        }
+        break;
+    }
+    const bool contiguous_last = (S[3] == 1 || dst_shape[3] == 1);
+    if (!contiguous_last && !splat) vb = eb;      // strided last dim that is not a broadcast: scalar gather
+    const uint32_t per = (uint32_t)(vb / eb);
+    const uint64_t nvec = n / per;
+    RT_REQUIRE(nvec <= 0xffffffffull - (uint64_t)BLOCK * UNROLL, RT_ERR_SIZE, "%s: %llu vectors exceed the 32-bit index space",
+               who, (unsigned long long)nvec);
+    GatherArgs p;
+    p.d3 = make_fastdiv(dst_shape[3] / per);
+    p.d2 = make_fastdiv(dst_shape[2]);
+    p.d1 = make_fastdiv(dst_shape[1]);
+    p.nvec = (uint32_t)nvec;
+    const unsigned blocks = blocks_for(nvec, BLOCK * UNROLL);
+    if (splat) {
+        p.base = base_elems;
+        for (int i = 0; i < 4; i++) p.s[i] = S[i];
+#define RT_SPLAT(ET, VT) \
+    hipLaunchKernelGGL((gather_splat_kernel<ET, VT>), dim3(blocks), dim3(BLOCK), 0, dev->stream, (const ET*)x, (VT*)y, p)
+        if (eb == 4) {
+            if (vb == 16) RT_SPLAT(uint32_t, uint4);
+            else if (vb == 8) RT_SPLAT(uint32_t, uint2);
+            else RT_SPLAT(uint32_t, uint32_t);
+        } else {
+            if (vb == 16) RT_SPLAT(uint16_t, uint4);
+            else if (vb == 8) RT_SPLAT(uint16_t, uint2);
+            else if (vb == 4) RT_SPLAT(uint16_t, uint32_t);
+            else RT_SPLAT(uint16_t, uint16_t);
+        }
+#undef RT_SPLAT
+    } else {
+        // convert to vector units; with per == 1 a strided last dim keeps its element stride
+        p.base = base_elems / per;
+        for (int i = 0; i < 3; i++) p.s[i] = (dst_shape[i] > 1) ? S[i] / per : 0;
+        p.s[3] = (per > 1 || dst_shape[3] == 1) ? (dst_shape[3] == 1 ? 0 : 1) : S[3];
+#define RT_GATHER(VT) hipLaunchKernelGGL((gather_vec_kernel<VT>), dim3(blocks), dim3(BLOCK), 0, dev->stream, (const VT*)x, (VT*)y, p)
+        if (vb == 16) RT_GATHER(uint4);
+        else if (vb == 8) RT_GATHER(uint2);
+        else if (vb == 4) RT_GATHER(uint32_t);
+        else RT_GATHER(uint16_t);
+#undef RT_GATHER
+    }
+    RT_CHECK_LAUNCH(who);
+    return RT_OK;
+}
+
+int validate_common(int elem_bytes, const void* x, const void* y, const char* who) {
+    RT_REQUIRE(elem_bytes == 2 || elem_bytes == 4, RT_ERR_ARG, "%s: elem_bytes must be 2 or 4, got %d", who, elem_bytes);
+    RT_REQUIRE(x && y, RT_ERR_NULL_POINTER, "%s: NULL operand", who);
+    RT_REQUIRE(rt_aligned(x, (size_t)elem_bytes) && rt_aligned(y, (size_t)elem_bytes), RT_ERR_ALIGN, "%s: misaligned pointer", who);
+    return RT_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uint32_t src_shape[4], const uint32_t perm[4]) {
+    RT_REQUIRE(src_shape && perm, RT_ERR_NULL_POINTER, "rt_permute: NULL shape or perm");
+    bool seen[4] = {false, false, false, false};
+    for (int i = 0; i < 4; i++) {
+        RT_REQUIRE(perm[i] < 4 && !seen[perm[i]], RT_ERR_PERM, "rt_permute: [%u,%u,%u,%u] is not a permutation of 0..3", perm[0],
+                   perm[1], perm[2], perm[3]);
+        seen[perm[i]] = true;
+    }
+    uint64_t n = 1;
+    for (int i = 0; i < 4; i++) {
+        RT_REQUIRE(src_shape[i] > 0, RT_ERR_SHAPE, "rt_permute: zero extent in dim %d", i);
+        n *= src_shape[i];
+    }
+    RT_REQUIRE(n <= RT_MAX_NUMEL, RT_ERR_SIZE, "rt_permute: tensor too large");
+    int rc = validate_common(elem_bytes, x, y, "rt_permute");
+    if (rc) return rc;
+    rc = rt_enter(dev);
+    if (rc) return rc;
+
+    uint64_t src_strides[4], S[4];
+    uint32_t dst_shape[4];
+    contiguous_strides(src_shape, src_strides);
+    for (int i = 0; i < 4; i++) {
+        dst_shape[i] = src_shape[perm[i]];           // permute.rs:53-56
+        S[i] = src_strides[perm[i]];
+    }
+    // Does the source's contiguous run survive?  Drop size-1 dims from the question: they carry no data movement.
+    if (S[3] == 1 || dst_shape[3] == 1) return launch_gather(dev, elem_bytes, x, y, dst_shape, S, 0, "rt_permute");
+
+    // find the dst dim fed by the source's innermost non-trivial dim
+    int q = -1;
+    for (int i = 0; i < 3; i++)
+        if (S[i] == 1 && dst_shape[i] > 1) q = i;
+    if (q < 0) {
+        // the source's last dim has extent 1, so "contiguous" is carried by a dim with stride > 1 everywhere: plain
+        // strided gather is as good as it gets
+        return launch_gather(dev, elem_bytes, x, y, dst_shape, S, 0, "rt_permute");
+    }
+    uint64_t dst_strides[4];
+    contiguous_strides(dst_shape, dst_strides);
+    int others[2], no = 0;
+    for (int i = 0; i < 3; i++)
+        if (i != q) others[no++] = i;
+    TransposeArgs p;
+    p.nq = dst_shape[q];
+    p.n3 = dst_shape[3];
+    p.s3 = S[3];
+    p.dq = dst_strides[q];
+    p.ob = make_fastdiv(dst_shape[others[1]]);
+    p.sa = S[others[0]];
+    p.sb = S[others[1]];
+    p.da = dst_strides[others[0]];
+    p.db = dst_strides[others[1]];
+    const uint64_t gz = (uint64_t)dst_shape[others[0]] * dst_shape[others[1]];
+    const uint64_t gx = (p.nq + TILE - 1) / TILE, gy = (p.n3 + TILE - 1) / TILE;
+    const uint64_t blocks = gx * gy * gz;
+    RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_permute: %llu tiles exceed the grid limit", (unsigned long long)blocks);
+    p.gx = make_fastdiv((uint32_t)gx);
+    p.gy = make_fastdiv((uint32_t)gy);
+    if (elem_bytes == 4) {
+        hipLaunchKernelGGL((transpose_kernel<uint32_t>), dim3((unsigned)blocks), dim3(BLOCK), 0, dev->stream, (const uint32_t*)x,
+                           (uint32_t*)y, p);
+    } else {
+        hipLaunchKernelGGL((transpose_kernel<uint16_t>), dim3((unsigned)blocks), dim3(BLOCK), 0, dev->stream, (const uint16_t*)x,
+                           (uint16_t*)y, p);
+    }
+    RT_CHECK_LAUNCH("transpose_kernel");
+    return RT_OK;
+}
+
+int rt_slice(rt_device* dev, int elem_bytes, const void* x, void* y, const uint32_t src_shape[4], const uint32_t start[4],
+             const uint32_t dst_shape[4]) {
+    RT_REQUIRE(src_shape && start && dst_shape, RT_ERR_NULL_POINTER, "rt_slice: NULL shape");
+    uint64_t n = 1;
+    for (int i = 0; i < 4; i++) {
+        // slice.rs:38-51 asserts start <= end <= dim; the CPU path additionally asserts start < end (cpu/reindex.rs:103-105)
+        RT_REQUIRE(dst_shape[i] > 0 && src_shape[i] > 0, RT_ERR_SHAPE, "rt_slice: empty range in dim %d", i);
+        RT_REQUIRE((uint64_t)start[i] + dst_shape[i] <= src_shape[i], RT_ERR_SHAPE, "rt_slice: dim %d: %u + %u exceeds %u", i,
+                   start[i], dst_shape[i], src_shape[i]);
+        n *= src_shape[i];
+    }
+    RT_REQUIRE(n <= RT_MAX_NUMEL, RT_ERR_SIZE, "rt_slice: tensor too large");
+    int rc = validate_common(elem_bytes, x, y, "rt_slice");
+    if (rc) return rc;
+    rc = rt_enter(dev);
+    if (rc) return rc;
+    uint64_t S[4], base = 0;
+    contiguous_strides(src_shape, S);
+    for (int i = 0; i < 4; i++) base += (uint64_t)start[i] * S[i];
+    return launch_gather(dev, elem_bytes, x, y, dst_shape, S, base, "rt_slice");
+}
+
+int rt_broadcast(rt_device* dev, int elem_bytes, const void* x, void* y, const uint32_t src_shape[4], const uint32_t dst_shape[4]) {
+    RT_REQUIRE(src_shape && dst_shape, RT_ERR_NULL_POINTER, "rt_broadcast: NULL shape");
+    uint64_t n = 1;
+    for (int i = 0; i < 4; i++) {
+        RT_REQUIRE(src_shape[i] > 0 && dst_shape[i] > 0, RT_ERR_SHAPE, "rt_broadcast: zero extent in dim %d", i);
+        // Broadcast::check_shapes (broadcast.rs:31-58)
+        RT_REQUIRE(src_shape[i] == 1 || src_shape[i] == dst_shape[i], RT_ERR_SHAPE,
+                   "rt_broadcast: source dimension %u cannot be broadcast to %u", src_shape[i], dst_shape[i]);
+        n *= dst_shape[i];
+    }
+    RT_REQUIRE(n <= RT_MAX_NUMEL, RT_ERR_SIZE, "rt_broadcast: tensor too large");
+    int rc = validate_common(elem_bytes, x, y, "rt_broadcast");
+    if (rc) return rc;
+    rc = rt_enter(dev);
+    if (rc) return rc;
+    uint64_t S[4];
+    contiguous_strides(src_shape, S);
+    for (int i = 0; i < 4; i++)
+        if (src_shape[i] == 1) S[i] = 0;
+    return launch_gather(dev, elem_bytes, x, y, dst_shape, S, 0, "rt_broadcast");
+}
+
+int rt_concat(rt_device* dev, int elem_bytes, int n_inputs, const void* const* xs, const uint32_t (*shapes)[4], int dim, void* y) {
+    RT_REQUIRE(elem_bytes == 2 || elem_bytes == 4, RT_ERR_ARG, "rt_concat: elem_bytes must be 2 or 4, got %d", elem_bytes);
+    // Concat::check_shapes (concat.rs:131-152)
+    RT_REQUIRE(n_inputs >= 2 && n_inputs <= 8, RT_ERR_ARG, "rt_concat: %d inputs (2..8 supported)", n_inputs);
+    RT_REQUIRE(dim >= 0 && dim < 4, RT_ERR_ARG, "rt_concat: dim %d out of range", dim);
+    RT_REQUIRE(xs && shapes && y, RT_ERR_NULL_POINTER, "rt_concat: NULL argument");
+    uint64_t a_dim = 1, block = 1, dst_dim = 0;
+    for (int k = 0; k < n_inputs; k++) {
+        RT_REQUIRE(xs[k], RT_ERR_NULL_POINTER, "rt_concat: input %d is NULL", k);
+        RT_REQUIRE(rt_aligned(xs[k], (size_t)elem_bytes), RT_ERR_ALIGN, "rt_concat: input %d misaligned", k);
+        for (int a = 0; a < 4; a++) {
+            RT_REQUIRE(shapes[k][a] > 0, RT_ERR_SHAPE, "rt_concat: input %d has a zero extent", k);
+            if (a != dim)
+                RT_REQUIRE(shapes[k][a] == shapes[0][a], RT_ERR_SHAPE, "rt_concat: input %d differs from input 0 in dim %d", k, a);
+        }
+        dst_dim += shapes[k][dim];
+    }
+    RT_REQUIRE(rt_aligned(y, (size_t)elem_bytes), RT_ERR_ALIGN, "rt_concat: output misaligned");
+    for (int a = 0; a < dim; a++) a_dim *= shapes[0][a];
+    for (int a = dim + 1; a < 4; a++) block *= shapes[0][a];
+    const uint64_t dst_s = block * dst_dim;
+    RT_REQUIRE(a_dim * dst_s <= RT_MAX_NUMEL, RT_ERR_SIZE, "rt_concat: output too large");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+
+    // widest vector that divides every segment length, every column offset and the destination row
+    int vb = 16;
+    for (; vb > elem_bytes; vb >>= 1) {
+        bool ok = rt_aligned(y, (size_t)vb) && (dst_s * elem_bytes) % vb == 0;
+        uint64_t off = 0;
+        for (int k = 0; k < n_inputs && ok; k++) {
+            const uint64_t b_dim = block * shapes[k][dim];
+            ok = rt_aligned(xs[k], (size_t)vb) && (b_dim * elem_bytes) % vb == 0 && (off * elem_bytes) % vb == 0;
+            off += b_dim;
+        }
+        if (ok) break;
+    }
+    const uint64_t per = (uint64_t)vb / elem_bytes;
+    ConcatArgs p;
+    uint64_t off = 0, max_nvec = 0;
+    RT_REQUIRE(dst_s / per <= 0xffffffffull, RT_ERR_SIZE, "rt_concat: destination row too long");
+    p.dst_sv = (uint32_t)(dst_s / per);
+    for (int k = 0; k < 8; k++) {
+        if (k < n_inputs) {
+            const uint64_t b_dim = block * shapes[k][dim];
+            const uint64_t nvec = a_dim * b_dim / per;
+            RT_REQUIRE(nvec <= 0xffffffffull - (uint64_t)BLOCK * UNROLL, RT_ERR_SIZE, "rt_concat: input %d too large", k);
+            p.src[k] = xs[k];
+            p.bv[k] = make_fastdiv((uint32_t)(b_dim / per));
+            p.dst_ov[k] = (uint32_t)(off / per);
+            p.nvec[k] = (uint32_t)nvec;
+            if (nvec > max_nvec) max_nvec = nvec;
+            off += b_dim;
+        } else {
+            p.src[k] = nullptr;
+            p.bv[k] = make_fastdiv(1);
+            p.dst_ov[k] = 0;
+            p.nvec[k] = 0;
+        }
+    }
+    const dim3 grid(blocks_for(max_nvec, BLOCK * UNROLL), (unsigned)n_inputs);
+    if (vb == 16) hipLaunchKernelGGL((concat_kernel<uint4>), grid, dim3(BLOCK), 0, dev->stream, (uint4*)y, p);
+    else if (vb == 8) hipLaunchKernelGGL((concat_kernel<uint2>), grid, dim3(BLOCK), 0, dev->stream, (uint2*)y, p);
+    else if (vb == 4) hipLaunchKernelGGL((concat_kernel<uint32_t>), grid, dim3(BLOCK), 0, dev->stream, (uint32_t*)y, p);
+    else hipLaunchKernelGGL((concat_kernel<uint16_t>), grid, dim3(BLOCK), 0, dev->stream, (uint16_t*)y, p);
+    RT_CHECK_LAUNCH("concat_kernel");
+    return RT_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,234 @@
+"""Thin object layer over the C ABI: Device (one HIP stream), Buffer (hipMalloc'd storage), op launchers.
+
+This mirrors the storage/dispatch seam of ratchet-core that the native library replaces:
+  Device  ~ WgpuDevice          (crates/ratchet-core/src/gpu/device.rs:18-30)
+  Buffer  ~ GPUBuffer           (crates/ratchet-core/src/storage/gpu_buffer.rs:20-27): ref-counted by Python, freed on drop
+  op methods ~ one CompiledOp dispatch each (crates/ratchet-core/src/executable.rs:33-59)
+Every method enqueues on the device's single stream; Device.sync() / Buffer.to_numpy() block.
+"""
+import ctypes
+
+import numpy as np
+
+from . import _lib
+from ._lib import RatchetError, check, shape4  # noqa: F401
+
+_NP_TO_DT = {np.dtype(np.float32): _lib.F32, np.dtype(np.float16): _lib.F16, np.dtype(np.int32): _lib.I32,
+             np.dtype(np.uint32): _lib.U32}
+_DT_BYTES = {_lib.F32: 4, _lib.F16: 2, _lib.BF16: 2, _lib.I32: 4, _lib.U32: 4}
+_DT_TO_NP = {_lib.F32: np.float32, _lib.F16: np.float16, _lib.BF16: np.uint16, _lib.I32: np.int32, _lib.U32: np.uint32}
+
+
+def dtype_code(np_dtype, bf16=False):
+    if bf16:
+        return _lib.BF16
+    return _NP_TO_DT[np.dtype(np_dtype)]
+
+
+class Buffer:
+    """A device allocation with a dtype code and a shape; owns its memory."""
+
+    def __init__(self, device, shape, dt):
+        self.device = device
+        self.shape = tuple(int(s) for s in shape)
+        self.dt = dt
+        self.numel = int(np.prod(self.shape, dtype=np.int64)) if self.shape else 1
+        self.nbytes = self.numel * _DT_BYTES[dt]
+        p = ctypes.c_void_p()
+        check(device.lib.rt_malloc(device.handle, self.nbytes, ctypes.byref(p)))
+        self.ptr = p
+
+    def __del__(self):
+        try:
+            if getattr(self, "ptr", None) is not None and self.device.handle is not None:
+                self.device.lib.rt_free(self.device.handle, self.ptr)
+                self.ptr = None
+        except Exception:
+            pass
+
+    def to_numpy(self):
+        out = np.empty(self.shape, dtype=_DT_TO_NP[self.dt])
+        check(self.device.lib.rt_d2h(self.device.handle, out.ctypes.data_as(ctypes.c_void_p), self.ptr, self.nbytes))
+        return out
+
+    def view(self, offset, shape):
+        return BufferView(self, offset, shape)
+
+    def reshape(self, shape):
+        return BufferView(self, 0, shape)
+
+    def zero_(self):
+        check(self.device.lib.rt_memset0(self.device.handle, self.ptr, self.nbytes))
+        return self
+
+
+class BufferView:
+    """A window into a Buffer starting `offset` elements in (keeps the parent alive); used for offset / misaligned operands."""
+
+    def __init__(self, parent, offset, shape):
+        self.device = parent.device
+        self.parent = parent
+        self.dt = parent.dt
+        self.shape = tuple(int(s) for s in shape)
+        self.numel = int(np.prod(self.shape, dtype=np.int64)) if self.shape else 1
+        self.nbytes = self.numel * _DT_BYTES[self.dt]
+        assert (offset + self.numel) <= parent.numel
+        self.ptr = ctypes.c_void_p(parent.ptr.value + offset * _DT_BYTES[self.dt])
+
+    def to_numpy(self):
+        out = np.empty(self.shape, dtype=_DT_TO_NP[self.dt])
+        check(self.device.lib.rt_d2h(self.device.handle, out.ctypes.data_as(ctypes.c_void_p), self.ptr, self.nbytes))
+        return out
+
+    def upload(self, array):
+        a = np.ascontiguousarray(array)
+        assert a.nbytes == self.nbytes
+        check(self.device.lib.rt_h2d(self.device.handle, self.ptr, a.ctypes.data_as(ctypes.c_void_p), a.nbytes))
+        return self
+
+
+class Event:
+    def __init__(self, device):
+        self.device = device
+        p = ctypes.c_void_p()
+        check(device.lib.rt_event_create(device.handle, ctypes.byref(p)))
+        self.ptr = p
+
+    def record(self):
+        check(self.device.lib.rt_event_record(self.device.handle, self.ptr))
+        return self
+
+    def elapsed_ms(self, stop):
+        ms = ctypes.c_float()
+        check(self.device.lib.rt_event_elapsed_ms(self.ptr, stop.ptr, ctypes.byref(ms)))
+        return float(ms.value)
+
+    def __del__(self):
+        try:
+            if getattr(self, "ptr", None) is not None:
+                self.device.lib.rt_event_destroy(self.ptr)
+                self.ptr = None
+        except Exception:
+            pass
+
+
+class Device:
+    def __init__(self, ordinal=0):
+        self.lib = _lib.load()
+        self.handle = None
+        h = ctypes.c_void_p()
+        check(self.lib.rt_device_create(ordinal, ctypes.byref(h)))
+        self.handle = h
+        self.ordinal = ordinal
+
+    @staticmethod
+    def count():
+        n = ctypes.c_int()
+        lib = _lib.load()
+        status = lib.rt_device_count(ctypes.byref(n))
+        return n.value if status == 0 else 0
+
+    def close(self):
+        if self.handle is not None:
+            self.lib.rt_device_destroy(self.handle)
+            self.handle = None
+
+    def sync(self):
+        check(self.lib.rt_sync(self.handle))
+
+    # ---- storage
+    def empty(self, shape, dt):
+        return Buffer(self, shape, dt)
+
+    def upload(self, array, bf16=False):
+        a = np.ascontiguousarray(array)
+        buf = Buffer(self, a.shape, dtype_code(a.dtype, bf16))
+        check(self.lib.rt_h2d(self.handle, buf.ptr, a.ctypes.data_as(ctypes.c_void_p), a.nbytes))
+        return buf
+
+    def event(self):
+        return Event(self)
+
+    # ---- ops (out may alias the first input where the C ABI allows it)
+    def binary(self, op, a, b, out=None):
+        op = _lib.BINARY_OPS.index(op) if isinstance(op, str) else op
+        if a.shape == b.shape:
+            out = out or Buffer(self, a.shape, a.dt)
+            check(self.lib.rt_binary(self.handle, op, a.dt, a.ptr, b.ptr, out.ptr, a.numel))
+            return out
+        shape = tuple(np.broadcast_shapes(a.shape, b.shape))
+        out = out or Buffer(self, shape, a.dt)
+        check(self.lib.rt_binary_bcast(self.handle, op, a.dt, a.ptr, shape4(a.shape), b.ptr, shape4(b.shape), out.ptr,
+                                       shape4(shape)))
+        return out
+
+    def unary(self, op, x, out=None):
+        op = _lib.UNARY_OPS.index(op) if isinstance(op, str) else op
+        out = out or Buffer(self, x.shape, x.dt)
+        check(self.lib.rt_unary(self.handle, op, x.dt, x.ptr, out.ptr, x.numel))
+        return out
+
+    def cast(self, x, dst_dt, out=None):
+        out = out or Buffer(self, x.shape, dst_dt)
+        check(self.lib.rt_cast(self.handle, x.dt, dst_dt, x.ptr, out.ptr, x.numel))
+        return out
+
+    def permute(self, x, dims, out=None):
+        dims = [int(d) for d in dims]
+        pad = 4 - len(dims)
+        perm = (ctypes.c_uint32 * 4)(*(list(range(pad)) + [d + pad for d in dims]))   # Permute::promote
+        out_shape = [x.shape[d] for d in dims]
+        out = out or Buffer(self, out_shape, x.dt)
+        check(self.lib.rt_permute(self.handle, _DT_BYTES[x.dt], x.ptr, out.ptr, shape4(x.shape), perm))
+        return out
+
+    def slice(self, x, ranges, out=None):
+        start = [int(r[0]) for r in ranges]
+        dst = [int(r[1]) - int(r[0]) for r in ranges]
+        out = out or Buffer(self, dst, x.dt)
+        pad = 4 - len(start)
+        check(self.lib.rt_slice(self.handle, _DT_BYTES[x.dt], x.ptr, out.ptr, shape4(x.shape),
+                                (ctypes.c_uint32 * 4)(*([0] * pad + start)), shape4(dst)))
+        return out
+
+    def broadcast_to(self, x, shape, out=None):
+        out = out or Buffer(self, shape, x.dt)
+        check(self.lib.rt_broadcast(self.handle, _DT_BYTES[x.dt], x.ptr, out.ptr, shape4(x.shape), shape4(shape)))
+        return out
+
+    def concat(self, xs, dim, out=None):
+        rank = len(xs[0].shape)
+        out_shape = list(xs[0].shape)
+        out_shape[dim] = sum(x.shape[dim] for x in xs)
+        out = out or Buffer(self, out_shape, xs[0].dt)
+        ptrs = (ctypes.c_void_p * len(xs))(*[x.ptr.value for x in xs])
+        shapes = ((ctypes.c_uint32 * 4) * len(xs))(*[shape4(x.shape) for x in xs])
+        check(self.lib.rt_concat(self.handle, _DT_BYTES[xs[0].dt], len(xs), ptrs, shapes, dim + (4 - rank), out.ptr))
+        return out
+
+    def softmax(self, x, out=None, mode=_lib.SOFTMAX_REFERENCE):
+        cols = x.shape[-1]
+        out = out or Buffer(self, x.shape, x.dt)
+        check(self.lib.rt_softmax(self.handle, x.dt, x.ptr, out.ptr, x.numel // cols, cols, mode))
+        return out
+
+    def layer_norm(self, x, scale, bias, eps=1e-5, out=None):
+        cols = x.shape[-1]
+        out = out or Buffer(self, x.shape, x.dt)
+        check(self.lib.rt_layer_norm(self.handle, x.dt, x.ptr, scale.ptr, bias.ptr if bias is not None else None, out.ptr,
+                                     x.numel // cols, cols, eps))
+        return out
+
+    def rms_norm(self, x, scale, eps=1e-5, out=None):
+        cols = x.shape[-1]
+        out = out or Buffer(self, x.shape, x.dt)
+        check(self.lib.rt_rms_norm(self.handle, x.dt, x.ptr, scale.ptr, out.ptr, x.numel // cols, cols, eps))
+        return out
+
+    def group_norm(self, x, groups, scale, bias, eps=1e-5, out=None):
+        B, C = x.shape[0], x.shape[1]
+        L = x.numel // (B * C)
+        out = out or Buffer(self, x.shape, x.dt)
+        check(self.lib.rt_group_norm(self.handle, x.dt, x.ptr, scale.ptr if scale is not None else None,
+                                     bias.ptr if bias is not None else None, out.ptr, B, C, L, groups, eps))
+        return out

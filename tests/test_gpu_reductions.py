@@ -1,0 +1,187 @@
+"""GPU parity: softmax, layer_norm, rms_norm, group_norm against the CPU oracle, through the C ABI.
+
+Bars: f32 <= 1e-5, f16 <= 1e-3 with the reference's all_close rule (|a-b| <= tol + tol*|b|, NaN == NaN).
+f16 softmax replays the reference's sequential f16 accumulation and is expected to be bit-exact.
+Problem spaces follow crates/ratchet-core/src/ops/softmax.rs:308-365 and ops/norm/mod.rs:400-512.
+"""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from gpu_util import mismatch_count, randn, same_bits
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    from ratchet_amd import Device
+
+    d = Device(0)
+    yield d
+    d.close()
+
+
+SOFTMAX_SHAPES = [(3, 256, 256), (1, 7, 33), (2, 1, 1), (1, 5, 255), (2, 64, 1500), (1, 3, 2048), (1, 2, 2052), (1, 130, 8),
+                  (1, 3, 5000)]
+
+
+@pytest.mark.parametrize("shape", SOFTMAX_SHAPES)
+def test_softmax_f32(dev, oracle, shape):
+    rng = np.random.default_rng(300)
+    x = randn(rng, shape, np.float32, 3.0)
+    want = oracle.softmax(x)
+    got = dev.softmax(dev.upload(x)).to_numpy()
+    bad, mx = oracle.count_not_close(got, want, 1e-5, 1e-5)
+    assert bad == 0, (shape, bad, mx)
+    ref = F.softmax(torch.from_numpy(x), dim=-1).numpy()               # the reference test's own referee and tolerance
+    bad, mx = oracle.count_not_close(got, ref, 1e-6, 1e-6)
+    assert bad == 0, (shape, bad, mx)
+
+
+def test_softmax_f32_masks_overflow_in_place(dev, oracle):
+    ninf = -np.inf
+    x = np.zeros((4, 64), np.float32)
+    x[0, 1:] = ninf
+    x[1, 2:] = ninf
+    x[1, :2] = 1.0
+    x[2, 0] = 100.0                                                    # exp overflows: NaN there, 0 elsewhere
+    x[3, :] = ninf                                                     # fully masked row: 0/0
+    want = oracle.softmax(x)
+    dx = dev.upload(x)
+    dev.softmax(dx, out=dx)
+    got = dx.to_numpy()
+    assert same_bits(got, want)
+    assert np.isnan(got[2, 0]) and np.all(got[2, 1:] == 0) and np.all(np.isnan(got[3]))
+
+
+@pytest.mark.parametrize("shape", [(3, 64, 256), (1, 7, 33), (2, 1, 1), (1, 70, 1000), (1, 65, 4096), (1, 3, 4100), (1, 129, 8)])
+def test_softmax_f16_reference_sequence(dev, oracle, shape):
+    rng = np.random.default_rng(301)
+    x = randn(rng, shape, np.float16, 2.0)
+    if shape[-1] >= 256:                                                # causal-style -inf tail and one overflow row
+        x[0, 0, shape[-1] // 2:] = -np.inf
+        x[0, 1, 5] = 12.0
+    want = oracle.softmax(x)
+    got = dev.softmax(dev.upload(x)).to_numpy()
+    bad, mx = oracle.count_not_close(got, want, 1e-3, 1e-3)
+    assert bad == 0, (shape, bad, mx)
+    assert mismatch_count(got, want) == 0, (shape, mismatch_count(got, want))
+
+
+def test_softmax_f16_order_dependence_is_reproduced(dev, oracle):
+    # 2048 + 1 + 1 + ... never grows in f16: the kernel must reproduce that, not the mathematically exact sum
+    row = np.zeros(512, np.float16)
+    row[0] = np.float16(np.log(2048.0))
+    x = np.stack([row, row[::-1]])
+    want = oracle.softmax(x)
+    got = dev.softmax(dev.upload(x)).to_numpy()
+    assert same_bits(got, want)
+    assert got[0, 1] != got[1, 0]
+
+
+def test_softmax_bf16_and_stable_mode(dev, oracle):
+    from ratchet_amd import _lib
+
+    rng = np.random.default_rng(302)
+    xb = oracle.cast((rng.standard_normal((2, 9, 320)) * 2).astype(np.float32), np.uint16, dst_bf16=True)
+    got = dev.softmax(dev.upload(xb, bf16=True)).to_numpy()
+    assert np.array_equal(got, oracle.softmax(xb, bf16=True))
+    # stable mode: max-subtracted, f32 accumulation; compare with torch in f32
+    for dtype, tol in ((np.float32, 1e-6), (np.float16, 1e-3)):
+        x = randn(rng, (2, 33, 1000), dtype, 3.0)
+        x[0, 0, 0] = 30000.0 if dtype == np.float16 else 1000.0         # would overflow without max subtraction
+        got = dev.softmax(dev.upload(x), mode=_lib.SOFTMAX_STABLE).to_numpy()
+        ref = F.softmax(torch.from_numpy(x.astype(np.float32)), dim=-1).numpy().astype(dtype)
+        bad, mx = oracle.count_not_close(got, ref, tol, tol)
+        assert bad == 0, (dtype, bad, mx)
+
+
+NORM_SHAPES = [(3, 256, 256), (2, 57, 1001), (1, 1, 1), (1, 13, 7), (1, 150, 384), (2, 9, 2048), (1, 5, 2052), (1, 3, 6000)]
+
+
+@pytest.mark.parametrize("shape", NORM_SHAPES)
+def test_layer_norm_f32(dev, oracle, shape):
+    rng = np.random.default_rng(310)
+    n = shape[-1]
+    x = randn(rng, shape, np.float32)
+    w = randn(rng, n, np.float32)
+    b = randn(rng, n, np.float32)
+    for bias in (b, None):
+        want = oracle.layer_norm(x, w, bias, 1e-5, intended=True)
+        got = dev.layer_norm(dev.upload(x), dev.upload(w), dev.upload(bias) if bias is not None else None, 1e-5).to_numpy()
+        bad, mx = oracle.count_not_close(got, want, 1e-5, 1e-5)
+        if n == 1:
+            assert same_bits(got, want)
+        else:
+            assert bad == 0, (shape, bias is None, bad, mx)
+    if n > 1:
+        ref = F.layer_norm(torch.from_numpy(x), (n,), torch.from_numpy(w), torch.from_numpy(b), eps=1e-5).numpy()
+        got = dev.layer_norm(dev.upload(x), dev.upload(w), dev.upload(b), 1e-5).to_numpy()
+        bad, mx = oracle.count_not_close(got, ref, 1e-4, 1e-4)          # the reference test's tolerance
+        assert bad == 0, (shape, bad, mx)
+
+
+@pytest.mark.parametrize("shape", NORM_SHAPES)
+def test_rms_norm_f32(dev, oracle, shape):
+    rng = np.random.default_rng(311)
+    n = shape[-1]
+    x = randn(rng, shape, np.float32)
+    w = randn(rng, n, np.float32)
+    want = oracle.rms_norm(x, w, 1e-5, intended=True)
+    got = dev.rms_norm(dev.upload(x), dev.upload(w), 1e-5).to_numpy()
+    bad, mx = oracle.count_not_close(got, want, 1e-5, 1e-5)
+    assert bad == 0, (shape, bad, mx)
+
+
+@pytest.mark.parametrize("shape", [(2, 64, 2560), (1, 33, 3072), (1, 9, 384), (1, 7, 100), (1, 3, 4104), (16, 128, 256), (1, 5, 1)])
+def test_norms_f16(dev, oracle, shape):
+    rng = np.random.default_rng(312)
+    n = shape[-1]
+    x = randn(rng, shape, np.float16)
+    w = (1 + 0.02 * rng.standard_normal(n)).astype(np.float16)
+    b = (0.02 * rng.standard_normal(n)).astype(np.float16)
+    want = oracle.layer_norm(x, w, b, 1e-5, intended=True)
+    got = dev.layer_norm(dev.upload(x), dev.upload(w), dev.upload(b), 1e-5).to_numpy()
+    bad, mx = oracle.count_not_close(got, want, 1e-3, 1e-3)
+    assert bad == 0, ("layer", shape, bad, mx)
+    # the rounding sequence and the f32 accumulation order are replayed exactly
+    assert mismatch_count(got, want) == 0, mismatch_count(got, want)
+    want = oracle.rms_norm(x, w, 1e-5, intended=True)
+    got = dev.rms_norm(dev.upload(x), dev.upload(w), 1e-5).to_numpy()
+    bad, mx = oracle.count_not_close(got, want, 1e-3, 1e-3)
+    assert bad == 0, ("rms", shape, bad, mx)
+    assert mismatch_count(got, want) == 0, mismatch_count(got, want)
+
+
+def test_layer_norm_variance_form_matches_reference(dev, oracle):
+    # E[x^2] - mu^2 loses digits with a large common offset; the kernel must lose them the same way (not use two passes)
+    rng = np.random.default_rng(313)
+    x = (rng.standard_normal((8, 256)) * 0.5 + 30).astype(np.float32)
+    w = np.ones(256, np.float32)
+    want = oracle.layer_norm(x, w, None, 1e-5, intended=True)
+    got = dev.layer_norm(dev.upload(x), dev.upload(w), None, 1e-5).to_numpy()
+    two_pass = F.layer_norm(torch.from_numpy(x), (256,), eps=1e-5).numpy()
+    assert np.nanmax(np.abs(got - want)) < np.nanmax(np.abs(two_pass - want)) or np.allclose(two_pass, want, atol=1e-4)
+
+
+@pytest.mark.parametrize("B,C,L,G", [(1, 3, 1, 1), (2, 8, 5, 4), (1, 6, 7, 6), (3, 4, 9, 1), (1, 64, 3000, 32), (2, 32, 17, 8)])
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_group_norm(dev, oracle, B, C, L, G, dtype):
+    rng = np.random.default_rng(320)
+    x = randn(rng, (B, C, L), dtype)
+    w = randn(rng, C, dtype)
+    b = randn(rng, C, dtype)
+    tol = 1e-5 if dtype == np.float32 else 1e-3
+    want = oracle.group_norm(x, G, w, b, 1e-5)
+    got = dev.group_norm(dev.upload(x), G, dev.upload(w), dev.upload(b), 1e-5).to_numpy()
+    bad, mx = oracle.count_not_close(got, want, tol, tol)
+    assert bad == 0, (bad, mx)
+    ref = F.group_norm(torch.from_numpy(x.astype(np.float32)), G, torch.from_numpy(w.astype(np.float32)),
+                       torch.from_numpy(b.astype(np.float32)), eps=1e-5).numpy().astype(dtype)
+    bad, mx = oracle.count_not_close(got, ref, max(tol, 1e-4), max(tol, 1e-4))      # the reference test's tolerance
+    assert bad == 0, (bad, mx)
+    got = dev.group_norm(dev.upload(x), G, None, None, 1e-5).to_numpy()
+    bad, mx = oracle.count_not_close(got, oracle.group_norm(x, G, None, None, 1e-5), tol, tol)
+    assert bad == 0, (bad, mx)

@@ -1,0 +1,145 @@
+"""GPU parity: permute / slice / broadcast_to / concat against the CPU oracle (bit-exact), through the C ABI.
+
+Problem spaces follow the reference's own tests (crates/ratchet-core/src/ops/reindex/{permute,slice,broadcast}.rs,
+ops/concat.rs) plus the BASELINE shapes and alignment / odd-size edge cases.
+"""
+import itertools
+
+import numpy as np
+import pytest
+
+from gpu_util import randn
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    from ratchet_amd import Device
+
+    d = Device(0)
+    yield d
+    d.close()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_permute_all_orders(dev, oracle, dtype):
+    rng = np.random.default_rng(200)
+    for shape in [(2, 3, 5, 7), (1, 4, 66, 130), (2, 1, 8, 64), (3, 5, 1, 16)]:
+        x = randn(rng, shape, dtype)
+        dx = dev.upload(x)
+        for perm in itertools.permutations(range(4)):
+            want = oracle.permute(x, perm)
+            got = dev.permute(dx, perm).to_numpy()
+            assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (shape, perm)
+
+
+def test_permute_lower_rank_and_baseline_shapes(dev, oracle):
+    rng = np.random.default_rng(201)
+    x3 = randn(rng, (4, 100, 80), np.float16)
+    for perm in itertools.permutations(range(3)):
+        assert np.array_equal(dev.permute(dev.upload(x3), perm).to_numpy(), oracle.permute(x3, perm)), perm
+    x2 = randn(rng, (257, 129), np.float32)
+    assert np.array_equal(dev.permute(dev.upload(x2), (1, 0)).to_numpy(), x2.T)
+    q = randn(rng, (1, 1500, 6, 64), np.float32)                       # Whisper-tiny heads
+    p = dev.permute(dev.upload(q), (0, 2, 1, 3))
+    assert np.array_equal(p.to_numpy(), oracle.permute(q, (0, 2, 1, 3)))
+    assert np.array_equal(dev.permute(p, (0, 2, 1, 3)).to_numpy(), q)   # and back
+    k = randn(rng, (1, 256, 32, 80), np.float16)                        # Phi-2 heads (shorter sequence)
+    assert np.array_equal(dev.permute(dev.upload(k), (0, 2, 1, 3)).to_numpy(), oracle.permute(k, (0, 2, 1, 3)))
+    assert np.array_equal(dev.permute(dev.upload(k), (0, 2, 3, 1)).to_numpy(), oracle.permute(k, (0, 2, 3, 1)))
+
+
+def test_permute_rejects_duplicates(dev):
+    from ratchet_amd import RatchetError
+
+    x = dev.upload(np.zeros((2, 2, 2, 2), np.float32))
+    with pytest.raises(RatchetError) as e:
+        dev.permute(x, (0, 1, 1, 3))
+    assert e.value.status == 5
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_slice(dev, oracle, dtype):
+    rng = np.random.default_rng(202)
+    x = randn(rng, (6, 5, 9, 40), dtype)
+    dx = dev.upload(x)
+    for ranges in [[(1, 4), (0, 5), (3, 8), (8, 32)], [(0, 6), (0, 5), (0, 9), (0, 40)], [(2, 3), (1, 2), (4, 5), (39, 40)],
+                   [(0, 6), (0, 5), (0, 9), (1, 9)], [(3, 6), (0, 5), (0, 9), (0, 40)], [(0, 6), (2, 4), (0, 9), (0, 40)]]:
+        want = oracle.slice_(x, ranges)
+        got = dev.slice(dx, ranges).to_numpy()
+        assert np.array_equal(got, want), ranges
+    # random sub-ranges as in the reference test (ops/reindex/slice.rs:71-187)
+    for _ in range(16):
+        shape = [int(rng.integers(2, 17)) for _ in range(3)] + [int(rng.integers(2, 129))]
+        y = randn(rng, shape, dtype)
+        ranges = []
+        for s in shape:
+            a = int(rng.integers(0, s))
+            b = int(rng.integers(a + 1, s + 1))
+            ranges.append((a, b))
+        assert np.array_equal(dev.slice(dev.upload(y), ranges).to_numpy(), oracle.slice_(y, ranges)), (shape, ranges)
+    # Phi-3 style split of a fused projection: [1, S, 3*D] -> [1, S, D]
+    z = randn(rng, (1, 64, 3 * 96), dtype)
+    for k in range(3):
+        r = [(0, 1), (0, 64), (k * 96, (k + 1) * 96)]
+        assert np.array_equal(dev.slice(dev.upload(z), r).to_numpy(), oracle.slice_(z, r))
+
+
+def test_slice_rejects_out_of_bounds(dev):
+    from ratchet_amd import RatchetError
+
+    x = dev.upload(np.zeros((2, 3), np.float32))
+    with pytest.raises(RatchetError) as e:
+        dev.slice(x, [(0, 2), (1, 4)])
+    assert e.value.status == 4
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_broadcast(dev, oracle, dtype):
+    rng = np.random.default_rng(203)
+    cases = [((1, 5, 1, 16), (3, 5, 4, 16)), ((1,), (4, 32, 8, 8)), ((2, 1, 1, 1), (2, 3, 4, 5)), ((7,), (2, 7)), ((3, 1), (3, 4)),
+             ((1, 1, 6), (2, 5, 6)), ((1, 32, 64, 1), (1, 32, 64, 64)), ((1, 1, 1, 64), (1, 4, 64, 64)), ((5, 1), (5, 3)),
+             ((2, 1, 3), (2, 7, 3)), ((1, 8, 1, 128), (2, 8, 2, 128)), ((16, 16), (1, 8, 16, 16))]
+    for src, dst in cases:
+        x = randn(rng, src, dtype)
+        want = oracle.broadcast(x, dst, numpy_semantics=True)
+        got = dev.broadcast_to(dev.upload(x), dst).to_numpy()
+        assert np.array_equal(got, want), (src, dst)
+        assert np.array_equal(want, np.broadcast_to(x, dst))
+
+
+def test_broadcast_rejects_invalid(dev):
+    from ratchet_amd import RatchetError
+
+    with pytest.raises(RatchetError) as e:
+        dev.broadcast_to(dev.upload(np.zeros((2, 3), np.float32)), (2, 4))
+    assert e.value.status == 4
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_concat(dev, oracle, dtype):
+    rng = np.random.default_rng(204)
+    # the reference's own case (ops/concat.rs:273-359)
+    xs = [randn(rng, (4, 2, k, 128), dtype) for k in (50, 13, 77, 55, 11)]
+    got = dev.concat([dev.upload(x) for x in xs], 2).to_numpy()
+    assert np.array_equal(got, oracle.concat(xs, 2))
+    for dim, shapes in [(0, [(2, 3), (5, 3), (1, 3)]), (1, [(3, 1), (3, 4)]), (3, [(2, 2, 3, 5), (2, 2, 3, 8)]),
+                        (2, [(1, 4, 31, 80), (1, 4, 1, 80)]), (1, [(2, 7, 3), (2, 9, 3), (2, 1, 3), (2, 2, 3), (2, 5, 3), (2, 6, 3),
+                                                                    (2, 1, 3), (2, 8, 3)])]:
+        ys = [randn(rng, s, dtype) for s in shapes]
+        got = dev.concat([dev.upload(y) for y in ys], dim).to_numpy()
+        assert np.array_equal(got, oracle.concat(ys, dim)), (dim, shapes)
+
+
+def test_concat_rejects_bad_arguments(dev):
+    from ratchet_amd import RatchetError
+
+    a = dev.upload(np.zeros((2, 3), np.float32))
+    b = dev.upload(np.zeros((3, 4), np.float32))
+    with pytest.raises(RatchetError) as e:
+        dev.concat([a, b], 0)
+    assert e.value.status == 4
+    with pytest.raises(RatchetError) as e:
+        dev.concat([a], 0)
+    assert e.value.status == 7
