@@ -1,0 +1,353 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X backend for ratchet-core's memory-bound tensor ops.
+
+A "step" is one pass over every op of BASELINE configs[1..4] (Whisper-tiny attention softmax + reindex, the Phi-2 and
+Phi-3 prefill elementwise blocks, the broadcast/reindex stress set), each op launched once through the C ABI on the
+device's single stream with its inputs already resident in HBM.  A step moves about 5.6 GB, far more than the 256 MB
+Infinity Cache, and every op has its own buffers, so each op sees cache-cold inputs on every step.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops REGEX] [--no-cpu] [--no-check]
+
+Prints ONE JSON line: whole-step throughput (algorithmic bytes / time), per-op microseconds / GB/s / fraction of the
+8 TB/s HBM roofline (HIP events around each launch), the roofline object for the dominant kernel (the f16 softmax over
+[1,32,4096,4096]) and the CPU baseline (the C++ restatement of ratchet's CPU executor on one host core, on a bounded
+sample of the same workload).
+"""
+import argparse
+import json
+import os
+import re
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBPS = 8000.0
+F32, F16 = 0, 1
+
+
+def stream_rng(seed, stream):
+    """One documented counter-based generator: Philox keyed by RATCHET_SEED, one counter block per tensor."""
+    return np.random.Generator(np.random.Philox(key=seed, counter=[0, 0, 0, stream]))
+
+
+def normal(seed, stream, shape, std, dtype, mean=0.0):
+    """N(mean, std) sampled in f32, then rounded once to the storage dtype (as Tensor::randn does, tensor.rs:543-548)."""
+    g = stream_rng(seed, stream)
+    return (g.standard_normal(shape, dtype=np.float32) * np.float32(std) + np.float32(mean)).astype(dtype)
+
+
+class Op:
+    """One benchmark row: device buffers, a launch closure, algorithmic bytes, and a CPU check/baseline closure."""
+
+    def __init__(self, cfg, name, dtype, shapes, alg_bytes, launch, cpu_sample, kernel=None):
+        self.cfg, self.name, self.dtype, self.shapes = cfg, name, dtype, shapes
+        self.alg_bytes = int(alg_bytes)
+        self.launch = launch
+        self.cpu_sample = cpu_sample        # () -> (want, got_fn, tol, sample_alg_bytes, run_fn)
+        self.kernel = kernel
+        self.us = []
+
+
+def build_workload(dev, seed):
+    from ratchet_amd import _lib
+
+    np16, np32 = np.float16, np.float32
+    ops = []
+    st = [100]
+
+    def nxt():
+        st[0] += 1
+        return st[0]
+
+    def up(a):
+        return dev.upload(a)
+
+    # ------------------------------------------------------------------ cfg 1: Whisper-tiny attention softmax + reindex
+    scores1 = normal(seed, nxt(), (1, 6, 1500, 1500), 3.0, np32)
+    d_scores1 = up(scores1)
+    d_soft1 = dev.empty(scores1.shape, F32)
+    ops.append(Op(1, "softmax", "f32", "[1,6,1500,1500]", 2 * scores1.nbytes, lambda: dev.softmax(d_scores1, out=d_soft1),
+                  dict(kind="softmax", x=scores1, out=d_soft1, rows=2048, tol=1e-5), kernel="softmax_wave_kernel"))
+    q1 = normal(seed, nxt(), (1, 1500, 6, 64), 1.0, np32)
+    d_q1 = up(q1)
+    d_q1p = dev.empty((1, 6, 1500, 64), F32)
+    d_q1b = dev.empty((1, 1500, 6, 64), F32)
+    q1p = np.ascontiguousarray(q1.transpose(0, 2, 1, 3))
+    ops.append(Op(1, "permute[0,2,1,3]", "f32", "[1,1500,6,64]->[1,6,1500,64]", 2 * q1.nbytes,
+                  lambda: dev.permute(d_q1, (0, 2, 1, 3), out=d_q1p),
+                  dict(kind="exact", out=d_q1p, run=lambda o: o.permute(q1, (0, 2, 1, 3)), bytes=2 * q1.nbytes)))
+    ops.append(Op(1, "permute back", "f32", "[1,6,1500,64]->[1,1500,6,64]", 2 * q1.nbytes,
+                  lambda: dev.permute(d_q1p, (0, 2, 1, 3), out=d_q1b),
+                  dict(kind="exact", out=d_q1b, run=lambda o: o.permute(q1p, (0, 2, 1, 3)), bytes=2 * q1.nbytes)))
+
+    # ------------------------------------------------------------------ cfg 2: Phi-2 prefill elementwise block, f16
+    x2 = normal(seed, nxt(), (1, 2048, 2560), 1.0, np16)
+    a2 = normal(seed, nxt(), (1, 2048, 2560), 0.5, np16)
+    g2 = normal(seed, nxt(), (2560,), 0.02, np16, mean=1.0)
+    b2 = normal(seed, nxt(), (2560,), 0.02, np16)
+    h2 = normal(seed, nxt(), (1, 2048, 10240), 1.0, np16)
+    d_x2, d_a2, d_g2, d_b2, d_h2 = up(x2), up(a2), up(g2), up(b2), up(h2)
+    d_res2, d_ln2, d_gelu2 = dev.empty(x2.shape, F16), dev.empty(x2.shape, F16), dev.empty(h2.shape, F16)
+    d_x2f32, d_x2f16 = dev.empty(x2.shape, F32), dev.empty(x2.shape, F16)
+    x2_f32 = x2.astype(np32)
+    ops.append(Op(2, "residual add", "f16", "[1,2048,2560]x2", 3 * x2.nbytes, lambda: dev.binary("add", d_x2, d_a2, out=d_res2),
+                  dict(kind="exact", out=d_res2, run=lambda o: o.binary("add", x2, a2), bytes=3 * x2.nbytes)))
+    ops.append(Op(2, "layer_norm", "f16", "2048x2560", 2 * x2.nbytes + g2.nbytes + b2.nbytes,
+                  lambda: dev.layer_norm(d_x2, d_g2, d_b2, 1e-5, out=d_ln2),
+                  dict(kind="rows", out=d_ln2, x=x2, rows=2048, tol=1e-3, fn=lambda o, xs: o.layer_norm(xs, g2, b2, 1e-5, intended=True)),
+                  kernel="norm_seq16_kernel"))
+    ops.append(Op(2, "gelu", "f16", "[1,2048,10240]", 2 * h2.nbytes, lambda: dev.unary("gelu", d_h2, out=d_gelu2),
+                  dict(kind="rows", out=d_gelu2, x=h2, rows=2048, tol=1e-3, fn=lambda o, xs: o.unary("gelu", xs)), kernel="unary_vec_kernel"))
+    ops.append(Op(2, "cast f16->f32", "f16->f32", "[1,2048,2560]", x2.nbytes * 3, lambda: dev.cast(d_x2, F32, out=d_x2f32),
+                  dict(kind="exact", out=d_x2f32, run=lambda o: o.cast(x2, np32), bytes=3 * x2.nbytes)))
+    ops.append(Op(2, "cast f32->f16", "f32->f16", "[1,2048,2560]", x2.nbytes * 3, lambda: dev.cast(d_x2f32, F16, out=d_x2f16),
+                  dict(kind="exact", out=d_x2f16, run=lambda o: o.cast(x2_f32, np16), bytes=3 * x2.nbytes)))
+
+    # ------------------------------------------------------------------ cfg 3: Phi-3-mini prefill, f16
+    x3 = normal(seed, nxt(), (1, 4096, 3072), 1.0, np16)
+    g3 = normal(seed, nxt(), (3072,), 0.02, np16, mean=1.0)
+    gate3 = normal(seed, nxt(), (1, 4096, 8192), 1.0, np16)
+    up3 = normal(seed, nxt(), (1, 4096, 8192), 1.0, np16)
+    d_x3, d_g3, d_gate3, d_up3 = up(x3), up(g3), up(gate3), up(up3)
+    d_rms3, d_silu3, d_swiglu3 = dev.empty(x3.shape, F16), dev.empty(gate3.shape, F16), dev.empty(gate3.shape, F16)
+    ops.append(Op(3, "rms_norm", "f16", "4096x3072", 2 * x3.nbytes + g3.nbytes, lambda: dev.rms_norm(d_x3, d_g3, 1e-5, out=d_rms3),
+                  dict(kind="rows", out=d_rms3, x=x3, rows=4096, tol=1e-3, fn=lambda o, xs: o.rms_norm(xs, g3, 1e-5, intended=True)),
+                  kernel="norm_seq16_kernel"))
+    ops.append(Op(3, "silu(gate)", "f16", "[1,4096,8192]", 2 * gate3.nbytes, lambda: dev.unary("silu", d_gate3, out=d_silu3),
+                  dict(kind="rows", out=d_silu3, x=gate3, rows=1024, tol=1e-3, fn=lambda o, xs: o.unary("silu", xs)), kernel="unary_vec_kernel"))
+    ops.append(Op(3, "mul silu(gate)*up", "f16", "[1,4096,8192]x2", 3 * gate3.nbytes, lambda: dev.binary("mul", d_up3, d_silu3, out=d_swiglu3),
+                  dict(kind="rows2", out=d_swiglu3, rows=512,
+                       fn=lambda o, n: o.binary("mul", up3.reshape(4096, 8192)[:n], o.unary("silu", gate3.reshape(4096, 8192)[:n])),
+                       tol=0.0, bytes_per_row=3 * 8192 * 2)))
+    # scores [1,32,4096,4096]: one head of N(0,2) generated on the host, replicated over the 32 heads on the device
+    S, H = 4096, 32
+    head = normal(seed, nxt(), (S, S), 2.0, np16)
+    mask = np.triu(np.full((S, S), -np.inf, np16), k=1)                      # -inf above the diagonal, 0 elsewhere
+    d_head, d_mask = up(head), up(mask)
+    d_scores3 = dev.empty((1, H, S, S), F16)
+    for h in range(H):
+        _lib.check(dev.lib.rt_d2d(dev.handle, d_scores3.ptr.value + h * head.nbytes, d_head.ptr, head.nbytes))
+    d_masked3 = dev.empty((1, H, S, S), F16)
+    d_soft3 = dev.empty((1, H, S, S), F16)
+    nb = H * head.nbytes
+    ops.append(Op(3, "scores + causal mask (broadcast fused)", "f16", "[1,32,4096,4096]+[4096,4096]", 2 * nb + mask.nbytes,
+                  lambda: dev.binary("add", d_scores3, d_mask, out=d_masked3),
+                  dict(kind="rows2", out=d_masked3, rows=2048, tol=0.0, bytes_per_row=2 * S * 2 + S * 2,
+                       fn=lambda o, n: o.binary("add", head[:n], mask[:n]).reshape(1, 1, n, S)), kernel="binary_suffix_kernel"))
+    ops.append(Op(3, "softmax (causal)", "f16", "131072x4096", 2 * nb, lambda: dev.softmax(d_masked3, out=d_soft3),
+                  dict(kind="rows2", out=d_soft3, rows=2048, tol=0.0, bytes_per_row=2 * S * 2,
+                       fn=lambda o, n: o.softmax(o.binary("add", head[:n], mask[:n])).reshape(1, 1, n, S)), kernel="softmax_seq16_kernel"))
+
+    # ------------------------------------------------------------------ cfg 4: broadcast / reindex stress, f16
+    kv_a = normal(seed, nxt(), (1, 32, 1984, 80), 1.0, np16)
+    kv_b = normal(seed, nxt(), (1, 32, 64, 80), 1.0, np16)
+    d_kva, d_kvb = up(kv_a), up(kv_b)
+    d_kv = dev.empty((1, 32, 2048, 80), F16)
+    ops.append(Op(4, "concat dim 2", "f16", "[1,32,1984,80]+[1,32,64,80]", 2 * (kv_a.nbytes + kv_b.nbytes),
+                  lambda: dev.concat([d_kva, d_kvb], 2, out=d_kv),
+                  dict(kind="exact", out=d_kv, run=lambda o: o.concat([kv_a, kv_b], 2), bytes=2 * (kv_a.nbytes + kv_b.nbytes))))
+    gx = normal(seed, nxt(), (1, 512, 3000), 1.0, np16)
+    gw = normal(seed, nxt(), (512,), 0.02, np16, mean=1.0)
+    gb = normal(seed, nxt(), (512,), 0.02, np16)
+    d_gx, d_gw, d_gb = up(gx), up(gw), up(gb)
+    d_gn = dev.empty(gx.shape, F16)
+    ops.append(Op(4, "group_norm G=32", "f16", "[1,512,3000]", 2 * gx.nbytes + gw.nbytes + gb.nbytes,
+                  lambda: dev.group_norm(d_gx, 32, d_gw, d_gb, 1e-5, out=d_gn),
+                  dict(kind="close", out=d_gn, tol=1e-3, run=lambda o: o.group_norm(gx, 32, gw, gb, 1e-5), bytes=2 * gx.nbytes)))
+    ma = normal(seed, nxt(), (1, 32, 2048, 1), 1.0, np16)
+    mb = normal(seed, nxt(), (1, 1, 1, 2048), 1.0, np16)
+    d_ma, d_mb = up(ma), up(mb)
+    d_mm = dev.empty((1, 32, 2048, 2048), F16)
+    ops.append(Op(4, "mul two-sided broadcast (fused)", "f16", "[1,32,2048,1]x[1,1,1,2048]", ma.nbytes + mb.nbytes + d_mm.nbytes,
+                  lambda: dev.binary("mul", d_ma, d_mb, out=d_mm),
+                  dict(kind="rows2", out=d_mm, rows=2048, tol=0.0, bytes_per_row=2048 * 2,
+                       fn=lambda o, n: o.binary("mul", np.ascontiguousarray(np.broadcast_to(ma[0, 0, :n], (n, 2048))),
+                                                np.ascontiguousarray(np.broadcast_to(mb[0, 0], (n, 2048)))).reshape(1, 1, n, 2048))))
+    p4 = normal(seed, nxt(), (1, 2048, 32, 80), 1.0, np16)
+    d_p4 = up(p4)
+    d_p4o = dev.empty((1, 32, 2048, 80), F16)
+    ops.append(Op(4, "permute[0,2,1,3]", "f16", "[1,2048,32,80]->[1,32,2048,80]", 2 * p4.nbytes,
+                  lambda: dev.permute(d_p4, (0, 2, 1, 3), out=d_p4o),
+                  dict(kind="exact", out=d_p4o, run=lambda o: o.permute(p4, (0, 2, 1, 3)), bytes=2 * p4.nbytes)))
+    return ops
+
+
+def download_rows(dev, buf, nrows, row_elems, np_dtype):
+    """first nrows rows (row_elems each) of a device buffer"""
+    import ctypes
+
+    from ratchet_amd import _lib
+
+    out = np.empty((nrows, row_elems), dtype=np_dtype)
+    _lib.check(dev.lib.rt_d2h(dev.handle, out.ctypes.data_as(ctypes.c_void_p), buf.ptr, out.nbytes))
+    return out
+
+
+def check_and_time_cpu(dev, op, oracle):
+    """Parity of the timed output buffer against the oracle on a bounded sample; returns (ok, cpu_seconds, cpu_bytes)."""
+    c = op.cpu_sample
+    kind = c["kind"]
+    np_dt = {"f32": np.float32, "f16": np.float16, "f16->f32": np.float32, "f32->f16": np.float16}[op.dtype]
+    t_cpu, b_cpu = 0.0, 0
+
+    def timed(fn):
+        nonlocal t_cpu
+        t0 = time.perf_counter()
+        r = fn()
+        t_cpu += time.perf_counter() - t0
+        return r
+
+    if kind == "exact":
+        want = timed(lambda: c["run"](oracle))
+        b_cpu = c["bytes"]
+        got = c["out"].to_numpy()
+        ok = np.array_equal(got.view(np.uint8), np.ascontiguousarray(want).view(np.uint8))
+    elif kind == "close":
+        want = timed(lambda: c["run"](oracle))
+        b_cpu = c["bytes"]
+        bad, _ = oracle.count_not_close(c["out"].to_numpy(), want, c["tol"], c["tol"])
+        ok = bad == 0
+    elif kind == "softmax":
+        x = c["x"].reshape(-1, c["x"].shape[-1])[: c["rows"]]
+        want = timed(lambda: oracle.softmax(x))
+        b_cpu = 2 * x.nbytes
+        got = download_rows(dev, c["out"], c["rows"], x.shape[-1], np_dt)
+        bad, _ = oracle.count_not_close(got, want, c["tol"], c["tol"])
+        ok = bad == 0
+    elif kind == "rows":
+        x = c["x"].reshape(-1, c["x"].shape[-1])[: c["rows"]]
+        want = timed(lambda: c["fn"](oracle, x))
+        b_cpu = 2 * x.nbytes
+        got = download_rows(dev, c["out"], c["rows"], x.shape[-1], np_dt)
+        bad, _ = oracle.count_not_close(got, want, c["tol"], c["tol"])
+        ok = bad == 0
+    else:  # rows2: closure builds the expected first n rows itself
+        n = c["rows"]
+        want = timed(lambda: c["fn"](oracle, n))
+        want = want.reshape(n, -1)
+        b_cpu = n * c["bytes_per_row"]
+        got = download_rows(dev, c["out"], n, want.shape[-1], np_dt)
+        if c["tol"] == 0.0:
+            ok = np.array_equal(got.view(np.uint16), want.view(np.uint16)) or bool(
+                np.all((got.view(np.uint16) == want.view(np.uint16)) | (np.isnan(got) & np.isnan(want))))
+        else:
+            bad, _ = oracle.count_not_close(got, want, c["tol"], c["tol"])
+            ok = bad == 0
+    return bool(ok), t_cpu, b_cpu
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--ops", type=str, default=None, help="regex selecting ops by 'cfgN name'")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline timing")
+    ap.add_argument("--no-check", action="store_true", help="skip the parity check of the timed buffers")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (every op is row/element parallel; there is no multi-GPU path). "
+              "Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    from ratchet_amd import Device
+
+    seed = int(os.environ.get("RATCHET_SEED", "0"))
+    dev = Device(0)
+    t_setup = time.perf_counter()
+    ops = build_workload(dev, seed)
+    if args.ops:
+        rx = re.compile(args.ops)
+        ops = [o for o in ops if rx.search(f"cfg{o.cfg} {o.name}")]
+    dev.sync()
+    t_setup = time.perf_counter() - t_setup
+
+    ev = [(dev.event(), dev.event()) for _ in ops]
+    step_start, step_stop = dev.event(), dev.event()
+
+    for _ in range(args.warmup):
+        for o in ops:
+            o.launch()
+    dev.sync()
+
+    step_ms = []
+    wall0 = time.perf_counter()
+    for _ in range(args.steps):
+        step_start.record()
+        for o, (e0, e1) in zip(ops, ev):
+            e0.record()
+            o.launch()
+            e1.record()
+        step_stop.record()
+        step_ms.append(step_start.elapsed_ms(step_stop))          # waits for the step to finish
+        for o, (e0, e1) in zip(ops, ev):
+            o.us.append(e0.elapsed_ms(e1) * 1e3)
+    dev.sync()
+    wall = time.perf_counter() - wall0
+
+    total_bytes = sum(o.alg_bytes for o in ops)
+    ms_per_step = float(np.mean(step_ms))
+    value = total_bytes / (ms_per_step * 1e-3) / 1e9
+
+    oracle = None
+    parity_ok, cpu_t, cpu_b = True, 0.0, 0
+    per_op_cpu = {}
+    if not (args.no_check and args.no_cpu):
+        from oracle import cpu_oracle as oracle          # the checker / CPU baseline only; never on the measured path
+
+        oracle.lib()
+        oracle.set_reference_copies(True)
+        for o in ops:
+            ok, t, b = check_and_time_cpu(dev, o, oracle)
+            parity_ok = parity_ok and ok
+            if not ok:
+                print(f"bench.py: PARITY FAILURE in cfg{o.cfg} {o.name}", file=sys.stderr)
+            cpu_t += t
+            cpu_b += b
+            per_op_cpu[id(o)] = (t, b)
+
+    rows = []
+    for o in ops:
+        med = float(np.median(o.us))
+        gbps = o.alg_bytes / (med * 1e-6) / 1e9
+        t, b = per_op_cpu.get(id(o), (0.0, 0))
+        rows.append({"cfg": o.cfg, "op": o.name, "dtype": o.dtype, "shape": o.shapes, "alg_MB": round(o.alg_bytes / 1e6, 3),
+                     "us": round(med, 2), "us_mean": round(float(np.mean(o.us)), 2), "GBps": round(gbps, 1),
+                     "frac_hbm": round(gbps / PEAK_HBM_GBPS, 4),
+                     "cpu_GBps": round(b / t / 1e9, 4) if t > 0 else None})
+
+    dom = max(ops, key=lambda o: float(np.mean(o.us)))
+    dom_avg_us = float(np.mean(dom.us))
+    dom_gbps = dom.alg_bytes / (dom_avg_us * 1e-6) / 1e9
+    result = {
+        "metric": "HBM GB/s over one pass of every op in BASELINE configs[1..4] (per-op us / GB/s / % of 8 TB/s in 'ops')",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic (Philox, RATCHET_SEED=%d; the [4096,4096] score head is replicated over 32 heads)" % seed,
+        "config": {"workload": "all ops of BASELINE configs[1..4]: Whisper-tiny softmax+permute (f32), Phi-2 prefill block (f16), "
+                               "Phi-3-mini prefill block incl. [1,32,4096,4096] causal softmax (f16), broadcast/reindex stress (f16)",
+                   "ops": len(ops), "algorithmic_GB_per_step": round(total_bytes / 1e9, 3), "cache": "cold (5.6 GB/step >> 256 MB)"},
+        "roofline": {"bound": "hbm", "kernel": dom.kernel or dom.name, "op": f"cfg{dom.cfg} {dom.name}",
+                     "achieved": round(dom_gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(dom_gbps / PEAK_HBM_GBPS, 4),
+                     "avg_launch_us": round(dom_avg_us, 2), "algorithmic_bytes": dom.alg_bytes, "traffic": None},
+        "cpu_baseline": None if args.no_cpu or cpu_t == 0 else {
+            "value": round(cpu_b / cpu_t / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "every op of the step on one host core with the reference's to_vec/store copies: whole tensors for ops <= 42 MB, "
+                      "the first 512-4096 rows for the large ones (%.1f MB algorithmic, %.1f s)" % (cpu_b / 1e6, cpu_t),
+            "host_cpus": os.cpu_count()},
+        "parity_ok": bool(parity_ok) if not args.no_check else None,
+        "ops": rows,
+        "wall_s": round(wall, 3), "setup_s": round(t_setup, 2),
+    }
+    print(json.dumps(result))
+    dev.close()
+    if not args.no_check and not parity_ok:
+        sys.exit(1)
+
+
+if __name__ == "__main__":
+    main()

@@ -115,8 +115,9 @@ int rt_device_destroy(rt_device* dev) {
     int rc = rt_enter(dev);
     if (rc) return rc;
     (void)hipStreamSynchronize(dev->stream);
-    for (int i = 0; i < RT_UNARY_COUNT; i++)
-        if (dev->unary_lut[i]) (void)hipFree(dev->unary_lut[i]);
+    for (int t = 0; t < 2; t++)
+        for (int i = 0; i < RT_UNARY_COUNT; i++)
+            if (dev->unary_lut[t][i]) (void)hipFree(dev->unary_lut[t][i]);
     if (dev->gn_scratch) (void)hipFree(dev->gn_scratch);
     hipError_t e = hipStreamDestroy(dev->stream);
     delete dev;

@@ -3,6 +3,8 @@
 // All of them are streaming kernels bounded by HBM bandwidth: every lane moves 16 bytes per access (dwordx4), a
 // 256-thread block covers UNROLL consecutive 4 KiB slabs per operand so that a wave always touches one contiguous
 // 1 KiB span, and loads of a whole tile are issued before the first store.  Arithmetic follows rt_arith.h.
+#include <type_traits>
+
 #include "rt_arith.h"
 #include "rt_internal.h"
 
@@ -10,6 +12,8 @@ namespace {
 
 constexpr int BLOCK = 256;
 constexpr int UNROLL = 4;
+// below this many elements the table fill (128 KiB per CU) costs more than computing
+constexpr uint64_t RT_LUT_MIN_NUMEL = 1u << 21;
 
 // ------------------------------------------------------------------------------------------------ binary, contiguous
 template <typename T, int OP>
@@ -182,6 +186,64 @@ __global__ void __launch_bounds__(BLOCK) unary_scalar_kernel(const T* x, T* y, u
     if (i < numel) y[i] = ar_unary<OP, T>(x[i]);
 }
 
+// ------------------------------------------------------------------------------------------------ unary via lookup table
+// A 16-bit type has only 65536 values, so any unary op on it is a 128 KiB table.  The table is produced once per
+// (device, op, type) by the exact kernel above applied to all 65536 bit patterns, which makes the lookup bit-identical
+// to computing.  Each block copies the table into LDS (gfx950 has 160 KiB per CU) and then streams its share of the
+// tensor: 16-byte loads, eight ds_read_u16 lookups per load, 16-byte stores.  The transcendental ops (fdlibm tanh, the
+// double-precision exp, two divisions for GELU/SiLU) cost 5-10x the HBM time when computed per element; the lookup
+// costs less than the memory traffic.
+constexpr int LUT_BLOCK = 1024;
+constexpr int LUT_UNROLL = 4;
+constexpr size_t LUT_BYTES = 65536 * sizeof(uint16_t);
+
+__global__ void iota16_kernel(uint16_t* p) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < 65536) p[i] = (uint16_t)i;
+}
+
+__global__ void __launch_bounds__(LUT_BLOCK) unary_lut_kernel(const uint16_t* __restrict__ table, const uint16_t* __restrict__ x,
+                                                              uint16_t* y, uint64_t numel) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t lut[];
+    {
+        const v4u* src = reinterpret_cast<const v4u*>(table);
+        v4u* dst = reinterpret_cast<v4u*>(lut);
+#pragma unroll
+        for (int i = 0; i < (int)(LUT_BYTES / 16 / LUT_BLOCK); i++) dst[i * LUT_BLOCK + threadIdx.x] = src[i * LUT_BLOCK + threadIdx.x];
+    }
+    __syncthreads();
+    const uint64_t nvec = numel / 8;
+    const v4u* xv = reinterpret_cast<const v4u*>(x);
+    v4u* yv = reinterpret_cast<v4u*>(y);
+    const uint64_t stride = (uint64_t)gridDim.x * (LUT_BLOCK * LUT_UNROLL);
+    for (uint64_t base = (uint64_t)blockIdx.x * (LUT_BLOCK * LUT_UNROLL) + threadIdx.x; base < nvec; base += stride) {
+        v4u in[LUT_UNROLL];
+#pragma unroll
+        for (int k = 0; k < LUT_UNROLL; k++) {
+            const uint64_t i = base + (uint64_t)k * LUT_BLOCK;
+            if (i < nvec) in[k] = xv[i];
+        }
+#pragma unroll
+        for (int k = 0; k < LUT_UNROLL; k++) {
+            const uint64_t i = base + (uint64_t)k * LUT_BLOCK;
+            if (i < nvec) {
+                v4u out;
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    const uint32_t lo = lut[in[k][w] & 0xffffu];
+                    const uint32_t hi = lut[in[k][w] >> 16];
+                    out[w] = lo | (hi << 16);
+                }
+                yv[i] = out;
+            }
+        }
+    }
+    if (blockIdx.x == 0) {
+        const uint64_t i = nvec * 8 + threadIdx.x;
+        if (i < numel) y[i] = lut[x[i]];
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ cast
 template <typename S, typename D> __device__ __forceinline__ D cast_one(S v);
 template <> __device__ __forceinline__ half_t cast_one<float, half_t>(float v) { return (half_t)v; }
@@ -313,6 +375,55 @@ template <typename T> int dispatch_unary(rt_device* dev, int op, const void* x, 
     }
 }
 
+// ops worth a table: everything with a libm call or a division in it
+inline bool lut_worthwhile(int op) {
+    switch (op) {
+        case RT_GELU: case RT_TANH: case RT_EXP: case RT_LOG: case RT_SIN: case RT_COS: case RT_SQRT: case RT_SILU: case RT_SIGMOID:
+            return true;
+        default: return false;
+    }
+}
+
+template <typename T> int build_unary_table(rt_device* dev, int ti, int op) {
+    if (dev->unary_lut[ti][op]) return RT_OK;
+    uint16_t* table = nullptr;
+    uint16_t* iota = nullptr;
+    RT_HIP(hipMalloc((void**)&table, LUT_BYTES));
+    hipError_t e = hipMalloc((void**)&iota, LUT_BYTES);
+    if (e != hipSuccess) {
+        (void)hipFree(table);
+        return rt_fail_hip(e, "hipMalloc(lut)");
+    }
+    hipLaunchKernelGGL(iota16_kernel, dim3(65536 / 256), dim3(256), 0, dev->stream, iota);
+    int rc = dispatch_unary<T>(dev, op, iota, table, 65536);          // the exact kernel defines the table
+    hipError_t es = hipStreamSynchronize(dev->stream);
+    (void)hipFree(iota);
+    if (rc != RT_OK || es != hipSuccess) {
+        (void)hipFree(table);
+        return rc != RT_OK ? rc : rt_fail_hip(es, "building the unary lookup table");
+    }
+    dev->unary_lut[ti][op] = table;
+    return RT_OK;
+}
+
+template <typename T> int unary_via_lut(rt_device* dev, int op, const void* x, void* y, uint64_t numel) {
+    const int ti = std::is_same<T, bf16_t>::value ? 1 : 0;
+    int rc = build_unary_table<T>(dev, ti, op);
+    if (rc) return rc;
+    if (!dev->lut_attr_set) {
+        RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(unary_lut_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)LUT_BYTES));
+        dev->lut_attr_set = 1;
+    }
+    uint64_t blocks = (numel / 8 + LUT_BLOCK * LUT_UNROLL - 1) / (LUT_BLOCK * LUT_UNROLL);
+    if (blocks > (uint64_t)dev->num_cus) blocks = dev->num_cus;          // one resident block per CU (128 KiB of LDS each)
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(unary_lut_kernel, dim3((unsigned)blocks), dim3(LUT_BLOCK), LUT_BYTES, dev->stream,
+                       (const uint16_t*)dev->unary_lut[ti][op], (const uint16_t*)x, (uint16_t*)y, numel);
+    RT_CHECK_LAUNCH("unary_lut_kernel");
+    return RT_OK;
+}
+
 template <typename S, typename D> int launch_cast(rt_device* dev, const void* x, void* y, uint64_t numel) {
     if (rt_aligned(x, 16) && rt_aligned(y, 16)) {
         hipLaunchKernelGGL((cast_vec_kernel<S, D>), dim3(blocks_for(numel / 8, BLOCK * 2)), dim3(BLOCK), 0, dev->stream,
@@ -431,6 +542,13 @@ int dispatch_bcast(rt_device* dev, int op, const void* a, const uint32_t as[4], 
 
 }  // namespace
 
+int rt_unary_table(rt_device* dev, int type_index, int op, const uint16_t** out) {
+    int rc = type_index == 1 ? build_unary_table<bf16_t>(dev, 1, op) : build_unary_table<half_t>(dev, 0, op);
+    if (rc) return rc;
+    *out = dev->unary_lut[type_index == 1 ? 1 : 0][op];
+    return RT_OK;
+}
+
 extern "C" {
 
 int rt_binary(rt_device* dev, int op, int dt, const void* a, const void* b, void* y, uint64_t numel) {
@@ -492,10 +610,12 @@ int rt_unary(rt_device* dev, int op, int dt, const void* x, void* y, uint64_t nu
     RT_REQUIRE(rt_aligned(x, eb) && rt_aligned(y, eb), RT_ERR_ALIGN, "rt_unary: misaligned pointer");
     int rc = rt_enter(dev);
     if (rc) return rc;
+    // large 16-bit tensors: table lookup (bit-identical to computing, see unary_lut_kernel)
+    const bool lut = dt != RT_F32 && numel >= RT_LUT_MIN_NUMEL && lut_worthwhile(op) && rt_aligned(x, 16) && rt_aligned(y, 16);
     switch (dt) {
         case RT_F32: return dispatch_unary<float>(dev, op, x, y, numel);
-        case RT_F16: return dispatch_unary<half_t>(dev, op, x, y, numel);
-        default: return dispatch_unary<bf16_t>(dev, op, x, y, numel);
+        case RT_F16: return lut ? unary_via_lut<half_t>(dev, op, x, y, numel) : dispatch_unary<half_t>(dev, op, x, y, numel);
+        default: return lut ? unary_via_lut<bf16_t>(dev, op, x, y, numel) : dispatch_unary<bf16_t>(dev, op, x, y, numel);
     }
 }
 

@@ -15,8 +15,9 @@ struct rt_device {
     // GroupNorm partial statistics: {mean, m2, count} triples, one per (group, split)
     float* gn_scratch;
     size_t gn_scratch_bytes;
-    // 65536-entry f16 -> f16 lookup tables, built on first use by the exact kernels (index = rt_unary_op)
-    uint16_t* unary_lut[RT_UNARY_COUNT];
+    // 65536-entry 16-bit -> 16-bit lookup tables, built on first use by the exact kernels ([0] = f16, [1] = bf16)
+    uint16_t* unary_lut[2][RT_UNARY_COUNT];
+    int lut_attr_set;
 };
 
 struct rt_event {
@@ -56,11 +57,19 @@ static inline int rt_dt_bytes(int dt) {
 }
 static inline bool rt_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
+// native clang vectors: arrays of these stay in registers (arrays of HIP's uint4 class type can end up in LDS scratch)
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+
 // the kernels index elements with 64-bit integers but grid sizes are 32-bit; 2^40 elements is far beyond 288 GB
 static const uint64_t RT_MAX_NUMEL = 1ull << 40;
 
 // Makes dev's ordinal current.  Every entry point calls it first.
 int rt_enter(rt_device* dev);
+
+// Device pointer to the 65536-entry table out[bits(x)] = bits(op(x)) for a 16-bit type (type_index 0 = f16, 1 = bf16),
+// built on first use by running the exact unary kernel over all bit patterns (blocks until the table is ready).
+int rt_unary_table(rt_device* dev, int type_index, int op, const uint16_t** out);
 
 // ---------------------------------------------------------------------------------------------------------
 // u32 division by a launch-time constant: q = (n * m) >> (32 + s), exact for all n < 2^32 (round-up method)

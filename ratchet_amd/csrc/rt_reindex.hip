@@ -213,12 +213,12 @@ int launch_gather(rt_device* dev, int eb, const void* x, void* y, const uint32_t
 #define RT_SPLAT(ET, VT) \
     hipLaunchKernelGGL((gather_splat_kernel<ET, VT>), dim3(blocks), dim3(BLOCK), 0, dev->stream, (const ET*)x, (VT*)y, p)
         if (eb == 4) {
-            if (vb == 16) RT_SPLAT(uint32_t, uint4);
-            else if (vb == 8) RT_SPLAT(uint32_t, uint2);
+            if (vb == 16) RT_SPLAT(uint32_t, v4u);
+            else if (vb == 8) RT_SPLAT(uint32_t, v2u);
             else RT_SPLAT(uint32_t, uint32_t);
         } else {
-            if (vb == 16) RT_SPLAT(uint16_t, uint4);
-            else if (vb == 8) RT_SPLAT(uint16_t, uint2);
+            if (vb == 16) RT_SPLAT(uint16_t, v4u);
+            else if (vb == 8) RT_SPLAT(uint16_t, v2u);
             else if (vb == 4) RT_SPLAT(uint16_t, uint32_t);
             else RT_SPLAT(uint16_t, uint16_t);
         }
@@ -229,8 +229,8 @@ int launch_gather(rt_device* dev, int eb, const void* x, void* y, const uint32_t
         for (int i = 0; i < 3; i++) p.s[i] = (dst_shape[i] > 1) ? S[i] / per : 0;
         p.s[3] = (per > 1 || dst_shape[3] == 1) ? (dst_shape[3] == 1 ? 0 : 1) : S[3];
 #define RT_GATHER(VT) hipLaunchKernelGGL((gather_vec_kernel<VT>), dim3(blocks), dim3(BLOCK), 0, dev->stream, (const VT*)x, (VT*)y, p)
-        if (vb == 16) RT_GATHER(uint4);
-        else if (vb == 8) RT_GATHER(uint2);
+        if (vb == 16) RT_GATHER(v4u);
+        else if (vb == 8) RT_GATHER(v2u);
         else if (vb == 4) RT_GATHER(uint32_t);
         else RT_GATHER(uint16_t);
 #undef RT_GATHER
@@ -425,8 +425,8 @@ int rt_concat(rt_device* dev, int elem_bytes, int n_inputs, const void* const* x
         }
     }
     const dim3 grid(blocks_for(max_nvec, BLOCK * UNROLL), (unsigned)n_inputs);
-    if (vb == 16) hipLaunchKernelGGL((concat_kernel<uint4>), grid, dim3(BLOCK), 0, dev->stream, (uint4*)y, p);
-    else if (vb == 8) hipLaunchKernelGGL((concat_kernel<uint2>), grid, dim3(BLOCK), 0, dev->stream, (uint2*)y, p);
+    if (vb == 16) hipLaunchKernelGGL((concat_kernel<v4u>), grid, dim3(BLOCK), 0, dev->stream, (v4u*)y, p);
+    else if (vb == 8) hipLaunchKernelGGL((concat_kernel<v2u>), grid, dim3(BLOCK), 0, dev->stream, (v2u*)y, p);
     else if (vb == 4) hipLaunchKernelGGL((concat_kernel<uint32_t>), grid, dim3(BLOCK), 0, dev->stream, (uint32_t*)y, p);
     else hipLaunchKernelGGL((concat_kernel<uint16_t>), grid, dim3(BLOCK), 0, dev->stream, (uint16_t*)y, p);
     RT_CHECK_LAUNCH("concat_kernel");

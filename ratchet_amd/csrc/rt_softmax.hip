@@ -2,9 +2,10 @@
 //
 // Arithmetic contract (REFERENCE mode) = crates/ratchet-core/src/cpu/softmax.rs:22-42: e_j = exp(x_j) with no max
 // subtraction, stored in the element type; sum accumulated over j ascending in the element type; y_j = e_j / sum.
-//   f32: the row lives in registers (one wave64 per row, 16-byte loads), one exp per element, the sum is a wave
-//        butterfly instead of a sequential fold (differs from the reference by float rounding order only), one
-//        IEEE division per element.  HBM traffic: one read, one write.
+//   f32: the row lives in registers (one wave64 per row, 16-byte loads), one exp per element (the device library's
+//        1-ulp expf; the 1e-5 bar leaves room for that), the sum is a wave butterfly instead of a sequential fold
+//        (differs from the reference by float rounding order only), one IEEE division per element.
+//        HBM traffic: one read, one write.
 //   f16/bf16: the sequential 16-bit accumulation is order dependent (terms below half an ulp of the running sum
 //        vanish), so it is replayed exactly: a block stages tiles of exp values through LDS and one lane per row walks
 //        its row left to right with v_add_f16; the second pass recomputes the same exp values and divides.
@@ -78,7 +79,7 @@ __global__ void __launch_bounds__(BLOCK) softmax_wave_kernel(const T* __restrict
             if (lane + k * WAVE < nvec)
 #pragma unroll
                 for (int q = 0; q < VE; q++) {
-                    e[k][q] = rt_expf(Ar<T>::widen(v[k].e[q]));
+                    e[k][q] = expf(Ar<T>::widen(v[k].e[q]));
                     s += e[k][q];
                 }
         s = wave_sum(s);
@@ -123,7 +124,7 @@ __global__ void __launch_bounds__(BLOCK) softmax_generic_kernel(const T* __restr
     }
     float s = 0.0f;
     for (uint32_t j = threadIdx.x; j < cols; j += BLOCK)
-        s += (MODE == 1) ? expf(Ar<T>::widen(xr[j]) - m) : rt_expf(Ar<T>::widen(xr[j]));
+        s += (MODE == 1) ? expf(Ar<T>::widen(xr[j]) - m) : expf(Ar<T>::widen(xr[j]));
     s = wave_sum(s);
     if (lane == 0) red[wave] = s;
     __syncthreads();
@@ -135,7 +136,7 @@ __global__ void __launch_bounds__(BLOCK) softmax_generic_kernel(const T* __restr
     __syncthreads();
     s = bcast;
     for (uint32_t j = threadIdx.x; j < cols; j += BLOCK) {
-        const float ev = (MODE == 1) ? expf(Ar<T>::widen(xr[j]) - m) : rt_expf(Ar<T>::widen(xr[j]));
+        const float ev = (MODE == 1) ? expf(Ar<T>::widen(xr[j]) - m) : expf(Ar<T>::widen(xr[j]));
         yr[j] = Ar<T>::conv(ev / s);
     }
 }
@@ -215,6 +216,202 @@ __global__ void __launch_bounds__(BLOCK) softmax_seq16_kernel(const T* __restric
     }
 }
 
+// ------------------------------------------------------------------------------------------------------------------
+// f16 reference arithmetic, single pass over HBM (cols <= NSLOT * 256, cols % 8 == 0, 16-byte aligned).
+//
+// One 1024-thread block per CU walks over groups of 30 rows.  Wave 0 does nothing but the sequential sums; in the other
+// 15 waves thread (r, cv) owns the 16-byte vectors at columns
+// t*256 + cv*8 of row r, t = 0..NSLOT-1, and keeps their exp values in registers (NSLOT * 4 VGPRs) until the row sum is
+// known, so x is read once and y written once.
+//   exp: a 16-bit type has 65536 values; the part of the exact exp table that is not saturated (x in about
+//        [-17.5, 11.1]; below gives 0, above inf) is 38384 entries = 75 KiB and sits in LDS.  One ds_read_u16 per element.
+//   sum: per 256-column tile the exp values also go to an LDS tile (double buffered); lanes 0..29 of wave 0 each walk
+//        one row of the tile left to right with dependent v_add_f16 (3 ns each on this chip).  A tile is 16 KiB in and
+//        15 KiB out of HBM per CU, about 1 us at a CU's share of 8 TB/s; the walk of 256 columns takes 0.8 us, which is
+//        why wave 0 is kept free of any other work and raises its issue priority.
+//   divide: the outputs of group g are produced while group g+1 streams in: y = e / sum with the quotient computed as
+//        q0 = e * (1/sum) plus one fma correction, which is the correctly rounded f16 quotient for normal finite sums
+//        (checked against IEEE division over operand pairs on the GPU); other sums take the IEEE path.
+// Global loads run two tiles ahead across group boundaries, so the pipeline never drains.
+// ------------------------------------------------------------------------------------------------------------------
+constexpr int SP_BLOCK = 1024;
+constexpr int SP_ROWS = 30;                  // 15 loader waves x 2 rows each; wave 0 only walks
+constexpr int SP_TC = 256;
+constexpr int SP_PAD = 8;
+constexpr uint32_t SP_LUT_POS = 0x4990;      // entries for bit patterns 0x0000 .. 0x498f  (last ones are +inf)
+constexpr uint32_t SP_LUT_NEG = 0x4c60;      // entries for bit patterns 0x8000 .. 0xcc5f  (last ones are +0)
+constexpr size_t SP_LUT_BYTES = (SP_LUT_POS + SP_LUT_NEG) * sizeof(uint16_t);
+constexpr size_t SP_TILE_BYTES = 2 * 32 * (SP_TC + SP_PAD) * sizeof(uint16_t);
+constexpr size_t SP_SMEM_BYTES = SP_LUT_BYTES + SP_TILE_BYTES + 2 * 32 * sizeof(uint16_t);
+
+__device__ __forceinline__ uint32_t sp_exp_lookup(const uint16_t* lut, uint32_t h) {
+    uint32_t idx;
+    if (h & 0x8000u) {
+        const uint32_t m = h - 0x8000u;
+        idx = SP_LUT_POS + (m < SP_LUT_NEG ? m : SP_LUT_NEG - 1);
+    } else {
+        idx = h < SP_LUT_POS ? h : SP_LUT_POS - 1;
+    }
+    uint32_t e = lut[idx];
+    if ((h & 0x7fffu) > 0x7c00u) e = 0x7e00u;            // exp(NaN) = NaN
+    return e;
+}
+
+template <int NSLOT>
+__global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint16_t* __restrict__ table, const half_t* x, half_t* y,
+                                                                      uint64_t rows, uint32_t cols) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    uint16_t* lut = reinterpret_cast<uint16_t*>(smem);
+    half_t (*tile)[32][SP_TC + SP_PAD] = reinterpret_cast<half_t (*)[32][SP_TC + SP_PAD]>(smem + SP_LUT_BYTES);
+    half_t (*sums)[32] = reinterpret_cast<half_t (*)[32]>(smem + SP_LUT_BYTES + SP_TILE_BYTES);
+
+    // table -> LDS (16-byte copies; both ranges start 16-byte aligned in the table and have multiple-of-8 lengths)
+    {
+        const v4u* src = reinterpret_cast<const v4u*>(table);
+        v4u* dst = reinterpret_cast<v4u*>(lut);
+        for (uint32_t i = threadIdx.x; i < SP_LUT_POS / 8; i += SP_BLOCK) dst[i] = src[i];
+        const v4u* srcn = reinterpret_cast<const v4u*>(table + 0x8000);
+        v4u* dstn = reinterpret_cast<v4u*>(lut + SP_LUT_POS);
+        for (uint32_t i = threadIdx.x; i < SP_LUT_NEG / 8; i += SP_BLOCK) dstn[i] = srcn[i];
+    }
+    const uint64_t ngroups = (rows + SP_ROWS - 1) / SP_ROWS;
+    __syncthreads();                                         // table visible
+
+    if (threadIdx.x < 64) {
+        // ------------------------------------------------------------------ wave 0: the walk, nothing else
+        __builtin_amdgcn_s_setprio(3);
+        const uint32_t lane = threadIdx.x;
+        const uint32_t wr = lane < SP_ROWS ? lane : 0;       // lanes 30..63 shadow row 0 and never publish
+        half_t run = (half_t)0.0f;
+        uint32_t gpar = 0;
+        for (uint64_t g = blockIdx.x; g < ngroups; g += gridDim.x) {
+#pragma unroll 1
+            for (int t = 0; t < NSLOT; t++) {
+                __syncthreads();                             // tile t is in LDS
+                const v4u* trow = reinterpret_cast<const v4u*>(tile[t & 1][wr]);
+                // 16 values per chunk; the LDS reads of the next chunk are in flight during the 16 dependent adds
+                v4u c0 = trow[0], c1 = trow[1];
+#pragma unroll
+                for (int c = 0; c < SP_TC / 16; c++) {
+                    v4u n0 = c0, n1 = c1;
+                    if (c + 1 < SP_TC / 16) {
+                        n0 = trow[(c + 1) * 2];
+                        n1 = trow[(c + 1) * 2 + 1];
+                    }
+#pragma unroll
+                    for (int w = 0; w < 4; w++) {
+                        run = run + bits_h((uint16_t)(c0[w] & 0xffffu));
+                        run = run + bits_h((uint16_t)(c0[w] >> 16));
+                    }
+#pragma unroll
+                    for (int w = 0; w < 4; w++) {
+                        run = run + bits_h((uint16_t)(c1[w] & 0xffffu));
+                        run = run + bits_h((uint16_t)(c1[w] >> 16));
+                    }
+                    c0 = n0;
+                    c1 = n1;
+                }
+            }
+            if (lane < SP_ROWS) sums[gpar][lane] = run;
+            run = (half_t)0.0f;
+            gpar ^= 1;
+        }
+        __syncthreads();                                     // drain barrier (matches the loaders')
+        return;
+    }
+
+    // ---------------------------------------------------------------------- waves 1..15: load, exp, park, divide, store
+    const uint32_t lt = threadIdx.x - 64;                    // 0..959
+    const uint32_t r = lt >> 5, cv = lt & 31;                // row in the group (0..29), vector in the tile
+    const uint32_t ccol = cv * 8;                            // column of this thread's vector inside a tile
+
+    auto load_x = [&](uint64_t g, uint32_t t, v4u& dst) {
+        const uint64_t row = g * SP_ROWS + r;
+        const uint32_t col = t * SP_TC + ccol;
+        if (g < ngroups && row < rows && col < cols) dst = *reinterpret_cast<const v4u*>(x + row * cols + col);
+    };
+
+    v4u e[NSLOT];                                            // exp values of the group in flight, 8 halves per slot
+    v4u pre0 = {0, 0, 0, 0}, pre1 = {0, 0, 0, 0};
+    uint64_t g = blockIdx.x;
+    load_x(g, 0, pre0);
+    load_x(g, 1, pre1);
+
+    bool have_prev = false;
+    uint64_t prev_row = 0;
+    float s_prev = 0.0f, rinv_prev = 0.0f;
+    bool fast_prev = false;
+    uint32_t gpar = 0;
+
+    auto flush_slot = [&](int t, const v4u& ev) {           // y[prev_row][slot t] = e / sum of the previous group
+        const uint32_t col = t * SP_TC + ccol;
+        if (prev_row < rows && col < cols) {
+            v4u out;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                uint32_t packed = 0;
+#pragma unroll
+                for (int hsel = 0; hsel < 2; hsel++) {
+                    const float ef = (float)bits_h((uint16_t)(hsel ? (ev[w] >> 16) : (ev[w] & 0xffffu)));
+                    float q;
+                    if (fast_prev) {
+                        const float q0 = ef * rinv_prev;
+                        const float err = __builtin_fmaf(-s_prev, q0, ef);
+                        q = __builtin_fmaf(err, rinv_prev, q0);
+                    } else {
+                        q = ef / s_prev;
+                    }
+                    packed |= (uint32_t)h_bits((half_t)q) << (16 * hsel);
+                }
+                out[w] = packed;
+            }
+            *reinterpret_cast<v4u*>(y + prev_row * cols + col) = out;
+        }
+    };
+    auto read_prev_sum = [&](uint32_t par) {
+        const float s = (float)sums[par][r];
+        s_prev = s;
+        // normal, finite, not tiny: the reciprocal-plus-correction quotient is exact there
+        fast_prev = (s >= 6.103515625e-05f) && (s < __builtin_huge_valf());
+        rinv_prev = fast_prev ? 1.0f / s : 0.0f;
+    };
+
+    for (; g < ngroups; g += gridDim.x) {
+        const uint64_t row = g * SP_ROWS + r;
+        const bool rvalid = row < rows;
+#pragma unroll
+        for (int t = 0; t < NSLOT; t++) {
+            v4u& pre = (t & 1) ? pre1 : pre0;
+            const uint32_t col = t * SP_TC + ccol;
+            // exp of the vector that arrived, parked in the LDS tile for the walk (zeros past the row end: adding +0 is a no-op)
+            v4u enew = {0, 0, 0, 0};
+            if (rvalid && col < cols) {
+#pragma unroll
+                for (int w = 0; w < 4; w++)
+                    enew[w] = sp_exp_lookup(lut, pre[w] & 0xffffu) | (sp_exp_lookup(lut, pre[w] >> 16) << 16);
+            }
+            *reinterpret_cast<v4u*>(&tile[t & 1][r][ccol]) = enew;
+            // next load for this register: two tiles ahead, possibly in the block's next group
+            if (t + 2 < NSLOT) load_x(g, t + 2, pre);
+            else load_x(g + gridDim.x, t + 2 - NSLOT, pre);
+            __syncthreads();
+            if (t == 0 && have_prev) read_prev_sum(gpar ^ 1);     // published by wave 0 before it reached this barrier
+            if (have_prev) flush_slot(t, e[t]);
+            e[t] = enew;
+        }
+        have_prev = true;
+        prev_row = row;
+        gpar ^= 1;
+    }
+    // drain: outputs of the block's last group
+    __syncthreads();
+    if (have_prev) {
+        read_prev_sum(gpar ^ 1);
+#pragma unroll
+        for (int t = 0; t < NSLOT; t++) flush_slot(t, e[t]);
+    }
+}
+
 template <typename T, int MODE> int launch_wave(rt_device* dev, const void* x, void* y, uint64_t rows, uint32_t cols) {
     constexpr int VE = 16 / sizeof(T);
     const uint32_t nvec = cols / VE;
@@ -242,6 +439,33 @@ template <typename T, int MODE> int launch_f32_style(rt_device* dev, const void*
     hipLaunchKernelGGL((softmax_generic_kernel<T, MODE>), dim3((unsigned)rows), dim3(BLOCK), 0, dev->stream, (const T*)x, (T*)y, rows,
                        cols);
     RT_CHECK_LAUNCH("softmax_generic_kernel");
+    return RT_OK;
+}
+
+int launch_f16_stream(rt_device* dev, const void* x, void* y, uint64_t rows, uint32_t cols) {
+    const uint16_t* table = nullptr;
+    int rc = rt_unary_table(dev, 0, RT_EXP, &table);
+    if (rc) return rc;
+    uint64_t blocks = (rows + SP_ROWS - 1) / SP_ROWS;
+    if (blocks > (uint64_t)dev->num_cus) blocks = dev->num_cus;      // one resident block per CU
+    const uint32_t nt = (cols + SP_TC - 1) / SP_TC;
+#define RT_SP(NS)                                                                                                                   \
+    do {                                                                                                                            \
+        static bool attr_done = false;                                                                                              \
+        if (!attr_done) {                                                                                                           \
+            RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(softmax_f16_stream_kernel<NS>),                                \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)SP_SMEM_BYTES));                            \
+            attr_done = true;                                                                                                       \
+        }                                                                                                                           \
+        hipLaunchKernelGGL((softmax_f16_stream_kernel<NS>), dim3((unsigned)blocks), dim3(SP_BLOCK), SP_SMEM_BYTES, dev->stream, table, \
+                           (const half_t*)x, (half_t*)y, rows, cols);                                                              \
+    } while (0)
+    if (nt <= 2) RT_SP(2);
+    else if (nt <= 4) RT_SP(4);
+    else if (nt <= 8) RT_SP(8);
+    else RT_SP(16);
+#undef RT_SP
+    RT_CHECK_LAUNCH("softmax_f16_stream_kernel");
     return RT_OK;
 }
 
@@ -283,7 +507,12 @@ extern "C" int rt_softmax(rt_device* dev, int dt, const void* x, void* y, uint64
     }
     switch (dt) {
         case RT_F32: return launch_f32_style<float, 0>(dev, x, y, rows, cols);
-        case RT_F16: return launch_seq16<half_t>(dev, x, y, rows, cols);
+        case RT_F16:
+            // rows of up to 4096 columns stream through registers in one pass once there is enough work to amortise the
+            // per-block table load; everything else takes the two-pass tile walker
+            if (cols % 8 == 0 && cols <= 16 * SP_TC && rows * cols >= (1u << 20) && rt_aligned(x, 16) && rt_aligned(y, 16))
+                return launch_f16_stream(dev, x, y, rows, cols);
+            return launch_seq16<half_t>(dev, x, y, rows, cols);
         default: return launch_seq16<bf16_t>(dev, x, y, rows, cols);
     }
 }

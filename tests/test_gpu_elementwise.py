@@ -188,3 +188,33 @@ def test_cast(dev, oracle):
     big = dev.empty((1000,), _lib.F32)
     v = big.view(1, (777,)).upload(y[:777])
     assert same_bits(dev.cast(v, _lib.F16).to_numpy(), oracle.cast(y[:777], np.float16))
+
+
+@pytest.mark.parametrize("op", ["gelu", "silu", "sigmoid", "tanh", "exp", "sqrt", "log"])
+def test_unary_f16_large_tensor_table_path(dev, oracle, op):
+    # tensors of 2^21 elements and more go through the LDS lookup table; it must equal the computed kernel bit for bit
+    rng = np.random.default_rng(120)
+    n = (1 << 22) + 5
+    x = ALL_F16[rng.integers(0, 65536, n)]
+    x[:65536] = ALL_F16
+    want = oracle.unary(op, x)
+    dx = dev.upload(x)
+    got = dev.unary(op, dx).to_numpy()
+    allowed = 8 * (n // 65536 + 1) if op == "log" else 0
+    assert mismatch_count(got, want) <= allowed, (op, mismatch_count(got, want))
+    small = dev.unary(op, dev.upload(ALL_F16)).to_numpy()        # computed path
+    assert same_bits(got[:65536], small)
+    dev.unary(op, dx, out=dx)                                    # in place
+    assert same_bits(dx.to_numpy(), got)
+
+
+def test_unary_bf16_large_tensor_table_path(dev, oracle):
+    rng = np.random.default_rng(121)
+    n = (1 << 21) + 3
+    x = rng.integers(0, 65536, n).astype(np.uint16)
+    x[:65536] = np.arange(65536, dtype=np.uint16)
+    for op in ("gelu", "silu"):
+        want = oracle.unary(op, x, bf16=True)
+        got = dev.unary(op, dev.upload(x, bf16=True)).to_numpy()
+        wf, gf = oracle.cast(want, np.float32, src_bf16=True), oracle.cast(got, np.float32, src_bf16=True)
+        assert np.all((got == want) | (np.isnan(wf) & np.isnan(gf))), op

@@ -70,6 +70,28 @@ def test_softmax_f16_reference_sequence(dev, oracle, shape):
     assert mismatch_count(got, want) == 0, (shape, mismatch_count(got, want))
 
 
+@pytest.mark.parametrize("shape", [(1, 300, 4096), (2, 601, 1000), (1, 2100, 512), (1, 4099, 264), (7, 64, 2560)])
+def test_softmax_f16_streaming_kernel(dev, oracle, shape):
+    # >= 2^20 elements with cols <= 4096 and cols % 8 == 0: the single-pass kernel (exp table in LDS, rows held in registers)
+    rng = np.random.default_rng(303)
+    x = randn(rng, shape, np.float16, 2.0)
+    n = shape[-1]
+    flat = x.reshape(-1, n)
+    for i in range(0, flat.shape[0], 3):                               # causal-style -inf tails of varying length
+        flat[i, (i * 37) % n + 1:] = -np.inf
+    flat[5, 7] = 12.0                                                  # overflow: inf sum, NaN at that element, 0 elsewhere
+    flat[11, :] = -np.inf                                              # fully masked row: 0/0
+    flat[13, 3] = np.nan
+    flat[17, :] = -20.0                                                # every exp underflows to 0
+    flat[19, :] = -16.0                                                # subnormal exps
+    want = oracle.softmax(x)
+    dx = dev.upload(x)
+    got = dev.softmax(dx).to_numpy()
+    assert mismatch_count(got, want) == 0, (shape, mismatch_count(got, want))
+    dev.softmax(dx, out=dx)                                            # in place, as the reference runs it
+    assert same_bits(dx.to_numpy(), want)
+
+
 def test_softmax_f16_order_dependence_is_reproduced(dev, oracle):
     # 2048 + 1 + 1 + ... never grows in f16: the kernel must reproduce that, not the mathematically exact sum
     row = np.zeros(512, np.float16)
