@@ -244,18 +244,22 @@ constexpr size_t SP_LUT_BYTES = (SP_LUT_POS + SP_LUT_NEG) * sizeof(uint16_t);
 constexpr size_t SP_TILE_BYTES = 2 * 32 * (SP_TC + SP_PAD) * sizeof(uint16_t);
 constexpr size_t SP_SMEM_BYTES = SP_LUT_BYTES + SP_TILE_BYTES + 2 * 32 * sizeof(uint16_t);
 
-__device__ __forceinline__ uint32_t sp_exp_lookup(const uint16_t* lut, uint32_t h) {
-    uint32_t idx;
-    if (h & 0x8000u) {
-        const uint32_t m = h - 0x8000u;
-        idx = SP_LUT_POS + (m < SP_LUT_NEG ? m : SP_LUT_NEG - 1);
-    } else {
-        idx = h < SP_LUT_POS ? h : SP_LUT_POS - 1;
-    }
-    uint32_t e = lut[idx];
-    if ((h & 0x7fffu) > 0x7c00u) e = 0x7e00u;            // exp(NaN) = NaN
-    return e;
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+typedef short i16x2 __attribute__((ext_vector_type(2)));
+
+// exp of two packed f16 bit patterns through the LDS table, branch free: both halves are clamped into the stored range
+// with packed 16-bit min/sub (the saturated ends of the table hold +inf and +0), then looked up.  NaNs are patched by
+// the caller.
+__device__ __forceinline__ uint32_t sp_exp_pair(const uint16_t* lut, uint32_t p) {
+    const u16x2 h = __builtin_bit_cast(u16x2, p);
+    const u16x2 neg = __builtin_bit_cast(u16x2, __builtin_bit_cast(i16x2, p) >> 15);       // 0xffff where the sign bit is set
+    const u16x2 top = (neg & (u16x2)(0x8000 + SP_LUT_NEG - SP_LUT_POS)) + (u16x2)(SP_LUT_POS - 1);
+    const u16x2 clamped = __builtin_elementwise_min(h, top);
+    const u16x2 idx = clamped - (neg & (u16x2)(0x8000 - SP_LUT_POS));
+    return (uint32_t)lut[idx.x] | ((uint32_t)lut[idx.y] << 16);
 }
+// bit 15 / bit 31 set where the corresponding half of p is a NaN: (h & 0x7fff) > 0x7c00  <=>  (h & 0x7fff) + 0x3ff >= 0x8000
+__device__ __forceinline__ uint32_t sp_nan_bits(uint32_t p) { return ((p & 0x7fff7fffu) + 0x03ff03ffu) & 0x80008000u; }
 
 template <int NSLOT>
 __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint16_t* __restrict__ table, const half_t* x, half_t* y,
@@ -347,23 +351,24 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
         const uint32_t col = t * SP_TC + ccol;
         if (prev_row < rows && col < cols) {
             v4u out;
+            if (fast_prev) {
 #pragma unroll
-            for (int w = 0; w < 4; w++) {
-                uint32_t packed = 0;
-#pragma unroll
-                for (int hsel = 0; hsel < 2; hsel++) {
-                    const float ef = (float)bits_h((uint16_t)(hsel ? (ev[w] >> 16) : (ev[w] & 0xffffu)));
-                    float q;
-                    if (fast_prev) {
-                        const float q0 = ef * rinv_prev;
-                        const float err = __builtin_fmaf(-s_prev, q0, ef);
-                        q = __builtin_fmaf(err, rinv_prev, q0);
-                    } else {
-                        q = ef / s_prev;
-                    }
-                    packed |= (uint32_t)h_bits((half_t)q) << (16 * hsel);
+                for (int w = 0; w < 4; w++) {
+                    const float e0 = (float)bits_h((uint16_t)(ev[w] & 0xffffu)), e1 = (float)bits_h((uint16_t)(ev[w] >> 16));
+                    const float a0 = e0 * rinv_prev, a1 = e1 * rinv_prev;
+                    float q0 = __builtin_fmaf(__builtin_fmaf(-s_prev, a0, e0), rinv_prev, a0);
+                    float q1 = __builtin_fmaf(__builtin_fmaf(-s_prev, a1, e1), rinv_prev, a1);
+                    // keep the f32 quotient and its conversion apart: fused into v_fma_mixlo_f16 the pair rounds
+                    // subnormal f16 results differently from fma-then-convert
+                    asm volatile("" : "+v"(q0), "+v"(q1));
+                    out[w] = (uint32_t)h_bits((half_t)q0) | ((uint32_t)h_bits((half_t)q1) << 16);
                 }
-                out[w] = packed;
+            } else {
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    const float e0 = (float)bits_h((uint16_t)(ev[w] & 0xffffu)), e1 = (float)bits_h((uint16_t)(ev[w] >> 16));
+                    out[w] = (uint32_t)h_bits((half_t)(e0 / s_prev)) | ((uint32_t)h_bits((half_t)(e1 / s_prev)) << 16);
+                }
             }
             *reinterpret_cast<v4u*>(y + prev_row * cols + col) = out;
         }
@@ -387,8 +392,16 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
             v4u enew = {0, 0, 0, 0};
             if (rvalid && col < cols) {
 #pragma unroll
-                for (int w = 0; w < 4; w++)
-                    enew[w] = sp_exp_lookup(lut, pre[w] & 0xffffu) | (sp_exp_lookup(lut, pre[w] >> 16) << 16);
+                for (int w = 0; w < 4; w++) enew[w] = sp_exp_pair(lut, pre[w]);
+                const uint32_t nans = sp_nan_bits(pre[0]) | sp_nan_bits(pre[1]) | sp_nan_bits(pre[2]) | sp_nan_bits(pre[3]);
+                if (nans) {                                  // exp(NaN) = NaN; rare, so patched out of line
+#pragma unroll
+                    for (int w = 0; w < 4; w++) {
+                        const uint32_t nb = sp_nan_bits(pre[w]);
+                        if (nb & 0x8000u) enew[w] = (enew[w] & 0xffff0000u) | 0x7e00u;
+                        if (nb & 0x80000000u) enew[w] = (enew[w] & 0x0000ffffu) | 0x7e000000u;
+                    }
+                }
             }
             *reinterpret_cast<v4u*>(&tile[t & 1][r][ccol]) = enew;
             // next load for this register: two tiles ahead, possibly in the block's next group

@@ -41,3 +41,14 @@ def ulp_diff(a, b):
 
 def randn(rng, shape, dtype, scale=1.0):
     return (rng.standard_normal(shape) * scale).astype(np.float32).astype(dtype)
+
+
+def describe_mismatch(got, want, x=None, limit=8):
+    """human-readable list of the first few differing elements (flat index, input, got, want)"""
+    g, w = np.asarray(got).reshape(-1), np.asarray(want).reshape(-1)
+    bad = np.flatnonzero(~((bits(g) == bits(w)) | (np.isnan(g) & np.isnan(w))))
+    xs = np.asarray(x).reshape(-1) if x is not None and np.asarray(x).size == g.size else None
+    rows = []
+    for i in bad[:limit]:
+        rows.append((int(i), None if xs is None else float(xs[i]), float(g[i]), float(w[i]), hex(int(bits(g)[i])), hex(int(bits(w)[i]))))
+    return {"count": int(bad.size), "first": rows}

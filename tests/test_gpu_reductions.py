@@ -9,7 +9,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from gpu_util import mismatch_count, randn, same_bits
+from gpu_util import describe_mismatch, mismatch_count, randn, same_bits
 
 pytestmark = pytest.mark.gpu
 
@@ -87,7 +87,7 @@ def test_softmax_f16_streaming_kernel(dev, oracle, shape):
     want = oracle.softmax(x)
     dx = dev.upload(x)
     got = dev.softmax(dx).to_numpy()
-    assert mismatch_count(got, want) == 0, (shape, mismatch_count(got, want))
+    assert mismatch_count(got, want) == 0, (shape, describe_mismatch(got, want, x))
     dev.softmax(dx, out=dx)                                            # in place, as the reference runs it
     assert same_bits(dx.to_numpy(), want)
 
