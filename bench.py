@@ -71,7 +71,7 @@ def build_workload(dev, seed):
     d_scores1 = up(scores1)
     d_soft1 = dev.empty(scores1.shape, F32)
     ops.append(Op(1, "softmax", "f32", "[1,6,1500,1500]", 2 * scores1.nbytes, lambda: dev.softmax(d_scores1, out=d_soft1),
-                  dict(kind="softmax", x=scores1, out=d_soft1, rows=2048, tol=1e-5), kernel="softmax_wave_kernel"))
+                  dict(kind="softmax", x=scores1, out=d_soft1, rows=9000, tol=1e-5), kernel="softmax_wave_kernel"))
     q1 = normal(seed, nxt(), (1, 1500, 6, 64), 1.0, np32)
     d_q1 = up(q1)
     d_q1p = dev.empty((1, 6, 1500, 64), F32)
@@ -99,9 +99,9 @@ def build_workload(dev, seed):
     ops.append(Op(2, "layer_norm", "f16", "2048x2560", 2 * x2.nbytes + g2.nbytes + b2.nbytes,
                   lambda: dev.layer_norm(d_x2, d_g2, d_b2, 1e-5, out=d_ln2),
                   dict(kind="rows", out=d_ln2, x=x2, rows=2048, tol=1e-3, fn=lambda o, xs: o.layer_norm(xs, g2, b2, 1e-5, intended=True)),
-                  kernel="norm_seq16_kernel"))
+                  kernel="norm_pipe16_kernel"))
     ops.append(Op(2, "gelu", "f16", "[1,2048,10240]", 2 * h2.nbytes, lambda: dev.unary("gelu", d_h2, out=d_gelu2),
-                  dict(kind="rows", out=d_gelu2, x=h2, rows=2048, tol=1e-3, fn=lambda o, xs: o.unary("gelu", xs)), kernel="unary_vec_kernel"))
+                  dict(kind="rows", out=d_gelu2, x=h2, rows=2048, tol=1e-3, fn=lambda o, xs: o.unary("gelu", xs)), kernel="unary_lut_kernel"))
     ops.append(Op(2, "cast f16->f32", "f16->f32", "[1,2048,2560]", x2.nbytes * 3, lambda: dev.cast(d_x2, F32, out=d_x2f32),
                   dict(kind="exact", out=d_x2f32, run=lambda o: o.cast(x2, np32), bytes=3 * x2.nbytes)))
     ops.append(Op(2, "cast f32->f16", "f32->f16", "[1,2048,2560]", x2.nbytes * 3, lambda: dev.cast(d_x2f32, F16, out=d_x2f16),
@@ -116,11 +116,11 @@ def build_workload(dev, seed):
     d_rms3, d_silu3, d_swiglu3 = dev.empty(x3.shape, F16), dev.empty(gate3.shape, F16), dev.empty(gate3.shape, F16)
     ops.append(Op(3, "rms_norm", "f16", "4096x3072", 2 * x3.nbytes + g3.nbytes, lambda: dev.rms_norm(d_x3, d_g3, 1e-5, out=d_rms3),
                   dict(kind="rows", out=d_rms3, x=x3, rows=4096, tol=1e-3, fn=lambda o, xs: o.rms_norm(xs, g3, 1e-5, intended=True)),
-                  kernel="norm_seq16_kernel"))
+                  kernel="norm_pipe16_kernel"))
     ops.append(Op(3, "silu(gate)", "f16", "[1,4096,8192]", 2 * gate3.nbytes, lambda: dev.unary("silu", d_gate3, out=d_silu3),
-                  dict(kind="rows", out=d_silu3, x=gate3, rows=1024, tol=1e-3, fn=lambda o, xs: o.unary("silu", xs)), kernel="unary_vec_kernel"))
+                  dict(kind="rows", out=d_silu3, x=gate3, rows=4096, tol=1e-3, fn=lambda o, xs: o.unary("silu", xs)), kernel="unary_lut_kernel"))
     ops.append(Op(3, "mul silu(gate)*up", "f16", "[1,4096,8192]x2", 3 * gate3.nbytes, lambda: dev.binary("mul", d_up3, d_silu3, out=d_swiglu3),
-                  dict(kind="rows2", out=d_swiglu3, rows=512,
+                  dict(kind="rows2", out=d_swiglu3, rows=4096,
                        fn=lambda o, n: o.binary("mul", up3.reshape(4096, 8192)[:n], o.unary("silu", gate3.reshape(4096, 8192)[:n])),
                        tol=0.0, bytes_per_row=3 * 8192 * 2)))
     # scores [1,32,4096,4096]: one head of N(0,2) generated on the host, replicated over the 32 heads on the device
@@ -136,11 +136,11 @@ def build_workload(dev, seed):
     nb = H * head.nbytes
     ops.append(Op(3, "scores + causal mask (broadcast fused)", "f16", "[1,32,4096,4096]+[4096,4096]", 2 * nb + mask.nbytes,
                   lambda: dev.binary("add", d_scores3, d_mask, out=d_masked3),
-                  dict(kind="rows2", out=d_masked3, rows=2048, tol=0.0, bytes_per_row=2 * S * 2 + S * 2,
-                       fn=lambda o, n: o.binary("add", head[:n], mask[:n]).reshape(1, 1, n, S)), kernel="binary_suffix_kernel"))
+                  dict(kind="rows2", out=d_masked3, rows=16384, tol=0.0, bytes_per_row=2 * S * 2 + S * 2,
+                       fn=lambda o, n: np.tile(o.binary("add", head, mask), (n // S, 1))), kernel="binary_bcast_kernel"))
     ops.append(Op(3, "softmax (causal)", "f16", "131072x4096", 2 * nb, lambda: dev.softmax(d_masked3, out=d_soft3),
-                  dict(kind="rows2", out=d_soft3, rows=2048, tol=0.0, bytes_per_row=2 * S * 2,
-                       fn=lambda o, n: o.softmax(o.binary("add", head[:n], mask[:n])).reshape(1, 1, n, S)), kernel="softmax_seq16_kernel"))
+                  dict(kind="rows2", out=d_soft3, rows=16384, tol=0.0, bytes_per_row=2 * S * 2,
+                       fn=lambda o, n: o.softmax(np.tile(o.binary("add", head, mask), (n // S, 1)))), kernel="softmax_f16_stream_kernel"))
 
     # ------------------------------------------------------------------ cfg 4: broadcast / reindex stress, f16
     kv_a = normal(seed, nxt(), (1, 32, 1984, 80), 1.0, np16)
@@ -164,16 +164,40 @@ def build_workload(dev, seed):
     d_mm = dev.empty((1, 32, 2048, 2048), F16)
     ops.append(Op(4, "mul two-sided broadcast (fused)", "f16", "[1,32,2048,1]x[1,1,1,2048]", ma.nbytes + mb.nbytes + d_mm.nbytes,
                   lambda: dev.binary("mul", d_ma, d_mb, out=d_mm),
-                  dict(kind="rows2", out=d_mm, rows=2048, tol=0.0, bytes_per_row=2048 * 2,
-                       fn=lambda o, n: o.binary("mul", np.ascontiguousarray(np.broadcast_to(ma[0, 0, :n], (n, 2048))),
-                                                np.ascontiguousarray(np.broadcast_to(mb[0, 0], (n, 2048)))).reshape(1, 1, n, 2048))))
+                  dict(kind="rows2", out=d_mm, rows=65536, tol=0.0, bytes_per_row=2048 * 2,
+                       fn=lambda o, n: o.binary("mul", np.ascontiguousarray(np.broadcast_to(ma.reshape(-1, 1)[:n], (n, 2048))),
+                                                np.ascontiguousarray(np.broadcast_to(mb.reshape(1, 2048), (n, 2048)))))))
     p4 = normal(seed, nxt(), (1, 2048, 32, 80), 1.0, np16)
     d_p4 = up(p4)
     d_p4o = dev.empty((1, 32, 2048, 80), F16)
     ops.append(Op(4, "permute[0,2,1,3]", "f16", "[1,2048,32,80]->[1,32,2048,80]", 2 * p4.nbytes,
                   lambda: dev.permute(d_p4, (0, 2, 1, 3), out=d_p4o),
                   dict(kind="exact", out=d_p4o, run=lambda o: o.permute(p4, (0, 2, 1, 3)), bytes=2 * p4.nbytes)))
+    ops_extra["copy_pair"] = (d_scores3, d_masked3)
     return ops
+
+
+ops_extra = {}
+
+
+def copy_ceiling(dev):
+    """What a plain copy kernel reaches on this chip on a 1 GiB tensor (1 GiB read + 1 GiB written): the practical HBM
+    ceiling for a streaming kernel, quoted beside the 8 TB/s peak."""
+    from ratchet_amd import _lib
+
+    src, dst = ops_extra["copy_pair"]
+    e0, e1 = dev.event(), dev.event()
+    times = []
+    for i in range(4):
+        e0.record()
+        _lib.check(dev.lib.rt_cast(dev.handle, F16, F16, src.ptr, dst.ptr, src.numel))
+        e1.record()
+        t = e0.elapsed_ms(e1)
+        if i:
+            times.append(t)
+    ms = float(np.mean(times))
+    return {"kernel": "copy_vec_kernel", "bytes": 2 * src.nbytes, "us": round(ms * 1e3, 1), "GBps": round(2 * src.nbytes / ms / 1e6, 1),
+            "frac_of_peak": round(2 * src.nbytes / ms / 1e6 / PEAK_HBM_GBPS, 4)}
 
 
 def download_rows(dev, buf, nrows, row_elems, np_dtype):
@@ -310,6 +334,8 @@ def main():
             cpu_b += b
             per_op_cpu[id(o)] = (t, b)
 
+    ceiling = copy_ceiling(dev) if not args.ops else None      # after the parity check: it overwrites an output buffer
+
     rows = []
     for o in ops:
         med = float(np.median(o.us))
@@ -336,9 +362,10 @@ def main():
                      "avg_launch_us": round(dom_avg_us, 2), "algorithmic_bytes": dom.alg_bytes, "traffic": None},
         "cpu_baseline": None if args.no_cpu or cpu_t == 0 else {
             "value": round(cpu_b / cpu_t / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": "every op of the step on one host core with the reference's to_vec/store copies: whole tensors for ops <= 42 MB, "
-                      "the first 512-4096 rows for the large ones (%.1f MB algorithmic, %.1f s)" % (cpu_b / 1e6, cpu_t),
+            "sample": "every op of the step on one host core with the reference's to_vec/store copies: whole tensors, except the first "
+                      "16384 of 131072 rows (4 heads) for the two ops on [1,32,4096,4096] (%.1f MB algorithmic, %.1f s)" % (cpu_b / 1e6, cpu_t),
             "host_cpus": os.cpu_count()},
+        "hbm_copy_ceiling": ceiling,
         "parity_ok": bool(parity_ok) if not args.no_check else None,
         "ops": rows,
         "wall_s": round(wall, 3), "setup_s": round(t_setup, 2),

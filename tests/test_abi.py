@@ -1,0 +1,137 @@
+"""CPU-only checks of the C ABI: the library loads without a GPU, exports every symbol include/ratchet_hip.h declares, and
+rejects bad arguments before touching HIP (so these paths are testable here; no compute call needs a device).
+
+Error behaviour mirrors the reference's guards: Permute duplicate dims (ops/reindex/permute.rs:49-52), Broadcast shape
+rule (ops/reindex/broadcast.rs:31-58), Slice bounds (ops/reindex/slice.rs:38-51), Concat arity/shape rule
+(ops/concat.rs:131-152), float-only dtypes for binary/unary/softmax/norm (ops/binary.rs:247-270, ops/softmax.rs:36-39).
+"""
+import ctypes
+import os
+import re
+
+import pytest
+
+from ratchet_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _lib.load()
+
+
+def u4(*v):
+    return (ctypes.c_uint32 * 4)(*v)
+
+
+def test_header_and_library_agree(lib):
+    header = open(os.path.join(ROOT, "include", "ratchet_hip.h")).read()
+    declared = sorted(set(re.findall(r"^(?:int|const char\*)\s+(rt_[a-z0-9_]+)\(", header, flags=re.M)))
+    assert declared, "no declarations parsed"
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in ratchet_hip.h but not exported"
+    assert sorted(_lib.EXPORTS) == declared
+
+
+def test_status_names(lib):
+    for code, name in _lib.STATUS_NAMES.items():
+        assert lib.rt_status_name(code).decode() == name
+    assert lib.rt_status_name(-2).decode() == "HIP_ERROR"
+
+
+def test_no_device_is_reported_not_hidden(lib):
+    n = ctypes.c_int(-1)
+    rc = lib.rt_device_count(ctypes.byref(n))
+    if rc != 0:                       # this container has no GPU: a HIP error code, never a silent fallback
+        assert rc < 0 and n.value == 0
+        h = ctypes.c_void_p()
+        assert lib.rt_device_create(0, ctypes.byref(h)) < 0
+        assert h.value is None
+        assert b"hip" in lib.rt_last_error().lower()
+
+
+SOME = ctypes.c_void_p(0x1000)        # a non-null, 16-byte aligned fake pointer: validation must reject before using it
+ODD = ctypes.c_void_p(0x1001)
+
+
+def test_binary_validation(lib):
+    assert lib.rt_binary(None, 9, _lib.F32, SOME, SOME, SOME, 8) == 3                 # RT_ERR_OP
+    assert lib.rt_binary(None, _lib.ADD, _lib.I32, SOME, SOME, SOME, 8) == 2          # RT_ERR_DTYPE
+    assert lib.rt_binary(None, _lib.ADD, _lib.F32, None, SOME, SOME, 8) == 1          # RT_ERR_NULL_POINTER
+    assert lib.rt_binary(None, _lib.ADD, _lib.F32, SOME, SOME, ODD, 8) == 9           # RT_ERR_ALIGN
+    assert lib.rt_binary(None, _lib.ADD, _lib.F32, SOME, SOME, SOME, 1 << 41) == 6    # RT_ERR_SIZE
+    assert lib.rt_binary(None, _lib.ADD, _lib.F32, SOME, SOME, SOME, 8) == 8          # all fine but no device
+    assert b"NULL" in lib.rt_last_error()
+
+
+def test_broadcast_binary_validation(lib):
+    ok = (None, _lib.MUL, _lib.F16, SOME, u4(1, 32, 64, 1), SOME, u4(1, 1, 1, 64), SOME, u4(1, 32, 64, 64))
+    assert lib.rt_binary_bcast(*ok) == 8
+    bad = (None, _lib.MUL, _lib.F16, SOME, u4(1, 32, 64, 3), SOME, u4(1, 1, 1, 64), SOME, u4(1, 32, 64, 64))
+    assert lib.rt_binary_bcast(*bad) == 4                                             # BroadcastingFailed
+    bad = (None, _lib.MUL, _lib.F16, SOME, u4(1, 32, 64, 1), SOME, u4(1, 1, 1, 64), SOME, u4(1, 32, 64, 128))
+    assert lib.rt_binary_bcast(*bad) == 4
+    zero = (None, _lib.MUL, _lib.F16, SOME, u4(1, 0, 64, 1), SOME, u4(1, 1, 1, 64), SOME, u4(1, 0, 64, 64))
+    assert lib.rt_binary_bcast(*zero) == 4
+
+
+def test_unary_and_cast_validation(lib):
+    assert lib.rt_unary(None, 14, _lib.F32, SOME, SOME, 8) == 3
+    assert lib.rt_unary(None, 0, _lib.U32, SOME, SOME, 8) == 2
+    assert lib.rt_unary(None, 0, _lib.F16, SOME, None, 8) == 1
+    assert lib.rt_unary(None, 0, _lib.F16, SOME, SOME, 8) == 8
+    assert lib.rt_cast(None, _lib.F16, _lib.I32, SOME, SOME, 8) == 2                  # unimplemented!() in the reference
+    assert lib.rt_cast(None, _lib.F16, _lib.BF16, SOME, SOME, 8) == 2
+    assert lib.rt_cast(None, 7, _lib.F32, SOME, SOME, 8) == 2
+    assert lib.rt_cast(None, _lib.F32, _lib.F16, SOME, SOME, 8) == 8
+    assert lib.rt_cast(None, _lib.F32, _lib.U32, SOME, SOME, 8) == 8
+
+
+def test_reindex_validation(lib):
+    shp = u4(2, 3, 4, 5)
+    assert lib.rt_permute(None, 4, SOME, SOME, shp, u4(0, 1, 1, 3)) == 5              # DuplicateDims
+    assert lib.rt_permute(None, 4, SOME, SOME, shp, u4(0, 1, 2, 4)) == 5
+    assert lib.rt_permute(None, 3, SOME, SOME, shp, u4(0, 1, 2, 3)) == 7              # elem_bytes
+    assert lib.rt_permute(None, 4, SOME, SOME, shp, u4(3, 2, 1, 0)) == 8
+    assert lib.rt_slice(None, 2, SOME, SOME, shp, u4(0, 0, 0, 3), u4(2, 3, 4, 3)) == 4   # 3 + 3 > 5
+    assert lib.rt_slice(None, 2, SOME, SOME, shp, u4(0, 0, 0, 0), u4(2, 3, 4, 0)) == 4   # empty range
+    assert lib.rt_slice(None, 2, SOME, SOME, shp, u4(1, 0, 0, 2), u4(1, 3, 4, 3)) == 8
+    assert lib.rt_broadcast(None, 4, SOME, SOME, u4(1, 3, 1, 5), u4(2, 3, 4, 6)) == 4
+    assert lib.rt_broadcast(None, 4, SOME, SOME, u4(1, 3, 1, 5), u4(2, 3, 4, 5)) == 8
+    shapes = ((ctypes.c_uint32 * 4) * 2)(u4(1, 2, 3, 4), u4(1, 2, 5, 4))
+    ptrs = (ctypes.c_void_p * 2)(0x1000, 0x2000)
+    assert lib.rt_concat(None, 4, 2, ptrs, shapes, 2, SOME) == 8
+    assert lib.rt_concat(None, 4, 2, ptrs, shapes, 1, SOME) == 4                      # differs outside the concat dim
+    assert lib.rt_concat(None, 4, 1, ptrs, shapes, 2, SOME) == 7                      # needs 2..8 inputs
+    assert lib.rt_concat(None, 4, 9, ptrs, shapes, 2, SOME) == 7
+    assert lib.rt_concat(None, 4, 2, ptrs, shapes, 4, SOME) == 7
+
+
+def test_reduction_validation(lib):
+    assert lib.rt_softmax(None, _lib.I32, SOME, SOME, 4, 8, 0) == 2
+    assert lib.rt_softmax(None, _lib.F32, SOME, SOME, 4, 8, 5) == 7                   # unknown mode
+    assert lib.rt_softmax(None, _lib.F32, SOME, SOME, 4, 0, 0) == 4
+    assert lib.rt_softmax(None, _lib.F32, SOME, SOME, 4, 8, 0) == 8
+    assert lib.rt_layer_norm(None, _lib.F32, SOME, None, None, SOME, 4, 8, 1e-5) == 1   # scale is required
+    assert lib.rt_layer_norm(None, _lib.F32, SOME, SOME, None, SOME, 4, 8, 1e-5) == 8   # bias is optional
+    assert lib.rt_layer_norm(None, _lib.F32, SOME, SOME, None, SOME, 4, 8, float("nan")) == 7
+    assert lib.rt_rms_norm(None, _lib.U32, SOME, SOME, SOME, 4, 8, 1e-5) == 2
+    assert lib.rt_group_norm(None, _lib.F16, SOME, None, None, SOME, 1, 6, 4, 4, 1e-5) == 7   # 6 channels, 4 groups
+    assert lib.rt_group_norm(None, _lib.F16, SOME, None, None, SOME, 1, 8, 4, 4, 1e-5) == 8
+
+
+def test_storage_validation(lib):
+    p = ctypes.c_void_p()
+    assert lib.rt_malloc(None, 16, ctypes.byref(p)) == 8
+    assert lib.rt_malloc(None, 16, None) == 1
+    assert lib.rt_sync(None) == 8
+    assert lib.rt_h2d(None, None, None, 16) == 1
+    assert lib.rt_event_elapsed_ms(None, None, None) == 1
+
+
+def test_python_binding_fails_loudly_without_library(tmp_path, monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "missing.so"))
+    with pytest.raises(ImportError):
+        _lib.load()
