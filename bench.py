@@ -26,6 +26,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBPS = 8000.0
+# HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same script (KiB counters scaled by
+# what a 1 GiB copy kernel reads on them, x2.000 and x1.000); bench.py cannot collect counters itself
+PMC_TRAFFIC_BYTES = {"softmax_f16_stream_kernel": int((1049831.1 + 1048576.0) * 1024)}
 F32, F16 = 0, 1
 
 
@@ -359,7 +362,9 @@ def main():
                    "ops": len(ops), "algorithmic_GB_per_step": round(total_bytes / 1e9, 3), "cache": "cold (5.6 GB/step >> 256 MB)"},
         "roofline": {"bound": "hbm", "kernel": dom.kernel or dom.name, "op": f"cfg{dom.cfg} {dom.name}",
                      "achieved": round(dom_gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(dom_gbps / PEAK_HBM_GBPS, 4),
-                     "avg_launch_us": round(dom_avg_us, 2), "algorithmic_bytes": dom.alg_bytes, "traffic": None},
+                     "avg_launch_us": round(dom_avg_us, 2), "algorithmic_bytes": dom.alg_bytes,
+                     # FETCH_SIZE + WRITE_SIZE per launch, scaled by a 1 GiB copy kernel (profiles/bench_step_hbm_traffic_pmc.txt)
+                     "traffic": PMC_TRAFFIC_BYTES.get(dom.kernel)},
         "cpu_baseline": None if args.no_cpu or cpu_t == 0 else {
             "value": round(cpu_b / cpu_t / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": "every op of the step on one host core with the reference's to_vec/store copies: whole tensors, except the first "
