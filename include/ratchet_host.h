@@ -1,0 +1,64 @@
+/*
+ * ratchet_host.h - C view of the C++ host mirror of ratchet-core's lazy Tensor API (ratchet_amd/csrc/host/ratchet.hpp),
+ * exported by libratchet_host.so.  It exists so that non-C++ callers (the Python parity tests) can drive the same graph
+ * building and resolve() code path; the device work itself goes through ratchet_hip.h.
+ *
+ * Handles are opaque and owned by the caller: release every rth_tensor / rth_device that a call returned.
+ * Builders return NULL on error; other calls return non-zero.  rth_last_error_kind() is the invariant that failed
+ * (the reference's InvariantError / assert it corresponds to, e.g. "BroadcastingFailed", "DuplicateDims",
+ * "DTypeMismatch"), rth_last_error() the full message; both are thread-local.
+ */
+#ifndef RATCHET_HOST_H
+#define RATCHET_HOST_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct rth_device rth_device;
+typedef struct rth_tensor rth_tensor;
+
+const char* rth_last_error(void);
+const char* rth_last_error_kind(void);
+
+rth_device* rth_device_request(int ordinal);                          /* Device::request_device (device.rs:61-77) */
+void rth_device_release(rth_device* dev);
+
+/* Tensor::from_data + to(device) (tensor.rs:553-571,874-892); dt codes as in ratchet_hip.h */
+rth_tensor* rth_from_host(rth_device* dev, const void* data, int rank, const uint64_t* shape, int dt);
+/* shape-only constant without storage: graph building and its errors can be exercised without a GPU; cannot be resolved */
+rth_tensor* rth_placeholder(int rank, const uint64_t* shape, int dt);
+void rth_release(rth_tensor* t);
+int rth_rank(const rth_tensor* t);
+int rth_shape(const rth_tensor* t, uint64_t* dims /* rank entries */);
+int rth_dtype(const rth_tensor* t);
+int rth_resolved(const rth_tensor* t);
+const char* rth_op_name(const rth_tensor* t);
+
+/* op builders (tensor.rs:294-495): record a node, run nothing */
+rth_tensor* rth_binary(const rth_tensor* a, const rth_tensor* b, int op);         /* add/sub/mul/div = 0..3 */
+rth_tensor* rth_unary(const rth_tensor* x, int op);                               /* UnaryOp order, gelu = 0 */
+rth_tensor* rth_cast(const rth_tensor* x, int dst_dt);
+rth_tensor* rth_layer_norm(const rth_tensor* x, const rth_tensor* weight, const rth_tensor* bias /* nullable */, float eps);
+rth_tensor* rth_rms_norm(const rth_tensor* x, const rth_tensor* weight, float eps);
+rth_tensor* rth_group_norm(const rth_tensor* x, size_t num_groups, const rth_tensor* weight, const rth_tensor* bias, float eps);
+rth_tensor* rth_softmax(const rth_tensor* x, size_t dim, int mode);
+rth_tensor* rth_slice(const rth_tensor* x, int n, const uint64_t* starts, const uint64_t* ends);
+rth_tensor* rth_view(const rth_tensor* x, int rank, const uint64_t* shape);
+rth_tensor* rth_cat(const rth_tensor* const* xs, int n, size_t dim);
+rth_tensor* rth_permute(const rth_tensor* x, int n, const uint64_t* dims);
+rth_tensor* rth_broadcast_to(const rth_tensor* x, int rank, const uint64_t* shape);
+
+int rth_resolve(rth_tensor* t);                                        /* Tensor::resolve (tensor.rs:861-863) */
+int rth_to_host(const rth_tensor* t, void* out);                       /* to(&Device::CPU) (tensor.rs:957-975) */
+long rth_last_resolve_launches(const rth_tensor* t);                   /* kernels launched by the last rth_resolve(t) */
+int rth_execution_order(const rth_tensor* t, uint64_t* ids, int cap);  /* ids in execution order; returns the count */
+uint64_t rth_id(const rth_tensor* t);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

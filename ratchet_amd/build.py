@@ -18,6 +18,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(HERE, "libratchet_hip.so")
+HOST_DIR = os.path.join(CSRC, "host")
+HOST_LIB_PATH = os.path.join(HERE, "libratchet_host.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -55,6 +57,22 @@ def _compile(src, force):
     return obj
 
 
+def build_host(force=False):
+    """libratchet_host.so: the C++ mirror of ratchet's lazy Tensor API (host code only, g++), linked against
+    libratchet_hip.so in the same directory."""
+    srcs = sorted(glob.glob(os.path.join(HOST_DIR, "*.cpp")))
+    deps = srcs + glob.glob(os.path.join(HOST_DIR, "*.hpp")) + headers() + [LIB_PATH]
+    if force or _newer(HOST_LIB_PATH, deps):
+        cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-o", HOST_LIB_PATH] + srcs + [
+            "-L" + HERE, "-lratchet_hip", "-Wl,-rpath,$ORIGIN"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("host library build failed:\n%s\n%s" % (" ".join(cmd), r.stderr[-8000:]))
+        if r.stderr.strip():
+            sys.stderr.write(r.stderr[-4000:])
+    return HOST_LIB_PATH
+
+
 def build(force=False, jobs=4):
     os.makedirs(OBJ_DIR, exist_ok=True)
     with ThreadPoolExecutor(max_workers=jobs) as ex:
@@ -64,6 +82,7 @@ def build(force=False, jobs=4):
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError("link failed:\n%s\n%s" % (" ".join(cmd), r.stderr[-8000:]))
+    build_host(force)
     return LIB_PATH
 
 

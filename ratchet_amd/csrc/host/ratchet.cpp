@@ -1,0 +1,564 @@
+// Implementation of the C++ host mirror (see ratchet.hpp).  Host code only: it talks to the GPU through the C ABI of
+// libratchet_hip.so and contains no arithmetic on tensor data.
+#include "ratchet.hpp"
+
+#include <algorithm>
+#include <atomic>
+#include <sstream>
+#include <unordered_set>
+
+#include "../../../include/ratchet_hip.h"
+
+namespace ratchet {
+
+// ------------------------------------------------------------------------------------------------------------ basics
+size_t size_of(DType dt) { return (dt == DType::F16 || dt == DType::BF16) ? 2 : 4; }
+bool is_float(DType dt) { return dt == DType::F32 || dt == DType::F16 || dt == DType::BF16; }
+const char* as_str(DType dt) {
+    switch (dt) {
+        case DType::F32: return "F32";
+        case DType::F16: return "F16";
+        case DType::BF16: return "BF16";
+        case DType::I32: return "I32";
+        default: return "U32";
+    }
+}
+
+size_t Shape::numel() const {
+    size_t n = 1;
+    for (size_t d : dims_) n *= d;
+    return n;
+}
+bool Shape::is_scalar() const {
+    return std::all_of(dims_.begin(), dims_.end(), [](size_t d) { return d == 1; });
+}
+Shape Shape::promote(const Shape& s, size_t rank) {
+    std::vector<size_t> d(s.dims_);
+    while (d.size() < rank) d.insert(d.begin(), 1);
+    return Shape(d);
+}
+bool Shape::multi_broadcast(const std::vector<const Shape*>& shapes, Shape* out) {
+    size_t max_rank = 0;
+    for (const Shape* s : shapes) max_rank = std::max(max_rank, s->rank());
+    std::vector<size_t> dims(max_rank, 1);
+    for (size_t i = 0; i < max_rank; i++) {
+        size_t cur = 1;
+        for (const Shape* s : shapes) {
+            const size_t len = s->rank();
+            const size_t d = i < len ? (*s)[len - i - 1] : 1;
+            if (d != 1) {
+                if (cur != 1 && d != cur) return false;
+                cur = d;
+            }
+        }
+        dims[max_rank - 1 - i] = cur;
+    }
+    *out = Shape(dims);
+    return true;
+}
+std::string Shape::to_string() const {
+    std::ostringstream o;
+    o << "[";
+    for (size_t i = 0; i < dims_.size(); i++) o << (i ? "," : "") << dims_[i];
+    o << "]";
+    return o.str();
+}
+std::vector<ptrdiff_t> contiguous_strides(const Shape& s) {
+    std::vector<ptrdiff_t> st(s.rank());
+    ptrdiff_t acc = 1;
+    for (size_t i = s.rank(); i-- > 0;) {
+        st[i] = acc;
+        acc *= (ptrdiff_t)s[i];
+    }
+    return st;
+}
+
+static void check_rt(int status, const char* what) {
+    if (status != 0) throw Error(status < 0 ? "DeviceError" : rt_status_name(status), std::string(what) + ": " + rt_last_error());
+}
+
+// ------------------------------------------------------------------------------------------------------------ device
+Device::Inner::~Inner() {
+    if (raw) rt_device_destroy(raw);
+}
+Device Device::request(int ordinal) {
+    Device d;
+    d.inner_ = std::make_shared<Inner>();
+    check_rt(rt_device_create(ordinal, &d.inner_->raw), "rt_device_create");
+    return d;
+}
+void Device::sync() const { check_rt(rt_sync(raw()), "rt_sync"); }
+
+Buffer::Buffer(const Device& d, size_t n) : device(d), bytes(n) { check_rt(rt_malloc(d.raw(), n, &ptr), "rt_malloc"); }
+Buffer::~Buffer() {
+    if (ptr) rt_free(device.raw(), ptr);
+}
+
+// ------------------------------------------------------------------------------------------------------------ graph
+enum class Kind { Const, Binary, Unary, Cast, Permute, Slice, Broadcast, Concat, Softmax, LayerNorm, RMSNorm, GroupNorm, View };
+
+struct Node {
+    uint64_t id = 0;
+    Kind kind = Kind::Const;
+    Shape shape;
+    DType dt = DType::F32;
+    Device device;
+    std::vector<Tensor> srcs;                 // Operation::srcs(), in bind order
+    BinaryOp bop = BinaryOp::Add;
+    UnaryOp uop = UnaryOp::Gelu;
+    std::vector<size_t> dims;                 // permute dims
+    std::vector<std::pair<size_t, size_t>> ranges;
+    size_t dim = 0;                           // concat / softmax
+    size_t groups = 0;
+    float eps = 0.0f;
+    bool has_bias = false;
+    SoftmaxMode mode = SoftmaxMode::Reference;
+    std::shared_ptr<Buffer> storage;          // Some(..) once resolved
+    size_t last_launches = 0;
+
+    static Node* of(const Tensor& t) { return t.node_.get(); }
+    static long holders(const Tensor& t) { return t.node_.use_count(); }
+    static Tensor wrap(std::shared_ptr<Node> n) { return Tensor(std::move(n)); }
+};
+
+static std::atomic<uint64_t> g_next_id{1};
+
+static std::shared_ptr<Node> new_node(Kind k, const Shape& shape, DType dt, const Device& dev) {
+    auto n = std::make_shared<Node>();
+    n->id = g_next_id++;
+    n->kind = k;
+    n->shape = shape;
+    n->dt = dt;
+    n->device = dev;
+    return n;
+}
+
+static void require_same_device(const Tensor& a, const Tensor& b) {
+    if (!(a.device() == b.device())) throw Error("DeviceMismatch", "operands live on different devices");
+}
+static void require_rank4(const Shape& s, const char* who) {
+    if (s.rank() == 0 || s.rank() > 4) throw Error("RankMismatch", std::string(who) + ": rank " + std::to_string(s.rank()) + " (1..4 supported)");
+}
+
+const Shape& Tensor::shape() const { return node_->shape; }
+DType Tensor::dt() const { return node_->dt; }
+const Device& Tensor::device() const { return node_->device; }
+bool Tensor::resolved() const { return node_ && node_->storage != nullptr; }
+uint64_t Tensor::id() const { return node_->id; }
+size_t Tensor::last_resolve_launches() const { return node_->last_launches; }
+const char* Tensor::op_name() const {
+    switch (node_->kind) {
+        case Kind::Const: return "Const";
+        case Kind::Binary: {
+            static const char* n[] = {"Add", "Sub", "Mul", "Div"};
+            return n[(int)node_->bop];
+        }
+        case Kind::Unary: {
+            static const char* n[] = {"Gelu", "Tanh", "Exp", "Log", "Sin", "Cos", "Abs", "Sqrt", "Relu", "Floor", "Ceil", "Neg", "Silu", "Sigmoid"};
+            return n[(int)node_->uop];
+        }
+        case Kind::Cast: return "Cast";
+        case Kind::Permute: return "Permute";
+        case Kind::Slice: return "Slice";
+        case Kind::Broadcast: return "Broadcast";
+        case Kind::Concat: return "Concat";
+        case Kind::Softmax: return "Softmax";
+        case Kind::View: return "View";
+        default: return "Norm";
+    }
+}
+
+Tensor Tensor::from_host(const void* data, const Shape& shape, DType dt, const Device& device) {
+    require_rank4(shape, "from_host");
+    auto n = new_node(Kind::Const, shape, dt, device);
+    const size_t bytes = shape.numel() * size_of(dt);
+    n->storage = std::make_shared<Buffer>(device, bytes);
+    check_rt(rt_h2d(device.raw(), n->storage->ptr, data, bytes), "rt_h2d");
+    return Tensor(n);
+}
+Tensor Tensor::zeros(const Shape& shape, DType dt, const Device& device) {
+    require_rank4(shape, "zeros");
+    auto n = new_node(Kind::Const, shape, dt, device);
+    const size_t bytes = shape.numel() * size_of(dt);
+    n->storage = std::make_shared<Buffer>(device, bytes);
+    check_rt(rt_memset0(device.raw(), n->storage->ptr, bytes), "rt_memset0");
+    return Tensor(n);
+}
+
+Tensor Tensor::placeholder(const Shape& shape, DType dt) {
+    require_rank4(shape, "placeholder");
+    return Tensor(new_node(Kind::Const, shape, dt, Device()));
+}
+
+// impl_binary_op! (tensor.rs:249-280) + Binary guards (ops/binary.rs:135-145)
+Tensor Tensor::binary(const Tensor& other, BinaryOp op) const {
+    require_same_device(*this, other);
+    if (dt() != other.dt()) throw Error("DTypeMismatch", std::string("expected ") + as_str(dt()) + ", got " + as_str(other.dt()));
+    if (!is_float(dt())) throw Error("UnsupportedDType", as_str(dt()));
+    Shape out;
+    if (!Shape::multi_broadcast({&shape(), &other.shape()}, &out))
+        throw Error("BroadcastingFailed", shape().to_string() + " vs " + other.shape().to_string());
+    Tensor lhs = *this, rhs = other;
+    if (lhs.shape() != out) lhs = lhs.broadcast_to(out);       // the reference stops after the first one that needs it
+    if (rhs.shape() != out) rhs = rhs.broadcast_to(out);
+    auto n = new_node(Kind::Binary, out, dt(), device());
+    n->bop = op;
+    n->srcs = {lhs, rhs};
+    return Tensor(n);
+}
+
+Tensor Tensor::unary(UnaryOp op) const {
+    if (!is_float(dt())) throw Error("UnsupportedDType", as_str(dt()));
+    auto n = new_node(Kind::Unary, shape(), dt(), device());
+    n->uop = op;
+    n->srcs = {*this};
+    return Tensor(n);
+}
+
+Tensor Tensor::cast(DType dst) const {
+    if (dt() == dst) return *this;
+    const DType s = dt();
+    const bool numeric = (s == DType::F32 && (dst == DType::F16 || dst == DType::BF16)) ||
+                         ((s == DType::F16 || s == DType::BF16) && dst == DType::F32);
+    const bool reinterpret = (s == DType::F32 && (dst == DType::I32 || dst == DType::U32)) ||
+                             ((s == DType::I32 || s == DType::U32) && dst == DType::F32);
+    if (!numeric && !reinterpret) throw Error("UnsupportedCast", std::string(as_str(s)) + " -> " + as_str(dst));   // unimplemented!() in cpu_cast
+    auto n = new_node(Kind::Cast, shape(), dst, device());
+    n->srcs = {*this};
+    return Tensor(n);
+}
+
+static void check_norm_operands(const Tensor& x, const Tensor& w, const Tensor* b, size_t expect) {
+    if (x.rank() < 2) throw Error("RankMismatch", "norm input needs rank >= 2");            // NormOp::check_shapes
+    if (!is_float(x.dt())) throw Error("UnsupportedDType", as_str(x.dt()));
+    if (w.dt() != x.dt()) throw Error("DTypeMismatch", std::string("expected ") + as_str(x.dt()) + ", got " + as_str(w.dt()));
+    if (b && b->dt() != x.dt()) throw Error("DTypeMismatch", std::string("expected ") + as_str(x.dt()) + ", got " + as_str(b->dt()));
+    if (w.numel() != expect || (b && b->numel() != expect))
+        throw Error("ShapeMismatch", "scale/bias must hold " + std::to_string(expect) + " elements");
+}
+
+Tensor Tensor::layer_norm(const Tensor& weight, const Tensor* bias, float eps) const {
+    check_norm_operands(*this, weight, bias, shape()[rank() - 1]);
+    auto n = new_node(Kind::LayerNorm, shape(), dt(), device());
+    n->eps = eps;
+    n->has_bias = bias != nullptr;
+    n->srcs = {*this, weight};
+    if (bias) n->srcs.push_back(*bias);
+    return Tensor(n);
+}
+Tensor Tensor::rms_norm(const Tensor& weight, float eps) const {
+    check_norm_operands(*this, weight, nullptr, shape()[rank() - 1]);
+    auto n = new_node(Kind::RMSNorm, shape(), dt(), device());
+    n->eps = eps;
+    n->srcs = {*this, weight};
+    return Tensor(n);
+}
+Tensor Tensor::group_norm(size_t num_groups, const Tensor& weight, const Tensor* bias, float eps) const {
+    if (rank() < 2) throw Error("RankMismatch", "group_norm input needs rank >= 2");
+    const size_t C = shape()[1];
+    if (num_groups == 0 || C % num_groups != 0)
+        throw Error("InvalidGroups", std::to_string(C) + " channels do not split into " + std::to_string(num_groups) + " groups");
+    check_norm_operands(*this, weight, bias, C);
+    auto n = new_node(Kind::GroupNorm, shape(), dt(), device());
+    n->eps = eps;
+    n->groups = num_groups;
+    n->has_bias = bias != nullptr;
+    n->srcs = {*this, weight};
+    if (bias) n->srcs.push_back(*bias);
+    return Tensor(n);
+}
+
+Tensor Tensor::softmax(size_t dim, SoftmaxMode mode) const {
+    if (rank() < 2) throw Error("RankMismatch", "softmax input needs rank >= 2");            // Softmax::check_shapes
+    if (dim >= rank()) throw Error("DimOutOfRange", "softmax dim " + std::to_string(dim));
+    if (!is_float(dt())) throw Error("UnsupportedDType", as_str(dt()));
+    if (dim != rank() - 1) throw Error("UnsupportedSoftmaxDim", "only the last dimension is implemented (as in the reference's kernels)");
+    auto n = new_node(Kind::Softmax, shape(), dt(), device());
+    n->dim = dim;
+    n->mode = mode;
+    n->srcs = {*this};
+    return Tensor(n);
+}
+
+Tensor Tensor::slice(const std::vector<std::pair<size_t, size_t>>& ranges) const {
+    if (ranges.size() != rank()) throw Error("RankMismatch", "slice needs one range per dimension");
+    std::vector<size_t> out;
+    for (size_t i = 0; i < ranges.size(); i++) {
+        const auto& r = ranges[i];
+        if (r.first > r.second || r.second > shape()[i])                                      // Slice::check_shapes
+            throw Error("SliceOutOfBounds", "dim " + std::to_string(i) + ": " + std::to_string(r.first) + ".." + std::to_string(r.second));
+        if (r.first == r.second) throw Error("EmptySlice", "dim " + std::to_string(i));   // cpu/reindex.rs:103-105 asserts start < end
+        out.push_back(r.second - r.first);
+    }
+    auto n = new_node(Kind::Slice, Shape(out), dt(), device());
+    n->ranges = ranges;
+    n->srcs = {*this};
+    return Tensor(n);
+}
+
+Tensor Tensor::view(const Shape& shape_) const {
+    if (shape_.rank() != rank()) throw Error("RankMismatch", "view keeps the rank (View::check_shapes)");
+    if (shape_.numel() != numel()) throw Error("ShapeMismatch", "view keeps the element count");
+    auto n = new_node(Kind::View, shape_, dt(), device());
+    n->srcs = {*this};
+    n->storage = node_->storage;               // Tensor::shallow shares the storage when it already exists
+    return Tensor(n);
+}
+
+Tensor Tensor::cat(const std::vector<Tensor>& tensors, size_t dim) {
+    if (tensors.size() < 2 || tensors.size() > 8) throw Error("ConcatArity", std::to_string(tensors.size()) + " inputs (2..8 supported)");
+    const Tensor& first = tensors[0];
+    require_rank4(first.shape(), "cat");
+    if (dim >= first.rank()) throw Error("DimOutOfRange", "cat dim " + std::to_string(dim));
+    size_t stacked = 0;
+    for (const Tensor& t : tensors) {
+        require_same_device(first, t);
+        if (t.dt() != first.dt()) throw Error("DTypeMismatch", std::string("expected ") + as_str(first.dt()) + ", got " + as_str(t.dt()));
+        if (t.rank() != first.rank()) throw Error("RankMismatch", "cat inputs must have one rank");
+        for (size_t a = 0; a < first.rank(); a++)
+            if (a != dim && t.shape()[a] != first.shape()[a]) throw Error("ConcatShapeMismatch", t.shape().to_string() + " vs " + first.shape().to_string());
+        stacked += t.shape()[dim];
+    }
+    Shape out = first.shape();
+    out[dim] = stacked;
+    auto n = new_node(Kind::Concat, out, first.dt(), first.device());
+    n->dim = dim;
+    n->srcs = tensors;
+    return Tensor(n);
+}
+
+Tensor Tensor::permute(const std::vector<size_t>& dims) const {
+    if (dims.size() != rank()) throw Error("RankMismatch", "permute needs one index per dimension");    // Permute::check_shapes
+    std::vector<bool> seen(rank(), false);
+    std::vector<size_t> out(rank());
+    for (size_t i = 0; i < dims.size(); i++) {
+        if (dims[i] >= rank()) throw Error("DimOutOfRange", "permute index " + std::to_string(dims[i]));
+        if (seen[dims[i]]) throw Error("DuplicateDims", "permute indices repeat");                       // InvariantError::DuplicateDims
+        seen[dims[i]] = true;
+        out[i] = shape()[dims[i]];
+    }
+    auto n = new_node(Kind::Permute, Shape(out), dt(), device());
+    n->dims = dims;
+    n->srcs = {*this};
+    return Tensor(n);
+}
+
+Tensor Tensor::broadcast_to(const Shape& to) const {
+    require_rank4(to, "broadcast_to");
+    if (rank() > to.rank())
+        throw Error("InvalidBroadcast", "source has more dimensions than the target: " + shape().to_string() + " -> " + to.to_string());
+    for (size_t i = 0; i < rank(); i++) {                                                           // Broadcast::check_shapes
+        const size_t s = shape()[rank() - 1 - i], d = to[to.rank() - 1 - i];
+        if (s != 1 && s != d) throw Error("InvalidBroadcast", std::to_string(s) + " cannot be broadcast to " + std::to_string(d));
+    }
+    auto n = new_node(Kind::Broadcast, to, dt(), device());
+    n->srcs = {*this};
+    return Tensor(n);
+}
+
+// ------------------------------------------------------------------------------------------------------------ resolve
+static void shape4(const Shape& s, uint32_t out[4]) {
+    const Shape p = Shape::promote(s, 4);
+    for (int i = 0; i < 4; i++) out[i] = (uint32_t)p[i];
+}
+
+// iterative post-order DFS over srcs, sources that have sources of their own first (tensor.rs:696-740)
+static std::vector<Node*> execution_order(Node* root) {
+    std::unordered_set<uint64_t> done, pending;
+    std::vector<Node*> order;
+    std::vector<std::pair<Node*, size_t>> stack{{root, 0}};
+    while (!stack.empty()) {
+        auto [cur, idx] = stack.back();
+        stack.pop_back();
+        if (idx == cur->srcs.size()) {
+            done.insert(cur->id);
+            pending.erase(cur->id);
+            order.push_back(cur);
+            continue;
+        }
+        std::vector<Node*> all;
+        for (const Tensor& s : cur->srcs)
+            if (!Node::of(s)->srcs.empty()) all.push_back(Node::of(s));
+        for (const Tensor& s : cur->srcs)
+            if (Node::of(s)->srcs.empty()) all.push_back(Node::of(s));
+        Node* pre = all[idx];
+        if (done.count(pre->id)) {
+            stack.push_back({cur, idx + 1});
+        } else if (pending.count(pre->id)) {
+            throw Error("CycleDetected", "cycle through tensor " + std::to_string(pre->id));
+        } else {
+            pending.insert(pre->id);
+            stack.push_back({cur, idx});
+            stack.push_back({pre, 0});
+        }
+    }
+    return order;
+}
+
+std::vector<uint64_t> Tensor::execution_order_ids() const {
+    std::vector<uint64_t> ids;
+    for (Node* n : execution_order(node_.get())) ids.push_back(n->id);
+    return ids;
+}
+
+struct Resolver {
+    // a Broadcast node nobody else holds, not yet materialised, feeding a Binary: fused into the binary kernel
+    static bool fusable_broadcast(const Tensor& operand) {
+        Node* b = Node::of(operand);
+        return b->kind == Kind::Broadcast && !b->storage && Node::holders(operand) == 1;
+    }
+
+    static void run(Node* n, size_t& launches) {
+        rt_device* dev = n->device.raw();
+        const int dt = (int)n->dt;
+        auto src = [&](size_t i) -> Node* { return Node::of(n->srcs[i]); };
+        auto out_buffer = [&]() { n->storage = std::make_shared<Buffer>(n->device, n->shape.numel() * size_of(n->dt)); };
+        // tensor.rs:823-824: supports_inplace() && Arc::strong_count(srcs[0]) == 1 (and here: nobody else shares the buffer)
+        auto take_src0_if_unshared = [&]() {
+            Node* s0 = src(0);
+            if (Node::holders(n->srcs[0]) == 1 && s0->storage.use_count() == 1 && s0->shape == n->shape && s0->dt == n->dt) {
+                n->storage = s0->storage;
+                return true;
+            }
+            return false;
+        };
+        switch (n->kind) {
+            case Kind::Const: throw Error("Unresolved", "constant tensor " + std::to_string(n->id) + " has no storage (placeholder)");
+            case Kind::View: n->storage = src(0)->storage; return;
+            case Kind::Binary: {
+                const bool fa = fusable_broadcast(n->srcs[0]), fb = fusable_broadcast(n->srcs[1]);
+                Node* a = fa ? Node::of(src(0)->srcs[0]) : src(0);
+                Node* b = fb ? Node::of(src(1)->srcs[0]) : src(1);
+                if (fa || fb) {
+                    uint32_t as[4], bs[4], ys[4];
+                    shape4(a->shape, as);
+                    shape4(b->shape, bs);
+                    shape4(n->shape, ys);
+                    out_buffer();
+                    check_rt(rt_binary_bcast(dev, (int)n->bop, dt, a->storage->ptr, as, b->storage->ptr, bs, n->storage->ptr, ys), "rt_binary_bcast");
+                } else {
+                    if (!take_src0_if_unshared()) out_buffer();
+                    check_rt(rt_binary(dev, (int)n->bop, dt, a->storage->ptr, b->storage->ptr, n->storage->ptr, n->shape.numel()), "rt_binary");
+                }
+                launches++;
+                return;
+            }
+            case Kind::Unary:
+                if (!take_src0_if_unshared()) out_buffer();
+                check_rt(rt_unary(dev, (int)n->uop, dt, src(0)->storage->ptr, n->storage->ptr, n->shape.numel()), "rt_unary");
+                launches++;
+                return;
+            case Kind::Softmax: {
+                if (!take_src0_if_unshared()) out_buffer();
+                const size_t cols = n->shape[n->shape.rank() - 1];
+                check_rt(rt_softmax(dev, dt, src(0)->storage->ptr, n->storage->ptr, n->shape.numel() / cols, (uint32_t)cols, (int)n->mode),
+                         "rt_softmax");
+                launches++;
+                return;
+            }
+            case Kind::Cast:
+                out_buffer();                                  // Cast::supports_inplace() is false (ops/cast.rs:128-131)
+                check_rt(rt_cast(dev, (int)src(0)->dt, dt, src(0)->storage->ptr, n->storage->ptr, n->shape.numel()), "rt_cast");
+                launches++;
+                return;
+            case Kind::Permute: {
+                uint32_t ss[4], perm[4];
+                shape4(src(0)->shape, ss);
+                const size_t pad = 4 - n->dims.size();         // Permute::promote (ops/reindex/permute.rs:29-38)
+                for (size_t i = 0; i < pad; i++) perm[i] = (uint32_t)i;
+                for (size_t i = 0; i < n->dims.size(); i++) perm[pad + i] = (uint32_t)(n->dims[i] + pad);
+                out_buffer();
+                check_rt(rt_permute(dev, (int)size_of(n->dt), src(0)->storage->ptr, n->storage->ptr, ss, perm), "rt_permute");
+                launches++;
+                return;
+            }
+            case Kind::Slice: {
+                uint32_t ss[4], st[4] = {0, 0, 0, 0}, ds[4];
+                shape4(src(0)->shape, ss);
+                shape4(n->shape, ds);
+                const size_t pad = 4 - n->ranges.size();
+                for (size_t i = 0; i < n->ranges.size(); i++) st[pad + i] = (uint32_t)n->ranges[i].first;
+                out_buffer();
+                check_rt(rt_slice(dev, (int)size_of(n->dt), src(0)->storage->ptr, n->storage->ptr, ss, st, ds), "rt_slice");
+                launches++;
+                return;
+            }
+            case Kind::Broadcast: {
+                uint32_t ss[4], ds[4];
+                shape4(src(0)->shape, ss);
+                shape4(n->shape, ds);
+                out_buffer();
+                check_rt(rt_broadcast(dev, (int)size_of(n->dt), src(0)->storage->ptr, n->storage->ptr, ss, ds), "rt_broadcast");
+                launches++;
+                return;
+            }
+            case Kind::Concat: {
+                const void* ptrs[8];
+                uint32_t shapes[8][4];
+                for (size_t i = 0; i < n->srcs.size(); i++) {
+                    ptrs[i] = src(i)->storage->ptr;
+                    shape4(src(i)->shape, shapes[i]);
+                }
+                out_buffer();
+                check_rt(rt_concat(dev, (int)size_of(n->dt), (int)n->srcs.size(), ptrs, shapes, (int)(n->dim + 4 - n->shape.rank()), n->storage->ptr),
+                         "rt_concat");
+                launches++;
+                return;
+            }
+            case Kind::LayerNorm:
+            case Kind::RMSNorm: {
+                const size_t cols = n->shape[n->shape.rank() - 1];
+                out_buffer();
+                if (n->kind == Kind::LayerNorm)
+                    check_rt(rt_layer_norm(dev, dt, src(0)->storage->ptr, src(1)->storage->ptr, n->has_bias ? src(2)->storage->ptr : nullptr,
+                                           n->storage->ptr, n->shape.numel() / cols, (uint32_t)cols, n->eps),
+                             "rt_layer_norm");
+                else
+                    check_rt(rt_rms_norm(dev, dt, src(0)->storage->ptr, src(1)->storage->ptr, n->storage->ptr, n->shape.numel() / cols,
+                                         (uint32_t)cols, n->eps),
+                             "rt_rms_norm");
+                launches++;
+                return;
+            }
+            case Kind::GroupNorm: {
+                const size_t B = n->shape[0], C = n->shape[1];
+                out_buffer();
+                check_rt(rt_group_norm(dev, dt, src(0)->storage->ptr, src(1)->storage->ptr, n->has_bias ? src(2)->storage->ptr : nullptr,
+                                       n->storage->ptr, (uint32_t)B, (uint32_t)C, (uint32_t)(n->shape.numel() / (B * C)), (uint32_t)n->groups, n->eps),
+                         "rt_group_norm");
+                launches++;
+                return;
+            }
+        }
+    }
+
+    static void resolve(Node* root) {
+        size_t launches = 0;
+        const std::vector<Node*> order = execution_order(root);
+        // broadcasts that their (single) binary consumer will absorb are not materialised
+        std::unordered_set<Node*> skip;
+        for (Node* n : order)
+            if (n->kind == Kind::Binary && !n->storage)
+                for (const Tensor& s : n->srcs)
+                    if (fusable_broadcast(s)) skip.insert(Node::of(s));
+        for (Node* n : order) {
+            if (n->storage || skip.count(n)) continue;         // already resolved (tensor.rs:783) or fused away
+            run(n, launches);
+        }
+        check_rt(rt_sync(root->device.raw()), "rt_sync");      // resolve returns after completion (tensor.rs:855-856)
+        root->last_launches = launches;
+    }
+};
+
+Tensor Tensor::resolve() const {
+    if (!node_) throw Error("NullTensor", "resolve on an empty tensor");
+    Resolver::resolve(node_.get());
+    return *this;
+}
+
+void Tensor::to_host(void* out) const {
+    if (!resolved()) throw Error("Unresolved", "to_host needs a resolved tensor (call resolve() first)");
+    check_rt(rt_d2h(node_->device.raw(), out, node_->storage->ptr, numel() * size_of(dt())), "rt_d2h");
+}
+
+}  // namespace ratchet

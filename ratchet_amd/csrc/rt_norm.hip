@@ -239,13 +239,15 @@ __global__ void __launch_bounds__(BLOCK) norm_seq16_kernel(const T* __restrict__
 }
 
 // Pipelined form of the kernel above for the common case (cols % 8 == 0, 16-byte aligned operands).
-// 8 rows per block, 256-column tiles, one 16-byte vector per thread per tile.  Global loads run two tiles ahead of the
-// LDS stage, LDS tiles are double buffered and there is one barrier per tile, so the lanes that walk (8 for RMSNorm, 16
-// for LayerNorm, all in wave 0) never wait for memory: the kernel runs at the speed of the dependent v_add_f32 chain.
+// 8 rows per 320-thread block, 256-column tiles.  Wave 0 does nothing but walk (8 lanes for RMSNorm, 16 for LayerNorm)
+// and raises its issue priority; the four loader waves fetch one 16-byte vector per thread per tile two tiles ahead,
+// widen x and T(x*x) to f32 and park them in double-buffered LDS tiles; one barrier per tile.  The kernel runs at the
+// speed of the dependent v_add_f32 chain (about 3 ns per column on this chip).
+constexpr int NP_BLOCK = 320;
 template <typename T, int KIND>
-__global__ void __launch_bounds__(BLOCK) norm_pipe16_kernel(const T* __restrict__ x, const T* __restrict__ scale,
-                                                            const T* __restrict__ bias, T* __restrict__ y, uint64_t rows, uint32_t cols,
-                                                            float eps) {
+__global__ void __launch_bounds__(NP_BLOCK) norm_pipe16_kernel(const T* __restrict__ x, const T* __restrict__ scale,
+                                                               const T* __restrict__ bias, T* __restrict__ y, uint64_t rows, uint32_t cols,
+                                                               float eps) {
     constexpr int RB = 8, TC = 256, PAD = 4;
     constexpr int NSUM = (KIND == NORM_LAYER) ? 2 : 1;
     __shared__ __attribute__((aligned(16))) float tile[2][NSUM][RB][TC + PAD];   // [.][0] = squares, [.][1] = values
@@ -253,13 +255,54 @@ __global__ void __launch_bounds__(BLOCK) norm_pipe16_kernel(const T* __restrict_
     __shared__ T s_mu[RB], s_r[RB];
     const uint64_t row0 = (uint64_t)blockIdx.x * RB;
     const uint32_t nrows = (rows - row0 < (uint64_t)RB) ? (uint32_t)(rows - row0) : (uint32_t)RB;
-    const uint32_t r = threadIdx.x >> 5, cv = threadIdx.x & 31;                 // loader role: row, vector within the tile
+    const uint32_t ntiles = (cols + TC - 1) / TC;
+
+    if (threadIdx.x < 64) {
+        // ---------------------------------------------------------------- wave 0: the sequential sums
+        __builtin_amdgcn_s_setprio(3);
+        const uint32_t wrow = threadIdx.x % RB, wsum = (threadIdx.x / RB) % NSUM;   // lanes beyond NSUM*RB shadow and never publish
+        const bool publish = (threadIdx.x < NSUM * RB) && (wrow < nrows);
+        float run = 0.0f;
+        for (uint32_t t = 0; t < ntiles; t++) {
+            __syncthreads();                                                    // tile t is in LDS
+            // fixed trip count (tiles are zero padded): LDS reads of the next 32 values are issued before the 32 dependent
+            // adds of the current ones
+            const float4* trow = reinterpret_cast<const float4*>(tile[t & 1][wsum][wrow]);
+            float4 cur[8], nxt[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) cur[k] = trow[k];
+#pragma unroll
+            for (int c = 0; c < TC / 32; c++) {
+                if (c + 1 < TC / 32) {
+#pragma unroll
+                    for (int k = 0; k < 8; k++) nxt[k] = trow[(c + 1) * 8 + k];
+                }
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    run += cur[k].x; run += cur[k].y; run += cur[k].z; run += cur[k].w;
+                }
+#pragma unroll
+                for (int k = 0; k < 8; k++) cur[k] = nxt[k];
+            }
+        }
+        if (publish) sums[wsum][wrow] = run;
+        __builtin_amdgcn_s_setprio(0);
+        __syncthreads();                                                        // sums published
+        if (threadIdx.x < nrows) {
+            const RowStats<T> st = finish_stats<T, KIND>(KIND == NORM_LAYER ? sums[NSUM - 1][threadIdx.x] : 0.0f, sums[0][threadIdx.x],
+                                                         cols, eps);
+            s_mu[threadIdx.x] = st.mu;
+            s_r[threadIdx.x] = st.r;
+        }
+        __syncthreads();                                                        // row statistics published
+        return;
+    }
+
+    // -------------------------------------------------------------------- waves 1..4: loads, widening, second pass
+    const uint32_t lt = threadIdx.x - 64;
+    const uint32_t r = lt >> 5, cv = lt & 31;                                   // row, vector within the tile
     const bool rvalid = r < nrows;
     const T* xrow = x + (row0 + (rvalid ? r : 0)) * cols;
-    const uint32_t wrow = threadIdx.x % RB, wsum = threadIdx.x / RB;            // walker role
-    const bool walker = (threadIdx.x < NSUM * RB) && (wrow < nrows);
-    const uint32_t ntiles = (cols + TC - 1) / TC;
-    float run = 0.0f;
     v4u pre0 = {0, 0, 0, 0}, pre1 = {0, 0, 0, 0};
 
     auto issue = [&](uint32_t t, v4u& dst) {
@@ -295,26 +338,6 @@ __global__ void __launch_bounds__(BLOCK) norm_pipe16_kernel(const T* __restrict_
         }
         issue(t + 2, reg);
         __syncthreads();
-        if (walker) {
-            // fixed trip count: LDS reads of the next 32 values are issued before the 32 dependent adds of the current ones
-            const float4* trow = reinterpret_cast<const float4*>(tile[buf][wsum][wrow]);
-            float4 cur[8], nxt[8];
-#pragma unroll
-            for (int k = 0; k < 8; k++) cur[k] = trow[k];
-#pragma unroll
-            for (int c = 0; c < TC / 32; c++) {
-                if (c + 1 < TC / 32) {
-#pragma unroll
-                    for (int k = 0; k < 8; k++) nxt[k] = trow[(c + 1) * 8 + k];
-                }
-#pragma unroll
-                for (int k = 0; k < 8; k++) {
-                    run += cur[k].x; run += cur[k].y; run += cur[k].z; run += cur[k].w;
-                }
-#pragma unroll
-                for (int k = 0; k < 8; k++) cur[k] = nxt[k];
-            }
-        }
     };
 
     issue(0, pre0);
@@ -323,15 +346,8 @@ __global__ void __launch_bounds__(BLOCK) norm_pipe16_kernel(const T* __restrict_
         step(t, pre0);
         if (t + 1 < ntiles) step(t + 1, pre1);
     }
-    if (walker) sums[wsum][wrow] = run;
-    __syncthreads();
-    if (threadIdx.x < nrows) {
-        const RowStats<T> st = finish_stats<T, KIND>(KIND == NORM_LAYER ? sums[NSUM - 1][threadIdx.x] : 0.0f, sums[0][threadIdx.x],
-                                                     cols, eps);
-        s_mu[threadIdx.x] = st.mu;
-        s_r[threadIdx.x] = st.r;
-    }
-    __syncthreads();
+    __syncthreads();                                                            // sums published (wave 0 finishes the stats)
+    __syncthreads();                                                            // row statistics published
     if (!rvalid) return;
     RowStats<T> st;
     st.mu = s_mu[r];
@@ -356,7 +372,8 @@ __global__ void __launch_bounds__(BLOCK) norm_pipe16_kernel(const T* __restrict_
 // apply kernel: same grid; every block combines the group's partials (Chan et al.), then normalises its slice:
 //               y = (x - mean) * rstd * w[c] + b[c], f32 arithmetic, rounded to T once.
 // ------------------------------------------------------------------------------------------------------------------
-template <typename T>
+// VE = elements per access: 16 / sizeof(T) on the vector path (slices, L and base pointers are multiples of it), 1 otherwise
+template <typename T, int VE>
 __global__ void __launch_bounds__(BLOCK) gn_stats_kernel(const T* __restrict__ x, float* __restrict__ part, uint32_t glen,
                                                          uint32_t chunk, uint32_t splits) {
     __shared__ float red[WAVES];
@@ -367,7 +384,16 @@ __global__ void __launch_bounds__(BLOCK) gn_stats_kernel(const T* __restrict__ x
     const uint32_t c1 = (c0 + chunk < glen) ? c0 + chunk : glen;
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
     float acc = 0.0f;
-    for (uint32_t i = c0 + threadIdx.x; i < c1; i += BLOCK) acc += Ar<T>::widen(xs[i]);
+    for (uint32_t i = c0 + threadIdx.x * VE; i < c1; i += BLOCK * VE) {
+        if (VE > 1) {
+            Vec16<T> v;
+            v.u = *reinterpret_cast<const uint4*>(xs + i);
+#pragma unroll
+            for (int q = 0; q < VE; q++) acc += Ar<T>::widen(v.e[q]);
+        } else {
+            acc += Ar<T>::widen(xs[i]);
+        }
+    }
     acc = wave_sum(acc);
     if (lane == 0) red[wave] = acc;
     __syncthreads();
@@ -379,9 +405,19 @@ __global__ void __launch_bounds__(BLOCK) gn_stats_kernel(const T* __restrict__ x
     __syncthreads();
     const float mean = bc;
     float m2 = 0.0f;
-    for (uint32_t i = c0 + threadIdx.x; i < c1; i += BLOCK) {
-        const float d = Ar<T>::widen(xs[i]) - mean;
-        m2 += d * d;
+    for (uint32_t i = c0 + threadIdx.x * VE; i < c1; i += BLOCK * VE) {     // second pass: the slice is in cache
+        if (VE > 1) {
+            Vec16<T> v;
+            v.u = *reinterpret_cast<const uint4*>(xs + i);
+#pragma unroll
+            for (int q = 0; q < VE; q++) {
+                const float d = Ar<T>::widen(v.e[q]) - mean;
+                m2 += d * d;
+            }
+        } else {
+            const float d = Ar<T>::widen(xs[i]) - mean;
+            m2 += d * d;
+        }
     }
     m2 = wave_sum(m2);
     __syncthreads();
@@ -397,36 +433,52 @@ __global__ void __launch_bounds__(BLOCK) gn_stats_kernel(const T* __restrict__ x
     }
 }
 
-template <typename T>
+template <typename T, int VE>
 __global__ void __launch_bounds__(BLOCK) gn_apply_kernel(const T* __restrict__ x, const T* __restrict__ scale,
                                                          const T* __restrict__ bias, T* __restrict__ y,
                                                          const float* __restrict__ part, uint32_t glen, uint32_t chunk, uint32_t splits,
                                                          uint32_t cpg, uint32_t groups, FastDiv L, float eps) {
+    __shared__ float s_mean, s_rstd;
     const uint32_t s = blockIdx.y, grp = blockIdx.x;
-    // every thread combines the (few) partials itself: no shared memory, no barrier
-    double n = 0.0, mean = 0.0, m2 = 0.0;
-    const float* p = part + (uint64_t)grp * splits * 3;
-    for (uint32_t k = 0; k < splits; k++) {
-        const double nb = (double)p[3 * k + 2], mb = (double)p[3 * k], m2b = (double)p[3 * k + 1];
-        const double nt = n + nb;
-        const double delta = mb - mean;
-        mean += delta * (nb / nt);
-        m2 += m2b + delta * delta * (n * nb / nt);
-        n = nt;
+    if (threadIdx.x == 0) {
+        // combine the group's partials (Chan et al.) in double
+        double n = 0.0, mean = 0.0, m2 = 0.0;
+        const float* p = part + (uint64_t)grp * splits * 3;
+        for (uint32_t k = 0; k < splits; k++) {
+            const double nb = (double)p[3 * k + 2], mb = (double)p[3 * k], m2b = (double)p[3 * k + 1];
+            const double nt = n + nb;
+            const double delta = mb - mean;
+            mean += delta * (nb / nt);
+            m2 += m2b + delta * delta * (n * nb / nt);
+            n = nt;
+        }
+        s_mean = (float)mean;
+        s_rstd = (float)(1.0 / sqrt(m2 / n + (double)eps));
     }
-    const float meanf = (float)mean;
-    const float rstd = (float)(1.0 / sqrt(m2 / n + (double)eps));
+    __syncthreads();
+    const float meanf = s_mean, rstd = s_rstd;
     const uint32_t g = grp % groups;
     const T* xs = x + (uint64_t)grp * glen;
     T* ys = y + (uint64_t)grp * glen;
     const uint32_t c0 = s * chunk;
     const uint32_t c1 = (c0 + chunk < glen) ? c0 + chunk : glen;
-    for (uint32_t i = c0 + threadIdx.x; i < c1; i += BLOCK) {
-        const uint32_t c = g * cpg + fd_div(i, L);
+    for (uint32_t i = c0 + threadIdx.x * VE; i < c1; i += BLOCK * VE) {
+        const uint32_t c = g * cpg + fd_div(i, L);                            // with VE > 1, L % VE == 0: one channel per vector
         const float w = scale ? Ar<T>::widen(scale[c]) : 1.0f;
         const float b = bias ? Ar<T>::widen(bias[c]) : 0.0f;
-        const float v = (Ar<T>::widen(xs[i]) - meanf) * rstd;
-        ys[i] = Ar<T>::conv(v * w + b);
+        if (VE > 1) {
+            Vec16<T> v, o;
+            v.u = *reinterpret_cast<const uint4*>(xs + i);
+#pragma unroll
+            for (int q = 0; q < VE; q++) {
+                const float t = (Ar<T>::widen(v.e[q]) - meanf) * rstd;
+                o.e[q] = Ar<T>::conv(t * w + b);
+            }
+            *reinterpret_cast<uint4*>(ys + i) = o.u;
+        } else {
+            const float t = (Ar<T>::widen(xs[i]) - meanf) * rstd;
+            ys[i] = Ar<T>::conv(t * w + b);
+        }
     }
 }
 
@@ -484,7 +536,7 @@ int launch_norm16(rt_device* dev, const void* x, const void* scale, const void* 
     if (vec_ok) {
         const uint64_t blocks = (rows + 7) / 8;
         RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
-        hipLaunchKernelGGL((norm_pipe16_kernel<T, KIND>), dim3((unsigned)blocks), dim3(BLOCK), 0, dev->stream, (const T*)x, (const T*)scale,
+        hipLaunchKernelGGL((norm_pipe16_kernel<T, KIND>), dim3((unsigned)blocks), dim3(NP_BLOCK), 0, dev->stream, (const T*)x, (const T*)scale,
                            (const T*)bias, (T*)y, rows, cols, eps);
         RT_CHECK_LAUNCH("norm_pipe16_kernel");
         return RT_OK;
@@ -531,7 +583,10 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
     if (splits > max_splits) splits = max_splits;
     if (splits > 64) splits = 64;
     if (splits < 1) splits = 1;
-    const uint32_t chunk = (glen + splits - 1) / splits;
+    constexpr int VEMAX = 16 / sizeof(T);
+    const bool vec = (L % VEMAX == 0) && rt_aligned(x, 16) && rt_aligned(y, 16);       // then glen % VEMAX == 0 too
+    uint32_t chunk = (glen + splits - 1) / splits;
+    if (vec) chunk = (chunk + VEMAX - 1) / VEMAX * VEMAX;                               // slices start on vector boundaries
     splits = (glen + chunk - 1) / chunk;
     const size_t need = (size_t)bg * splits * 3 * sizeof(float);
     if (need > dev->gn_scratch_bytes) {
@@ -543,10 +598,17 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
         dev->gn_scratch_bytes = need;
     }
     const dim3 grid(bg, splits), block(BLOCK);
-    hipLaunchKernelGGL((gn_stats_kernel<T>), grid, block, 0, dev->stream, (const T*)x, dev->gn_scratch, glen, chunk, splits);
-    RT_CHECK_LAUNCH("gn_stats_kernel");
-    hipLaunchKernelGGL((gn_apply_kernel<T>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, (T*)y,
-                       (const float*)dev->gn_scratch, glen, chunk, splits, cpg, groups, make_fastdiv(L), eps);
+    if (vec) {
+        hipLaunchKernelGGL((gn_stats_kernel<T, VEMAX>), grid, block, 0, dev->stream, (const T*)x, dev->gn_scratch, glen, chunk, splits);
+        RT_CHECK_LAUNCH("gn_stats_kernel");
+        hipLaunchKernelGGL((gn_apply_kernel<T, VEMAX>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, (T*)y,
+                           (const float*)dev->gn_scratch, glen, chunk, splits, cpg, groups, make_fastdiv(L), eps);
+    } else {
+        hipLaunchKernelGGL((gn_stats_kernel<T, 1>), grid, block, 0, dev->stream, (const T*)x, dev->gn_scratch, glen, chunk, splits);
+        RT_CHECK_LAUNCH("gn_stats_kernel");
+        hipLaunchKernelGGL((gn_apply_kernel<T, 1>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, (T*)y,
+                           (const float*)dev->gn_scratch, glen, chunk, splits, cpg, groups, make_fastdiv(L), eps);
+    }
     RT_CHECK_LAUNCH("gn_apply_kernel");
     return RT_OK;
 }

@@ -83,13 +83,17 @@ __global__ void __launch_bounds__(BLOCK) softmax_wave_kernel(const T* __restrict
                     s += e[k][q];
                 }
         s = wave_sum(s);
+        // e / s as e * (1/s): one correctly rounded reciprocal per row, at most 1 ulp from the quotient (bar: 1e-5).
+        // A zero, subnormal, inf or NaN sum keeps the division so that 0/0, x/inf and inf/inf come out as the reference's do.
+        const bool plain = (s >= 1.17549435e-38f) && (s < __builtin_huge_valf());
+        const float rs = 1.0f / s;
 #pragma unroll
         for (int k = 0; k < NV; k++) {
             const uint32_t i = lane + k * WAVE;
             if (i < nvec) {
                 Vec16<T> o;
 #pragma unroll
-                for (int q = 0; q < VE; q++) o.e[q] = Ar<T>::conv(e[k][q] / s);
+                for (int q = 0; q < VE; q++) o.e[q] = Ar<T>::conv(plain ? e[k][q] * rs : e[k][q] / s);
                 yr[i] = o.u;
             }
         }

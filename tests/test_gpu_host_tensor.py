@@ -1,0 +1,190 @@
+"""GPU tests through the C++ host mirror of ratchet's Tensor API: the reference's own per-op trials (same problem spaces,
+torch as referee, the reference's tolerances) plus graph-level behaviour (multi-op graphs, the in-place rule, fused
+broadcasts) checked against the CPU oracle.
+
+Reference trials mirrored: ops/binary.rs:275-334, ops/unary.rs:365-461, ops/softmax.rs:308-365, ops/norm/mod.rs:400-512,
+ops/norm/groupnorm.rs:11-87, ops/cast.rs:217-282, ops/concat.rs:273-359, ops/reindex/{permute,slice,broadcast}.rs tests,
+and the multi-op attention graph of crates/ratchet-core/tests/attn_tests.rs (without its matmuls).
+"""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from gpu_util import same_bits
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hdev():
+    from ratchet_amd.host import HostDevice
+
+    d = HostDevice(0)
+    yield d
+    d.close()
+
+
+def T(a, dev):
+    from ratchet_amd.host import Tensor
+
+    return Tensor.from_numpy(a, dev)
+
+
+def close(oracle, got, want, tol):
+    bad, mx = oracle.count_not_close(np.ascontiguousarray(got), np.ascontiguousarray(want), tol, tol)
+    return bad == 0, (bad, mx)
+
+
+def test_binary_trials(hdev, oracle):
+    rng = np.random.default_rng(400)
+    for _ in range(8):
+        shape = (int(rng.integers(1, 5)), int(rng.integers(1, 5)), 1, int(rng.integers(1, 257)))
+        a, b = rng.standard_normal(shape).astype(np.float32), rng.standard_normal(shape).astype(np.float32)
+        for name, tf in (("add", torch.add), ("sub", torch.sub), ("mul", torch.mul), ("div", torch.div)):
+            got = getattr(T(a, hdev), name)(T(b, hdev)).resolve().to_numpy()
+            ok, info = close(oracle, got, tf(torch.from_numpy(a), torch.from_numpy(b)).numpy(), 1e-4)
+            assert ok, (name, shape, info)
+            assert same_bits(got, oracle.binary(name, a, b))
+
+
+def test_unary_trials(hdev, oracle):
+    rng = np.random.default_rng(401)
+    tf = {"gelu": lambda t: F.gelu(t, approximate="tanh"), "tanh": torch.tanh, "exp": torch.exp, "log": torch.log, "sin": torch.sin,
+          "cos": torch.cos, "abs": torch.abs, "sqrt": torch.sqrt, "relu": torch.relu, "floor": torch.floor, "ceil": torch.ceil,
+          "neg": torch.neg, "silu": F.silu, "sigmoid": torch.sigmoid}
+    for name, fn in tf.items():
+        x = rng.standard_normal((int(rng.integers(1, 3)), int(rng.integers(1, 129)))).astype(np.float32)
+        got = getattr(T(x, hdev), name)().resolve().to_numpy()
+        with np.errstate(all="ignore"):
+            want = fn(torch.from_numpy(x)).numpy()
+        tol = 5e-2 if name in ("gelu", "tanh") else 1e-4
+        ok, info = close(oracle, got, want, tol)
+        assert ok, (name, info)
+
+
+def test_softmax_norm_groupnorm_trials(hdev, oracle):
+    rng = np.random.default_rng(402)
+    for _ in range(6):
+        shape = (int(rng.integers(1, 4)), int(rng.integers(1, 257)), int(rng.integers(1, 257)))
+        x = rng.standard_normal(shape).astype(np.float32)
+        n = shape[-1]
+        got = T(x, hdev).softmax(2).resolve().to_numpy()
+        ok, info = close(oracle, got, F.softmax(torch.from_numpy(x), dim=-1).numpy(), 1e-6)
+        assert ok, ("softmax", shape, info)
+        w, b = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+        got = T(x, hdev).layer_norm(T(w, hdev), T(b, hdev), 1e-5).resolve().to_numpy()
+        want = F.layer_norm(torch.from_numpy(x), (n,), torch.from_numpy(w), torch.from_numpy(b), eps=1e-5).numpy()
+        ok, info = close(oracle, got, want, 1e-4)
+        assert ok, ("layer_norm", shape, info)
+        t = torch.from_numpy(x)
+        want = (t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + 1e-5) * torch.from_numpy(w)).numpy()
+        got = T(x, hdev).rms_norm(T(w, hdev), 1e-5).resolve().to_numpy()
+        ok, info = close(oracle, got, want, 1e-4)
+        assert ok, ("rms_norm", shape, info)
+    for B, C, L, G in ((1, 3, 1, 1), (2, 8, 5, 4), (1, 64, 40, 32)):
+        x = rng.standard_normal((B, C, L)).astype(np.float32)
+        w, b = rng.standard_normal(C).astype(np.float32), rng.standard_normal(C).astype(np.float32)
+        got = T(x, hdev).group_norm(G, T(w, hdev), T(b, hdev), 1e-5).resolve().to_numpy()
+        want = F.group_norm(torch.from_numpy(x), G, torch.from_numpy(w), torch.from_numpy(b), eps=1e-5).numpy()
+        ok, info = close(oracle, got, want, 1e-4)
+        assert ok, ("group_norm", (B, C, L, G), info)
+
+
+def test_cast_and_reindex_trials(hdev, oracle):
+    from ratchet_amd import _lib
+    from ratchet_amd.host import Tensor
+
+    rng = np.random.default_rng(403)
+    x = rng.standard_normal((2, 100, 77)).astype(np.float32)
+    h = T(x, hdev).cast(_lib.F16).resolve().to_numpy()
+    assert same_bits(h, x.astype(np.float16))
+    assert np.array_equal(T(x, hdev).cast(_lib.I32).resolve().to_numpy(), x.view(np.int32))
+    assert same_bits(T(h, hdev).full().resolve().to_numpy(), h.astype(np.float32))
+    xs = [rng.standard_normal((4, 2, k, 128)).astype(np.float32) for k in (50, 13, 77, 55, 11)]
+    got = Tensor.cat([T(a, hdev) for a in xs], 2).resolve().to_numpy()
+    assert np.array_equal(got, np.concatenate(xs, axis=2))
+    for _ in range(8):
+        shape = (int(rng.integers(1, 3)), int(rng.integers(1, 5)), int(rng.integers(1, 257)), int(rng.integers(1, 257)))
+        perm = [int(p) for p in rng.permutation(4)]
+        a = rng.standard_normal(shape).astype(np.float32)
+        assert np.array_equal(T(a, hdev).permute(perm).resolve().to_numpy(), np.ascontiguousarray(a.transpose(perm))), (shape, perm)
+    for _ in range(8):
+        shape = [int(rng.integers(2, 17)) for _ in range(3)] + [int(rng.integers(2, 129))]
+        a = rng.standard_normal(shape).astype(np.float32)
+        ranges = []
+        for s in shape:
+            lo = int(rng.integers(0, s))
+            ranges.append((lo, int(rng.integers(lo + 1, s + 1))))
+        want = a[tuple(slice(lo, hi) for lo, hi in ranges)]
+        assert np.array_equal(T(a, hdev).slice(ranges).resolve().to_numpy(), want), (shape, ranges)
+    for _ in range(8):
+        src = [int(rng.integers(1, 3)), int(rng.integers(1, 9)), int(rng.integers(1, 3)), int(rng.integers(1, 129))]
+        dst = [s if s != 1 else int(rng.integers(1, 9)) for s in src]
+        a = rng.standard_normal(src).astype(np.float32)
+        assert np.array_equal(T(a, hdev).broadcast_to(dst).resolve().to_numpy(), np.broadcast_to(a, dst)), (src, dst)
+    one = np.array([3.5], np.float32)                                 # the reference's debug case [1] -> [4,32,128,128]
+    assert np.all(T(one, hdev).broadcast_to((4, 32, 128, 128)).resolve().to_numpy() == 3.5)
+    v = rng.standard_normal((2, 6)).astype(np.float32)
+    assert np.array_equal(T(v, hdev).view((3, 4)).gelu().resolve().to_numpy(), oracle.unary("gelu", v.reshape(3, 4)))
+
+
+def test_whisper_bias_gelu_layer_norm_graph(hdev, oracle):
+    # BASELINE config 0 as ONE lazy graph: bias add (broadcast fused) -> tanh GELU -> LayerNorm, f32
+    rng = np.random.default_rng(404)
+    x = rng.standard_normal((1, 1500, 384)).astype(np.float32)
+    bias = (0.02 * rng.standard_normal(384)).astype(np.float32)
+    g = (1 + 0.02 * rng.standard_normal(384)).astype(np.float32)
+    b = (0.02 * rng.standard_normal(384)).astype(np.float32)
+    y = T(x, hdev).add(T(bias, hdev)).gelu().layer_norm(T(g, hdev), T(b, hdev), 1e-5).resolve()
+    # three kernels: the Broadcast node is absorbed by the add, GELU runs in place on the add's buffer
+    assert y.last_resolve_launches() == 3
+    h = oracle.unary("gelu", oracle.binary("add", x, np.ascontiguousarray(np.broadcast_to(bias, x.shape))))
+    want = oracle.layer_norm(h, g, b, 1e-5)
+    ok, info = close(oracle, y.to_numpy(), want, 1e-5)
+    assert ok, info
+
+
+def test_phi3_style_attention_tail_graph(hdev, oracle):
+    # scores.add(mask) -> full -> softmax(3) -> cast(f16), the pattern of models/phi3/attn.rs:148-153, and SwiGLU
+    # up.mul(gate.full().silu().cast(f16)) of models/phi3/mlp.rs:37, in f16 with an f32 mask broadcast over heads
+    from ratchet_amd import _lib
+
+    rng = np.random.default_rng(405)
+    S, H = 128, 4
+    scores = (2 * rng.standard_normal((1, H, S, S))).astype(np.float32)
+    mask = np.triu(np.full((S, S), -np.inf, np.float32), k=1)
+    y = T(scores, hdev).add(T(mask, hdev)).softmax(3).cast(_lib.F16).resolve()
+    want = oracle.cast(oracle.softmax(oracle.binary("add", scores, np.ascontiguousarray(np.broadcast_to(mask, scores.shape)))),
+                       np.float16)
+    ok, info = close(oracle, y.to_numpy(), want, 1e-3)
+    assert ok, info
+    assert y.last_resolve_launches() == 3
+    gate = rng.standard_normal((1, 64, 512)).astype(np.float16)
+    up = rng.standard_normal((1, 64, 512)).astype(np.float16)
+    z = T(up, hdev).mul(T(gate, hdev).full().silu().cast(_lib.F16)).resolve().to_numpy()
+    want = oracle.binary("mul", up, oracle.cast(oracle.unary("silu", oracle.cast(gate, np.float32)), np.float16))
+    assert same_bits(z, want)
+
+
+def test_two_sided_broadcast_and_inplace_rule(hdev, oracle):
+    rng = np.random.default_rng(406)
+    a = rng.standard_normal((1, 8, 64, 1)).astype(np.float16)
+    b = rng.standard_normal((1, 1, 1, 96)).astype(np.float16)
+    y = T(a, hdev).mul(T(b, hdev)).resolve()                        # the reference mis-builds this graph (tensor.rs:266-272)
+    assert y.shape == (1, 8, 64, 96) and y.last_resolve_launches() == 1
+    want = oracle.binary("mul", np.ascontiguousarray(np.broadcast_to(a, y.shape)), np.ascontiguousarray(np.broadcast_to(b, y.shape)))
+    assert same_bits(y.to_numpy(), want)
+    # in-place rule (tensor.rs:823-824): a source somebody else still holds must keep its contents
+    x = rng.standard_normal((4, 100)).astype(np.float32)
+    tx = T(x, hdev)
+    g = tx.gelu().resolve()
+    assert same_bits(tx.resolve().to_numpy(), x)                    # tx is held here, so gelu must not have written into it
+    assert same_bits(g.to_numpy(), oracle.unary("gelu", x))
+    s = tx.add(tx).resolve()                                        # both operands are the same tensor
+    assert same_bits(s.to_numpy(), x + x) and same_bits(tx.to_numpy(), x)
+    # a materialised broadcast held by the caller stays a separate tensor
+    bt = T(b, hdev).broadcast_to((1, 8, 64, 96))
+    y2 = T(a, hdev).mul(bt).resolve()
+    assert same_bits(y2.to_numpy(), want)
+    assert same_bits(bt.resolve().to_numpy(), np.broadcast_to(b, (1, 8, 64, 96)))

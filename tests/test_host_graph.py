@@ -1,0 +1,138 @@
+"""CPU-only checks of the C++ host mirror's graph building: shape/dtype rules, the errors the reference raises, and the
+topological order.  Tensors here are placeholders (no storage), so no GPU is needed.
+
+Known answers come from the reference's own rules: Shape::multi_broadcast (shape.rs:118-136, numpy rules), Permute output
+shape (ops/reindex/permute.rs:53-56), Concat output shape (ops/concat.rs:116-124), Strides [2,3,4] -> [12,4,1]
+(strides.rs:173-179 is the reference's own unit test).
+"""
+import numpy as np
+import pytest
+
+from ratchet_amd import _lib
+from ratchet_amd.host import HostError, Tensor
+
+F32, F16 = _lib.F32, _lib.F16
+
+
+def P(*shape, dt=F32):
+    return Tensor.placeholder(shape, dt)
+
+
+@pytest.mark.parametrize("a,b", [((1, 1500, 384), (384,)), ((1, 32, 2048, 1), (1, 1, 1, 2048)), ((3, 1, 5), (1, 7, 1)), ((5, 7), (1,)),
+                                 ((1,), (2, 9)), ((4, 1, 8), (4, 6, 8)), ((2, 3), (2, 3))])
+def test_binary_shape_is_numpy_broadcast(a, b):
+    y = P(*a).add(P(*b))
+    assert y.shape == tuple(np.broadcast_shapes(a, b))
+    assert y.op_name() == "Add" and not y.resolved()
+
+
+def test_binary_errors():
+    with pytest.raises(HostError) as e:
+        P(2, 3).mul(P(2, 4))
+    assert e.value.kind == "BroadcastingFailed"                      # InvariantError::BroadcastingFailed (tensor.rs:258-261)
+    with pytest.raises(HostError) as e:
+        P(2, 3).mul(P(2, 3, dt=F16))
+    assert e.value.kind == "DTypeMismatch"                           # Binary::check_dtypes (ops/binary.rs:142-144)
+    with pytest.raises(HostError) as e:
+        P(2, 3, dt=_lib.I32).add(P(2, 3, dt=_lib.I32))
+    assert e.value.kind == "UnsupportedDType"
+
+
+def test_cast_rules():
+    x = P(2, 3)
+    assert x.cast(F32).id == x.id                                    # same dtype returns self (tensor.rs:316-318)
+    assert x.half().dt == F16 and x.half().full().dt == F32
+    assert x.cast(_lib.U32).dt == _lib.U32
+    with pytest.raises(HostError) as e:
+        P(2, 3, dt=F16).cast(_lib.I32)                               # unimplemented!() in cpu_cast (cpu/mod.rs:152)
+    assert e.value.kind == "UnsupportedCast"
+
+
+def test_permute_rules():
+    x = P(1, 1500, 6, 64)
+    assert x.permute((0, 2, 1, 3)).shape == (1, 6, 1500, 64)
+    assert P(4, 5, 6).permute((2, 0, 1)).shape == (6, 4, 5)
+    with pytest.raises(HostError) as e:
+        x.permute((0, 1, 1, 3))
+    assert e.value.kind == "DuplicateDims"                           # InvariantError::DuplicateDims (permute.rs:49-52)
+    with pytest.raises(HostError) as e:
+        x.permute((0, 1, 2))
+    assert e.value.kind == "RankMismatch"                            # assert!(rank == dims.len()) (permute.rs:69)
+
+
+def test_slice_broadcast_view_cat_rules():
+    x = P(6, 5, 9, 40)
+    assert x.slice([(1, 4), (0, 5), (3, 8), (8, 32)]).shape == (3, 5, 5, 24)
+    for ranges, kind in (([(0, 7), (0, 5), (0, 9), (0, 40)], "SliceOutOfBounds"), ([(2, 2), (0, 5), (0, 9), (0, 40)], "EmptySlice"),
+                         ([(0, 6), (0, 5)], "RankMismatch")):
+        with pytest.raises(HostError) as e:
+            x.slice(ranges)
+        assert e.value.kind == kind
+    assert P(1, 5, 1, 16).broadcast_to((3, 5, 4, 16)).shape == (3, 5, 4, 16)
+    assert P(7).broadcast_to((2, 7)).shape == (2, 7)
+    for src, dst in (((2, 3), (2, 4)), ((2, 3, 4), (3, 4))):
+        with pytest.raises(HostError) as e:
+            P(*src).broadcast_to(dst)
+        assert e.value.kind == "InvalidBroadcast"                    # Broadcast::check_shapes panics (broadcast.rs:31-58)
+    assert P(2, 6).view((3, 4)).shape == (3, 4)
+    with pytest.raises(HostError) as e:
+        P(2, 6).view((12,))                                          # View::check_shapes asserts equal rank (ops/view.rs:19-23)
+    assert e.value.kind == "RankMismatch"
+    with pytest.raises(HostError) as e:
+        P(2, 6).view((3, 5))
+    assert e.value.kind == "ShapeMismatch"
+    xs = [P(4, 2, k, 128) for k in (50, 13, 77, 55, 11)]             # the reference's concat test (ops/concat.rs:273-359)
+    assert Tensor.cat(xs, 2).shape == (4, 2, 206, 128)
+    with pytest.raises(HostError) as e:
+        Tensor.cat([P(2, 3)], 0)
+    assert e.value.kind == "ConcatArity"
+    with pytest.raises(HostError) as e:
+        Tensor.cat([P(2, 3), P(3, 4)], 0)
+    assert e.value.kind == "ConcatShapeMismatch"
+    with pytest.raises(HostError) as e:
+        Tensor.cat([P(2, 3)] * 9, 0)
+    assert e.value.kind == "ConcatArity"
+
+
+def test_softmax_and_norm_rules():
+    x = P(1, 6, 1500, 1500)
+    assert x.softmax(3).shape == x.shape
+    for t, dim, kind in ((P(8), 0, "RankMismatch"), (x, 4, "DimOutOfRange"), (x, 1, "UnsupportedSoftmaxDim"),
+                         (P(2, 3, dt=_lib.I32), 1, "UnsupportedDType")):
+        with pytest.raises(HostError) as e:
+            t.softmax(dim)
+        assert e.value.kind == kind
+    h = P(1, 2048, 2560, dt=F16)
+    w, b = P(2560, dt=F16), P(2560, dt=F16)
+    assert h.layer_norm(w, b, 1e-5).shape == h.shape and h.layer_norm(w, None, 1e-5).op_name() == "Norm"
+    assert h.rms_norm(w, 1e-5).shape == h.shape
+    with pytest.raises(HostError) as e:
+        h.layer_norm(P(2560), b, 1e-5)
+    assert e.value.kind == "DTypeMismatch"                           # apply_layer_norm's dtype check (cpu/norm.rs:34-49)
+    with pytest.raises(HostError) as e:
+        h.rms_norm(P(2561, dt=F16), 1e-5)
+    assert e.value.kind == "ShapeMismatch"
+    g = P(1, 512, 3000, dt=F16)
+    assert g.group_norm(32, P(512, dt=F16), P(512, dt=F16), 1e-5).shape == g.shape
+    with pytest.raises(HostError) as e:
+        g.group_norm(30, P(512, dt=F16), None, 1e-5)
+    assert e.value.kind == "InvalidGroups"
+
+
+def test_execution_order_is_topological_and_dedups_shared_nodes():
+    a, b = P(4, 8), P(8)
+    s = a.add(b)                    # Broadcast(b) + Add
+    g = s.gelu()
+    y = g.mul(s)                    # s is used twice
+    order = y.execution_order()
+    assert len(order) == len(set(order))
+    pos = {i: k for k, i in enumerate(order)}
+    assert pos[a.id] < pos[s.id] and pos[b.id] < pos[s.id] < pos[g.id] < pos[y.id]
+    assert order[-1] == y.id
+    assert len(order) == 6          # a, b, Broadcast(b), s, g, y
+
+
+def test_placeholders_cannot_be_resolved():
+    with pytest.raises(HostError) as e:
+        P(2, 3).gelu().resolve()
+    assert e.value.kind == "Unresolved"
