@@ -116,6 +116,13 @@ int rt_broadcast(rt_device* dev, int elem_bytes, const void* x, void* y, const u
 int rt_concat(rt_device* dev, int elem_bytes, int n_inputs, const void* const* xs, const uint32_t (*shapes)[4],
               int dim, void* y);
 
+/* Cache, the KV-cache append (ops/cache.rs:17-105, Tensor::cache tensor.rs:481-486; callers models/phi2/attn.rs:129-135,
+ * models/whisper/mha.rs:72-79): dst = cat(cache[.. 0:offset ..], source) along dim, shape = cache shape with
+ * dim := offset + source_shape[dim] (:139-147), and source is also written into cache at offset (cache is updated in
+ * place; it must not alias dst).  The reference has no CPU implementation; its test's ground truth is that cat. */
+int rt_cache(rt_device* dev, int elem_bytes, void* cache, const uint32_t cache_shape[4], const void* source,
+             const uint32_t source_shape[4], int dim, uint32_t offset, void* dst);
+
 /* Softmax over the last dimension (ops/softmax.rs:14-39,183-199; cpu/softmax.rs:22-42): rows x cols, contiguous.
  * y may alias x (the reference kernel is in-place only, ops/softmax.rs:47-49).  dt: F32, F16, BF16. */
 int rt_softmax(rt_device* dev, int dt, const void* x, void* y, uint64_t rows, uint32_t cols, int mode);

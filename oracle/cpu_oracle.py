@@ -42,6 +42,7 @@ def lib():
         L.orc_slice.argtypes = [i, vp, vp, i, vp, vp, vp]
         L.orc_broadcast.argtypes = [i, vp, vp, i, vp, i, vp, i]
         L.orc_concat.argtypes = [i, i, vp, i, vp, i, vp]
+        L.orc_cache.argtypes = [i, vp, i, vp, vp, vp, i, ctypes.c_uint64, vp]
         L.orc_softmax.argtypes = [i, vp, vp, sz, sz]
         L.orc_layer_norm.argtypes = [i, vp, vp, vp, vp, sz, sz, f, sz]
         L.orc_rms_norm.argtypes = [i, vp, vp, vp, sz, sz, f, sz]
@@ -160,6 +161,18 @@ def concat(xs, dim):
     y = np.empty(out_shape, dtype=xs[0].dtype)
     ptrs = (ctypes.c_void_p * len(xs))(*[x.ctypes.data for x in xs])
     _check(lib().orc_concat(xs[0].dtype.itemsize, len(xs), ptrs, rank, _p(shapes), dim, _p(y)), "concat")
+    return y
+
+
+def cache(cache_arr, source, dim, offset):
+    """KV-cache append: returns dst; cache_arr (C-contiguous, writable) is updated in place as the reference's kernel does."""
+    assert cache_arr.flags["C_CONTIGUOUS"] and cache_arr.flags["WRITEABLE"]
+    source = _c(source)
+    out_shape = list(cache_arr.shape)
+    out_shape[dim] = offset + source.shape[dim]
+    y = np.empty(out_shape, dtype=cache_arr.dtype)
+    _check(lib().orc_cache(cache_arr.dtype.itemsize, _p(cache_arr), cache_arr.ndim, _p(_u64(cache_arr.shape)), _p(source),
+                           _p(_u64(source.shape)), dim, offset, _p(y)), "cache")
     return y
 
 

@@ -11,6 +11,7 @@ struct OrcTable {
     int (*slice)(int, const void*, void*, int, const uint64_t*, const uint64_t*, const uint64_t*);
     int (*broadcast)(int, const void*, void*, int, const uint64_t*, int, const uint64_t*, int);
     int (*concat)(int, int, const void* const*, int, const uint64_t*, int, void*);
+    int (*cache)(int, void*, int, const uint64_t*, const void*, const uint64_t*, int, uint64_t, void*);
     int (*softmax)(int, const void*, void*, size_t, size_t);
     int (*layer_norm)(int, const void*, const void*, const void*, void*, size_t, size_t, float, size_t);
     int (*rms_norm)(int, const void*, const void*, void*, size_t, size_t, float, size_t);

@@ -28,6 +28,10 @@ int orc_broadcast(int eb, const void* x, void* y, int sr, const uint64_t* ss, in
 int orc_concat(int eb, int n, const void* const* xs, int rank, const uint64_t* shapes, int dim, void* y) {
     return table().concat(eb, n, xs, rank, shapes, dim, y);
 }
+int orc_cache(int eb, void* cache, int rank, const uint64_t* cs, const void* source, const uint64_t* ss, int dim, uint64_t offset,
+              void* dst) {
+    return table().cache(eb, cache, rank, cs, source, ss, dim, offset, dst);
+}
 int orc_softmax(int dt, const void* x, void* y, size_t rows, size_t cols) { return table().softmax(dt, x, y, rows, cols); }
 int orc_layer_norm(int dt, const void* x, const void* s, const void* b, void* y, size_t rows, size_t cols, float eps,
                    size_t shape0) {

@@ -58,6 +58,11 @@ int orc_broadcast(int elem_bytes, const void* x, void* y, int src_rank, const ui
 int orc_concat(int elem_bytes, int n_inputs, const void* const* xs, int rank, const uint64_t* shapes /* n*rank */,
                int dim, void* y);
 
+/* KV-cache append (crates/ratchet-core/src/ops/cache.rs:64-105; the reference has no CPU implementation, its test uses cat as
+ * ground truth): dst = cat(cache[.. :offset ..], source) along dim, and source is also written into cache at offset. */
+int orc_cache(int elem_bytes, void* cache, int rank, const uint64_t* cache_shape, const void* source, const uint64_t* source_shape,
+              int dim, uint64_t offset, void* dst);
+
 int orc_softmax(int dt, const void* x, void* y, size_t rows, size_t cols);
 /* shape0 = size of the input's first dimension: the reference broadcasts scale/bias with a
  * vector special case that depends on it (pass 1 to get the mathematically intended result) */

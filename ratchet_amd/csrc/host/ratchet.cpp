@@ -95,7 +95,7 @@ Buffer::~Buffer() {
 }
 
 // ------------------------------------------------------------------------------------------------------------ graph
-enum class Kind { Const, Binary, Unary, Cast, Permute, Slice, Broadcast, Concat, Softmax, LayerNorm, RMSNorm, GroupNorm, View };
+enum class Kind { Const, Binary, Unary, Cast, Permute, Slice, Broadcast, Concat, Cache, Softmax, LayerNorm, RMSNorm, GroupNorm, View };
 
 struct Node {
     uint64_t id = 0;
@@ -162,6 +162,7 @@ const char* Tensor::op_name() const {
         case Kind::Slice: return "Slice";
         case Kind::Broadcast: return "Broadcast";
         case Kind::Concat: return "Concat";
+        case Kind::Cache: return "Cache";
         case Kind::Softmax: return "Softmax";
         case Kind::View: return "View";
         default: return "Norm";
@@ -324,6 +325,27 @@ Tensor Tensor::cat(const std::vector<Tensor>& tensors, size_t dim) {
     auto n = new_node(Kind::Concat, out, first.dt(), first.device());
     n->dim = dim;
     n->srcs = tensors;
+    return Tensor(n);
+}
+
+// Cache guards: ops/cache.rs:124-133
+Tensor Tensor::cache(const Tensor& source, size_t dim, size_t offset) const {
+    require_same_device(*this, source);
+    if (rank() < 3 || rank() > 4) throw Error("RankMismatch", "cache needs rank 3 or 4");
+    if (source.rank() != rank()) throw Error("RankMismatch", "cache and source must have one rank");
+    if (dt() != source.dt()) throw Error("DTypeMismatch", std::string("expected ") + as_str(dt()) + ", got " + as_str(source.dt()));
+    if (dim >= rank()) throw Error("DimOutOfRange", "cache dim " + std::to_string(dim));
+    for (size_t a = 0; a < rank(); a++)
+        if (a != dim && source.shape()[a] != shape()[a]) throw Error("ShapeMismatch", source.shape().to_string() + " vs " + shape().to_string());
+    if (offset > shape()[dim] || offset + source.shape()[dim] > shape()[dim])
+        throw Error("CacheOverflow", "offset " + std::to_string(offset) + " + " + std::to_string(source.shape()[dim]) + " rows exceed " +
+                                         std::to_string(shape()[dim]));
+    Shape out = shape();
+    out[dim] = offset + source.shape()[dim];
+    auto n = new_node(Kind::Cache, out, dt(), device());
+    n->dim = dim;
+    n->groups = offset;                        // reuses the integer slot: the write offset
+    n->srcs = {*this, source};
     return Tensor(n);
 }
 
@@ -502,6 +524,17 @@ struct Resolver {
                 out_buffer();
                 check_rt(rt_concat(dev, (int)size_of(n->dt), (int)n->srcs.size(), ptrs, shapes, (int)(n->dim + 4 - n->shape.rank()), n->storage->ptr),
                          "rt_concat");
+                launches++;
+                return;
+            }
+            case Kind::Cache: {
+                uint32_t cs[4], ss[4];
+                shape4(src(0)->shape, cs);
+                shape4(src(1)->shape, ss);
+                out_buffer();                                  // Cache::supports_inplace() is false (ops/cache.rs:150-152)
+                check_rt(rt_cache(dev, (int)size_of(n->dt), src(0)->storage->ptr, cs, src(1)->storage->ptr, ss,
+                                  (int)(n->dim + 4 - n->shape.rank()), (uint32_t)n->groups, n->storage->ptr),
+                         "rt_cache");
                 launches++;
                 return;
             }

@@ -146,6 +146,9 @@ class Tensor {
     Tensor view(const Shape& shape) const;                                                               // tensor.rs:454-461
     static Tensor cat(const std::vector<Tensor>& tensors, size_t dim);                                   // tensor.rs:463-470
     Tensor permute(const std::vector<size_t>& dims) const;                                               // tensor.rs:472-479
+    // self is the cache (tensor.rs:481-486): result = cat(self[.. :offset ..], source) along dim; resolve() also writes
+    // source into the cache's storage at offset
+    Tensor cache(const Tensor& source, size_t dim, size_t offset) const;
     Tensor broadcast_to(const Shape& shape) const;                                                       // tensor.rs:488-495
 
     // tensor.rs:861-863: runs every unresolved node this tensor depends on; returns after completion

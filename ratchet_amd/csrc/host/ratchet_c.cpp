@@ -114,6 +114,9 @@ rth_tensor* rth_cat(const rth_tensor* const* xs, int n, size_t dim) {
         return Tensor::cat(ts, dim);
     });
 }
+rth_tensor* rth_cache(const rth_tensor* cache, const rth_tensor* source, size_t dim, size_t offset) {
+    return build([&] { return cache->t.cache(source->t, dim, offset); });
+}
 rth_tensor* rth_permute(const rth_tensor* x, int n, const uint64_t* dims) {
     return build([&] {
         std::vector<size_t> d(dims, dims + (n > 0 ? n : 0));

@@ -139,6 +139,52 @@ __global__ void __launch_bounds__(BLOCK) concat_kernel(VecT* __restrict__ y, Con
     }
 }
 
+// KV-cache append: blockIdx.y == 0 copies the filled prefix of the cache into dst, blockIdx.y == 1 writes the new rows
+// into both the cache (at `offset`) and dst.  All quantities are in vectors of sizeof(VecT) bytes.
+struct CacheArgs {
+    FastDiv pv, sv;          // prefix / source vectors per outer row
+    uint32_t cap_v, dst_v;   // cache / dst vectors per outer row
+    uint32_t off_v;          // offset, in vectors, inside an outer row
+    uint32_t n_prefix, n_src;
+};
+
+template <typename VecT>
+__global__ void __launch_bounds__(BLOCK) cache_kernel(VecT* __restrict__ cache, const VecT* __restrict__ src, VecT* __restrict__ dst,
+                                                      CacheArgs p) {
+    const uint32_t base = blockIdx.x * (BLOCK * UNROLL) + threadIdx.x;
+    if (blockIdx.y == 0) {
+        if (blockIdx.x * (BLOCK * UNROLL) >= p.n_prefix) return;
+        VecT r[UNROLL];
+        uint32_t row[UNROLL], col[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            const uint32_t v = base + u * BLOCK;
+            if (v < p.n_prefix) {
+                fd_divmod(v, p.pv, row[u], col[u]);
+                r[u] = cache[(uint64_t)row[u] * p.cap_v + col[u]];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            const uint32_t v = base + u * BLOCK;
+            if (v < p.n_prefix) dst[(uint64_t)row[u] * p.dst_v + col[u]] = r[u];
+        }
+    } else {
+        if (blockIdx.x * (BLOCK * UNROLL) >= p.n_src) return;
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            const uint32_t v = base + u * BLOCK;
+            if (v < p.n_src) {
+                uint32_t row, col;
+                fd_divmod(v, p.sv, row, col);
+                const VecT val = src[v];
+                cache[(uint64_t)row * p.cap_v + p.off_v + col] = val;
+                dst[(uint64_t)row * p.dst_v + p.off_v + col] = val;
+            }
+        }
+    }
+}
+
 inline unsigned blocks_for(uint64_t items, uint64_t per_block) {
     const uint64_t b = (items + per_block - 1) / per_block;
     return (unsigned)(b ? b : 1);
@@ -430,6 +476,59 @@ int rt_concat(rt_device* dev, int elem_bytes, int n_inputs, const void* const* x
     else if (vb == 4) hipLaunchKernelGGL((concat_kernel<uint32_t>), grid, dim3(BLOCK), 0, dev->stream, (uint32_t*)y, p);
     else hipLaunchKernelGGL((concat_kernel<uint16_t>), grid, dim3(BLOCK), 0, dev->stream, (uint16_t*)y, p);
     RT_CHECK_LAUNCH("concat_kernel");
+    return RT_OK;
+}
+
+int rt_cache(rt_device* dev, int elem_bytes, void* cache, const uint32_t cache_shape[4], const void* source, const uint32_t source_shape[4],
+             int dim, uint32_t offset, void* dst) {
+    RT_REQUIRE(elem_bytes == 2 || elem_bytes == 4, RT_ERR_ARG, "rt_cache: elem_bytes must be 2 or 4, got %d", elem_bytes);
+    RT_REQUIRE(dim >= 0 && dim < 4, RT_ERR_ARG, "rt_cache: dim %d out of range", dim);
+    RT_REQUIRE(cache_shape && source_shape, RT_ERR_NULL_POINTER, "rt_cache: NULL shape");
+    uint64_t outer = 1, inner = 1;
+    for (int a = 0; a < 4; a++) {
+        RT_REQUIRE(cache_shape[a] > 0 && source_shape[a] > 0, RT_ERR_SHAPE, "rt_cache: zero extent in dim %d", a);
+        if (a != dim)
+            RT_REQUIRE(cache_shape[a] == source_shape[a], RT_ERR_SHAPE, "rt_cache: source differs from the cache in dim %d", a);
+        if (a < dim) outer *= cache_shape[a];
+        if (a > dim) inner *= cache_shape[a];
+    }
+    const uint64_t cap = cache_shape[dim], s = source_shape[dim];
+    // Cache::check_shapes (ops/cache.rs:125-128): offset <= cache extent; the write itself must also fit
+    RT_REQUIRE(offset <= cap && (uint64_t)offset + s <= cap, RT_ERR_SHAPE, "rt_cache: offset %u + %llu rows exceed the cache's %llu", offset,
+               (unsigned long long)s, (unsigned long long)cap);
+    RT_REQUIRE(cache && source && dst, RT_ERR_NULL_POINTER, "rt_cache: NULL operand");
+    RT_REQUIRE(rt_aligned(cache, (size_t)elem_bytes) && rt_aligned(source, (size_t)elem_bytes) && rt_aligned(dst, (size_t)elem_bytes),
+               RT_ERR_ALIGN, "rt_cache: misaligned pointer");
+    RT_REQUIRE(outer * cap * inner <= RT_MAX_NUMEL, RT_ERR_SIZE, "rt_cache: cache too large");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    const uint64_t pre_b = (uint64_t)offset * inner * elem_bytes, src_b = s * inner * elem_bytes, cap_b = cap * inner * elem_bytes,
+                   dst_b = ((uint64_t)offset + s) * inner * elem_bytes;
+    int vb = 16;
+    for (; vb > elem_bytes; vb >>= 1)
+        if (pre_b % vb == 0 && src_b % vb == 0 && cap_b % vb == 0 && dst_b % vb == 0 && rt_aligned(cache, (size_t)vb) &&
+            rt_aligned(source, (size_t)vb) && rt_aligned(dst, (size_t)vb))
+            break;
+    CacheArgs p;
+    const uint64_t n_prefix = outer * pre_b / vb, n_src = outer * src_b / vb;
+    RT_REQUIRE(n_prefix <= 0xffffffffull - (uint64_t)BLOCK * UNROLL && n_src <= 0xffffffffull - (uint64_t)BLOCK * UNROLL &&
+                   cap_b / vb <= 0xffffffffull,
+               RT_ERR_SIZE, "rt_cache: tensor too large for 32-bit vector indices");
+    p.pv = make_fastdiv((uint32_t)(pre_b / vb ? pre_b / vb : 1));
+    p.sv = make_fastdiv((uint32_t)(src_b / vb));
+    p.cap_v = (uint32_t)(cap_b / vb);
+    p.dst_v = (uint32_t)(dst_b / vb);
+    p.off_v = (uint32_t)(pre_b / vb);
+    p.n_prefix = (uint32_t)n_prefix;
+    p.n_src = (uint32_t)n_src;
+    const dim3 grid(blocks_for(n_prefix > n_src ? n_prefix : n_src, BLOCK * UNROLL), 2);
+    if (vb == 16) hipLaunchKernelGGL((cache_kernel<v4u>), grid, dim3(BLOCK), 0, dev->stream, (v4u*)cache, (const v4u*)source, (v4u*)dst, p);
+    else if (vb == 8) hipLaunchKernelGGL((cache_kernel<v2u>), grid, dim3(BLOCK), 0, dev->stream, (v2u*)cache, (const v2u*)source, (v2u*)dst, p);
+    else if (vb == 4)
+        hipLaunchKernelGGL((cache_kernel<uint32_t>), grid, dim3(BLOCK), 0, dev->stream, (uint32_t*)cache, (const uint32_t*)source, (uint32_t*)dst, p);
+    else
+        hipLaunchKernelGGL((cache_kernel<uint16_t>), grid, dim3(BLOCK), 0, dev->stream, (uint16_t*)cache, (const uint16_t*)source, (uint16_t*)dst, p);
+    RT_CHECK_LAUNCH("cache_kernel");
     return RT_OK;
 }
 

@@ -54,7 +54,7 @@ def load():
         "rth_from_host": [vp, vp, i, u64p, i], "rth_placeholder": [i, u64p, i], "rth_binary": [vp, vp, i], "rth_unary": [vp, i],
         "rth_cast": [vp, i], "rth_layer_norm": [vp, vp, vp, f], "rth_rms_norm": [vp, vp, f], "rth_group_norm": [vp, sz, vp, vp, f],
         "rth_softmax": [vp, sz, i], "rth_slice": [vp, i, u64p, u64p], "rth_view": [vp, i, u64p],
-        "rth_cat": [ctypes.POINTER(vp), i, sz], "rth_permute": [vp, i, u64p], "rth_broadcast_to": [vp, i, u64p],
+        "rth_cat": [ctypes.POINTER(vp), i, sz], "rth_cache": [vp, vp, sz, sz], "rth_permute": [vp, i, u64p], "rth_broadcast_to": [vp, i, u64p],
     }.items():
         fn = getattr(H, name)
         fn.argtypes = args
@@ -196,6 +196,9 @@ class Tensor:
     def cat(tensors, dim):
         arr = (ctypes.c_void_p * len(tensors))(*[t.handle for t in tensors])
         return Tensor(load().rth_cat(arr, len(tensors), dim))
+
+    def cache(self, source, dim, offset):
+        return Tensor(self.H.rth_cache(self.handle, source.handle, dim, offset))
 
     def permute(self, dims):
         return Tensor(self.H.rth_permute(self.handle, len(dims), _u64(dims)))

@@ -206,6 +206,16 @@ class Device:
         check(self.lib.rt_concat(self.handle, _DT_BYTES[xs[0].dt], len(xs), ptrs, shapes, dim + (4 - rank), out.ptr))
         return out
 
+    def cache(self, cache, source, dim, offset, out=None):
+        """KV-cache append: returns cat(cache[:offset], source) along dim and writes source into cache at offset."""
+        rank = len(cache.shape)
+        out_shape = list(cache.shape)
+        out_shape[dim] = offset + source.shape[dim]
+        out = out or Buffer(self, out_shape, cache.dt)
+        check(self.lib.rt_cache(self.handle, _DT_BYTES[cache.dt], cache.ptr, shape4(cache.shape), source.ptr, shape4(source.shape),
+                                dim + (4 - rank), offset, out.ptr))
+        return out
+
     def softmax(self, x, out=None, mode=_lib.SOFTMAX_REFERENCE):
         cols = x.shape[-1]
         out = out or Buffer(self, x.shape, x.dt)

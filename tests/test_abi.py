@@ -106,6 +106,14 @@ def test_reindex_validation(lib):
     assert lib.rt_concat(None, 4, 1, ptrs, shapes, 2, SOME) == 7                      # needs 2..8 inputs
     assert lib.rt_concat(None, 4, 9, ptrs, shapes, 2, SOME) == 7
     assert lib.rt_concat(None, 4, 2, ptrs, shapes, 4, SOME) == 7
+    cs, ss = u4(1, 2, 6, 16), u4(1, 2, 1, 16)
+    assert lib.rt_cache(None, 4, SOME, cs, SOME, ss, 2, 2, SOME) == 8
+    assert lib.rt_cache(None, 4, SOME, cs, SOME, ss, 2, 6, SOME) == 4                 # offset 6 + 1 row > 6
+    assert lib.rt_cache(None, 4, SOME, cs, SOME, ss, 2, 7, SOME) == 4                 # offset > cache extent (ops/cache.rs:127)
+    assert lib.rt_cache(None, 4, SOME, cs, SOME, u4(1, 3, 1, 16), 2, 0, SOME) == 4    # differs outside dim
+    assert lib.rt_cache(None, 4, SOME, cs, SOME, ss, 4, 0, SOME) == 7
+    assert lib.rt_cache(None, 8, SOME, cs, SOME, ss, 2, 0, SOME) == 7
+    assert lib.rt_cache(None, 4, None, cs, SOME, ss, 2, 0, SOME) == 1
 
 
 def test_reduction_validation(lib):

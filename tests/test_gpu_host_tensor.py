@@ -188,3 +188,22 @@ def test_two_sided_broadcast_and_inplace_rule(hdev, oracle):
     y2 = T(a, hdev).mul(bt).resolve()
     assert same_bits(y2.to_numpy(), want)
     assert same_bits(bt.resolve().to_numpy(), np.broadcast_to(b, (1, 8, 64, 96)))
+
+
+def test_cache_decode_loop(hdev, oracle):
+    """phi2's KV append (models/phi2/attn.rs:129-135): the cache tensor is reused across steps and each step's result is
+    cat(cache[:offset], new rows); ground truth as in the reference's test (ops/cache.rs:162-217)."""
+    from ratchet_amd import _lib
+
+    rng = np.random.default_rng(405)
+    cache_np = np.zeros((1, 4, 24, 80), np.float16)
+    cache = T(cache_np, hdev)
+    rows, off = [], 0
+    for n in (7, 1, 1, 1):
+        src = rng.standard_normal((1, 4, n, 80)).astype(np.float16)
+        rows.append(src)
+        got = cache.cache(T(src, hdev), 2, off).resolve().to_numpy()
+        off += n
+        assert np.array_equal(got, np.concatenate(rows, axis=2))
+        assert np.array_equal(got, oracle.cache(cache_np, src, 2, off - n))
+    assert np.array_equal(cache.to_numpy(), cache_np)

@@ -143,3 +143,42 @@ def test_concat_rejects_bad_arguments(dev):
     with pytest.raises(RatchetError) as e:
         dev.concat([a], 0)
     assert e.value.status == 7
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_cache(dev, oracle, dtype):
+    rng = np.random.default_rng(205)
+    # the reference's own case (ops/cache.rs:162-217)
+    populated = randn(rng, (1, 2, 2, 16), dtype)
+    source = randn(rng, (1, 2, 1, 16), dtype)
+    cache = np.concatenate([populated, np.zeros((1, 2, 4, 16), dtype)], axis=2)
+    d_cache = dev.upload(cache)
+    got = dev.cache(d_cache, dev.upload(source), 2, 2).to_numpy()
+    want = oracle.cache(cache, source, 2, 2)
+    assert np.array_equal(got, want) and np.array_equal(got, np.concatenate([populated, source], axis=2))
+    assert np.array_equal(d_cache.to_numpy(), cache)
+    # decode loops in phi2's (dim 2) and whisper's (dim 1) layouts, odd extents for every vector width, prompt then single rows
+    for dim, shape, chunks in ((2, (1, 32, 40, 80), (17, 1, 1, 1, 20)), (1, (1, 24, 384), (5, 1, 1, 17)), (2, (2, 3, 9, 5), (2, 3, 1, 3)),
+                               (3, (1, 2, 3, 11), (4, 7)), (1, (2, 6, 4, 6), (1, 5)), (0, (6, 2, 4), (6,)), (2, (1, 1, 2048, 128), (2047, 1))):
+        cache = randn(rng, shape, dtype)                       # stale contents beyond the fill must never reach dst
+        d_cache = dev.upload(cache)
+        off = 0
+        for n in chunks:
+            sshape = list(shape)
+            sshape[dim] = n
+            src = randn(rng, sshape, dtype)
+            got = dev.cache(d_cache, dev.upload(src), dim, off).to_numpy()
+            want = oracle.cache(cache, src, dim, off)
+            off += n
+            assert np.array_equal(got, want), (dim, shape, off)
+            assert np.array_equal(d_cache.to_numpy(), cache), (dim, shape, off)
+
+
+def test_cache_rejects_overflow(dev):
+    from ratchet_amd import RatchetError
+
+    c = dev.upload(np.zeros((1, 2, 4, 8), np.float32))
+    s = dev.upload(np.zeros((1, 2, 2, 8), np.float32))
+    with pytest.raises(RatchetError) as e:
+        dev.cache(c, s, 2, 3)
+    assert e.value.status == 4

@@ -94,6 +94,20 @@ def test_slice_broadcast_view_cat_rules():
     assert e.value.kind == "ConcatArity"
 
 
+def test_cache_rules():
+    # Cache::compute_view and check_shapes (ops/cache.rs:124-147)
+    kv = P(1, 32, 2048, 80, dt=F16)
+    y = kv.cache(P(1, 32, 1, 80, dt=F16), 2, 17)
+    assert y.shape == (1, 32, 18, 80) and y.op_name() == "Cache"
+    assert P(1, 1500, 384).cache(P(1, 3, 384), 1, 0).shape == (1, 3, 384)     # whisper's layout (models/whisper/mha.rs:72-79)
+    for cache, src, dim, off, kind in ((P(64, 80), P(1, 80), 0, 0, "RankMismatch"), (kv, P(1, 32, 1, 80), 2, 0, "DTypeMismatch"),
+                                       (kv, P(1, 32, 1, 80, dt=F16), 2, 2049, "CacheOverflow"), (kv, P(1, 32, 2, 80, dt=F16), 2, 2047, "CacheOverflow"),
+                                       (kv, P(1, 16, 1, 80, dt=F16), 2, 0, "ShapeMismatch"), (kv, P(1, 32, 1, 80, dt=F16), 4, 0, "DimOutOfRange")):
+        with pytest.raises(HostError) as e:
+            cache.cache(src, dim, off)
+        assert e.value.kind == kind, (kind, e.value.kind)
+
+
 def test_softmax_and_norm_rules():
     x = P(1, 6, 1500, 1500)
     assert x.softmax(3).shape == x.shape

@@ -351,3 +351,34 @@ def test_concat_reference_case(oracle):
     assert np.array_equal(oracle.concat(zs, 0), np.concatenate(zs, axis=0))
     with pytest.raises(ValueError):
         oracle.concat([np.zeros((2, 3), np.float32), np.zeros((3, 4), np.float32)], 0)
+
+
+def test_cache_reference_case_and_properties(oracle):
+    # crates/ratchet-core/src/ops/cache.rs:162-217: populated [1,2,2,16] + zeros [1,2,4,16] along dim 2, source [1,2,1,16],
+    # offset 2; the ground truth the reference's test uses is cat(populated, source)
+    rng = np.random.default_rng(77)
+    populated = rng.standard_normal((1, 2, 2, 16)).astype(np.float32)
+    source = rng.standard_normal((1, 2, 1, 16)).astype(np.float32)
+    cache = np.concatenate([populated, np.zeros((1, 2, 4, 16), np.float32)], axis=2)
+    dst = oracle.cache(cache, source, 2, 2)
+    assert dst.shape == (1, 2, 3, 16)
+    assert np.array_equal(dst, np.concatenate([populated, source], axis=2))
+    assert np.array_equal(cache[:, :, 2:3], source) and np.array_equal(cache[:, :, :2], populated) and not cache[:, :, 3:].any()
+    # a decode loop fills the cache row by row; after the last step the cache equals the concatenation of every source
+    for dim, shape, dtype in ((1, (3, 9, 20), np.float16), (2, (2, 3, 7, 5), np.float32), (3, (1, 2, 3, 11), np.float16), (0, (6, 2, 4), np.float32)):
+        cache = np.zeros(shape, dtype)
+        steps, off = [], 0
+        while off < shape[dim]:
+            n = min(int(rng.integers(1, 4)), shape[dim] - off)
+            sshape = list(shape)
+            sshape[dim] = n
+            src = rng.standard_normal(sshape).astype(dtype)
+            steps.append(src)
+            dst = oracle.cache(cache, src, dim, off)
+            off += n
+            assert np.array_equal(dst, np.concatenate(steps, axis=dim)), (dim, shape, off)
+        assert np.array_equal(cache, np.concatenate(steps, axis=dim))
+    with pytest.raises(ValueError):
+        oracle.cache(np.zeros((1, 2, 4, 8), np.float32), np.zeros((1, 2, 2, 8), np.float32), 2, 3)     # 3 + 2 > 4
+    with pytest.raises(ValueError):
+        oracle.cache(np.zeros((4, 8), np.float32), np.zeros((1, 8), np.float32), 0, 0)                  # rank < 3 (cache.rs:125)
