@@ -9,6 +9,7 @@
 #define RT_ARITH_H
 
 #include "../../include/ratchet_hip.h"
+#include "rt_internal.h"
 #include "rt_math.h"
 
 struct bf16_t {
@@ -116,7 +117,7 @@ template <int OP, typename T> __device__ __forceinline__ T ar_binary(T a, T b) {
 
 // 16-byte register vector viewed as elements of T
 template <typename T> union Vec16 {
-    uint4 u;
+    v4u u;
     T e[16 / sizeof(T)];
     __device__ __forceinline__ Vec16() {}
 };

@@ -61,6 +61,12 @@ static inline bool rt_aligned(const void* p, size_t a) { return (reinterpret_cas
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 typedef unsigned int v2u __attribute__((ext_vector_type(2)));
 
+// Streaming accesses for data that is touched once: the non-temporal hint keeps it from displacing cache lines and,
+// measured on MI355X with a 1 GiB copy, lifts a kernel from 5.7-6.2 TB/s to 6.5 TB/s.  Operands that are re-read
+// (broadcast rows, tables, a second pass over the same tile) keep ordinary loads.
+template <typename V> __device__ __forceinline__ V ld_stream(const V* p) { return __builtin_nontemporal_load(p); }
+template <typename V> __device__ __forceinline__ void st_stream(V* p, V v) { __builtin_nontemporal_store(v, p); }
+
 // the kernels index elements with 64-bit integers but grid sizes are 32-bit; 2^40 elements is far beyond 288 GB
 static const uint64_t RT_MAX_NUMEL = 1ull << 40;
 

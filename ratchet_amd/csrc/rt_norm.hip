@@ -69,13 +69,13 @@ __global__ void __launch_bounds__(BLOCK) norm_wave_kernel(const T* __restrict__ 
     if (row >= rows) return;
     const int lane = threadIdx.x & (WAVE - 1);
     const uint32_t nvec = cols / VE;
-    const uint4* xr = reinterpret_cast<const uint4*>(x + row * cols);
-    uint4* yr = reinterpret_cast<uint4*>(y + row * cols);
+    const v4u* xr = reinterpret_cast<const v4u*>(x + row * cols);
+    v4u* yr = reinterpret_cast<v4u*>(y + row * cols);
     Vec16<T> v[NV];
 #pragma unroll
     for (int k = 0; k < NV; k++) {
         const uint32_t i = lane + k * WAVE;
-        if (i < nvec) v[k].u = xr[i];
+        if (i < nvec) v[k].u = ld_stream(xr + i);
     }
     float sx = 0.0f, sq = 0.0f;
 #pragma unroll
@@ -90,8 +90,8 @@ __global__ void __launch_bounds__(BLOCK) norm_wave_kernel(const T* __restrict__ 
     if (KIND == NORM_LAYER) sx = wave_sum(sx);
     sq = wave_sum(sq);
     const RowStats<T> st = finish_stats<T, KIND>(sx, sq, cols, eps);
-    const uint4* sv = reinterpret_cast<const uint4*>(scale);
-    const uint4* bv = reinterpret_cast<const uint4*>(bias);
+    const v4u* sv = reinterpret_cast<const v4u*>(scale);
+    const v4u* bv = reinterpret_cast<const v4u*>(bias);
 #pragma unroll
     for (int k = 0; k < NV; k++) {
         const uint32_t i = lane + k * WAVE;
@@ -101,7 +101,7 @@ __global__ void __launch_bounds__(BLOCK) norm_wave_kernel(const T* __restrict__ 
             if (KIND == NORM_LAYER && bias) b.u = bv[i];
 #pragma unroll
             for (int q = 0; q < VE; q++) o.e[q] = norm_one<T, KIND>(v[k].e[q], st, s.e[q], b.e[q], bias != nullptr);
-            yr[i] = o.u;
+            st_stream(yr + i, o.u);
         }
     }
 }
@@ -167,7 +167,7 @@ __global__ void __launch_bounds__(BLOCK) norm_seq16_kernel(const T* __restrict__
                 const T* src = x + (row0 + r) * cols + c0 + col;
                 if (VEC) {
                     Vec16<T> in;
-                    in.u = *reinterpret_cast<const uint4*>(src);
+                    in.u = *reinterpret_cast<const v4u*>(src);
                     float sq[8], xv[8];
 #pragma unroll
                     for (int q = 0; q < 8; q++) {
@@ -224,12 +224,12 @@ __global__ void __launch_bounds__(BLOCK) norm_seq16_kernel(const T* __restrict__
         for (uint32_t cv = threadIdx.x; cv < cvec; cv += BLOCK) {
             if (VEC) {
                 Vec16<T> in, sc, bi, out;
-                in.u = reinterpret_cast<const uint4*>(src)[cv];
-                sc.u = reinterpret_cast<const uint4*>(scale)[cv];
-                if (KIND == NORM_LAYER && bias) bi.u = reinterpret_cast<const uint4*>(bias)[cv];
+                in.u = reinterpret_cast<const v4u*>(src)[cv];
+                sc.u = reinterpret_cast<const v4u*>(scale)[cv];
+                if (KIND == NORM_LAYER && bias) bi.u = reinterpret_cast<const v4u*>(bias)[cv];
 #pragma unroll
                 for (int q = 0; q < 8; q++) out.e[q] = norm_one<T, KIND>(in.e[q], st, sc.e[q], bi.e[q], bias != nullptr);
-                reinterpret_cast<uint4*>(dst)[cv] = out.u;
+                st_stream(reinterpret_cast<v4u*>(dst) + cv, out.u);
             } else {
                 const T b = (KIND == NORM_LAYER && bias) ? bias[cv] : Ar<T>::conv(0.0f);
                 dst[cv] = norm_one<T, KIND>(src[cv], st, scale[cv], b, bias != nullptr);
@@ -316,7 +316,7 @@ __global__ void __launch_bounds__(NP_BLOCK) norm_pipe16_kernel(const T* __restri
             float sq[8], xv[8];
             if (col < cols) {
                 Vec16<T> in;
-                in.u = __builtin_bit_cast(uint4, reg);
+                in.u = __builtin_bit_cast(v4u, reg);
 #pragma unroll
                 for (int q = 0; q < 8; q++) {
                     sq[q] = Ar<T>::widen(Ar<T>::mul(in.e[q], in.e[q]));
@@ -356,12 +356,12 @@ __global__ void __launch_bounds__(NP_BLOCK) norm_pipe16_kernel(const T* __restri
     const uint32_t cvec = cols / 8;
     for (uint32_t c = cv; c < cvec; c += 32) {
         Vec16<T> in, sc, bi, out;
-        in.u = reinterpret_cast<const uint4*>(xrow)[c];
-        sc.u = reinterpret_cast<const uint4*>(scale)[c];
-        if (KIND == NORM_LAYER && bias) bi.u = reinterpret_cast<const uint4*>(bias)[c];
+        in.u = ld_stream(reinterpret_cast<const v4u*>(xrow) + c);
+        sc.u = reinterpret_cast<const v4u*>(scale)[c];
+        if (KIND == NORM_LAYER && bias) bi.u = reinterpret_cast<const v4u*>(bias)[c];
 #pragma unroll
         for (int q = 0; q < 8; q++) out.e[q] = norm_one<T, KIND>(in.e[q], st, sc.e[q], bi.e[q], bias != nullptr);
-        reinterpret_cast<uint4*>(yrow)[c] = out.u;
+        st_stream(reinterpret_cast<v4u*>(yrow) + c, out.u);
     }
 }
 
@@ -387,7 +387,7 @@ __global__ void __launch_bounds__(BLOCK) gn_stats_kernel(const T* __restrict__ x
     for (uint32_t i = c0 + threadIdx.x * VE; i < c1; i += BLOCK * VE) {
         if (VE > 1) {
             Vec16<T> v;
-            v.u = *reinterpret_cast<const uint4*>(xs + i);
+            v.u = *reinterpret_cast<const v4u*>(xs + i);
 #pragma unroll
             for (int q = 0; q < VE; q++) acc += Ar<T>::widen(v.e[q]);
         } else {
@@ -408,7 +408,7 @@ __global__ void __launch_bounds__(BLOCK) gn_stats_kernel(const T* __restrict__ x
     for (uint32_t i = c0 + threadIdx.x * VE; i < c1; i += BLOCK * VE) {     // second pass: the slice is in cache
         if (VE > 1) {
             Vec16<T> v;
-            v.u = *reinterpret_cast<const uint4*>(xs + i);
+            v.u = *reinterpret_cast<const v4u*>(xs + i);
 #pragma unroll
             for (int q = 0; q < VE; q++) {
                 const float d = Ar<T>::widen(v.e[q]) - mean;
@@ -468,13 +468,13 @@ __global__ void __launch_bounds__(BLOCK) gn_apply_kernel(const T* __restrict__ x
         const float b = bias ? Ar<T>::widen(bias[c]) : 0.0f;
         if (VE > 1) {
             Vec16<T> v, o;
-            v.u = *reinterpret_cast<const uint4*>(xs + i);
+            v.u = *reinterpret_cast<const v4u*>(xs + i);
 #pragma unroll
             for (int q = 0; q < VE; q++) {
                 const float t = (Ar<T>::widen(v.e[q]) - meanf) * rstd;
                 o.e[q] = Ar<T>::conv(t * w + b);
             }
-            *reinterpret_cast<uint4*>(ys + i) = o.u;
+            st_stream(reinterpret_cast<v4u*>(ys + i), o.u);
         } else {
             const float t = (Ar<T>::widen(xs[i]) - meanf) * rstd;
             ys[i] = Ar<T>::conv(t * w + b);

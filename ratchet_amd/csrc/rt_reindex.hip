@@ -39,7 +39,7 @@ __global__ void __launch_bounds__(BLOCK) gather_vec_kernel(const VecT* __restric
 #pragma unroll
     for (int k = 0; k < UNROLL; k++) {
         const uint32_t v = base + k * BLOCK;
-        if (v < p.nvec) y[v] = r[k];
+        if (v < p.nvec) st_stream(y + v, r[k]);
     }
 }
 
@@ -61,7 +61,7 @@ __global__ void __launch_bounds__(BLOCK) gather_splat_kernel(const ElemT* __rest
             union { VecT v; ElemT e[PER]; } u;
 #pragma unroll
             for (int q = 0; q < PER; q++) u.e[q] = e;
-            y[v] = u.v;
+            st_stream(y + v, u.v);
         }
     }
 }
@@ -126,7 +126,7 @@ __global__ void __launch_bounds__(BLOCK) concat_kernel(VecT* __restrict__ y, Con
 #pragma unroll
     for (int u = 0; u < UNROLL; u++) {
         const uint32_t v = base + u * BLOCK;
-        if (v < nvec) r[u] = x[v];
+        if (v < nvec) r[u] = ld_stream(x + v);
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; u++) {
@@ -134,7 +134,7 @@ __global__ void __launch_bounds__(BLOCK) concat_kernel(VecT* __restrict__ y, Con
         if (v < nvec) {
             uint32_t row, col;
             fd_divmod(v, p.bv[k], row, col);
-            y[(uint64_t)row * p.dst_sv + p.dst_ov[k] + col] = r[u];
+            st_stream(y + ((uint64_t)row * p.dst_sv + p.dst_ov[k] + col), r[u]);
         }
     }
 }

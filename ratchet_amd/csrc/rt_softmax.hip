@@ -34,13 +34,13 @@ __global__ void __launch_bounds__(BLOCK) softmax_wave_kernel(const T* __restrict
     if (row >= rows) return;
     const int lane = threadIdx.x & (WAVE - 1);
     const uint32_t nvec = cols / VE;
-    const uint4* xr = reinterpret_cast<const uint4*>(x + row * cols);
-    uint4* yr = reinterpret_cast<uint4*>(y + row * cols);
+    const v4u* xr = reinterpret_cast<const v4u*>(x + row * cols);
+    v4u* yr = reinterpret_cast<v4u*>(y + row * cols);
     Vec16<T> v[NV];
 #pragma unroll
     for (int k = 0; k < NV; k++) {
         const uint32_t i = lane + k * WAVE;
-        if (i < nvec) v[k].u = xr[i];
+        if (i < nvec) v[k].u = ld_stream(xr + i);
     }
     float e[NV][VE];
     if (MODE == 1) {
@@ -69,7 +69,7 @@ __global__ void __launch_bounds__(BLOCK) softmax_wave_kernel(const T* __restrict
                 Vec16<T> o;
 #pragma unroll
                 for (int q = 0; q < VE; q++) o.e[q] = Ar<T>::conv(e[k][q] / s);
-                yr[i] = o.u;
+                st_stream(yr + i, o.u);
             }
         }
     } else {
@@ -94,7 +94,7 @@ __global__ void __launch_bounds__(BLOCK) softmax_wave_kernel(const T* __restrict
                 Vec16<T> o;
 #pragma unroll
                 for (int q = 0; q < VE; q++) o.e[q] = Ar<T>::conv(plain ? e[k][q] * rs : e[k][q] / s);
-                yr[i] = o.u;
+                st_stream(yr + i, o.u);
             }
         }
     }
@@ -172,10 +172,10 @@ __global__ void __launch_bounds__(BLOCK) softmax_seq16_kernel(const T* __restric
                 const T* src = x + (row0 + r) * cols + c0 + col;
                 if (VEC) {
                     Vec16<T> in, out;
-                    in.u = *reinterpret_cast<const uint4*>(src);
+                    in.u = *reinterpret_cast<const v4u*>(src);
 #pragma unroll
                     for (int q = 0; q < 8; q++) out.e[q] = ar_exp<T>(in.e[q]);
-                    *reinterpret_cast<uint4*>(&tile[r][col]) = out.u;
+                    *reinterpret_cast<v4u*>(&tile[r][col]) = out.u;
                 } else {
                     tile[r][col] = ar_exp<T>(*src);
                 }
@@ -188,7 +188,7 @@ __global__ void __launch_bounds__(BLOCK) softmax_seq16_kernel(const T* __restric
                 // ncol is a multiple of 8 here (cols % 8 == 0 and TC % 8 == 0)
                 for (uint32_t j = 0; j < ncol; j += 8) {
                     Vec16<T> t;
-                    t.u = *reinterpret_cast<const uint4*>(trow + j);
+                    t.u = *reinterpret_cast<const v4u*>(trow + j);
 #pragma unroll
                     for (int q = 0; q < 8; q++) run = Ar<T>::add(run, t.e[q]);
                 }
@@ -209,10 +209,10 @@ __global__ void __launch_bounds__(BLOCK) softmax_seq16_kernel(const T* __restric
         for (uint32_t cv = threadIdx.x; cv < cvec; cv += BLOCK) {
             if (VEC) {
                 Vec16<T> in, out;
-                in.u = reinterpret_cast<const uint4*>(src)[cv];
+                in.u = reinterpret_cast<const v4u*>(src)[cv];
 #pragma unroll
                 for (int q = 0; q < 8; q++) out.e[q] = Ar<T>::div(ar_exp<T>(in.e[q]), sum);
-                reinterpret_cast<uint4*>(dst)[cv] = out.u;
+                st_stream(reinterpret_cast<v4u*>(dst) + cv, out.u);
             } else {
                 dst[cv] = Ar<T>::div(ar_exp<T>(src[cv]), sum);
             }
@@ -336,7 +336,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
     auto load_x = [&](uint64_t g, uint32_t t, v4u& dst) {
         const uint64_t row = g * SP_ROWS + r;
         const uint32_t col = t * SP_TC + ccol;
-        if (g < ngroups && row < rows && col < cols) dst = *reinterpret_cast<const v4u*>(x + row * cols + col);
+        if (g < ngroups && row < rows && col < cols) dst = ld_stream(reinterpret_cast<const v4u*>(x + row * cols + col));
     };
 
     v4u e[NSLOT];                                            // exp values of the group in flight, 8 halves per slot
@@ -374,7 +374,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
                     out[w] = (uint32_t)h_bits((half_t)(e0 / s_prev)) | ((uint32_t)h_bits((half_t)(e1 / s_prev)) << 16);
                 }
             }
-            *reinterpret_cast<v4u*>(y + prev_row * cols + col) = out;
+            st_stream(reinterpret_cast<v4u*>(y + prev_row * cols + col), out);
         }
     };
     auto read_prev_sum = [&](uint32_t par) {
