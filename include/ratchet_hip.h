@@ -142,6 +142,32 @@ int rt_rms_norm(rt_device* dev, int dt, const void* x, const void* scale, void* 
 int rt_group_norm(rt_device* dev, int dt, const void* x, const void* scale, const void* bias, void* y, uint32_t B,
                   uint32_t C, uint32_t L, uint32_t groups, float eps);
 
+/* ---- Caller patterns in one pass --------------------------------------------------------------------------------
+ * The models wrap every 16-bit norm, softmax and activation in full() ... cast(dt): widen to f32, run the f32 op,
+ * round back.  These entry points produce what that op sequence produces (same rounding points: 16-bit add for the
+ * mask, f32 arithmetic inside, one rounding at the end) without the f32 tensors ever reaching memory.  io_dt is
+ * RT_F16 or RT_BF16. */
+
+/* x.full().layer_norm(w, b, eps).cast(dt) (kind 0) / x.full().rms_norm(w, eps).cast(dt) (kind 1): LayerNorm and
+ * RMSNorm modules, crates/ratchet-nn/src/norm.rs:35-44 and :61-70.  scale/bias are f32 (Norm::check_dtypes makes them
+ * match the widened input); bias may be NULL and is ignored for kind 1. */
+int rt_norm_via_f32(rt_device* dev, int kind, int io_dt, const void* x, const float* scale, const float* bias, void* y,
+                    uint64_t rows, uint32_t cols, float eps);
+
+/* scores.add(mask.cast(dt)).full().softmax(3).cast(dt): crates/ratchet-models/src/phi3/attn.rs:143-153,
+ * phi2/attn.rs:143-150, whisper/mha.rs:115-124.  mask may be NULL (no add); otherwise each mask extent is 1 or the
+ * scores' extent.  mode as rt_softmax. */
+int rt_softmax_via_f32(rt_device* dev, int io_dt, const void* x, const uint32_t x_shape[4], const void* mask,
+                       const uint32_t mask_shape[4], void* y, int mode);
+
+/* x.full().<op>().cast(dt) for any rt_unary op (activations: crates/ratchet-models/src/phi2/mlp.rs, whisper/residual_block.rs). */
+int rt_unary_via_f32(rt_device* dev, int op, int io_dt, const void* x, void* y, uint64_t numel);
+
+/* up.mul(gate.full().<op>().cast(dt)) with gate and up given as row-strided [rows, cols] views (strides in elements),
+ * so the two slices of the fused projection need no copies: crates/ratchet-models/src/phi3/mlp.rs:32-38. */
+int rt_gated_mul_via_f32(rt_device* dev, int op, int io_dt, const void* gate, uint64_t gate_row_stride, const void* up,
+                         uint64_t up_row_stride, void* y, uint64_t rows, uint32_t cols);
+
 #ifdef __cplusplus
 }
 #endif

@@ -117,7 +117,10 @@ int rt_device_destroy(rt_device* dev) {
     (void)hipStreamSynchronize(dev->stream);
     for (int t = 0; t < 2; t++)
         for (int i = 0; i < RT_UNARY_COUNT; i++)
+        {
             if (dev->unary_lut[t][i]) (void)hipFree(dev->unary_lut[t][i]);
+            if (dev->unary_lut_via32[t][i]) (void)hipFree(dev->unary_lut_via32[t][i]);
+        }
     if (dev->gn_scratch) (void)hipFree(dev->gn_scratch);
     hipError_t e = hipStreamDestroy(dev->stream);
     delete dev;

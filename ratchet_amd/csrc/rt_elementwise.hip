@@ -143,7 +143,13 @@ __global__ void __launch_bounds__(BLOCK) binary_bcast_kernel(const T* __restrict
 }
 
 // ------------------------------------------------------------------------------------------------ unary
-template <typename T, int OP>
+// VIA32: the caller pattern x.full().<op>().cast(dt) on a 16-bit tensor in one pass: widen, the f32 op, one rounding
+template <typename T, int OP, bool VIA32> __device__ __forceinline__ T apply_unary(T v) {
+    if (VIA32) return Ar<T>::conv(ar_unary<OP, float>(Ar<T>::widen(v)));
+    return ar_unary<OP, T>(v);
+}
+
+template <typename T, int OP, bool VIA32>
 __global__ void __launch_bounds__(BLOCK) unary_vec_kernel(const T* __restrict__ x, T* y, uint64_t numel) {
     constexpr int VE = 16 / sizeof(T);
     const uint64_t nvec = numel / VE;
@@ -162,20 +168,20 @@ __global__ void __launch_bounds__(BLOCK) unary_vec_kernel(const T* __restrict__ 
         if (i < nvec) {
             Vec16<T> r;
 #pragma unroll
-            for (int e = 0; e < VE; e++) r.e[e] = ar_unary<OP, T>(rx[k].e[e]);
+            for (int e = 0; e < VE; e++) r.e[e] = apply_unary<T, OP, VIA32>(rx[k].e[e]);
             st_stream(yv + i, r.u);
         }
     }
     if (blockIdx.x == 0) {
         const uint64_t i = nvec * VE + threadIdx.x;
-        if (i < numel) y[i] = ar_unary<OP, T>(x[i]);
+        if (i < numel) y[i] = apply_unary<T, OP, VIA32>(x[i]);
     }
 }
 
-template <typename T, int OP>
+template <typename T, int OP, bool VIA32>
 __global__ void __launch_bounds__(BLOCK) unary_scalar_kernel(const T* x, T* y, uint64_t numel) {
     const uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
-    if (i < numel) y[i] = ar_unary<OP, T>(x[i]);
+    if (i < numel) y[i] = apply_unary<T, OP, VIA32>(x[i]);
 }
 
 // ------------------------------------------------------------------------------------------------ unary via lookup table
@@ -234,6 +240,59 @@ __global__ void __launch_bounds__(LUT_BLOCK) unary_lut_kernel(const uint16_t* __
         const uint64_t i = nvec * 8 + threadIdx.x;
         if (i < numel) y[i] = lut[x[i]];
     }
+}
+
+// ------------------------------------------------------------------------------------------------ gated multiply
+// y[r, c] = up[r, c] * act(gate[r, c]) with act = cast(op(full(gate))), the feed-forward gate of phi3
+// (ratchet-models/src/phi3/mlp.rs:32-38: up.mul(gate.full().silu().cast(dt)) on the two halves of one projection).
+// gate and up are row-strided views, so the two slices are never materialised.  act comes from the same kind of LDS
+// table as unary_lut_kernel (built by the exact kernels for "widen, f32 op, round"); the product is the type's own.
+struct GatedArgs {
+    FastDiv cv;              // vectors (or elements, scalar kernel) per row
+    uint64_t gs, us;         // row strides of gate and up, in elements
+    uint64_t nvec;           // rows * vectors per row
+};
+
+template <typename T>
+__global__ void __launch_bounds__(LUT_BLOCK) gated_lut_kernel(const uint16_t* __restrict__ table, const T* __restrict__ gate,
+                                                              const T* __restrict__ up, T* __restrict__ y, GatedArgs p) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t lut[];
+    {
+        const v4u* src = reinterpret_cast<const v4u*>(table);
+        v4u* dst = reinterpret_cast<v4u*>(lut);
+#pragma unroll
+        for (int i = 0; i < (int)(LUT_BYTES / 16 / LUT_BLOCK); i++) dst[i * LUT_BLOCK + threadIdx.x] = src[i * LUT_BLOCK + threadIdx.x];
+    }
+    __syncthreads();
+    const uint64_t stride = (uint64_t)gridDim.x * LUT_BLOCK;
+    for (uint64_t v = (uint64_t)blockIdx.x * LUT_BLOCK + threadIdx.x; v < p.nvec; v += stride) {
+        uint32_t row, c;
+        fd_divmod((uint32_t)v, p.cv, row, c);
+        Vec16<T> g, u, o;
+        g.u = ld_stream(reinterpret_cast<const v4u*>(gate + (uint64_t)row * p.gs) + c);
+        u.u = ld_stream(reinterpret_cast<const v4u*>(up + (uint64_t)row * p.us) + c);
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const uint32_t lo = lut[g.u[w] & 0xffffu];
+            const uint32_t hi = lut[g.u[w] >> 16];
+            g.u[w] = lo | (hi << 16);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) o.e[e] = Ar<T>::mul(u.e[e], g.e[e]);
+        st_stream(reinterpret_cast<v4u*>(y) + v, o.u);
+    }
+}
+
+// any size / alignment: one element per thread, computed directly
+template <typename T, int OP>
+__global__ void __launch_bounds__(BLOCK) gated_scalar_kernel(const T* __restrict__ gate, const T* __restrict__ up, T* __restrict__ y,
+                                                             GatedArgs p) {
+    const uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+    if (i >= p.nvec) return;
+    uint32_t row, c;
+    fd_divmod((uint32_t)i, p.cv, row, c);
+    const T act = apply_unary<T, OP, true>(gate[(uint64_t)row * p.gs + c]);
+    y[i] = Ar<T>::mul(up[(uint64_t)row * p.us + c], act);
 }
 
 // ------------------------------------------------------------------------------------------------ cast
@@ -342,24 +401,24 @@ int dispatch_binary(rt_device* dev, int op, const void* a, const void* b, void* 
     }
 }
 
-template <typename T, int OP>
+template <typename T, int OP, bool VIA32>
 int launch_unary(rt_device* dev, const void* x, void* y, uint64_t numel) {
     const bool vec = rt_aligned(x, 16) && rt_aligned(y, 16);
     if (vec) {
         constexpr int VE = 16 / sizeof(T);
-        hipLaunchKernelGGL((unary_vec_kernel<T, OP>), dim3(blocks_for(numel / VE, BLOCK * UNROLL)), dim3(BLOCK), 0,
+        hipLaunchKernelGGL((unary_vec_kernel<T, OP, VIA32>), dim3(blocks_for(numel / VE, BLOCK * UNROLL)), dim3(BLOCK), 0,
                            dev->stream, (const T*)x, (T*)y, numel);
     } else {
-        hipLaunchKernelGGL((unary_scalar_kernel<T, OP>), dim3(blocks_for(numel, BLOCK)), dim3(BLOCK), 0, dev->stream,
+        hipLaunchKernelGGL((unary_scalar_kernel<T, OP, VIA32>), dim3(blocks_for(numel, BLOCK)), dim3(BLOCK), 0, dev->stream,
                            (const T*)x, (T*)y, numel);
     }
     RT_CHECK_LAUNCH("unary kernel");
     return RT_OK;
 }
 
-template <typename T> int dispatch_unary(rt_device* dev, int op, const void* x, void* y, uint64_t numel) {
+template <typename T, bool VIA32 = false> int dispatch_unary(rt_device* dev, int op, const void* x, void* y, uint64_t numel) {
     switch (op) {
-#define RT_CASE(OPC) case OPC: return launch_unary<T, OPC>(dev, x, y, numel);
+#define RT_CASE(OPC) case OPC: return launch_unary<T, OPC, VIA32>(dev, x, y, numel);
         RT_CASE(RT_GELU) RT_CASE(RT_TANH) RT_CASE(RT_EXP) RT_CASE(RT_LOG) RT_CASE(RT_SIN) RT_CASE(RT_COS)
         RT_CASE(RT_ABS) RT_CASE(RT_SQRT) RT_CASE(RT_RELU) RT_CASE(RT_FLOOR) RT_CASE(RT_CEIL) RT_CASE(RT_NEG)
         RT_CASE(RT_SILU) RT_CASE(RT_SIGMOID)
@@ -377,8 +436,9 @@ inline bool lut_worthwhile(int op) {
     }
 }
 
-template <typename T> int build_unary_table(rt_device* dev, int ti, int op) {
-    if (dev->unary_lut[ti][op]) return RT_OK;
+template <typename T, bool VIA32 = false> int build_unary_table(rt_device* dev, int ti, int op) {
+    uint16_t*& slot = VIA32 ? dev->unary_lut_via32[ti][op] : dev->unary_lut[ti][op];
+    if (slot) return RT_OK;
     uint16_t* table = nullptr;
     uint16_t* iota = nullptr;
     RT_HIP(hipMalloc((void**)&table, LUT_BYTES));
@@ -388,20 +448,20 @@ template <typename T> int build_unary_table(rt_device* dev, int ti, int op) {
         return rt_fail_hip(e, "hipMalloc(lut)");
     }
     hipLaunchKernelGGL(iota16_kernel, dim3(65536 / 256), dim3(256), 0, dev->stream, iota);
-    int rc = dispatch_unary<T>(dev, op, iota, table, 65536);          // the exact kernel defines the table
+    int rc = dispatch_unary<T, VIA32>(dev, op, iota, table, 65536);   // the exact kernel defines the table
     hipError_t es = hipStreamSynchronize(dev->stream);
     (void)hipFree(iota);
     if (rc != RT_OK || es != hipSuccess) {
         (void)hipFree(table);
         return rc != RT_OK ? rc : rt_fail_hip(es, "building the unary lookup table");
     }
-    dev->unary_lut[ti][op] = table;
+    slot = table;
     return RT_OK;
 }
 
-template <typename T> int unary_via_lut(rt_device* dev, int op, const void* x, void* y, uint64_t numel) {
+template <typename T, bool VIA32 = false> int unary_via_lut(rt_device* dev, int op, const void* x, void* y, uint64_t numel) {
     const int ti = std::is_same<T, bf16_t>::value ? 1 : 0;
-    int rc = build_unary_table<T>(dev, ti, op);
+    int rc = build_unary_table<T, VIA32>(dev, ti, op);
     if (rc) return rc;
     if (!dev->lut_attr_set) {
         RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(unary_lut_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -412,8 +472,49 @@ template <typename T> int unary_via_lut(rt_device* dev, int op, const void* x, v
     if (blocks > (uint64_t)dev->num_cus) blocks = dev->num_cus;          // one resident block per CU (128 KiB of LDS each)
     if (blocks < 1) blocks = 1;
     hipLaunchKernelGGL(unary_lut_kernel, dim3((unsigned)blocks), dim3(LUT_BLOCK), LUT_BYTES, dev->stream,
-                       (const uint16_t*)dev->unary_lut[ti][op], (const uint16_t*)x, (uint16_t*)y, numel);
+                       (const uint16_t*)(VIA32 ? dev->unary_lut_via32[ti][op] : dev->unary_lut[ti][op]), (const uint16_t*)x,
+                       (uint16_t*)y, numel);
     RT_CHECK_LAUNCH("unary_lut_kernel");
+    return RT_OK;
+}
+
+template <typename T>
+int launch_gated(rt_device* dev, int op, const void* gate, uint64_t gs, const void* up, uint64_t us, void* y, uint64_t rows, uint32_t cols) {
+    const int ti = std::is_same<T, bf16_t>::value ? 1 : 0;
+    const uint64_t numel = rows * cols;
+    GatedArgs p;
+    p.gs = gs;
+    p.us = us;
+    const bool vec = cols % 8 == 0 && gs % 8 == 0 && us % 8 == 0 && rt_aligned(gate, 16) && rt_aligned(up, 16) && rt_aligned(y, 16);
+    if (vec && numel >= RT_LUT_MIN_NUMEL) {
+        int rc = build_unary_table<T, true>(dev, ti, op);
+        if (rc) return rc;
+        if (!dev->gated_attr_set[ti]) {
+            RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gated_lut_kernel<T>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)LUT_BYTES));
+            dev->gated_attr_set[ti] = 1;
+        }
+        p.cv = make_fastdiv(cols / 8);
+        p.nvec = numel / 8;
+        uint64_t blocks = (p.nvec + LUT_BLOCK - 1) / LUT_BLOCK;
+        if (blocks > (uint64_t)dev->num_cus) blocks = dev->num_cus;
+        hipLaunchKernelGGL((gated_lut_kernel<T>), dim3((unsigned)blocks), dim3(LUT_BLOCK), LUT_BYTES, dev->stream,
+                           (const uint16_t*)dev->unary_lut_via32[ti][op], (const T*)gate, (const T*)up, (T*)y, p);
+        RT_CHECK_LAUNCH("gated_lut_kernel");
+        return RT_OK;
+    }
+    p.cv = make_fastdiv(cols);
+    p.nvec = numel;
+    const dim3 grid(blocks_for(numel, BLOCK)), block(BLOCK);
+    switch (op) {
+#define RT_CASE(OPC) case OPC: hipLaunchKernelGGL((gated_scalar_kernel<T, OPC>), grid, block, 0, dev->stream, (const T*)gate, (const T*)up, (T*)y, p); break;
+        RT_CASE(RT_GELU) RT_CASE(RT_TANH) RT_CASE(RT_EXP) RT_CASE(RT_LOG) RT_CASE(RT_SIN) RT_CASE(RT_COS)
+        RT_CASE(RT_ABS) RT_CASE(RT_SQRT) RT_CASE(RT_RELU) RT_CASE(RT_FLOOR) RT_CASE(RT_CEIL) RT_CASE(RT_NEG)
+        RT_CASE(RT_SILU) RT_CASE(RT_SIGMOID)
+#undef RT_CASE
+        default: return rt_fail(RT_ERR_OP, "rt_gated_mul_via_f32: op %d out of range", op);
+    }
+    RT_CHECK_LAUNCH("gated_scalar_kernel");
     return RT_OK;
 }
 
@@ -605,6 +706,38 @@ int rt_unary(rt_device* dev, int op, int dt, const void* x, void* y, uint64_t nu
         case RT_F16: return lut ? unary_via_lut<half_t>(dev, op, x, y, numel) : dispatch_unary<half_t>(dev, op, x, y, numel);
         default: return lut ? unary_via_lut<bf16_t>(dev, op, x, y, numel) : dispatch_unary<bf16_t>(dev, op, x, y, numel);
     }
+}
+
+int rt_unary_via_f32(rt_device* dev, int op, int io_dt, const void* x, void* y, uint64_t numel) {
+    RT_REQUIRE(op >= 0 && op < RT_UNARY_COUNT, RT_ERR_OP, "rt_unary_via_f32: op %d out of range", op);
+    RT_REQUIRE(io_dt == RT_F16 || io_dt == RT_BF16, RT_ERR_DTYPE, "rt_unary_via_f32: dtype %d is not F16/BF16", io_dt);
+    RT_REQUIRE(numel <= RT_MAX_NUMEL, RT_ERR_SIZE, "rt_unary_via_f32: numel %llu too large", (unsigned long long)numel);
+    if (numel == 0) return dev ? RT_OK : rt_fail(RT_ERR_NULL_DEVICE, "rt_device is NULL");
+    RT_REQUIRE(x && y, RT_ERR_NULL_POINTER, "rt_unary_via_f32: NULL operand");
+    RT_REQUIRE(rt_aligned(x, 2) && rt_aligned(y, 2), RT_ERR_ALIGN, "rt_unary_via_f32: misaligned pointer");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    const bool lut = numel >= RT_LUT_MIN_NUMEL && lut_worthwhile(op) && rt_aligned(x, 16) && rt_aligned(y, 16);
+    if (io_dt == RT_F16) return lut ? unary_via_lut<half_t, true>(dev, op, x, y, numel) : dispatch_unary<half_t, true>(dev, op, x, y, numel);
+    return lut ? unary_via_lut<bf16_t, true>(dev, op, x, y, numel) : dispatch_unary<bf16_t, true>(dev, op, x, y, numel);
+}
+
+int rt_gated_mul_via_f32(rt_device* dev, int op, int io_dt, const void* gate, uint64_t gate_row_stride, const void* up,
+                         uint64_t up_row_stride, void* y, uint64_t rows, uint32_t cols) {
+    RT_REQUIRE(op >= 0 && op < RT_UNARY_COUNT, RT_ERR_OP, "rt_gated_mul_via_f32: op %d out of range", op);
+    RT_REQUIRE(io_dt == RT_F16 || io_dt == RT_BF16, RT_ERR_DTYPE, "rt_gated_mul_via_f32: dtype %d is not F16/BF16", io_dt);
+    RT_REQUIRE(cols > 0 || rows == 0, RT_ERR_SHAPE, "rt_gated_mul_via_f32: cols is 0");
+    RT_REQUIRE(gate_row_stride >= cols && up_row_stride >= cols, RT_ERR_SHAPE, "rt_gated_mul_via_f32: a row stride is shorter than a row");
+    RT_REQUIRE(rows <= RT_MAX_NUMEL && rows * (uint64_t)cols <= 0xffffffffull && rows * gate_row_stride <= RT_MAX_NUMEL &&
+                   rows * up_row_stride <= RT_MAX_NUMEL,
+               RT_ERR_SIZE, "rt_gated_mul_via_f32: tensor too large");
+    if (rows == 0) return dev ? RT_OK : rt_fail(RT_ERR_NULL_DEVICE, "rt_device is NULL");
+    RT_REQUIRE(gate && up && y, RT_ERR_NULL_POINTER, "rt_gated_mul_via_f32: NULL operand");
+    RT_REQUIRE(rt_aligned(gate, 2) && rt_aligned(up, 2) && rt_aligned(y, 2), RT_ERR_ALIGN, "rt_gated_mul_via_f32: misaligned pointer");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    if (io_dt == RT_F16) return launch_gated<half_t>(dev, op, gate, gate_row_stride, up, up_row_stride, y, rows, cols);
+    return launch_gated<bf16_t>(dev, op, gate, gate_row_stride, up, up_row_stride, y, rows, cols);
 }
 
 int rt_cast(rt_device* dev, int src_dt, int dst_dt, const void* x, void* y, uint64_t numel) {

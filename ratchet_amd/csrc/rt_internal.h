@@ -17,7 +17,10 @@ struct rt_device {
     size_t gn_scratch_bytes;
     // 65536-entry 16-bit -> 16-bit lookup tables, built on first use by the exact kernels ([0] = f16, [1] = bf16)
     uint16_t* unary_lut[2][RT_UNARY_COUNT];
+    // the same for "widen to f32, f32 op, round once" (the full -> op -> cast caller pattern)
+    uint16_t* unary_lut_via32[2][RT_UNARY_COUNT];
     int lut_attr_set;
+    int gated_attr_set[2];
 };
 
 struct rt_event {

@@ -136,6 +136,93 @@ __global__ void __launch_bounds__(BLOCK) norm_generic_kernel(const T* __restrict
 }
 
 // ------------------------------------------------------------------------------------------------------------------
+// The caller pattern of ratchet-nn (src/norm.rs:35-44, 61-70): x.full().layer_norm(w, b, eps).cast(src_dt) on a
+// 16-bit x with f32 weights, in one pass: the row is widened into registers, the f32 norm arithmetic above is applied
+// (butterfly sums) and the result is rounded once.  4 bytes of traffic per element instead of the 16 of the three
+// separate ops, and no sequential chain: the f32 sums need no replay because the parity bar after the cast is the
+// 16-bit one.
+// ------------------------------------------------------------------------------------------------------------------
+template <typename T, int NV, int KIND>
+__global__ void __launch_bounds__(BLOCK) norm_via32_wave_kernel(const T* __restrict__ x, const float* __restrict__ scale,
+                                                                const float* __restrict__ bias, T* __restrict__ y, uint64_t rows,
+                                                                uint32_t cols, float eps) {
+    const uint64_t row = (uint64_t)blockIdx.x * WAVES + (threadIdx.x / WAVE);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & (WAVE - 1);
+    const uint32_t nvec = cols / 8;
+    const v4u* xr = reinterpret_cast<const v4u*>(x + row * cols);
+    v4u* yr = reinterpret_cast<v4u*>(y + row * cols);
+    Vec16<T> v[NV];
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        const uint32_t i = lane + k * WAVE;
+        if (i < nvec) v[k].u = ld_stream(xr + i);
+    }
+    float sx = 0.0f, sq = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NV; k++)
+        if (lane + k * WAVE < nvec)
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                const float e = Ar<T>::widen(v[k].e[q]);
+                if (KIND == NORM_LAYER) sx += e;
+                sq += e * e;
+            }
+    if (KIND == NORM_LAYER) sx = wave_sum(sx);
+    sq = wave_sum(sq);
+    const RowStats<float> st = finish_stats<float, KIND>(sx, sq, cols, eps);
+    const float4* sv = reinterpret_cast<const float4*>(scale);
+    const float4* bv = reinterpret_cast<const float4*>(bias);
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        const uint32_t i = lane + k * WAVE;
+        if (i < nvec) {
+            float s[8], b[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            *reinterpret_cast<float4*>(s) = sv[2 * i];
+            *reinterpret_cast<float4*>(s + 4) = sv[2 * i + 1];
+            if (KIND == NORM_LAYER && bias) {
+                *reinterpret_cast<float4*>(b) = bv[2 * i];
+                *reinterpret_cast<float4*>(b + 4) = bv[2 * i + 1];
+            }
+            Vec16<T> o;
+#pragma unroll
+            for (int q = 0; q < 8; q++)
+                o.e[q] = Ar<T>::conv(norm_one<float, KIND>(Ar<T>::widen(v[k].e[q]), st, s[q], b[q], bias != nullptr));
+            st_stream(yr + i, o.u);
+        }
+    }
+}
+
+// any cols / alignment: one block per row, scalar accesses, the row is re-read from cache for the second pass
+template <typename T, int KIND>
+__global__ void __launch_bounds__(BLOCK) norm_via32_generic_kernel(const T* __restrict__ x, const float* __restrict__ scale,
+                                                                   const float* __restrict__ bias, T* __restrict__ y, uint64_t rows,
+                                                                   uint32_t cols, float eps) {
+    __shared__ float red[2][WAVES];
+    const uint64_t row = blockIdx.x;
+    const T* xr = x + row * cols;
+    T* yr = y + row * cols;
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    float sx = 0.0f, sq = 0.0f;
+    for (uint32_t j = threadIdx.x; j < cols; j += BLOCK) {
+        const float e = Ar<T>::widen(xr[j]);
+        sx += e;
+        sq += e * e;
+    }
+    sx = wave_sum(sx);
+    sq = wave_sum(sq);
+    if (lane == 0) { red[0][wave] = sx; red[1][wave] = sq; }
+    __syncthreads();
+    sx = red[0][0]; sq = red[1][0];
+    for (int w = 1; w < WAVES; w++) { sx += red[0][w]; sq += red[1][w]; }
+    const RowStats<float> st = finish_stats<float, KIND>(sx, sq, cols, eps);
+    for (uint32_t j = threadIdx.x; j < cols; j += BLOCK) {
+        const float b = (KIND == NORM_LAYER && bias) ? bias[j] : 0.0f;
+        yr[j] = Ar<T>::conv(norm_one<float, KIND>(Ar<T>::widen(xr[j]), st, scale[j], b, bias != nullptr));
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------------
 // 16-bit LayerNorm / RMSNorm with the reference's sequential f32 accumulation.
 // A block owns RB consecutive rows.  Pass A: per column tile, all threads load 16-byte vectors, widen x and T(x*x) to
 // f32 and park them in LDS; lanes [0, RB) then add the squares of "their" row left to right, lanes [RB, 2RB) the values
@@ -613,9 +700,57 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
     return RT_OK;
 }
 
+template <typename T, int KIND>
+int launch_norm_via32(rt_device* dev, const void* x, const float* scale, const float* bias, void* y, uint64_t rows, uint32_t cols, float eps) {
+    const uint32_t nvec = cols / 8;
+    const bool vec_ok = (cols % 8 == 0) && rt_aligned(x, 16) && rt_aligned(y, 16) && rt_aligned(scale, 16) && (!bias || rt_aligned(bias, 16)) &&
+                        nvec <= (uint32_t)(WAVE * 8);
+    if (vec_ok) {
+        const uint32_t nv = (nvec + WAVE - 1) / WAVE;
+        const uint64_t blocks = (rows + WAVES - 1) / WAVES;
+        RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_norm_via_f32: too many rows");
+        const dim3 grid((unsigned)blocks), block(BLOCK);
+#define RT_NV(NVC) hipLaunchKernelGGL((norm_via32_wave_kernel<T, NVC, KIND>), grid, block, 0, dev->stream, (const T*)x, scale, bias, (T*)y, rows, cols, eps)
+        if (nv <= 1) RT_NV(1);
+        else if (nv <= 2) RT_NV(2);
+        else if (nv <= 4) RT_NV(4);
+        else if (nv <= 6) RT_NV(6);
+        else RT_NV(8);
+#undef RT_NV
+        RT_CHECK_LAUNCH("norm_via32_wave_kernel");
+        return RT_OK;
+    }
+    RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "rt_norm_via_f32: too many rows");
+    hipLaunchKernelGGL((norm_via32_generic_kernel<T, KIND>), dim3((unsigned)rows), dim3(BLOCK), 0, dev->stream, (const T*)x, scale, bias,
+                       (T*)y, rows, cols, eps);
+    RT_CHECK_LAUNCH("norm_via32_generic_kernel");
+    return RT_OK;
+}
+
 }  // namespace
 
 extern "C" {
+
+int rt_norm_via_f32(rt_device* dev, int kind, int io_dt, const void* x, const float* scale, const float* bias, void* y, uint64_t rows,
+                    uint32_t cols, float eps) {
+    RT_REQUIRE(kind == NORM_LAYER || kind == NORM_RMS, RT_ERR_ARG, "rt_norm_via_f32: kind %d is not 0 (layer) or 1 (rms)", kind);
+    RT_REQUIRE(io_dt == RT_F16 || io_dt == RT_BF16, RT_ERR_DTYPE, "rt_norm_via_f32: dtype %d is not F16/BF16", io_dt);
+    RT_REQUIRE(cols > 0, RT_ERR_SHAPE, "rt_norm_via_f32: cols is 0");
+    RT_REQUIRE(rows <= RT_MAX_NUMEL / cols, RT_ERR_SIZE, "rt_norm_via_f32: tensor too large");
+    RT_REQUIRE(eps == eps, RT_ERR_ARG, "rt_norm_via_f32: eps is NaN");
+    if (rows == 0) return dev ? RT_OK : rt_fail(RT_ERR_NULL_DEVICE, "rt_device is NULL");
+    RT_REQUIRE(x && scale && y, RT_ERR_NULL_POINTER, "rt_norm_via_f32: NULL operand");
+    RT_REQUIRE(rt_aligned(x, 2) && rt_aligned(y, 2) && rt_aligned(scale, 4) && (!bias || rt_aligned(bias, 4)), RT_ERR_ALIGN,
+               "rt_norm_via_f32: misaligned pointer");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    if (kind == NORM_RMS) bias = nullptr;
+    if (io_dt == RT_F16)
+        return kind == NORM_LAYER ? launch_norm_via32<half_t, NORM_LAYER>(dev, x, scale, bias, y, rows, cols, eps)
+                                  : launch_norm_via32<half_t, NORM_RMS>(dev, x, scale, bias, y, rows, cols, eps);
+    return kind == NORM_LAYER ? launch_norm_via32<bf16_t, NORM_LAYER>(dev, x, scale, bias, y, rows, cols, eps)
+                              : launch_norm_via32<bf16_t, NORM_RMS>(dev, x, scale, bias, y, rows, cols, eps);
+}
 
 int rt_layer_norm(rt_device* dev, int dt, const void* x, const void* scale, const void* bias, void* y, uint64_t rows, uint32_t cols,
                   float eps) {

@@ -429,6 +429,156 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
     }
 }
 
+// ------------------------------------------------------------------------------------------------------------------
+// The attention caller pattern (ratchet-models/src/phi3/attn.rs:148-153, phi2/attn.rs:143-150, whisper/mha.rs:115-124):
+//     w = scores.add(mask.cast(dt)).full().softmax(3).cast(dt)
+// on 16-bit scores in one pass: the mask (broadcast over batch / heads, optional) is added in the 16-bit type as the
+// separate add would, the sum is widened, the f32 softmax above is applied in registers and the result rounded once.
+// 4 bytes of HBM traffic per element against 26 for the four separate ops (6 + 6 + 8 + 6).
+// Blocks take the XCD-aware order of binary_bcast_kernel so that the heads sharing a mask row run on one XCD.
+// ------------------------------------------------------------------------------------------------------------------
+struct MaskArgs {
+    FastDiv d2, d1;          // x extents of dims 2 and 1 (rows = d0 * d1 * d2)
+    uint32_t ms[3];          // mask row strides in elements over dims 0..2 (0 where the mask extent is 1)
+    uint32_t mlast;          // 1: the mask has a full last dim, 0: one value per row
+    FastDiv reps;            // XCD-aware order (see BcastArgs in the elementwise kernels); slabs == 0: identity
+    uint32_t slabs;
+};
+constexpr uint32_t SM_XCDS = 8;
+
+template <typename T> __device__ __forceinline__ uint64_t mask_row_offset(uint64_t row, const MaskArgs& p) {
+    uint32_t t, i2, i1, i0;
+    fd_divmod((uint32_t)row, p.d2, t, i2);
+    fd_divmod(t, p.d1, i0, i1);
+    return (uint64_t)i0 * p.ms[0] + (uint64_t)i1 * p.ms[1] + (uint64_t)i2 * p.ms[2];
+}
+
+template <typename T, int NV, int MODE, bool MASK>
+__global__ void __launch_bounds__(BLOCK) softmax_via32_wave_kernel(const T* __restrict__ x, const T* __restrict__ mask,
+                                                                   T* __restrict__ y, uint64_t rows, uint32_t cols, MaskArgs p) {
+    uint32_t blk = blockIdx.x;
+    if (MASK && p.slabs) {
+        uint32_t rep, grp;
+        fd_divmod(blk / SM_XCDS, p.reps, grp, rep);
+        blk = rep * p.slabs + grp * SM_XCDS + (blk % SM_XCDS);
+    }
+    const uint64_t row = (uint64_t)blk * WAVES + (threadIdx.x / WAVE);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & (WAVE - 1);
+    const uint32_t nvec = cols / 8;
+    const v4u* xr = reinterpret_cast<const v4u*>(x + row * cols);
+    v4u* yr = reinterpret_cast<v4u*>(y + row * cols);
+    Vec16<T> v[NV];
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        const uint32_t i = lane + k * WAVE;
+        if (i < nvec) v[k].u = ld_stream(xr + i);
+    }
+    if (MASK) {
+        const T* mr = mask + mask_row_offset<T>(row, p);
+        if (p.mlast) {
+            const v4u* mv = reinterpret_cast<const v4u*>(mr);
+#pragma unroll
+            for (int k = 0; k < NV; k++) {
+                const uint32_t i = lane + k * WAVE;
+                if (i < nvec) {
+                    Vec16<T> m;
+                    m.u = mv[i];
+#pragma unroll
+                    for (int q = 0; q < 8; q++) v[k].e[q] = Ar<T>::add(v[k].e[q], m.e[q]);
+                }
+            }
+        } else {
+            const T m = mr[0];
+#pragma unroll
+            for (int k = 0; k < NV; k++)
+#pragma unroll
+                for (int q = 0; q < 8; q++) v[k].e[q] = Ar<T>::add(v[k].e[q], m);
+        }
+    }
+    float e[NV][8];
+    float m = 0.0f;
+    if (MODE == 1) {
+        m = -__builtin_huge_valf();
+#pragma unroll
+        for (int k = 0; k < NV; k++)
+            if (lane + k * WAVE < nvec)
+#pragma unroll
+                for (int q = 0; q < 8; q++) m = fmaxf(m, Ar<T>::widen(v[k].e[q]));
+        m = wave_max(m);
+        if (m == -__builtin_huge_valf()) m = 0.0f;
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NV; k++)
+        if (lane + k * WAVE < nvec)
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                e[k][q] = expf(Ar<T>::widen(v[k].e[q]) - m);
+                s += e[k][q];
+            }
+    s = wave_sum(s);
+    const bool plain = (s >= 1.17549435e-38f) && (s < __builtin_huge_valf());
+    const float rs = 1.0f / s;
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        const uint32_t i = lane + k * WAVE;
+        if (i < nvec) {
+            Vec16<T> o;
+#pragma unroll
+            for (int q = 0; q < 8; q++) o.e[q] = Ar<T>::conv(plain ? e[k][q] * rs : e[k][q] / s);
+            st_stream(yr + i, o.u);
+        }
+    }
+}
+
+// any cols / alignment: one block per row, scalar accesses, the row re-read from cache between passes
+template <typename T, int MODE, bool MASK>
+__global__ void __launch_bounds__(BLOCK) softmax_via32_generic_kernel(const T* __restrict__ x, const T* __restrict__ mask,
+                                                                      T* __restrict__ y, uint64_t rows, uint32_t cols, MaskArgs p) {
+    __shared__ float red[WAVES];
+    __shared__ float bcast;
+    const uint64_t row = blockIdx.x;
+    const T* xr = x + row * cols;
+    T* yr = y + row * cols;
+    const T* mr = MASK ? mask + mask_row_offset<T>(row, p) : nullptr;
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    auto elem = [&](uint32_t j) -> float {
+        T v = xr[j];
+        if (MASK) v = Ar<T>::add(v, mr[p.mlast ? j : 0]);
+        return Ar<T>::widen(v);
+    };
+    float m = 0.0f;
+    if (MODE == 1) {
+        float lm = -__builtin_huge_valf();
+        for (uint32_t j = threadIdx.x; j < cols; j += BLOCK) lm = fmaxf(lm, elem(j));
+        lm = wave_max(lm);
+        if (lane == 0) red[wave] = lm;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float t = red[0];
+            for (int w = 1; w < WAVES; w++) t = fmaxf(t, red[w]);
+            bcast = (t == -__builtin_huge_valf()) ? 0.0f : t;
+        }
+        __syncthreads();
+        m = bcast;
+        __syncthreads();
+    }
+    float s = 0.0f;
+    for (uint32_t j = threadIdx.x; j < cols; j += BLOCK) s += expf(elem(j) - m);
+    s = wave_sum(s);
+    if (lane == 0) red[wave] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = red[0];
+        for (int w = 1; w < WAVES; w++) t += red[w];
+        bcast = t;
+    }
+    __syncthreads();
+    s = bcast;
+    for (uint32_t j = threadIdx.x; j < cols; j += BLOCK) yr[j] = Ar<T>::conv(expf(elem(j) - m) / s);
+}
+
 template <typename T, int MODE> int launch_wave(rt_device* dev, const void* x, void* y, uint64_t rows, uint32_t cols) {
     constexpr int VE = 16 / sizeof(T);
     const uint32_t nvec = cols / VE;
@@ -502,7 +652,107 @@ template <typename T> int launch_seq16(rt_device* dev, const void* x, void* y, u
     return RT_OK;
 }
 
+template <typename T, int MODE, bool MASK>
+int launch_via32(rt_device* dev, const void* x, const void* mask, void* y, uint64_t rows, uint32_t cols, const MaskArgs& p, bool mask_vec_ok) {
+    const uint32_t nvec = cols / 8;
+    const bool vec_ok = (cols % 8 == 0) && rt_aligned(x, 16) && rt_aligned(y, 16) && nvec <= (uint32_t)(WAVE * 8) && (!MASK || mask_vec_ok);
+    if (vec_ok) {
+        const uint32_t nv = (nvec + WAVE - 1) / WAVE;
+        const uint64_t blocks = (rows + WAVES - 1) / WAVES;
+        RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax_via_f32: too many rows");
+        const dim3 grid((unsigned)blocks), block(BLOCK);
+#define RT_SV(NVC)                                                                                                                 \
+    hipLaunchKernelGGL((softmax_via32_wave_kernel<T, NVC, MODE, MASK>), grid, block, 0, dev->stream, (const T*)x, (const T*)mask, (T*)y, \
+                       rows, cols, p)
+        if (nv <= 1) RT_SV(1);
+        else if (nv <= 2) RT_SV(2);
+        else if (nv <= 4) RT_SV(4);
+        else if (nv <= 6) RT_SV(6);
+        else RT_SV(8);
+#undef RT_SV
+        RT_CHECK_LAUNCH("softmax_via32_wave_kernel");
+        return RT_OK;
+    }
+    RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax_via_f32: too many rows");
+    hipLaunchKernelGGL((softmax_via32_generic_kernel<T, MODE, MASK>), dim3((unsigned)rows), dim3(BLOCK), 0, dev->stream, (const T*)x,
+                       (const T*)mask, (T*)y, rows, cols, p);
+    RT_CHECK_LAUNCH("softmax_via32_generic_kernel");
+    return RT_OK;
+}
+
+template <typename T>
+int dispatch_via32(rt_device* dev, const void* x, const void* mask, void* y, uint64_t rows, uint32_t cols, const MaskArgs& p, bool mask_vec_ok,
+                   int mode) {
+    if (mask) {
+        return mode == RT_SOFTMAX_STABLE ? launch_via32<T, 1, true>(dev, x, mask, y, rows, cols, p, mask_vec_ok)
+                                         : launch_via32<T, 0, true>(dev, x, mask, y, rows, cols, p, mask_vec_ok);
+    }
+    return mode == RT_SOFTMAX_STABLE ? launch_via32<T, 1, false>(dev, x, mask, y, rows, cols, p, mask_vec_ok)
+                                     : launch_via32<T, 0, false>(dev, x, mask, y, rows, cols, p, mask_vec_ok);
+}
+
 }  // namespace
+
+extern "C" int rt_softmax_via_f32(rt_device* dev, int io_dt, const void* x, const uint32_t x_shape[4], const void* mask,
+                                  const uint32_t mask_shape[4], void* y, int mode) {
+    RT_REQUIRE(io_dt == RT_F16 || io_dt == RT_BF16, RT_ERR_DTYPE, "rt_softmax_via_f32: dtype %d is not F16/BF16", io_dt);
+    RT_REQUIRE(mode == RT_SOFTMAX_REFERENCE || mode == RT_SOFTMAX_STABLE, RT_ERR_ARG, "rt_softmax_via_f32: unknown mode %d", mode);
+    RT_REQUIRE(x_shape && (!mask || mask_shape), RT_ERR_NULL_POINTER, "rt_softmax_via_f32: NULL shape");
+    uint64_t n = 1;
+    for (int i = 0; i < 4; i++) {
+        RT_REQUIRE(x_shape[i] > 0, RT_ERR_SHAPE, "rt_softmax_via_f32: zero extent in dim %d", i);
+        // the add's broadcast rule with the scores as the larger side (Shape::multi_broadcast, shape.rs:118-136)
+        if (mask)
+            RT_REQUIRE(mask_shape[i] == 1 || mask_shape[i] == x_shape[i], RT_ERR_SHAPE,
+                       "rt_softmax_via_f32: mask dim %d: %u does not broadcast to %u", i, mask_shape[i], x_shape[i]);
+        n *= x_shape[i];
+        RT_REQUIRE(n <= 0xffffffffull * 8, RT_ERR_SIZE, "rt_softmax_via_f32: tensor too large");
+    }
+    const uint32_t cols = x_shape[3];
+    const uint64_t rows = n / cols;
+    RT_REQUIRE(rows <= 0xffffffffull, RT_ERR_SIZE, "rt_softmax_via_f32: too many rows");
+    RT_REQUIRE(x && y, RT_ERR_NULL_POINTER, "rt_softmax_via_f32: NULL operand");
+    RT_REQUIRE(rt_aligned(x, 2) && rt_aligned(y, 2) && (!mask || rt_aligned(mask, 2)), RT_ERR_ALIGN, "rt_softmax_via_f32: misaligned pointer");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    MaskArgs p;
+    p.d2 = make_fastdiv(x_shape[2]);
+    p.d1 = make_fastdiv(x_shape[1]);
+    p.ms[0] = p.ms[1] = p.ms[2] = 0;
+    p.mlast = 0;
+    p.reps = make_fastdiv(1);
+    p.slabs = 0;
+    bool mask_vec_ok = true;
+    if (mask) {
+        uint64_t st = 1;
+        p.mlast = mask_shape[3] != 1 || cols == 1;
+        st = mask_shape[3];
+        for (int i = 2; i >= 0; i--) {
+            RT_REQUIRE(st <= 0xffffffffull, RT_ERR_SIZE, "rt_softmax_via_f32: mask too large");
+            p.ms[i] = mask_shape[i] == 1 ? 0u : (uint32_t)st;
+            st *= mask_shape[i];
+        }
+        mask_vec_ok = !p.mlast || (rt_aligned(mask, 16) && cols % 8 == 0);
+        // a mask repeated over the leading dims and larger than an XCD's L2 keeps comfortably: XCD-aware block order
+        int lead = 0;
+        while (lead < 3 && mask_shape[lead] == 1) lead++;
+        bool prefix = lead > 0;
+        uint64_t reps = 1, inner_rows = 1;
+        for (int i = 0; i < 3; i++) {
+            if (i < lead) reps *= x_shape[i];
+            else {
+                inner_rows *= x_shape[i];
+                if (mask_shape[i] != x_shape[i]) prefix = false;
+            }
+        }
+        if (prefix && p.mlast && reps > 1 && inner_rows * cols * 2 >= (1u << 20) && inner_rows % (WAVES * SM_XCDS) == 0) {
+            p.reps = make_fastdiv((uint32_t)reps);
+            p.slabs = (uint32_t)(inner_rows / WAVES);
+        }
+    }
+    if (io_dt == RT_F16) return dispatch_via32<half_t>(dev, x, mask, y, rows, cols, p, mask_vec_ok, mode);
+    return dispatch_via32<bf16_t>(dev, x, mask, y, rows, cols, p, mask_vec_ok, mode);
+}
 
 extern "C" int rt_softmax(rt_device* dev, int dt, const void* x, void* y, uint64_t rows, uint32_t cols, int mode) {
     RT_REQUIRE(rt_is_float_dt(dt), RT_ERR_DTYPE, "rt_softmax: dtype %d is not F32/F16/BF16", dt);   // Softmax::check_dtypes

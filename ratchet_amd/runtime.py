@@ -62,6 +62,10 @@ class Buffer:
         return self
 
 
+def _unary_code(op):
+    return _lib.UNARY_OPS.index(op) if isinstance(op, str) else op
+
+
 class BufferView:
     """A window into a Buffer starting `offset` elements in (keeps the parent alive); used for offset / misaligned operands."""
 
@@ -233,6 +237,34 @@ class Device:
         cols = x.shape[-1]
         out = out or Buffer(self, x.shape, x.dt)
         check(self.lib.rt_rms_norm(self.handle, x.dt, x.ptr, scale.ptr, out.ptr, x.numel // cols, cols, eps))
+        return out
+
+    # ---- caller patterns in one pass: what full() -> op -> cast(dt) yields on a 16-bit tensor
+    def norm_via_f32(self, kind, x, scale, bias=None, eps=1e-5, out=None):
+        """kind 'layer' | 'rms'; x 16-bit, scale / bias f32 buffers."""
+        cols = x.shape[-1]
+        out = out or Buffer(self, x.shape, x.dt)
+        check(self.lib.rt_norm_via_f32(self.handle, {"layer": 0, "rms": 1}[kind], x.dt, x.ptr, scale.ptr,
+                                       bias.ptr if bias is not None else None, out.ptr, x.numel // cols, cols, eps))
+        return out
+
+    def softmax_via_f32(self, x, mask=None, out=None, mode=_lib.SOFTMAX_REFERENCE):
+        """softmax over the last dim of (x + mask) with the mask broadcast over x's leading dims."""
+        out = out or Buffer(self, x.shape, x.dt)
+        check(self.lib.rt_softmax_via_f32(self.handle, x.dt, x.ptr, shape4(x.shape), mask.ptr if mask is not None else None,
+                                          shape4(mask.shape) if mask is not None else None, out.ptr, mode))
+        return out
+
+    def unary_via_f32(self, op, x, out=None):
+        out = out or Buffer(self, x.shape, x.dt)
+        check(self.lib.rt_unary_via_f32(self.handle, _unary_code(op), x.dt, x.ptr, out.ptr, x.numel))
+        return out
+
+    def gated_mul_via_f32(self, op, gate, up, rows, cols, gate_row_stride=None, up_row_stride=None, out=None):
+        """out[r, c] = up[r, c] * cast(op(full(gate[r, c]))); gate / up may be views with a row stride (elements)."""
+        out = out or Buffer(self, (rows, cols), gate.dt)
+        check(self.lib.rt_gated_mul_via_f32(self.handle, _unary_code(op), gate.dt, gate.ptr, gate_row_stride or cols, up.ptr,
+                                            up_row_stride or cols, out.ptr, rows, cols))
         return out
 
     def group_norm(self, x, groups, scale, bias, eps=1e-5, out=None):

@@ -129,6 +129,27 @@ def test_reduction_validation(lib):
     assert lib.rt_group_norm(None, _lib.F16, SOME, None, None, SOME, 1, 8, 4, 4, 1e-5) == 8
 
 
+def test_fused_pattern_validation(lib):
+    f32p = ctypes.cast(ctypes.c_void_p(0x1000), ctypes.c_void_p)
+    assert lib.rt_norm_via_f32(None, 0, _lib.F16, SOME, f32p, None, SOME, 4, 8, 1e-5) == 8
+    assert lib.rt_norm_via_f32(None, 2, _lib.F16, SOME, f32p, None, SOME, 4, 8, 1e-5) == 7      # kind
+    assert lib.rt_norm_via_f32(None, 0, _lib.F32, SOME, f32p, None, SOME, 4, 8, 1e-5) == 2      # f32 needs no full()/cast()
+    assert lib.rt_norm_via_f32(None, 1, _lib.BF16, SOME, None, None, SOME, 4, 8, 1e-5) == 1
+    shp = u4(1, 2, 4, 8)
+    assert lib.rt_softmax_via_f32(None, _lib.F16, SOME, shp, None, None, SOME, 0) == 8
+    assert lib.rt_softmax_via_f32(None, _lib.F16, SOME, shp, SOME, u4(1, 1, 4, 8), SOME, 0) == 8
+    assert lib.rt_softmax_via_f32(None, _lib.F16, SOME, shp, SOME, u4(1, 3, 4, 8), SOME, 0) == 4
+    assert lib.rt_softmax_via_f32(None, _lib.F16, SOME, shp, SOME, None, SOME, 0) == 1
+    assert lib.rt_softmax_via_f32(None, _lib.F32, SOME, shp, None, None, SOME, 0) == 2
+    assert lib.rt_softmax_via_f32(None, _lib.F16, SOME, shp, None, None, SOME, 3) == 7
+    assert lib.rt_unary_via_f32(None, 0, _lib.F16, SOME, SOME, 16) == 8
+    assert lib.rt_unary_via_f32(None, 14, _lib.F16, SOME, SOME, 16) == 3
+    assert lib.rt_unary_via_f32(None, 0, _lib.I32, SOME, SOME, 16) == 2
+    assert lib.rt_gated_mul_via_f32(None, 12, _lib.F16, SOME, 16, SOME, 16, SOME, 4, 8) == 8
+    assert lib.rt_gated_mul_via_f32(None, 12, _lib.F16, SOME, 4, SOME, 16, SOME, 4, 8) == 4      # stride shorter than a row
+    assert lib.rt_gated_mul_via_f32(None, 12, _lib.F32, SOME, 16, SOME, 16, SOME, 4, 8) == 2
+
+
 def test_storage_validation(lib):
     p = ctypes.c_void_p()
     assert lib.rt_malloc(None, 16, ctypes.byref(p)) == 8
