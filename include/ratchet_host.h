@@ -49,6 +49,8 @@ rth_tensor* rth_softmax(const rth_tensor* x, size_t dim, int mode);
 rth_tensor* rth_slice(const rth_tensor* x, int n, const uint64_t* starts, const uint64_t* ends);
 rth_tensor* rth_view(const rth_tensor* x, int rank, const uint64_t* shape);
 rth_tensor* rth_cat(const rth_tensor* const* xs, int n, size_t dim);
+/* one-launch replacements of full() -> norm / softmax / activation -> cast(dt) at resolve(); on by default */
+void rth_set_pattern_fusion(int on);
 rth_tensor* rth_cache(const rth_tensor* cache, const rth_tensor* source, size_t dim, size_t offset);   /* tensor.rs:481-486 */
 rth_tensor* rth_permute(const rth_tensor* x, int n, const uint64_t* dims);
 rth_tensor* rth_broadcast_to(const rth_tensor* x, int rank, const uint64_t* shape);

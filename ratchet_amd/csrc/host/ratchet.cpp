@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <atomic>
 #include <sstream>
+#include <unordered_map>
 #include <unordered_set>
 
 #include "../../../include/ratchet_hip.h"
@@ -423,11 +424,174 @@ std::vector<uint64_t> Tensor::execution_order_ids() const {
     return ids;
 }
 
+static std::atomic<bool> g_fuse_patterns{true};
+void set_pattern_fusion(bool on) { g_fuse_patterns = on; }
+bool pattern_fusion() { return g_fuse_patterns; }
+
+// One-pass replacements for the op sequences the models always emit around 16-bit tensors (full() ... cast(dt)).
+// The graph the user built is unchanged; resolve() runs one launch at the sequence's last node and never materialises
+// the interior nodes, which must be unresolved and held by nobody but their single consumer.
+struct FusedPlan {
+    enum What { NormVia32, SoftmaxVia32, UnaryVia32, GatedMul } what;
+    Node* x = nullptr;            // 16-bit input (gate for GatedMul)
+    Node* aux = nullptr;          // norm node (scale / bias / eps / kind), softmax node (mode), unary node (op)
+    Node* mask = nullptr;         // SoftmaxVia32: tensor added to x before the softmax (nullptr: none)
+    Node* up = nullptr;           // GatedMul: the multiplied operand
+    uint64_t x_off = 0, up_off = 0, x_stride = 0, up_stride = 0;   // GatedMul views, in elements
+};
+
 struct Resolver {
     // a Broadcast node nobody else holds, not yet materialised, feeding a Binary: fused into the binary kernel
     static bool fusable_broadcast(const Tensor& operand) {
         Node* b = Node::of(operand);
         return b->kind == Kind::Broadcast && !b->storage && Node::holders(operand) == 1;
+    }
+    // an interior node of a pattern: not yet computed and invisible to everybody but its consumer
+    static bool interior(const Tensor& t, Kind k) {
+        Node* n = Node::of(t);
+        return n->kind == k && !n->storage && Node::holders(t) == 1;
+    }
+    static bool is16(DType d) { return d == DType::F16 || d == DType::BF16; }
+
+    // `n` is a Cast f32 -> 16-bit whose source chain is <16-bit x>.full().<op>(): fills plan, lists the interior nodes
+    static bool match_via32(Node* n, FusedPlan& plan, std::vector<Node*>& inner) {
+        if (n->kind != Kind::Cast || !is16(n->dt) || n->storage) return false;
+        const Tensor& opT = n->srcs[0];
+        Node* op = Node::of(opT);
+        if (op->dt != DType::F32 || op->storage || Node::holders(opT) != 1) return false;
+        if (op->kind != Kind::LayerNorm && op->kind != Kind::RMSNorm && op->kind != Kind::Softmax && op->kind != Kind::Unary) return false;
+        if (!interior(op->srcs[0], Kind::Cast)) return false;
+        Node* widen = Node::of(op->srcs[0]);
+        Node* x = Node::of(widen->srcs[0]);
+        if (x->dt != n->dt) return false;                          // full() of a 16-bit tensor, cast back to the same type
+        plan.x = x;
+        plan.aux = op;
+        inner = {op, widen};
+        if (op->kind == Kind::Unary) {
+            plan.what = FusedPlan::UnaryVia32;
+            return true;
+        }
+        if (op->kind == Kind::LayerNorm || op->kind == Kind::RMSNorm) {
+            plan.what = FusedPlan::NormVia32;
+            return true;
+        }
+        if (op->dim != op->shape.rank() - 1) return false;
+        plan.what = FusedPlan::SoftmaxVia32;
+        // scores.add(mask): a Binary add nobody else sees, scores at full shape, the mask broadcast (or already full)
+        if (interior(widen->srcs[0], Kind::Binary) && x->bop == BinaryOp::Add) {
+            Node* scores = Node::of(x->srcs[0]);
+            const Tensor& mT = x->srcs[1];
+            Node* m = Node::of(mT);
+            if (scores->shape == x->shape && !(scores->kind == Kind::Broadcast && !scores->storage)) {
+                if (fusable_broadcast(mT)) {
+                    inner.push_back(x);
+                    inner.push_back(m);
+                    plan.mask = Node::of(m->srcs[0]);
+                    plan.x = scores;
+                } else if (m->kind != Kind::Broadcast || m->storage) {
+                    inner.push_back(x);
+                    plan.mask = m;
+                    plan.x = scores;
+                }
+            }
+        }
+        return true;
+    }
+
+    // a Slice that only narrows the last dim, not yet materialised and seen by its consumer alone: a row-strided view
+    static bool last_dim_view(const Tensor& t, Node*& base, uint64_t& off, uint64_t& stride) {
+        Node* n = Node::of(t);
+        if (n->kind != Kind::Slice || n->storage || Node::holders(t) != 1) return false;
+        Node* src = Node::of(n->srcs[0]);
+        const size_t r = src->shape.rank();
+        if (n->ranges.size() != r) return false;
+        for (size_t i = 0; i + 1 < r; i++)
+            if (n->ranges[i].first != 0 || n->ranges[i].second != src->shape[i]) return false;
+        base = src;
+        off = n->ranges[r - 1].first;
+        stride = src->shape[r - 1];
+        return true;
+    }
+
+    // up.mul(gate.full().<op>().cast(dt)), either operand order
+    static bool match_gated(Node* n, FusedPlan& plan, std::vector<Node*>& inner) {
+        if (n->kind != Kind::Binary || n->bop != BinaryOp::Mul || !is16(n->dt) || n->storage) return false;
+        for (int side = 0; side < 2; side++) {
+            const Tensor& actT = n->srcs[side ^ 1];
+            const Tensor& upT = n->srcs[side];
+            if (!interior(actT, Kind::Cast)) continue;
+            FusedPlan act;
+            std::vector<Node*> act_inner;
+            if (!match_via32(Node::of(actT), act, act_inner) || act.what != FusedPlan::UnaryVia32) continue;
+            Node* up = Node::of(upT);
+            if (up->shape != n->shape || (up->kind == Kind::Broadcast && !up->storage)) continue;
+            plan.what = FusedPlan::GatedMul;
+            plan.aux = act.aux;
+            plan.x = act.x;
+            plan.up = up;
+            inner = act_inner;
+            inner.push_back(Node::of(actT));
+            const uint64_t cols = n->shape[n->shape.rank() - 1];
+            plan.x_stride = plan.up_stride = cols;
+            // the gate's slice hangs off the widening cast, the other operand's off the multiply
+            Node* widen = act_inner[1];
+            Node* base = nullptr;
+            uint64_t off = 0, stride = 0;
+            if (last_dim_view(widen->srcs[0], base, off, stride)) {
+                inner.push_back(plan.x);
+                plan.x = base;
+                plan.x_off = off;
+                plan.x_stride = stride;
+            }
+            if (last_dim_view(upT, base, off, stride)) {
+                inner.push_back(plan.up);
+                plan.up = base;
+                plan.up_off = off;
+                plan.up_stride = stride;
+            }
+            return true;
+        }
+        return false;
+    }
+
+    static void run_fused(Node* n, const FusedPlan& plan, size_t& launches) {
+        rt_device* dev = n->device.raw();
+        const int dt = (int)n->dt;
+        n->storage = std::make_shared<Buffer>(n->device, n->shape.numel() * size_of(n->dt));
+        const size_t cols = n->shape[n->shape.rank() - 1];
+        const uint64_t rows = n->shape.numel() / cols;
+        switch (plan.what) {
+            case FusedPlan::NormVia32: {
+                Node* op = plan.aux;
+                const bool layer = op->kind == Kind::LayerNorm;
+                const float* scale = static_cast<const float*>(Node::of(op->srcs[1])->storage->ptr);
+                const float* bias = (layer && op->has_bias) ? static_cast<const float*>(Node::of(op->srcs[2])->storage->ptr) : nullptr;
+                check_rt(rt_norm_via_f32(dev, layer ? 0 : 1, dt, plan.x->storage->ptr, scale, bias, n->storage->ptr, rows, (uint32_t)cols, op->eps),
+                         "rt_norm_via_f32");
+                break;
+            }
+            case FusedPlan::SoftmaxVia32: {
+                uint32_t xs[4], ms[4];
+                shape4(n->shape, xs);
+                if (plan.mask) shape4(plan.mask->shape, ms);
+                check_rt(rt_softmax_via_f32(dev, dt, plan.x->storage->ptr, xs, plan.mask ? plan.mask->storage->ptr : nullptr, plan.mask ? ms : nullptr,
+                                            n->storage->ptr, (int)plan.aux->mode),
+                         "rt_softmax_via_f32");
+                break;
+            }
+            case FusedPlan::UnaryVia32:
+                check_rt(rt_unary_via_f32(dev, (int)plan.aux->uop, dt, plan.x->storage->ptr, n->storage->ptr, n->shape.numel()), "rt_unary_via_f32");
+                break;
+            case FusedPlan::GatedMul: {
+                const size_t eb = size_of(n->dt);
+                const char* gate = static_cast<const char*>(plan.x->storage->ptr) + plan.x_off * eb;
+                const char* up = static_cast<const char*>(plan.up->storage->ptr) + plan.up_off * eb;
+                check_rt(rt_gated_mul_via_f32(dev, (int)plan.aux->uop, dt, gate, plan.x_stride, up, plan.up_stride, n->storage->ptr, rows, (uint32_t)cols),
+                         "rt_gated_mul_via_f32");
+                break;
+            }
+        }
+        launches++;
     }
 
     static void run(Node* n, size_t& launches) {
@@ -568,15 +732,31 @@ struct Resolver {
     static void resolve(Node* root) {
         size_t launches = 0;
         const std::vector<Node*> order = execution_order(root);
-        // broadcasts that their (single) binary consumer will absorb are not materialised
         std::unordered_set<Node*> skip;
+        // caller patterns, consumers first so that the longest sequence wins (the gated multiply contains a unary one)
+        std::unordered_map<Node*, FusedPlan> fused;
+        if (g_fuse_patterns) {
+            for (auto it = order.rbegin(); it != order.rend(); ++it) {
+                Node* n = *it;
+                if (n->storage || skip.count(n)) continue;
+                FusedPlan plan;
+                std::vector<Node*> inner;
+                if (match_gated(n, plan, inner) || match_via32(n, plan, inner)) {
+                    fused.emplace(n, plan);
+                    for (Node* i : inner) skip.insert(i);
+                }
+            }
+        }
+        // broadcasts that their (single) binary consumer will absorb are not materialised
         for (Node* n : order)
-            if (n->kind == Kind::Binary && !n->storage)
+            if (n->kind == Kind::Binary && !n->storage && !skip.count(n) && !fused.count(n))
                 for (const Tensor& s : n->srcs)
                     if (fusable_broadcast(s)) skip.insert(Node::of(s));
         for (Node* n : order) {
             if (n->storage || skip.count(n)) continue;         // already resolved (tensor.rs:783) or fused away
-            run(n, launches);
+            auto f = fused.find(n);
+            if (f != fused.end()) run_fused(n, f->second, launches);
+            else run(n, launches);
         }
         check_rt(rt_sync(root->device.raw()), "rt_sync");      // resolve returns after completion (tensor.rs:855-856)
         root->last_launches = launches;

@@ -90,6 +90,11 @@ struct Buffer {
     Buffer& operator=(const Buffer&) = delete;
 };
 
+// resolve() replaces the models' full() -> norm / softmax / activation -> cast(dt) sequences on 16-bit tensors (and
+// phi3's gated multiply) by one launch each when the intermediate tensors are visible to nobody else.  On by default.
+void set_pattern_fusion(bool on);
+bool pattern_fusion();
+
 class Tensor;
 struct Node;                                                  // LazyOp + operands (op.rs:14-31)
 

@@ -114,6 +114,7 @@ rth_tensor* rth_cat(const rth_tensor* const* xs, int n, size_t dim) {
         return Tensor::cat(ts, dim);
     });
 }
+void rth_set_pattern_fusion(int on) { ratchet::set_pattern_fusion(on != 0); }
 rth_tensor* rth_cache(const rth_tensor* cache, const rth_tensor* source, size_t dim, size_t offset) {
     return build([&] { return cache->t.cache(source->t, dim, offset); });
 }

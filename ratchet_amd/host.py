@@ -68,8 +68,15 @@ def load():
     H.rth_last_resolve_launches.restype = ctypes.c_long
     H.rth_id.argtypes = [vp]
     H.rth_id.restype = ctypes.c_uint64
+    H.rth_set_pattern_fusion.argtypes = [i]
+    H.rth_set_pattern_fusion.restype = None
     _h = H
     return H
+
+
+def set_pattern_fusion(on):
+    """resolve() folds full() -> norm / softmax / activation -> cast(dt) sequences into one launch each (default on)."""
+    load().rth_set_pattern_fusion(int(bool(on)))
 
 
 def _raise():

@@ -207,3 +207,71 @@ def test_cache_decode_loop(hdev, oracle):
         assert np.array_equal(got, np.concatenate(rows, axis=2))
         assert np.array_equal(got, oracle.cache(cache_np, src, 2, off - n))
     assert np.array_equal(cache.to_numpy(), cache_np)
+
+
+def test_caller_patterns_resolve_in_one_launch(hdev, oracle):
+    """The models' full() -> op -> cast(dt) sequences (ratchet-nn/src/norm.rs:35-44, ratchet-models/src/phi3/attn.rs:143-153,
+    phi3/mlp.rs:32-38) are folded by resolve() when nobody else sees the intermediate tensors; results stay within the op
+    sequence's own bars and the graph the user built is unchanged."""
+    from ratchet_amd import _lib
+    from ratchet_amd.host import set_pattern_fusion
+
+    F16, F32 = _lib.F16, _lib.F32
+    rng = np.random.default_rng(406)
+    x = (rng.standard_normal((2, 64, 2560)) * 2).astype(np.float16)
+    w = rng.standard_normal(2560).astype(np.float32)
+    b = rng.standard_normal(2560).astype(np.float32)
+    S, H = 128, 4
+    scores = (2 * rng.standard_normal((1, H, S, S))).astype(np.float16)
+    mask = np.triu(np.full((S, S), -np.inf, np.float16), k=1)
+    proj = rng.standard_normal((1, 64, 1024)).astype(np.float16)
+
+    def graphs():
+        ln = T(x, hdev).full().layer_norm(T(w, hdev), T(b, hdev), 1e-5).cast(F16)
+        rms = T(x, hdev).full().rms_norm(T(w, hdev), 1e-5).cast(F16)
+        attn = T(scores, hdev).add(T(mask, hdev)).full().softmax(3).cast(F16)
+        act = T(x, hdev).full().gelu().cast(F16)
+        p = T(proj, hdev)
+        gate, up = p.slice([(0, 1), (0, 64), (0, 512)]), p.slice([(0, 1), (0, 64), (512, 1024)])
+        glu = up.mul(gate.full().silu().cast(F16))
+        return {"ln": ln, "rms": rms, "attn": attn, "act": act, "glu": glu}
+
+    set_pattern_fusion(False)
+    try:
+        plain = {k: (g.resolve().to_numpy(), g.last_resolve_launches()) for k, g in graphs().items()}
+    finally:
+        set_pattern_fusion(True)
+    fused = {k: (g.resolve().to_numpy(), g.last_resolve_launches()) for k, g in graphs().items()}
+    assert {k: v[1] for k, v in plain.items()} == {"ln": 3, "rms": 3, "attn": 4, "act": 3, "glu": 6}
+    assert {k: v[1] for k, v in fused.items()} == {"ln": 1, "rms": 1, "attn": 1, "act": 1, "glu": 1}
+    for k in ("act", "glu"):
+        assert same_bits(fused[k][0], plain[k][0]), k
+    for k in ("ln", "rms", "attn"):
+        ok, info = close(oracle, fused[k][0], plain[k][0], 1e-3)
+        assert ok, (k, info)
+    # against the oracle's op sequence as well
+    x32 = oracle.cast(x, np.float32)
+    ok, info = close(oracle, fused["ln"][0], oracle.cast(oracle.layer_norm(x32, w, b, 1e-5, intended=True), np.float16), 1e-3)
+    assert ok, info
+    want = oracle.cast(oracle.softmax(oracle.cast(oracle.binary("add", scores, np.ascontiguousarray(np.broadcast_to(mask, scores.shape))),
+                                                  np.float32)), np.float16)
+    ok, info = close(oracle, fused["attn"][0], want, 1e-3)
+    assert ok, info
+    gate_np, up_np = np.ascontiguousarray(proj[..., :512]), np.ascontiguousarray(proj[..., 512:])
+    want = oracle.binary("mul", up_np, oracle.cast(oracle.unary("silu", oracle.cast(gate_np, np.float32)), np.float16))
+    assert same_bits(fused["glu"][0], want)
+
+
+def test_pattern_with_a_visible_intermediate_is_not_folded(hdev, oracle):
+    from ratchet_amd import _lib
+
+    rng = np.random.default_rng(407)
+    x = rng.standard_normal((4, 256)).astype(np.float16)
+    w = rng.standard_normal(256).astype(np.float32)
+    wide = T(x, hdev).full()                                   # the caller keeps the f32 tensor: it must be materialised
+    y = wide.rms_norm(T(w, hdev), 1e-5).cast(_lib.F16).resolve()
+    assert y.last_resolve_launches() == 3
+    assert wide.resolved() and same_bits(wide.to_numpy(), x.astype(np.float32))
+    want = oracle.cast(oracle.rms_norm(oracle.cast(x, np.float32), w, 1e-5, intended=True), np.float16)
+    ok, info = close(oracle, y.to_numpy(), want, 1e-3)
+    assert ok, info
