@@ -177,6 +177,7 @@ def build_workload(dev, seed):
                   lambda: dev.permute(d_p4, (0, 2, 1, 3), out=d_p4o),
                   dict(kind="exact", out=d_p4o, run=lambda o: o.permute(p4, (0, 2, 1, 3)), bytes=2 * p4.nbytes)))
     ops_extra["copy_pair"] = (d_scores3, d_masked3)
+    ops_extra["attn"] = (d_scores3, d_mask, d_masked3, d_soft3)
     return ops
 
 
@@ -201,6 +202,101 @@ def copy_ceiling(dev):
     ms = float(np.mean(times))
     return {"kernel": "copy_vec_kernel", "bytes": 2 * src.nbytes, "us": round(ms * 1e3, 1), "GBps": round(2 * src.nbytes / ms / 1e6, 1),
             "frac_of_peak": round(2 * src.nbytes / ms / 1e6 / PEAK_HBM_GBPS, 4)}
+
+
+def one_pass_patterns(dev, seed, oracle):
+    """The models wrap 16-bit norms, softmax and activations in full() ... cast(dt); the library has one-pass entry points
+    for those sequences.  Reported beside the step (never part of `value`): time of the one-pass launch and of the op
+    sequence it replaces, both with HIP events on the device's stream, at the shapes of BASELINE configs 2 and 3."""
+    from ratchet_amd.runtime import BufferView
+
+    np16, np32 = np.float16, np.float32
+
+    def timeit(fn, n=10):
+        for _ in range(2):
+            fn()
+        e0, e1 = dev.event(), dev.event()
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        return e0.elapsed_ms(e1) / n * 1e3
+
+    out = []
+
+    def row(name, shape, alg_bytes, seq_bytes, launches, fused, seq, got, want, exact):
+        us_f, us_s = timeit(fused), timeit(seq)
+        ok = None
+        if oracle is not None:
+            a, b = download_rows(dev, got, 256, shape_cols[0], np16), download_rows(dev, want, 256, shape_cols[0], np16)
+            if exact:
+                ok = bool(np.all((a.view(np.uint16) == b.view(np.uint16)) | (np.isnan(a) & np.isnan(b))))
+            else:
+                ok = oracle.count_not_close(a, b, 1e-3, 1e-3)[0] == 0
+        out.append({"pattern": name, "shape": shape, "one_pass_us": round(us_f, 1), "sequence_us": round(us_s, 1),
+                    "launches_replaced": launches, "alg_MB": round(alg_bytes / 1e6, 1), "sequence_alg_MB": round(seq_bytes / 1e6, 1),
+                    "GBps": round(alg_bytes / us_f / 1e3, 1), "frac_hbm": round(alg_bytes / us_f / 1e3 / PEAK_HBM_GBPS, 4),
+                    "matches_sequence": ok})
+
+    shape_cols = [0]
+    # cfg 2: LayerNorm module on [1,2048,2560] f16 with f32 weights; GELU between full() and cast()
+    x = normal(seed, 901, (2048, 2560), 1.0, np16)
+    w, b = normal(seed, 902, (2560,), 0.02, np32, mean=1.0), normal(seed, 903, (2560,), 0.02, np32)
+    dx, dw, db = dev.upload(x), dev.upload(w), dev.upload(b)
+    f32a, f32b = dev.empty(x.shape, F32), dev.empty(x.shape, F32)
+    y1, y2 = dev.empty(x.shape, F16), dev.empty(x.shape, F16)
+    shape_cols[0] = 2560
+    row("full -> layer_norm -> cast", "[1,2048,2560] f16", 2 * x.nbytes, 10 * x.nbytes, 3,
+        lambda: dev.norm_via_f32("layer", dx, dw, db, 1e-5, out=y1),
+        lambda: (dev.cast(dx, F32, out=f32a), dev.layer_norm(f32a, dw, db, 1e-5, out=f32b), dev.cast(f32b, F16, out=y2)), y1, y2, False)
+    del f32a, f32b
+    h = normal(seed, 904, (2048, 10240), 1.0, np16)
+    dh = dev.upload(h)
+    f32a = dev.empty(h.shape, F32)
+    y1, y2 = dev.empty(h.shape, F16), dev.empty(h.shape, F16)
+    shape_cols[0] = 10240
+    row("full -> gelu -> cast", "[1,2048,10240] f16", 2 * h.nbytes, 10 * h.nbytes, 3,
+        lambda: dev.unary_via_f32("gelu", dh, out=y1),
+        lambda: (dev.cast(dh, F32, out=f32a), dev.unary("gelu", f32a, out=f32a), dev.cast(f32a, F16, out=y2)), y1, y2, True)
+    del f32a, dh
+    # cfg 3: RMSNorm module on [1,4096,3072]; gated multiply on the [1,4096,16384] gate_up projection; attention softmax
+    x = normal(seed, 905, (4096, 3072), 1.0, np16)
+    w = normal(seed, 906, (3072,), 0.02, np32, mean=1.0)
+    dx, dw = dev.upload(x), dev.upload(w)
+    f32a, f32b = dev.empty(x.shape, F32), dev.empty(x.shape, F32)
+    y1, y2 = dev.empty(x.shape, F16), dev.empty(x.shape, F16)
+    shape_cols[0] = 3072
+    row("full -> rms_norm -> cast", "[1,4096,3072] f16", 2 * x.nbytes, 10 * x.nbytes, 3,
+        lambda: dev.norm_via_f32("rms", dx, dw, None, 1e-5, out=y1),
+        lambda: (dev.cast(dx, F32, out=f32a), dev.rms_norm(f32a, dw, 1e-5, out=f32b), dev.cast(f32b, F16, out=y2)), y1, y2, False)
+    del f32a, f32b
+    proj = normal(seed, 907, (4096, 16384), 1.0, np16)
+    dp = dev.upload(proj)
+    half = (4096, 8192)
+    g16, u16, act16 = dev.empty(half, F16), dev.empty(half, F16), dev.empty(half, F16)
+    g32 = dev.empty(half, F32)
+    y1, y2 = dev.empty(half, F16), dev.empty(half, F16)
+    gate_v = BufferView(dp, 0, (proj.size - 8192,))
+    up_v = BufferView(dp, 8192, (proj.size - 8192,))
+    hb = 4096 * 8192 * 2
+    shape_cols[0] = 8192
+    row("slice x2 -> full -> silu -> cast -> mul", "[1,4096,16384] f16 -> [1,4096,8192]", 3 * hb, 17 * hb, 6,
+        lambda: dev.gated_mul_via_f32("silu", gate_v, up_v, 4096, 8192, gate_row_stride=16384, up_row_stride=16384, out=y1),
+        lambda: (dev.slice(dp, [(0, 4096), (0, 8192)], out=g16), dev.slice(dp, [(0, 4096), (8192, 16384)], out=u16),
+                 dev.cast(g16, F32, out=g32), dev.unary("silu", g32, out=g32), dev.cast(g32, F16, out=act16),
+                 dev.binary("mul", u16, act16, out=y2)), y1, y2, True)
+    del g16, u16, act16, g32, dp
+    S, H = 4096, 32
+    scores, mask, masked, _ = ops_extra["attn"]
+    s32a = dev.empty((1, H, S, S), F32)
+    y1, y2 = dev.empty((1, H, S, S), F16), dev.empty((1, H, S, S), F16)
+    nb = H * S * S * 2
+    shape_cols[0] = S
+    row("add(mask) -> full -> softmax -> cast", "[1,32,4096,4096]+[4096,4096] f16", 2 * nb + S * S * 2, 12 * nb + S * S * 2, 4,
+        lambda: dev.softmax_via_f32(scores, mask, out=y1),
+        lambda: (dev.binary("add", scores, mask, out=masked), dev.cast(masked, F32, out=s32a), dev.softmax(s32a, out=s32a),
+                 dev.cast(s32a, F16, out=y2)), y1, y2, False)
+    return out
 
 
 def download_rows(dev, buf, nrows, row_elems, np_dtype):
@@ -275,6 +371,7 @@ def main():
     ap.add_argument("--ops", type=str, default=None, help="regex selecting ops by 'cfgN name'")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline timing")
     ap.add_argument("--no-check", action="store_true", help="skip the parity check of the timed buffers")
+    ap.add_argument("--no-patterns", action="store_true", help="skip the one-pass caller-pattern timings reported beside the step")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (every op is row/element parallel; there is no multi-GPU path). "
@@ -338,6 +435,7 @@ def main():
             per_op_cpu[id(o)] = (t, b)
 
     ceiling = copy_ceiling(dev) if not args.ops else None      # after the parity check: it overwrites an output buffer
+    patterns = one_pass_patterns(dev, seed, oracle if not args.no_check else None) if not (args.ops or args.no_patterns) else None
 
     rows = []
     for o in ops:
@@ -371,6 +469,7 @@ def main():
                       "16384 of 131072 rows (4 heads) for the two ops on [1,32,4096,4096] (%.1f MB algorithmic, %.1f s)" % (cpu_b / 1e6, cpu_t),
             "host_cpus": os.cpu_count()},
         "hbm_copy_ceiling": ceiling,
+        "one_pass_patterns": patterns,
         "parity_ok": bool(parity_ok) if not args.no_check else None,
         "ops": rows,
         "wall_s": round(wall, 3), "setup_s": round(t_setup, 2),
