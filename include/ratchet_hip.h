@@ -123,6 +123,24 @@ int rt_concat(rt_device* dev, int elem_bytes, int n_inputs, const void* const* x
 int rt_cache(rt_device* dev, int elem_bytes, void* cache, const uint32_t cache_shape[4], const void* source,
              const uint32_t source_shape[4], int dim, uint32_t offset, void* dst);
 
+/* IndexSelect (ops/select.rs:20-79, cpu/mod.rs:44-84; the embedding lookup of every model):
+ * dst[left, i, right] = src[left, indices[i], right] along dim, i32 indices on the device.  The reference panics on an
+ * index outside [0, src_shape[dim]); here such a row is filled with zeros. */
+int rt_index_select(rt_device* dev, int elem_bytes, const void* src, const uint32_t src_shape[4], const int32_t* indices,
+                    uint32_t n_indices, int dim, void* dst);
+
+/* IndexWrite (ops/index_write.rs:14-111): dst, in place, receives the src_numel elements of src as one flat run that
+ * starts at the element write_start addresses (D[offset(write_start) + i] = S[i], :96-104).  A run that would leave dst
+ * is rejected (the reference's kernel has no bound). */
+int rt_index_write(rt_device* dev, int elem_bytes, void* dst, const uint32_t dst_shape[4], const void* src, uint64_t src_numel,
+                   const uint32_t write_start[4]);
+
+/* RoPE on [B, H, S, D] (ops/rope.rs:17-95; arithmetic of cpu/rope.rs:23-143): the first `dim` columns are rotated in
+ * halves by theta[p, i] = (offset + p) * base^(-i / (dim/2)), the rest pass through.  y may be x (the reference's GPU
+ * kernel is in-place only).  F16/BF16 are widened, rotated in f32 and rounded once, which is what the models'
+ * x.full().rope(..).cast(dt) yields; the reference's CPU path implements F32 only. */
+int rt_rope(rt_device* dev, int dt, const void* x, void* y, const uint32_t shape[4], uint32_t dim, float base, uint32_t offset);
+
 /* Softmax over the last dimension (ops/softmax.rs:14-39,183-199; cpu/softmax.rs:22-42): rows x cols, contiguous.
  * y may alias x (the reference kernel is in-place only, ops/softmax.rs:47-49).  dt: F32, F16, BF16. */
 int rt_softmax(rt_device* dev, int dt, const void* x, void* y, uint64_t rows, uint32_t cols, int mode);

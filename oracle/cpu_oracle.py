@@ -43,6 +43,9 @@ def lib():
         L.orc_broadcast.argtypes = [i, vp, vp, i, vp, i, vp, i]
         L.orc_concat.argtypes = [i, i, vp, i, vp, i, vp]
         L.orc_cache.argtypes = [i, vp, i, vp, vp, vp, i, ctypes.c_uint64, vp]
+        L.orc_rope.argtypes = [i, vp, vp, vp, ctypes.c_uint64, f, ctypes.c_uint64]
+        L.orc_index_select.argtypes = [i, vp, i, vp, vp, ctypes.c_uint64, i, vp]
+        L.orc_index_write.argtypes = [i, vp, i, vp, vp, ctypes.c_uint64, vp]
         L.orc_softmax.argtypes = [i, vp, vp, sz, sz]
         L.orc_layer_norm.argtypes = [i, vp, vp, vp, vp, sz, sz, f, sz]
         L.orc_rms_norm.argtypes = [i, vp, vp, vp, sz, sz, f, sz]
@@ -174,6 +177,35 @@ def cache(cache_arr, source, dim, offset):
     _check(lib().orc_cache(cache_arr.dtype.itemsize, _p(cache_arr), cache_arr.ndim, _p(_u64(cache_arr.shape)), _p(source),
                            _p(_u64(source.shape)), dim, offset, _p(y)), "cache")
     return y
+
+
+def rope(x, dim, base, offset):
+    """x [B, H, S, D] float32 (the only dtype the reference's CPU path implements)."""
+    x = _c(x)
+    assert x.ndim == 4
+    y = np.empty_like(x)
+    _check(lib().orc_rope(dt_code(x.dtype), _p(x), _p(y), _p(_u64(x.shape)), dim, base, offset), "rope")
+    return y
+
+
+def index_select(src, indices, dim):
+    src = _c(src)
+    indices = np.ascontiguousarray(indices, dtype=np.int32)
+    out_shape = list(src.shape)
+    out_shape[dim] = indices.shape[0]
+    y = np.empty(out_shape, dtype=src.dtype)
+    _check(lib().orc_index_select(src.dtype.itemsize, _p(src), src.ndim, _p(_u64(src.shape)), _p(indices), indices.shape[0], dim, _p(y)),
+           "index_select")
+    return y
+
+
+def index_write(dst, src, write_start):
+    """Writes src (flattened) into dst (C-contiguous, writable, modified in place) from the element write_start addresses."""
+    assert dst.flags["C_CONTIGUOUS"] and dst.flags["WRITEABLE"]
+    src = _c(src)
+    _check(lib().orc_index_write(dst.dtype.itemsize, _p(dst), dst.ndim, _p(_u64(dst.shape)), _p(src), src.size, _p(_u64(write_start))),
+           "index_write")
+    return dst
 
 
 def softmax(x, bf16=False):

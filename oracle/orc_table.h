@@ -12,6 +12,9 @@ struct OrcTable {
     int (*broadcast)(int, const void*, void*, int, const uint64_t*, int, const uint64_t*, int);
     int (*concat)(int, int, const void* const*, int, const uint64_t*, int, void*);
     int (*cache)(int, void*, int, const uint64_t*, const void*, const uint64_t*, int, uint64_t, void*);
+    int (*rope)(int, const void*, void*, const uint64_t*, uint64_t, float, uint64_t);
+    int (*index_select)(int, const void*, int, const uint64_t*, const int32_t*, uint64_t, int, void*);
+    int (*index_write)(int, void*, int, const uint64_t*, const void*, uint64_t, const uint64_t*);
     int (*softmax)(int, const void*, void*, size_t, size_t);
     int (*layer_norm)(int, const void*, const void*, const void*, void*, size_t, size_t, float, size_t);
     int (*rms_norm)(int, const void*, const void*, void*, size_t, size_t, float, size_t);

@@ -32,6 +32,15 @@ int orc_cache(int eb, void* cache, int rank, const uint64_t* cs, const void* sou
               void* dst) {
     return table().cache(eb, cache, rank, cs, source, ss, dim, offset, dst);
 }
+int orc_rope(int dt, const void* x, void* y, const uint64_t* shape, uint64_t dim, float base, uint64_t offset) {
+    return table().rope(dt, x, y, shape, dim, base, offset);
+}
+int orc_index_select(int eb, const void* src, int rank, const uint64_t* ss, const int32_t* indices, uint64_t n, int dim, void* dst) {
+    return table().index_select(eb, src, rank, ss, indices, n, dim, dst);
+}
+int orc_index_write(int eb, void* dst, int rank, const uint64_t* ds, const void* src, uint64_t n, const uint64_t* write_start) {
+    return table().index_write(eb, dst, rank, ds, src, n, write_start);
+}
 int orc_softmax(int dt, const void* x, void* y, size_t rows, size_t cols) { return table().softmax(dt, x, y, rows, cols); }
 int orc_layer_norm(int dt, const void* x, const void* s, const void* b, void* y, size_t rows, size_t cols, float eps,
                    size_t shape0) {

@@ -18,6 +18,9 @@
  *   unary f16 ............................ exhaustive (65536 inputs) against a numpy float16 model
  *   softmax, layer_norm, rms_norm ........ torch at the reference's own tolerances + invariants
  *   group_norm ........................... torch F.group_norm (the reference CPU path is a no-op)
+ *   cache, index_select, index_write ..... numpy concatenate / take / flat assignment and the reference's own test cases
+ *   rope ................................. float64 closed form of the half-rotation RoPE (what the reference's mlx ground
+ *                                          truth computes), rotation invariants, offset additivity
  *   PARITY UNPINNED: the accumulation type of `Sum for f16` inside `mean` (assumed: f32
  *   accumulation, one rounding; switchable with orc_set_f16_sum_mode) - the `half` crate is
  *   not present in the reference tree and no reference test exercises the f16 CPU path.
@@ -62,6 +65,14 @@ int orc_concat(int elem_bytes, int n_inputs, const void* const* xs, int rank, co
  * ground truth): dst = cat(cache[.. :offset ..], source) along dim, and source is also written into cache at offset. */
 int orc_cache(int elem_bytes, void* cache, int rank, const uint64_t* cache_shape, const void* source, const uint64_t* source_shape,
               int dim, uint64_t offset, void* dst);
+
+/* RoPE on [B, H, S, D] (crates/ratchet-core/src/cpu/rope.rs:7-143): F32 only, as in the reference; returns 1 for other dtypes */
+int orc_rope(int dt, const void* x, void* y, const uint64_t* shape4, uint64_t dim, float base, uint64_t offset);
+/* IndexSelect (cpu/mod.rs:44-84) and IndexWrite (ops/index_write.rs:96-104); an out-of-range index / run is an error */
+int orc_index_select(int elem_bytes, const void* src, int rank, const uint64_t* src_shape, const int32_t* indices, uint64_t n_indices,
+                     int dim, void* dst);
+int orc_index_write(int elem_bytes, void* dst, int rank, const uint64_t* dst_shape, const void* src, uint64_t src_numel,
+                    const uint64_t* write_start);
 
 int orc_softmax(int dt, const void* x, void* y, size_t rows, size_t cols);
 /* shape0 = size of the input's first dimension: the reference broadcasts scale/bias with a

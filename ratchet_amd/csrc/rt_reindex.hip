@@ -185,6 +185,39 @@ __global__ void __launch_bounds__(BLOCK) cache_kernel(VecT* __restrict__ cache, 
     }
 }
 
+// IndexSelect: dst[left, i, right] = src[left, indices[i], right].  One thread per vector of the `right` run; an index
+// outside [0, src_dim) (the reference panics on it) yields a row of zeros rather than a wild read.
+struct SelectArgs {
+    FastDiv rv;              // vectors per `right` run
+    FastDiv n_ids;
+    uint32_t src_dim;
+    uint32_t nvec;
+};
+
+template <typename VecT>
+__global__ void __launch_bounds__(BLOCK) index_select_kernel(const VecT* __restrict__ src, const int32_t* __restrict__ indices,
+                                                             VecT* __restrict__ dst, SelectArgs p) {
+    const uint32_t v = blockIdx.x * BLOCK + threadIdx.x;
+    if (v >= p.nvec) return;
+    uint32_t row, col, left, i;
+    fd_divmod(v, p.rv, row, col);
+    fd_divmod(row, p.n_ids, left, i);
+    const uint32_t idx = (uint32_t)indices[i];
+    VecT val = {};
+    if (idx < p.src_dim) val = src[((uint64_t)left * p.src_dim + idx) * p.rv.d + col];
+    st_stream(dst + v, val);
+}
+
+// IndexWrite: a flat run of src copied into dst from a linear offset (bytes here)
+__global__ void __launch_bounds__(BLOCK) index_write_vec_kernel(v4u* __restrict__ dst, const v4u* __restrict__ src, uint64_t nvec) {
+    const uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+    if (i < nvec) dst[i] = ld_stream(src + i);
+}
+__global__ void __launch_bounds__(BLOCK) index_write_u16_kernel(uint16_t* __restrict__ dst, const uint16_t* __restrict__ src, uint64_t n) {
+    const uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+    if (i < n) dst[i] = src[i];
+}
+
 inline unsigned blocks_for(uint64_t items, uint64_t per_block) {
     const uint64_t b = (items + per_block - 1) / per_block;
     return (unsigned)(b ? b : 1);
@@ -529,6 +562,79 @@ int rt_cache(rt_device* dev, int elem_bytes, void* cache, const uint32_t cache_s
     else
         hipLaunchKernelGGL((cache_kernel<uint16_t>), grid, dim3(BLOCK), 0, dev->stream, (uint16_t*)cache, (const uint16_t*)source, (uint16_t*)dst, p);
     RT_CHECK_LAUNCH("cache_kernel");
+    return RT_OK;
+}
+
+int rt_index_select(rt_device* dev, int elem_bytes, const void* src, const uint32_t src_shape[4], const int32_t* indices,
+                    uint32_t n_indices, int dim, void* dst) {
+    RT_REQUIRE(elem_bytes == 2 || elem_bytes == 4, RT_ERR_ARG, "rt_index_select: elem_bytes must be 2 or 4, got %d", elem_bytes);
+    RT_REQUIRE(dim >= 0 && dim < 4, RT_ERR_ARG, "rt_index_select: dim %d out of range", dim);
+    RT_REQUIRE(src_shape, RT_ERR_NULL_POINTER, "rt_index_select: NULL shape");
+    RT_REQUIRE(n_indices > 0, RT_ERR_SHAPE, "rt_index_select: no indices");
+    uint64_t left = 1, right = 1;
+    for (int a = 0; a < 4; a++) {
+        RT_REQUIRE(src_shape[a] > 0, RT_ERR_SHAPE, "rt_index_select: zero extent in dim %d", a);
+        if (a < dim) left *= src_shape[a];
+        if (a > dim) right *= src_shape[a];
+    }
+    RT_REQUIRE(left * src_shape[dim] * right <= RT_MAX_NUMEL, RT_ERR_SIZE, "rt_index_select: source too large");
+    RT_REQUIRE(src && indices && dst, RT_ERR_NULL_POINTER, "rt_index_select: NULL operand");
+    RT_REQUIRE(rt_aligned(src, (size_t)elem_bytes) && rt_aligned(dst, (size_t)elem_bytes) && rt_aligned(indices, 4), RT_ERR_ALIGN,
+               "rt_index_select: misaligned pointer");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    const uint64_t run_b = right * elem_bytes;
+    int vb = 16;
+    for (; vb > elem_bytes; vb >>= 1)
+        if (run_b % vb == 0 && rt_aligned(src, (size_t)vb) && rt_aligned(dst, (size_t)vb)) break;
+    const uint64_t nvec = left * n_indices * (run_b / vb);
+    RT_REQUIRE(nvec <= 0xffffffffull - BLOCK && left * n_indices <= 0xffffffffull && run_b / vb <= 0xffffffffull, RT_ERR_SIZE,
+               "rt_index_select: output too large for 32-bit vector indices");
+    SelectArgs p;
+    p.rv = make_fastdiv((uint32_t)(run_b / vb));
+    p.n_ids = make_fastdiv(n_indices);
+    p.src_dim = src_shape[dim];
+    p.nvec = (uint32_t)nvec;
+    const dim3 grid(blocks_for(nvec, BLOCK)), block(BLOCK);
+    if (vb == 16) hipLaunchKernelGGL((index_select_kernel<v4u>), grid, block, 0, dev->stream, (const v4u*)src, indices, (v4u*)dst, p);
+    else if (vb == 8) hipLaunchKernelGGL((index_select_kernel<v2u>), grid, block, 0, dev->stream, (const v2u*)src, indices, (v2u*)dst, p);
+    else if (vb == 4) hipLaunchKernelGGL((index_select_kernel<uint32_t>), grid, block, 0, dev->stream, (const uint32_t*)src, indices, (uint32_t*)dst, p);
+    else hipLaunchKernelGGL((index_select_kernel<uint16_t>), grid, block, 0, dev->stream, (const uint16_t*)src, indices, (uint16_t*)dst, p);
+    RT_CHECK_LAUNCH("index_select_kernel");
+    return RT_OK;
+}
+
+int rt_index_write(rt_device* dev, int elem_bytes, void* dst, const uint32_t dst_shape[4], const void* src, uint64_t src_numel,
+                   const uint32_t write_start[4]) {
+    RT_REQUIRE(elem_bytes == 2 || elem_bytes == 4, RT_ERR_ARG, "rt_index_write: elem_bytes must be 2 or 4, got %d", elem_bytes);
+    RT_REQUIRE(dst_shape && write_start, RT_ERR_NULL_POINTER, "rt_index_write: NULL shape");
+    uint64_t numel = 1, off = 0;
+    for (int a = 0; a < 4; a++) {
+        RT_REQUIRE(dst_shape[a] > 0, RT_ERR_SHAPE, "rt_index_write: zero extent in dim %d", a);
+        RT_REQUIRE(write_start[a] < dst_shape[a], RT_ERR_SHAPE, "rt_index_write: write_start[%d] = %u outside extent %u", a, write_start[a],
+                   dst_shape[a]);
+        off = off * dst_shape[a] + write_start[a];
+        numel *= dst_shape[a];
+        RT_REQUIRE(numel <= RT_MAX_NUMEL, RT_ERR_SIZE, "rt_index_write: destination too large");
+    }
+    // the reference's kernel writes D[offset + i] for i < src_numel with no bound (ops/index_write.rs:96-104)
+    RT_REQUIRE(src_numel <= numel && off + src_numel <= numel, RT_ERR_SHAPE, "rt_index_write: %llu elements from offset %llu leave the destination",
+               (unsigned long long)src_numel, (unsigned long long)off);
+    if (src_numel == 0) return dev ? RT_OK : rt_fail(RT_ERR_NULL_DEVICE, "rt_device is NULL");
+    RT_REQUIRE(dst && src, RT_ERR_NULL_POINTER, "rt_index_write: NULL operand");
+    RT_REQUIRE(rt_aligned(dst, (size_t)elem_bytes) && rt_aligned(src, (size_t)elem_bytes), RT_ERR_ALIGN, "rt_index_write: misaligned pointer");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    unsigned char* d = static_cast<unsigned char*>(dst) + off * elem_bytes;
+    const uint64_t bytes = src_numel * elem_bytes;
+    if (rt_aligned(d, 16) && rt_aligned(src, 16) && bytes % 16 == 0) {
+        hipLaunchKernelGGL(index_write_vec_kernel, dim3(blocks_for(bytes / 16, BLOCK)), dim3(BLOCK), 0, dev->stream, (v4u*)d, (const v4u*)src,
+                           bytes / 16);
+    } else {
+        hipLaunchKernelGGL(index_write_u16_kernel, dim3(blocks_for(bytes / 2, BLOCK)), dim3(BLOCK), 0, dev->stream, (uint16_t*)d,
+                           (const uint16_t*)src, bytes / 2);
+    }
+    RT_CHECK_LAUNCH("index_write kernel");
     return RT_OK;
 }
 

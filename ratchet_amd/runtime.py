@@ -220,6 +220,29 @@ class Device:
                                 dim + (4 - rank), offset, out.ptr))
         return out
 
+    def index_select(self, src, indices, dim, out=None):
+        """indices: 1-D I32 buffer."""
+        rank = len(src.shape)
+        out_shape = list(src.shape)
+        out_shape[dim] = indices.numel
+        out = out or Buffer(self, out_shape, src.dt)
+        check(self.lib.rt_index_select(self.handle, _DT_BYTES[src.dt], src.ptr, shape4(src.shape), indices.ptr, indices.numel,
+                                       dim + (4 - rank), out.ptr))
+        return out
+
+    def index_write(self, dst, src, write_start):
+        """dst is modified in place and returned."""
+        pad = 4 - len(dst.shape)
+        check(self.lib.rt_index_write(self.handle, _DT_BYTES[dst.dt], dst.ptr, shape4(dst.shape), src.ptr, src.numel,
+                                      (ctypes.c_uint32 * 4)(*([0] * pad + [int(w) for w in write_start]))))
+        return dst
+
+    def rope(self, x, dim, base, offset, out=None):
+        """x [B, H, S, D]; out may be x."""
+        out = out or Buffer(self, x.shape, x.dt)
+        check(self.lib.rt_rope(self.handle, x.dt, x.ptr, out.ptr, shape4(x.shape), dim, base, offset))
+        return out
+
     def softmax(self, x, out=None, mode=_lib.SOFTMAX_REFERENCE):
         cols = x.shape[-1]
         out = out or Buffer(self, x.shape, x.dt)

@@ -129,6 +129,22 @@ def test_reduction_validation(lib):
     assert lib.rt_group_norm(None, _lib.F16, SOME, None, None, SOME, 1, 8, 4, 4, 1e-5) == 8
 
 
+def test_rope_and_index_validation(lib):
+    shp = u4(1, 2, 4, 24)
+    assert lib.rt_rope(None, _lib.F32, SOME, SOME, shp, 16, 10000.0, 0) == 8
+    assert lib.rt_rope(None, _lib.F32, SOME, SOME, shp, 12, 10000.0, 0) == 4                 # dim % 8 (ops/rope.rs:57)
+    assert lib.rt_rope(None, _lib.F32, SOME, SOME, shp, 32, 10000.0, 0) == 4                 # dim > head_dim (ops/rope.rs:56)
+    assert lib.rt_rope(None, _lib.I32, SOME, SOME, shp, 16, 10000.0, 0) == 2
+    assert lib.rt_rope(None, _lib.F32, SOME, SOME, shp, 16, -1.0, 0) == 7
+    assert lib.rt_index_select(None, 4, SOME, u4(1, 1, 8, 4), SOME, 3, 2, SOME) == 8
+    assert lib.rt_index_select(None, 4, SOME, u4(1, 1, 8, 4), SOME, 0, 2, SOME) == 4
+    assert lib.rt_index_select(None, 4, SOME, u4(1, 1, 8, 4), None, 3, 2, SOME) == 1
+    assert lib.rt_index_select(None, 1, SOME, u4(1, 1, 8, 4), SOME, 3, 2, SOME) == 7
+    assert lib.rt_index_write(None, 4, SOME, u4(1, 1, 3, 2), SOME, 2, u4(0, 0, 2, 0)) == 8
+    assert lib.rt_index_write(None, 4, SOME, u4(1, 1, 3, 2), SOME, 3, u4(0, 0, 2, 0)) == 4   # the run would leave dst
+    assert lib.rt_index_write(None, 4, SOME, u4(1, 1, 3, 2), SOME, 1, u4(0, 0, 3, 0)) == 4   # write_start outside dst
+
+
 def test_fused_pattern_validation(lib):
     f32p = ctypes.cast(ctypes.c_void_p(0x1000), ctypes.c_void_p)
     assert lib.rt_norm_via_f32(None, 0, _lib.F16, SOME, f32p, None, SOME, 4, 8, 1e-5) == 8

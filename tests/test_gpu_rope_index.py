@@ -1,0 +1,89 @@
+"""GPU parity of RoPE, IndexSelect and IndexWrite against the oracle (crates/ratchet-core/src/cpu/rope.rs:23-143,
+cpu/mod.rs:44-84, ops/index_write.rs:96-104).  IndexSelect / IndexWrite: bit-exact.  RoPE f32: the rounding points are the
+oracle's; only sin / cos may differ from the host C library's by an ulp, so the bar is 1e-6 (the reference tests at 1e-2)."""
+import numpy as np
+import pytest
+
+from gpu_util import randn, same_bits
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    from ratchet_amd import Device
+
+    return Device(0)
+
+
+@pytest.mark.parametrize("shape,dim,offset", [((1, 2, 5, 16), 16, 0), ((2, 3, 7, 32), 16, 5), ((1, 32, 128, 96), 96, 0), ((1, 32, 1, 96), 96, 4095),
+                                              ((1, 4, 1, 80), 32, 1023), ((2, 1, 300, 128), 64, 17), ((1, 32, 512, 80), 32, 0)])
+def test_rope_f32(dev, oracle, shape, dim, offset):
+    rng = np.random.default_rng(601)
+    x = rng.standard_normal(shape).astype(np.float32)
+    want = oracle.rope(x, dim, 10000.0, offset)
+    d = dev.upload(x)
+    got = dev.rope(d, dim, 10000.0, offset).to_numpy()
+    bad, mx = oracle.count_not_close(got, want, 1e-6, 1e-6)
+    assert bad == 0, (bad, mx)
+    assert (got.view(np.uint32) != want.view(np.uint32)).mean() < 0.1                       # mostly the same bits (one sin/cos ulp moves a column of all heads)
+    assert np.array_equal(got[..., dim:], x[..., dim:])
+    inplace = dev.rope(d, dim, 10000.0, offset, out=d).to_numpy()                            # the reference's GPU kernel is in-place only
+    assert same_bits(inplace, got)
+
+
+def test_rope_16bit_is_widen_rotate_round(dev, oracle):
+    rng = np.random.default_rng(602)
+    x = randn(rng, (1, 8, 40, 96), np.float16)
+    want = oracle.cast(oracle.rope(oracle.cast(x, np.float32), 96, 10000.0, 7), np.float16)
+    got = dev.rope(dev.upload(x), 96, 10000.0, 7).to_numpy()
+    bad, mx = oracle.count_not_close(got, want, 1e-3, 1e-3)
+    assert bad == 0, (bad, mx)
+    assert (got.view(np.uint16) != want.view(np.uint16)).mean() < 0.001
+
+
+def test_rope_rejects_bad_arguments(dev):
+    from ratchet_amd import RatchetError
+
+    x = dev.upload(np.zeros((1, 2, 4, 24), np.float32))
+    for dim, base in ((12, 10000.0), (32, 10000.0), (16, 0.0)):
+        with pytest.raises(RatchetError) as e:
+            dev.rope(x, dim, base, 0)
+        assert e.value.status in (4, 7)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_index_select(dev, oracle, dtype):
+    rng = np.random.default_rng(603)
+    cases = [((256, 32), 0, [64, 192, 255]),                     # the reference's fixed case (ops/select.rs:350-357)
+             ((32064, 256), 0, rng.integers(0, 32064, 77)),      # an embedding table
+             ((51, 384), 0, rng.integers(0, 51, 1)), ((7, 9), 1, rng.integers(0, 9, 20)), ((3, 5, 11), 1, rng.integers(0, 5, 6)),
+             ((2, 3, 4, 6), 2, rng.integers(0, 4, 9)), ((64, 3), 0, rng.integers(0, 64, 40)), ((10, 7), 0, rng.integers(0, 10, 5))]
+    for shape, dim, idx in cases:
+        src = randn(rng, shape, dtype)
+        idx = np.asarray(idx, dtype=np.int32)
+        got = dev.index_select(dev.upload(src), dev.upload(idx), dim).to_numpy()
+        assert np.array_equal(got, oracle.index_select(src, idx, dim)), (shape, dim)
+        assert np.array_equal(got, np.take(src, idx, axis=dim))
+    src = randn(rng, (16, 8), dtype)
+    got = dev.index_select(dev.upload(src), dev.upload(np.array([3, 16, -1, 0], np.int32)), 0).to_numpy()
+    assert np.array_equal(got[[0, 3]], src[[3, 0]]) and not got[[1, 2]].any()                # out-of-range rows come back as zeros
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_index_write(dev, oracle, dtype):
+    rng = np.random.default_rng(604)
+    dst = np.array([1, 2, 3, 4, 5, 6], dtype).reshape(3, 2)     # the reference's own test (ops/index_write.rs:203-224)
+    d = dev.upload(dst)
+    dev.index_write(d, dev.upload(np.array([[7, 8]], dtype)), [2, 0])
+    assert np.array_equal(d.to_numpy(), np.array([[1, 2], [3, 4], [7, 8]], dtype))
+    for shape, sshape, start in (((1, 32, 64, 80), (1, 32, 1, 80), (0, 0, 17, 0)), ((4, 100), (37,), (1, 3)), ((2, 3, 8), (2, 8), (0, 1, 0)),
+                                 ((1024, 1024), (512, 1024), (512, 0)), ((5, 7), (1,), (4, 6))):
+        dst, src = randn(rng, shape, dtype), randn(rng, sshape, dtype)
+        d = dev.upload(dst)
+        dev.index_write(d, dev.upload(src), start)
+        assert np.array_equal(d.to_numpy(), oracle.index_write(dst.copy(), src, start)), (shape, sshape, start)
+    from ratchet_amd import RatchetError
+    with pytest.raises(RatchetError) as e:
+        dev.index_write(dev.upload(np.zeros((2, 3), dtype)), dev.upload(np.zeros(3, dtype)), [1, 1])
+    assert e.value.status == 4

@@ -382,3 +382,80 @@ def test_cache_reference_case_and_properties(oracle):
         oracle.cache(np.zeros((1, 2, 4, 8), np.float32), np.zeros((1, 2, 2, 8), np.float32), 2, 3)     # 3 + 2 > 4
     with pytest.raises(ValueError):
         oracle.cache(np.zeros((4, 8), np.float32), np.zeros((1, 8), np.float32), 0, 0)                  # rank < 3 (cache.rs:125)
+
+
+# ------------------------------------------------------------------------------------------- rope / index_select / index_write
+def _rope_f64(x, dim, base, offset):
+    """Half-rotation RoPE in float64: what mlx.nn.RoPE(dim, traditional=False), the ground truth of the reference's own test
+    (ops/rope.rs:275-300), computes."""
+    half = dim // 2
+    S = x.shape[2]
+    pos = np.arange(offset, offset + S, dtype=np.float64)[:, None]
+    inv = np.float64(base) ** (-np.arange(half, dtype=np.float64) / half)
+    th = pos * inv
+    c, s = np.cos(th), np.sin(th)
+    x1, x2 = x[..., :half].astype(np.float64), x[..., half:dim].astype(np.float64)
+    return np.concatenate([x1 * c - x2 * s, x1 * s + x2 * c, x[..., dim:].astype(np.float64)], axis=-1)
+
+
+@pytest.mark.parametrize("shape,dim,offset", [((1, 2, 5, 16), 16, 0), ((2, 3, 7, 32), 16, 5), ((1, 32, 64, 96), 96, 0), ((1, 4, 1, 80), 32, 1023),
+                                              ((1, 1, 300, 128), 64, 17)])
+def test_rope_matches_float64_closed_form(oracle, shape, dim, offset):
+    rng = np.random.default_rng(31)
+    x = rng.standard_normal(shape).astype(np.float32)
+    y = oracle.rope(x, dim, 10000.0, offset)
+    want = _rope_f64(x, dim, 10000.0, offset)
+    # f32 theta carries |theta| * 2^-24 of phase error (positions up to ~1300 here), so ~1e-4 absolute; the reference's bar is 1e-2
+    assert np.abs(y - want).max() < 2e-4 * max(1.0, (offset + shape[2]) / 1000.0)
+    assert np.array_equal(y[..., dim:], x[..., dim:])                                       # pass-through columns untouched
+
+
+def test_rope_invariants(oracle):
+    rng = np.random.default_rng(32)
+    x = rng.standard_normal((2, 2, 9, 24)).astype(np.float32)
+    half = 8
+    y = oracle.rope(x, 16, 10000.0, 0)
+    assert np.array_equal(y[:, :, 0], x[:, :, 0])                                           # position 0: theta = 0, cos 1, sin 0
+    n_in = x[..., :half].astype(np.float64) ** 2 + x[..., half:16].astype(np.float64) ** 2
+    n_out = y[..., :half].astype(np.float64) ** 2 + y[..., half:16].astype(np.float64) ** 2
+    assert np.allclose(n_in, n_out, rtol=1e-5, atol=1e-6)                                   # a rotation keeps each pair's norm
+    # the offset only shifts positions: rows 3.. of offset 0 equal rows 0.. of offset 3, bit for bit
+    z = oracle.rope(np.ascontiguousarray(x[:, :, 3:]), 16, 10000.0, 3)
+    assert np.array_equal(z, y[:, :, 3:])
+    # a transposed pairing (interleaved "traditional" RoPE) or a swapped sign would not pass this known answer:
+    # x1 = 1, x2 = 0 at position 1, frequency 0 -> (cos 1, sin 1)
+    e = np.zeros((1, 1, 2, 8), np.float32)
+    e[0, 0, 1, 0] = 1.0
+    r = oracle.rope(e, 8, 10000.0, 0)
+    assert abs(r[0, 0, 1, 0] - np.cos(1.0)) < 1e-7 and abs(r[0, 0, 1, 4] - np.sin(1.0)) < 1e-7 and r[0, 0, 1, 1] == 0
+    with pytest.raises(ValueError):
+        oracle.rope(x, 12, 10000.0, 0)                                                      # dim % 8 != 0 (ops/rope.rs:57)
+    with pytest.raises(ValueError):
+        oracle.rope(x.astype(np.float16), 16, 10000.0, 0)                                   # todo!() in cpu_rope for f16
+
+
+def test_index_select_is_numpy_take(oracle):
+    rng = np.random.default_rng(33)
+    for shape, dim, dtype in (((256, 32), 0, np.float32), ((51, 384), 0, np.float16), ((7, 9), 1, np.float32), ((3, 5, 11), 1, np.float16),
+                              ((2, 3, 4, 6), 2, np.float32)):
+        src = rng.standard_normal(shape).astype(dtype)
+        idx = rng.integers(0, shape[dim], size=int(rng.integers(1, 64))).astype(np.int32)
+        assert np.array_equal(oracle.index_select(src, idx, dim), np.take(src, idx, axis=dim)), (shape, dim)
+    # the reference's fixed case (ops/select.rs:350-357): rows 64, 192, 255 of a [256, 32] table
+    src = rng.standard_normal((256, 32)).astype(np.float32)
+    assert np.array_equal(oracle.index_select(src, [64, 192, 255], 0), src[[64, 192, 255]])
+    with pytest.raises(ValueError):
+        oracle.index_select(src, [256], 0)
+
+
+def test_index_write_reference_case(oracle):
+    # crates/ratchet-core/src/ops/index_write.rs:203-224: dst [[1,2],[3,4],[5,6]], src [[7,8]], write_start [2,0] -> [[1,2],[3,4],[7,8]]
+    dst = np.array([1, 2, 3, 4, 5, 6], np.float32).reshape(3, 2)
+    oracle.index_write(dst, np.array([[7, 8]], np.float32), [2, 0])
+    assert np.array_equal(dst, np.array([[1, 2], [3, 4], [7, 8]], np.float32))
+    # a flat run, not a sub-block: three elements from [0,1] of a [2,3] tensor wrap into the next row
+    d = np.zeros((2, 3), np.float16)
+    oracle.index_write(d, np.array([1, 2, 3], np.float16), [0, 1])
+    assert np.array_equal(d, np.array([[0, 1, 2], [3, 0, 0]], np.float16))
+    with pytest.raises(ValueError):
+        oracle.index_write(d, np.array([1, 2, 3], np.float16), [1, 1])                      # would leave dst
