@@ -52,6 +52,9 @@ rth_tensor* rth_cat(const rth_tensor* const* xs, int n, size_t dim);
 /* one-launch replacements of full() -> norm / softmax / activation -> cast(dt) at resolve(); on by default */
 void rth_set_pattern_fusion(int on);
 rth_tensor* rth_cache(const rth_tensor* cache, const rth_tensor* source, size_t dim, size_t offset);   /* tensor.rs:481-486 */
+rth_tensor* rth_rope(const rth_tensor* x, size_t dim, float base, size_t offset);                       /* tensor.rs:392-397 */
+rth_tensor* rth_index_select(const rth_tensor* x, const rth_tensor* indices, size_t dim);               /* tensor.rs:497-502 */
+rth_tensor* rth_index_write(const rth_tensor* dst, const rth_tensor* src, int rank, const uint64_t* write_start);   /* tensor.rs:504-510 */
 rth_tensor* rth_permute(const rth_tensor* x, int n, const uint64_t* dims);
 rth_tensor* rth_broadcast_to(const rth_tensor* x, int rank, const uint64_t* shape);
 

@@ -96,7 +96,7 @@ Buffer::~Buffer() {
 }
 
 // ------------------------------------------------------------------------------------------------------------ graph
-enum class Kind { Const, Binary, Unary, Cast, Permute, Slice, Broadcast, Concat, Cache, Softmax, LayerNorm, RMSNorm, GroupNorm, View };
+enum class Kind { Const, Binary, Unary, Cast, Permute, Slice, Broadcast, Concat, Cache, RoPE, IndexSelect, IndexWrite, Softmax, LayerNorm, RMSNorm, GroupNorm, View };
 
 struct Node {
     uint64_t id = 0;
@@ -164,6 +164,9 @@ const char* Tensor::op_name() const {
         case Kind::Broadcast: return "Broadcast";
         case Kind::Concat: return "Concat";
         case Kind::Cache: return "Cache";
+        case Kind::RoPE: return "RoPE";
+        case Kind::IndexSelect: return "IndexSelect";
+        case Kind::IndexWrite: return "IndexWrite";
         case Kind::Softmax: return "Softmax";
         case Kind::View: return "View";
         default: return "Norm";
@@ -347,6 +350,54 @@ Tensor Tensor::cache(const Tensor& source, size_t dim, size_t offset) const {
     n->dim = dim;
     n->groups = offset;                        // reuses the integer slot: the write offset
     n->srcs = {*this, source};
+    return Tensor(n);
+}
+
+// RoPE guards: ops/rope.rs:52-66
+Tensor Tensor::rope(size_t dim, float base, size_t offset) const {
+    if (rank() != 4) throw Error("RankMismatch", "rope needs rank 4, got " + std::to_string(rank()));
+    if (shape()[3] < dim) throw Error("ShapeMismatch", "rope dim " + std::to_string(dim) + " exceeds head dim " + std::to_string(shape()[3]));
+    if (dim == 0 || dim % 8 != 0) throw Error("ShapeMismatch", "rope dim " + std::to_string(dim) + " is not a multiple of 8");
+    if (!is_float(dt())) throw Error("UnsupportedDType", as_str(dt()));
+    auto n = new_node(Kind::RoPE, shape(), dt(), device());
+    n->dim = dim;
+    n->groups = offset;                        // integer slot: the position offset
+    n->eps = base;                             // float slot: the frequency base
+    n->srcs = {*this};
+    return Tensor(n);
+}
+
+// IndexSelect guards: ops/select.rs:67-79 (rank-2 source, rank-1 I32 indices) and compute_view :48-60
+Tensor Tensor::index_select(const Tensor& indices, size_t dim) const {
+    require_same_device(*this, indices);
+    if (rank() != 2) throw Error("RankMismatch", "index_select source must have rank 2, got " + std::to_string(rank()));
+    if (indices.rank() != 1) throw Error("RankMismatch", "index_select indices must have rank 1, got " + std::to_string(indices.rank()));
+    if (indices.dt() != DType::I32) throw Error("DTypeMismatch", std::string("expected I32, got ") + as_str(indices.dt()));
+    if (dim >= rank()) throw Error("DimOutOfRange", "index_select dim " + std::to_string(dim));
+    if (size_of(dt()) != 2 && size_of(dt()) != 4) throw Error("UnsupportedDType", as_str(dt()));
+    Shape out = shape();
+    out[dim] = indices.shape()[0];
+    auto n = new_node(Kind::IndexSelect, out, dt(), device());
+    n->dim = dim;
+    n->srcs = {*this, indices};
+    return Tensor(n);
+}
+
+// IndexWrite has no guards in the reference (ops/index_write.rs:29-33); the run it writes must stay inside dst
+Tensor Tensor::index_write(const Tensor& src, const std::vector<size_t>& write_start) const {
+    require_same_device(*this, src);
+    require_rank4(shape(), "index_write");
+    if (dt() != src.dt()) throw Error("DTypeMismatch", std::string("expected ") + as_str(dt()) + ", got " + as_str(src.dt()));
+    if (write_start.size() != rank()) throw Error("RankMismatch", "write_start must have one entry per dimension");
+    size_t off = 0;
+    for (size_t i = 0; i < rank(); i++) {
+        if (write_start[i] >= shape()[i]) throw Error("IndexOutOfBounds", "write_start[" + std::to_string(i) + "] = " + std::to_string(write_start[i]));
+        off = off * shape()[i] + write_start[i];
+    }
+    if (off + src.numel() > numel()) throw Error("IndexOutOfBounds", "the written run leaves the destination");
+    auto n = new_node(Kind::IndexWrite, shape(), dt(), device());
+    n->dims = write_start;
+    n->srcs = {*this, src};
     return Tensor(n);
 }
 
@@ -699,6 +750,35 @@ struct Resolver {
                 check_rt(rt_cache(dev, (int)size_of(n->dt), src(0)->storage->ptr, cs, src(1)->storage->ptr, ss,
                                   (int)(n->dim + 4 - n->shape.rank()), (uint32_t)n->groups, n->storage->ptr),
                          "rt_cache");
+                launches++;
+                return;
+            }
+            case Kind::RoPE: {
+                uint32_t xs[4];
+                shape4(n->shape, xs);
+                if (!take_src0_if_unshared()) out_buffer();    // RoPE::supports_inplace() (ops/rope.rs:80-82)
+                check_rt(rt_rope(dev, dt, src(0)->storage->ptr, n->storage->ptr, xs, (uint32_t)n->dim, n->eps, (uint32_t)n->groups), "rt_rope");
+                launches++;
+                return;
+            }
+            case Kind::IndexSelect: {
+                uint32_t ss[4];
+                shape4(src(0)->shape, ss);
+                out_buffer();
+                check_rt(rt_index_select(dev, (int)size_of(n->dt), src(0)->storage->ptr, ss, static_cast<const int32_t*>(src(1)->storage->ptr),
+                                         (uint32_t)src(1)->shape[0], (int)(n->dim + 4 - n->shape.rank()), n->storage->ptr),
+                         "rt_index_select");
+                launches++;
+                return;
+            }
+            case Kind::IndexWrite: {
+                uint32_t ds[4], ws[4] = {0, 0, 0, 0};
+                shape4(n->shape, ds);
+                const size_t pad = 4 - n->dims.size();
+                for (size_t i = 0; i < n->dims.size(); i++) ws[pad + i] = (uint32_t)n->dims[i];
+                n->storage = src(0)->storage;                  // the destination's buffer is the result (ops/index_write.rs:40-50)
+                check_rt(rt_index_write(dev, (int)size_of(n->dt), n->storage->ptr, ds, src(1)->storage->ptr, src(1)->shape.numel(), ws),
+                         "rt_index_write");
                 launches++;
                 return;
             }

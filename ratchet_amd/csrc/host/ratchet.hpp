@@ -155,6 +155,10 @@ class Tensor {
     // source into the cache's storage at offset
     Tensor cache(const Tensor& source, size_t dim, size_t offset) const;
     Tensor broadcast_to(const Shape& shape) const;                                                       // tensor.rs:488-495
+    Tensor rope(size_t dim, float base, size_t offset) const;                                            // tensor.rs:392-397
+    Tensor index_select(const Tensor& indices, size_t dim) const;                                        // tensor.rs:497-502
+    // self is the destination (tensor.rs:504-510): resolve() writes src into self's storage as a flat run from write_start
+    Tensor index_write(const Tensor& src, const std::vector<size_t>& write_start) const;
 
     // tensor.rs:861-863: runs every unresolved node this tensor depends on; returns after completion
     Tensor resolve() const;

@@ -118,6 +118,18 @@ void rth_set_pattern_fusion(int on) { ratchet::set_pattern_fusion(on != 0); }
 rth_tensor* rth_cache(const rth_tensor* cache, const rth_tensor* source, size_t dim, size_t offset) {
     return build([&] { return cache->t.cache(source->t, dim, offset); });
 }
+rth_tensor* rth_rope(const rth_tensor* x, size_t dim, float base, size_t offset) {
+    return build([&] { return x->t.rope(dim, base, offset); });
+}
+rth_tensor* rth_index_select(const rth_tensor* x, const rth_tensor* indices, size_t dim) {
+    return build([&] { return x->t.index_select(indices->t, dim); });
+}
+rth_tensor* rth_index_write(const rth_tensor* dst, const rth_tensor* src, int rank, const uint64_t* write_start) {
+    return build([&] {
+        std::vector<size_t> ws(write_start, write_start + rank);
+        return dst->t.index_write(src->t, ws);
+    });
+}
 rth_tensor* rth_permute(const rth_tensor* x, int n, const uint64_t* dims) {
     return build([&] {
         std::vector<size_t> d(dims, dims + (n > 0 ? n : 0));

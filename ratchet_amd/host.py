@@ -54,7 +54,8 @@ def load():
         "rth_from_host": [vp, vp, i, u64p, i], "rth_placeholder": [i, u64p, i], "rth_binary": [vp, vp, i], "rth_unary": [vp, i],
         "rth_cast": [vp, i], "rth_layer_norm": [vp, vp, vp, f], "rth_rms_norm": [vp, vp, f], "rth_group_norm": [vp, sz, vp, vp, f],
         "rth_softmax": [vp, sz, i], "rth_slice": [vp, i, u64p, u64p], "rth_view": [vp, i, u64p],
-        "rth_cat": [ctypes.POINTER(vp), i, sz], "rth_cache": [vp, vp, sz, sz], "rth_permute": [vp, i, u64p], "rth_broadcast_to": [vp, i, u64p],
+        "rth_cat": [ctypes.POINTER(vp), i, sz], "rth_cache": [vp, vp, sz, sz], "rth_rope": [vp, sz, f, sz], "rth_index_select": [vp, vp, sz],
+        "rth_index_write": [vp, vp, i, u64p], "rth_permute": [vp, i, u64p], "rth_broadcast_to": [vp, i, u64p],
     }.items():
         fn = getattr(H, name)
         fn.argtypes = args
@@ -206,6 +207,15 @@ class Tensor:
 
     def cache(self, source, dim, offset):
         return Tensor(self.H.rth_cache(self.handle, source.handle, dim, offset))
+
+    def rope(self, dim, base, offset):
+        return Tensor(self.H.rth_rope(self.handle, dim, base, offset))
+
+    def index_select(self, indices, dim):
+        return Tensor(self.H.rth_index_select(self.handle, indices.handle, dim))
+
+    def index_write(self, src, write_start):
+        return Tensor(self.H.rth_index_write(self.handle, src.handle, len(write_start), _u64(write_start)))
 
     def permute(self, dims):
         return Tensor(self.H.rth_permute(self.handle, len(dims), _u64(dims)))

@@ -275,3 +275,28 @@ def test_pattern_with_a_visible_intermediate_is_not_folded(hdev, oracle):
     want = oracle.cast(oracle.rms_norm(oracle.cast(x, np.float32), w, 1e-5, intended=True), np.float16)
     ok, info = close(oracle, y.to_numpy(), want, 1e-3)
     assert ok, info
+
+
+def test_rope_index_select_index_write_graphs(hdev, oracle):
+    """phi3's attention head prep (ratchet-models/src/phi3/attn.rs:118-133): x.full().rope(dim, base, offset).cast(dt); the embedding
+    lookup (index_select, dim 0); index_write with the reference's own case (ops/index_write.rs:203-224)."""
+    from ratchet_amd import _lib
+
+    rng = np.random.default_rng(408)
+    q = rng.standard_normal((1, 8, 33, 96)).astype(np.float32)
+    got = T(q, hdev).rope(96, 10000.0, 5).resolve().to_numpy()
+    bad, mx = oracle.count_not_close(got, oracle.rope(q, 96, 10000.0, 5), 1e-6, 1e-6)
+    assert bad == 0, (bad, mx)
+    q16 = q.astype(np.float16)
+    got16 = T(q16, hdev).full().rope(96, 10000.0, 5).cast(_lib.F16).resolve().to_numpy()
+    want16 = oracle.cast(oracle.rope(oracle.cast(q16, np.float32), 96, 10000.0, 5), np.float16)
+    ok, info = close(oracle, got16, want16, 1e-3)
+    assert ok, info
+    table = rng.standard_normal((1000, 64)).astype(np.float16)
+    ids = rng.integers(0, 1000, 19).astype(np.int32)
+    got = T(table, hdev).index_select(T(ids, hdev), 0).resolve().to_numpy()
+    assert np.array_equal(got, table[ids])
+    dst = T(np.array([1, 2, 3, 4, 5, 6], np.float32).reshape(3, 2), hdev)
+    out = dst.index_write(T(np.array([[7, 8]], np.float32), hdev), [2, 0]).resolve()
+    assert np.array_equal(out.to_numpy(), np.array([[1, 2], [3, 4], [7, 8]], np.float32))
+    assert np.array_equal(dst.to_numpy(), out.to_numpy())                      # in place: the destination's buffer is the result

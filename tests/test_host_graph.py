@@ -108,6 +108,32 @@ def test_cache_rules():
         assert e.value.kind == kind, (kind, e.value.kind)
 
 
+def test_rope_and_index_rules():
+    q = P(1, 32, 4096, 96)
+    assert q.rope(96, 10000.0, 0).shape == q.shape and q.rope(32, 10000.0, 7).op_name() == "RoPE"
+    for t, dim, kind in ((P(32, 4096, 96), 96, "RankMismatch"), (q, 128, "ShapeMismatch"), (q, 20, "ShapeMismatch"),
+                         (P(1, 2, 3, 8, dt=_lib.I32), 8, "UnsupportedDType")):     # RoPE::check_shapes / check_dtypes (ops/rope.rs:52-66)
+        with pytest.raises(HostError) as e:
+            t.rope(dim, 10000.0, 0)
+        assert e.value.kind == kind
+    table, ids = P(51865, 384, dt=F16), P(7, dt=_lib.I32)
+    y = table.index_select(ids, 0)                                               # IndexSelect::compute_view (ops/select.rs:48-60)
+    assert y.shape == (7, 384) and y.dt == F16 and y.op_name() == "IndexSelect"
+    assert table.index_select(ids, 1).shape == (51865, 7)
+    for src, idx, dim, kind in ((P(2, 3, 4), ids, 0, "RankMismatch"), (table, P(7, 1, dt=_lib.I32), 0, "RankMismatch"),
+                                (table, P(7), 0, "DTypeMismatch"), (table, ids, 2, "DimOutOfRange")):   # ops/select.rs:67-79
+        with pytest.raises(HostError) as e:
+            src.index_select(idx, dim)
+        assert e.value.kind == kind
+    dst = P(3, 2)
+    assert dst.index_write(P(1, 2), [2, 0]).shape == (3, 2)                      # the reference's test (ops/index_write.rs:203-224)
+    for src, ws, kind in ((P(1, 2), [3, 0], "IndexOutOfBounds"), (P(2, 2), [2, 0], "IndexOutOfBounds"), (P(1, 2), [2], "RankMismatch"),
+                          (P(1, 2, dt=F16), [2, 0], "DTypeMismatch")):
+        with pytest.raises(HostError) as e:
+            dst.index_write(src, ws)
+        assert e.value.kind == kind
+
+
 def test_softmax_and_norm_rules():
     x = P(1, 6, 1500, 1500)
     assert x.softmax(3).shape == x.shape
