@@ -227,8 +227,10 @@ __global__ void __launch_bounds__(BLOCK) softmax_seq16_kernel(const T* __restric
 // 15 waves thread (r, cv) owns the 16-byte vectors at columns
 // t*256 + cv*8 of row r, t = 0..NSLOT-1, and keeps their exp values in registers (NSLOT * 4 VGPRs) until the row sum is
 // known, so x is read once and y written once.
-//   exp: a 16-bit type has 65536 values; the part of the exact exp table that is not saturated (x in about
-//        [-17.5, 11.1]; below gives 0, above inf) is 38384 entries = 75 KiB and sits in LDS.  One ds_read_u16 per element.
+//   exp: a 16-bit type has 65536 values; the whole exact exp table (128 KiB) sits in LDS next to the 31 KiB of tiles
+//        (162 880 of the CU's 163 840 bytes), so exp is one ds_read_u16 per element with the bit pattern as the index:
+//        no range clamping, no NaN special case.  The kernel is bound by vector instruction issue as much as by HBM
+//        (removing two of ~16 VALU instructions per element moved it by 10 %), which is why the index math was cut.
 //   sum: per 256-column tile the exp values also go to an LDS tile (double buffered); lanes 0..29 of wave 0 each walk
 //        one row of the tile left to right with dependent v_add_f16 (3 ns each on this chip).  A tile is 16 KiB in and
 //        15 KiB out of HBM per CU, about 1 us at a CU's share of 8 TB/s; the walk of 256 columns takes 0.8 us, which is
@@ -242,45 +244,33 @@ constexpr int SP_BLOCK = 1024;
 constexpr int SP_ROWS = 30;                  // 15 loader waves x 2 rows each; wave 0 only walks
 constexpr int SP_TC = 256;
 constexpr int SP_PAD = 8;
-constexpr uint32_t SP_LUT_POS = 0x4990;      // entries for bit patterns 0x0000 .. 0x498f  (last ones are +inf)
-constexpr uint32_t SP_LUT_NEG = 0x4c60;      // entries for bit patterns 0x8000 .. 0xcc5f  (last ones are +0)
-constexpr size_t SP_LUT_BYTES = (SP_LUT_POS + SP_LUT_NEG) * sizeof(uint16_t);
-constexpr size_t SP_TILE_BYTES = 2 * 32 * (SP_TC + SP_PAD) * sizeof(uint16_t);
-constexpr size_t SP_SMEM_BYTES = SP_LUT_BYTES + SP_TILE_BYTES + 2 * 32 * sizeof(uint16_t);
+constexpr int SP_PF = 4;                     // tiles loaded ahead
+constexpr size_t SP_LUT_BYTES = 65536 * sizeof(uint16_t);
+constexpr size_t SP_TILE_BYTES = 2 * SP_ROWS * (SP_TC + SP_PAD) * sizeof(uint16_t);
+constexpr size_t SP_SMEM_BYTES = SP_LUT_BYTES + SP_TILE_BYTES + 2 * 32 * sizeof(uint16_t);      // 162 880 of the CU's 163 840 bytes
 
-typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
-typedef short i16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 
-// exp of two packed f16 bit patterns through the LDS table, branch free: both halves are clamped into the stored range
-// with packed 16-bit min/sub (the saturated ends of the table hold +inf and +0), then looked up.  NaNs are patched by
-// the caller.
+// exp of two packed f16 bit patterns: two lookups in the full 65536-entry table (NaN, inf and the saturated ends included)
 __device__ __forceinline__ uint32_t sp_exp_pair(const uint16_t* lut, uint32_t p) {
-    const u16x2 h = __builtin_bit_cast(u16x2, p);
-    const u16x2 neg = __builtin_bit_cast(u16x2, __builtin_bit_cast(i16x2, p) >> 15);       // 0xffff where the sign bit is set
-    const u16x2 top = (neg & (u16x2)(0x8000 + SP_LUT_NEG - SP_LUT_POS)) + (u16x2)(SP_LUT_POS - 1);
-    const u16x2 clamped = __builtin_elementwise_min(h, top);
-    const u16x2 idx = clamped - (neg & (u16x2)(0x8000 - SP_LUT_POS));
-    return (uint32_t)lut[idx.x] | ((uint32_t)lut[idx.y] << 16);
+    return (uint32_t)lut[p & 0xffffu] | ((uint32_t)lut[p >> 16] << 16);
 }
-// bit 15 / bit 31 set where the corresponding half of p is a NaN: (h & 0x7fff) > 0x7c00  <=>  (h & 0x7fff) + 0x3ff >= 0x8000
-__device__ __forceinline__ uint32_t sp_nan_bits(uint32_t p) { return ((p & 0x7fff7fffu) + 0x03ff03ffu) & 0x80008000u; }
 
-template <int NSLOT>
+template <int NSLOT, bool FULL>
 __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint16_t* __restrict__ table, const half_t* x, half_t* y,
                                                                       uint64_t rows, uint32_t cols) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint16_t* lut = reinterpret_cast<uint16_t*>(smem);
-    half_t (*tile)[32][SP_TC + SP_PAD] = reinterpret_cast<half_t (*)[32][SP_TC + SP_PAD]>(smem + SP_LUT_BYTES);
+    half_t (*tile)[SP_ROWS][SP_TC + SP_PAD] = reinterpret_cast<half_t (*)[SP_ROWS][SP_TC + SP_PAD]>(smem + SP_LUT_BYTES);
     half_t (*sums)[32] = reinterpret_cast<half_t (*)[32]>(smem + SP_LUT_BYTES + SP_TILE_BYTES);
 
-    // table -> LDS (16-byte copies; both ranges start 16-byte aligned in the table and have multiple-of-8 lengths)
+    // table -> LDS
     {
         const v4u* src = reinterpret_cast<const v4u*>(table);
         v4u* dst = reinterpret_cast<v4u*>(lut);
-        for (uint32_t i = threadIdx.x; i < SP_LUT_POS / 8; i += SP_BLOCK) dst[i] = src[i];
-        const v4u* srcn = reinterpret_cast<const v4u*>(table + 0x8000);
-        v4u* dstn = reinterpret_cast<v4u*>(lut + SP_LUT_POS);
-        for (uint32_t i = threadIdx.x; i < SP_LUT_NEG / 8; i += SP_BLOCK) dstn[i] = srcn[i];
+#pragma unroll
+        for (uint32_t i = 0; i < SP_LUT_BYTES / 16 / SP_BLOCK; i++) dst[i * SP_BLOCK + threadIdx.x] = src[i * SP_BLOCK + threadIdx.x];
     }
     const uint64_t ngroups = (rows + SP_ROWS - 1) / SP_ROWS;
     __syncthreads();                                         // table visible
@@ -329,53 +319,68 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
     }
 
     // ---------------------------------------------------------------------- waves 1..15: load, exp, park, divide, store
+    // Global accesses are raw buffer loads / stores: an access whose target does not exist (rows past the end, columns
+    // past a short row, the store of "the previous group" during the first one) gets an offset outside the buffer and
+    // the hardware drops it.  That keeps the loop free of branches around memory instructions, so the compiler can
+    // count exactly how many of them may stay in flight at each wait (with branches it waits for all of them, the
+    // store issued a moment ago included, and the prefetch distance collapses).
     const uint32_t lt = threadIdx.x - 64;                    // 0..959
     const uint32_t r = lt >> 5, cv = lt & 31;                // row in the group (0..29), vector in the tile
     const uint32_t ccol = cv * 8;                            // column of this thread's vector inside a tile
+    const uint32_t row_bytes = cols * 2;
+    const uint32_t nbytes = (uint32_t)(rows * row_bytes);    // the launcher keeps this below 2^31
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(x), 0, nbytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(y, 0, nbytes, 0x00020000);
+    constexpr uint32_t OOB = 0x80000000u;                    // >= nbytes, and stays so after adding a column offset
+    constexpr int PF = NSLOT < SP_PF ? NSLOT : SP_PF;        // tiles in flight per thread
+    const uint32_t G = gridDim.x;
 
-    auto load_x = [&](uint64_t g, uint32_t t, v4u& dst) {
+    auto group_off = [&](uint64_t g) -> uint32_t {           // byte offset of (row r of group g, column ccol), or OOB
         const uint64_t row = g * SP_ROWS + r;
-        const uint32_t col = t * SP_TC + ccol;
-        if (g < ngroups && row < rows && col < cols) dst = ld_stream(reinterpret_cast<const v4u*>(x + row * cols + col));
+        return (g < ngroups && row < rows) ? (uint32_t)row * row_bytes + ccol * 2 : OOB;
     };
+    auto slot_off = [&](uint32_t base, int t) -> uint32_t {
+        if (!FULL && (uint32_t)t * SP_TC + ccol >= cols) return OOB;
+        return base + (uint32_t)t * (SP_TC * 2);
+    };
+    auto load_x = [&](uint32_t off) -> v4u { return __builtin_amdgcn_raw_buffer_load_b128(rx, off, 0, 2); };   // 2: non-temporal
 
-    v4u e[NSLOT];                                            // exp values of the group in flight, 8 halves per slot
-    v4u pre0 = {0, 0, 0, 0}, pre1 = {0, 0, 0, 0};
     uint64_t g = blockIdx.x;
-    load_x(g, 0, pre0);
-    load_x(g, 1, pre1);
+    uint32_t cur = group_off(g), nxt = group_off(g + G), prev = OOB;
+    v4u e[NSLOT];                                            // exp values of the group in flight, 8 halves per slot
+    v4u pre[PF];
+#pragma unroll
+    for (int t = 0; t < NSLOT; t++) e[t] = v4u{0, 0, 0, 0};
+#pragma unroll
+    for (int k = 0; k < PF; k++) pre[k] = load_x(slot_off(cur, k));
 
-    bool have_prev = false;
-    uint64_t prev_row = 0;
-    float s_prev = 0.0f, rinv_prev = 0.0f;
-    bool fast_prev = false;
+    float s_prev = 1.0f, rinv_prev = 1.0f;
+    bool fast_prev = true;
     uint32_t gpar = 0;
 
-    auto flush_slot = [&](int t, const v4u& ev) {           // y[prev_row][slot t] = e / sum of the previous group
-        const uint32_t col = t * SP_TC + ccol;
-        if (prev_row < rows && col < cols) {
-            v4u out;
-            if (fast_prev) {
+    auto quotients = [&](const v4u& ev) -> v4u {             // e / sum of the previous group
+        v4u out;
+        if (fast_prev) {
 #pragma unroll
-                for (int w = 0; w < 4; w++) {
-                    const float e0 = (float)bits_h((uint16_t)(ev[w] & 0xffffu)), e1 = (float)bits_h((uint16_t)(ev[w] >> 16));
-                    const float a0 = e0 * rinv_prev, a1 = e1 * rinv_prev;
-                    float q0 = __builtin_fmaf(__builtin_fmaf(-s_prev, a0, e0), rinv_prev, a0);
-                    float q1 = __builtin_fmaf(__builtin_fmaf(-s_prev, a1, e1), rinv_prev, a1);
-                    // keep the f32 quotient and its conversion apart: fused into v_fma_mixlo_f16 the pair rounds
-                    // subnormal f16 results differently from fma-then-convert
-                    asm volatile("" : "+v"(q0), "+v"(q1));
-                    out[w] = (uint32_t)h_bits((half_t)q0) | ((uint32_t)h_bits((half_t)q1) << 16);
-                }
-            } else {
-#pragma unroll
-                for (int w = 0; w < 4; w++) {
-                    const float e0 = (float)bits_h((uint16_t)(ev[w] & 0xffffu)), e1 = (float)bits_h((uint16_t)(ev[w] >> 16));
-                    out[w] = (uint32_t)h_bits((half_t)(e0 / s_prev)) | ((uint32_t)h_bits((half_t)(e1 / s_prev)) << 16);
-                }
+            for (int w = 0; w < 4; w++) {
+                const float e0 = (float)bits_h((uint16_t)(ev[w] & 0xffffu)), e1 = (float)bits_h((uint16_t)(ev[w] >> 16));
+                const float a0 = e0 * rinv_prev, a1 = e1 * rinv_prev;
+                float q0 = __builtin_fmaf(__builtin_fmaf(-s_prev, a0, e0), rinv_prev, a0);
+                float q1 = __builtin_fmaf(__builtin_fmaf(-s_prev, a1, e1), rinv_prev, a1);
+                // keep the f32 quotient and its conversion apart: fused into v_fma_mixlo_f16 the pair rounds
+                // subnormal f16 results differently from fma-then-convert
+                asm volatile("" : "+v"(q0), "+v"(q1));
+                const f32x2 q = {q0, q1};
+                out[w] = __builtin_bit_cast(uint32_t, __builtin_convertvector(q, h16x2));
             }
-            st_stream(reinterpret_cast<v4u*>(y + prev_row * cols + col), out);
+        } else {
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                const float e0 = (float)bits_h((uint16_t)(ev[w] & 0xffffu)), e1 = (float)bits_h((uint16_t)(ev[w] >> 16));
+                out[w] = (uint32_t)h_bits((half_t)(e0 / s_prev)) | ((uint32_t)h_bits((half_t)(e1 / s_prev)) << 16);
+            }
         }
+        return out;
     };
     auto read_prev_sum = [&](uint32_t par) {
         const float s = (float)sums[par][r];
@@ -385,48 +390,35 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
         rinv_prev = fast_prev ? 1.0f / s : 0.0f;
     };
 
-    for (; g < ngroups; g += gridDim.x) {
-        const uint64_t row = g * SP_ROWS + r;
-        const bool rvalid = row < rows;
+    for (; g < ngroups; g += G) {
 #pragma unroll
         for (int t = 0; t < NSLOT; t++) {
-            v4u& pre = (t & 1) ? pre1 : pre0;
-            const uint32_t col = t * SP_TC + ccol;
-            // exp of the vector that arrived, parked in the LDS tile for the walk (zeros past the row end: adding +0 is a no-op)
-            v4u enew = {0, 0, 0, 0};
-            if (rvalid && col < cols) {
+            v4u& in = pre[t % PF];
+            // exp of the vector that arrived, parked in the LDS tile for the walk (zeros past the row end: adding +0 is a no-op;
+            // rows past the tensor's end read zeros and their sums are never used)
+            v4u enew;
 #pragma unroll
-                for (int w = 0; w < 4; w++) enew[w] = sp_exp_pair(lut, pre[w]);
-                const uint32_t nans = sp_nan_bits(pre[0]) | sp_nan_bits(pre[1]) | sp_nan_bits(pre[2]) | sp_nan_bits(pre[3]);
-                if (nans) {                                  // exp(NaN) = NaN; rare, so patched out of line
-#pragma unroll
-                    for (int w = 0; w < 4; w++) {
-                        const uint32_t nb = sp_nan_bits(pre[w]);
-                        if (nb & 0x8000u) enew[w] = (enew[w] & 0xffff0000u) | 0x7e00u;
-                        if (nb & 0x80000000u) enew[w] = (enew[w] & 0x0000ffffu) | 0x7e000000u;
-                    }
-                }
-            }
+            for (int w = 0; w < 4; w++) enew[w] = sp_exp_pair(lut, in[w]);
+            if (!FULL && (uint32_t)t * SP_TC + ccol >= cols) enew = v4u{0, 0, 0, 0};
             *reinterpret_cast<v4u*>(&tile[t & 1][r][ccol]) = enew;
-            // next load for this register: two tiles ahead, possibly in the block's next group
-            if (t + 2 < NSLOT) load_x(g, t + 2, pre);
-            else load_x(g + gridDim.x, t + 2 - NSLOT, pre);
+            // next load for this register: PF tiles ahead, possibly in the block's next group
+            in = (t + PF < NSLOT) ? load_x(slot_off(cur, t + PF)) : load_x(slot_off(nxt, t + PF - NSLOT));
             __syncthreads();
-            if (t == 0 && have_prev) read_prev_sum(gpar ^ 1);     // published by wave 0 before it reached this barrier
-            if (have_prev) flush_slot(t, e[t]);
+            if (t == 0) read_prev_sum(gpar ^ 1);              // published by wave 0 before it reached this barrier
+            const v4u out = quotients(e[t]);                  // first group: prev is OOB, the store is dropped
+            __builtin_amdgcn_raw_buffer_store_b128(out, ry, slot_off(prev, t), 0, 2);
             e[t] = enew;
         }
-        have_prev = true;
-        prev_row = row;
+        prev = cur;
+        cur = nxt;
+        nxt = group_off(g + 2 * (uint64_t)G);
         gpar ^= 1;
     }
     // drain: outputs of the block's last group
     __syncthreads();
-    if (have_prev) {
-        read_prev_sum(gpar ^ 1);
+    read_prev_sum(gpar ^ 1);
 #pragma unroll
-        for (int t = 0; t < NSLOT; t++) flush_slot(t, e[t]);
-    }
+    for (int t = 0; t < NSLOT; t++) __builtin_amdgcn_raw_buffer_store_b128(quotients(e[t]), ry, slot_off(prev, t), 0, 2);
 }
 
 // ------------------------------------------------------------------------------------------------------------------
@@ -613,26 +605,41 @@ int launch_f16_stream(rt_device* dev, const void* x, void* y, uint64_t rows, uin
     const uint16_t* table = nullptr;
     int rc = rt_unary_table(dev, 0, RT_EXP, &table);
     if (rc) return rc;
-    uint64_t blocks = (rows + SP_ROWS - 1) / SP_ROWS;
-    if (blocks > (uint64_t)dev->num_cus) blocks = dev->num_cus;      // one resident block per CU
     const uint32_t nt = (cols + SP_TC - 1) / SP_TC;
-#define RT_SP(NS)                                                                                                                   \
-    do {                                                                                                                            \
-        static bool attr_done = false;                                                                                              \
-        if (!attr_done) {                                                                                                           \
-            RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(softmax_f16_stream_kernel<NS>),                                \
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)SP_SMEM_BYTES));                            \
-            attr_done = true;                                                                                                       \
-        }                                                                                                                           \
-        hipLaunchKernelGGL((softmax_f16_stream_kernel<NS>), dim3((unsigned)blocks), dim3(SP_BLOCK), SP_SMEM_BYTES, dev->stream, table, \
-                           (const half_t*)x, (half_t*)y, rows, cols);                                                              \
+    const bool full = cols % SP_TC == 0 && (nt == 2 || nt == 4 || nt == 8 || nt == 16);
+    // the kernel addresses the tensor with 32-bit byte offsets below 2^31: larger tensors go in row chunks
+    const uint64_t max_rows = (0x7fffffffull / ((uint64_t)cols * 2)) / SP_ROWS * SP_ROWS;
+#define RT_SP(NS, F)                                                                                                                 \
+    do {                                                                                                                             \
+        static bool attr_done = false;                                                                                               \
+        if (!attr_done) {                                                                                                            \
+            RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(softmax_f16_stream_kernel<NS, F>),                              \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)SP_SMEM_BYTES));                             \
+            attr_done = true;                                                                                                        \
+        }                                                                                                                            \
+        hipLaunchKernelGGL((softmax_f16_stream_kernel<NS, F>), dim3((unsigned)blocks), dim3(SP_BLOCK), SP_SMEM_BYTES, dev->stream,   \
+                           table, xc, yc, n, cols);                                                                                  \
     } while (0)
-    if (nt <= 2) RT_SP(2);
-    else if (nt <= 4) RT_SP(4);
-    else if (nt <= 8) RT_SP(8);
-    else RT_SP(16);
+    for (uint64_t row0 = 0; row0 < rows; row0 += max_rows) {
+        const uint64_t n = rows - row0 < max_rows ? rows - row0 : max_rows;
+        const half_t* xc = (const half_t*)x + row0 * cols;
+        half_t* yc = (half_t*)y + row0 * cols;
+        uint64_t blocks = (n + SP_ROWS - 1) / SP_ROWS;
+        if (blocks > (uint64_t)dev->num_cus) blocks = dev->num_cus;      // one resident block per CU
+        if (full) {
+            if (nt == 2) RT_SP(2, true);
+            else if (nt == 4) RT_SP(4, true);
+            else if (nt == 8) RT_SP(8, true);
+            else RT_SP(16, true);
+        } else {
+            if (nt <= 2) RT_SP(2, false);
+            else if (nt <= 4) RT_SP(4, false);
+            else if (nt <= 8) RT_SP(8, false);
+            else RT_SP(16, false);
+        }
+        RT_CHECK_LAUNCH("softmax_f16_stream_kernel");
+    }
 #undef RT_SP
-    RT_CHECK_LAUNCH("softmax_f16_stream_kernel");
     return RT_OK;
 }
 
