@@ -92,6 +92,24 @@ def test_softmax_f16_streaming_kernel(dev, oracle, shape):
     assert same_bits(dx.to_numpy(), want)
 
 
+def test_softmax_f16_streaming_kernel_beyond_2_gib(dev, oracle):
+    # the kernel addresses a launch with 32-bit byte offsets below 2^31, so a larger tensor is split into row chunks
+    # (262 140 rows of 4096 f16 each); rows on both sides of the split and at the end are compared with the oracle
+    rows, n = 262140 + 47, 4096
+    rng = np.random.default_rng(304)
+    block = randn(rng, (1021, n), np.float16, 2.0)
+    block[::3, 1000:] = -np.inf
+    x = np.tile(block, (rows // 1021 + 1, 1))[:rows]
+    got = dev.softmax(dev.upload(x)).to_numpy()
+    for lo, hi in ((0, 64), (262100, rows)):
+        want = oracle.softmax(x[lo:hi])
+        assert mismatch_count(got[lo:hi], want) == 0, (lo, hi)
+    # every row equals the result of its source row in the repeated block
+    want_block = oracle.softmax(block)
+    reps = rows // 1021
+    assert same_bits(got[: reps * 1021].reshape(reps, 1021, n), np.broadcast_to(want_block, (reps, 1021, n)))
+
+
 def test_softmax_f16_order_dependence_is_reproduced(dev, oracle):
     # 2048 + 1 + 1 + ... never grows in f16: the kernel must reproduce that, not the mathematically exact sum
     row = np.zeros(512, np.float16)
