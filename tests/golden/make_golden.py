@@ -68,6 +68,43 @@ def main():
     out["broadcast_x"] = bsrc
     out["broadcast_y"] = orc.broadcast(bsrc, (2, 3, 4, 5))
     out["concat_y"] = orc.concat([r, r[:, :, :2] * -1, r[:, :, 1:2] + 0.5], 2)
+    # ---- KV-cache append, index ops, RoPE (appended after the vectors above so that those keep their values)
+    kv = rng.standard_normal((1, 2, 6, 16)).astype(np.float32)
+    kv[:, :, 2:] = 0
+    src = rng.standard_normal((1, 2, 1, 16)).astype(np.float32)
+    out["cache_in"], out["cache_src"] = kv.copy(), src
+    out["cache_dst"] = orc.cache(kv, src, 2, 2)                 # the reference test's layout (ops/cache.rs:162-217)
+    out["cache_after"] = kv
+    table = rng.standard_normal((50, 12)).astype(np.float16)
+    ids = np.array([7, 0, 49, 7, 23], np.int32)
+    out["select_table"], out["select_ids"] = table, ids
+    out["select_rows"] = orc.index_select(table, ids, 0)
+    out["select_cols"] = orc.index_select(table, np.array([11, 0, 5], np.int32), 1)
+    iw = np.array([1, 2, 3, 4, 5, 6], np.float32).reshape(3, 2)
+    out["index_write_y"] = orc.index_write(iw, np.array([[7, 8]], np.float32), [2, 0])    # ops/index_write.rs:203-224
+    q = rng.standard_normal((1, 2, 5, 24)).astype(np.float32)
+    out["rope_x"] = q
+    out["rope_dim16_off3"] = orc.rope(q, 16, 10000.0, 3)
+    out["rope_dim24_off0"] = orc.rope(q, 24, 10000.0, 0)
+    # ---- the models' full() -> op -> cast(dt) sequences on f16 tensors, as the oracle's op sequence gives them
+    h = np.concatenate([edge_values(np.float16), (rng.standard_normal(33) * 3).astype(np.float16)])
+    out["via32_x"] = h
+    for op in ("gelu", "silu", "exp", "tanh", "sigmoid"):
+        out[f"via32_{op}"] = orc.cast(orc.unary(op, orc.cast(h, np.float32)), np.float16)
+    nx16 = rng.standard_normal((4, 64)).astype(np.float16)
+    w32, b32 = (1 + 0.02 * rng.standard_normal(64)).astype(np.float32), (0.02 * rng.standard_normal(64)).astype(np.float32)
+    out["via32_norm_x"], out["via32_norm_w"], out["via32_norm_b"] = nx16, w32, b32
+    out["via32_layer_norm"] = orc.cast(orc.layer_norm(orc.cast(nx16, np.float32), w32, b32, 1e-5, intended=True), np.float16)
+    out["via32_rms_norm"] = orc.cast(orc.rms_norm(orc.cast(nx16, np.float32), w32, 1e-5, intended=True), np.float16)
+    sc = (rng.standard_normal((1, 2, 8, 16)) * 2).astype(np.float16)
+    mask = np.triu(np.full((8, 16), -np.inf, np.float16), k=9)
+    out["via32_scores"], out["via32_mask"] = sc, mask
+    masked = orc.binary("add", sc, np.ascontiguousarray(np.broadcast_to(mask, sc.shape)))
+    out["via32_softmax"] = orc.cast(orc.softmax(orc.cast(masked, np.float32)), np.float16)
+    proj = rng.standard_normal((3, 32)).astype(np.float16)
+    out["via32_proj"] = proj
+    act = orc.cast(orc.unary("silu", orc.cast(np.ascontiguousarray(proj[:, :16]), np.float32)), np.float16)
+    out["via32_gated"] = orc.binary("mul", np.ascontiguousarray(proj[:, 16:]), act)
     path = os.path.join(HERE, "vectors.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path), "bytes,", len(out), "arrays")

@@ -36,6 +36,17 @@ def test_oracle_reproduces_the_recorded_vectors(oracle):
     assert np.array_equal(GOLD["permute_0213"], r.transpose(0, 2, 1, 3))
     assert np.array_equal(oracle.slice_(r, [(1, 2), (0, 3), (1, 3), (2, 5)]), GOLD["slice_mid"])
     assert np.array_equal(GOLD["broadcast_y"], np.broadcast_to(GOLD["broadcast_x"], (2, 3, 4, 5)))
+    kv = GOLD["cache_in"].copy()
+    assert np.array_equal(oracle.cache(kv, GOLD["cache_src"], 2, 2), GOLD["cache_dst"]) and np.array_equal(kv, GOLD["cache_after"])
+    assert np.array_equal(GOLD["cache_dst"], np.concatenate([GOLD["cache_in"][:, :, :2], GOLD["cache_src"]], axis=2))
+    assert np.array_equal(oracle.index_select(GOLD["select_table"], GOLD["select_ids"], 0), GOLD["select_rows"])
+    assert np.array_equal(GOLD["select_rows"], GOLD["select_table"][GOLD["select_ids"]])
+    assert np.array_equal(GOLD["index_write_y"], np.array([[1, 2], [3, 4], [7, 8]], np.float32))
+    assert same(oracle.rope(GOLD["rope_x"], 16, 10000.0, 3), GOLD["rope_dim16_off3"])
+    assert same(oracle.rope(GOLD["rope_x"], 24, 10000.0, 0), GOLD["rope_dim24_off0"])
+    h32 = oracle.cast(GOLD["via32_x"], np.float32)
+    for op in ("gelu", "silu", "exp", "tanh", "sigmoid"):
+        assert same(oracle.cast(oracle.unary(op, h32), np.float16), GOLD[f"via32_{op}"]), op
 
 
 @pytest.mark.gpu
@@ -83,5 +94,31 @@ def test_kernels_reproduce_the_recorded_vectors(oracle):
         rr = GOLD["reindex_x"]
         parts = [rr, np.ascontiguousarray(rr[:, :, :2] * -1), np.ascontiguousarray(rr[:, :, 1:2] + 0.5)]
         assert np.array_equal(dev.concat([dev.upload(p) for p in parts], 2).to_numpy(), GOLD["concat_y"])
+        kv = dev.upload(GOLD["cache_in"])
+        assert np.array_equal(dev.cache(kv, dev.upload(GOLD["cache_src"]), 2, 2).to_numpy(), GOLD["cache_dst"])
+        assert np.array_equal(kv.to_numpy(), GOLD["cache_after"])
+        t = dev.upload(GOLD["select_table"])
+        assert np.array_equal(dev.index_select(t, dev.upload(GOLD["select_ids"]), 0).to_numpy(), GOLD["select_rows"])
+        assert np.array_equal(dev.index_select(t, dev.upload(np.array([11, 0, 5], np.int32)), 1).to_numpy(), GOLD["select_cols"])
+        iw = dev.upload(np.array([1, 2, 3, 4, 5, 6], np.float32).reshape(3, 2))
+        assert np.array_equal(dev.index_write(iw, dev.upload(np.array([[7, 8]], np.float32)), [2, 0]).to_numpy(), GOLD["index_write_y"])
+        q = dev.upload(GOLD["rope_x"])
+        for dim, off, key in ((16, 3, "rope_dim16_off3"), (24, 0, "rope_dim24_off0")):
+            bad, mx = oracle.count_not_close(dev.rope(q, dim, 10000.0, off).to_numpy(), GOLD[key], 1e-6, 1e-6)
+            assert bad == 0, (key, mx)
+        h = dev.upload(GOLD["via32_x"])
+        for op in ("gelu", "silu", "exp", "tanh", "sigmoid"):
+            assert same(dev.unary_via_f32(op, h).to_numpy(), GOLD[f"via32_{op}"]), op
+        nx, w, b = dev.upload(GOLD["via32_norm_x"]), dev.upload(GOLD["via32_norm_w"]), dev.upload(GOLD["via32_norm_b"])
+        for got, key in ((dev.norm_via_f32("layer", nx, w, b, 1e-5), "via32_layer_norm"), (dev.norm_via_f32("rms", nx, w, None, 1e-5), "via32_rms_norm")):
+            bad, mx = oracle.count_not_close(got.to_numpy(), GOLD[key], 1e-3, 1e-3)
+            assert bad == 0, (key, mx)
+        got = dev.softmax_via_f32(dev.upload(GOLD["via32_scores"]), dev.upload(GOLD["via32_mask"])).to_numpy()
+        bad, mx = oracle.count_not_close(got, GOLD["via32_softmax"], 1e-3, 1e-3)
+        assert bad == 0, mx
+        from ratchet_amd.runtime import BufferView
+        proj = dev.upload(GOLD["via32_proj"])
+        got = dev.gated_mul_via_f32("silu", BufferView(proj, 0, (80,)), BufferView(proj, 16, (80,)), 3, 16, gate_row_stride=32, up_row_stride=32)
+        assert same(got.to_numpy(), GOLD["via32_gated"])
     finally:
         dev.close()

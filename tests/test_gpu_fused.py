@@ -172,3 +172,47 @@ def test_fused_entry_points_reject_bad_arguments(dev):
     with pytest.raises(RatchetError) as e:
         dev.softmax_via_f32(h, dev.upload(np.zeros((2, 3, 4, 5), np.float16)))
     assert e.value.status == 4
+
+
+def test_bf16_patterns(dev, oracle):
+    """The same four entry points on bf16 (carried as uint16 bit patterns on the host)."""
+    rng = np.random.default_rng(505)
+
+    def bf(a):
+        return oracle.cast(np.ascontiguousarray(a, dtype=np.float32), np.uint16, dst_bf16=True)
+
+    def wide(u):
+        return oracle.cast(u, np.float32, src_bf16=True)
+
+    def close_bf16(got, want, tol):
+        bad, mx = oracle.count_not_close(got, want, tol, tol, bf16=True)
+        return bad == 0, (bad, mx)
+
+    # norms: f32 arithmetic, one rounding to bf16 (8 significand bits: the bar is the reference's 16-bit one, relative 1e-2 here)
+    x = bf(rng.standard_normal((33, 1024)) * 2 + 0.25)
+    w, b = rng.standard_normal(1024).astype(np.float32), rng.standard_normal(1024).astype(np.float32)
+    want = bf(oracle.layer_norm(wide(x), w, b, 1e-5, intended=True))
+    got = dev.norm_via_f32("layer", dev.upload(x, bf16=True), dev.upload(w), dev.upload(b), 1e-5).to_numpy()
+    ok, info = close_bf16(got, want, 1e-2)
+    assert ok, info
+    assert (got != want).mean() < 0.01
+    want = bf(oracle.rms_norm(wide(x), w, 1e-5, intended=True))
+    got = dev.norm_via_f32("rms", dev.upload(x, bf16=True), dev.upload(w), None, 1e-5).to_numpy()
+    assert (got != want).mean() < 0.01
+    # masked softmax
+    s = bf(rng.standard_normal((1, 3, 40, 256)) * 2)
+    mask = bf(np.triu(np.full((40, 256), -np.inf, np.float32), k=217))
+    masked = oracle.binary("add", s, np.ascontiguousarray(np.broadcast_to(mask, s.shape)), bf16=True)
+    want = bf(oracle.softmax(wide(masked)))
+    got = dev.softmax_via_f32(dev.upload(s, bf16=True), dev.upload(mask, bf16=True)).to_numpy()
+    ok, info = close_bf16(got, want, 1e-2)
+    assert ok, info
+    assert (got != want).mean() < 0.01
+    # gated multiply: bit-exact (table path and direct path)
+    for shape in ((600, 4096), (5, 24)):
+        gate, up = bf(rng.standard_normal(shape) * 2), bf(rng.standard_normal(shape))
+        act = bf(oracle.unary("silu", wide(gate)))
+        want = oracle.binary("mul", up, act, bf16=True)
+        got = dev.gated_mul_via_f32("silu", dev.upload(gate, bf16=True), dev.upload(up, bf16=True), shape[0], shape[1]).to_numpy()
+        nan = ((want & 0x7fff) > 0x7f80)
+        assert np.array_equal(got[~nan], want[~nan]), shape
