@@ -67,6 +67,13 @@ const char* rt_status_name(int status);
 int rt_malloc(rt_device* dev, size_t bytes, void** dptr);    /* BufferPool::get_or_create (buffer_pool.rs:68-116): sizes
                                                                 are rounded up to 4 B, minimum 16 B (:82-93) */
 int rt_free(rt_device* dev, void* dptr);                     /* last drop of a PooledGPUBuffer */
+/* rt_malloc / rt_free sit on a per-device pool (the role of gpu/pools/buffer_pool.rs:60-112): a freed block is parked
+ * and handed out again to a later request of about its size; since every kernel and copy of a device runs on its one
+ * in-order stream, neither call synchronises.  rt_pool_trim returns the parked blocks to the driver (it waits for
+ * queued work first); rt_pool_stats reports bytes handed out, bytes parked, and how many requests the pool served
+ * (hits) or passed to hipMalloc (misses); any out pointer may be NULL. */
+int rt_pool_trim(rt_device* dev);
+int rt_pool_stats(rt_device* dev, uint64_t* live_bytes, uint64_t* parked_bytes, uint64_t* hits, uint64_t* misses);
 int rt_memset0(rt_device* dev, void* dptr, size_t bytes);    /* GPUBuffer::zeros (gpu_buffer.rs:29-37) */
 int rt_h2d(rt_device* dev, void* dptr, const void* host, size_t bytes);   /* GPUBuffer::from_bytes (:49-59), blocking */
 int rt_d2h(rt_device* dev, void* host, const void* dptr, size_t bytes);   /* GPUBuffer::to_cpu (:199-218), blocking */

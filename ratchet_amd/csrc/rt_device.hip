@@ -4,8 +4,19 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <map>
+#include <mutex>
+#include <unordered_map>
 
 #include "rt_internal.h"
+
+struct rt_pool {
+    std::mutex mu;
+    std::multimap<size_t, void*> parked;            // block size -> block, free for reuse
+    std::unordered_map<void*, size_t> live;         // blocks handed out by rt_malloc
+    size_t parked_bytes = 0;
+    uint64_t hits = 0, misses = 0;
+};
 
 static thread_local char g_err[512] = "";
 
@@ -93,10 +104,12 @@ int rt_device_create(int ordinal, rt_device** out) {
                        prop.gcnArchName);
     rt_device* dev = new rt_device();
     memset(dev, 0, sizeof(*dev));
+    dev->pool = new rt_pool();
     dev->ordinal = ordinal;
     dev->num_cus = prop.multiProcessorCount;
     hipError_t e = hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking);   // default priority
     if (e != hipSuccess) {
+        delete dev->pool;
         delete dev;
         return rt_fail_hip(e, "hipStreamCreateWithFlags");
     }
@@ -104,6 +117,7 @@ int rt_device_create(int ordinal, rt_device** out) {
     e = hipMalloc((void**)&dev->gn_scratch, dev->gn_scratch_bytes);
     if (e != hipSuccess) {
         (void)hipStreamDestroy(dev->stream);
+        delete dev->pool;
         delete dev;
         return rt_fail_hip(e, "hipMalloc(scratch)");
     }
@@ -122,6 +136,10 @@ int rt_device_destroy(rt_device* dev) {
             if (dev->unary_lut_via32[t][i]) (void)hipFree(dev->unary_lut_via32[t][i]);
         }
     if (dev->gn_scratch) (void)hipFree(dev->gn_scratch);
+    // buffers the caller never returned are released with the device, like the parked ones
+    for (auto& kv : dev->pool->parked) (void)hipFree(kv.second);
+    for (auto& kv : dev->pool->live) (void)hipFree(kv.first);
+    delete dev->pool;
     hipError_t e = hipStreamDestroy(dev->stream);
     delete dev;
     if (e != hipSuccess) return rt_fail_hip(e, "hipStreamDestroy");
@@ -135,15 +153,55 @@ int rt_sync(rt_device* dev) {
     return RT_OK;
 }
 
+// Storage pool.  The reference keeps freed GPU buffers in a pool keyed by size and hands them out again
+// (crates/ratchet-core/src/gpu/pools/buffer_pool.rs:60-112) because creating a buffer per op per step is what costs.
+// Here: rt_free parks the block, rt_malloc takes the smallest parked block that fits without wasting more than a
+// quarter of it.  Every kernel and copy of a device runs on that device's one stream, so a block handed out again is
+// only touched by work queued after the work of its previous owner: no synchronisation is needed on either call.
+// hipMalloc / hipFree (which synchronise the device) happen only on a pool miss, in rt_pool_trim and at destroy.
+static size_t pool_round(size_t bytes) {
+    // the reference rounds sizes up to 4 bytes and never allocates less than 16 (buffer_pool.rs:82-93); blocks are
+    // further rounded so that near-equal requests share a size: 512 B steps up to 1 MiB, 1/16 of the size above
+    size_t sz = (bytes + 3) & ~(size_t)3;
+    if (sz < 16) sz = 16;
+    if (sz <= (1u << 20)) return (sz + 511) & ~(size_t)511;
+    size_t step = 1;
+    while (step * 32 <= sz) step <<= 1;                          // step = 2^floor(log2(sz)) / 16
+    return (sz + step - 1) / step * step;
+}
+
 int rt_malloc(rt_device* dev, size_t bytes, void** dptr) {
     RT_REQUIRE(dptr, RT_ERR_NULL_POINTER, "rt_malloc: dptr is NULL");
     *dptr = nullptr;
     int rc = rt_enter(dev);
     if (rc) return rc;
-    // the reference rounds sizes up to 4 bytes and never allocates less than 16 (buffer_pool.rs:82-93)
-    size_t sz = (bytes + 3) & ~(size_t)3;
-    if (sz < 16) sz = 16;
-    RT_HIP(hipMalloc(dptr, sz));
+    const size_t sz = pool_round(bytes);
+    rt_pool* pool = dev->pool;
+    std::lock_guard<std::mutex> lock(pool->mu);
+    auto it = pool->parked.lower_bound(sz);
+    if (it != pool->parked.end() && it->first <= sz + sz / 4) {
+        *dptr = it->second;
+        pool->live.emplace(it->second, it->first);
+        pool->parked_bytes -= it->first;
+        pool->parked.erase(it);
+        pool->hits++;
+        return RT_OK;
+    }
+    hipError_t e = hipMalloc(dptr, sz);
+    if (e == hipErrorOutOfMemory && !pool->parked.empty()) {   // give the parked blocks back and try once more
+        (void)hipGetLastError();
+        (void)hipStreamSynchronize(dev->stream);
+        for (auto& kv : pool->parked) (void)hipFree(kv.second);
+        pool->parked.clear();
+        pool->parked_bytes = 0;
+        e = hipMalloc(dptr, sz);
+    }
+    if (e != hipSuccess) {
+        *dptr = nullptr;
+        return rt_fail_hip(e, "hipMalloc");
+    }
+    pool->live.emplace(*dptr, sz);
+    pool->misses++;
     return RT_OK;
 }
 
@@ -151,9 +209,43 @@ int rt_free(rt_device* dev, void* dptr) {
     int rc = rt_enter(dev);
     if (rc) return rc;
     if (!dptr) return RT_OK;
-    // work queued on the stream may still use the buffer
-    RT_HIP(hipStreamSynchronize(dev->stream));
-    RT_HIP(hipFree(dptr));
+    rt_pool* pool = dev->pool;
+    std::lock_guard<std::mutex> lock(pool->mu);
+    auto it = pool->live.find(dptr);
+    RT_REQUIRE(it != pool->live.end(), RT_ERR_ARG, "rt_free: %p was not allocated by rt_malloc on this device (or was freed twice)", dptr);
+    pool->parked.emplace(it->second, dptr);
+    pool->parked_bytes += it->second;
+    pool->live.erase(it);
+    return RT_OK;
+}
+
+int rt_pool_trim(rt_device* dev) {
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    RT_HIP(hipStreamSynchronize(dev->stream));                  // queued work may still use a parked block
+    rt_pool* pool = dev->pool;
+    std::lock_guard<std::mutex> lock(pool->mu);
+    hipError_t first = hipSuccess;
+    for (auto& kv : pool->parked) {
+        hipError_t e = hipFree(kv.second);
+        if (e != hipSuccess && first == hipSuccess) first = e;
+    }
+    pool->parked.clear();
+    pool->parked_bytes = 0;
+    if (first != hipSuccess) return rt_fail_hip(first, "hipFree");
+    return RT_OK;
+}
+
+int rt_pool_stats(rt_device* dev, uint64_t* live_bytes, uint64_t* parked_bytes, uint64_t* hits, uint64_t* misses) {
+    RT_REQUIRE(dev, RT_ERR_NULL_DEVICE, "rt_device is NULL");
+    rt_pool* pool = dev->pool;
+    std::lock_guard<std::mutex> lock(pool->mu);
+    uint64_t live = 0;
+    for (auto& kv : pool->live) live += kv.second;
+    if (live_bytes) *live_bytes = live;
+    if (parked_bytes) *parked_bytes = pool->parked_bytes;
+    if (hits) *hits = pool->hits;
+    if (misses) *misses = pool->misses;
     return RT_OK;
 }
 

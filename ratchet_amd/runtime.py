@@ -140,6 +140,15 @@ class Device:
     def sync(self):
         check(self.lib.rt_sync(self.handle))
 
+    def pool_stats(self):
+        """(bytes handed out, bytes parked for reuse, requests served by the pool, requests passed to hipMalloc)"""
+        v = [ctypes.c_uint64() for _ in range(4)]
+        check(self.lib.rt_pool_stats(self.handle, *[ctypes.byref(x) for x in v]))
+        return tuple(int(x.value) for x in v)
+
+    def pool_trim(self):
+        check(self.lib.rt_pool_trim(self.handle))
+
     # ---- storage
     def empty(self, shape, dt):
         return Buffer(self, shape, dt)

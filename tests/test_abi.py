@@ -166,6 +166,11 @@ def test_fused_pattern_validation(lib):
     assert lib.rt_gated_mul_via_f32(None, 12, _lib.F32, SOME, 16, SOME, 16, SOME, 4, 8) == 2
 
 
+def test_pool_validation(lib):
+    assert lib.rt_pool_trim(None) == 8
+    assert lib.rt_pool_stats(None, None, None, None, None) == 8
+
+
 def test_storage_validation(lib):
     p = ctypes.c_void_p()
     assert lib.rt_malloc(None, 16, ctypes.byref(p)) == 8

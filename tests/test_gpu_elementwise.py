@@ -222,3 +222,45 @@ def test_unary_bf16_large_tensor_table_path(dev, oracle):
         got = dev.unary(op, dev.upload(x, bf16=True)).to_numpy()
         wf, gf = oracle.cast(want, np.float32, src_bf16=True), oracle.cast(got, np.float32, src_bf16=True)
         assert np.all((got == want) | (np.isnan(wf) & np.isnan(gf))), op
+
+
+def test_storage_pool_reuses_blocks_in_stream_order(oracle):
+    """rt_free parks a block, the next rt_malloc of about that size gets it back without a device synchronisation
+    (the role of the reference's BufferPool, gpu/pools/buffer_pool.rs:60-112); results stay right because every launch of a
+    device goes through one in-order stream."""
+    from ratchet_amd import Device, RatchetError
+
+    d = Device(0)
+    try:
+        rng = np.random.default_rng(120)
+        x = randn(rng, (1 << 20,), np.float32)
+        dx = d.upload(x)
+        live0, parked0, hits0, misses0 = d.pool_stats()
+        a = d.unary("neg", dx)
+        pa = a.ptr.value
+        del a                                                 # parked while the kernel may still be running
+        b = d.unary("abs", dx)                                # same size: the parked block comes back
+        assert b.ptr.value == pa
+        assert np.array_equal(b.to_numpy(), np.abs(x))
+        live, parked, hits, misses = d.pool_stats()
+        assert hits == hits0 + 1 and misses == misses0 + 1 and live == live0 + 4 * (1 << 20) and parked == parked0
+        # a chain that frees every intermediate immediately: correct values, two blocks cycle
+        y = dx
+        want = x
+        for op in ("neg", "abs", "sqrt", "neg", "exp"):
+            y = d.unary(op, y)
+            want = oracle.unary(op, want)
+        assert same_bits(y.to_numpy(), want)
+        assert d.pool_stats()[3] <= misses + 2
+        small = d.empty((3,), 0)                              # sizes are rounded: 12 bytes -> one 512-byte class
+        ps = small.ptr.value
+        del small
+        assert d.empty((100,), 0).ptr.value == ps
+        del b, y
+        assert d.pool_stats()[1] > 0
+        d.pool_trim()
+        assert d.pool_stats()[1] == 0
+        import ctypes
+        assert d.lib.rt_free(d.handle, ctypes.c_void_p(0x1000)) == 7      # not a block of this pool
+    finally:
+        d.close()
