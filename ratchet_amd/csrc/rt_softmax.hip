@@ -617,11 +617,11 @@ int launch_f16_stream(rt_device* dev, const void* x, void* y, uint64_t rows, uin
     const uint64_t max_rows = (0x7fffffffull / ((uint64_t)cols * 2)) / SP_ROWS * SP_ROWS;
 #define RT_SP(NS, F)                                                                                                                 \
     do {                                                                                                                             \
-        static bool attr_done = false;                                                                                               \
-        if (!attr_done) {                                                                                                            \
+        const unsigned bit = 1u << ((NS == 2 ? 0 : NS == 4 ? 1 : NS == 8 ? 2 : 3) + (F ? 4 : 0));                                   \
+        if (!(dev->sp_attr_set & bit)) {               /* the LDS opt-in is per function and per device */                           \
             RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(softmax_f16_stream_kernel<NS, F>),                              \
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)SP_SMEM_BYTES));                             \
-            attr_done = true;                                                                                                        \
+            dev->sp_attr_set |= bit;                                                                                                 \
         }                                                                                                                            \
         hipLaunchKernelGGL((softmax_f16_stream_kernel<NS, F>), dim3((unsigned)blocks), dim3(SP_BLOCK), SP_SMEM_BYTES, dev->stream,   \
                            table, xc, yc, n, cols);                                                                                  \
