@@ -1,0 +1,130 @@
+"""Properties at the full sizes of the benchmark configurations (too large for the oracle to walk in test time): round
+trips, row sums, repetition over heads, agreement between two independent paths of the library.  Small-size parity against
+the oracle lives in the other test_gpu_* files; here the question is whether indexing, chunking and grid mapping hold up
+at 2^29-element tensors."""
+import numpy as np
+import pytest
+
+from gpu_util import same_bits
+
+pytestmark = pytest.mark.gpu
+
+F32, F16 = 0, 1
+
+
+@pytest.fixture(scope="module")
+def dev():
+    from ratchet_amd import Device
+
+    d = Device(0)
+    yield d
+    d.close()
+
+
+def test_whisper_scores_softmax_rows_sum_to_one_and_permute_round_trip(dev, oracle):
+    rng = np.random.default_rng(701)
+    scores = (3 * rng.standard_normal((1, 6, 1500, 1500))).astype(np.float32)
+    y = dev.softmax(dev.upload(scores)).to_numpy()
+    sums = y.sum(axis=-1, dtype=np.float64)
+    assert np.abs(sums - 1).max() < 1e-5
+    assert (y >= 0).all() and np.array_equal(y.argmax(-1), scores.argmax(-1))
+    bad, mx = oracle.count_not_close(y[0, 3, 700:764], oracle.softmax(scores[0, 3, 700:764]), 1e-5, 1e-5)   # a slab from the middle
+    assert bad == 0, mx
+    q = rng.standard_normal((1, 1500, 6, 64)).astype(np.float32)
+    dq = dev.upload(q)
+    p = dev.permute(dq, (0, 2, 1, 3))
+    assert np.array_equal(p.to_numpy(), q.transpose(0, 2, 1, 3))
+    assert same_bits(dev.permute(p, (0, 2, 1, 3)).to_numpy(), q)
+
+
+def test_phi2_block_identities(dev, oracle):
+    rng = np.random.default_rng(702)
+    x = rng.standard_normal((1, 2048, 2560)).astype(np.float16)
+    a = (0.5 * rng.standard_normal((1, 2048, 2560))).astype(np.float16)
+    dx, da = dev.upload(x), dev.upload(a)
+    r = dev.binary("add", dx, da)
+    assert same_bits(dev.binary("sub", r, da).to_numpy(), oracle.binary("sub", oracle.binary("add", x, a), a))    # whole tensor, exact
+    assert same_bits(dev.cast(dev.cast(dx, F32), F16).to_numpy(), x)                                               # f16 -> f32 -> f16 is the identity
+    g = (1 + 0.02 * rng.standard_normal(2560)).astype(np.float16)
+    b = (0.02 * rng.standard_normal(2560)).astype(np.float16)
+    ln = dev.layer_norm(r, dev.upload(g), dev.upload(b), 1e-5).to_numpy()
+    rr = r.to_numpy()
+    rows = [0, 1, 777, 2047]
+    want = oracle.layer_norm(rr[0, rows], g, b, 1e-5, intended=True)
+    assert same_bits(ln[0, rows], want)
+    h = rng.standard_normal((1, 2048, 10240)).astype(np.float16)
+    ge = dev.unary("gelu", dev.upload(h)).to_numpy()
+    table = oracle.unary("gelu", np.arange(65536, dtype=np.uint16).view(np.float16))                               # every f16 input, once
+    assert same_bits(ge, table[h.view(np.uint16)])
+
+
+def test_phi3_attention_tail_at_full_size(dev, oracle):
+    S, H = 4096, 32
+    rng = np.random.default_rng(703)
+    head = (2 * rng.standard_normal((S, S))).astype(np.float16)
+    mask = np.triu(np.full((S, S), -np.inf, np.float16), k=1)
+    scores = dev.empty((1, H, S, S), F16)
+    dh = dev.upload(head)
+    from ratchet_amd import _lib
+    for h in range(H):
+        _lib.check(dev.lib.rt_d2d(dev.handle, scores.ptr.value + h * head.nbytes, dh.ptr, head.nbytes))
+    masked = dev.binary("add", scores, dev.upload(mask))
+    soft = dev.softmax(masked)
+    out = soft.to_numpy()
+    # every head holds the same data, so every head must hold the same result, bit for bit (catches any grid / chunk mapping slip)
+    assert all(same_bits(out[0, h], out[0, 0]) for h in range(1, H))
+    rows = list(range(0, 64)) + list(range(2016, 2080)) + list(range(4032, 4096))
+    want = oracle.softmax(oracle.binary("add", head[rows], mask[rows]))
+    assert same_bits(out[0, 0, rows], want)
+    assert not out[0, 0][np.triu_indices(S, k=1)].any()                            # masked positions are exactly zero
+    # no "rows sum to one" here: the reference accumulates the 4096 exp terms in f16, terms below half an ulp of the running
+    # sum vanish, and long rows come out up to ~10 % heavy; the oracle rows above pin exactly that behaviour
+    # the one-pass path (f32 inside) agrees with the f16 path within the 16-bit bar, and is again identical across heads
+    fused = dev.softmax_via_f32(scores, dev.upload(mask)).to_numpy()
+    assert all(same_bits(fused[0, h], fused[0, 0]) for h in (1, 13, 31))
+    want = oracle.cast(oracle.softmax(oracle.cast(oracle.binary("add", head[rows], mask[rows]), np.float32)), np.float16)
+    bad, mx = oracle.count_not_close(fused[0, 0, rows], want, 1e-3, 1e-3)
+    assert bad == 0, mx
+    assert np.abs(fused[0, 0].astype(np.float64).sum(-1) - 1).max() < 1e-3         # f32 sums inside: these rows do sum to one
+
+
+def test_phi3_mlp_and_norm_at_full_size(dev, oracle):
+    rng = np.random.default_rng(704)
+    gate = rng.standard_normal((1, 4096, 8192)).astype(np.float16)
+    up = rng.standard_normal((1, 4096, 8192)).astype(np.float16)
+    dg, du = dev.upload(gate), dev.upload(up)
+    table = oracle.unary("silu", np.arange(65536, dtype=np.uint16).view(np.float16))
+    act = dev.unary("silu", dg)
+    assert same_bits(act.to_numpy(), table[gate.view(np.uint16)])
+    got = dev.binary("mul", du, act).to_numpy()
+    assert same_bits(got[0, 1000:1016], oracle.binary("mul", up[0, 1000:1016], table[gate[0, 1000:1016].view(np.uint16)]))
+    x = rng.standard_normal((1, 4096, 3072)).astype(np.float16)
+    g = (1 + 0.02 * rng.standard_normal(3072)).astype(np.float16)
+    rn = dev.rms_norm(dev.upload(x), dev.upload(g), 1e-5).to_numpy()
+    rows = [0, 5, 2048, 4095]
+    assert same_bits(rn[0, rows], oracle.rms_norm(x[0, rows], g, 1e-5, intended=True))
+
+
+def test_reindex_stress_round_trips(dev, oracle):
+    rng = np.random.default_rng(705)
+    ka = rng.standard_normal((1, 32, 1984, 80)).astype(np.float16)
+    kb = rng.standard_normal((1, 32, 64, 80)).astype(np.float16)
+    cat = dev.concat([dev.upload(ka), dev.upload(kb)], 2)
+    assert same_bits(dev.slice(cat, [(0, 1), (0, 32), (0, 1984), (0, 80)]).to_numpy(), ka)       # concat then slice gives the parts back
+    assert same_bits(dev.slice(cat, [(0, 1), (0, 32), (1984, 2048), (0, 80)]).to_numpy(), kb)
+    cache = dev.upload(np.concatenate([ka, np.zeros_like(kb)], axis=2))
+    assert same_bits(dev.cache(cache, dev.upload(kb), 2, 1984).to_numpy(), cat.to_numpy())          # the KV append builds the same tensor
+    a = rng.standard_normal((1, 32, 2048, 1)).astype(np.float16)
+    b = rng.standard_normal((1, 1, 1, 2048)).astype(np.float16)
+    m = dev.binary("mul", dev.upload(a), dev.upload(b)).to_numpy()
+    assert same_bits(m, a * b)                                                                    # numpy's f16 product is correctly rounded too
+    p = rng.standard_normal((1, 2048, 32, 80)).astype(np.float16)
+    dp = dev.upload(p)
+    t = dev.permute(dp, (0, 2, 1, 3))
+    assert np.array_equal(t.to_numpy(), p.transpose(0, 2, 1, 3))
+    assert same_bits(dev.permute(t, (0, 2, 1, 3)).to_numpy(), p)
+    gx = rng.standard_normal((1, 512, 3000)).astype(np.float16)
+    gw, gb = rng.standard_normal(512).astype(np.float16), rng.standard_normal(512).astype(np.float16)
+    gn = dev.group_norm(dev.upload(gx), 32, dev.upload(gw), dev.upload(gb), 1e-5).to_numpy()
+    bad, mx = oracle.count_not_close(gn, oracle.group_norm(gx, 32, gw, gb, 1e-5), 1e-3, 1e-3)
+    assert bad == 0, mx
