@@ -38,7 +38,8 @@ enum rt_status {
     RT_ERR_SIZE = 6,           /* element count overflows what the kernels index (2^40 elements) */
     RT_ERR_ARG = 7,            /* other bad argument (n_inputs, dim, groups, mode, elem_bytes, eps) */
     RT_ERR_NULL_DEVICE = 8,    /* rt_device* is NULL */
-    RT_ERR_ALIGN = 9           /* pointer not aligned to its element size */
+    RT_ERR_ALIGN = 9,          /* pointer not aligned to its element size */
+    RT_ERR_CAPTURE = 10        /* the call cannot run while the device is capturing a graph (or capture state is wrong) */
 };
 
 enum rt_dtype { RT_F32 = 0, RT_F16 = 1, RT_BF16 = 2, RT_I32 = 3, RT_U32 = 4 };
@@ -166,6 +167,21 @@ int rt_rms_norm(rt_device* dev, int dt, const void* x, const void* scale, void* 
  * the reference's own CPU implementation is a no-op (cpu/norm.rs:215-219). */
 int rt_group_norm(rt_device* dev, int dt, const void* x, const void* scale, const void* bias, void* y, uint32_t B,
                   uint32_t C, uint32_t L, uint32_t groups, float eps);
+
+/* ---- Replayable launch lists ---------------------------------------------------------------------------------------
+ * The reference encodes every compiled op of a graph into one command buffer and submits it once
+ * (Executable::dispatch, executable.rs:33-59).  The counterpart here is a HIP graph: between rt_capture_begin and
+ * rt_capture_end every launch the rt_* ops would enqueue on the device's stream is recorded instead of run;
+ * rt_graph_launch replays the whole list with one submission, in stream order with everything else on the device.
+ * While capturing, calls that wait for the device or go to the driver for memory return RT_ERR_CAPTURE: rt_sync,
+ * rt_h2d, rt_d2h, rt_pool_trim, event calls, an rt_malloc the pool cannot serve, and the first use of an op that builds
+ * a lookup table or grows scratch (run the sequence once eagerly first).  A graph holds raw pointers: every buffer it
+ * touches must stay allocated while the graph is in use. */
+typedef struct rt_graph rt_graph;
+int rt_capture_begin(rt_device* dev);
+int rt_capture_end(rt_device* dev, rt_graph** out);
+int rt_graph_launch(rt_device* dev, rt_graph* graph);
+int rt_graph_destroy(rt_graph* graph);
 
 /* ---- Caller patterns in one pass --------------------------------------------------------------------------------
  * The models wrap every 16-bit norm, softmax and activation in full() ... cast(dt): widen to f32, run the f32 op,

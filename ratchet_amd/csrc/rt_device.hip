@@ -10,6 +10,12 @@
 
 #include "rt_internal.h"
 
+struct rt_graph {
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+    int ordinal;
+};
+
 struct rt_pool {
     std::mutex mu;
     std::multimap<size_t, void*> parked;            // block size -> block, free for reuse
@@ -73,6 +79,7 @@ const char* rt_status_name(int status) {
         case RT_ERR_ARG: return "RT_ERR_ARG";
         case RT_ERR_NULL_DEVICE: return "RT_ERR_NULL_DEVICE";
         case RT_ERR_ALIGN: return "RT_ERR_ALIGN";
+        case RT_ERR_CAPTURE: return "RT_ERR_CAPTURE";
         default: return status < 0 ? "HIP_ERROR" : "RT_ERR_UNKNOWN";
     }
 }
@@ -128,6 +135,7 @@ int rt_device_create(int ordinal, rt_device** out) {
 int rt_device_destroy(rt_device* dev) {
     int rc = rt_enter(dev);
     if (rc) return rc;
+    RT_NO_CAPTURE(dev, "rt_device_destroy");
     (void)hipStreamSynchronize(dev->stream);
     for (int t = 0; t < 2; t++)
         for (int i = 0; i < RT_UNARY_COUNT; i++)
@@ -149,6 +157,7 @@ int rt_device_destroy(rt_device* dev) {
 int rt_sync(rt_device* dev) {
     int rc = rt_enter(dev);
     if (rc) return rc;
+    RT_NO_CAPTURE(dev, "rt_sync");
     RT_HIP(hipStreamSynchronize(dev->stream));
     return RT_OK;
 }
@@ -187,6 +196,7 @@ int rt_malloc(rt_device* dev, size_t bytes, void** dptr) {
         pool->hits++;
         return RT_OK;
     }
+    RT_NO_CAPTURE(dev, "rt_malloc of a size the pool holds no block for");
     hipError_t e = hipMalloc(dptr, sz);
     if (e == hipErrorOutOfMemory && !pool->parked.empty()) {   // give the parked blocks back and try once more
         (void)hipGetLastError();
@@ -222,6 +232,7 @@ int rt_free(rt_device* dev, void* dptr) {
 int rt_pool_trim(rt_device* dev) {
     int rc = rt_enter(dev);
     if (rc) return rc;
+    RT_NO_CAPTURE(dev, "rt_pool_trim");
     RT_HIP(hipStreamSynchronize(dev->stream));                  // queued work may still use a parked block
     rt_pool* pool = dev->pool;
     std::lock_guard<std::mutex> lock(pool->mu);
@@ -272,6 +283,7 @@ int rt_h2d(rt_device* dev, void* dptr, const void* host, size_t bytes) {
     int rc = rt_enter(dev);
     if (rc) return rc;
     if (bytes == 0) return RT_OK;
+    RT_NO_CAPTURE(dev, "rt_h2d");
     RT_HIP(hipMemcpyAsync(dptr, host, bytes, hipMemcpyHostToDevice, dev->stream));
     RT_HIP(hipStreamSynchronize(dev->stream));
     return RT_OK;
@@ -282,6 +294,7 @@ int rt_d2h(rt_device* dev, void* host, const void* dptr, size_t bytes) {
     int rc = rt_enter(dev);
     if (rc) return rc;
     if (bytes == 0) return RT_OK;
+    RT_NO_CAPTURE(dev, "rt_d2h");
     RT_HIP(hipMemcpyAsync(host, dptr, bytes, hipMemcpyDeviceToHost, dev->stream));
     RT_HIP(hipStreamSynchronize(dev->stream));
     return RT_OK;
@@ -293,6 +306,61 @@ int rt_d2d(rt_device* dev, void* dst, const void* src, size_t bytes) {
     if (rc) return rc;
     if (bytes == 0) return RT_OK;
     RT_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, dev->stream));
+    return RT_OK;
+}
+
+int rt_capture_begin(rt_device* dev) {
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    RT_REQUIRE(!dev->capturing, RT_ERR_CAPTURE, "rt_capture_begin: the device is already capturing");
+    // thread-local mode: only this thread's calls on this stream are checked, other threads and devices carry on
+    RT_HIP(hipStreamBeginCapture(dev->stream, hipStreamCaptureModeThreadLocal));
+    dev->capturing = 1;
+    return RT_OK;
+}
+
+int rt_capture_end(rt_device* dev, rt_graph** out) {
+    RT_REQUIRE(out, RT_ERR_NULL_POINTER, "rt_capture_end: out is NULL");
+    *out = nullptr;
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    RT_REQUIRE(dev->capturing, RT_ERR_CAPTURE, "rt_capture_end: the device is not capturing");
+    dev->capturing = 0;
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(dev->stream, &graph);
+    if (e != hipSuccess || !graph) return e != hipSuccess ? rt_fail_hip(e, "hipStreamEndCapture") : rt_fail(RT_ERR_CAPTURE, "rt_capture_end: empty capture");
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(graph);
+        return rt_fail_hip(e, "hipGraphInstantiate");
+    }
+    rt_graph* g = new rt_graph();
+    g->graph = graph;
+    g->exec = exec;
+    g->ordinal = dev->ordinal;
+    *out = g;
+    return RT_OK;
+}
+
+int rt_graph_launch(rt_device* dev, rt_graph* graph) {
+    RT_REQUIRE(graph, RT_ERR_NULL_POINTER, "rt_graph_launch: graph is NULL");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    RT_NO_CAPTURE(dev, "rt_graph_launch");
+    RT_REQUIRE(graph->ordinal == dev->ordinal, RT_ERR_ARG, "rt_graph_launch: the graph was captured on device %d", graph->ordinal);
+    RT_HIP(hipGraphLaunch(graph->exec, dev->stream));
+    return RT_OK;
+}
+
+int rt_graph_destroy(rt_graph* graph) {
+    if (!graph) return RT_OK;
+    (void)hipSetDevice(graph->ordinal);
+    hipError_t e1 = hipGraphExecDestroy(graph->exec);
+    hipError_t e2 = hipGraphDestroy(graph->graph);
+    delete graph;
+    if (e1 != hipSuccess) return rt_fail_hip(e1, "hipGraphExecDestroy");
+    if (e2 != hipSuccess) return rt_fail_hip(e2, "hipGraphDestroy");
     return RT_OK;
 }
 
@@ -325,6 +393,7 @@ int rt_event_record(rt_device* dev, rt_event* ev) {
     RT_REQUIRE(ev, RT_ERR_NULL_POINTER, "rt_event_record: event is NULL");
     int rc = rt_enter(dev);
     if (rc) return rc;
+    RT_NO_CAPTURE(dev, "rt_event_record");
     RT_HIP(hipEventRecord(ev->ev, dev->stream));
     return RT_OK;
 }

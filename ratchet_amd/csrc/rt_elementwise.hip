@@ -439,6 +439,7 @@ inline bool lut_worthwhile(int op) {
 template <typename T, bool VIA32 = false> int build_unary_table(rt_device* dev, int ti, int op) {
     uint16_t*& slot = VIA32 ? dev->unary_lut_via32[ti][op] : dev->unary_lut[ti][op];
     if (slot) return RT_OK;
+    RT_NO_CAPTURE(dev, "building a lookup table (first use of this op and type on the device)");
     uint16_t* table = nullptr;
     uint16_t* iota = nullptr;
     RT_HIP(hipMalloc((void**)&table, LUT_BYTES));

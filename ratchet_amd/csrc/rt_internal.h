@@ -24,6 +24,7 @@ struct rt_device {
     unsigned sp_attr_set;   // streaming softmax instantiations whose dynamic-LDS limit has been raised on this device
     // caching allocator behind rt_malloc / rt_free (defined in rt_device.hip)
     struct rt_pool* pool;
+    int capturing;          // between rt_capture_begin and rt_capture_end
 };
 
 struct rt_event {
@@ -44,6 +45,12 @@ int rt_fail_hip(hipError_t e, const char* what);
 #define RT_REQUIRE(cond, status, ...)                          \
     do {                                                       \
         if (!(cond)) return rt_fail((status), __VA_ARGS__);    \
+    } while (0)
+
+// Calls that wait for the device or ask the driver for memory cannot be recorded into a graph.
+#define RT_NO_CAPTURE(dev, who)                                                                                        \
+    do {                                                                                                               \
+        if ((dev)->capturing) return rt_fail(RT_ERR_CAPTURE, "%s cannot run while the device is capturing a graph", who); \
     } while (0)
 
 // Returns rt_fail_hip(...) if the launch that was just enqueued was rejected.

@@ -677,6 +677,7 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
     splits = (glen + chunk - 1) / chunk;
     const size_t need = (size_t)bg * splits * 3 * sizeof(float);
     if (need > dev->gn_scratch_bytes) {
+        RT_NO_CAPTURE(dev, "growing the GroupNorm scratch");
         RT_HIP(hipStreamSynchronize(dev->stream));
         RT_HIP(hipFree(dev->gn_scratch));
         dev->gn_scratch = nullptr;

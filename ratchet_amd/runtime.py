@@ -91,6 +91,47 @@ class BufferView:
         return self
 
 
+class Graph:
+    """A replayable list of launches recorded on a device (a HIP graph); the buffers it touches must outlive it."""
+
+    def __init__(self, device, handle):
+        self.device, self.handle = device, handle
+
+    def launch(self):
+        check(self.device.lib.rt_graph_launch(self.device.handle, self.handle))
+
+    def __del__(self):
+        try:
+            if self.handle is not None and self.device.handle is not None:
+                self.device.lib.rt_graph_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+class _Capture:
+    def __init__(self, device):
+        self.device = device
+        self.graph = None
+
+    def __enter__(self):
+        check(self.device.lib.rt_capture_begin(self.device.handle))
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        p = ctypes.c_void_p()
+        rc = self.device.lib.rt_capture_end(self.device.handle, ctypes.byref(p))
+        if exc_type is None:
+            check(rc)
+            self.graph = Graph(self.device, p)
+        elif rc == 0:
+            self.device.lib.rt_graph_destroy(p)
+        return False
+
+    def launch(self):
+        self.graph.launch()
+
+
 class Event:
     def __init__(self, device):
         self.device = device
@@ -139,6 +180,10 @@ class Device:
 
     def sync(self):
         check(self.lib.rt_sync(self.handle))
+
+    def capture(self):
+        """with dev.capture() as g: <launch ops> ... then g.launch() replays them with one submission."""
+        return _Capture(self)
 
     def pool_stats(self):
         """(bytes handed out, bytes parked for reuse, requests served by the pool, requests passed to hipMalloc)"""

@@ -166,6 +166,16 @@ def test_fused_pattern_validation(lib):
     assert lib.rt_gated_mul_via_f32(None, 12, _lib.F32, SOME, 16, SOME, 16, SOME, 4, 8) == 2
 
 
+def test_graph_validation(lib):
+    assert lib.rt_capture_begin(None) == 8
+    p = ctypes.c_void_p()
+    assert lib.rt_capture_end(None, ctypes.byref(p)) == 8
+    assert lib.rt_capture_end(None, None) == 1
+    assert lib.rt_graph_launch(None, None) == 1
+    assert lib.rt_graph_destroy(None) == 0
+    assert lib.rt_status_name(10) == b"RT_ERR_CAPTURE"
+
+
 def test_pool_validation(lib):
     assert lib.rt_pool_trim(None) == 8
     assert lib.rt_pool_stats(None, None, None, None, None) == 8

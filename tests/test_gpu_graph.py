@@ -1,0 +1,114 @@
+"""Replayable launch lists (HIP graphs) through the C ABI: the counterpart of the reference's encode-all-then-submit-once
+Executable::dispatch (crates/ratchet-core/src/executable.rs:33-59).  Every replay is compared bit for bit with eager execution,
+with eager work and synchronisations between replays."""
+import numpy as np
+import pytest
+
+from gpu_util import randn, same_bits
+
+pytestmark = pytest.mark.gpu
+
+F32, F16 = 0, 1
+
+
+@pytest.fixture()
+def dev():
+    from ratchet_amd import Device
+
+    d = Device(0)
+    yield d
+    d.close()
+
+
+def test_replays_match_eager_execution(dev, oracle):
+    rng = np.random.default_rng(801)
+    x = randn(rng, (1, 1024, 2560), np.float16)
+    bias = randn(rng, (2560,), np.float16, 0.02)
+    g = randn(rng, (2560,), np.float16, 0.02) + np.float16(1)
+    s = randn(rng, (1, 4, 512, 512), np.float16, 2.0)
+    mask = np.triu(np.full((512, 512), -np.inf, np.float16), k=1)
+    gx = randn(rng, (2, 64, 300), np.float16)
+    gw = randn(rng, (64,), np.float16)
+    dx, dbias, dg, ds, dmask, dgx, dgw = (dev.upload(a) for a in (x, bias, g, s, mask, gx, gw))
+    h = dev.empty(x.shape, F16)
+    act = dev.empty(x.shape, F16)
+    ln = dev.empty(x.shape, F16)
+    masked = dev.empty(s.shape, F16)
+    soft = dev.empty(s.shape, F16)
+    fused = dev.empty(s.shape, F16)
+    gn = dev.empty(gx.shape, F16)
+    cat = dev.empty((1, 2048, 2560), F16)
+    scratch = dev.empty((1024,), F32)
+
+    def sequence():
+        scratch.zero_()                                        # a fill kernel, not a memset node
+        dev.binary("add", dx, dbias, out=h)
+        dev.unary("gelu", h, out=act)                          # table path (2.6M elements)
+        dev.layer_norm(act, dg, dbias, 1e-5, out=ln)
+        dev.binary("add", ds, dmask, out=masked)
+        dev.softmax(masked, out=soft)                          # streaming kernel (1M elements)
+        dev.softmax_via_f32(ds, dmask, out=fused)
+        dev.group_norm(dgx, 8, dgw, None, 1e-5, out=gn)
+        dev.concat([ln, act], 1, out=cat)
+
+    outputs = (ln, soft, fused, gn, cat)
+    sequence()                                                 # eager: builds the tables, sizes the scratch, gives the expected values
+    want = [o.to_numpy() for o in outputs]
+    assert same_bits(want[1], oracle.softmax(oracle.binary("add", s, np.ascontiguousarray(np.broadcast_to(mask, s.shape)))))
+    with dev.capture() as cap:
+        sequence()
+    for o in outputs:                                          # capturing must not have run anything
+        o.zero_()
+    assert not soft.to_numpy().any()
+    for replay in range(4):
+        cap.launch()
+        got = [o.to_numpy() for o in outputs]
+        for k, (a, b) in enumerate(zip(got, want)):
+            assert same_bits(a, b), (replay, k)
+        # eager work and a synchronisation between replays, then scribble over the outputs so a replay that did nothing would show
+        dev.unary("neg", dx, out=h)
+        dev.sync()
+        for o in outputs:
+            o.zero_()
+    # a new input value flows through the same graph (pointers are fixed, contents are not)
+    x2 = randn(rng, x.shape, np.float16)
+    from ratchet_amd import _lib
+    import ctypes
+    _lib.check(dev.lib.rt_h2d(dev.handle, dx.ptr, x2.ctypes.data_as(ctypes.c_void_p), x2.nbytes))
+    cap.launch()
+    got_ln = ln.to_numpy()
+    sequence()
+    assert same_bits(got_ln, ln.to_numpy())
+
+
+def test_calls_that_cannot_be_captured_say_so(dev):
+    from ratchet_amd import RatchetError
+
+    x = dev.upload(np.ones((1 << 21,), np.float16))
+    y = dev.empty(x.shape, F16)
+    with pytest.raises(RatchetError) as e:
+        with dev.capture():
+            dev.sync()
+    assert e.value.status == 10
+    with pytest.raises(RatchetError) as e:
+        with dev.capture():
+            x.to_numpy()
+    assert e.value.status == 10
+    with pytest.raises(RatchetError) as e:
+        with dev.capture():
+            dev.unary("tanh", x, out=y)                        # first use: the lookup table would have to be built
+    assert e.value.status == 10
+    with pytest.raises(RatchetError) as e:
+        with dev.capture():
+            dev.empty((123457,), F32)                          # nothing of that size is parked in the pool
+    assert e.value.status == 10
+    # the device is usable again after each failed capture, and a nested begin is refused
+    dev.unary("tanh", x, out=y)
+    assert np.allclose(y.to_numpy()[:4].astype(np.float32), np.tanh(1.0), atol=1e-3)
+    with dev.capture() as cap:
+        dev.unary("tanh", x, out=y)
+        assert dev.lib.rt_capture_begin(dev.handle) == 10
+    y.zero_()
+    cap.launch()
+    assert np.allclose(y.to_numpy()[-4:].astype(np.float32), np.tanh(1.0), atol=1e-3)
+    assert dev.lib.rt_capture_end(dev.handle, None) == 1
