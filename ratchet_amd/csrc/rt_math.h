@@ -194,4 +194,33 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// Reduction over the LANES threads that share a row: one wave64 (LANES == 64) or a whole 256-thread block, whose four
+// wave results meet in LDS and are added in a fixed order.  Every thread of the block must call the block form.
+template <int LANES> __device__ __forceinline__ float row_sum(float v) {
+    v = wave_sum(v);
+    if constexpr (LANES != 64) {
+        __shared__ float red[LANES / 64];
+        __syncthreads();                                   // earlier readers of red are done
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+        __syncthreads();
+        v = red[0];
+#pragma unroll
+        for (int w = 1; w < LANES / 64; w++) v += red[w];
+    }
+    return v;
+}
+template <int LANES> __device__ __forceinline__ float row_max(float v) {
+    v = wave_max(v);
+    if constexpr (LANES != 64) {
+        __shared__ float red[LANES / 64];
+        __syncthreads();
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+        __syncthreads();
+        v = red[0];
+#pragma unroll
+        for (int w = 1; w < LANES / 64; w++) v = fmaxf(v, red[w]);
+    }
+    return v;
+}
+
 #endif

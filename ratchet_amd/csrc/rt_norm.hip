@@ -60,41 +60,41 @@ template <typename T, int KIND> __device__ __forceinline__ T norm_one(T x, const
 }
 
 // cols % VE == 0, rows 16-byte aligned, cols / VE <= 64 * NV
-template <typename T, int NV, int KIND>
+template <typename T, int NV, int KIND, int LANES>
 __global__ void __launch_bounds__(BLOCK) norm_wave_kernel(const T* __restrict__ x, const T* __restrict__ scale,
                                                           const T* __restrict__ bias, T* __restrict__ y, uint64_t rows, uint32_t cols,
                                                           float eps) {
     constexpr int VE = 16 / sizeof(T);
-    const uint64_t row = (uint64_t)blockIdx.x * WAVES + (threadIdx.x / WAVE);
+    const uint64_t row = (uint64_t)blockIdx.x * (BLOCK / LANES) + (threadIdx.x / LANES);
     if (row >= rows) return;
-    const int lane = threadIdx.x & (WAVE - 1);
+    const int lane = threadIdx.x & (LANES - 1);
     const uint32_t nvec = cols / VE;
     const v4u* xr = reinterpret_cast<const v4u*>(x + row * cols);
     v4u* yr = reinterpret_cast<v4u*>(y + row * cols);
     Vec16<T> v[NV];
 #pragma unroll
     for (int k = 0; k < NV; k++) {
-        const uint32_t i = lane + k * WAVE;
+        const uint32_t i = lane + k * LANES;
         if (i < nvec) v[k].u = ld_stream(xr + i);
     }
     float sx = 0.0f, sq = 0.0f;
 #pragma unroll
     for (int k = 0; k < NV; k++)
-        if (lane + k * WAVE < nvec)
+        if (lane + k * LANES < nvec)
 #pragma unroll
             for (int q = 0; q < VE; q++) {
                 const T e = v[k].e[q];
                 if (KIND == NORM_LAYER) sx += Ar<T>::widen(e);
                 sq += Ar<T>::widen(Ar<T>::mul(e, e));
             }
-    if (KIND == NORM_LAYER) sx = wave_sum(sx);
-    sq = wave_sum(sq);
+    if (KIND == NORM_LAYER) sx = row_sum<LANES>(sx);
+    sq = row_sum<LANES>(sq);
     const RowStats<T> st = finish_stats<T, KIND>(sx, sq, cols, eps);
     const v4u* sv = reinterpret_cast<const v4u*>(scale);
     const v4u* bv = reinterpret_cast<const v4u*>(bias);
 #pragma unroll
     for (int k = 0; k < NV; k++) {
-        const uint32_t i = lane + k * WAVE;
+        const uint32_t i = lane + k * LANES;
         if (i < nvec) {
             Vec16<T> s, b, o;
             s.u = sv[i];
@@ -142,40 +142,40 @@ __global__ void __launch_bounds__(BLOCK) norm_generic_kernel(const T* __restrict
 // separate ops, and no sequential chain: the f32 sums need no replay because the parity bar after the cast is the
 // 16-bit one.
 // ------------------------------------------------------------------------------------------------------------------
-template <typename T, int NV, int KIND>
+template <typename T, int NV, int KIND, int LANES>
 __global__ void __launch_bounds__(BLOCK) norm_via32_wave_kernel(const T* __restrict__ x, const float* __restrict__ scale,
                                                                 const float* __restrict__ bias, T* __restrict__ y, uint64_t rows,
                                                                 uint32_t cols, float eps) {
-    const uint64_t row = (uint64_t)blockIdx.x * WAVES + (threadIdx.x / WAVE);
+    const uint64_t row = (uint64_t)blockIdx.x * (BLOCK / LANES) + (threadIdx.x / LANES);
     if (row >= rows) return;
-    const int lane = threadIdx.x & (WAVE - 1);
+    const int lane = threadIdx.x & (LANES - 1);
     const uint32_t nvec = cols / 8;
     const v4u* xr = reinterpret_cast<const v4u*>(x + row * cols);
     v4u* yr = reinterpret_cast<v4u*>(y + row * cols);
     Vec16<T> v[NV];
 #pragma unroll
     for (int k = 0; k < NV; k++) {
-        const uint32_t i = lane + k * WAVE;
+        const uint32_t i = lane + k * LANES;
         if (i < nvec) v[k].u = ld_stream(xr + i);
     }
     float sx = 0.0f, sq = 0.0f;
 #pragma unroll
     for (int k = 0; k < NV; k++)
-        if (lane + k * WAVE < nvec)
+        if (lane + k * LANES < nvec)
 #pragma unroll
             for (int q = 0; q < 8; q++) {
                 const float e = Ar<T>::widen(v[k].e[q]);
                 if (KIND == NORM_LAYER) sx += e;
                 sq += e * e;
             }
-    if (KIND == NORM_LAYER) sx = wave_sum(sx);
-    sq = wave_sum(sq);
+    if (KIND == NORM_LAYER) sx = row_sum<LANES>(sx);
+    sq = row_sum<LANES>(sq);
     const RowStats<float> st = finish_stats<float, KIND>(sx, sq, cols, eps);
     const float4* sv = reinterpret_cast<const float4*>(scale);
     const float4* bv = reinterpret_cast<const float4*>(bias);
 #pragma unroll
     for (int k = 0; k < NV; k++) {
-        const uint32_t i = lane + k * WAVE;
+        const uint32_t i = lane + k * LANES;
         if (i < nvec) {
             float s[8], b[8] = {0, 0, 0, 0, 0, 0, 0, 0};
             *reinterpret_cast<float4*>(s) = sv[2 * i];
@@ -572,21 +572,37 @@ __global__ void __launch_bounds__(BLOCK) gn_apply_kernel(const T* __restrict__ x
 template <typename T, int KIND>
 int launch_norm(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint64_t rows, uint32_t cols, float eps) {
     constexpr int VE = 16 / sizeof(T);
+    const uint32_t nvec = cols / VE;
     const bool vec_ok = (cols % VE == 0) && rt_aligned(x, 16) && rt_aligned(y, 16) && rt_aligned(scale, 16) &&
-                        (!bias || rt_aligned(bias, 16)) && (cols / VE) <= (uint32_t)(WAVE * 8);
-    if (vec_ok) {
-        const uint32_t nv = (cols / VE + WAVE - 1) / WAVE;
+                        (!bias || rt_aligned(bias, 16)) && nvec <= (uint32_t)(BLOCK * 8);
+    if (vec_ok && nvec <= (uint32_t)(WAVE * 8)) {
+        const uint32_t nv = (nvec + WAVE - 1) / WAVE;
         const uint64_t blocks = (rows + WAVES - 1) / WAVES;
         RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
         const dim3 grid((unsigned)blocks), block(BLOCK);
-#define RT_NORM(NVC)                                                                                                           \
-    hipLaunchKernelGGL((norm_wave_kernel<T, NVC, KIND>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, \
+#define RT_NORM(NVC)                                                                                                                 \
+    hipLaunchKernelGGL((norm_wave_kernel<T, NVC, KIND, WAVE>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, \
                        (T*)y, rows, cols, eps)
         if (nv <= 1) RT_NORM(1);
         else if (nv <= 2) RT_NORM(2);
         else if (nv <= 3) RT_NORM(3);
         else if (nv <= 4) RT_NORM(4);
         else if (nv <= 5) RT_NORM(5);
+        else if (nv <= 6) RT_NORM(6);
+        else RT_NORM(8);
+#undef RT_NORM
+        RT_CHECK_LAUNCH("norm_wave_kernel");
+        return RT_OK;
+    }
+    if (vec_ok) {                                            // longer rows: the 256 threads of a block share one row
+        const uint32_t nv = (nvec + BLOCK - 1) / BLOCK;
+        RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
+        const dim3 grid((unsigned)rows), block(BLOCK);
+#define RT_NORM(NVC)                                                                                                                  \
+    hipLaunchKernelGGL((norm_wave_kernel<T, NVC, KIND, BLOCK>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, \
+                       (T*)y, rows, cols, eps)
+        if (nv <= 3) RT_NORM(3);
+        else if (nv <= 4) RT_NORM(4);
         else if (nv <= 6) RT_NORM(6);
         else RT_NORM(8);
 #undef RT_NORM
@@ -705,15 +721,28 @@ template <typename T, int KIND>
 int launch_norm_via32(rt_device* dev, const void* x, const float* scale, const float* bias, void* y, uint64_t rows, uint32_t cols, float eps) {
     const uint32_t nvec = cols / 8;
     const bool vec_ok = (cols % 8 == 0) && rt_aligned(x, 16) && rt_aligned(y, 16) && rt_aligned(scale, 16) && (!bias || rt_aligned(bias, 16)) &&
-                        nvec <= (uint32_t)(WAVE * 8);
-    if (vec_ok) {
+                        nvec <= (uint32_t)(BLOCK * 8);
+    if (vec_ok && nvec <= (uint32_t)(WAVE * 8)) {
         const uint32_t nv = (nvec + WAVE - 1) / WAVE;
         const uint64_t blocks = (rows + WAVES - 1) / WAVES;
         RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_norm_via_f32: too many rows");
         const dim3 grid((unsigned)blocks), block(BLOCK);
-#define RT_NV(NVC) hipLaunchKernelGGL((norm_via32_wave_kernel<T, NVC, KIND>), grid, block, 0, dev->stream, (const T*)x, scale, bias, (T*)y, rows, cols, eps)
+#define RT_NV(NVC) hipLaunchKernelGGL((norm_via32_wave_kernel<T, NVC, KIND, WAVE>), grid, block, 0, dev->stream, (const T*)x, scale, bias, (T*)y, rows, cols, eps)
         if (nv <= 1) RT_NV(1);
         else if (nv <= 2) RT_NV(2);
+        else if (nv <= 4) RT_NV(4);
+        else if (nv <= 6) RT_NV(6);
+        else RT_NV(8);
+#undef RT_NV
+        RT_CHECK_LAUNCH("norm_via32_wave_kernel");
+        return RT_OK;
+    }
+    if (vec_ok) {
+        const uint32_t nv = (nvec + BLOCK - 1) / BLOCK;
+        RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "rt_norm_via_f32: too many rows");
+        const dim3 grid((unsigned)rows), block(BLOCK);
+#define RT_NV(NVC) hipLaunchKernelGGL((norm_via32_wave_kernel<T, NVC, KIND, BLOCK>), grid, block, 0, dev->stream, (const T*)x, scale, bias, (T*)y, rows, cols, eps)
+        if (nv <= 3) RT_NV(3);
         else if (nv <= 4) RT_NV(4);
         else if (nv <= 6) RT_NV(6);
         else RT_NV(8);

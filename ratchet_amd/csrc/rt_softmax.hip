@@ -22,24 +22,26 @@ constexpr int WAVES = BLOCK / WAVE;
 template <typename T> __device__ __forceinline__ float stable_exp(float v) { return expf(v); }
 
 // ------------------------------------------------------------------------------------------------------------------
-// wave-per-row, row held in registers.  Requires cols % VE == 0, 16-byte aligned rows, cols / VE <= 64 * NV.
+// Row held in registers by the LANES threads that share it: a wave64 (four rows per block) for rows of up to 512
+// vectors, the whole 256-thread block for rows of up to 2048 vectors (8192 f32 / 16384 16-bit columns).
+// Requires cols % VE == 0, 16-byte aligned rows, cols / VE <= LANES * NV.
 // MODE 0: reference arithmetic for f32 (exp, tree sum, divide).  MODE 1: stable (max subtraction, f32 accumulate) for
 // any T; results are rounded to T once.
 // ------------------------------------------------------------------------------------------------------------------
-template <typename T, int NV, int MODE>
+template <typename T, int NV, int MODE, int LANES>
 __global__ void __launch_bounds__(BLOCK) softmax_wave_kernel(const T* __restrict__ x, T* __restrict__ y, uint64_t rows,
                                                              uint32_t cols) {
     constexpr int VE = 16 / sizeof(T);
-    const uint64_t row = (uint64_t)blockIdx.x * WAVES + (threadIdx.x / WAVE);
+    const uint64_t row = (uint64_t)blockIdx.x * (BLOCK / LANES) + (threadIdx.x / LANES);
     if (row >= rows) return;
-    const int lane = threadIdx.x & (WAVE - 1);
+    const int lane = threadIdx.x & (LANES - 1);
     const uint32_t nvec = cols / VE;
     const v4u* xr = reinterpret_cast<const v4u*>(x + row * cols);
     v4u* yr = reinterpret_cast<v4u*>(y + row * cols);
     Vec16<T> v[NV];
 #pragma unroll
     for (int k = 0; k < NV; k++) {
-        const uint32_t i = lane + k * WAVE;
+        const uint32_t i = lane + k * LANES;
         if (i < nvec) v[k].u = ld_stream(xr + i);
     }
     float e[NV][VE];
@@ -47,24 +49,24 @@ __global__ void __launch_bounds__(BLOCK) softmax_wave_kernel(const T* __restrict
         float m = -__builtin_huge_valf();
 #pragma unroll
         for (int k = 0; k < NV; k++)
-            if (lane + k * WAVE < nvec)
+            if (lane + k * LANES < nvec)
 #pragma unroll
                 for (int q = 0; q < VE; q++) m = fmaxf(m, Ar<T>::widen(v[k].e[q]));
-        m = wave_max(m);
+        m = row_max<LANES>(m);
         if (m == -__builtin_huge_valf()) m = 0.0f;           // fully masked row: exp(-inf - 0) = 0, 0/0 = NaN as torch does
         float s = 0.0f;
 #pragma unroll
         for (int k = 0; k < NV; k++)
-            if (lane + k * WAVE < nvec)
+            if (lane + k * LANES < nvec)
 #pragma unroll
                 for (int q = 0; q < VE; q++) {
                     e[k][q] = expf(Ar<T>::widen(v[k].e[q]) - m);
                     s += e[k][q];
                 }
-        s = wave_sum(s);
+        s = row_sum<LANES>(s);
 #pragma unroll
         for (int k = 0; k < NV; k++) {
-            const uint32_t i = lane + k * WAVE;
+            const uint32_t i = lane + k * LANES;
             if (i < nvec) {
                 Vec16<T> o;
 #pragma unroll
@@ -76,20 +78,20 @@ __global__ void __launch_bounds__(BLOCK) softmax_wave_kernel(const T* __restrict
         float s = 0.0f;
 #pragma unroll
         for (int k = 0; k < NV; k++)
-            if (lane + k * WAVE < nvec)
+            if (lane + k * LANES < nvec)
 #pragma unroll
                 for (int q = 0; q < VE; q++) {
                     e[k][q] = expf(Ar<T>::widen(v[k].e[q]));
                     s += e[k][q];
                 }
-        s = wave_sum(s);
+        s = row_sum<LANES>(s);
         // e / s as e * (1/s): one correctly rounded reciprocal per row, at most 1 ulp from the quotient (bar: 1e-5).
         // A zero, subnormal, inf or NaN sum keeps the division so that 0/0, x/inf and inf/inf come out as the reference's do.
         const bool plain = (s >= 1.17549435e-38f) && (s < __builtin_huge_valf());
         const float rs = 1.0f / s;
 #pragma unroll
         for (int k = 0; k < NV; k++) {
-            const uint32_t i = lane + k * WAVE;
+            const uint32_t i = lane + k * LANES;
             if (i < nvec) {
                 Vec16<T> o;
 #pragma unroll
@@ -451,7 +453,7 @@ template <typename T> __device__ __forceinline__ uint64_t mask_row_offset(uint64
 // library expf the f32 softmax uses costs about four times as many instructions.
 __device__ __forceinline__ float via32_exp(float v) { return __builtin_amdgcn_exp2f(v * 1.44269504088896341f); }
 
-template <typename T, int NV, int MODE, bool MASK>
+template <typename T, int NV, int MODE, bool MASK, int LANES>
 __global__ void __launch_bounds__(BLOCK) softmax_via32_wave_kernel(const T* __restrict__ x, const T* __restrict__ mask,
                                                                    T* __restrict__ y, uint64_t rows, uint32_t cols, MaskArgs p) {
     uint32_t blk = blockIdx.x;
@@ -460,16 +462,16 @@ __global__ void __launch_bounds__(BLOCK) softmax_via32_wave_kernel(const T* __re
         fd_divmod(blk / SM_XCDS, p.reps, grp, rep);
         blk = rep * p.slabs + grp * SM_XCDS + (blk % SM_XCDS);
     }
-    const uint64_t row = (uint64_t)blk * WAVES + (threadIdx.x / WAVE);
+    const uint64_t row = (uint64_t)blk * (BLOCK / LANES) + (threadIdx.x / LANES);
     if (row >= rows) return;
-    const int lane = threadIdx.x & (WAVE - 1);
+    const int lane = threadIdx.x & (LANES - 1);
     const uint32_t nvec = cols / 8;
     const v4u* xr = reinterpret_cast<const v4u*>(x + row * cols);
     v4u* yr = reinterpret_cast<v4u*>(y + row * cols);
     Vec16<T> v[NV];
 #pragma unroll
     for (int k = 0; k < NV; k++) {
-        const uint32_t i = lane + k * WAVE;
+        const uint32_t i = lane + k * LANES;
         if (i < nvec) v[k].u = ld_stream(xr + i);
     }
     if (MASK) {
@@ -478,7 +480,7 @@ __global__ void __launch_bounds__(BLOCK) softmax_via32_wave_kernel(const T* __re
             const v4u* mv = reinterpret_cast<const v4u*>(mr);
 #pragma unroll
             for (int k = 0; k < NV; k++) {
-                const uint32_t i = lane + k * WAVE;
+                const uint32_t i = lane + k * LANES;
                 if (i < nvec) {
                     Vec16<T> m;
                     m.u = mv[i];
@@ -500,27 +502,27 @@ __global__ void __launch_bounds__(BLOCK) softmax_via32_wave_kernel(const T* __re
         m = -__builtin_huge_valf();
 #pragma unroll
         for (int k = 0; k < NV; k++)
-            if (lane + k * WAVE < nvec)
+            if (lane + k * LANES < nvec)
 #pragma unroll
                 for (int q = 0; q < 8; q++) m = fmaxf(m, Ar<T>::widen(v[k].e[q]));
-        m = wave_max(m);
+        m = row_max<LANES>(m);
         if (m == -__builtin_huge_valf()) m = 0.0f;
     }
     float s = 0.0f;
 #pragma unroll
     for (int k = 0; k < NV; k++)
-        if (lane + k * WAVE < nvec)
+        if (lane + k * LANES < nvec)
 #pragma unroll
             for (int q = 0; q < 8; q++) {
                 e[k][q] = via32_exp(Ar<T>::widen(v[k].e[q]) - m);
                 s += e[k][q];
             }
-    s = wave_sum(s);
+    s = row_sum<LANES>(s);
     const bool plain = (s >= 1.17549435e-38f) && (s < __builtin_huge_valf());
     const float rs = 1.0f / s;
 #pragma unroll
     for (int k = 0; k < NV; k++) {
-        const uint32_t i = lane + k * WAVE;
+        const uint32_t i = lane + k * LANES;
         if (i < nvec) {
             Vec16<T> o;
 #pragma unroll
@@ -580,25 +582,37 @@ __global__ void __launch_bounds__(BLOCK) softmax_via32_generic_kernel(const T* _
 template <typename T, int MODE> int launch_wave(rt_device* dev, const void* x, void* y, uint64_t rows, uint32_t cols) {
     constexpr int VE = 16 / sizeof(T);
     const uint32_t nvec = cols / VE;
-    const uint32_t nv = (nvec + WAVE - 1) / WAVE;
-    const uint64_t blocks = (rows + WAVES - 1) / WAVES;
-    RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax: too many rows");
-    const dim3 grid((unsigned)blocks), block(BLOCK);
-#define RT_SM(NVC) hipLaunchKernelGGL((softmax_wave_kernel<T, NVC, MODE>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols)
-    if (nv <= 1) RT_SM(1);
-    else if (nv <= 2) RT_SM(2);
-    else if (nv <= 3) RT_SM(3);
-    else if (nv <= 4) RT_SM(4);
-    else if (nv <= 6) RT_SM(6);
-    else RT_SM(8);
+    if (nvec <= (uint32_t)(WAVE * 8)) {
+        const uint32_t nv = (nvec + WAVE - 1) / WAVE;
+        const uint64_t blocks = (rows + WAVES - 1) / WAVES;
+        RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax: too many rows");
+        const dim3 grid((unsigned)blocks), block(BLOCK);
+#define RT_SM(NVC) hipLaunchKernelGGL((softmax_wave_kernel<T, NVC, MODE, WAVE>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols)
+        if (nv <= 1) RT_SM(1);
+        else if (nv <= 2) RT_SM(2);
+        else if (nv <= 3) RT_SM(3);
+        else if (nv <= 4) RT_SM(4);
+        else if (nv <= 6) RT_SM(6);
+        else RT_SM(8);
 #undef RT_SM
+    } else {
+        const uint32_t nv = (nvec + BLOCK - 1) / BLOCK;
+        RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax: too many rows");
+        const dim3 grid((unsigned)rows), block(BLOCK);
+#define RT_SM(NVC) hipLaunchKernelGGL((softmax_wave_kernel<T, NVC, MODE, BLOCK>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols)
+        if (nv <= 3) RT_SM(3);
+        else if (nv <= 4) RT_SM(4);
+        else if (nv <= 6) RT_SM(6);
+        else RT_SM(8);
+#undef RT_SM
+    }
     RT_CHECK_LAUNCH("softmax_wave_kernel");
     return RT_OK;
 }
 
 template <typename T, int MODE> int launch_f32_style(rt_device* dev, const void* x, void* y, uint64_t rows, uint32_t cols) {
     constexpr int VE = 16 / sizeof(T);
-    const bool vec_ok = (cols % VE == 0) && rt_aligned(x, 16) && rt_aligned(y, 16) && (cols / VE) <= (uint32_t)(WAVE * 8);
+    const bool vec_ok = (cols % VE == 0) && rt_aligned(x, 16) && rt_aligned(y, 16) && (cols / VE) <= (uint32_t)(BLOCK * 8);
     if (vec_ok) return launch_wave<T, MODE>(dev, x, y, rows, cols);
     RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax: too many rows");
     hipLaunchKernelGGL((softmax_generic_kernel<T, MODE>), dim3((unsigned)rows), dim3(BLOCK), 0, dev->stream, (const T*)x, (T*)y, rows,
@@ -668,17 +682,34 @@ template <typename T> int launch_seq16(rt_device* dev, const void* x, void* y, u
 template <typename T, int MODE, bool MASK>
 int launch_via32(rt_device* dev, const void* x, const void* mask, void* y, uint64_t rows, uint32_t cols, const MaskArgs& p, bool mask_vec_ok) {
     const uint32_t nvec = cols / 8;
-    const bool vec_ok = (cols % 8 == 0) && rt_aligned(x, 16) && rt_aligned(y, 16) && nvec <= (uint32_t)(WAVE * 8) && (!MASK || mask_vec_ok);
-    if (vec_ok) {
+    const bool vec_ok = (cols % 8 == 0) && rt_aligned(x, 16) && rt_aligned(y, 16) && nvec <= (uint32_t)(BLOCK * 8) && (!MASK || mask_vec_ok);
+    if (vec_ok && nvec <= (uint32_t)(WAVE * 8)) {
         const uint32_t nv = (nvec + WAVE - 1) / WAVE;
         const uint64_t blocks = (rows + WAVES - 1) / WAVES;
         RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax_via_f32: too many rows");
         const dim3 grid((unsigned)blocks), block(BLOCK);
 #define RT_SV(NVC)                                                                                                                 \
-    hipLaunchKernelGGL((softmax_via32_wave_kernel<T, NVC, MODE, MASK>), grid, block, 0, dev->stream, (const T*)x, (const T*)mask, (T*)y, \
-                       rows, cols, p)
+    hipLaunchKernelGGL((softmax_via32_wave_kernel<T, NVC, MODE, MASK, WAVE>), grid, block, 0, dev->stream, (const T*)x, (const T*)mask, \
+                       (T*)y, rows, cols, p)
         if (nv <= 1) RT_SV(1);
         else if (nv <= 2) RT_SV(2);
+        else if (nv <= 4) RT_SV(4);
+        else if (nv <= 6) RT_SV(6);
+        else RT_SV(8);
+#undef RT_SV
+        RT_CHECK_LAUNCH("softmax_via32_wave_kernel");
+        return RT_OK;
+    }
+    if (vec_ok) {                                            // rows of up to 16384 columns: the block shares the row
+        MaskArgs q = p;
+        q.slabs = 0;                                         // the XCD-aware order is laid out for four rows per block
+        const uint32_t nv = (nvec + BLOCK - 1) / BLOCK;
+        RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax_via_f32: too many rows");
+        const dim3 grid((unsigned)rows), block(BLOCK);
+#define RT_SV(NVC)                                                                                                                  \
+    hipLaunchKernelGGL((softmax_via32_wave_kernel<T, NVC, MODE, MASK, BLOCK>), grid, block, 0, dev->stream, (const T*)x, (const T*)mask, \
+                       (T*)y, rows, cols, q)
+        if (nv <= 3) RT_SV(3);
         else if (nv <= 4) RT_SV(4);
         else if (nv <= 6) RT_SV(6);
         else RT_SV(8);

@@ -88,7 +88,8 @@ def test_gated_mul_matches_the_op_sequence(dev, oracle, shape, split):
 
 
 @pytest.mark.parametrize("kind", ["layer", "rms"])
-@pytest.mark.parametrize("rows,cols", [(64, 2560), (100, 3072), (257, 384), (9, 4096), (5, 1000), (3, 77), (2, 8192)])
+@pytest.mark.parametrize("rows,cols", [(64, 2560), (100, 3072), (257, 384), (9, 4096), (5, 1000), (3, 77), (2, 8192), (3, 5120), (2, 16384),
+                                       (2, 16392)])
 def test_norm_via_f32(dev, oracle, kind, rows, cols):
     rng = np.random.default_rng(503)
     x = (randn(rng, (rows, cols), np.float16) * np.float16(3) + np.float16(0.5)).astype(np.float16)
@@ -129,7 +130,9 @@ def _attn_case(rng, B, H, S, T, mask_kind, dtype=np.float16):
 
 @pytest.mark.parametrize("B,H,S,T,mask_kind", [(1, 4, 128, 128, "causal"), (2, 3, 64, 200, "causal4"), (1, 6, 100, 1500, None),
                                                (2, 2, 33, 77, "per_batch"), (1, 2, 40, 64, "row_scalar"), (1, 8, 512, 1024, "causal"),
-                                               (1, 2, 7, 4096, "causal"), (1, 1, 3, 8200, None), (1, 3, 5, 4100, "causal")])
+                                               (1, 2, 7, 4096, "causal"), (1, 1, 3, 8200, None), (1, 3, 5, 4100, "causal"),
+                                               (1, 2, 6, 8192, "causal"), (2, 1, 3, 16384, "per_batch"), (1, 2, 4, 6000, None),
+                                               (1, 1, 2, 16392, None)])
 def test_softmax_via_f32(dev, oracle, B, H, S, T, mask_kind):
     rng = np.random.default_rng(504)
     x, mask = _attn_case(rng, B, H, S, T, mask_kind)

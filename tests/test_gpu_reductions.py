@@ -24,7 +24,7 @@ def dev():
 
 
 SOFTMAX_SHAPES = [(3, 256, 256), (1, 7, 33), (2, 1, 1), (1, 5, 255), (2, 64, 1500), (1, 3, 2048), (1, 2, 2052), (1, 130, 8),
-                  (1, 3, 5000)]
+                  (1, 3, 5000), (2, 9, 4096), (1, 5, 3072), (1, 3, 8192), (1, 2, 8196), (1, 2, 6148)]   # > 2048 columns: a block per row
 
 
 @pytest.mark.parametrize("shape", SOFTMAX_SHAPES)
@@ -138,7 +138,8 @@ def test_softmax_bf16_and_stable_mode(dev, oracle):
         assert bad == 0, (dtype, bad, mx)
 
 
-NORM_SHAPES = [(3, 256, 256), (2, 57, 1001), (1, 1, 1), (1, 13, 7), (1, 150, 384), (2, 9, 2048), (1, 5, 2052), (1, 3, 6000)]
+NORM_SHAPES = [(3, 256, 256), (2, 57, 1001), (1, 1, 1), (1, 13, 7), (1, 150, 384), (2, 9, 2048), (1, 5, 2052), (1, 3, 6000),
+               (2, 33, 2560), (1, 9, 3072), (1, 3, 8192), (1, 2, 8196)]                             # > 2048 columns: a block per row
 
 
 @pytest.mark.parametrize("shape", NORM_SHAPES)
