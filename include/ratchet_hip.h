@@ -168,6 +168,14 @@ int rt_rms_norm(rt_device* dev, int dt, const void* x, const void* scale, void* 
 int rt_group_norm(rt_device* dev, int dt, const void* x, const void* scale, const void* bias, void* y, uint32_t B,
                   uint32_t C, uint32_t L, uint32_t groups, float eps);
 
+/* scores.add(mask).softmax(last dim) in the tensors' own arithmetic (the 16-bit sum is rounded as the separate add
+ * rounds it, then Softmax's contract applies), result bit-identical to rt_binary_bcast(RT_ADD) followed by rt_softmax
+ * but the sum never reaches memory when the shape allows (f16, reference mode, up to 4096 columns, a mask that covers
+ * whole trailing dims and repeats over the leading ones).  Each mask extent is 1 or the scores' extent; y may be x.
+ * Binary: ops/binary.rs:27-119 via tensor.rs:249-280; Softmax: ops/softmax.rs:17-73, cpu/softmax.rs:22-42. */
+int rt_softmax_masked(rt_device* dev, int dt, const void* x, const uint32_t x_shape[4], const void* mask,
+                      const uint32_t mask_shape[4], void* y, int mode);
+
 /* ---- Replayable launch lists ---------------------------------------------------------------------------------------
  * The reference encodes every compiled op of a graph into one command buffer and submits it once
  * (Executable::dispatch, executable.rs:33-59).  The counterpart here is a HIP graph: between rt_capture_begin and

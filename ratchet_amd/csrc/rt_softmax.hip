@@ -252,6 +252,7 @@ constexpr size_t SP_TILE_BYTES = 2 * SP_ROWS * (SP_TC + SP_PAD) * sizeof(uint16_
 constexpr size_t SP_SMEM_BYTES = SP_LUT_BYTES + SP_TILE_BYTES + 2 * 32 * sizeof(uint16_t);      // 162 880 of the CU's 163 840 bytes
 
 typedef _Float16 h16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 // exp of two packed f16 bit patterns: two lookups in the full 65536-entry table (NaN, inf and the saturated ends included)
@@ -259,9 +260,42 @@ __device__ __forceinline__ uint32_t sp_exp_pair(const uint16_t* lut, uint32_t p)
     return (uint32_t)lut[p & 0xffffu] | ((uint32_t)lut[p >> 16] << 16);
 }
 
-template <int NSLOT, bool FULL>
-__global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint16_t* __restrict__ table, const half_t* x, half_t* y,
-                                                                      uint64_t rows, uint32_t cols) {
+// Which 30-row groups a block works on, and in which order.  Rows come in `reps` periods of P rows (P = all rows when
+// nothing repeats; P = the rows one mask covers when a mask is added, e.g. S rows per head for an [S, T] mask under
+// B * H heads); a period holds GP = ceil(P / 30) groups, none of which straddles two periods.
+//   xcd == 0: item w = block + i * grid  ->  (rep, group) = (w / GP, w % GP).
+//   xcd == 1: the hardware places block b on XCD b % 8.  XCD k takes the groups pg = k, k + 8, ... of every period and
+//             walks them repeat-fastest, so the blocks of one XCD work on the same mask rows at the same time and the
+//             XCD's L2 fetches each mask row once instead of once per head.
+struct SpSched {
+    uint32_t P, GP, reps, xcd;
+    FastDiv gp_div, reps_div;
+};
+constexpr uint32_t SP_XCDS = 8;
+
+__device__ __forceinline__ uint32_t sp_item_count(const SpSched& s, uint32_t b, uint32_t G) {
+    if (!s.xcd) {
+        const uint32_t total = s.GP * s.reps;
+        return b < total ? (total - b + G - 1) / G : 0;
+    }
+    const uint32_t k = b % SP_XCDS, j0 = b / SP_XCDS, gx = G / SP_XCDS;
+    const uint32_t total = (s.GP > k ? (s.GP - k + SP_XCDS - 1) / SP_XCDS : 0) * s.reps;
+    return j0 < total ? (total - j0 + gx - 1) / gx : 0;
+}
+__device__ __forceinline__ void sp_item(const SpSched& s, uint32_t b, uint32_t G, uint32_t it, uint32_t& rep, uint32_t& pg) {
+    if (!s.xcd) {
+        fd_divmod(b + it * G, s.gp_div, rep, pg);
+    } else {
+        uint32_t pgl;
+        fd_divmod(b / SP_XCDS + it * (G / SP_XCDS), s.reps_div, pgl, rep);
+        pg = pgl * SP_XCDS + b % SP_XCDS;
+    }
+}
+
+template <int NSLOT, bool FULL, bool MASK>
+__global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint16_t* __restrict__ table, const half_t* x,
+                                                                      const half_t* mask, half_t* y, uint64_t rows, uint32_t cols,
+                                                                      SpSched sch) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint16_t* lut = reinterpret_cast<uint16_t*>(smem);
     half_t (*tile)[SP_ROWS][SP_TC + SP_PAD] = reinterpret_cast<half_t (*)[SP_ROWS][SP_TC + SP_PAD]>(smem + SP_LUT_BYTES);
@@ -274,7 +308,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
 #pragma unroll
         for (uint32_t i = 0; i < SP_LUT_BYTES / 16 / SP_BLOCK; i++) dst[i * SP_BLOCK + threadIdx.x] = src[i * SP_BLOCK + threadIdx.x];
     }
-    const uint64_t ngroups = (rows + SP_ROWS - 1) / SP_ROWS;
+    const uint32_t n_items = sp_item_count(sch, blockIdx.x, gridDim.x);
     __syncthreads();                                         // table visible
 
     if (threadIdx.x < 64) {
@@ -284,7 +318,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
         const uint32_t wr = lane < SP_ROWS ? lane : 0;       // lanes 30..63 shadow row 0 and never publish
         half_t run = (half_t)0.0f;
         uint32_t gpar = 0;
-        for (uint64_t g = blockIdx.x; g < ngroups; g += gridDim.x) {
+        for (uint32_t it = 0; it < n_items; it++) {
 #pragma unroll 1
             for (int t = 0; t < NSLOT; t++) {
                 __syncthreads();                             // tile t is in LDS
@@ -333,28 +367,40 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
     const uint32_t nbytes = (uint32_t)(rows * row_bytes);    // the launcher keeps this below 2^31
     const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(x), 0, nbytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(y, 0, nbytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rm =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(MASK ? mask : x), 0, MASK ? sch.P * row_bytes : nbytes, 0x00020000);
     constexpr uint32_t OOB = 0x80000000u;                    // >= nbytes, and stays so after adding a column offset
-    constexpr int PF = NSLOT < SP_PF ? NSLOT : SP_PF;        // tiles in flight per thread
+    constexpr int PF = MASK ? 2 : (NSLOT < SP_PF ? NSLOT : SP_PF);   // tiles in flight per thread (the mask doubles the registers)
     const uint32_t G = gridDim.x;
 
-    auto group_off = [&](uint64_t g) -> uint32_t {           // byte offset of (row r of group g, column ccol), or OOB
-        const uint64_t row = g * SP_ROWS + r;
-        return (g < ngroups && row < rows) ? (uint32_t)row * row_bytes + ccol * 2 : OOB;
+    // byte offsets of (row r of item `it`, column ccol) in x / y and in the mask, or OOB
+    auto item_off = [&](uint32_t it, uint32_t& xo, uint32_t& mo) {
+        uint32_t rep, pg;
+        sp_item(sch, blockIdx.x, G, it, rep, pg);
+        const uint32_t prow = pg * SP_ROWS + r;              // row inside the period
+        const bool ok = it < n_items && prow < sch.P;
+        mo = ok ? prow * row_bytes + ccol * 2 : OOB;
+        xo = ok ? (rep * sch.P + prow) * row_bytes + ccol * 2 : OOB;
     };
     auto slot_off = [&](uint32_t base, int t) -> uint32_t {
         if (!FULL && (uint32_t)t * SP_TC + ccol >= cols) return OOB;
         return base + (uint32_t)t * (SP_TC * 2);
     };
     auto load_x = [&](uint32_t off) -> v4u { return __builtin_amdgcn_raw_buffer_load_b128(rx, off, 0, 2); };   // 2: non-temporal
+    auto load_m = [&](uint32_t off) -> v4u { return __builtin_amdgcn_raw_buffer_load_b128(rm, off, 0, 0); };   // re-read by other heads
 
-    uint64_t g = blockIdx.x;
-    uint32_t cur = group_off(g), nxt = group_off(g + G), prev = OOB;
+    uint32_t cur, nxt, mcur, mnxt, prev = OOB;
+    item_off(0, cur, mcur);
+    item_off(1, nxt, mnxt);
     v4u e[NSLOT];                                            // exp values of the group in flight, 8 halves per slot
-    v4u pre[PF];
+    v4u pre[PF], mpre[MASK ? PF : 1];
 #pragma unroll
     for (int t = 0; t < NSLOT; t++) e[t] = v4u{0, 0, 0, 0};
 #pragma unroll
-    for (int k = 0; k < PF; k++) pre[k] = load_x(slot_off(cur, k));
+    for (int k = 0; k < PF; k++) {
+        pre[k] = load_x(slot_off(cur, k));
+        if (MASK) mpre[k] = load_m(slot_off(mcur, k));
+    }
 
     float s_prev = 1.0f, rinv_prev = 1.0f;
     bool fast_prev = true;
@@ -392,10 +438,14 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
         rinv_prev = fast_prev ? 1.0f / s : 0.0f;
     };
 
-    for (; g < ngroups; g += G) {
+    for (uint32_t it = 0; it < n_items; it++) {
 #pragma unroll
         for (int t = 0; t < NSLOT; t++) {
             v4u& in = pre[t % PF];
+            if (MASK) {                                      // scores + mask in f16, as the separate add would round it
+                const h16x8 sum = __builtin_bit_cast(h16x8, in) + __builtin_bit_cast(h16x8, mpre[t % PF]);
+                in = __builtin_bit_cast(v4u, sum);
+            }
             // exp of the vector that arrived, parked in the LDS tile for the walk (zeros past the row end: adding +0 is a no-op;
             // rows past the tensor's end read zeros and their sums are never used)
             v4u enew;
@@ -404,7 +454,13 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
             if (!FULL && (uint32_t)t * SP_TC + ccol >= cols) enew = v4u{0, 0, 0, 0};
             *reinterpret_cast<v4u*>(&tile[t & 1][r][ccol]) = enew;
             // next load for this register: PF tiles ahead, possibly in the block's next group
-            in = (t + PF < NSLOT) ? load_x(slot_off(cur, t + PF)) : load_x(slot_off(nxt, t + PF - NSLOT));
+            if (t + PF < NSLOT) {
+                in = load_x(slot_off(cur, t + PF));
+                if (MASK) mpre[t % PF] = load_m(slot_off(mcur, t + PF));
+            } else {
+                in = load_x(slot_off(nxt, t + PF - NSLOT));
+                if (MASK) mpre[t % PF] = load_m(slot_off(mnxt, t + PF - NSLOT));
+            }
             __syncthreads();
             if (t == 0) read_prev_sum(gpar ^ 1);              // published by wave 0 before it reached this barrier
             const v4u out = quotients(e[t]);                  // first group: prev is OOB, the store is dropped
@@ -413,7 +469,8 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
         }
         prev = cur;
         cur = nxt;
-        nxt = group_off(g + 2 * (uint64_t)G);
+        mcur = mnxt;
+        item_off(it + 2, nxt, mnxt);
         gpar ^= 1;
     }
     // drain: outputs of the block's last group
@@ -621,45 +678,71 @@ template <typename T, int MODE> int launch_f32_style(rt_device* dev, const void*
     return RT_OK;
 }
 
-int launch_f16_stream(rt_device* dev, const void* x, void* y, uint64_t rows, uint32_t cols) {
+// mask == nullptr: plain softmax.  Otherwise the mask has `period` rows of `cols` columns and repeats every `period`
+// rows of x (rows % period == 0).  Returns RT_OK with *done = false when the shape does not fit this kernel.
+int launch_f16_stream(rt_device* dev, const void* x, const void* mask, uint64_t period, void* y, uint64_t rows, uint32_t cols, bool* done) {
+    *done = false;
+    const uint64_t row_bytes = (uint64_t)cols * 2;
+    if (!mask) period = rows;
+    // the kernel addresses a launch with 32-bit byte offsets below 2^31: larger tensors go in chunks of whole periods
+    // (whole 30-row groups when nothing repeats)
+    uint64_t chunk_rows;
+    if (mask) {
+        if (period * row_bytes > 0x7fffffffull) return RT_OK;
+        chunk_rows = (0x7fffffffull / (period * row_bytes)) * period;
+    } else {
+        chunk_rows = (0x7fffffffull / row_bytes) / SP_ROWS * SP_ROWS;
+    }
     const uint16_t* table = nullptr;
     int rc = rt_unary_table(dev, 0, RT_EXP, &table);
     if (rc) return rc;
     const uint32_t nt = (cols + SP_TC - 1) / SP_TC;
     const bool full = cols % SP_TC == 0 && (nt == 2 || nt == 4 || nt == 8 || nt == 16);
-    // the kernel addresses the tensor with 32-bit byte offsets below 2^31: larger tensors go in row chunks
-    const uint64_t max_rows = (0x7fffffffull / ((uint64_t)cols * 2)) / SP_ROWS * SP_ROWS;
-#define RT_SP(NS, F)                                                                                                                 \
+#define RT_SP(NS, F, M)                                                                                                              \
     do {                                                                                                                             \
-        const unsigned bit = 1u << ((NS == 2 ? 0 : NS == 4 ? 1 : NS == 8 ? 2 : 3) + (F ? 4 : 0));                                   \
+        const unsigned bit = 1u << ((NS == 2 ? 0 : NS == 4 ? 1 : NS == 8 ? 2 : 3) + (F ? 4 : 0) + (M ? 8 : 0));                      \
         if (!(dev->sp_attr_set & bit)) {               /* the LDS opt-in is per function and per device */                           \
-            RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(softmax_f16_stream_kernel<NS, F>),                              \
+            RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(softmax_f16_stream_kernel<NS, F, M>),                           \
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)SP_SMEM_BYTES));                             \
             dev->sp_attr_set |= bit;                                                                                                 \
         }                                                                                                                            \
-        hipLaunchKernelGGL((softmax_f16_stream_kernel<NS, F>), dim3((unsigned)blocks), dim3(SP_BLOCK), SP_SMEM_BYTES, dev->stream,   \
-                           table, xc, yc, n, cols);                                                                                  \
+        hipLaunchKernelGGL((softmax_f16_stream_kernel<NS, F, M>), dim3(blocks), dim3(SP_BLOCK), SP_SMEM_BYTES, dev->stream, table,   \
+                           xc, (const half_t*)mask, yc, n, cols, sch);                                                               \
     } while (0)
-    for (uint64_t row0 = 0; row0 < rows; row0 += max_rows) {
-        const uint64_t n = rows - row0 < max_rows ? rows - row0 : max_rows;
+#define RT_SP_NS(F, M)                                      \
+    do {                                                    \
+        if (nt <= 2) RT_SP(2, F, M);                        \
+        else if (nt <= 4) RT_SP(4, F, M);                   \
+        else if (nt <= 8) RT_SP(8, F, M);                   \
+        else RT_SP(16, F, M);                               \
+    } while (0)
+    for (uint64_t row0 = 0; row0 < rows; row0 += chunk_rows) {
+        const uint64_t n = rows - row0 < chunk_rows ? rows - row0 : chunk_rows;
         const half_t* xc = (const half_t*)x + row0 * cols;
         half_t* yc = (half_t*)y + row0 * cols;
-        uint64_t blocks = (n + SP_ROWS - 1) / SP_ROWS;
-        if (blocks > (uint64_t)dev->num_cus) blocks = dev->num_cus;      // one resident block per CU
-        if (full) {
-            if (nt == 2) RT_SP(2, true);
-            else if (nt == 4) RT_SP(4, true);
-            else if (nt == 8) RT_SP(8, true);
-            else RT_SP(16, true);
+        SpSched sch;
+        sch.P = (uint32_t)(mask ? period : n);
+        sch.GP = (sch.P + SP_ROWS - 1) / SP_ROWS;
+        sch.reps = (uint32_t)(n / sch.P);
+        sch.gp_div = make_fastdiv(sch.GP);
+        sch.reps_div = make_fastdiv(sch.reps);
+        const uint64_t items = (uint64_t)sch.GP * sch.reps;
+        unsigned blocks = (unsigned)(items < (uint64_t)dev->num_cus ? items : (uint64_t)dev->num_cus);      // one resident block per CU
+        // XCD-aware order: worth it when a mask row is shared by several periods and the grid splits evenly over the XCDs
+        sch.xcd = (mask && sch.reps > 1 && blocks >= 8 * SP_XCDS && sch.GP >= SP_XCDS) ? 1u : 0u;
+        if (sch.xcd) blocks = blocks / SP_XCDS * SP_XCDS;
+        if (mask) {
+            if (full) RT_SP_NS(true, true);
+            else RT_SP_NS(false, true);
         } else {
-            if (nt <= 2) RT_SP(2, false);
-            else if (nt <= 4) RT_SP(4, false);
-            else if (nt <= 8) RT_SP(8, false);
-            else RT_SP(16, false);
+            if (full) RT_SP_NS(true, false);
+            else RT_SP_NS(false, false);
         }
         RT_CHECK_LAUNCH("softmax_f16_stream_kernel");
     }
+#undef RT_SP_NS
 #undef RT_SP
+    *done = true;
     return RT_OK;
 }
 
@@ -821,9 +904,54 @@ extern "C" int rt_softmax(rt_device* dev, int dt, const void* x, void* y, uint64
         case RT_F16:
             // rows of up to 4096 columns stream through registers in one pass once there is enough work to amortise the
             // per-block table load; everything else takes the two-pass tile walker
-            if (cols % 8 == 0 && cols <= 16 * SP_TC && rows * cols >= (1u << 20) && rt_aligned(x, 16) && rt_aligned(y, 16))
-                return launch_f16_stream(dev, x, y, rows, cols);
+            if (cols % 8 == 0 && cols <= 16 * SP_TC && rows * cols >= (1u << 20) && rt_aligned(x, 16) && rt_aligned(y, 16)) {
+                bool done = false;
+                rc = launch_f16_stream(dev, x, nullptr, 0, y, rows, cols, &done);
+                if (rc || done) return rc;
+            }
             return launch_seq16<half_t>(dev, x, y, rows, cols);
         default: return launch_seq16<bf16_t>(dev, x, y, rows, cols);
     }
+}
+
+extern "C" int rt_softmax_masked(rt_device* dev, int dt, const void* x, const uint32_t x_shape[4], const void* mask,
+                                 const uint32_t mask_shape[4], void* y, int mode) {
+    RT_REQUIRE(rt_is_float_dt(dt), RT_ERR_DTYPE, "rt_softmax_masked: dtype %d is not F32/F16/BF16", dt);
+    RT_REQUIRE(mode == RT_SOFTMAX_REFERENCE || mode == RT_SOFTMAX_STABLE, RT_ERR_ARG, "rt_softmax_masked: unknown mode %d", mode);
+    RT_REQUIRE(x_shape && mask_shape, RT_ERR_NULL_POINTER, "rt_softmax_masked: NULL shape");
+    uint64_t n = 1;
+    for (int i = 0; i < 4; i++) {
+        RT_REQUIRE(x_shape[i] > 0, RT_ERR_SHAPE, "rt_softmax_masked: zero extent in dim %d", i);
+        // the add's broadcast rule with the scores as the larger side (Shape::multi_broadcast, shape.rs:118-136)
+        RT_REQUIRE(mask_shape[i] == 1 || mask_shape[i] == x_shape[i], RT_ERR_SHAPE, "rt_softmax_masked: mask dim %d: %u does not broadcast to %u",
+                   i, mask_shape[i], x_shape[i]);
+        n *= x_shape[i];
+        RT_REQUIRE(n <= RT_MAX_NUMEL, RT_ERR_SIZE, "rt_softmax_masked: tensor too large");
+    }
+    RT_REQUIRE(x && mask && y, RT_ERR_NULL_POINTER, "rt_softmax_masked: NULL operand");
+    const size_t eb = (size_t)rt_dt_bytes(dt);
+    RT_REQUIRE(rt_aligned(x, eb) && rt_aligned(y, eb) && rt_aligned(mask, eb), RT_ERR_ALIGN, "rt_softmax_masked: misaligned pointer");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    const uint32_t cols = x_shape[3];
+    const uint64_t rows = n / cols;
+    // one pass: f16, reference arithmetic, a mask that covers whole trailing dims and repeats over the leading ones
+    int lead = 0;
+    while (lead < 3 && mask_shape[lead] == 1) lead++;
+    bool whole = mask_shape[3] == cols;
+    uint64_t period = 1;
+    for (int i = lead; i < 3; i++) {
+        if (mask_shape[i] != x_shape[i]) whole = false;
+        period *= x_shape[i];
+    }
+    if (dt == RT_F16 && mode == RT_SOFTMAX_REFERENCE && whole && cols % 8 == 0 && cols <= 16 * SP_TC && rows * cols >= (1u << 20) &&
+        rt_aligned(x, 16) && rt_aligned(y, 16) && rt_aligned(mask, 16)) {
+        bool done = false;
+        rc = launch_f16_stream(dev, x, mask, period, y, rows, cols, &done);
+        if (rc || done) return rc;
+    }
+    // otherwise the two ops, the sum parked in y
+    rc = rt_binary_bcast(dev, RT_ADD, dt, x, x_shape, mask, mask_shape, y, x_shape);
+    if (rc) return rc;
+    return rt_softmax(dev, dt, y, y, rows, cols, mode);
 }

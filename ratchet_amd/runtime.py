@@ -303,6 +303,12 @@ class Device:
         check(self.lib.rt_softmax(self.handle, x.dt, x.ptr, out.ptr, x.numel // cols, cols, mode))
         return out
 
+    def softmax_masked(self, x, mask, out=None, mode=_lib.SOFTMAX_REFERENCE):
+        """softmax over the last dim of x + mask (mask broadcast over x's leading dims), in x's own arithmetic."""
+        out = out or Buffer(self, x.shape, x.dt)
+        check(self.lib.rt_softmax_masked(self.handle, x.dt, x.ptr, shape4(x.shape), mask.ptr, shape4(mask.shape), out.ptr, mode))
+        return out
+
     def layer_norm(self, x, scale, bias, eps=1e-5, out=None):
         cols = x.shape[-1]
         out = out or Buffer(self, x.shape, x.dt)

@@ -226,3 +226,47 @@ def test_group_norm(dev, oracle, B, C, L, G, dtype):
     got = dev.group_norm(dev.upload(x), G, None, None, 1e-5).to_numpy()
     bad, mx = oracle.count_not_close(got, oracle.group_norm(x, G, None, None, 1e-5), tol, tol)
     assert bad == 0, (bad, mx)
+
+
+@pytest.mark.parametrize("shape,mshape", [((1, 8, 512, 512), (512, 512)), ((2, 4, 300, 1024), (1, 1, 300, 1024)), ((1, 32, 100, 4096), (100, 4096)),
+                                          ((2, 3, 250, 1000), (2, 1, 250, 1000)), ((1, 5, 1000, 264), (1, 5, 1000, 264)),
+                                          ((1, 16, 256, 256), (1, 1, 1, 256)), ((1, 2, 40, 64), (40, 64)), ((3, 2, 1031, 512), (1031, 512))])
+def test_softmax_masked_equals_add_then_softmax(dev, oracle, shape, mshape):
+    """scores.add(mask).softmax(3) in f16: one launch where the streaming kernel applies (mask rows shared by periods of
+    whole heads, XCD-aware order), two launches otherwise; always the bits of the two separate ops."""
+    rng = np.random.default_rng(320)
+    x = randn(rng, shape, np.float16, 2.0)
+    S, T = mshape[-2], mshape[-1]
+    mask = np.zeros(mshape, np.float16)
+    m2 = mask.reshape(-1, S, T)
+    m2[:] = np.triu(np.full((S, T), -np.inf, np.float16), k=1 + max(T - S, 0)) if S > 1 else (randn(rng, (T,), np.float16) * np.float16(3))
+    m2[..., S // 2, :] = randn(rng, (T,), np.float16)                 # a finite row too: the 16-bit add must round as the separate op does
+    full_mask = np.ascontiguousarray(np.broadcast_to(mask.reshape((1,) * (4 - mask.ndim) + mask.shape), shape))
+    want = oracle.softmax(oracle.binary("add", x, full_mask))
+    dx, dm = dev.upload(x), dev.upload(mask)
+    got = dev.softmax_masked(dx, dm).to_numpy()
+    assert mismatch_count(got, want) == 0, (shape, mshape, describe_mismatch(got, want, x))
+    two = dev.softmax(dev.binary("add", dx, dm)).to_numpy()
+    assert same_bits(got, two)
+    dev.softmax_masked(dx, dm, out=dx)                                 # in place
+    assert same_bits(dx.to_numpy(), got)
+
+
+def test_softmax_masked_other_types_and_modes(dev, oracle):
+    from ratchet_amd import _lib, RatchetError
+
+    rng = np.random.default_rng(321)
+    x = randn(rng, (2, 3, 33, 200), np.float32, 2.0)
+    mask = np.triu(np.full((33, 200), -np.inf, np.float32), k=168)
+    got = dev.softmax_masked(dev.upload(x), dev.upload(mask)).to_numpy()
+    want = oracle.softmax(oracle.binary("add", x, np.ascontiguousarray(np.broadcast_to(mask, x.shape))))
+    bad, mx = oracle.count_not_close(got, want, 1e-5, 1e-5)
+    assert bad == 0, mx
+    h = x.astype(np.float16)
+    got = dev.softmax_masked(dev.upload(h), dev.upload(mask.astype(np.float16)), mode=_lib.SOFTMAX_STABLE).to_numpy()
+    ref = F.softmax(torch.from_numpy((h + mask.astype(np.float16)).astype(np.float32)), dim=-1).numpy().astype(np.float16)
+    bad, mx = oracle.count_not_close(got, ref, 1e-3, 1e-3)
+    assert bad == 0, mx
+    with pytest.raises(RatchetError) as e:
+        dev.softmax_masked(dev.upload(h), dev.upload(np.zeros((33, 100), np.float16)))
+    assert e.value.status == 4
