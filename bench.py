@@ -293,6 +293,11 @@ def one_pass_patterns(dev, seed, oracle):
     y1, y2 = dev.empty((1, H, S, S), F16), dev.empty((1, H, S, S), F16)
     nb = H * S * S * 2
     shape_cols[0] = S
+    y3 = dev.empty((1, H, S, S), F16)
+    row("add(mask) -> softmax (f16 arithmetic, bit-exact)", "[1,32,4096,4096]+[4096,4096] f16", 2 * nb + S * S * 2, 4 * nb + S * S * 2, 2,
+        lambda: dev.softmax_masked(scores, mask, out=y3),
+        lambda: (dev.binary("add", scores, mask, out=masked), dev.softmax(masked, out=y2)), y3, y2, True)
+    del y3
     row("add(mask) -> full -> softmax -> cast", "[1,32,4096,4096]+[4096,4096] f16", 2 * nb + S * S * 2, 12 * nb + S * S * 2, 4,
         lambda: dev.softmax_via_f32(scores, mask, out=y1),
         lambda: (dev.binary("add", scores, mask, out=masked), dev.cast(masked, F32, out=s32a), dev.softmax(s32a, out=s32a),

@@ -483,7 +483,7 @@ bool pattern_fusion() { return g_fuse_patterns; }
 // The graph the user built is unchanged; resolve() runs one launch at the sequence's last node and never materialises
 // the interior nodes, which must be unresolved and held by nobody but their single consumer.
 struct FusedPlan {
-    enum What { NormVia32, SoftmaxVia32, UnaryVia32, GatedMul } what;
+    enum What { NormVia32, SoftmaxVia32, UnaryVia32, GatedMul, SoftmaxMasked } what;
     Node* x = nullptr;            // 16-bit input (gate for GatedMul)
     Node* aux = nullptr;          // norm node (scale / bias / eps / kind), softmax node (mode), unary node (op)
     Node* mask = nullptr;         // SoftmaxVia32: tensor added to x before the softmax (nullptr: none)
@@ -545,6 +545,31 @@ struct Resolver {
                     plan.x = scores;
                 }
             }
+        }
+        return true;
+    }
+
+    // scores.add(mask).softmax(last dim) in one type: the add is absorbed when nobody else sees the sum
+    static bool match_masked_softmax(Node* n, FusedPlan& plan, std::vector<Node*>& inner) {
+        if (n->kind != Kind::Softmax || n->storage || n->dim != n->shape.rank() - 1) return false;
+        if (!interior(n->srcs[0], Kind::Binary)) return false;
+        Node* add = Node::of(n->srcs[0]);
+        if (add->bop != BinaryOp::Add) return false;
+        Node* scores = Node::of(add->srcs[0]);
+        const Tensor& mT = add->srcs[1];
+        Node* m = Node::of(mT);
+        if (scores->shape != add->shape || (scores->kind == Kind::Broadcast && !scores->storage)) return false;
+        plan.what = FusedPlan::SoftmaxMasked;
+        plan.aux = n;
+        plan.x = scores;
+        inner = {add};
+        if (fusable_broadcast(mT)) {
+            inner.push_back(m);
+            plan.mask = Node::of(m->srcs[0]);
+        } else if (m->kind != Kind::Broadcast || m->storage) {
+            plan.mask = m;
+        } else {
+            return false;
         }
         return true;
     }
@@ -628,6 +653,14 @@ struct Resolver {
                 check_rt(rt_softmax_via_f32(dev, dt, plan.x->storage->ptr, xs, plan.mask ? plan.mask->storage->ptr : nullptr, plan.mask ? ms : nullptr,
                                             n->storage->ptr, (int)plan.aux->mode),
                          "rt_softmax_via_f32");
+                break;
+            }
+            case FusedPlan::SoftmaxMasked: {
+                uint32_t xs[4], ms[4];
+                shape4(n->shape, xs);
+                shape4(plan.mask->shape, ms);
+                check_rt(rt_softmax_masked(dev, dt, plan.x->storage->ptr, xs, plan.mask->storage->ptr, ms, n->storage->ptr, (int)n->mode),
+                         "rt_softmax_masked");
                 break;
             }
             case FusedPlan::UnaryVia32:
@@ -821,7 +854,7 @@ struct Resolver {
                 if (n->storage || skip.count(n)) continue;
                 FusedPlan plan;
                 std::vector<Node*> inner;
-                if (match_gated(n, plan, inner) || match_via32(n, plan, inner)) {
+                if (match_gated(n, plan, inner) || match_via32(n, plan, inner) || match_masked_softmax(n, plan, inner)) {
                     fused.emplace(n, plan);
                     for (Node* i : inner) skip.insert(i);
                 }

@@ -247,6 +247,7 @@ constexpr int SP_ROWS = 30;                  // 15 loader waves x 2 rows each; w
 constexpr int SP_TC = 256;
 constexpr int SP_PAD = 8;
 constexpr int SP_PF = 4;                     // tiles loaded ahead
+constexpr int SP_MPF = 1;                    // mask tiles loaded ahead
 constexpr size_t SP_LUT_BYTES = 65536 * sizeof(uint16_t);
 constexpr size_t SP_TILE_BYTES = 2 * SP_ROWS * (SP_TC + SP_PAD) * sizeof(uint16_t);
 constexpr size_t SP_SMEM_BYTES = SP_LUT_BYTES + SP_TILE_BYTES + 2 * 32 * sizeof(uint16_t);      // 162 880 of the CU's 163 840 bytes
@@ -260,36 +261,23 @@ __device__ __forceinline__ uint32_t sp_exp_pair(const uint16_t* lut, uint32_t p)
     return (uint32_t)lut[p & 0xffffu] | ((uint32_t)lut[p >> 16] << 16);
 }
 
-// Which 30-row groups a block works on, and in which order.  Rows come in `reps` periods of P rows (P = all rows when
-// nothing repeats; P = the rows one mask covers when a mask is added, e.g. S rows per head for an [S, T] mask under
-// B * H heads); a period holds GP = ceil(P / 30) groups, none of which straddles two periods.
-//   xcd == 0: item w = block + i * grid  ->  (rep, group) = (w / GP, w % GP).
-//   xcd == 1: the hardware places block b on XCD b % 8.  XCD k takes the groups pg = k, k + 8, ... of every period and
-//             walks them repeat-fastest, so the blocks of one XCD work on the same mask rows at the same time and the
-//             XCD's L2 fetches each mask row once instead of once per head.
+// Which 30-row groups a block works on.  Rows come in `reps` periods of P rows (P = all rows when nothing repeats; P = the
+// rows one mask covers when a mask is added, e.g. S rows per head for an [S, T] mask under B * H heads); a period holds
+// GP = ceil(P / 30) groups, none of which straddles two periods.  Item w = block + i * grid -> (rep, group) = (w / GP, w % GP):
+// the blocks running at one time work on one contiguous window of x.  (An order that put all heads of one mask slab on one
+// XCD, as the broadcast add does, was measured slower here, 461 against 441 us on [1,32,4096,4096]: thirty-two streams
+// 32 MiB apart collide in the memory channels, and the mask re-reads it saves are served by the Infinity Cache anyway.)
 struct SpSched {
-    uint32_t P, GP, reps, xcd;
-    FastDiv gp_div, reps_div;
+    uint32_t P, GP, reps;
+    FastDiv gp_div;
 };
-constexpr uint32_t SP_XCDS = 8;
 
 __device__ __forceinline__ uint32_t sp_item_count(const SpSched& s, uint32_t b, uint32_t G) {
-    if (!s.xcd) {
-        const uint32_t total = s.GP * s.reps;
-        return b < total ? (total - b + G - 1) / G : 0;
-    }
-    const uint32_t k = b % SP_XCDS, j0 = b / SP_XCDS, gx = G / SP_XCDS;
-    const uint32_t total = (s.GP > k ? (s.GP - k + SP_XCDS - 1) / SP_XCDS : 0) * s.reps;
-    return j0 < total ? (total - j0 + gx - 1) / gx : 0;
+    const uint32_t total = s.GP * s.reps;
+    return b < total ? (total - b + G - 1) / G : 0;
 }
 __device__ __forceinline__ void sp_item(const SpSched& s, uint32_t b, uint32_t G, uint32_t it, uint32_t& rep, uint32_t& pg) {
-    if (!s.xcd) {
-        fd_divmod(b + it * G, s.gp_div, rep, pg);
-    } else {
-        uint32_t pgl;
-        fd_divmod(b / SP_XCDS + it * (G / SP_XCDS), s.reps_div, pgl, rep);
-        pg = pgl * SP_XCDS + b % SP_XCDS;
-    }
+    fd_divmod(b + it * G, s.gp_div, rep, pg);
 }
 
 template <int NSLOT, bool FULL, bool MASK>
@@ -370,7 +358,8 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
     const __amdgpu_buffer_rsrc_t rm =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(MASK ? mask : x), 0, MASK ? sch.P * row_bytes : nbytes, 0x00020000);
     constexpr uint32_t OOB = 0x80000000u;                    // >= nbytes, and stays so after adding a column offset
-    constexpr int PF = MASK ? 2 : (NSLOT < SP_PF ? NSLOT : SP_PF);   // tiles in flight per thread (the mask doubles the registers)
+    constexpr int PF = NSLOT < SP_PF ? NSLOT : SP_PF;        // tiles of x in flight per thread
+    constexpr int MPF = SP_MPF;                              // tiles of the mask in flight (L2 hits: a short distance is enough)
     const uint32_t G = gridDim.x;
 
     // byte offsets of (row r of item `it`, column ccol) in x / y and in the mask, or OOB
@@ -393,13 +382,14 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
     item_off(0, cur, mcur);
     item_off(1, nxt, mnxt);
     v4u e[NSLOT];                                            // exp values of the group in flight, 8 halves per slot
-    v4u pre[PF], mpre[MASK ? PF : 1];
+    v4u pre[PF], mpre[MPF];
 #pragma unroll
     for (int t = 0; t < NSLOT; t++) e[t] = v4u{0, 0, 0, 0};
 #pragma unroll
-    for (int k = 0; k < PF; k++) {
-        pre[k] = load_x(slot_off(cur, k));
-        if (MASK) mpre[k] = load_m(slot_off(mcur, k));
+    for (int k = 0; k < PF; k++) pre[k] = load_x(slot_off(cur, k));
+    if (MASK) {
+#pragma unroll
+        for (int k = 0; k < MPF; k++) mpre[k] = load_m(slot_off(mcur, k));
     }
 
     float s_prev = 1.0f, rinv_prev = 1.0f;
@@ -411,10 +401,14 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
         if (fast_prev) {
 #pragma unroll
             for (int w = 0; w < 4; w++) {
-                const float e0 = (float)bits_h((uint16_t)(ev[w] & 0xffffu)), e1 = (float)bits_h((uint16_t)(ev[w] >> 16));
-                const float a0 = e0 * rinv_prev, a1 = e1 * rinv_prev;
-                float q0 = __builtin_fmaf(__builtin_fmaf(-s_prev, a0, e0), rinv_prev, a0);
-                float q1 = __builtin_fmaf(__builtin_fmaf(-s_prev, a1, e1), rinv_prev, a1);
+                // v_fma_mix_f32 reads the f16 halves of ev[w] directly: a = e * r (+0), rem = e - s * a; no separate conversions
+                float a0, a1, m0, m1;
+                asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(a0) : "v"(ev[w]), "v"(rinv_prev));
+                asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(a1) : "v"(ev[w]), "v"(rinv_prev));
+                asm("v_fma_mix_f32 %0, -%1, %2, %3 op_sel_hi:[0,0,1]" : "=v"(m0) : "v"(s_prev), "v"(a0), "v"(ev[w]));
+                asm("v_fma_mix_f32 %0, -%1, %2, %3 op_sel:[0,0,1] op_sel_hi:[0,0,1]" : "=v"(m1) : "v"(s_prev), "v"(a1), "v"(ev[w]));
+                float q0 = __builtin_fmaf(m0, rinv_prev, a0);
+                float q1 = __builtin_fmaf(m1, rinv_prev, a1);
                 // keep the f32 quotient and its conversion apart: fused into v_fma_mixlo_f16 the pair rounds
                 // subnormal f16 results differently from fma-then-convert
                 asm volatile("" : "+v"(q0), "+v"(q1));
@@ -443,8 +437,9 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
         for (int t = 0; t < NSLOT; t++) {
             v4u& in = pre[t % PF];
             if (MASK) {                                      // scores + mask in f16, as the separate add would round it
-                const h16x8 sum = __builtin_bit_cast(h16x8, in) + __builtin_bit_cast(h16x8, mpre[t % PF]);
+                const h16x8 sum = __builtin_bit_cast(h16x8, in) + __builtin_bit_cast(h16x8, mpre[t % MPF]);
                 in = __builtin_bit_cast(v4u, sum);
+                mpre[t % MPF] = (t + MPF < NSLOT) ? load_m(slot_off(mcur, t + MPF)) : load_m(slot_off(mnxt, t + MPF - NSLOT));
             }
             // exp of the vector that arrived, parked in the LDS tile for the walk (zeros past the row end: adding +0 is a no-op;
             // rows past the tensor's end read zeros and their sums are never used)
@@ -454,13 +449,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
             if (!FULL && (uint32_t)t * SP_TC + ccol >= cols) enew = v4u{0, 0, 0, 0};
             *reinterpret_cast<v4u*>(&tile[t & 1][r][ccol]) = enew;
             // next load for this register: PF tiles ahead, possibly in the block's next group
-            if (t + PF < NSLOT) {
-                in = load_x(slot_off(cur, t + PF));
-                if (MASK) mpre[t % PF] = load_m(slot_off(mcur, t + PF));
-            } else {
-                in = load_x(slot_off(nxt, t + PF - NSLOT));
-                if (MASK) mpre[t % PF] = load_m(slot_off(mnxt, t + PF - NSLOT));
-            }
+            in = (t + PF < NSLOT) ? load_x(slot_off(cur, t + PF)) : load_x(slot_off(nxt, t + PF - NSLOT));
             __syncthreads();
             if (t == 0) read_prev_sum(gpar ^ 1);              // published by wave 0 before it reached this barrier
             const v4u out = quotients(e[t]);                  // first group: prev is OOB, the store is dropped
@@ -725,12 +714,9 @@ int launch_f16_stream(rt_device* dev, const void* x, const void* mask, uint64_t 
         sch.GP = (sch.P + SP_ROWS - 1) / SP_ROWS;
         sch.reps = (uint32_t)(n / sch.P);
         sch.gp_div = make_fastdiv(sch.GP);
-        sch.reps_div = make_fastdiv(sch.reps);
         const uint64_t items = (uint64_t)sch.GP * sch.reps;
-        unsigned blocks = (unsigned)(items < (uint64_t)dev->num_cus ? items : (uint64_t)dev->num_cus);      // one resident block per CU
-        // XCD-aware order: worth it when a mask row is shared by several periods and the grid splits evenly over the XCDs
-        sch.xcd = (mask && sch.reps > 1 && blocks >= 8 * SP_XCDS && sch.GP >= SP_XCDS) ? 1u : 0u;
-        if (sch.xcd) blocks = blocks / SP_XCDS * SP_XCDS;
+        RT_REQUIRE(items <= 0xffffffffull, RT_ERR_SIZE, "rt_softmax: too many row groups");
+        const unsigned blocks = (unsigned)(items < (uint64_t)dev->num_cus ? items : (uint64_t)dev->num_cus);   // one resident block per CU
         if (mask) {
             if (full) RT_SP_NS(true, true);
             else RT_SP_NS(false, true);

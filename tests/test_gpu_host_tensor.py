@@ -159,7 +159,7 @@ def test_phi3_style_attention_tail_graph(hdev, oracle):
                        np.float16)
     ok, info = close(oracle, y.to_numpy(), want, 1e-3)
     assert ok, info
-    assert y.last_resolve_launches() == 3
+    assert y.last_resolve_launches() == 2                            # add + softmax go through one call, then the cast
     gate = rng.standard_normal((1, 64, 512)).astype(np.float16)
     up = rng.standard_normal((1, 64, 512)).astype(np.float16)
     z = T(up, hdev).mul(T(gate, hdev).full().silu().cast(_lib.F16)).resolve().to_numpy()
@@ -230,11 +230,12 @@ def test_caller_patterns_resolve_in_one_launch(hdev, oracle):
         ln = T(x, hdev).full().layer_norm(T(w, hdev), T(b, hdev), 1e-5).cast(F16)
         rms = T(x, hdev).full().rms_norm(T(w, hdev), 1e-5).cast(F16)
         attn = T(scores, hdev).add(T(mask, hdev)).full().softmax(3).cast(F16)
+        attn16 = T(scores, hdev).add(T(mask, hdev)).softmax(3)
         act = T(x, hdev).full().gelu().cast(F16)
         p = T(proj, hdev)
         gate, up = p.slice([(0, 1), (0, 64), (0, 512)]), p.slice([(0, 1), (0, 64), (512, 1024)])
         glu = up.mul(gate.full().silu().cast(F16))
-        return {"ln": ln, "rms": rms, "attn": attn, "act": act, "glu": glu}
+        return {"ln": ln, "rms": rms, "attn": attn, "attn16": attn16, "act": act, "glu": glu}
 
     set_pattern_fusion(False)
     try:
@@ -242,9 +243,9 @@ def test_caller_patterns_resolve_in_one_launch(hdev, oracle):
     finally:
         set_pattern_fusion(True)
     fused = {k: (g.resolve().to_numpy(), g.last_resolve_launches()) for k, g in graphs().items()}
-    assert {k: v[1] for k, v in plain.items()} == {"ln": 3, "rms": 3, "attn": 4, "act": 3, "glu": 6}
-    assert {k: v[1] for k, v in fused.items()} == {"ln": 1, "rms": 1, "attn": 1, "act": 1, "glu": 1}
-    for k in ("act", "glu"):
+    assert {k: v[1] for k, v in plain.items()} == {"ln": 3, "rms": 3, "attn": 4, "attn16": 2, "act": 3, "glu": 6}
+    assert {k: v[1] for k, v in fused.items()} == {"ln": 1, "rms": 1, "attn": 1, "attn16": 1, "act": 1, "glu": 1}
+    for k in ("act", "glu", "attn16"):
         assert same_bits(fused[k][0], plain[k][0]), k
     for k in ("ln", "rms", "attn"):
         ok, info = close(oracle, fused[k][0], plain[k][0], 1e-3)

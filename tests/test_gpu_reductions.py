@@ -232,8 +232,8 @@ def test_group_norm(dev, oracle, B, C, L, G, dtype):
                                           ((2, 3, 250, 1000), (2, 1, 250, 1000)), ((1, 5, 1000, 264), (1, 5, 1000, 264)),
                                           ((1, 16, 256, 256), (1, 1, 1, 256)), ((1, 2, 40, 64), (40, 64)), ((3, 2, 1031, 512), (1031, 512))])
 def test_softmax_masked_equals_add_then_softmax(dev, oracle, shape, mshape):
-    """scores.add(mask).softmax(3) in f16: one launch where the streaming kernel applies (mask rows shared by periods of
-    whole heads, XCD-aware order), two launches otherwise; always the bits of the two separate ops."""
+    """scores.add(mask).softmax(3) in f16: one launch where the streaming kernel applies (a mask shared by periods of whole
+    heads), two launches otherwise; always the bits of the two separate ops."""
     rng = np.random.default_rng(320)
     x = randn(rng, shape, np.float16, 2.0)
     S, T = mshape[-2], mshape[-1]
