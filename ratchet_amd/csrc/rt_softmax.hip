@@ -475,16 +475,14 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
 // on 16-bit scores in one pass: the mask (broadcast over batch / heads, optional) is added in the 16-bit type as the
 // separate add would, the sum is widened, the f32 softmax above is applied in registers and the result rounded once.
 // 4 bytes of HBM traffic per element against 26 for the four separate ops (6 + 6 + 8 + 6).
-// Blocks take the XCD-aware order of binary_bcast_kernel so that the heads sharing a mask row run on one XCD.
+// (Ordering the blocks so that the heads sharing a mask row run on one XCD, as binary_bcast_kernel does, changed nothing
+// here: 380 us either way on [1,32,4096,4096]; the mask re-reads are served by the Infinity Cache.)
 // ------------------------------------------------------------------------------------------------------------------
 struct MaskArgs {
     FastDiv d2, d1;          // x extents of dims 2 and 1 (rows = d0 * d1 * d2)
     uint32_t ms[3];          // mask row strides in elements over dims 0..2 (0 where the mask extent is 1)
     uint32_t mlast;          // 1: the mask has a full last dim, 0: one value per row
-    FastDiv reps;            // XCD-aware order (see BcastArgs in the elementwise kernels); slabs == 0: identity
-    uint32_t slabs;
 };
-constexpr uint32_t SM_XCDS = 8;
 
 template <typename T> __device__ __forceinline__ uint64_t mask_row_offset(uint64_t row, const MaskArgs& p) {
     uint32_t t, i2, i1, i0;
@@ -502,13 +500,7 @@ __device__ __forceinline__ float via32_exp(float v) { return __builtin_amdgcn_ex
 template <typename T, int NV, int MODE, bool MASK, int LANES>
 __global__ void __launch_bounds__(BLOCK) softmax_via32_wave_kernel(const T* __restrict__ x, const T* __restrict__ mask,
                                                                    T* __restrict__ y, uint64_t rows, uint32_t cols, MaskArgs p) {
-    uint32_t blk = blockIdx.x;
-    if (MASK && p.slabs) {
-        uint32_t rep, grp;
-        fd_divmod(blk / SM_XCDS, p.reps, grp, rep);
-        blk = rep * p.slabs + grp * SM_XCDS + (blk % SM_XCDS);
-    }
-    const uint64_t row = (uint64_t)blk * (BLOCK / LANES) + (threadIdx.x / LANES);
+    const uint64_t row = (uint64_t)blockIdx.x * (BLOCK / LANES) + (threadIdx.x / LANES);
     if (row >= rows) return;
     const int lane = threadIdx.x & (LANES - 1);
     const uint32_t nvec = cols / 8;
@@ -770,14 +762,12 @@ int launch_via32(rt_device* dev, const void* x, const void* mask, void* y, uint6
         return RT_OK;
     }
     if (vec_ok) {                                            // rows of up to 16384 columns: the block shares the row
-        MaskArgs q = p;
-        q.slabs = 0;                                         // the XCD-aware order is laid out for four rows per block
         const uint32_t nv = (nvec + BLOCK - 1) / BLOCK;
         RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax_via_f32: too many rows");
         const dim3 grid((unsigned)rows), block(BLOCK);
 #define RT_SV(NVC)                                                                                                                  \
     hipLaunchKernelGGL((softmax_via32_wave_kernel<T, NVC, MODE, MASK, BLOCK>), grid, block, 0, dev->stream, (const T*)x, (const T*)mask, \
-                       (T*)y, rows, cols, q)
+                       (T*)y, rows, cols, p)
         if (nv <= 3) RT_SV(3);
         else if (nv <= 4) RT_SV(4);
         else if (nv <= 6) RT_SV(6);
@@ -833,8 +823,6 @@ extern "C" int rt_softmax_via_f32(rt_device* dev, int io_dt, const void* x, cons
     p.d1 = make_fastdiv(x_shape[1]);
     p.ms[0] = p.ms[1] = p.ms[2] = 0;
     p.mlast = 0;
-    p.reps = make_fastdiv(1);
-    p.slabs = 0;
     bool mask_vec_ok = true;
     if (mask) {
         uint64_t st = 1;
@@ -846,22 +834,6 @@ extern "C" int rt_softmax_via_f32(rt_device* dev, int io_dt, const void* x, cons
             st *= mask_shape[i];
         }
         mask_vec_ok = !p.mlast || (rt_aligned(mask, 16) && cols % 8 == 0);
-        // a mask repeated over the leading dims and larger than an XCD's L2 keeps comfortably: XCD-aware block order
-        int lead = 0;
-        while (lead < 3 && mask_shape[lead] == 1) lead++;
-        bool prefix = lead > 0;
-        uint64_t reps = 1, inner_rows = 1;
-        for (int i = 0; i < 3; i++) {
-            if (i < lead) reps *= x_shape[i];
-            else {
-                inner_rows *= x_shape[i];
-                if (mask_shape[i] != x_shape[i]) prefix = false;
-            }
-        }
-        if (prefix && p.mlast && reps > 1 && inner_rows * cols * 2 >= (1u << 20) && inner_rows % (WAVES * SM_XCDS) == 0) {
-            p.reps = make_fastdiv((uint32_t)reps);
-            p.slabs = (uint32_t)(inner_rows / WAVES);
-        }
     }
     if (io_dt == RT_F16) return dispatch_via32<half_t>(dev, x, mask, y, rows, cols, p, mask_vec_ok, mode);
     return dispatch_via32<bf16_t>(dev, x, mask, y, rows, cols, p, mask_vec_ok, mode);
