@@ -17,6 +17,8 @@
 //   (one dependent add per element), so many small row groups run side by side.
 // GroupNorm follows torch.nn.functional.group_norm, the ground truth of the reference's own test
 // (ops/norm/groupnorm.rs:24-31): statistics in f32 (Chan-combined partial mean/M2), f32 arithmetic, one final rounding.
+#include <type_traits>
+
 #include "rt_arith.h"
 #include "rt_internal.h"
 
@@ -677,6 +679,69 @@ int norm_entry(rt_device* dev, int kind, int dt, const void* x, const void* scal
     }
 }
 
+// Few, small groups (the latency-bound case: 32 groups of 96 KB in the reference's Whisper-style shape): one launch, one
+// 1024-thread block per (batch, group), the group staged in LDS once, then mean, squared deviations and the output all
+// come from LDS.  Same definitions as the two-kernel path (mean, then the variance about that mean, f32 arithmetic).
+constexpr int GN_LDS_BLOCK = 1024;
+constexpr size_t GN_LDS_MAX_BYTES = 144 * 1024;
+
+template <typename T>
+__global__ void __launch_bounds__(GN_LDS_BLOCK) gn_lds_kernel(const T* __restrict__ x, const T* __restrict__ scale, const T* __restrict__ bias,
+                                                              T* __restrict__ y, uint32_t glen, uint32_t cpg, uint32_t groups, FastDiv L,
+                                                              float eps) {
+    constexpr int VE = 16 / sizeof(T);
+    extern __shared__ __attribute__((aligned(16))) unsigned char gn_smem[];
+    v4u* stage = reinterpret_cast<v4u*>(gn_smem);
+    const uint32_t grp = blockIdx.x, g = grp % groups;
+    const v4u* xs = reinterpret_cast<const v4u*>(x + (uint64_t)grp * glen);
+    v4u* ys = reinterpret_cast<v4u*>(y + (uint64_t)grp * glen);
+    const uint32_t nvec = glen / VE;
+    float acc = 0.0f;
+    for (uint32_t i0 = threadIdx.x; i0 < nvec; i0 += GN_LDS_BLOCK * 8) {    // eight loads in flight per thread
+        Vec16<T> v[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const uint32_t i = i0 + k * GN_LDS_BLOCK;
+            if (i < nvec) v[k].u = ld_stream(xs + i);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const uint32_t i = i0 + k * GN_LDS_BLOCK;
+            if (i < nvec) {
+                stage[i] = v[k].u;
+#pragma unroll
+                for (int q = 0; q < VE; q++) acc += Ar<T>::widen(v[k].e[q]);
+            }
+        }
+    }
+    const float mean = row_sum<GN_LDS_BLOCK>(acc) / (float)glen;
+    float m2 = 0.0f;
+    for (uint32_t i = threadIdx.x; i < nvec; i += GN_LDS_BLOCK) {           // a thread re-reads what it wrote itself
+        Vec16<T> v;
+        v.u = stage[i];
+#pragma unroll
+        for (int q = 0; q < VE; q++) {
+            const float d = Ar<T>::widen(v.e[q]) - mean;
+            m2 += d * d;
+        }
+    }
+    const float var = row_sum<GN_LDS_BLOCK>(m2) / (float)glen;
+    const float rstd = 1.0f / __builtin_sqrtf(var + eps);
+    for (uint32_t i = threadIdx.x; i < nvec; i += GN_LDS_BLOCK) {
+        const uint32_t c = g * cpg + fd_div(i * VE, L);                      // L % VE == 0: one channel per vector
+        const float w = scale ? Ar<T>::widen(scale[c]) : 1.0f;
+        const float b = bias ? Ar<T>::widen(bias[c]) : 0.0f;
+        Vec16<T> v, o;
+        v.u = stage[i];
+#pragma unroll
+        for (int q = 0; q < VE; q++) {
+            const float t = (Ar<T>::widen(v.e[q]) - mean) * rstd;
+            o.e[q] = Ar<T>::conv(t * w + b);
+        }
+        st_stream(ys + i, o.u);
+    }
+}
+
 template <typename T>
 int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint32_t bg, uint32_t glen, uint32_t cpg,
               uint32_t groups, uint32_t L, float eps) {
@@ -688,6 +753,18 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
     if (splits < 1) splits = 1;
     constexpr int VEMAX = 16 / sizeof(T);
     const bool vec = (L % VEMAX == 0) && rt_aligned(x, 16) && rt_aligned(y, 16);       // then glen % VEMAX == 0 too
+    if (vec && (size_t)glen * sizeof(T) <= GN_LDS_MAX_BYTES && bg <= 2u * (uint32_t)dev->num_cus) {
+        const int ti = sizeof(T) == 4 ? 0 : (std::is_same<T, half_t>::value ? 1 : 2);
+        if (!(dev->gn_lds_attr_set & (1u << ti))) {
+            RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gn_lds_kernel<T>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)GN_LDS_MAX_BYTES));
+            dev->gn_lds_attr_set |= 1u << ti;
+        }
+        hipLaunchKernelGGL((gn_lds_kernel<T>), dim3(bg), dim3(GN_LDS_BLOCK), (size_t)glen * sizeof(T), dev->stream, (const T*)x, (const T*)scale,
+                           (const T*)bias, (T*)y, glen, cpg, groups, make_fastdiv(L), eps);
+        RT_CHECK_LAUNCH("gn_lds_kernel");
+        return RT_OK;
+    }
     uint32_t chunk = (glen + splits - 1) / splits;
     if (vec) chunk = (chunk + VEMAX - 1) / VEMAX * VEMAX;                               // slices start on vector boundaries
     splits = (glen + chunk - 1) / chunk;

@@ -207,7 +207,11 @@ def test_layer_norm_variance_form_matches_reference(dev, oracle):
     assert np.nanmax(np.abs(got - want)) < np.nanmax(np.abs(two_pass - want)) or np.allclose(two_pass, want, atol=1e-4)
 
 
-@pytest.mark.parametrize("B,C,L,G", [(1, 3, 1, 1), (2, 8, 5, 4), (1, 6, 7, 6), (3, 4, 9, 1), (1, 64, 3000, 32), (2, 32, 17, 8)])
+@pytest.mark.parametrize("B,C,L,G", [(1, 3, 1, 1), (2, 8, 5, 4), (1, 6, 7, 6), (3, 4, 9, 1), (1, 64, 3000, 32), (2, 32, 17, 8),
+                                     (1, 512, 3000, 32),          # the benchmark shape: 32 groups of 96 KB, staged in LDS, one launch
+                                     (9, 128, 40, 64),            # 576 groups: more than two per CU, the two-launch streaming path
+                                     (1, 8, 40000, 2),            # groups larger than LDS
+                                     (2, 16, 24, 4)])
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
 def test_group_norm(dev, oracle, B, C, L, G, dtype):
     rng = np.random.default_rng(320)
