@@ -231,8 +231,8 @@ __global__ void __launch_bounds__(BLOCK) softmax_seq16_kernel(const T* __restric
 // known, so x is read once and y written once.
 //   exp: a 16-bit type has 65536 values; the whole exact exp table (128 KiB) sits in LDS next to the 31 KiB of tiles
 //        (162 880 of the CU's 163 840 bytes), so exp is one ds_read_u16 per element with the bit pattern as the index:
-//        no range clamping, no NaN special case.  The kernel is bound by vector instruction issue as much as by HBM
-//        (removing two of ~16 VALU instructions per element moved it by 10 %), which is why the index math was cut.
+//        no range clamping, no NaN special case.  (With a 75 KiB table of the unsaturated range and clamping index math
+//        the kernel was bound by vector instruction issue, 16.5 VALU instructions per element; it is not any more.)
 //   sum: per 256-column tile the exp values also go to an LDS tile (double buffered); lanes 0..29 of wave 0 each walk
 //        one row of the tile left to right with dependent v_add_f16 (3 ns each on this chip).  A tile is 16 KiB in and
 //        15 KiB out of HBM per CU, about 1 us at a CU's share of 8 TB/s; the walk of 256 columns takes 0.8 us, which is
@@ -240,7 +240,10 @@ __global__ void __launch_bounds__(BLOCK) softmax_seq16_kernel(const T* __restric
 //   divide: the outputs of group g are produced while group g+1 streams in: y = e / sum with the quotient computed as
 //        q0 = e * (1/sum) plus one fma correction, which is the correctly rounded f16 quotient for normal finite sums
 //        (checked against IEEE division over operand pairs on the GPU); other sums take the IEEE path.
-// Global loads run two tiles ahead across group boundaries, so the pipeline never drains.
+//   mask: with MASK, a second operand (one [P, cols] block shared by every period of P rows, e.g. an [S, T] attention
+//        mask under B * H heads) is added to x in f16 as the vectors arrive: scores.add(mask).softmax() without the sum
+//        ever reaching memory, bit-identical to the two separate ops.
+// Global loads run SP_PF tiles ahead across group boundaries, so the pipeline never drains.
 // ------------------------------------------------------------------------------------------------------------------
 constexpr int SP_BLOCK = 1024;
 constexpr int SP_ROWS = 30;                  // 15 loader waves x 2 rows each; wave 0 only walks
