@@ -19,6 +19,7 @@ SOFTMAX_REFERENCE, SOFTMAX_STABLE = 0, 1
 STATUS_NAMES = {
     0: "RT_OK", 1: "RT_ERR_NULL_POINTER", 2: "RT_ERR_DTYPE", 3: "RT_ERR_OP", 4: "RT_ERR_SHAPE", 5: "RT_ERR_PERM",
     6: "RT_ERR_SIZE", 7: "RT_ERR_ARG", 8: "RT_ERR_NULL_DEVICE", 9: "RT_ERR_ALIGN",
+    10: "RT_ERR_CAPTURE",
 }
 
 EXPORTS = [

@@ -14,6 +14,21 @@ from ratchet_amd.host import HostError, Tensor
 F32, F16 = _lib.F32, _lib.F16
 
 
+def test_host_header_and_library_agree():
+    import os
+    import re
+
+    from ratchet_amd import host
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    header = open(os.path.join(root, "include", "ratchet_host.h")).read()
+    declared = sorted(set(re.findall(r"\b(rth_[a-z0-9_]+)\(", header)))
+    assert len(declared) > 30
+    H = host.load()
+    for name in declared:
+        assert hasattr(H, name), f"{name} is declared in ratchet_host.h but not exported by libratchet_host.so"
+
+
 def P(*shape, dt=F32):
     return Tensor.placeholder(shape, dt)
 
