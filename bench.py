@@ -305,6 +305,56 @@ def one_pass_patterns(dev, seed, oracle):
     return out
 
 
+def decode_step(dev, seed):
+    """A launch-bound sequence, reported beside the step: the memory-bound ops of one Phi-2-sized decode layer (one token,
+    2047 tokens already in the KV cache) launched one by one, and the same sequence replayed from a HIP graph."""
+    np16, np32 = np.float16, np.float32
+    H, D, N, T = 32, 80, 2560, 2047
+    table = dev.upload(normal(seed, 951, (4096, N), 1.0, np16))
+    ids = dev.upload(np.array([1234], np.int32))
+    w32, b32 = dev.upload(normal(seed, 952, (N,), 0.02, np32, mean=1.0)), dev.upload(normal(seed, 953, (N,), 0.02, np32))
+    x, h = dev.empty((1, N), F16), dev.empty((1, N), F16)
+    q, k, v = (dev.upload(normal(seed, 954 + i, (1, H, 1, D), 1.0, np16)) for i in range(3))
+    kc, vc = dev.empty((1, H, 2048, D), F16).zero_(), dev.empty((1, H, 2048, D), F16).zero_()
+    kd, vd = dev.empty((1, H, T + 1, D), F16), dev.empty((1, H, T + 1, D), F16)
+    scores = dev.upload(normal(seed, 957, (1, H, 1, T + 1), 2.0, np16))
+    probs = dev.empty((1, H, 1, T + 1), F16)
+    ff = dev.upload(normal(seed, 958, (1, 4 * N), 1.0, np16))
+    act, res = dev.empty((1, 4 * N), F16), dev.empty((1, N), F16)
+
+    def seq():
+        dev.index_select(table, ids, 0, out=x)                       # embedding row
+        dev.norm_via_f32("layer", x, w32, b32, 1e-5, out=h)          # input LayerNorm (full -> layer_norm -> cast)
+        dev.rope(q, 32, 10000.0, T, out=q)                           # rotary on q and k, in place
+        dev.rope(k, 32, 10000.0, T, out=k)
+        dev.cache(kc, k, 2, T, out=kd)                               # KV append
+        dev.cache(vc, v, 2, T, out=vd)
+        dev.softmax_via_f32(scores, None, out=probs)                 # attention weights over 2048 keys
+        dev.unary_via_f32("gelu", ff, out=act)                       # MLP activation
+        dev.binary("add", x, h, out=res)                             # residual
+
+    n_ops = 9
+    seq()
+    dev.sync()
+
+    def timed(fn, n=200):
+        dev.sync()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        dev.sync()
+        return (time.perf_counter() - t0) / n * 1e6
+
+    eager = timed(seq)
+    with dev.capture() as g:
+        seq()
+    g.launch()
+    replay = timed(g.launch)
+    return {"sequence": "index_select, layer_norm(via f32), rope x2, cache x2, softmax(via f32), gelu(via f32), add at Phi-2 decode shapes",
+            "launches": n_ops, "eager_us": round(eager, 1), "graph_replay_us": round(replay, 1),
+            "note": "eager = nine calls through ctypes on the device's stream; replay = one hipGraphLaunch of the captured sequence"}
+
+
 def download_rows(dev, buf, nrows, row_elems, np_dtype):
     """first nrows rows (row_elems each) of a device buffer"""
     import ctypes
@@ -489,6 +539,7 @@ def main():
 
     ceiling = copy_ceiling(dev) if not args.ops else None      # after the parity check: it overwrites an output buffer
     patterns = one_pass_patterns(dev, seed, oracle if not args.no_check else None) if not (args.ops or args.no_patterns) else None
+    decode = decode_step(dev, seed) if not (args.ops or args.no_patterns) else None
 
     rows = []
     for o in ops:
@@ -524,6 +575,7 @@ def main():
             "host_cpus": os.cpu_count()},
         "hbm_copy_ceiling": ceiling,
         "one_pass_patterns": patterns,
+        "decode_step": decode,
         "parity_ok": bool(parity_ok) if not args.no_check else None,
         "ops": rows,
         "wall_s": round(wall, 3), "setup_s": round(t_setup, 2),
