@@ -272,6 +272,7 @@ __device__ __forceinline__ uint32_t sp_exp_pair(const uint16_t* lut, uint32_t p)
 // 32 MiB apart collide in the memory channels, and the mask re-reads it saves are served by the Infinity Cache anyway.)
 struct SpSched {
     uint32_t P, GP, reps;
+    uint32_t R;              // rows per group actually used (<= SP_ROWS): chosen so that the groups fill whole rounds of the grid
     FastDiv gp_div;
 };
 
@@ -369,8 +370,8 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
     auto item_off = [&](uint32_t it, uint32_t& xo, uint32_t& mo) {
         uint32_t rep, pg;
         sp_item(sch, blockIdx.x, G, it, rep, pg);
-        const uint32_t prow = pg * SP_ROWS + r;              // row inside the period
-        const bool ok = it < n_items && prow < sch.P;
+        const uint32_t prow = pg * sch.R + r;                // row inside the period
+        const bool ok = it < n_items && r < sch.R && prow < sch.P;
         mo = ok ? prow * row_bytes + ccol * 2 : OOB;
         xo = ok ? (rep * sch.P + prow) * row_bytes + ccol * 2 : OOB;
     };
@@ -706,8 +707,24 @@ int launch_f16_stream(rt_device* dev, const void* x, const void* mask, uint64_t 
         half_t* yc = (half_t*)y + row0 * cols;
         SpSched sch;
         sch.P = (uint32_t)(mask ? period : n);
-        sch.GP = (sch.P + SP_ROWS - 1) / SP_ROWS;
         sch.reps = (uint32_t)(n / sch.P);
+        // rows per group: every block runs ceil(groups / grid) rounds of 16-or-fewer tile steps whatever the group holds, so
+        // 4370 groups of 30 rows on 256 CUs cost 18 rounds where 17.07 are needed; 27-row groups make 19 full rounds.
+        // Pick the size that minimises rounds x rows (time is proportional to the rows a round could have carried).
+        {
+            uint64_t best = ~0ull;
+            sch.R = SP_ROWS;
+            for (uint32_t R = SP_ROWS; R >= SP_ROWS - 6; R--) {
+                const uint64_t groups = (uint64_t)((sch.P + R - 1) / R) * sch.reps;
+                const uint64_t rounds = (groups + dev->num_cus - 1) / dev->num_cus;
+                const uint64_t cost = rounds * R + rounds / 4;          // the small second term: a round has a fixed cost too
+                if (cost < best) {
+                    best = cost;
+                    sch.R = R;
+                }
+            }
+        }
+        sch.GP = (sch.P + sch.R - 1) / sch.R;
         sch.gp_div = make_fastdiv(sch.GP);
         const uint64_t items = (uint64_t)sch.GP * sch.reps;
         RT_REQUIRE(items <= 0xffffffffull, RT_ERR_SIZE, "rt_softmax: too many row groups");
