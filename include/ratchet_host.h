@@ -26,6 +26,8 @@ const char* rth_last_error_kind(void);
 
 rth_device* rth_device_request(int ordinal);                          /* Device::request_device (device.rs:61-77) */
 void rth_device_release(rth_device* dev);
+/* {bytes handed out, bytes parked in the pool, requests served by the pool, requests passed to the driver} (rt_pool_stats) */
+int rth_pool_stats(rth_device* dev, uint64_t out[4]);
 
 /* Tensor::from_data + to(device) (tensor.rs:553-571,874-892); dt codes as in ratchet_hip.h */
 rth_tensor* rth_from_host(rth_device* dev, const void* data, int rank, const uint64_t* shape, int dt);

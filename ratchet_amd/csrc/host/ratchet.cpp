@@ -844,7 +844,22 @@ struct Resolver {
 
     static void resolve(Node* root) {
         size_t launches = 0;
-        const std::vector<Node*> order = execution_order(root);
+        const std::vector<Node*> full_order = execution_order(root);
+        // only what the root still needs: nothing below a tensor that already has its storage (tensor.rs:783 skips those;
+        // their own inputs may have given their buffers back, see below)
+        std::unordered_set<Node*> needed;
+        {
+            std::vector<Node*> todo{root};
+            while (!todo.empty()) {
+                Node* n = todo.back();
+                todo.pop_back();
+                if (!needed.insert(n).second || n->storage) continue;
+                for (const Tensor& s : n->srcs) todo.push_back(Node::of(s));
+            }
+        }
+        std::vector<Node*> order;
+        for (Node* n : full_order)
+            if (needed.count(n)) order.push_back(n);
         std::unordered_set<Node*> skip;
         // caller patterns, consumers first so that the longest sequence wins (the gated multiply contains a unary one)
         std::unordered_map<Node*, FusedPlan> fused;
@@ -865,11 +880,55 @@ struct Resolver {
             if (n->kind == Kind::Binary && !n->storage && !skip.count(n) && !fused.count(n))
                 for (const Tensor& s : n->srcs)
                     if (fusable_broadcast(s)) skip.insert(Node::of(s));
+
+        // Liveness, the job of the reference's allocation planner (gpu/buffer_allocator/allocator.rs:141-271): an
+        // intermediate that nobody outside this graph can see gives its buffer back to the device's pool right after the
+        // last launch that reads it, so a long graph holds a few live buffers instead of one per node.  Launches run in
+        // stream order, which makes the hand-over safe without waiting.
+        std::unordered_map<Node*, size_t> index_of, edges, last_use;
+        std::unordered_map<Node*, Node*> consumer;                 // of a skipped node: the one node that absorbs it
+        for (size_t i = 0; i < order.size(); i++) index_of[order[i]] = i;
         for (Node* n : order) {
-            if (n->storage || skip.count(n)) continue;         // already resolved (tensor.rs:783) or fused away
-            auto f = fused.find(n);
-            if (f != fused.end()) run_fused(n, f->second, launches);
-            else run(n, launches);
+            if (n->storage) continue;                              // a resolved node reads nothing
+            for (const Tensor& s : n->srcs) {
+                edges[Node::of(s)]++;
+                consumer[Node::of(s)] = n;
+            }
+        }
+        auto exec_index = [&](Node* n) {
+            while (skip.count(n)) n = consumer.at(n);
+            return index_of.at(n);
+        };
+        std::vector<std::vector<Node*>> release_at(order.size());
+        for (Node* n : order) {
+            if (n->storage) continue;
+            for (const Tensor& s : n->srcs) {
+                Node* src = Node::of(s);
+                const size_t at = exec_index(n);
+                auto it = last_use.find(src);
+                if (it == last_use.end() || it->second < at) last_use[src] = at;
+            }
+        }
+        for (Node* n : order) {
+            if (n->storage) continue;
+            for (const Tensor& s : n->srcs) {
+                Node* src = Node::of(s);
+                // every holder of the node is an edge of this graph: no user handle, no other graph
+                if (src != root && !src->srcs.empty() && (size_t)Node::holders(s) == edges[src] && last_use.count(src)) {
+                    release_at[last_use[src]].push_back(src);
+                    last_use.erase(src);
+                }
+            }
+        }
+
+        for (size_t i = 0; i < order.size(); i++) {
+            Node* n = order[i];
+            if (!n->storage && !skip.count(n)) {                   // else: already resolved or fused away
+                auto f = fused.find(n);
+                if (f != fused.end()) run_fused(n, f->second, launches);
+                else run(n, launches);
+            }
+            for (Node* dead : release_at[i]) dead->storage.reset();
         }
         check_rt(rt_sync(root->device.raw()), "rt_sync");      // resolve returns after completion (tensor.rs:855-856)
         root->last_launches = launches;

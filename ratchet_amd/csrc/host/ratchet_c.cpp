@@ -5,6 +5,7 @@
 
 #include "../../../include/ratchet_host.h"
 #include "ratchet.hpp"
+#include "../../../include/ratchet_hip.h"
 
 using namespace ratchet;
 
@@ -49,6 +50,9 @@ rth_device* rth_device_request(int ordinal) {
     }
 }
 void rth_device_release(rth_device* dev) { delete dev; }
+int rth_pool_stats(rth_device* dev, uint64_t out[4]) {
+    return rt_pool_stats(dev->dev.raw(), &out[0], &out[1], &out[2], &out[3]);
+}
 
 rth_tensor* rth_from_host(rth_device* dev, const void* data, int rank, const uint64_t* shape, int dt) {
     return build([&] { return Tensor::from_host(data, make_shape(rank, shape), (DType)dt, dev->dev); });

@@ -69,6 +69,8 @@ def load():
     H.rth_last_resolve_launches.restype = ctypes.c_long
     H.rth_id.argtypes = [vp]
     H.rth_id.restype = ctypes.c_uint64
+    H.rth_pool_stats.argtypes = [vp, u64p]
+    H.rth_pool_stats.restype = i
     H.rth_set_pattern_fusion.argtypes = [i]
     H.rth_set_pattern_fusion.restype = None
     _h = H
@@ -96,6 +98,13 @@ class HostDevice:
         self.handle = self.H.rth_device_request(ordinal)
         if not self.handle:
             _raise()
+
+    def pool_stats(self):
+        """(bytes handed out, bytes parked for reuse, requests served by the pool, requests passed to hipMalloc)"""
+        out = (ctypes.c_uint64 * 4)()
+        if self.H.rth_pool_stats(self.handle, out) != 0:
+            _raise()
+        return tuple(int(v) for v in out)
 
     def close(self):
         if self.handle:

@@ -301,3 +301,41 @@ def test_rope_index_select_index_write_graphs(hdev, oracle):
     out = dst.index_write(T(np.array([[7, 8]], np.float32), hdev), [2, 0]).resolve()
     assert np.array_equal(out.to_numpy(), np.array([[1, 2], [3, 4], [7, 8]], np.float32))
     assert np.array_equal(dst.to_numpy(), out.to_numpy())                      # in place: the destination's buffer is the result
+
+
+def test_intermediates_return_their_buffers_during_resolve(oracle):
+    """What the reference's allocation planner achieves (gpu/buffer_allocator/allocator.rs:141-271): a long graph holds a few
+    live buffers, not one per node.  Twelve alternating casts of an 8 MiB tensor (Cast never runs in place) need three
+    buffers from the driver, not twelve, and only the result stays allocated afterwards."""
+    from ratchet_amd import _lib
+    from ratchet_amd.host import HostDevice, set_pattern_fusion
+
+    d = HostDevice(0)
+    try:
+        rng = np.random.default_rng(409)
+        x = rng.standard_normal((1024, 4096)).astype(np.float16)
+        tx = T(x, d)
+        live0, _, _, misses0 = d.pool_stats()
+        set_pattern_fusion(False)                               # keep all twelve casts as launches
+        try:
+            y = tx
+            for _ in range(6):
+                y = y.full().half()
+            y.resolve()
+        finally:
+            set_pattern_fusion(True)
+        assert y.last_resolve_launches() == 12
+        assert same_bits(y.to_numpy(), x)
+        live, parked, _, misses = d.pool_stats()
+        assert misses - misses0 <= 3, misses - misses0
+        assert live - live0 == x.nbytes                         # the result; every intermediate is back in the pool
+        # a tensor the caller still holds keeps its buffer
+        mid = tx.full()
+        z = mid.neg().half().resolve()
+        assert mid.resolved() and same_bits(mid.to_numpy(), x.astype(np.float32))
+        assert same_bits(z.to_numpy(), oracle.cast(oracle.unary("neg", x.astype(np.float32)), np.float16))
+        # a resolved tensor whose inputs were released can still be built upon
+        w = y.full().neg().half().resolve()
+        assert same_bits(w.to_numpy(), (-x.astype(np.float32)).astype(np.float16))
+    finally:
+        d.close()
