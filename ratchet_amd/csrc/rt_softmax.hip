@@ -223,37 +223,39 @@ __global__ void __launch_bounds__(BLOCK) softmax_seq16_kernel(const T* __restric
 }
 
 // ------------------------------------------------------------------------------------------------------------------
-// f16 reference arithmetic, single pass over HBM (cols <= NSLOT * 256, cols % 8 == 0, 16-byte aligned).
+// f16 reference arithmetic, single pass over HBM (cols <= NSTEP * 512, cols % 8 == 0, 16-byte aligned).
 //
-// One 1024-thread block per CU walks over groups of 30 rows.  Wave 0 does nothing but the sequential sums; in the other
-// 15 waves thread (r, cv) owns the 16-byte vectors at columns
-// t*256 + cv*8 of row r, t = 0..NSLOT-1, and keeps their exp values in registers (NSLOT * 4 VGPRs) until the row sum is
-// known, so x is read once and y written once.
-//   exp: a 16-bit type has 65536 values; the whole exact exp table (128 KiB) sits in LDS next to the 31 KiB of tiles
-//        (162 880 of the CU's 163 840 bytes), so exp is one ds_read_u16 per element with the bit pattern as the index:
-//        no range clamping, no NaN special case.  (With a 75 KiB table of the unsaturated range and clamping index math
-//        the kernel was bound by vector instruction issue, 16.5 VALU instructions per element; it is not any more.)
-//   sum: per 256-column tile the exp values also go to an LDS tile (double buffered); lanes 0..29 of wave 0 each walk
-//        one row of the tile left to right with dependent v_add_f16 (3 ns each on this chip).  A tile is 16 KiB in and
-//        15 KiB out of HBM per CU, about 1 us at a CU's share of 8 TB/s; the walk of 256 columns takes 0.8 us, which is
-//        why wave 0 is kept free of any other work and raises its issue priority.
+// One 1024-thread block per CU walks over groups of 30 rows.  Wave 0 does nothing but the sequential sums; loader wave
+// w = 1..15 owns rows w-1 and w+14 of the group: in step t its 64 lanes cover the 1 KiB at columns t*512 .. t*512+511 of
+// each of the two rows (one fully contiguous 1 KiB per load instruction), and keep the exp values in registers
+// (NSTEP * 8 VGPRs) until the row sum is known, so x is read once and y written once.
+//   exp: a 16-bit type has 65536 values; the whole exact exp table (128 KiB) sits in LDS next to the 31 KiB tile
+//        (162 400 of the CU's 163 840 bytes), so exp is one ds_read_u16 per element with the bit pattern as the index:
+//        no range clamping, no NaN special case.
+//   sum: per 512-column step the exp values also go to an LDS tile; lanes 0..29 of wave 0 each walk one row of the
+//        tile left to right with dependent v_add_f16 (3 ns each on this chip, 1.5 us per step).  The tile is single
+//        buffered with two barriers per step: the loaders look up step t+1 into registers and divide / store the
+//        previous group's step t while wave 0 walks step t, and only the short LDS write of the tile sits between the
+//        barriers with wave 0 idle.  A step is 30 KiB in and 30 KiB out of HBM per CU, about 2 us at a CU's share of
+//        8 TB/s, so the walk stays hidden; wave 0 is kept free of any other work and raises its issue priority.
 //   divide: the outputs of group g are produced while group g+1 streams in: y = e / sum with the quotient computed as
 //        q0 = e * (1/sum) plus one fma correction, which is the correctly rounded f16 quotient for normal finite sums
 //        (checked against IEEE division over operand pairs on the GPU); other sums take the IEEE path.
 //   mask: with MASK, a second operand (one [P, cols] block shared by every period of P rows, e.g. an [S, T] attention
 //        mask under B * H heads) is added to x in f16 as the vectors arrive: scores.add(mask).softmax() without the sum
 //        ever reaching memory, bit-identical to the two separate ops.
-// Global loads run SP_PF tiles ahead across group boundaries, so the pipeline never drains.
+// Global loads run SP_PF steps ahead across group boundaries, so the pipeline never drains.
 // ------------------------------------------------------------------------------------------------------------------
 constexpr int SP_BLOCK = 1024;
 constexpr int SP_ROWS = 30;                  // 15 loader waves x 2 rows each; wave 0 only walks
-constexpr int SP_TC = 256;
+constexpr int SP_HALF = SP_ROWS / 2;
+constexpr int SP_TC = 512;                   // columns per step: 64 lanes x 8 halves
 constexpr int SP_PAD = 8;
-constexpr int SP_PF = 4;                     // tiles loaded ahead
-constexpr int SP_MPF = 1;                    // mask tiles loaded ahead
+constexpr int SP_PF = 2;                     // steps loaded ahead
+constexpr int SP_MAX_STEPS = 8;              // rows of up to 4096 columns
 constexpr size_t SP_LUT_BYTES = 65536 * sizeof(uint16_t);
-constexpr size_t SP_TILE_BYTES = 2 * SP_ROWS * (SP_TC + SP_PAD) * sizeof(uint16_t);
-constexpr size_t SP_SMEM_BYTES = SP_LUT_BYTES + SP_TILE_BYTES + 2 * 32 * sizeof(uint16_t);      // 162 880 of the CU's 163 840 bytes
+constexpr size_t SP_TILE_BYTES = SP_ROWS * (SP_TC + SP_PAD) * sizeof(uint16_t);
+constexpr size_t SP_SMEM_BYTES = SP_LUT_BYTES + SP_TILE_BYTES + 2 * 32 * sizeof(uint16_t);      // 162 400 of the CU's 163 840 bytes
 
 typedef _Float16 h16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 h16x8 __attribute__((ext_vector_type(8)));
@@ -284,13 +286,13 @@ __device__ __forceinline__ void sp_item(const SpSched& s, uint32_t b, uint32_t G
     fd_divmod(b + it * G, s.gp_div, rep, pg);
 }
 
-template <int NSLOT, bool FULL, bool MASK>
+template <int NSTEP, bool FULL, bool MASK>
 __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint16_t* __restrict__ table, const half_t* x,
                                                                       const half_t* mask, half_t* y, uint64_t rows, uint32_t cols,
                                                                       SpSched sch) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint16_t* lut = reinterpret_cast<uint16_t*>(smem);
-    half_t (*tile)[SP_ROWS][SP_TC + SP_PAD] = reinterpret_cast<half_t (*)[SP_ROWS][SP_TC + SP_PAD]>(smem + SP_LUT_BYTES);
+    half_t (*tile)[SP_TC + SP_PAD] = reinterpret_cast<half_t (*)[SP_TC + SP_PAD]>(smem + SP_LUT_BYTES);
     half_t (*sums)[32] = reinterpret_cast<half_t (*)[32]>(smem + SP_LUT_BYTES + SP_TILE_BYTES);
 
     // table -> LDS
@@ -303,18 +305,21 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
     const uint32_t n_items = sp_item_count(sch, blockIdx.x, gridDim.x);
     __syncthreads();                                         // table visible
 
+    // Every wave passes the same barriers: two per step (A: the walk of the previous tile is over, the tile may be
+    // overwritten; B: the new tile is complete) and one after the block's last group.
     if (threadIdx.x < 64) {
         // ------------------------------------------------------------------ wave 0: the walk, nothing else
         __builtin_amdgcn_s_setprio(3);
         const uint32_t lane = threadIdx.x;
         const uint32_t wr = lane < SP_ROWS ? lane : 0;       // lanes 30..63 shadow row 0 and never publish
+        const v4u* trow = reinterpret_cast<const v4u*>(tile[wr]);
         half_t run = (half_t)0.0f;
         uint32_t gpar = 0;
         for (uint32_t it = 0; it < n_items; it++) {
 #pragma unroll 1
-            for (int t = 0; t < NSLOT; t++) {
-                __syncthreads();                             // tile t is in LDS
-                const v4u* trow = reinterpret_cast<const v4u*>(tile[t & 1][wr]);
+            for (int t = 0; t < NSTEP; t++) {
+                __syncthreads();                             // A
+                __syncthreads();                             // B: tile t is in LDS
                 // 16 values per chunk; the LDS reads of the next chunk are in flight during the 16 dependent adds
                 v4u c0 = trow[0], c1 = trow[1];
 #pragma unroll
@@ -342,7 +347,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
             run = (half_t)0.0f;
             gpar ^= 1;
         }
-        __syncthreads();                                     // drain barrier (matches the loaders')
+        __syncthreads();                                     // after the last group: its sums are published
         return;
     }
 
@@ -353,8 +358,8 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
     // count exactly how many of them may stay in flight at each wait (with branches it waits for all of them, the
     // store issued a moment ago included, and the prefetch distance collapses).
     const uint32_t lt = threadIdx.x - 64;                    // 0..959
-    const uint32_t r = lt >> 5, cv = lt & 31;                // row in the group (0..29), vector in the tile
-    const uint32_t ccol = cv * 8;                            // column of this thread's vector inside a tile
+    const uint32_t rr = __builtin_amdgcn_readfirstlane(lt >> 6);   // rows rr and rr + 15 of the group: the same for the whole wave
+    const uint32_t ccol = (lt & 63) * 8;                     // column of this thread's vectors inside a step
     const uint32_t row_bytes = cols * 2;
     const uint32_t nbytes = (uint32_t)(rows * row_bytes);    // the launcher keeps this below 2^31
     const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(x), 0, nbytes, 0x00020000);
@@ -362,57 +367,73 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
     const __amdgpu_buffer_rsrc_t rm =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(MASK ? mask : x), 0, MASK ? sch.P * row_bytes : nbytes, 0x00020000);
     constexpr uint32_t OOB = 0x80000000u;                    // >= nbytes, and stays so after adding a column offset
-    constexpr int PF = NSLOT < SP_PF ? NSLOT : SP_PF;        // tiles of x in flight per thread
-    constexpr int MPF = SP_MPF;                              // tiles of the mask in flight (L2 hits: a short distance is enough)
+    constexpr int PF = NSTEP < SP_PF ? NSTEP : SP_PF;        // steps of x in flight per thread
     const uint32_t G = gridDim.x;
 
-    // byte offsets of (row r of item `it`, column ccol) in x / y and in the mask, or OOB
-    auto item_off = [&](uint32_t it, uint32_t& xo, uint32_t& mo) {
+    // Row offsets are the same for all lanes of a wave, so they live in scalar registers (the vector registers are all
+    // needed for data): byte offset of rows rr / rr + 15 of item `it` in x / y, or OOB, and of the item's period in x
+    // (x offset - period offset = mask offset; for a row that does not exist the mask offset is arbitrary, which is
+    // harmless: the load is range checked, and what is computed from it is never stored).
+    auto item_off = [&](uint32_t it, uint32_t (&xo)[2], uint32_t& period_off) {
         uint32_t rep, pg;
         sp_item(sch, blockIdx.x, G, it, rep, pg);
-        const uint32_t prow = pg * sch.R + r;                // row inside the period
-        const bool ok = it < n_items && r < sch.R && prow < sch.P;
-        mo = ok ? prow * row_bytes + ccol * 2 : OOB;
-        xo = ok ? (rep * sch.P + prow) * row_bytes + ccol * 2 : OOB;
+        period_off = __builtin_amdgcn_readfirstlane(rep * sch.P * row_bytes);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint32_t r = rr + h * SP_HALF;
+            const uint32_t prow = pg * sch.R + r;            // row inside the period
+            const bool ok = it < n_items && r < sch.R && prow < sch.P;
+            xo[h] = __builtin_amdgcn_readfirstlane(ok ? (rep * sch.P + prow) * row_bytes : OOB);
+        }
     };
-    auto slot_off = [&](uint32_t base, int t) -> uint32_t {
+    const uint32_t cbyte = ccol * 2;
+    auto step_off = [&](uint32_t row_off, int t) -> uint32_t {   // per-lane offset of this thread's vector in step t of a row
         if (!FULL && (uint32_t)t * SP_TC + ccol >= cols) return OOB;
-        return base + (uint32_t)t * (SP_TC * 2);
+        return row_off + (uint32_t)t * (SP_TC * 2) + cbyte;
     };
     auto load_x = [&](uint32_t off) -> v4u { return __builtin_amdgcn_raw_buffer_load_b128(rx, off, 0, 2); };   // 2: non-temporal
     auto load_m = [&](uint32_t off) -> v4u { return __builtin_amdgcn_raw_buffer_load_b128(rm, off, 0, 0); };   // re-read by other heads
 
-    uint32_t cur, nxt, mcur, mnxt, prev = OOB;
-    item_off(0, cur, mcur);
-    item_off(1, nxt, mnxt);
-    v4u e[NSLOT];                                            // exp values of the group in flight, 8 halves per slot
-    v4u pre[PF], mpre[MPF];
+    uint32_t cur[2], nxt[2], prev[2] = {OOB, OOB}, pcur, pnxt;
+    item_off(0, cur, pcur);
+    item_off(1, nxt, pnxt);
+    v4u e[NSTEP][2];                                         // exp values of the group in flight, 8 halves per vector
+    v4u pre[PF][2], mpre[2];                                 // x: PF steps in flight; mask: one (L2 hits: a short distance is enough)
 #pragma unroll
-    for (int t = 0; t < NSLOT; t++) e[t] = v4u{0, 0, 0, 0};
+    for (int t = 0; t < NSTEP; t++) e[t][0] = e[t][1] = v4u{0, 0, 0, 0};
+    // The pending memory operations at the top of the group loop are the same on entry as after a group (two loads, two
+    // stores, two loads, two stores: the stores here go nowhere), so the compiler can count them there too.
 #pragma unroll
-    for (int k = 0; k < PF; k++) pre[k] = load_x(slot_off(cur, k));
+    for (int k = 0; k < PF; k++) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) pre[k][h] = load_x(step_off(cur[h], k));
+#pragma unroll
+        for (int h = 0; h < 2; h++) __builtin_amdgcn_raw_buffer_store_b128(v4u{0, 0, 0, 0}, ry, OOB, 0, 2);
+    }
     if (MASK) {
 #pragma unroll
-        for (int k = 0; k < MPF; k++) mpre[k] = load_m(slot_off(mcur, k));
+        for (int h = 0; h < 2; h++) mpre[h] = load_m(step_off(cur[h] - pcur, 0));
     }
 
-    float s_prev = 1.0f, rinv_prev = 1.0f;
-    bool fast_prev = true;
+    // sum of the previous group's rows, reciprocal, and whether the short division applies: wave-uniform as well
+    float s_prev[2] = {1.0f, 1.0f}, rinv_prev[2] = {1.0f, 1.0f};
+    bool fast_prev[2] = {true, true};
     uint32_t gpar = 0;
 
-    auto quotients = [&](const v4u& ev) -> v4u {             // e / sum of the previous group
+    auto quotients = [&](const v4u& ev, int h) -> v4u {      // e / sum of the previous group
         v4u out;
-        if (fast_prev) {
+        const float s = s_prev[h], rinv = rinv_prev[h];
+        if (fast_prev[h]) {
 #pragma unroll
             for (int w = 0; w < 4; w++) {
                 // v_fma_mix_f32 reads the f16 halves of ev[w] directly: a = e * r (+0), rem = e - s * a; no separate conversions
                 float a0, a1, m0, m1;
-                asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(a0) : "v"(ev[w]), "v"(rinv_prev));
-                asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(a1) : "v"(ev[w]), "v"(rinv_prev));
-                asm("v_fma_mix_f32 %0, -%1, %2, %3 op_sel_hi:[0,0,1]" : "=v"(m0) : "v"(s_prev), "v"(a0), "v"(ev[w]));
-                asm("v_fma_mix_f32 %0, -%1, %2, %3 op_sel:[0,0,1] op_sel_hi:[0,0,1]" : "=v"(m1) : "v"(s_prev), "v"(a1), "v"(ev[w]));
-                float q0 = __builtin_fmaf(m0, rinv_prev, a0);
-                float q1 = __builtin_fmaf(m1, rinv_prev, a1);
+                asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(a0) : "v"(ev[w]), "s"(rinv));
+                asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(a1) : "v"(ev[w]), "s"(rinv));
+                asm("v_fma_mix_f32 %0, -%1, %2, %3 op_sel_hi:[0,0,1]" : "=v"(m0) : "s"(s), "v"(a0), "v"(ev[w]));
+                asm("v_fma_mix_f32 %0, -%1, %2, %3 op_sel:[0,0,1] op_sel_hi:[0,0,1]" : "=v"(m1) : "s"(s), "v"(a1), "v"(ev[w]));
+                float q0 = __builtin_fmaf(m0, rinv, a0);
+                float q1 = __builtin_fmaf(m1, rinv, a1);
                 // keep the f32 quotient and its conversion apart: fused into v_fma_mixlo_f16 the pair rounds
                 // subnormal f16 results differently from fma-then-convert
                 asm volatile("" : "+v"(q0), "+v"(q1));
@@ -423,54 +444,79 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
 #pragma unroll
             for (int w = 0; w < 4; w++) {
                 const float e0 = (float)bits_h((uint16_t)(ev[w] & 0xffffu)), e1 = (float)bits_h((uint16_t)(ev[w] >> 16));
-                out[w] = (uint32_t)h_bits((half_t)(e0 / s_prev)) | ((uint32_t)h_bits((half_t)(e1 / s_prev)) << 16);
+                out[w] = (uint32_t)h_bits((half_t)(e0 / s)) | ((uint32_t)h_bits((half_t)(e1 / s)) << 16);
             }
         }
         return out;
     };
     auto read_prev_sum = [&](uint32_t par) {
-        const float s = (float)sums[par][r];
-        s_prev = s;
-        // normal, finite, not tiny: the reciprocal-plus-correction quotient is exact there
-        fast_prev = (s >= 6.103515625e-05f) && (s < __builtin_huge_valf());
-        rinv_prev = fast_prev ? 1.0f / s : 0.0f;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint32_t sb = __builtin_amdgcn_readfirstlane((uint32_t)h_bits(sums[par][rr + h * SP_HALF]));
+            const float s = (float)bits_h((uint16_t)sb);
+            s_prev[h] = s;
+            // normal, finite, not tiny: the reciprocal-plus-correction quotient is exact there
+            fast_prev[h] = (s >= 6.103515625e-05f) && (s < __builtin_huge_valf());
+            rinv_prev[h] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, fast_prev[h] ? 1.0f / s : 0.0f)));
+        }
     };
 
     for (uint32_t it = 0; it < n_items; it++) {
 #pragma unroll
-        for (int t = 0; t < NSLOT; t++) {
-            v4u& in = pre[t % PF];
-            if (MASK) {                                      // scores + mask in f16, as the separate add would round it
-                const h16x8 sum = __builtin_bit_cast(h16x8, in) + __builtin_bit_cast(h16x8, mpre[t % MPF]);
-                in = __builtin_bit_cast(v4u, sum);
-                mpre[t % MPF] = (t + MPF < NSLOT) ? load_m(slot_off(mcur, t + MPF)) : load_m(slot_off(mnxt, t + MPF - NSLOT));
-            }
-            // exp of the vector that arrived, parked in the LDS tile for the walk (zeros past the row end: adding +0 is a no-op;
-            // rows past the tensor's end read zeros and their sums are never used)
-            v4u enew;
+        for (int t = 0; t < NSTEP; t++) {
+            // exp of the vectors that arrived, in place (zeros past the row end: adding +0 is a no-op; rows past the
+            // tensor's end read zeros and their sums are never used)
 #pragma unroll
-            for (int w = 0; w < 4; w++) enew[w] = sp_exp_pair(lut, in[w]);
-            if (!FULL && (uint32_t)t * SP_TC + ccol >= cols) enew = v4u{0, 0, 0, 0};
-            *reinterpret_cast<v4u*>(&tile[t & 1][r][ccol]) = enew;
-            // next load for this register: PF tiles ahead, possibly in the block's next group
-            in = (t + PF < NSLOT) ? load_x(slot_off(cur, t + PF)) : load_x(slot_off(nxt, t + PF - NSLOT));
-            __syncthreads();
-            if (t == 0) read_prev_sum(gpar ^ 1);              // published by wave 0 before it reached this barrier
-            const v4u out = quotients(e[t]);                  // first group: prev is OOB, the store is dropped
-            __builtin_amdgcn_raw_buffer_store_b128(out, ry, slot_off(prev, t), 0, 2);
-            e[t] = enew;
+            for (int h = 0; h < 2; h++) {
+                v4u& in = pre[t % PF][h];
+                if (MASK) {                                  // scores + mask in f16, as the separate add would round it
+                    const h16x8 sum = __builtin_bit_cast(h16x8, in) + __builtin_bit_cast(h16x8, mpre[h]);
+                    in = __builtin_bit_cast(v4u, sum);
+                }
+#pragma unroll
+                for (int w = 0; w < 4; w++) in[w] = sp_exp_pair(lut, in[w]);
+                if (!FULL && (uint32_t)t * SP_TC + ccol >= cols) in = v4u{0, 0, 0, 0};
+            }
+            __syncthreads();                                 // A: wave 0 has left the previous tile
+            *reinterpret_cast<v4u*>(&tile[rr][ccol]) = pre[t % PF][0];
+            *reinterpret_cast<v4u*>(&tile[rr + SP_HALF][ccol]) = pre[t % PF][1];
+            // the registers are free again: next loads, PF steps ahead, possibly in the block's next group
+            // (loads return in order: the mask of the next step goes first, so that waiting for it does not wait for x of
+            // the step after)
+            if (MASK) {
+#pragma unroll
+                for (int h = 0; h < 2; h++)
+                    mpre[h] = (t + 1 < NSTEP) ? load_m(step_off(cur[h] - pcur, t + 1)) : load_m(step_off(nxt[h] - pnxt, 0));
+            }
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+                pre[t % PF][h] = (t + PF < NSTEP) ? load_x(step_off(cur[h], t + PF)) : load_x(step_off(nxt[h], t + PF - NSTEP));
+            __syncthreads();                                 // B: parked for the walk
+            if (t == 0) read_prev_sum(gpar ^ 1);             // published by wave 0 before it reached barrier A
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const v4u out = quotients(e[t][h], h);       // first group: prev is OOB, the store is dropped
+                __builtin_amdgcn_raw_buffer_store_b128(out, ry, step_off(prev[h], t), 0, 2);
+                // this group's values come back from the tile, which stays intact until the next barrier A
+                e[t][h] = *reinterpret_cast<const v4u*>(&tile[rr + h * SP_HALF][ccol]);
+            }
         }
-        prev = cur;
-        cur = nxt;
-        mcur = mnxt;
-        item_off(it + 2, nxt, mnxt);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            prev[h] = cur[h];
+            cur[h] = nxt[h];
+        }
+        pcur = pnxt;
+        item_off(it + 2, nxt, pnxt);
         gpar ^= 1;
     }
     // drain: outputs of the block's last group
     __syncthreads();
     read_prev_sum(gpar ^ 1);
 #pragma unroll
-    for (int t = 0; t < NSLOT; t++) __builtin_amdgcn_raw_buffer_store_b128(quotients(e[t]), ry, slot_off(prev, t), 0, 2);
+    for (int t = 0; t < NSTEP; t++)
+#pragma unroll
+        for (int h = 0; h < 2; h++) __builtin_amdgcn_raw_buffer_store_b128(quotients(e[t][h], h), ry, step_off(prev[h], t), 0, 2);
 }
 
 // ------------------------------------------------------------------------------------------------------------------
@@ -682,10 +728,10 @@ int launch_f16_stream(rt_device* dev, const void* x, const void* mask, uint64_t 
     int rc = rt_unary_table(dev, 0, RT_EXP, &table);
     if (rc) return rc;
     const uint32_t nt = (cols + SP_TC - 1) / SP_TC;
-    const bool full = cols % SP_TC == 0 && (nt == 2 || nt == 4 || nt == 8 || nt == 16);
+    const bool full = cols % SP_TC == 0 && (nt == 1 || nt == 2 || nt == 4 || nt == 8);
 #define RT_SP(NS, F, M)                                                                                                              \
     do {                                                                                                                             \
-        const unsigned bit = 1u << ((NS == 2 ? 0 : NS == 4 ? 1 : NS == 8 ? 2 : 3) + (F ? 4 : 0) + (M ? 8 : 0));                      \
+        const unsigned bit = 1u << ((NS == 1 ? 0 : NS == 2 ? 1 : NS == 4 ? 2 : 3) + (F ? 4 : 0) + (M ? 8 : 0));                      \
         if (!(dev->sp_attr_set & bit)) {               /* the LDS opt-in is per function and per device */                           \
             RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(softmax_f16_stream_kernel<NS, F, M>),                           \
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)SP_SMEM_BYTES));                             \
@@ -696,10 +742,10 @@ int launch_f16_stream(rt_device* dev, const void* x, const void* mask, uint64_t 
     } while (0)
 #define RT_SP_NS(F, M)                                      \
     do {                                                    \
-        if (nt <= 2) RT_SP(2, F, M);                        \
+        if (nt <= 1) RT_SP(1, F, M);                        \
+        else if (nt <= 2) RT_SP(2, F, M);                   \
         else if (nt <= 4) RT_SP(4, F, M);                   \
-        else if (nt <= 8) RT_SP(8, F, M);                   \
-        else RT_SP(16, F, M);                               \
+        else RT_SP(8, F, M);                                \
     } while (0)
     for (uint64_t row0 = 0; row0 < rows; row0 += chunk_rows) {
         const uint64_t n = rows - row0 < chunk_rows ? rows - row0 : chunk_rows;
@@ -708,7 +754,7 @@ int launch_f16_stream(rt_device* dev, const void* x, const void* mask, uint64_t 
         SpSched sch;
         sch.P = (uint32_t)(mask ? period : n);
         sch.reps = (uint32_t)(n / sch.P);
-        // rows per group: every block runs ceil(groups / grid) rounds of 16-or-fewer tile steps whatever the group holds, so
+        // rows per group: every block runs ceil(groups / grid) rounds of 8-or-fewer steps whatever the group holds, so
         // 4370 groups of 30 rows on 256 CUs cost 18 rounds where 17.07 are needed; 27-row groups make 19 full rounds.
         // Pick the size that minimises rounds x rows (time is proportional to the rows a round could have carried).
         {
@@ -882,7 +928,7 @@ extern "C" int rt_softmax(rt_device* dev, int dt, const void* x, void* y, uint64
         case RT_F16:
             // rows of up to 4096 columns stream through registers in one pass once there is enough work to amortise the
             // per-block table load; everything else takes the two-pass tile walker
-            if (cols % 8 == 0 && cols <= 16 * SP_TC && rows * cols >= (1u << 20) && rt_aligned(x, 16) && rt_aligned(y, 16)) {
+            if (cols % 8 == 0 && cols <= SP_MAX_STEPS * SP_TC && rows * cols >= (1u << 20) && rt_aligned(x, 16) && rt_aligned(y, 16)) {
                 bool done = false;
                 rc = launch_f16_stream(dev, x, nullptr, 0, y, rows, cols, &done);
                 if (rc || done) return rc;
@@ -922,7 +968,7 @@ extern "C" int rt_softmax_masked(rt_device* dev, int dt, const void* x, const ui
         if (mask_shape[i] != x_shape[i]) whole = false;
         period *= x_shape[i];
     }
-    if (dt == RT_F16 && mode == RT_SOFTMAX_REFERENCE && whole && cols % 8 == 0 && cols <= 16 * SP_TC && rows * cols >= (1u << 20) &&
+    if (dt == RT_F16 && mode == RT_SOFTMAX_REFERENCE && whole && cols % 8 == 0 && cols <= SP_MAX_STEPS * SP_TC && rows * cols >= (1u << 20) &&
         rt_aligned(x, 16) && rt_aligned(y, 16) && rt_aligned(mask, 16)) {
         bool done = false;
         rc = launch_f16_stream(dev, x, mask, period, y, rows, cols, &done);
