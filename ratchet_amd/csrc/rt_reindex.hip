@@ -5,7 +5,8 @@
 // op into "dst[i0,i1,i2,i3] = src[base + i0*S0 + i1*S1 + i2*S2 + i3*S3]" with strides resolved at launch, picks the
 // widest vector (16/8/4/2 bytes) that keeps every source and destination access aligned, and each thread moves whole
 // vectors along the destination's last dimension with multiply-shift index math.  A permutation that moves the
-// source's contiguous dimension goes through an LDS tile so both the read and the write side stay coalesced.
+// source's contiguous dimension is transposed in V x V blocks in registers when rows are whole 16-byte vectors, and
+// through an LDS tile otherwise, so both the read and the write side stay coalesced.
 #include "rt_internal.h"
 
 namespace {
@@ -68,8 +69,10 @@ __global__ void __launch_bounds__(BLOCK) gather_splat_kernel(const ElemT* __rest
 
 // Tiled transpose for permutations that move the source's contiguous dimension.
 // Destination dims: `q` is the one fed by the source's last dim; 3 is fed by source dim with stride sj.
-// A block owns a TILE x TILE patch over (dst dim q, dst dim 3); the two remaining dims are flattened in blockIdx.z.
-constexpr int TILE = 64;
+// A block owns a TQ x TJ patch over (dst dim q, dst dim 3), 4096 elements; the two remaining dims are flattened into the
+// block index.  The patch is square unless one side is short (channel-last images, [H,W,3] <-> [3,H,W]), where a
+// 64 x 64 patch would be mostly empty.
+constexpr int TILE_ELEMS = 4096;
 struct TransposeArgs {
     uint32_t nq, n3;         // extents of dst dim q and dst dim 3
     uint64_t s3;             // source stride (elements) of the dim that becomes dst dim 3
@@ -80,30 +83,88 @@ struct TransposeArgs {
     uint64_t da, db;         // destination strides of the other dims
 };
 
-template <typename ElemT>
+template <typename ElemT, int TQ>
 __global__ void __launch_bounds__(BLOCK) transpose_kernel(const ElemT* __restrict__ x, ElemT* __restrict__ y, TransposeArgs p) {
-    __shared__ ElemT tile[TILE][TILE + (sizeof(ElemT) == 4 ? 1 : 2)];
+    constexpr int TJ = TILE_ELEMS / TQ;
+    // the pitch is an odd number of 4-byte words: the column reads below touch every bank once
+    __shared__ ElemT tile[TJ][TQ + (sizeof(ElemT) == 4 ? 1 : 2)];
     uint32_t oa, obi, bz, byx, by, bx;
     fd_divmod(blockIdx.x, p.gx, byx, bx);
     fd_divmod(byx, p.gy, bz, by);
     fd_divmod(bz, p.ob, oa, obi);
     const uint64_t src0 = oa * p.sa + obi * p.sb;
     const uint64_t dst0 = oa * p.da + obi * p.db;
-    const uint32_t q0 = bx * TILE, j0 = by * TILE;                     // origin in (dst dim q, dst dim 3)
-    const uint32_t tx = threadIdx.x & (TILE - 1), ty = threadIdx.x / TILE;   // 64 x 4
+    const uint32_t q0 = bx * TQ, j0 = by * TJ;                         // origin in (dst dim q, dst dim 3)
     // read: rows = dst-dim-3 index (source stride s3), columns = source's contiguous dim (dst dim q)
 #pragma unroll 4
-    for (uint32_t r = ty; r < TILE; r += BLOCK / TILE) {
-        const uint32_t j = j0 + r, q = q0 + tx;
-        if (j < p.n3 && q < p.nq) tile[r][tx] = x[src0 + (uint64_t)j * p.s3 + q];
+    for (uint32_t i = threadIdx.x; i < TILE_ELEMS; i += BLOCK) {
+        const uint32_t r = i / TQ, c = i % TQ;
+        const uint32_t j = j0 + r, q = q0 + c;
+        if (j < p.n3 && q < p.nq) tile[r][c] = x[src0 + (uint64_t)j * p.s3 + q];
     }
     __syncthreads();
     // write: rows = dst dim q, columns = dst dim 3 (contiguous in the destination)
 #pragma unroll 4
-    for (uint32_t r = ty; r < TILE; r += BLOCK / TILE) {
-        const uint32_t q = q0 + r, j = j0 + tx;
-        if (q < p.nq && j < p.n3) y[dst0 + (uint64_t)q * p.dq + j] = tile[tx][r];
+    for (uint32_t i = threadIdx.x; i < TILE_ELEMS; i += BLOCK) {
+        const uint32_t r = i / TJ, c = i % TJ;
+        const uint32_t q = q0 + r, j = j0 + c;
+        if (q < p.nq && j < p.n3) y[dst0 + (uint64_t)q * p.dq + j] = tile[c][r];
     }
+}
+
+// The same permutations when every row on both sides is a whole number of aligned 16-byte vectors (the attention
+// transposes: [B,H,T,D] -> [B,H,D,T], [B,T,H,D] -> [B,H,D,T]): no LDS.  A thread loads V rows of one 16-byte vector
+// (V = 8 halves or 4 words: a V x V block), transposes the block in its registers and stores V vectors.  The 64 lanes of
+// a wave are laid out as QB blocks along the source's contiguous dim by JB blocks along the destination's, so a load
+// instruction reads JB runs of QB * 16 bytes and a store instruction writes QB runs of JB * 16 bytes; QB covers the
+// whole source row when that is short (head dims up to 96 halves), which makes the source patch one contiguous run.
+struct TransposeRegArgs {
+    uint32_t nqb, njb;       // blocks of V elements along dst dim q / dst dim 3
+    uint32_t QB, JB;         // blocks per wave along q / along j (QB * JB <= 64)
+    FastDiv qb_div;          // lane -> (jb, qb)
+    uint64_t s3;             // source stride (elements) of the dim that becomes dst dim 3
+    uint64_t dq;             // destination stride (elements) of dim q
+    FastDiv gx, gy;          // tile counts along q (QB blocks each) and along j (4 waves x JB blocks each)
+    FastDiv ob;
+    uint64_t sa, sb, da, db;
+};
+
+__device__ __forceinline__ void transpose_block(const v4u (&in)[8], v4u (&out)[8], uint16_t) {
+    // out[k] holds element k of each of the 8 input rows: halves (2w, 2w+1) of out[k] come from in[2w], in[2w+1]
+#pragma unroll
+    for (int k = 0; k < 8; k++)
+#pragma unroll
+        for (int w = 0; w < 4; w++)
+            out[k][w] = __builtin_amdgcn_perm(in[2 * w + 1][k / 2], in[2 * w][k / 2], (k & 1) ? 0x07060302u : 0x05040100u);
+}
+__device__ __forceinline__ void transpose_block(const v4u (&in)[4], v4u (&out)[4], uint32_t) {
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+#pragma unroll
+        for (int w = 0; w < 4; w++) out[k][w] = in[w][k];
+}
+
+template <typename ElemT>
+__global__ void __launch_bounds__(BLOCK) transpose_reg_kernel(const ElemT* __restrict__ x, ElemT* __restrict__ y, TransposeRegArgs p) {
+    constexpr int V = 16 / sizeof(ElemT);
+    uint32_t oa, obi, bz, byx, by, bx;
+    fd_divmod(blockIdx.x, p.gx, byx, bx);
+    fd_divmod(byx, p.gy, bz, by);
+    fd_divmod(bz, p.ob, oa, obi);
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t jb, qb;
+    fd_divmod(lane, p.qb_div, jb, qb);
+    qb += bx * p.QB;
+    const uint32_t jblk = (by * (BLOCK / 64) + wave) * p.JB + jb;
+    if (jb >= p.JB || qb >= p.nqb || jblk >= p.njb) return;
+    const ElemT* src = x + oa * p.sa + obi * p.sb + (uint64_t)jblk * V * p.s3 + (uint64_t)qb * V;
+    ElemT* dst = y + oa * p.da + obi * p.db + (uint64_t)qb * V * p.dq + (uint64_t)jblk * V;
+    v4u in[V], out[V];
+#pragma unroll
+    for (int i = 0; i < V; i++) in[i] = ld_stream(reinterpret_cast<const v4u*>(src + (uint64_t)i * p.s3));
+    transpose_block(in, out, ElemT());
+#pragma unroll
+    for (int k = 0; k < V; k++) st_stream(reinterpret_cast<v4u*>(dst + (uint64_t)k * p.dq), out[k]);
 }
 
 // concat: input k is [a_dim, bv[k]] vectors, copied into dst rows of dst_sv vectors at column dst_ov[k]
@@ -372,6 +433,41 @@ int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uin
     int others[2], no = 0;
     for (int i = 0; i < 3; i++)
         if (i != q) others[no++] = i;
+    {
+        // whole aligned 16-byte vectors on both sides: the register transpose
+        const uint32_t V = 16u / (uint32_t)elem_bytes;
+        if (dst_shape[q] % V == 0 && dst_shape[3] % V == 0 && rt_aligned(x, 16) && rt_aligned(y, 16)) {
+            TransposeRegArgs r;
+            r.nqb = dst_shape[q] / V;
+            r.njb = dst_shape[3] / V;
+            r.QB = r.nqb <= 12 ? r.nqb : 8;
+            r.JB = 64 / r.QB;
+            if (r.JB > r.njb) r.JB = r.njb;
+            r.qb_div = make_fastdiv(r.QB);
+            r.s3 = S[3];
+            r.dq = dst_strides[q];
+            r.ob = make_fastdiv(dst_shape[others[1]]);
+            r.sa = S[others[0]];
+            r.sb = S[others[1]];
+            r.da = dst_strides[others[0]];
+            r.db = dst_strides[others[1]];
+            const uint64_t gz = (uint64_t)dst_shape[others[0]] * dst_shape[others[1]];
+            const uint64_t gx = (r.nqb + r.QB - 1) / r.QB, gy = (r.njb + (BLOCK / 64) * r.JB - 1) / ((BLOCK / 64) * r.JB);
+            const uint64_t blocks = gx * gy * gz;
+            RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_permute: %llu tiles exceed the grid limit", (unsigned long long)blocks);
+            r.gx = make_fastdiv((uint32_t)gx);
+            r.gy = make_fastdiv((uint32_t)gy);
+            if (elem_bytes == 4) {
+                hipLaunchKernelGGL((transpose_reg_kernel<uint32_t>), dim3((unsigned)blocks), dim3(BLOCK), 0, dev->stream,
+                                   (const uint32_t*)x, (uint32_t*)y, r);
+            } else {
+                hipLaunchKernelGGL((transpose_reg_kernel<uint16_t>), dim3((unsigned)blocks), dim3(BLOCK), 0, dev->stream,
+                                   (const uint16_t*)x, (uint16_t*)y, r);
+            }
+            RT_CHECK_LAUNCH("transpose_reg_kernel");
+            return RT_OK;
+        }
+    }
     TransposeArgs p;
     p.nq = dst_shape[q];
     p.n3 = dst_shape[3];
@@ -383,18 +479,25 @@ int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uin
     p.da = dst_strides[others[0]];
     p.db = dst_strides[others[1]];
     const uint64_t gz = (uint64_t)dst_shape[others[0]] * dst_shape[others[1]];
-    const uint64_t gx = (p.nq + TILE - 1) / TILE, gy = (p.n3 + TILE - 1) / TILE;
+    const uint32_t tq = p.nq <= 8 ? 8 : p.nq <= 16 ? 16 : p.n3 <= 8 ? 512 : p.n3 <= 16 ? 256 : 64, tj = TILE_ELEMS / tq;
+    const uint64_t gx = (p.nq + tq - 1) / tq, gy = (p.n3 + tj - 1) / tj;
     const uint64_t blocks = gx * gy * gz;
     RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_permute: %llu tiles exceed the grid limit", (unsigned long long)blocks);
     p.gx = make_fastdiv((uint32_t)gx);
     p.gy = make_fastdiv((uint32_t)gy);
-    if (elem_bytes == 4) {
-        hipLaunchKernelGGL((transpose_kernel<uint32_t>), dim3((unsigned)blocks), dim3(BLOCK), 0, dev->stream, (const uint32_t*)x,
-                           (uint32_t*)y, p);
-    } else {
-        hipLaunchKernelGGL((transpose_kernel<uint16_t>), dim3((unsigned)blocks), dim3(BLOCK), 0, dev->stream, (const uint16_t*)x,
-                           (uint16_t*)y, p);
-    }
+#define RT_TR(E, TQ) hipLaunchKernelGGL((transpose_kernel<E, TQ>), dim3((unsigned)blocks), dim3(BLOCK), 0, dev->stream, (const E*)x, (E*)y, p)
+#define RT_TR_E(E)                       \
+    do {                                 \
+        if (tq == 8) RT_TR(E, 8);        \
+        else if (tq == 16) RT_TR(E, 16); \
+        else if (tq == 64) RT_TR(E, 64); \
+        else if (tq == 256) RT_TR(E, 256); \
+        else RT_TR(E, 512);              \
+    } while (0)
+    if (elem_bytes == 4) RT_TR_E(uint32_t);
+    else RT_TR_E(uint16_t);
+#undef RT_TR_E
+#undef RT_TR
     RT_CHECK_LAUNCH("transpose_kernel");
     return RT_OK;
 }

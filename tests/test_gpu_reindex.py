@@ -50,6 +50,35 @@ def test_permute_lower_rank_and_baseline_shapes(dev, oracle):
     assert np.array_equal(dev.permute(dev.upload(k), (0, 2, 3, 1)).to_numpy(), oracle.permute(k, (0, 2, 3, 1)))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_permute_transposes_of_whole_vectors(dev, oracle, dtype):
+    """Permutations that move the contiguous dim, on shapes whose rows are whole 16-byte vectors on both sides
+    (K^T in phi2/attn.rs:140, whisper/mha.rs:106, moondream/vision_encoder.rs:58): every order, head dims 64..128,
+    extents that leave partial tiles, and a slice-shaped source offset through views of a larger upload."""
+    rng = np.random.default_rng(202)
+    for shape in [(2, 3, 40, 80), (1, 6, 1504, 64), (2, 2, 264, 96), (1, 4, 72, 128), (3, 8, 16, 8), (1, 2, 520, 200), (2, 16, 8, 1032)]:
+        x = randn(rng, shape, dtype)
+        dx = dev.upload(x)
+        for perm in itertools.permutations(range(4)):
+            if perm[3] == 3:
+                continue                                    # the contiguous dim stays: covered above
+            want = oracle.permute(x, perm)
+            got = dev.permute(dx, perm).to_numpy()
+            assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (shape, perm)
+    # rank 3 ([B, C, T] -> [B, T, C]: whisper/encoder.rs:53) and rank 2
+    x3 = randn(rng, (2, 384, 1504), dtype)
+    assert np.array_equal(dev.permute(dev.upload(x3), (0, 2, 1)).to_numpy(), np.ascontiguousarray(x3.transpose(0, 2, 1)))
+    x2 = randn(rng, (1000, 136), dtype)
+    assert np.array_equal(dev.permute(dev.upload(x2), (1, 0)).to_numpy(), np.ascontiguousarray(x2.T))
+    # channel-last image to channel-first and back (moondream/generate.rs:42,140): one side of the transpose is 3 long
+    img = randn(rng, (378, 378, 3), dtype)
+    chw = dev.permute(dev.upload(img), (2, 0, 1))
+    assert np.array_equal(chw.to_numpy(), np.ascontiguousarray(img.transpose(2, 0, 1)))
+    assert np.array_equal(dev.permute(chw, (1, 2, 0)).to_numpy(), img)
+    wide = randn(rng, (2, 700, 12), dtype)
+    assert np.array_equal(dev.permute(dev.upload(wide), (0, 2, 1)).to_numpy(), np.ascontiguousarray(wide.transpose(0, 2, 1)))
+
+
 def test_permute_rejects_duplicates(dev):
     from ratchet_amd import RatchetError
 
