@@ -203,21 +203,20 @@ __global__ void __launch_bounds__(BLOCK) softmax_seq16_kernel(const T* __restric
     if (threadIdx.x < nrows) sums[threadIdx.x] = run;
     __syncthreads();
 
+    // the block's rows are one contiguous run of nrows * cols elements: all threads sweep it, whatever the row length
     const uint32_t cvec = cols / VE;
-    for (uint32_t r = 0; r < nrows; r++) {
-        const T sum = sums[r];
-        const T* src = x + (row0 + r) * cols;
-        T* dst = y + (row0 + r) * cols;
-        for (uint32_t cv = threadIdx.x; cv < cvec; cv += BLOCK) {
-            if (VEC) {
-                Vec16<T> in, out;
-                in.u = reinterpret_cast<const v4u*>(src)[cv];
+    const T* src = x + row0 * cols;
+    T* dst = y + row0 * cols;
+    for (uint64_t i = threadIdx.x; i < (uint64_t)nrows * cvec; i += BLOCK) {
+        const T sum = sums[i / cvec];
+        if (VEC) {
+            Vec16<T> in, out;
+            in.u = reinterpret_cast<const v4u*>(src)[i];
 #pragma unroll
-                for (int q = 0; q < 8; q++) out.e[q] = Ar<T>::div(ar_exp<T>(in.e[q]), sum);
-                st_stream(reinterpret_cast<v4u*>(dst) + cv, out.u);
-            } else {
-                dst[cv] = Ar<T>::div(ar_exp<T>(src[cv]), sum);
-            }
+            for (int q = 0; q < 8; q++) out.e[q] = Ar<T>::div(ar_exp<T>(in.e[q]), sum);
+            st_stream(reinterpret_cast<v4u*>(dst) + i, out.u);
+        } else {
+            dst[i] = Ar<T>::div(ar_exp<T>(src[i]), sum);
         }
     }
 }
@@ -757,10 +756,11 @@ int launch_f16_stream(rt_device* dev, const void* x, const void* mask, uint64_t 
         // rows per group: every block runs ceil(groups / grid) rounds of 8-or-fewer steps whatever the group holds, so
         // 4370 groups of 30 rows on 256 CUs cost 18 rounds where 17.07 are needed; 27-row groups make 19 full rounds.
         // Pick the size that minimises rounds x rows (time is proportional to the rows a round could have carried).
+        // Few rows (a decode step's [B * H, T] scores) spread over the CUs the same way: 32 rows run as 32 one-row groups.
         {
             uint64_t best = ~0ull;
             sch.R = SP_ROWS;
-            for (uint32_t R = SP_ROWS; R >= SP_ROWS - 6; R--) {
+            for (uint32_t R = SP_ROWS; R >= 1; R--) {
                 const uint64_t groups = (uint64_t)((sch.P + R - 1) / R) * sch.reps;
                 const uint64_t rounds = (groups + dev->num_cus - 1) / dev->num_cus;
                 const uint64_t cost = rounds * R + rounds / 4;          // the small second term: a round has a fixed cost too
@@ -926,9 +926,10 @@ extern "C" int rt_softmax(rt_device* dev, int dt, const void* x, void* y, uint64
     switch (dt) {
         case RT_F32: return launch_f32_style<float, 0>(dev, x, y, rows, cols);
         case RT_F16:
-            // rows of up to 4096 columns stream through registers in one pass once there is enough work to amortise the
-            // per-block table load; everything else takes the two-pass tile walker
-            if (cols % 8 == 0 && cols <= SP_MAX_STEPS * SP_TC && rows * cols >= (1u << 20) && rt_aligned(x, 16) && rt_aligned(y, 16)) {
+            // rows of up to 4096 columns that are whole aligned vectors stream through registers in one pass (also small
+            // problems: the per-block table load costs about 5 us, the two-pass walker more); everything else takes
+            // the two-pass tile walker
+            if (cols % 8 == 0 && cols <= SP_MAX_STEPS * SP_TC && rt_aligned(x, 16) && rt_aligned(y, 16)) {
                 bool done = false;
                 rc = launch_f16_stream(dev, x, nullptr, 0, y, rows, cols, &done);
                 if (rc || done) return rc;
@@ -968,7 +969,7 @@ extern "C" int rt_softmax_masked(rt_device* dev, int dt, const void* x, const ui
         if (mask_shape[i] != x_shape[i]) whole = false;
         period *= x_shape[i];
     }
-    if (dt == RT_F16 && mode == RT_SOFTMAX_REFERENCE && whole && cols % 8 == 0 && cols <= SP_MAX_STEPS * SP_TC && rows * cols >= (1u << 20) &&
+    if (dt == RT_F16 && mode == RT_SOFTMAX_REFERENCE && whole && cols % 8 == 0 && cols <= SP_MAX_STEPS * SP_TC &&
         rt_aligned(x, 16) && rt_aligned(y, 16) && rt_aligned(mask, 16)) {
         bool done = false;
         rc = launch_f16_stream(dev, x, mask, period, y, rows, cols, &done);

@@ -70,9 +70,11 @@ def test_softmax_f16_reference_sequence(dev, oracle, shape):
     assert mismatch_count(got, want) == 0, (shape, mismatch_count(got, want))
 
 
-@pytest.mark.parametrize("shape", [(1, 300, 4096), (2, 601, 1000), (1, 2100, 512), (1, 4099, 264), (7, 64, 2560)])
+@pytest.mark.parametrize("shape", [(1, 300, 4096), (2, 601, 1000), (1, 2100, 512), (1, 4099, 264), (7, 64, 2560),
+                                   (32, 1, 4096), (32, 1, 1000), (1, 20, 8), (1, 257, 520), (1, 31, 2056), (16, 61, 72)])
 def test_softmax_f16_streaming_kernel(dev, oracle, shape):
-    # >= 2^20 elements with cols <= 4096 and cols % 8 == 0: the single-pass kernel (exp table in LDS, rows held in registers)
+    # cols <= 4096 and cols % 8 == 0: the single-pass kernel (exp table in LDS, rows held in registers), from the large
+    # prefill shapes down to a decode step's [B * H, 1, T] scores, where every row becomes a group of its own
     rng = np.random.default_rng(303)
     x = randn(rng, shape, np.float16, 2.0)
     n = shape[-1]
@@ -84,6 +86,7 @@ def test_softmax_f16_streaming_kernel(dev, oracle, shape):
     flat[13, 3] = np.nan
     flat[17, :] = -20.0                                                # every exp underflows to 0
     flat[19, :] = -16.0                                                # subnormal exps
+    flat[-1, : n // 2] = -12.0                                         # the last row: tiny terms first, then ordinary ones
     want = oracle.softmax(x)
     dx = dev.upload(x)
     got = dev.softmax(dx).to_numpy()
