@@ -302,32 +302,40 @@ template <> __device__ __forceinline__ float cast_one<half_t, float>(half_t v) {
 template <> __device__ __forceinline__ bf16_t cast_one<float, bf16_t>(float v) { return Ar<bf16_t>::conv(v); }
 template <> __device__ __forceinline__ float cast_one<bf16_t, float>(bf16_t v) { return Ar<bf16_t>::widen(v); }
 
-// 8 elements per thread: 16 bytes on the 2-byte side, 2 x 16 bytes on the 4-byte side
-constexpr int CAST_UNROLL = 2;
+// Four elements per thread and access: 8 bytes on the 2-byte side, 16 bytes on the 4-byte side, so that every load
+// and every store instruction of a wave covers one contiguous run (512 B / 1 KiB).  (Eight elements per thread make the
+// 4-byte side two 16-byte accesses 32 bytes apart per lane: each instruction then touches half of every 32 bytes, and
+// the kernel ran at 4.6 TB/s where this layout reaches 6.)
+constexpr int CAST_UNROLL = 4;
+template <int BYTES> struct CastVec;
+template <> struct CastVec<8> { typedef v2u type; };
+template <> struct CastVec<16> { typedef v4u type; };
+
 template <typename S, typename D>
 __global__ void __launch_bounds__(BLOCK) cast_vec_kernel(const S* __restrict__ x, D* __restrict__ y, uint64_t numel) {
-    constexpr int PER = 8;
+    constexpr int PER = 4;
+    typedef typename CastVec<PER * sizeof(S)>::type SV;
+    typedef typename CastVec<PER * sizeof(D)>::type DV;
     const uint64_t ngrp = numel / PER;
     const uint64_t base = (uint64_t)blockIdx.x * (BLOCK * CAST_UNROLL) + threadIdx.x;
+    SV raw[CAST_UNROLL];
+#pragma unroll
+    for (int k = 0; k < CAST_UNROLL; k++) {
+        const uint64_t g = base + (uint64_t)k * BLOCK;
+        if (g < ngrp) raw[k] = ld_stream(reinterpret_cast<const SV*>(x) + g);
+    }
 #pragma unroll
     for (int k = 0; k < CAST_UNROLL; k++) {
         const uint64_t g = base + (uint64_t)k * BLOCK;
         if (g < ngrp) {
             S in[PER];
             D out[PER];
-            const v4u* src = reinterpret_cast<const v4u*>(x + g * PER);
-            constexpr int NS = PER * sizeof(S) / 16, ND = PER * sizeof(D) / 16;
-            v4u raw[NS];
-#pragma unroll
-            for (int q = 0; q < NS; q++) raw[q] = ld_stream(src + q);
-            __builtin_memcpy(in, raw, sizeof(in));
+            __builtin_memcpy(in, &raw[k], sizeof(in));
 #pragma unroll
             for (int e = 0; e < PER; e++) out[e] = cast_one<S, D>(in[e]);
-            v4u o[ND];
-            __builtin_memcpy(o, out, sizeof(out));
-            v4u* dst = reinterpret_cast<v4u*>(y + g * PER);
-#pragma unroll
-            for (int q = 0; q < ND; q++) st_stream(dst + q, o[q]);
+            DV o;
+            __builtin_memcpy(&o, out, sizeof(out));
+            st_stream(reinterpret_cast<DV*>(y) + g, o);
         }
     }
     if (blockIdx.x == 0) {
@@ -521,7 +529,7 @@ int launch_gated(rt_device* dev, int op, const void* gate, uint64_t gs, const vo
 
 template <typename S, typename D> int launch_cast(rt_device* dev, const void* x, void* y, uint64_t numel) {
     if (rt_aligned(x, 16) && rt_aligned(y, 16)) {
-        hipLaunchKernelGGL((cast_vec_kernel<S, D>), dim3(blocks_for(numel / 8, BLOCK * CAST_UNROLL)), dim3(BLOCK), 0, dev->stream,
+        hipLaunchKernelGGL((cast_vec_kernel<S, D>), dim3(blocks_for(numel / 4, BLOCK * CAST_UNROLL)), dim3(BLOCK), 0, dev->stream,
                            (const S*)x, (D*)y, numel);
     } else {
         hipLaunchKernelGGL((cast_scalar_kernel<S, D>), dim3(blocks_for(numel, BLOCK)), dim3(BLOCK), 0, dev->stream,
