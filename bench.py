@@ -28,7 +28,7 @@ sys.path.insert(0, ROOT)
 PEAK_HBM_GBPS = 8000.0
 # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same script (KiB counters scaled by
 # what a 1 GiB copy kernel reads on them, x2.000 and x1.000); bench.py cannot collect counters itself
-PMC_TRAFFIC_BYTES = {"softmax_f16_stream_kernel": int((1050142.0 + 1048100.8) * 1024),
+PMC_TRAFFIC_BYTES = {"softmax16_stream_kernel": int((1050142.0 + 1048100.8) * 1024),
                      "binary_bcast_kernel": int((1081371.9 + 1047757.7) * 1024)}
 F32, F16 = 0, 1
 
@@ -144,7 +144,7 @@ def build_workload(dev, seed):
                        fn=lambda o, n: np.tile(o.binary("add", head, mask), (n // S, 1))), kernel="binary_bcast_kernel"))
     ops.append(Op(3, "softmax (causal)", "f16", "131072x4096", 2 * nb, lambda: dev.softmax(d_masked3, out=d_soft3),
                   dict(kind="rows2", out=d_soft3, rows=16384, tol=0.0, bytes_per_row=2 * S * 2,
-                       fn=lambda o, n: o.softmax(np.tile(o.binary("add", head, mask), (n // S, 1)))), kernel="softmax_f16_stream_kernel"))
+                       fn=lambda o, n: o.softmax(np.tile(o.binary("add", head, mask), (n // S, 1)))), kernel="softmax16_stream_kernel"))
 
     # ------------------------------------------------------------------ cfg 4: broadcast / reindex stress, f16
     kv_a = normal(seed, nxt(), (1, 32, 1984, 80), 1.0, np16)

@@ -22,7 +22,7 @@ struct rt_device {
     int lut_attr_set;
     int gated_attr_set[2];
     unsigned gn_lds_attr_set;
-    unsigned sp_attr_set;   // streaming softmax instantiations whose dynamic-LDS limit has been raised on this device
+    uint64_t sp_attr_set;   // streaming softmax instantiations whose dynamic-LDS limit has been raised on this device
     // caching allocator behind rt_malloc / rt_free (defined in rt_device.hip)
     struct rt_pool* pool;
     int capturing;          // between rt_capture_begin and rt_capture_end

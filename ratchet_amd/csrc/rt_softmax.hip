@@ -274,6 +274,7 @@ __device__ __forceinline__ uint32_t sp_exp_pair(const uint16_t* lut, uint32_t p)
 struct SpSched {
     uint32_t P, GP, reps;
     uint32_t R;              // rows per group actually used (<= SP_ROWS): chosen so that the groups fill whole rounds of the grid
+    uint32_t nsteps;         // 512-column steps per row, rounded up to an even number (used by the long-row variant)
     FastDiv gp_div;
 };
 
@@ -285,14 +286,64 @@ __device__ __forceinline__ void sp_item(const SpSched& s, uint32_t b, uint32_t G
     fd_divmod(b + it * G, s.gp_div, rep, pg);
 }
 
-template <int NSTEP, bool FULL, bool MASK>
-__global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint16_t* __restrict__ table, const half_t* x,
-                                                                      const half_t* mask, half_t* y, uint64_t rows, uint32_t cols,
-                                                                      SpSched sch) {
+// What differs between the two 16-bit types: the walker's running sum and how a packed pair is divided by the row sum.
+template <typename T> struct SpType;
+template <> struct SpType<half_t> {
+    typedef half_t Run;
+    static __device__ __forceinline__ Run zero() { return (half_t)0.0f; }
+    static __device__ __forceinline__ void add_pair(Run& run, uint32_t w) {        // two dependent v_add_f16
+        run = run + bits_h((uint16_t)(w & 0xffffu));
+        run = run + bits_h((uint16_t)(w >> 16));
+    }
+    static __device__ __forceinline__ uint16_t run_bits(Run run) { return h_bits(run); }
+    static __device__ __forceinline__ float widen_bits(uint32_t b) { return (float)bits_h((uint16_t)b); }
+    static __device__ __forceinline__ uint32_t round_pair(float q0, float q1) {
+        const f32x2 q = {q0, q1};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(q, h16x2));
+    }
+    static __device__ __forceinline__ v4u add_vec(const v4u& a, const v4u& b) {    // eight f16 sums, rounded as the separate add does
+        return __builtin_bit_cast(v4u, __builtin_bit_cast(h16x8, a) + __builtin_bit_cast(h16x8, b));
+    }
+    static constexpr bool SHORT_DIVISION = true;
+};
+template <> struct SpType<bf16_t> {
+    typedef float Run;                                                            // always a bf16 value, held widened
+    static __device__ __forceinline__ Run zero() { return 0.0f; }
+    // bf16(a + b): both operands have 16 zero low bits, so a NaN sum has them too and the rounding increment cannot carry
+    // into the exponent; everything else is plain round-to-nearest-even on the bit pattern
+    static __device__ __forceinline__ float add_round(float a, float b) {
+        const uint32_t x = f2u(a + b);
+        return u2f((x + 0x7fffu + ((x >> 16) & 1u)) & 0xffff0000u);
+    }
+    static __device__ __forceinline__ void add_pair(Run& run, uint32_t w) {
+        run = add_round(run, u2f(w << 16));
+        run = add_round(run, u2f(w & 0xffff0000u));
+    }
+    static __device__ __forceinline__ uint16_t run_bits(Run run) { return (uint16_t)(f2u(run) >> 16); }
+    static __device__ __forceinline__ float widen_bits(uint32_t b) { return u2f(b << 16); }
+    static __device__ __forceinline__ uint32_t round_pair(float q0, float q1) { return (uint32_t)f2bf(q0) | ((uint32_t)f2bf(q1) << 16); }
+    static __device__ __forceinline__ v4u add_vec(const v4u& a, const v4u& b) {
+        v4u r;
+#pragma unroll
+        for (int w = 0; w < 4; w++)
+            r[w] = (uint32_t)f2bf(u2f(a[w] << 16) + u2f(b[w] << 16)) | ((uint32_t)f2bf(u2f(a[w] & 0xffff0000u) + u2f(b[w] & 0xffff0000u)) << 16);
+        return r;
+    }
+    static constexpr bool SHORT_DIVISION = false;                                 // the quotient's range is f32's: always the IEEE division
+};
+
+// NSTEP > 0: rows of up to NSTEP * 512 columns, exp values parked in registers.  NSTEP == 0: longer rows; the exp values
+// are parked in y instead and read back (by the thread that wrote them) when the row sum is known: 4 bytes of traffic per
+// element and byte of the type instead of 2, any row length.
+template <typename T, int NSTEP, bool FULL, bool MASK>
+__global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16_t* __restrict__ table, const T* x, const T* mask, T* y,
+                                                                    uint64_t rows, uint32_t cols, SpSched sch) {
+    typedef SpType<T> ST;
+    constexpr bool PARK = NSTEP > 0;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint16_t* lut = reinterpret_cast<uint16_t*>(smem);
-    half_t (*tile)[SP_TC + SP_PAD] = reinterpret_cast<half_t (*)[SP_TC + SP_PAD]>(smem + SP_LUT_BYTES);
-    half_t (*sums)[32] = reinterpret_cast<half_t (*)[32]>(smem + SP_LUT_BYTES + SP_TILE_BYTES);
+    uint16_t (*tile)[SP_TC + SP_PAD] = reinterpret_cast<uint16_t (*)[SP_TC + SP_PAD]>(smem + SP_LUT_BYTES);
+    uint16_t (*sums)[32] = reinterpret_cast<uint16_t (*)[32]>(smem + SP_LUT_BYTES + SP_TILE_BYTES);
 
     // table -> LDS
     {
@@ -302,6 +353,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
         for (uint32_t i = 0; i < SP_LUT_BYTES / 16 / SP_BLOCK; i++) dst[i * SP_BLOCK + threadIdx.x] = src[i * SP_BLOCK + threadIdx.x];
     }
     const uint32_t n_items = sp_item_count(sch, blockIdx.x, gridDim.x);
+    const uint32_t nsteps = PARK ? (uint32_t)NSTEP : sch.nsteps;
     __syncthreads();                                         // table visible
 
     // Every wave passes the same barriers: two per step (A: the walk of the previous tile is over, the tile may be
@@ -312,11 +364,11 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
         const uint32_t lane = threadIdx.x;
         const uint32_t wr = lane < SP_ROWS ? lane : 0;       // lanes 30..63 shadow row 0 and never publish
         const v4u* trow = reinterpret_cast<const v4u*>(tile[wr]);
-        half_t run = (half_t)0.0f;
+        typename ST::Run run = ST::zero();
         uint32_t gpar = 0;
         for (uint32_t it = 0; it < n_items; it++) {
 #pragma unroll 1
-            for (int t = 0; t < NSTEP; t++) {
+            for (uint32_t t = 0; t < nsteps; t++) {
                 __syncthreads();                             // A
                 __syncthreads();                             // B: tile t is in LDS
                 // 16 values per chunk; the LDS reads of the next chunk are in flight during the 16 dependent adds
@@ -329,21 +381,15 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
                         n1 = trow[(c + 1) * 2 + 1];
                     }
 #pragma unroll
-                    for (int w = 0; w < 4; w++) {
-                        run = run + bits_h((uint16_t)(c0[w] & 0xffffu));
-                        run = run + bits_h((uint16_t)(c0[w] >> 16));
-                    }
+                    for (int w = 0; w < 4; w++) ST::add_pair(run, c0[w]);
 #pragma unroll
-                    for (int w = 0; w < 4; w++) {
-                        run = run + bits_h((uint16_t)(c1[w] & 0xffffu));
-                        run = run + bits_h((uint16_t)(c1[w] >> 16));
-                    }
+                    for (int w = 0; w < 4; w++) ST::add_pair(run, c1[w]);
                     c0 = n0;
                     c1 = n1;
                 }
             }
-            if (lane < SP_ROWS) sums[gpar][lane] = run;
-            run = (half_t)0.0f;
+            if (lane < SP_ROWS) sums[gpar][lane] = ST::run_bits(run);
+            run = ST::zero();
             gpar ^= 1;
         }
         __syncthreads();                                     // after the last group: its sums are published
@@ -361,12 +407,11 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
     const uint32_t ccol = (lt & 63) * 8;                     // column of this thread's vectors inside a step
     const uint32_t row_bytes = cols * 2;
     const uint32_t nbytes = (uint32_t)(rows * row_bytes);    // the launcher keeps this below 2^31
-    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(x), 0, nbytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(x), 0, nbytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(y, 0, nbytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t rm =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(MASK ? mask : x), 0, MASK ? sch.P * row_bytes : nbytes, 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(MASK ? mask : x), 0, MASK ? sch.P * row_bytes : nbytes, 0x00020000);
     constexpr uint32_t OOB = 0x80000000u;                    // >= nbytes, and stays so after adding a column offset
-    constexpr int PF = NSTEP < SP_PF ? NSTEP : SP_PF;        // steps of x in flight per thread
     const uint32_t G = gridDim.x;
 
     // Row offsets are the same for all lanes of a wave, so they live in scalar registers (the vector registers are all
@@ -386,43 +431,25 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
         }
     };
     const uint32_t cbyte = ccol * 2;
-    auto step_off = [&](uint32_t row_off, int t) -> uint32_t {   // per-lane offset of this thread's vector in step t of a row
-        if (!FULL && (uint32_t)t * SP_TC + ccol >= cols) return OOB;
-        return row_off + (uint32_t)t * (SP_TC * 2) + cbyte;
+    auto past_end = [&](uint32_t t) -> bool { return !(PARK && FULL) && t * SP_TC + ccol >= cols; };
+    auto step_off = [&](uint32_t row_off, uint32_t t) -> uint32_t {   // per-lane offset of this thread's vector in step t of a row
+        if (past_end(t)) return OOB;
+        return row_off + t * (SP_TC * 2) + cbyte;
     };
     auto load_x = [&](uint32_t off) -> v4u { return __builtin_amdgcn_raw_buffer_load_b128(rx, off, 0, 2); };   // 2: non-temporal
     auto load_m = [&](uint32_t off) -> v4u { return __builtin_amdgcn_raw_buffer_load_b128(rm, off, 0, 0); };   // re-read by other heads
-
-    uint32_t cur[2], nxt[2], prev[2] = {OOB, OOB}, pcur, pnxt;
-    item_off(0, cur, pcur);
-    item_off(1, nxt, pnxt);
-    v4u e[NSTEP][2];                                         // exp values of the group in flight, 8 halves per vector
-    v4u pre[PF][2], mpre[2];                                 // x: PF steps in flight; mask: one (L2 hits: a short distance is enough)
-#pragma unroll
-    for (int t = 0; t < NSTEP; t++) e[t][0] = e[t][1] = v4u{0, 0, 0, 0};
-    // The pending memory operations at the top of the group loop are the same on entry as after a group (two loads, two
-    // stores, two loads, two stores: the stores here go nowhere), so the compiler can count them there too.
-#pragma unroll
-    for (int k = 0; k < PF; k++) {
-#pragma unroll
-        for (int h = 0; h < 2; h++) pre[k][h] = load_x(step_off(cur[h], k));
-#pragma unroll
-        for (int h = 0; h < 2; h++) __builtin_amdgcn_raw_buffer_store_b128(v4u{0, 0, 0, 0}, ry, OOB, 0, 2);
-    }
-    if (MASK) {
-#pragma unroll
-        for (int h = 0; h < 2; h++) mpre[h] = load_m(step_off(cur[h] - pcur, 0));
-    }
+    auto load_y = [&](uint32_t off) -> v4u { return __builtin_amdgcn_raw_buffer_load_b128(ry, off, 0, 0); };
+    auto store_y = [&](const v4u& v, uint32_t off) { __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, 2); };      // results: non-temporal
+    auto store_park = [&](const v4u& v, uint32_t off) { __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, 0); };   // read back soon
 
     // sum of the previous group's rows, reciprocal, and whether the short division applies: wave-uniform as well
     float s_prev[2] = {1.0f, 1.0f}, rinv_prev[2] = {1.0f, 1.0f};
     bool fast_prev[2] = {true, true};
-    uint32_t gpar = 0;
 
     auto quotients = [&](const v4u& ev, int h) -> v4u {      // e / sum of the previous group
         v4u out;
         const float s = s_prev[h], rinv = rinv_prev[h];
-        if (fast_prev[h]) {
+        if (ST::SHORT_DIVISION && fast_prev[h]) {
 #pragma unroll
             for (int w = 0; w < 4; w++) {
                 // v_fma_mix_f32 reads the f16 halves of ev[w] directly: a = e * r (+0), rem = e - s * a; no separate conversions
@@ -436,86 +463,183 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax_f16_stream_kernel(const uint
                 // keep the f32 quotient and its conversion apart: fused into v_fma_mixlo_f16 the pair rounds
                 // subnormal f16 results differently from fma-then-convert
                 asm volatile("" : "+v"(q0), "+v"(q1));
-                const f32x2 q = {q0, q1};
-                out[w] = __builtin_bit_cast(uint32_t, __builtin_convertvector(q, h16x2));
+                out[w] = ST::round_pair(q0, q1);
             }
         } else {
 #pragma unroll
-            for (int w = 0; w < 4; w++) {
-                const float e0 = (float)bits_h((uint16_t)(ev[w] & 0xffffu)), e1 = (float)bits_h((uint16_t)(ev[w] >> 16));
-                out[w] = (uint32_t)h_bits((half_t)(e0 / s)) | ((uint32_t)h_bits((half_t)(e1 / s)) << 16);
-            }
+            for (int w = 0; w < 4; w++) out[w] = ST::round_pair(ST::widen_bits(ev[w] & 0xffffu) / s, ST::widen_bits(ev[w] >> 16) / s);
         }
         return out;
     };
     auto read_prev_sum = [&](uint32_t par) {
 #pragma unroll
         for (int h = 0; h < 2; h++) {
-            const uint32_t sb = __builtin_amdgcn_readfirstlane((uint32_t)h_bits(sums[par][rr + h * SP_HALF]));
-            const float s = (float)bits_h((uint16_t)sb);
+            const uint32_t sb = __builtin_amdgcn_readfirstlane((uint32_t)sums[par][rr + h * SP_HALF]);
+            const float s = ST::widen_bits(sb);
             s_prev[h] = s;
             // normal, finite, not tiny: the reciprocal-plus-correction quotient is exact there
             fast_prev[h] = (s >= 6.103515625e-05f) && (s < __builtin_huge_valf());
             rinv_prev[h] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, fast_prev[h] ? 1.0f / s : 0.0f)));
         }
     };
+    // exp of the vector that arrived, in place (zeros past the row end: adding +0 is a no-op; rows past the tensor's end
+    // read zeros and their sums are never used)
+    auto exp_in_place = [&](v4u& in, const v4u& m, uint32_t t) {
+        if (MASK) in = ST::add_vec(in, m);                   // scores + mask in the 16-bit type, as the separate add would round it
+#pragma unroll
+        for (int w = 0; w < 4; w++) in[w] = sp_exp_pair(lut, in[w]);
+        if (past_end(t)) in = v4u{0, 0, 0, 0};
+    };
 
-    for (uint32_t it = 0; it < n_items; it++) {
+    uint32_t cur[2], nxt[2], prev[2] = {OOB, OOB}, pcur, pnxt;
+    item_off(0, cur, pcur);
+    item_off(1, nxt, pnxt);
+    uint32_t gpar = 0;
+
+    if constexpr (PARK) {
+        constexpr int PF = NSTEP < SP_PF ? NSTEP : SP_PF;    // steps of x in flight per thread
+        v4u e[NSTEP][2];                                     // exp values of the group in flight, 8 halves per vector
+        v4u pre[PF][2], mpre[2];                             // x: PF steps in flight; mask: one (L2 hits: a short distance is enough)
 #pragma unroll
-        for (int t = 0; t < NSTEP; t++) {
-            // exp of the vectors that arrived, in place (zeros past the row end: adding +0 is a no-op; rows past the
-            // tensor's end read zeros and their sums are never used)
+        for (int t = 0; t < NSTEP; t++) e[t][0] = e[t][1] = v4u{0, 0, 0, 0};
+        // The pending memory operations at the top of the group loop are the same on entry as after a group (two loads, two
+        // stores, two loads, two stores: the stores here go nowhere), so the compiler can count them there too.
 #pragma unroll
-            for (int h = 0; h < 2; h++) {
-                v4u& in = pre[t % PF][h];
-                if (MASK) {                                  // scores + mask in f16, as the separate add would round it
-                    const h16x8 sum = __builtin_bit_cast(h16x8, in) + __builtin_bit_cast(h16x8, mpre[h]);
-                    in = __builtin_bit_cast(v4u, sum);
+        for (int k = 0; k < PF; k++) {
+#pragma unroll
+            for (int h = 0; h < 2; h++) pre[k][h] = load_x(step_off(cur[h], k));
+#pragma unroll
+            for (int h = 0; h < 2; h++) store_y(v4u{0, 0, 0, 0}, OOB);
+        }
+        if (MASK) {
+#pragma unroll
+            for (int h = 0; h < 2; h++) mpre[h] = load_m(step_off(cur[h] - pcur, 0));
+        }
+
+        for (uint32_t it = 0; it < n_items; it++) {
+#pragma unroll
+            for (int t = 0; t < NSTEP; t++) {
+#pragma unroll
+                for (int h = 0; h < 2; h++) exp_in_place(pre[t % PF][h], mpre[h], t);
+                __syncthreads();                             // A: wave 0 has left the previous tile
+                *reinterpret_cast<v4u*>(&tile[rr][ccol]) = pre[t % PF][0];
+                *reinterpret_cast<v4u*>(&tile[rr + SP_HALF][ccol]) = pre[t % PF][1];
+                // the registers are free again: next loads, PF steps ahead, possibly in the block's next group
+                // (loads return in order: the mask of the next step goes first, so that waiting for it does not wait for x
+                // of the step after)
+                if (MASK) {
+#pragma unroll
+                    for (int h = 0; h < 2; h++)
+                        mpre[h] = (t + 1 < NSTEP) ? load_m(step_off(cur[h] - pcur, t + 1)) : load_m(step_off(nxt[h] - pnxt, 0));
                 }
 #pragma unroll
-                for (int w = 0; w < 4; w++) in[w] = sp_exp_pair(lut, in[w]);
-                if (!FULL && (uint32_t)t * SP_TC + ccol >= cols) in = v4u{0, 0, 0, 0};
-            }
-            __syncthreads();                                 // A: wave 0 has left the previous tile
-            *reinterpret_cast<v4u*>(&tile[rr][ccol]) = pre[t % PF][0];
-            *reinterpret_cast<v4u*>(&tile[rr + SP_HALF][ccol]) = pre[t % PF][1];
-            // the registers are free again: next loads, PF steps ahead, possibly in the block's next group
-            // (loads return in order: the mask of the next step goes first, so that waiting for it does not wait for x of
-            // the step after)
-            if (MASK) {
-#pragma unroll
                 for (int h = 0; h < 2; h++)
-                    mpre[h] = (t + 1 < NSTEP) ? load_m(step_off(cur[h] - pcur, t + 1)) : load_m(step_off(nxt[h] - pnxt, 0));
-            }
+                    pre[t % PF][h] = (t + PF < NSTEP) ? load_x(step_off(cur[h], t + PF)) : load_x(step_off(nxt[h], t + PF - NSTEP));
+                __syncthreads();                             // B: parked for the walk
+                if (t == 0) read_prev_sum(gpar ^ 1);         // published by wave 0 before it reached barrier A
 #pragma unroll
-            for (int h = 0; h < 2; h++)
-                pre[t % PF][h] = (t + PF < NSTEP) ? load_x(step_off(cur[h], t + PF)) : load_x(step_off(nxt[h], t + PF - NSTEP));
-            __syncthreads();                                 // B: parked for the walk
-            if (t == 0) read_prev_sum(gpar ^ 1);             // published by wave 0 before it reached barrier A
+                for (int h = 0; h < 2; h++) {
+                    store_y(quotients(e[t][h], h), step_off(prev[h], t));   // first group: prev is OOB, the store is dropped
+                    // this group's values come back from the tile, which stays intact until the next barrier A
+                    e[t][h] = *reinterpret_cast<const v4u*>(&tile[rr + h * SP_HALF][ccol]);
+                }
+            }
 #pragma unroll
             for (int h = 0; h < 2; h++) {
-                const v4u out = quotients(e[t][h], h);       // first group: prev is OOB, the store is dropped
-                __builtin_amdgcn_raw_buffer_store_b128(out, ry, step_off(prev[h], t), 0, 2);
-                // this group's values come back from the tile, which stays intact until the next barrier A
-                e[t][h] = *reinterpret_cast<const v4u*>(&tile[rr + h * SP_HALF][ccol]);
+                prev[h] = cur[h];
+                cur[h] = nxt[h];
+            }
+            pcur = pnxt;
+            item_off(it + 2, nxt, pnxt);
+            gpar ^= 1;
+        }
+        // drain: outputs of the block's last group
+        __syncthreads();
+        read_prev_sum(gpar ^ 1);
+#pragma unroll
+        for (int t = 0; t < NSTEP; t++)
+#pragma unroll
+            for (int h = 0; h < 2; h++) store_y(quotients(e[t][h], h), step_off(prev[h], t));
+    } else {
+        // One flat loop over the steps of all groups, two steps per trip (nsteps is even; a step past the row end moves
+        // nothing).  Per step and row: exp values to the tile and to y, x of two steps ahead, the previous group's exp
+        // values of this step (loaded two steps ago from y, where this thread put them a group ago) divided and stored,
+        // and the load of those of two steps ahead.  The prologue issues the same sequence with targets that do not exist.
+        v4u pre[2][2], qpre[2][2], mpre[2];
+        uint32_t qnext[2] = {OOB, OOB};                      // rows whose parked values the next two loads fetch: prev, then cur
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+#pragma unroll
+            for (int h = 0; h < 2; h++) store_park(v4u{0, 0, 0, 0}, OOB);
+            if (MASK) {
+#pragma unroll
+                for (int h = 0; h < 2; h++) mpre[h] = load_m(step_off(cur[h] - pcur, 0));
+            }
+#pragma unroll
+            for (int h = 0; h < 2; h++) pre[k][h] = load_x(step_off(cur[h], k));
+#pragma unroll
+            for (int h = 0; h < 2; h++) store_y(v4u{0, 0, 0, 0}, OOB);
+#pragma unroll
+            for (int h = 0; h < 2; h++) qpre[k][h] = load_y(OOB);
+        }
+        uint32_t t0 = 0;                                     // first step of the trip within its group
+        const uint32_t trips = n_items * (nsteps / 2);
+        for (uint32_t trip = 0; trip < trips; trip++) {
+#pragma unroll
+            for (int k = 0; k < 2; k++) {
+                const uint32_t t = t0 + k;
+#pragma unroll
+                for (int h = 0; h < 2; h++) exp_in_place(pre[k][h], mpre[h], t);
+                __syncthreads();                             // A
+                *reinterpret_cast<v4u*>(&tile[rr][ccol]) = pre[k][0];
+                *reinterpret_cast<v4u*>(&tile[rr + SP_HALF][ccol]) = pre[k][1];
+#pragma unroll
+                for (int h = 0; h < 2; h++) store_park(pre[k][h], step_off(cur[h], t));      // parked in y (kept in cache: read back soon)
+                const bool wrap = t + 2 >= nsteps;           // two steps ahead is in the block's next group
+                const uint32_t ta = wrap ? t + 2 - nsteps : t + 2;
+                if (MASK) {
+                    const bool w1 = t + 1 >= nsteps;
+#pragma unroll
+                    for (int h = 0; h < 2; h++) mpre[h] = load_m(step_off(w1 ? nxt[h] - pnxt : cur[h] - pcur, w1 ? 0 : t + 1));
+                }
+#pragma unroll
+                for (int h = 0; h < 2; h++) pre[k][h] = load_x(step_off(wrap ? nxt[h] : cur[h], ta));
+                __syncthreads();                             // B
+                if (t == 0) read_prev_sum(gpar ^ 1);
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    store_y(quotients(qpre[k][h], h), step_off(prev[h], t));
+                    qpre[k][h] = load_y(step_off(wrap ? cur[h] : prev[h], ta));
+                }
+            }
+            t0 += 2;
+            if (t0 >= nsteps) {                              // next group
+                t0 = 0;
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    prev[h] = cur[h];
+                    cur[h] = nxt[h];
+                }
+                pcur = pnxt;
+                item_off(trip / (nsteps / 2) + 2, nxt, pnxt);
+                gpar ^= 1;
             }
         }
+        // drain: the last group's parked values (steps 0 and 1 are already here; the values of the last steps were stored
+        // a moment ago, so everything this wave has in flight completes first)
+        __syncthreads();
+        __builtin_amdgcn_s_waitcnt(0);
+        read_prev_sum(gpar ^ 1);
+        for (uint32_t t = 0; t < nsteps; t += 2) {
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
-            prev[h] = cur[h];
-            cur[h] = nxt[h];
+            for (int k = 0; k < 2; k++)
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    store_y(quotients(qpre[k][h], h), step_off(prev[h], t + k));
+                    qpre[k][h] = load_y(step_off(prev[h], t + k + 2 < nsteps ? t + k + 2 : 0xffffu));
+                }
         }
-        pcur = pnxt;
-        item_off(it + 2, nxt, pnxt);
-        gpar ^= 1;
     }
-    // drain: outputs of the block's last group
-    __syncthreads();
-    read_prev_sum(gpar ^ 1);
-#pragma unroll
-    for (int t = 0; t < NSTEP; t++)
-#pragma unroll
-        for (int h = 0; h < 2; h++) __builtin_amdgcn_raw_buffer_store_b128(quotients(e[t][h], h), ry, step_off(prev[h], t), 0, 2);
 }
 
 // ------------------------------------------------------------------------------------------------------------------
@@ -710,8 +834,10 @@ template <typename T, int MODE> int launch_f32_style(rt_device* dev, const void*
 
 // mask == nullptr: plain softmax.  Otherwise the mask has `period` rows of `cols` columns and repeats every `period`
 // rows of x (rows % period == 0).  Returns RT_OK with *done = false when the shape does not fit this kernel.
-int launch_f16_stream(rt_device* dev, const void* x, const void* mask, uint64_t period, void* y, uint64_t rows, uint32_t cols, bool* done) {
+template <typename T>
+int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t period, void* y, uint64_t rows, uint32_t cols, bool* done) {
     *done = false;
+    constexpr int TI = sizeof(typename SpType<T>::Run) == 4 ? 1 : 0;         // table and attribute index: 0 f16, 1 bf16
     const uint64_t row_bytes = (uint64_t)cols * 2;
     if (!mask) period = rows;
     // the kernel addresses a launch with 32-bit byte offsets below 2^31: larger tensors go in chunks of whole periods
@@ -722,22 +848,23 @@ int launch_f16_stream(rt_device* dev, const void* x, const void* mask, uint64_t 
         chunk_rows = (0x7fffffffull / (period * row_bytes)) * period;
     } else {
         chunk_rows = (0x7fffffffull / row_bytes) / SP_ROWS * SP_ROWS;
+        if (chunk_rows == 0) return RT_OK;
     }
     const uint16_t* table = nullptr;
-    int rc = rt_unary_table(dev, 0, RT_EXP, &table);
+    int rc = rt_unary_table(dev, TI, RT_EXP, &table);
     if (rc) return rc;
     const uint32_t nt = (cols + SP_TC - 1) / SP_TC;
     const bool full = cols % SP_TC == 0 && (nt == 1 || nt == 2 || nt == 4 || nt == 8);
 #define RT_SP(NS, F, M)                                                                                                              \
     do {                                                                                                                             \
-        const unsigned bit = 1u << ((NS == 1 ? 0 : NS == 2 ? 1 : NS == 4 ? 2 : 3) + (F ? 4 : 0) + (M ? 8 : 0));                      \
+        const uint64_t bit = 1ull << (TI * 20 + (NS == 0 ? 4 : NS == 1 ? 0 : NS == 2 ? 1 : NS == 4 ? 2 : 3) * 4 + (F ? 2 : 0) + (M ? 1 : 0)); \
         if (!(dev->sp_attr_set & bit)) {               /* the LDS opt-in is per function and per device */                           \
-            RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(softmax_f16_stream_kernel<NS, F, M>),                           \
+            RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(softmax16_stream_kernel<T, NS, F, M>),                          \
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)SP_SMEM_BYTES));                             \
             dev->sp_attr_set |= bit;                                                                                                 \
         }                                                                                                                            \
-        hipLaunchKernelGGL((softmax_f16_stream_kernel<NS, F, M>), dim3(blocks), dim3(SP_BLOCK), SP_SMEM_BYTES, dev->stream, table,   \
-                           xc, (const half_t*)mask, yc, n, cols, sch);                                                               \
+        hipLaunchKernelGGL((softmax16_stream_kernel<T, NS, F, M>), dim3(blocks), dim3(SP_BLOCK), SP_SMEM_BYTES, dev->stream, table,  \
+                           xc, (const T*)mask, yc, n, cols, sch);                                                                    \
     } while (0)
 #define RT_SP_NS(F, M)                                      \
     do {                                                    \
@@ -748,23 +875,26 @@ int launch_f16_stream(rt_device* dev, const void* x, const void* mask, uint64_t 
     } while (0)
     for (uint64_t row0 = 0; row0 < rows; row0 += chunk_rows) {
         const uint64_t n = rows - row0 < chunk_rows ? rows - row0 : chunk_rows;
-        const half_t* xc = (const half_t*)x + row0 * cols;
-        half_t* yc = (half_t*)y + row0 * cols;
+        const T* xc = (const T*)x + row0 * cols;
+        T* yc = (T*)y + row0 * cols;
         SpSched sch;
         sch.P = (uint32_t)(mask ? period : n);
         sch.reps = (uint32_t)(n / sch.P);
+        sch.nsteps = (nt + 1) & ~1u;
         // rows per group: every block runs ceil(groups / grid) rounds of 8-or-fewer steps whatever the group holds, so
         // 4370 groups of 30 rows on 256 CUs cost 18 rounds where 17.07 are needed; 27-row groups make 19 full rounds.
-        // Pick the size that minimises rounds x rows (time is proportional to the rows a round could have carried).
-        // Few rows (a decode step's [B * H, T] scores) spread over the CUs the same way: 32 rows run as 32 one-row groups.
+        // A step takes the longer of the walk (1.5 us whatever the group holds) and the group's memory time (2 KiB per
+        // row at a CU's share of the bandwidth: about 0.09 us per row), so a round costs max(R + 1, 18) in units of a
+        // row's memory time; pick the size with the cheapest total, the smallest such size on a tie.  Few rows (a decode
+        // step's [B * H, T] scores) spread over the CUs the same way: 32 rows run as 32 one-row groups.
         {
             uint64_t best = ~0ull;
             sch.R = SP_ROWS;
             for (uint32_t R = SP_ROWS; R >= 1; R--) {
                 const uint64_t groups = (uint64_t)((sch.P + R - 1) / R) * sch.reps;
                 const uint64_t rounds = (groups + dev->num_cus - 1) / dev->num_cus;
-                const uint64_t cost = rounds * R + rounds / 4;          // the small second term: a round has a fixed cost too
-                if (cost < best) {
+                const uint64_t cost = rounds * (R + 1 > 18 ? R + 1 : 18);
+                if (cost <= best) {
                     best = cost;
                     sch.R = R;
                 }
@@ -775,14 +905,17 @@ int launch_f16_stream(rt_device* dev, const void* x, const void* mask, uint64_t 
         const uint64_t items = (uint64_t)sch.GP * sch.reps;
         RT_REQUIRE(items <= 0xffffffffull, RT_ERR_SIZE, "rt_softmax: too many row groups");
         const unsigned blocks = (unsigned)(items < (uint64_t)dev->num_cus ? items : (uint64_t)dev->num_cus);   // one resident block per CU
-        if (mask) {
+        if (nt > SP_MAX_STEPS) {                         // long rows: exp values parked in y
+            if (mask) RT_SP(0, false, true);
+            else RT_SP(0, false, false);
+        } else if (mask) {
             if (full) RT_SP_NS(true, true);
             else RT_SP_NS(false, true);
         } else {
             if (full) RT_SP_NS(true, false);
             else RT_SP_NS(false, false);
         }
-        RT_CHECK_LAUNCH("softmax_f16_stream_kernel");
+        RT_CHECK_LAUNCH("softmax16_stream_kernel");
     }
 #undef RT_SP_NS
 #undef RT_SP
@@ -925,17 +1058,18 @@ extern "C" int rt_softmax(rt_device* dev, int dt, const void* x, void* y, uint64
     }
     switch (dt) {
         case RT_F32: return launch_f32_style<float, 0>(dev, x, y, rows, cols);
-        case RT_F16:
-            // rows of up to 4096 columns that are whole aligned vectors stream through registers in one pass (also small
-            // problems: the per-block table load costs about 5 us, the two-pass walker more); everything else takes
-            // the two-pass tile walker
-            if (cols % 8 == 0 && cols <= SP_MAX_STEPS * SP_TC && rt_aligned(x, 16) && rt_aligned(y, 16)) {
+        default: {
+            // 16-bit types, rows that are whole aligned vectors: one pass, rows of up to 4096 columns held in registers,
+            // longer ones parked in y (also small problems: the per-block table load costs about 5 us, the two-pass walker
+            // more); everything else takes the two-pass tile walker
+            if (cols % 8 == 0 && rt_aligned(x, 16) && rt_aligned(y, 16)) {
                 bool done = false;
-                rc = launch_f16_stream(dev, x, nullptr, 0, y, rows, cols, &done);
+                rc = dt == RT_F16 ? launch_stream16<half_t>(dev, x, nullptr, 0, y, rows, cols, &done)
+                                  : launch_stream16<bf16_t>(dev, x, nullptr, 0, y, rows, cols, &done);
                 if (rc || done) return rc;
             }
-            return launch_seq16<half_t>(dev, x, y, rows, cols);
-        default: return launch_seq16<bf16_t>(dev, x, y, rows, cols);
+            return dt == RT_F16 ? launch_seq16<half_t>(dev, x, y, rows, cols) : launch_seq16<bf16_t>(dev, x, y, rows, cols);
+        }
     }
 }
 
@@ -969,10 +1103,11 @@ extern "C" int rt_softmax_masked(rt_device* dev, int dt, const void* x, const ui
         if (mask_shape[i] != x_shape[i]) whole = false;
         period *= x_shape[i];
     }
-    if (dt == RT_F16 && mode == RT_SOFTMAX_REFERENCE && whole && cols % 8 == 0 && cols <= SP_MAX_STEPS * SP_TC &&
-        rt_aligned(x, 16) && rt_aligned(y, 16) && rt_aligned(mask, 16)) {
+    if (dt != RT_F32 && mode == RT_SOFTMAX_REFERENCE && whole && cols % 8 == 0 && rt_aligned(x, 16) && rt_aligned(y, 16) &&
+        rt_aligned(mask, 16)) {
         bool done = false;
-        rc = launch_f16_stream(dev, x, mask, period, y, rows, cols, &done);
+        rc = dt == RT_F16 ? launch_stream16<half_t>(dev, x, mask, period, y, rows, cols, &done)
+                          : launch_stream16<bf16_t>(dev, x, mask, period, y, rows, cols, &done);
         if (rc || done) return rc;
     }
     // otherwise the two ops, the sum parked in y

@@ -113,6 +113,71 @@ def test_softmax_f16_streaming_kernel_beyond_2_gib(dev, oracle):
     assert same_bits(got[: reps * 1021].reshape(reps, 1021, n), np.broadcast_to(want_block, (reps, 1021, n)))
 
 
+def _bf16(oracle, a):
+    return oracle.cast(np.asarray(a, np.float32), np.uint16, dst_bf16=True)
+
+
+def _special_rows(flat, n):
+    """the edge rows of test_softmax_f16_streaming_kernel, on an f32 array that is rounded to the 16-bit type afterwards"""
+    for i in range(0, flat.shape[0], 3):
+        flat[i, (i * 37) % n + 1:] = -np.inf
+    flat[5, 7] = 95.0                                                   # overflows both 16-bit types' exp: inf sum, NaN there
+    flat[11, :] = -np.inf
+    flat[13, 3] = np.nan
+    flat[17, :] = -110.0                                                # every exp underflows to 0 (bf16 and f16)
+    flat[19, :] = -16.0                                                 # subnormal exps in f16
+    flat[-1, : n // 2] = -12.0
+
+
+@pytest.mark.parametrize("shape", [(1, 300, 4096), (2, 601, 1000), (1, 2100, 512), (32, 1, 4096), (1, 20, 8), (1, 31, 2056), (16, 61, 72)])
+def test_softmax_bf16_streaming_kernel(dev, oracle, shape):
+    """bf16 rows that are whole vectors take the same single-pass kernel: the sum is the reference's sequence of
+    bf16(f32(sum) + f32(e)), the quotient bf16(f32(e) / f32(sum))."""
+    rng = np.random.default_rng(305)
+    n = shape[-1]
+    xf = (rng.standard_normal(shape) * 2).astype(np.float32)
+    _special_rows(xf.reshape(-1, n), n)
+    xb = _bf16(oracle, xf)
+    want = oracle.softmax(xb, bf16=True)
+    dx = dev.upload(xb, bf16=True)
+    got = dev.softmax(dx).to_numpy()
+    isnan = lambda b: (b & 0x7fff) > 0x7f80
+    bad = (got != want) & ~(isnan(got) & isnan(want))
+    assert not bad.any(), (shape, int(bad.sum()), np.flatnonzero(bad.reshape(-1))[:8], got.reshape(-1)[bad.reshape(-1)][:8], want.reshape(-1)[bad.reshape(-1)][:8])
+    dev.softmax(dx, out=dx)
+    got2 = dx.to_numpy()
+    assert not ((got2 != want) & ~(isnan(got2) & isnan(want))).any()
+
+
+@pytest.mark.parametrize("shape,kind", [((1, 70, 8192), "f16"), ((2, 33, 4104), "f16"), ((1, 3, 51200), "f16"), ((1, 100, 6008), "f16"),
+                                        ((1, 40, 8192), "bf16"), ((1, 5, 20000), "bf16")])
+def test_softmax_16_bit_long_rows(dev, oracle, shape, kind):
+    """rows of more than 4096 columns: the exp values are parked in y and read back once the row sum is known; also in place"""
+    rng = np.random.default_rng(306)
+    n = shape[-1]
+    xf = (rng.standard_normal(shape) * 2).astype(np.float32)
+    _special_rows(xf.reshape(-1, n), n) if xf.reshape(-1, n).shape[0] >= 20 else None
+    xf.reshape(-1, n)[0, n // 3:] = -np.inf
+    if kind == "f16":
+        x = xf.astype(np.float16)
+        want = oracle.softmax(x)
+        dx = dev.upload(x)
+        got = dev.softmax(dx).to_numpy()
+        assert mismatch_count(got, want) == 0, (shape, describe_mismatch(got, want, x))
+        dev.softmax(dx, out=dx)
+        assert same_bits(dx.to_numpy(), want)
+    else:
+        xb = _bf16(oracle, xf)
+        want = oracle.softmax(xb, bf16=True)
+        dx = dev.upload(xb, bf16=True)
+        isnan = lambda b: (b & 0x7fff) > 0x7f80
+        got = dev.softmax(dx).to_numpy()
+        assert not ((got != want) & ~(isnan(got) & isnan(want))).any(), shape
+        dev.softmax(dx, out=dx)
+        got = dx.to_numpy()
+        assert not ((got != want) & ~(isnan(got) & isnan(want))).any(), shape
+
+
 def test_softmax_f16_order_dependence_is_reproduced(dev, oracle):
     # 2048 + 1 + 1 + ... never grows in f16: the kernel must reproduce that, not the mathematically exact sum
     row = np.zeros(512, np.float16)
@@ -257,6 +322,34 @@ def test_softmax_masked_equals_add_then_softmax(dev, oracle, shape, mshape):
     assert same_bits(got, two)
     dev.softmax_masked(dx, dm, out=dx)                                 # in place
     assert same_bits(dx.to_numpy(), got)
+
+
+@pytest.mark.parametrize("shape,mshape,kind", [((1, 4, 50, 8192), (50, 8192), "f16"), ((2, 2, 33, 4200), (1, 1, 33, 4200), "f16"),
+                                               ((1, 8, 128, 512), (128, 512), "bf16"), ((1, 3, 40, 6000), (40, 6000), "bf16")])
+def test_softmax_masked_long_rows_and_bf16(dev, oracle, shape, mshape, kind):
+    """the one-launch masked softmax beyond 4096 columns (values parked in y) and in bf16: the bits of add-then-softmax"""
+    rng = np.random.default_rng(322)
+    bf = kind == "bf16"
+    S, T = mshape[-2], mshape[-1]
+    xf = (rng.standard_normal(shape) * 2).astype(np.float32)
+    mf = np.triu(np.full((S, T), -np.inf, np.float32), k=1 + max(T - S, 0))
+    mf[S // 2, :] = rng.standard_normal(T).astype(np.float32)
+    mf = np.ascontiguousarray(np.broadcast_to(mf, mshape))
+    if bf:
+        x, m = _bf16(oracle, xf), _bf16(oracle, mf)
+    else:
+        x, m = xf.astype(np.float16), mf.astype(np.float16)
+    full_mask = np.ascontiguousarray(np.broadcast_to(m.reshape((1,) * (4 - m.ndim) + m.shape), shape))
+    want = oracle.softmax(oracle.binary("add", x, full_mask, bf16=bf), bf16=bf)
+    dx, dm = dev.upload(x, bf16=bf), dev.upload(m, bf16=bf)
+    got = dev.softmax_masked(dx, dm).to_numpy()
+    if bf:
+        isnan = lambda b: (b & 0x7fff) > 0x7f80
+        assert not ((got != want) & ~(isnan(got) & isnan(want))).any(), (shape, mshape)
+    else:
+        assert mismatch_count(got, want) == 0, (shape, mshape, describe_mismatch(got, want, x))
+    dev.softmax_masked(dx, dm, out=dx)                                 # in place
+    assert np.array_equal(dx.to_numpy().view(np.uint16), got.view(np.uint16))
 
 
 def test_softmax_masked_other_types_and_modes(dev, oracle):
