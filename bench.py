@@ -28,8 +28,8 @@ sys.path.insert(0, ROOT)
 PEAK_HBM_GBPS = 8000.0
 # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same script (KiB counters scaled by
 # what a 1 GiB copy kernel reads on them, x2.000 and x1.000); bench.py cannot collect counters itself
-PMC_TRAFFIC_BYTES = {"softmax16_stream_kernel": int((1050142.0 + 1048100.8) * 1024),
-                     "binary_bcast_kernel": int((1081371.9 + 1047757.7) * 1024)}
+PMC_TRAFFIC_BYTES = {"softmax16_stream_kernel": int((1050201.0 + 1048126.2) * 1024),
+                     "binary_bcast_kernel": int((1081372.1 + 1047819.4) * 1024)}
 F32, F16 = 0, 1
 
 
