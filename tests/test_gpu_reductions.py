@@ -178,6 +178,29 @@ def test_softmax_16_bit_long_rows(dev, oracle, shape, kind):
         assert not ((got != want) & ~(isnan(got) & isnan(want))).any(), shape
 
 
+@pytest.mark.parametrize("rows,cols,kind", [(40000, 8, "f16"), (33001, 72, "f16"), (32768 + 5, 128, "f16"), (50000, 24, "bf16"), (32800, 104, "bf16")])
+def test_softmax_16_bit_many_narrow_rows(dev, oracle, rows, cols, kind):
+    """tens of thousands of rows of at most 128 columns: the kernel with one lane per row; also in place"""
+    rng = np.random.default_rng(307)
+    xf = (rng.standard_normal((rows, cols)) * 2).astype(np.float32)
+    _special_rows(xf, cols)
+    xf[rows - 2, :] = 95.0 if kind == "bf16" else 12.0                  # a row in the last (partial) block that overflows
+    bf = kind == "bf16"
+    x = _bf16(oracle, xf) if bf else xf.astype(np.float16)
+    want = oracle.softmax(x, bf16=bf)
+    dx = dev.upload(x, bf16=bf)
+    got = dev.softmax(dx).to_numpy()
+    dev.softmax(dx, out=dx)
+    got2 = dx.to_numpy()
+    if bf:
+        isnan = lambda b: (b & 0x7fff) > 0x7f80
+        assert not ((got != want) & ~(isnan(got) & isnan(want))).any()
+        assert not ((got2 != want) & ~(isnan(got2) & isnan(want))).any()
+    else:
+        assert mismatch_count(got, want) == 0, describe_mismatch(got, want, x)
+        assert same_bits(got2, want)
+
+
 def test_softmax_f16_order_dependence_is_reproduced(dev, oracle):
     # 2048 + 1 + 1 + ... never grows in f16: the kernel must reproduce that, not the mathematically exact sum
     row = np.zeros(512, np.float16)
