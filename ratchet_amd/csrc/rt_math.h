@@ -194,11 +194,15 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
-// Reduction over the LANES threads that share a row: one wave64 (LANES == 64) or a whole 256-thread block, whose four
-// wave results meet in LDS and are added in a fixed order.  Every thread of the block must call the block form.
+// Reduction over the LANES threads that share a row: a group of 2..64 neighbouring lanes of a wave (a butterfly over the
+// group; LANES == 64 is the whole wave), or a whole 256-thread block, whose four wave results meet in LDS and are added
+// in a fixed order.  Every thread of the block must call the block form.
 template <int LANES> __device__ __forceinline__ float row_sum(float v) {
-    v = wave_sum(v);
-    if constexpr (LANES != 64) {
+    if constexpr (LANES <= 64) {
+#pragma unroll
+        for (int off = LANES / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    } else {
+        v = wave_sum(v);
         __shared__ float red[LANES / 64];
         __syncthreads();                                   // earlier readers of red are done
         if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
@@ -210,8 +214,11 @@ template <int LANES> __device__ __forceinline__ float row_sum(float v) {
     return v;
 }
 template <int LANES> __device__ __forceinline__ float row_max(float v) {
-    v = wave_max(v);
-    if constexpr (LANES != 64) {
+    if constexpr (LANES <= 64) {
+#pragma unroll
+        for (int off = LANES / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    } else {
+        v = wave_max(v);
         __shared__ float red[LANES / 64];
         __syncthreads();
         if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;

@@ -577,6 +577,23 @@ int launch_norm(rt_device* dev, const void* x, const void* scale, const void* bi
     const uint32_t nvec = cols / VE;
     const bool vec_ok = (cols % VE == 0) && rt_aligned(x, 16) && rt_aligned(y, 16) && rt_aligned(scale, 16) &&
                         (!bias || rt_aligned(bias, 16)) && nvec <= (uint32_t)(BLOCK * 8);
+    if (vec_ok && nvec <= 32) {
+        // rows of at most 32 vectors: a group of 2..32 lanes per row (one vector each), so that a wave carries 2..32 rows
+        // and as many bytes as with long rows
+        const uint32_t lanes = nvec <= 2 ? 2 : nvec <= 4 ? 4 : nvec <= 8 ? 8 : nvec <= 16 ? 16 : 32;
+        const uint64_t blocks = (rows + BLOCK / lanes - 1) / (BLOCK / lanes);
+        RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
+        const dim3 grid((unsigned)blocks), block(BLOCK);
+#define RT_NARROW(L) hipLaunchKernelGGL((norm_wave_kernel<T, 1, KIND, L>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, (T*)y, rows, cols, eps)
+        if (lanes == 2) RT_NARROW(2);
+        else if (lanes == 4) RT_NARROW(4);
+        else if (lanes == 8) RT_NARROW(8);
+        else if (lanes == 16) RT_NARROW(16);
+        else RT_NARROW(32);
+#undef RT_NARROW
+        RT_CHECK_LAUNCH("norm_wave_kernel");
+        return RT_OK;
+    }
     if (vec_ok && nvec <= (uint32_t)(WAVE * 8)) {
         const uint32_t nv = (nvec + WAVE - 1) / WAVE;
         const uint64_t blocks = (rows + WAVES - 1) / WAVES;
@@ -618,6 +635,69 @@ int launch_norm(rt_device* dev, const void* x, const void* scale, const void* bi
     return RT_OK;
 }
 
+// 16-bit reference arithmetic, many rows of at most 128 columns (whole aligned vectors): one lane per row.  A block's
+// 256 rows are one contiguous run that passes through LDS with coalesced 16-byte accesses (row pitch 16 bytes more than
+// the row, so neighbouring lanes' LDS accesses fall into different banks); the sequential f32 sums are short chains
+// inside the lane.  (The tile walker above carries 8 rows per block however short they are: a million rows of 8 columns
+// took it 479 us.)
+template <typename T, int KIND, int NV>
+__global__ void __launch_bounds__(BLOCK) norm16_lane_kernel(const T* x, const T* __restrict__ scale, const T* __restrict__ bias, T* y,
+                                                            uint64_t rows, float eps) {
+    __shared__ v4u stage[BLOCK * (NV + 1)];
+    const uint64_t row0 = (uint64_t)blockIdx.x * BLOCK;
+    const uint32_t nrows = rows - row0 < (uint64_t)BLOCK ? (uint32_t)(rows - row0) : (uint32_t)BLOCK;
+    const v4u* xb = reinterpret_cast<const v4u*>(x) + row0 * NV;
+    v4u* yb = reinterpret_cast<v4u*>(y) + row0 * NV;
+    const uint32_t nvec = nrows * NV;
+    for (uint32_t i = threadIdx.x; i < nvec; i += BLOCK) stage[(i / NV) * (NV + 1) + i % NV] = ld_stream(xb + i);
+    __syncthreads();
+    if (threadIdx.x < nrows) {
+        v4u* mine = stage + threadIdx.x * (NV + 1);
+        Vec16<T> v[NV];
+#pragma unroll
+        for (int k = 0; k < NV; k++) v[k].u = mine[k];
+        float sx = 0.0f, sq = 0.0f;                          // the reference's order: element 0 first
+#pragma unroll
+        for (int k = 0; k < NV; k++)
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                sq += Ar<T>::widen(Ar<T>::mul(v[k].e[q], v[k].e[q]));
+                if (KIND == NORM_LAYER) sx += Ar<T>::widen(v[k].e[q]);
+            }
+        const RowStats<T> st = finish_stats<T, KIND>(sx, sq, NV * 8, eps);
+#pragma unroll
+        for (int k = 0; k < NV; k++) {
+            Vec16<T> sc, bi;
+            sc.u = reinterpret_cast<const v4u*>(scale)[k];
+            if (KIND == NORM_LAYER && bias) bi.u = reinterpret_cast<const v4u*>(bias)[k];
+#pragma unroll
+            for (int q = 0; q < 8; q++) v[k].e[q] = norm_one<T, KIND>(v[k].e[q], st, sc.e[q], bi.e[q], bias != nullptr);
+            mine[k] = v[k].u;
+        }
+    }
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i < nvec; i += BLOCK) st_stream(yb + i, stage[(i / NV) * (NV + 1) + i % NV]);
+}
+
+template <typename T, int KIND>
+int launch_norm16_lane(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint64_t rows, uint32_t cols, float eps) {
+    const uint64_t blocks = (rows + BLOCK - 1) / BLOCK;
+    RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
+#define RT_LANE(NV)                                                                                                              \
+    case NV:                                                                                                                     \
+        hipLaunchKernelGGL((norm16_lane_kernel<T, KIND, NV>), dim3((unsigned)blocks), dim3(BLOCK), 0, dev->stream, (const T*)x, \
+                           (const T*)scale, (const T*)bias, (T*)y, rows, eps);                                                   \
+        break
+    switch (cols / 8) {
+        RT_LANE(1); RT_LANE(2); RT_LANE(3); RT_LANE(4); RT_LANE(5); RT_LANE(6); RT_LANE(7); RT_LANE(8);
+        RT_LANE(9); RT_LANE(10); RT_LANE(11); RT_LANE(12); RT_LANE(13); RT_LANE(14); RT_LANE(15); RT_LANE(16);
+        default: return rt_fail(RT_ERR_ARG, "norm: internal: %u columns in the one-lane-per-row kernel", cols);
+    }
+#undef RT_LANE
+    RT_CHECK_LAUNCH("norm16_lane_kernel");
+    return RT_OK;
+}
+
 template <typename T, int KIND, int RB>
 int launch_norm16_rb(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint64_t rows, uint32_t cols, float eps) {
     const uint64_t blocks = (rows + RB - 1) / RB;
@@ -638,6 +718,7 @@ int launch_norm16_rb(rt_device* dev, const void* x, const void* scale, const voi
 template <typename T, int KIND>
 int launch_norm16(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint64_t rows, uint32_t cols, float eps) {
     const bool vec_ok = (cols % 8 == 0) && rt_aligned(x, 16) && rt_aligned(y, 16) && rt_aligned(scale, 16) && (!bias || rt_aligned(bias, 16));
+    if (vec_ok && cols <= 128 && rows >= 16384) return launch_norm16_lane<T, KIND>(dev, x, scale, bias, y, rows, cols, eps);
     if (vec_ok) {
         const uint64_t blocks = (rows + 7) / 8;
         RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
@@ -799,6 +880,23 @@ int launch_norm_via32(rt_device* dev, const void* x, const float* scale, const f
     const uint32_t nvec = cols / 8;
     const bool vec_ok = (cols % 8 == 0) && rt_aligned(x, 16) && rt_aligned(y, 16) && rt_aligned(scale, 16) && (!bias || rt_aligned(bias, 16)) &&
                         nvec <= (uint32_t)(BLOCK * 8);
+    if (vec_ok && nvec <= 32) {
+        // rows of at most 32 vectors: a group of 2..32 lanes per row (one vector each), so that a wave carries 2..32 rows
+        // and as many bytes as with long rows
+        const uint32_t lanes = nvec <= 2 ? 2 : nvec <= 4 ? 4 : nvec <= 8 ? 8 : nvec <= 16 ? 16 : 32;
+        const uint64_t blocks = (rows + BLOCK / lanes - 1) / (BLOCK / lanes);
+        RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_norm_via_f32: too many rows");
+        const dim3 grid((unsigned)blocks), block(BLOCK);
+#define RT_NARROW(L) hipLaunchKernelGGL((norm_via32_wave_kernel<T, 1, KIND, L>), grid, block, 0, dev->stream, (const T*)x, scale, bias, (T*)y, rows, cols, eps)
+        if (lanes == 2) RT_NARROW(2);
+        else if (lanes == 4) RT_NARROW(4);
+        else if (lanes == 8) RT_NARROW(8);
+        else if (lanes == 16) RT_NARROW(16);
+        else RT_NARROW(32);
+#undef RT_NARROW
+        RT_CHECK_LAUNCH("norm_via32_wave_kernel");
+        return RT_OK;
+    }
     if (vec_ok && nvec <= (uint32_t)(WAVE * 8)) {
         const uint32_t nv = (nvec + WAVE - 1) / WAVE;
         const uint64_t blocks = (rows + WAVES - 1) / WAVES;

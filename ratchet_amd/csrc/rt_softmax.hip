@@ -628,7 +628,6 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
         // values of this step (loaded two steps ago from y, where this thread put them a group ago) divided and stored,
         // and the load of those of two steps ahead.  The prologue issues the same sequence with targets that do not exist.
         v4u pre[2][2], qpre[2][2], mpre[2];
-        uint32_t qnext[2] = {OOB, OOB};                      // rows whose parked values the next two loads fetch: prev, then cur
 #pragma unroll
         for (int k = 0; k < 2; k++) {
 #pragma unroll
@@ -855,6 +854,24 @@ __global__ void __launch_bounds__(BLOCK) softmax_via32_generic_kernel(const T* _
 template <typename T, int MODE> int launch_wave(rt_device* dev, const void* x, void* y, uint64_t rows, uint32_t cols) {
     constexpr int VE = 16 / sizeof(T);
     const uint32_t nvec = cols / VE;
+    const bool vec_ok = true;
+    if (vec_ok && nvec <= 32) {
+        // rows of at most 32 vectors: a group of 2..32 lanes per row (one vector each), so that a wave carries 2..32 rows
+        // and as many bytes as with long rows
+        const uint32_t lanes = nvec <= 2 ? 2 : nvec <= 4 ? 4 : nvec <= 8 ? 8 : nvec <= 16 ? 16 : 32;
+        const uint64_t blocks = (rows + BLOCK / lanes - 1) / (BLOCK / lanes);
+        RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax: too many rows");
+        const dim3 grid((unsigned)blocks), block(BLOCK);
+#define RT_NARROW(L) hipLaunchKernelGGL((softmax_wave_kernel<T, 1, MODE, L>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols)
+        if (lanes == 2) RT_NARROW(2);
+        else if (lanes == 4) RT_NARROW(4);
+        else if (lanes == 8) RT_NARROW(8);
+        else if (lanes == 16) RT_NARROW(16);
+        else RT_NARROW(32);
+#undef RT_NARROW
+        RT_CHECK_LAUNCH("softmax_wave_kernel");
+        return RT_OK;
+    }
     if (nvec <= (uint32_t)(WAVE * 8)) {
         const uint32_t nv = (nvec + WAVE - 1) / WAVE;
         const uint64_t blocks = (rows + WAVES - 1) / WAVES;
@@ -1005,6 +1022,23 @@ template <typename T, int MODE, bool MASK>
 int launch_via32(rt_device* dev, const void* x, const void* mask, void* y, uint64_t rows, uint32_t cols, const MaskArgs& p, bool mask_vec_ok) {
     const uint32_t nvec = cols / 8;
     const bool vec_ok = (cols % 8 == 0) && rt_aligned(x, 16) && rt_aligned(y, 16) && nvec <= (uint32_t)(BLOCK * 8) && (!MASK || mask_vec_ok);
+    if (vec_ok && nvec <= 32) {
+        // rows of at most 32 vectors: a group of 2..32 lanes per row (one vector each), so that a wave carries 2..32 rows
+        // and as many bytes as with long rows
+        const uint32_t lanes = nvec <= 2 ? 2 : nvec <= 4 ? 4 : nvec <= 8 ? 8 : nvec <= 16 ? 16 : 32;
+        const uint64_t blocks = (rows + BLOCK / lanes - 1) / (BLOCK / lanes);
+        RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax_via_f32: too many rows");
+        const dim3 grid((unsigned)blocks), block(BLOCK);
+#define RT_NARROW(L) hipLaunchKernelGGL((softmax_via32_wave_kernel<T, 1, MODE, MASK, L>), grid, block, 0, dev->stream, (const T*)x, (const T*)mask, (T*)y, rows, cols, p)
+        if (lanes == 2) RT_NARROW(2);
+        else if (lanes == 4) RT_NARROW(4);
+        else if (lanes == 8) RT_NARROW(8);
+        else if (lanes == 16) RT_NARROW(16);
+        else RT_NARROW(32);
+#undef RT_NARROW
+        RT_CHECK_LAUNCH("softmax_via32_wave_kernel");
+        return RT_OK;
+    }
     if (vec_ok && nvec <= (uint32_t)(WAVE * 8)) {
         const uint32_t nv = (nvec + WAVE - 1) / WAVE;
         const uint64_t blocks = (rows + WAVES - 1) / WAVES;

@@ -287,6 +287,22 @@ def test_norms_f16(dev, oracle, shape):
     assert mismatch_count(got, want) == 0, mismatch_count(got, want)
 
 
+@pytest.mark.parametrize("rows,cols,kind", [(20000, 8, "f16"), (16384 + 3, 64, "f16"), (17000, 128, "f16"), (30000, 24, "bf16"), (16500, 120, "bf16")])
+def test_norms_16_bit_many_narrow_rows(dev, oracle, rows, cols, kind):
+    """tens of thousands of rows of at most 128 columns take a kernel with one lane per row; same bits as the walkers"""
+    rng = np.random.default_rng(314)
+    bf = kind == "bf16"
+    conv = (lambda a: _bf16(oracle, a)) if bf else (lambda a: np.asarray(a, np.float32).astype(np.float16))
+    x = conv(rng.standard_normal((rows, cols)) * 1.5 + 0.25)
+    w = conv(1 + 0.02 * rng.standard_normal(cols))
+    b = conv(0.02 * rng.standard_normal(cols))
+    dx, dw, db = dev.upload(x, bf16=bf), dev.upload(w, bf16=bf), dev.upload(b, bf16=bf)
+    for name, want, got in (("layer", oracle.layer_norm(x, w, b, 1e-5, bf16=bf, intended=True), dev.layer_norm(dx, dw, db, 1e-5).to_numpy()),
+                            ("layer, no bias", oracle.layer_norm(x, w, None, 1e-5, bf16=bf, intended=True), dev.layer_norm(dx, dw, None, 1e-5).to_numpy()),
+                            ("rms", oracle.rms_norm(x, w, 1e-5, bf16=bf, intended=True), dev.rms_norm(dx, dw, 1e-5).to_numpy())):
+        assert np.array_equal(np.asarray(got).view(np.uint16), np.asarray(want).view(np.uint16)), (name, rows, cols, kind)
+
+
 def test_layer_norm_variance_form_matches_reference(dev, oracle):
     # E[x^2] - mu^2 loses digits with a large common offset; the kernel must lose them the same way (not use two passes)
     rng = np.random.default_rng(313)
