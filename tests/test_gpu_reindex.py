@@ -159,6 +159,14 @@ def test_concat(dev, oracle, dtype):
         ys = [randn(rng, s, dtype) for s in shapes]
         got = dev.concat([dev.upload(y) for y in ys], dim).to_numpy()
         assert np.array_equal(got, oracle.concat(ys, dim)), (dim, shapes)
+    # short segments take the kernel that walks the destination: the rotary / pass-through halves of a head
+    # (phi2/attn.rs:119-127 via rope), eight narrow inputs, segments of 1..3 vectors, odd widths, many rows
+    for dim, shapes in [(3, [(1, 32, 300, 32), (1, 32, 300, 48)]), (3, [(2, 4, 100, 16), (2, 4, 100, 64)]), (1, [(5000, 8), (5000, 8)]),
+                        (1, [(3000, 3), (3000, 5)]), (1, [(1000, 33), (1000, 31)]), (2, [(7, 9, k, 4) for k in (1, 2, 3, 4, 5, 6, 7, 8)]),
+                        (3, [(2, 3, 70, 24), (2, 3, 70, 8), (2, 3, 70, 40)]), (2, [(3, 500, 1, 8), (3, 500, 2, 8)])]:
+        ys = [randn(rng, s, dtype) for s in shapes]
+        got = dev.concat([dev.upload(y) for y in ys], dim).to_numpy()
+        assert np.array_equal(got, oracle.concat(ys, dim)), (dim, shapes)
 
 
 def test_concat_rejects_bad_arguments(dev):
