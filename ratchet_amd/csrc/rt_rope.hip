@@ -60,6 +60,133 @@ __global__ void __launch_bounds__(BLOCK) rope_kernel(const T* x, T* y, RopeArgs 
     }
 }
 
+// The same work in 16-byte vectors, for head layouts whose rotated half, rotated width and head dim are whole aligned
+// vectors (every model: 32/80, 96/96, 128/128 columns).  A rotary block owns BLOCK / VE items, an item being (position,
+// vector of VE frequencies): first every thread computes one (position, frequency) sin / cos pair into LDS (the double
+// precision sin and cos are the long pole: one pair per thread, not VE), then thread (item, sub) rotates the item's two
+// vectors in rows sub, sub + VE, ... of the block's share of batch * heads.  Blocks past the rotary ones copy the
+// pass-through vectors the same way.
+struct RopeVecArgs {
+    FastDiv hv_div, pv_div;  // rotated vectors per half row; pass-through vectors per row
+    uint32_t S, half, offset;
+    uint32_t hv, pv, row_v;  // vectors: per half, pass-through, per row
+    uint32_t nbh, bh_chunk;
+    uint32_t rot_items, pass_items, rot_blocks;
+    float ln_base;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(BLOCK) rope_vec_kernel(const T* x, T* y, RopeVecArgs a) {
+    constexpr int VE = 16 / sizeof(T), ITEMS = BLOCK / VE;
+    __shared__ float s_sn[BLOCK], s_cs[BLOCK];
+    const uint32_t bh0 = blockIdx.y * a.bh_chunk;
+    const uint32_t bh1 = (bh0 + a.bh_chunk < a.nbh) ? bh0 + a.bh_chunk : a.nbh;
+    const v4u* xv = reinterpret_cast<const v4u*>(x);
+    v4u* yv = reinterpret_cast<v4u*>(y);
+    const uint32_t it = threadIdx.x % ITEMS, sub = threadIdx.x / ITEMS;
+    const uint64_t row_stride = (uint64_t)a.S * a.row_v;
+    if (blockIdx.x < a.rot_blocks) {
+        {
+            const uint32_t item = blockIdx.x * ITEMS + threadIdx.x / VE, e = threadIdx.x % VE;
+            if (item < a.rot_items) {
+                uint32_t p, slot;
+                fd_divmod(item, a.hv_div, p, slot);
+                const float neg_i = -(float)(slot * VE + e);
+                const float inv = rt_expf(neg_i * a.ln_base / (float)a.half);
+                const float theta = (float)(a.offset + p) * inv;
+                s_sn[threadIdx.x] = rt_sinf(theta);
+                s_cs[threadIdx.x] = rt_cosf(theta);
+            }
+        }
+        __syncthreads();
+        const uint32_t item = blockIdx.x * ITEMS + it;
+        if (item >= a.rot_items) return;
+        uint32_t p, slot;
+        fd_divmod(item, a.hv_div, p, slot);
+        float sn[VE], cs[VE];
+#pragma unroll
+        for (int e = 0; e < VE; e++) {
+            sn[e] = s_sn[it * VE + e];
+            cs[e] = s_cs[it * VE + e];
+        }
+        auto rotate = [&](Vec16<T>& lo, Vec16<T>& hi) {
+#pragma unroll
+            for (int e = 0; e < VE; e++) {
+                const float x1 = Ar<T>::widen(lo.e[e]), x2 = Ar<T>::widen(hi.e[e]);
+                const float r1 = x1 * cs[e] - x2 * sn[e];
+                const float r2 = x1 * sn[e] + x2 * cs[e];
+                lo.e[e] = Ar<T>::conv(r1);
+                hi.e[e] = Ar<T>::conv(r2);
+            }
+        };
+        const uint64_t at_p = (uint64_t)p * a.row_v + slot;
+        for (uint32_t bh = bh0 + sub; bh < bh1; bh += 2 * VE) {     // two rows per trip, all four loads before the first store
+            const uint64_t at0 = (uint64_t)bh * row_stride + at_p;
+            const bool two = bh + VE < bh1;
+            const uint64_t at1 = two ? at0 + (uint64_t)VE * row_stride : at0;
+            Vec16<T> lo0, hi0, lo1, hi1;
+            lo0.u = ld_stream(xv + at0);
+            hi0.u = ld_stream(xv + at0 + a.hv);
+            lo1.u = ld_stream(xv + at1);
+            hi1.u = ld_stream(xv + at1 + a.hv);
+            rotate(lo0, hi0);
+            st_stream(yv + at0, lo0.u);
+            st_stream(yv + at0 + a.hv, hi0.u);
+            if (two) {
+                rotate(lo1, hi1);
+                st_stream(yv + at1, lo1.u);
+                st_stream(yv + at1 + a.hv, hi1.u);
+            }
+        }
+    } else {
+        const uint32_t item = (blockIdx.x - a.rot_blocks) * ITEMS + it;
+        if (item >= a.pass_items) return;
+        uint32_t p, slot;
+        fd_divmod(item, a.pv_div, p, slot);
+        const uint64_t at_p = (uint64_t)p * a.row_v + 2 * a.hv + slot;
+        for (uint32_t bh = bh0 + sub; bh < bh1; bh += 2 * VE) {
+            const uint64_t at0 = (uint64_t)bh * row_stride + at_p;
+            const bool two = bh + VE < bh1;
+            const uint64_t at1 = two ? at0 + (uint64_t)VE * row_stride : at0;
+            const v4u v0 = ld_stream(xv + at0), v1 = ld_stream(xv + at1);
+            st_stream(yv + at0, v0);
+            if (two) st_stream(yv + at1, v1);
+        }
+    }
+}
+
+template <typename T> int launch_rope_vec(rt_device* dev, const void* x, void* y, const uint32_t shape[4], uint32_t dim, uint32_t offset, float ln_base) {
+    constexpr uint32_t VE = 16 / sizeof(T), ITEMS = BLOCK / VE;
+    RopeVecArgs a;
+    a.S = shape[2];
+    a.half = dim / 2;
+    a.offset = offset;
+    a.hv = a.half / VE;
+    a.pv = (shape[3] - dim) / VE;
+    a.row_v = shape[3] / VE;
+    a.nbh = shape[0] * shape[1];
+    a.ln_base = ln_base;
+    a.hv_div = make_fastdiv(a.hv);
+    a.pv_div = make_fastdiv(a.pv ? a.pv : 1);
+    const uint64_t rot_items = (uint64_t)a.S * a.hv, pass_items = (x == y) ? 0 : (uint64_t)a.S * a.pv;   // in place: nothing to copy
+    RT_REQUIRE(rot_items + pass_items <= 0x7fffffffull, RT_ERR_SIZE, "rt_rope: seq_len * head_dim too large");
+    a.rot_items = (uint32_t)rot_items;
+    a.pass_items = (uint32_t)pass_items;
+    a.rot_blocks = (uint32_t)((rot_items + ITEMS - 1) / ITEMS);
+    const uint64_t blocks_x = a.rot_blocks + (pass_items + ITEMS - 1) / ITEMS;
+    // batch * heads is split over blockIdx.y until about four blocks per CU exist, but not below one row per sub-thread
+    uint64_t chunks = ((uint64_t)dev->num_cus * 4 + blocks_x - 1) / blocks_x;
+    const uint64_t max_chunks = (a.nbh + VE - 1) / VE;
+    if (chunks > max_chunks) chunks = max_chunks;
+    if (chunks > 65535) chunks = 65535;
+    if (chunks < 1) chunks = 1;
+    a.bh_chunk = (uint32_t)((a.nbh + chunks - 1) / chunks);
+    chunks = (a.nbh + a.bh_chunk - 1) / a.bh_chunk;
+    hipLaunchKernelGGL((rope_vec_kernel<T>), dim3((unsigned)blocks_x, (unsigned)chunks), dim3(BLOCK), 0, dev->stream, (const T*)x, (T*)y, a);
+    RT_CHECK_LAUNCH("rope_vec_kernel");
+    return RT_OK;
+}
+
 template <typename T> int launch_rope(rt_device* dev, const void* x, void* y, const RopeArgs& a, unsigned chunks) {
     const dim3 grid((a.n_items + BLOCK - 1) / BLOCK, chunks);
     hipLaunchKernelGGL((rope_kernel<T>), grid, dim3(BLOCK), 0, dev->stream, (const T*)x, (T*)y, a);
@@ -95,6 +222,14 @@ extern "C" int rt_rope(rt_device* dev, int dt, const void* x, void* y, const uin
     a.half = dim / 2;
     a.offset = offset;
     a.nbh = shape[0] * shape[1];
+    const uint32_t ve = 16u / (uint32_t)eb;
+    if ((dim / 2) % ve == 0 && shape[3] % ve == 0 && rt_aligned(x, 16) && rt_aligned(y, 16)) {
+        switch (dt) {
+            case RT_F32: return launch_rope_vec<float>(dev, x, y, shape, dim, offset, logf(base));
+            case RT_F16: return launch_rope_vec<half_t>(dev, x, y, shape, dim, offset, logf(base));
+            default: return launch_rope_vec<bf16_t>(dev, x, y, shape, dim, offset, logf(base));
+        }
+    }
     const uint32_t per_row = a.half + (a.D - dim);
     a.per_row = make_fastdiv(per_row);
     const uint64_t items = (uint64_t)a.S * per_row;

@@ -42,6 +42,42 @@ def test_rope_16bit_is_widen_rotate_round(dev, oracle):
     assert (got.view(np.uint16) != want.view(np.uint16)).mean() < 0.001
 
 
+@pytest.mark.parametrize("shape,dim,offset", [((2, 5, 33, 80), 32, 3), ((1, 3, 9, 80), 40, 0), ((3, 7, 4, 128), 128, 100), ((1, 1, 70, 64), 48, 9),
+                                              ((1, 19, 1, 96), 96, 2047), ((1, 2, 6, 24), 24, 1)])
+def test_rope_16bit_layouts(dev, oracle, shape, dim, offset):
+    """f16 / bf16 in the vector layout (half the rotated width a multiple of 8) and outside it (dim 40, 24), odd
+    batch * heads counts, with and without pass-through columns, out of place and in place"""
+    rng = np.random.default_rng(605)
+    xf = rng.standard_normal(shape).astype(np.float32)
+    for bf in (False, True):
+        x = oracle.cast(xf, np.uint16, dst_bf16=True) if bf else xf.astype(np.float16)
+        x32 = oracle.cast(x, np.float32, src_bf16=bf)
+        want = oracle.cast(oracle.rope(x32, dim, 10000.0, offset), np.uint16 if bf else np.float16, dst_bf16=bf)
+        d = dev.upload(x, bf16=bf)
+        got = dev.rope(d, dim, 10000.0, offset).to_numpy()
+        diff = got.view(np.uint16) != np.asarray(want).view(np.uint16)
+        assert diff.mean() < 0.002, (shape, dim, bf, diff.mean())                              # one sin / cos ulp may move a rounding
+        bad, mx = oracle.count_not_close(got, want, 1e-2 if bf else 1e-3, 1e-2 if bf else 1e-3, bf16=bf)
+        assert bad == 0, (shape, dim, bf, bad, mx)
+        assert np.array_equal(got[..., dim:].view(np.uint16), x[..., dim:].view(np.uint16))
+        inplace = dev.rope(d, dim, 10000.0, offset, out=d).to_numpy()
+        assert np.array_equal(inplace.view(np.uint16), got.view(np.uint16))
+
+
+def test_rope_f32_off_vector_alignment(dev, oracle):
+    """an operand 4 bytes off 16-byte alignment takes the scalar kernel: same results as the aligned call"""
+    rng = np.random.default_rng(606)
+    shape = (1, 4, 37, 80)
+    x = rng.standard_normal(shape).astype(np.float32)
+    aligned = dev.rope(dev.upload(x), 32, 10000.0, 11).to_numpy()
+    big = dev.empty((x.size + 4,), 0)
+    view = big.view(1, shape)
+    view.upload(x)
+    out = dev.empty((x.size + 4,), 0).view(1, shape)
+    dev.rope(view, 32, 10000.0, 11, out=out)
+    assert same_bits(out.to_numpy(), aligned)
+
+
 def test_rope_rejects_bad_arguments(dev):
     from ratchet_amd import RatchetError
 
