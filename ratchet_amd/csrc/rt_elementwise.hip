@@ -487,6 +487,40 @@ template <typename T, bool VIA32 = false> int unary_via_lut(rt_device* dev, int 
     return RT_OK;
 }
 
+// Below the size where a per-block copy of the table into LDS pays (one 128 KiB load per block), the same table is read
+// where it lies: the 128 KiB stay in L2 (and largely in the CUs' L1) and every element is one 2-byte load.  For the heavy
+// ops this is still far cheaper than computing: gelu on [64, 10240] f16 took 11.8 us computed, of which most is the
+// dependent chain of one thread's eight exact tanh evaluations.
+__global__ void __launch_bounds__(BLOCK) unary_table_gather_kernel(const uint16_t* __restrict__ table, const uint16_t* x, uint16_t* y,
+                                                                   uint64_t numel) {
+    const uint64_t nvec = numel / 8;
+    const uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+    if (i < nvec) {
+        const v4u in = ld_stream(reinterpret_cast<const v4u*>(x) + i);
+        v4u out;
+#pragma unroll
+        for (int w = 0; w < 4; w++) out[w] = (uint32_t)table[in[w] & 0xffffu] | ((uint32_t)table[in[w] >> 16] << 16);
+        st_stream(reinterpret_cast<v4u*>(y) + i, out);
+    }
+    if (blockIdx.x == 0) {
+        const uint64_t j = nvec * 8 + threadIdx.x;
+        if (j < numel) y[j] = table[x[j]];
+    }
+}
+
+constexpr uint64_t RT_GATHER_MIN_NUMEL = 2048;
+
+template <typename T, bool VIA32 = false> int unary_via_table_gather(rt_device* dev, int op, const void* x, void* y, uint64_t numel) {
+    const int ti = std::is_same<T, bf16_t>::value ? 1 : 0;
+    int rc = build_unary_table<T, VIA32>(dev, ti, op);
+    if (rc) return rc;
+    hipLaunchKernelGGL(unary_table_gather_kernel, dim3(blocks_for(numel / 8 ? numel / 8 : 1, BLOCK)), dim3(BLOCK), 0, dev->stream,
+                       (const uint16_t*)(VIA32 ? dev->unary_lut_via32[ti][op] : dev->unary_lut[ti][op]), (const uint16_t*)x, (uint16_t*)y,
+                       numel);
+    RT_CHECK_LAUNCH("unary_table_gather_kernel");
+    return RT_OK;
+}
+
 template <typename T>
 int launch_gated(rt_device* dev, int op, const void* gate, uint64_t gs, const void* up, uint64_t us, void* y, uint64_t rows, uint32_t cols) {
     const int ti = std::is_same<T, bf16_t>::value ? 1 : 0;
@@ -710,10 +744,17 @@ int rt_unary(rt_device* dev, int op, int dt, const void* x, void* y, uint64_t nu
     if (rc) return rc;
     // large 16-bit tensors: table lookup (bit-identical to computing, see unary_lut_kernel)
     const bool lut = dt != RT_F32 && numel >= RT_LUT_MIN_NUMEL && lut_worthwhile(op) && rt_aligned(x, 16) && rt_aligned(y, 16);
+    // in between: the table read in place (while a graph is being captured only if the table exists already)
+    const bool gather = dt != RT_F32 && !lut && numel >= RT_GATHER_MIN_NUMEL && lut_worthwhile(op) && rt_aligned(x, 16) && rt_aligned(y, 16) &&
+                        (!dev->capturing || dev->unary_lut[dt == RT_BF16 ? 1 : 0][op]);
     switch (dt) {
         case RT_F32: return dispatch_unary<float>(dev, op, x, y, numel);
-        case RT_F16: return lut ? unary_via_lut<half_t>(dev, op, x, y, numel) : dispatch_unary<half_t>(dev, op, x, y, numel);
-        default: return lut ? unary_via_lut<bf16_t>(dev, op, x, y, numel) : dispatch_unary<bf16_t>(dev, op, x, y, numel);
+        case RT_F16:
+            return lut ? unary_via_lut<half_t>(dev, op, x, y, numel)
+                       : gather ? unary_via_table_gather<half_t>(dev, op, x, y, numel) : dispatch_unary<half_t>(dev, op, x, y, numel);
+        default:
+            return lut ? unary_via_lut<bf16_t>(dev, op, x, y, numel)
+                       : gather ? unary_via_table_gather<bf16_t>(dev, op, x, y, numel) : dispatch_unary<bf16_t>(dev, op, x, y, numel);
     }
 }
 
@@ -727,8 +768,13 @@ int rt_unary_via_f32(rt_device* dev, int op, int io_dt, const void* x, void* y, 
     int rc = rt_enter(dev);
     if (rc) return rc;
     const bool lut = numel >= RT_LUT_MIN_NUMEL && lut_worthwhile(op) && rt_aligned(x, 16) && rt_aligned(y, 16);
-    if (io_dt == RT_F16) return lut ? unary_via_lut<half_t, true>(dev, op, x, y, numel) : dispatch_unary<half_t, true>(dev, op, x, y, numel);
-    return lut ? unary_via_lut<bf16_t, true>(dev, op, x, y, numel) : dispatch_unary<bf16_t, true>(dev, op, x, y, numel);
+    const bool gather = !lut && numel >= RT_GATHER_MIN_NUMEL && lut_worthwhile(op) && rt_aligned(x, 16) && rt_aligned(y, 16) &&
+                        (!dev->capturing || dev->unary_lut_via32[io_dt == RT_BF16 ? 1 : 0][op]);
+    if (io_dt == RT_F16)
+        return lut ? unary_via_lut<half_t, true>(dev, op, x, y, numel)
+                   : gather ? unary_via_table_gather<half_t, true>(dev, op, x, y, numel) : dispatch_unary<half_t, true>(dev, op, x, y, numel);
+    return lut ? unary_via_lut<bf16_t, true>(dev, op, x, y, numel)
+               : gather ? unary_via_table_gather<bf16_t, true>(dev, op, x, y, numel) : dispatch_unary<bf16_t, true>(dev, op, x, y, numel);
 }
 
 int rt_gated_mul_via_f32(rt_device* dev, int op, int io_dt, const void* gate, uint64_t gate_row_stride, const void* up,
