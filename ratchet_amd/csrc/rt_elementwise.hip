@@ -283,6 +283,24 @@ __global__ void __launch_bounds__(LUT_BLOCK) gated_lut_kernel(const uint16_t* __
     }
 }
 
+// mid-size tensors: the table read where it lies (see unary_table_gather_kernel), one vector per thread
+template <typename T>
+__global__ void __launch_bounds__(BLOCK) gated_gather_kernel(const uint16_t* __restrict__ table, const T* __restrict__ gate,
+                                                             const T* __restrict__ up, T* __restrict__ y, GatedArgs p) {
+    const uint64_t v = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+    if (v >= p.nvec) return;
+    uint32_t row, c;
+    fd_divmod((uint32_t)v, p.cv, row, c);
+    Vec16<T> g, u, o;
+    g.u = ld_stream(reinterpret_cast<const v4u*>(gate + (uint64_t)row * p.gs) + c);
+    u.u = ld_stream(reinterpret_cast<const v4u*>(up + (uint64_t)row * p.us) + c);
+#pragma unroll
+    for (int w = 0; w < 4; w++) g.u[w] = (uint32_t)table[g.u[w] & 0xffffu] | ((uint32_t)table[g.u[w] >> 16] << 16);
+#pragma unroll
+    for (int e = 0; e < 8; e++) o.e[e] = Ar<T>::mul(u.e[e], g.e[e]);
+    st_stream(reinterpret_cast<v4u*>(y) + v, o.u);
+}
+
 // any size / alignment: one element per thread, computed directly
 template <typename T, int OP>
 __global__ void __launch_bounds__(BLOCK) gated_scalar_kernel(const T* __restrict__ gate, const T* __restrict__ up, T* __restrict__ y,
@@ -544,6 +562,16 @@ int launch_gated(rt_device* dev, int op, const void* gate, uint64_t gs, const vo
         hipLaunchKernelGGL((gated_lut_kernel<T>), dim3((unsigned)blocks), dim3(LUT_BLOCK), LUT_BYTES, dev->stream,
                            (const uint16_t*)dev->unary_lut_via32[ti][op], (const T*)gate, (const T*)up, (T*)y, p);
         RT_CHECK_LAUNCH("gated_lut_kernel");
+        return RT_OK;
+    }
+    if (vec && numel >= RT_GATHER_MIN_NUMEL && lut_worthwhile(op) && (!dev->capturing || dev->unary_lut_via32[ti][op])) {
+        int rc = build_unary_table<T, true>(dev, ti, op);
+        if (rc) return rc;
+        p.cv = make_fastdiv(cols / 8);
+        p.nvec = numel / 8;
+        hipLaunchKernelGGL((gated_gather_kernel<T>), dim3(blocks_for(p.nvec, BLOCK)), dim3(BLOCK), 0, dev->stream,
+                           (const uint16_t*)dev->unary_lut_via32[ti][op], (const T*)gate, (const T*)up, (T*)y, p);
+        RT_CHECK_LAUNCH("gated_gather_kernel");
         return RT_OK;
     }
     p.cv = make_fastdiv(cols);

@@ -65,7 +65,7 @@ def _bf16_nan(u):
 
 
 @pytest.mark.parametrize("shape,split", [((2, 1024, 4096), True), ((1, 7, 48), True), ((3, 5, 22), True), ((600, 4096), False),
-                                         ((33, 77), False)])
+                                         ((33, 77), False), ((1, 64, 16384), True), ((100, 512), False), ((1, 30, 144), True)])
 def test_gated_mul_matches_the_op_sequence(dev, oracle, shape, split):
     """phi3's MLP: up_states.slice(second half).mul(up_states.slice(first half).full().silu().cast(dt))."""
     rng = np.random.default_rng(502)
@@ -212,7 +212,7 @@ def test_bf16_patterns(dev, oracle):
     assert ok, info
     assert (got != want).mean() < 0.01
     # gated multiply: bit-exact (table path and direct path)
-    for shape in ((600, 4096), (5, 24)):
+    for shape in ((600, 4096), (5, 24), (40, 512)):
         gate, up = bf(rng.standard_normal(shape) * 2), bf(rng.standard_normal(shape))
         act = bf(oracle.unary("silu", wide(gate)))
         want = oracle.binary("mul", up, act, bf16=True)
