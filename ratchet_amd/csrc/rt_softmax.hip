@@ -284,7 +284,8 @@ template <typename T> int launch_lane16(rt_device* dev, const void* x, void* y, 
 }
 
 // ------------------------------------------------------------------------------------------------------------------
-// f16 reference arithmetic, single pass over HBM (cols <= NSTEP * 512, cols % 8 == 0, 16-byte aligned).
+// 16-bit reference arithmetic (f16, bf16), single pass over HBM (cols % 8 == 0, 16-byte aligned; the description is of
+// the variant for rows of at most 4096 columns, whose differences from the long-row variant are stated at the kernel).
 //
 // One 1024-thread block per CU walks over groups of 30 rows.  Wave 0 does nothing but the sequential sums; loader wave
 // w = 1..15 owns rows w-1 and w+14 of the group: in step t its 64 lanes cover the 1 KiB at columns t*512 .. t*512+511 of
@@ -294,16 +295,17 @@ template <typename T> int launch_lane16(rt_device* dev, const void* x, void* y, 
 //        (162 400 of the CU's 163 840 bytes), so exp is one ds_read_u16 per element with the bit pattern as the index:
 //        no range clamping, no NaN special case.
 //   sum: per 512-column step the exp values also go to an LDS tile; lanes 0..29 of wave 0 each walk one row of the
-//        tile left to right with dependent v_add_f16 (3 ns each on this chip, 1.5 us per step).  The tile is single
+//        tile left to right with dependent v_add_f16 (3 ns each on this chip, 1.5 us per step; bf16: add, round on the
+//        bit pattern, 12 ns).  The tile is single
 //        buffered with two barriers per step: the loaders look up step t+1 into registers and divide / store the
 //        previous group's step t while wave 0 walks step t, and only the short LDS write of the tile sits between the
 //        barriers with wave 0 idle.  A step is 30 KiB in and 30 KiB out of HBM per CU, about 2 us at a CU's share of
 //        8 TB/s, so the walk stays hidden; wave 0 is kept free of any other work and raises its issue priority.
 //   divide: the outputs of group g are produced while group g+1 streams in: y = e / sum with the quotient computed as
 //        q0 = e * (1/sum) plus one fma correction, which is the correctly rounded f16 quotient for normal finite sums
-//        (checked against IEEE division over operand pairs on the GPU); other sums take the IEEE path.
+//        (checked against IEEE division over operand pairs on the GPU); other sums, and bf16, take the IEEE path.
 //   mask: with MASK, a second operand (one [P, cols] block shared by every period of P rows, e.g. an [S, T] attention
-//        mask under B * H heads) is added to x in f16 as the vectors arrive: scores.add(mask).softmax() without the sum
+//        mask under B * H heads) is added to x in the 16-bit type as the vectors arrive: scores.add(mask).softmax() without the sum
 //        ever reaching memory, bit-identical to the two separate ops.
 // Global loads run SP_PF steps ahead across group boundaries, so the pipeline never drains.
 // ------------------------------------------------------------------------------------------------------------------
