@@ -823,14 +823,52 @@ __global__ void __launch_bounds__(GN_LDS_BLOCK) gn_lds_kernel(const T* __restric
     }
 }
 
+// Many slices per group (few, very large groups): the partials of a group are combined once, by one block, into a
+// single (mean, M2, count) triple that the apply kernel then reads as if the group had one slice.
+__global__ void __launch_bounds__(BLOCK) gn_combine_kernel(const float* __restrict__ part, float* __restrict__ out, uint32_t splits) {
+    __shared__ double s_n[BLOCK], s_mean[BLOCK], s_m2[BLOCK];
+    const float* p = part + (uint64_t)blockIdx.x * splits * 3;
+    double n = 0.0, mean = 0.0, m2 = 0.0;
+    auto merge = [&](double nb, double mb, double m2b) {                       // Chan et al.
+        if (nb == 0.0) return;
+        const double nt = n + nb;
+        const double delta = mb - mean;
+        mean += delta * (nb / nt);
+        m2 += m2b + delta * delta * (n * nb / nt);
+        n = nt;
+    };
+    for (uint32_t k = threadIdx.x; k < splits; k += BLOCK) merge((double)p[3 * k + 2], (double)p[3 * k], (double)p[3 * k + 1]);
+    s_n[threadIdx.x] = n;
+    s_mean[threadIdx.x] = mean;
+    s_m2[threadIdx.x] = m2;
+    __syncthreads();
+    for (int off = BLOCK / 2; off > 0; off >>= 1) {
+        if ((int)threadIdx.x < off) {
+            merge(s_n[threadIdx.x + off], s_mean[threadIdx.x + off], s_m2[threadIdx.x + off]);
+            s_n[threadIdx.x] = n;
+            s_mean[threadIdx.x] = mean;
+            s_m2[threadIdx.x] = m2;
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        float* o = out + (uint64_t)blockIdx.x * 3;
+        o[0] = (float)mean;
+        o[1] = (float)m2;
+        o[2] = (float)n;
+    }
+}
+
 template <typename T>
 int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint32_t bg, uint32_t glen, uint32_t cpg,
               uint32_t groups, uint32_t L, float eps) {
-    // enough blocks to cover the chip, slices of at least 2048 elements
+    // enough blocks to cover the chip, slices of at least 2048 elements; beyond 64 slices per group the partials are
+    // combined by a launch of their own instead of by every apply block
+    constexpr uint32_t FUSED_COMBINE_MAX = 64;
     uint32_t splits = (2048 + bg - 1) / bg;
     const uint32_t max_splits = (glen + 2047) / 2048;
     if (splits > max_splits) splits = max_splits;
-    if (splits > 64) splits = 64;
+    if (splits > 2048) splits = 2048;
     if (splits < 1) splits = 1;
     constexpr int VEMAX = 16 / sizeof(T);
     const bool vec = (L % VEMAX == 0) && rt_aligned(x, 16) && rt_aligned(y, 16);       // then glen % VEMAX == 0 too
@@ -849,7 +887,7 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
     uint32_t chunk = (glen + splits - 1) / splits;
     if (vec) chunk = (chunk + VEMAX - 1) / VEMAX * VEMAX;                               // slices start on vector boundaries
     splits = (glen + chunk - 1) / chunk;
-    const size_t need = (size_t)bg * splits * 3 * sizeof(float);
+    const size_t need = ((size_t)bg * splits + bg) * 3 * sizeof(float);           // partials, then one combined triple per group
     if (need > dev->gn_scratch_bytes) {
         RT_NO_CAPTURE(dev, "growing the GroupNorm scratch");
         RT_HIP(hipStreamSynchronize(dev->stream));
@@ -860,16 +898,23 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
         dev->gn_scratch_bytes = need;
     }
     const dim3 grid(bg, splits), block(BLOCK);
+    const bool separate = splits > FUSED_COMBINE_MAX;
+    const float* stats = separate ? dev->gn_scratch + (size_t)bg * splits * 3 : dev->gn_scratch;
+    const uint32_t stat_splits = separate ? 1 : splits;
+    if (vec) hipLaunchKernelGGL((gn_stats_kernel<T, VEMAX>), grid, block, 0, dev->stream, (const T*)x, dev->gn_scratch, glen, chunk, splits);
+    else hipLaunchKernelGGL((gn_stats_kernel<T, 1>), grid, block, 0, dev->stream, (const T*)x, dev->gn_scratch, glen, chunk, splits);
+    RT_CHECK_LAUNCH("gn_stats_kernel");
+    if (separate) {
+        hipLaunchKernelGGL(gn_combine_kernel, dim3(bg), block, 0, dev->stream, (const float*)dev->gn_scratch,
+                           dev->gn_scratch + (size_t)bg * splits * 3, splits);
+        RT_CHECK_LAUNCH("gn_combine_kernel");
+    }
     if (vec) {
-        hipLaunchKernelGGL((gn_stats_kernel<T, VEMAX>), grid, block, 0, dev->stream, (const T*)x, dev->gn_scratch, glen, chunk, splits);
-        RT_CHECK_LAUNCH("gn_stats_kernel");
-        hipLaunchKernelGGL((gn_apply_kernel<T, VEMAX>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, (T*)y,
-                           (const float*)dev->gn_scratch, glen, chunk, splits, cpg, groups, make_fastdiv(L), eps);
+        hipLaunchKernelGGL((gn_apply_kernel<T, VEMAX>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, (T*)y, stats,
+                           glen, chunk, stat_splits, cpg, groups, make_fastdiv(L), eps);
     } else {
-        hipLaunchKernelGGL((gn_stats_kernel<T, 1>), grid, block, 0, dev->stream, (const T*)x, dev->gn_scratch, glen, chunk, splits);
-        RT_CHECK_LAUNCH("gn_stats_kernel");
-        hipLaunchKernelGGL((gn_apply_kernel<T, 1>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, (T*)y,
-                           (const float*)dev->gn_scratch, glen, chunk, splits, cpg, groups, make_fastdiv(L), eps);
+        hipLaunchKernelGGL((gn_apply_kernel<T, 1>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, (T*)y, stats,
+                           glen, chunk, stat_splits, cpg, groups, make_fastdiv(L), eps);
     }
     RT_CHECK_LAUNCH("gn_apply_kernel");
     return RT_OK;

@@ -318,6 +318,7 @@ def test_layer_norm_variance_form_matches_reference(dev, oracle):
                                      (1, 512, 3000, 32),          # the benchmark shape: 32 groups of 96 KB, staged in LDS, one launch
                                      (9, 128, 40, 64),            # 576 groups: more than two per CU, the two-launch streaming path
                                      (1, 8, 40000, 2),            # groups larger than LDS
+                                     (1, 4, 300000, 1),           # one group of 1.2 M elements: hundreds of slices, combined by a launch of their own
                                      (2, 16, 24, 4)])
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
 def test_group_norm(dev, oracle, B, C, L, G, dtype):
