@@ -340,6 +340,8 @@ struct SpSched {
     uint32_t R;              // rows per group actually used (<= SP_ROWS): chosen so that the groups fill whole rounds of the grid
     uint32_t nsteps;         // 512-column steps per row, rounded up to an even number (used by the long-row variant)
     FastDiv gp_div;
+    FastDiv pm_div;          // rows of the mask: row (rep * P + r) of x takes mask row (rep * P + r) % PM.  PM == P unless the
+    uint32_t PM;             // mask is only a few rows tall, where groups that stop at every period would be nearly empty
 };
 
 __device__ __forceinline__ uint32_t sp_item_count(const SpSched& s, uint32_t b, uint32_t G) {
@@ -474,24 +476,31 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
     const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(x), 0, nbytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(y, 0, nbytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t rm =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(MASK ? mask : x), 0, MASK ? sch.P * row_bytes : nbytes, 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(MASK ? mask : x), 0, MASK ? sch.PM * row_bytes : nbytes, 0x00020000);
     constexpr uint32_t OOB = 0x80000000u;                    // >= nbytes, and stays so after adding a column offset
     const uint32_t G = gridDim.x;
 
     // Row offsets are the same for all lanes of a wave, so they live in scalar registers (the vector registers are all
-    // needed for data): byte offset of rows rr / rr + 15 of item `it` in x / y, or OOB, and of the item's period in x
-    // (x offset - period offset = mask offset; for a row that does not exist the mask offset is arbitrary, which is
-    // harmless: the load is range checked, and what is computed from it is never stored).
-    auto item_off = [&](uint32_t it, uint32_t (&xo)[2], uint32_t& period_off) {
+    // needed for data): byte offset of rows rr / rr + 15 of item `it` in x / y, or OOB, and the difference between that
+    // and the row's offset in the mask (for a row that does not exist the mask offset is arbitrary, which is harmless:
+    // the load is range checked, and what is computed from it is never stored).
+    auto item_off = [&](uint32_t it, uint32_t (&xo)[2], uint32_t (&mdiff)[2]) {
         uint32_t rep, pg;
         sp_item(sch, blockIdx.x, G, it, rep, pg);
-        period_off = __builtin_amdgcn_readfirstlane(rep * sch.P * row_bytes);
 #pragma unroll
         for (int h = 0; h < 2; h++) {
             const uint32_t r = rr + h * SP_HALF;
             const uint32_t prow = pg * sch.R + r;            // row inside the period
             const bool ok = it < n_items && r < sch.R && prow < sch.P;
-            xo[h] = __builtin_amdgcn_readfirstlane(ok ? (rep * sch.P + prow) * row_bytes : OOB);
+            const uint32_t row = rep * sch.P + prow;
+            xo[h] = __builtin_amdgcn_readfirstlane(ok ? row * row_bytes : OOB);
+            if (MASK) {
+                uint32_t q, mrow;
+                fd_divmod(row, sch.pm_div, q, mrow);
+                mdiff[h] = __builtin_amdgcn_readfirstlane((row - mrow) * row_bytes);
+            } else {
+                mdiff[h] = 0;
+            }
         }
     };
     const uint32_t cbyte = ccol * 2;
@@ -555,7 +564,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
         if (past_end(t)) in = v4u{0, 0, 0, 0};
     };
 
-    uint32_t cur[2], nxt[2], prev[2] = {OOB, OOB}, pcur, pnxt;
+    uint32_t cur[2], nxt[2], prev[2] = {OOB, OOB}, pcur[2], pnxt[2];
     item_off(0, cur, pcur);
     item_off(1, nxt, pnxt);
     uint32_t gpar = 0;
@@ -577,7 +586,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
         }
         if (MASK) {
 #pragma unroll
-            for (int h = 0; h < 2; h++) mpre[h] = load_m(step_off(cur[h] - pcur, 0));
+            for (int h = 0; h < 2; h++) mpre[h] = load_m(step_off(cur[h] - pcur[h], 0));
         }
 
         for (uint32_t it = 0; it < n_items; it++) {
@@ -594,7 +603,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                 if (MASK) {
 #pragma unroll
                     for (int h = 0; h < 2; h++)
-                        mpre[h] = (t + 1 < NSTEP) ? load_m(step_off(cur[h] - pcur, t + 1)) : load_m(step_off(nxt[h] - pnxt, 0));
+                        mpre[h] = (t + 1 < NSTEP) ? load_m(step_off(cur[h] - pcur[h], t + 1)) : load_m(step_off(nxt[h] - pnxt[h], 0));
                 }
 #pragma unroll
                 for (int h = 0; h < 2; h++)
@@ -613,7 +622,8 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                 prev[h] = cur[h];
                 cur[h] = nxt[h];
             }
-            pcur = pnxt;
+            pcur[0] = pnxt[0];
+            pcur[1] = pnxt[1];
             item_off(it + 2, nxt, pnxt);
             gpar ^= 1;
         }
@@ -636,7 +646,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
             for (int h = 0; h < 2; h++) store_park(v4u{0, 0, 0, 0}, OOB);
             if (MASK) {
 #pragma unroll
-                for (int h = 0; h < 2; h++) mpre[h] = load_m(step_off(cur[h] - pcur, 0));
+                for (int h = 0; h < 2; h++) mpre[h] = load_m(step_off(cur[h] - pcur[h], 0));
             }
 #pragma unroll
             for (int h = 0; h < 2; h++) pre[k][h] = load_x(step_off(cur[h], k));
@@ -663,7 +673,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                 if (MASK) {
                     const bool w1 = t + 1 >= nsteps;
 #pragma unroll
-                    for (int h = 0; h < 2; h++) mpre[h] = load_m(step_off(w1 ? nxt[h] - pnxt : cur[h] - pcur, w1 ? 0 : t + 1));
+                    for (int h = 0; h < 2; h++) mpre[h] = load_m(step_off(w1 ? nxt[h] - pnxt[h] : cur[h] - pcur[h], w1 ? 0 : t + 1));
                 }
 #pragma unroll
                 for (int h = 0; h < 2; h++) pre[k][h] = load_x(step_off(wrap ? nxt[h] : cur[h], ta));
@@ -683,7 +693,8 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                     prev[h] = cur[h];
                     cur[h] = nxt[h];
                 }
-                pcur = pnxt;
+                pcur[0] = pnxt[0];
+                pcur[1] = pnxt[1];
                 item_off(trip / (nsteps / 2) + 2, nxt, pnxt);
                 gpar ^= 1;
             }
@@ -959,7 +970,10 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
         const T* xc = (const T*)x + row0 * cols;
         T* yc = (T*)y + row0 * cols;
         SpSched sch;
-        sch.P = (uint32_t)(mask ? period : n);
+        // a mask of few rows (a [1, T] padding mask, a short prefill): groups run across its periods
+        sch.PM = (uint32_t)(mask ? period : n);
+        sch.pm_div = make_fastdiv(sch.PM);
+        sch.P = (uint32_t)(mask && period >= 8 * SP_ROWS ? period : n);
         sch.reps = (uint32_t)(n / sch.P);
         sch.nsteps = (nt + 1) & ~1u;
         // rows per group: every block runs ceil(groups / grid) rounds of 8-or-fewer steps whatever the group holds, so
