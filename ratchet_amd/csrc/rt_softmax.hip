@@ -729,6 +729,7 @@ struct MaskArgs {
     FastDiv d2, d1;          // x extents of dims 2 and 1 (rows = d0 * d1 * d2)
     uint32_t ms[3];          // mask row strides in elements over dims 0..2 (0 where the mask extent is 1)
     uint32_t mlast;          // 1: the mask has a full last dim, 0: one value per row
+    uint32_t mvec;           // the mask starts on a 16-byte boundary (the span kernel may read it in aligned vectors)
 };
 
 template <typename T> __device__ __forceinline__ uint64_t mask_row_offset(uint64_t row, const MaskArgs& p) {
@@ -813,6 +814,141 @@ __global__ void __launch_bounds__(BLOCK) softmax_via32_wave_kernel(const T* __re
 #pragma unroll
             for (int q = 0; q < 8; q++) o.e[q] = Ar<T>::conv(plain ? e[k][q] * rs : e[k][q] / s);
             st_stream(yr + i, o.u);
+        }
+    }
+}
+
+// Rows that are not whole aligned vectors (a prompt of 1001 tokens: [B, H, 1001, 1001] scores): the same kernel over the
+// span of aligned 16-byte vectors that covers the row.  Row r starts `shift` = (r * cols) % 8 elements into its first
+// vector; elements of the span outside the row belong to the neighbouring rows, are ignored on the way in and are not
+// written on the way out (the two ragged vectors of a row are stored element by element).  An aligned vector that
+// holds one byte of the tensor lies in a mapped page, so the loads are safe at the tensor's ends too.  The mask row has
+// an alignment of its own and is read one element at a time (cache hits).  x and y themselves must be 16-byte aligned.
+template <typename T, int NV, int MODE, bool MASK, int LANES>
+__global__ void __launch_bounds__(BLOCK) softmax_via32_span_kernel(const T* x, const T* __restrict__ mask, T* y, uint64_t rows,
+                                                                   uint32_t cols, MaskArgs p) {
+    const uint64_t row = (uint64_t)blockIdx.x * (BLOCK / LANES) + (threadIdx.x / LANES);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & (LANES - 1);
+    const uint64_t first = row * cols;
+    const uint32_t shift = (uint32_t)(first & 7);
+    const uint32_t nspan = (shift + cols + 7) >> 3;
+    const v4u* xv = reinterpret_cast<const v4u*>(x) + (first >> 3);
+    v4u* yv = reinterpret_cast<v4u*>(y) + (first >> 3);
+    T* yrow = y + first;
+    Vec16<T> v[NV];
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        const uint32_t i = lane + k * LANES;
+        if (i < nspan) v[k].u = ld_stream(xv + i);
+    }
+    // column of element q of span vector i: i * 8 + q - shift, valid when below cols (elements before the row wrap around)
+    auto column = [&](uint32_t i, int q) -> uint32_t { return i * 8 + (uint32_t)q - shift; };
+    if (MASK) {
+        const uint64_t mfirst = mask_row_offset<T>(row, p);
+        const T* mr = mask + mfirst;
+        if (p.mlast && p.mvec) {
+            // The mask element of span element (i, q) sits at mask element mfirst - shift + i * 8 + q: the eight of a span
+            // vector straddle two aligned mask vectors, d elements into the first (d is the same for the whole row).
+            const int64_t base = (int64_t)mfirst - (int64_t)shift;
+            const int64_t a0 = base >> 3;                    // floor: -1 when the row starts the mask and shift > 0
+            const uint32_t d = (uint32_t)(base - a0 * 8);
+            const int64_t mend = (int64_t)mfirst + cols;     // one past the row's last mask element
+            const v4u* mv = reinterpret_cast<const v4u*>(mask);
+#pragma unroll
+            for (int k = 0; k < NV; k++) {
+                const uint32_t i = lane + k * LANES;
+                const int64_t a = a0 + i;
+                v4u lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+                if (a >= 0 && a * 8 < mend) lo = mv[a];      // also the lane after the span: its vector may end the row's mask
+                // the second vector is the first one of the next lane; the last lane of a wave loads its own
+                const bool own = LANES != 64 || lane == 63;
+                if (LANES == 64) {
+#pragma unroll
+                    for (int w = 0; w < 4; w++) hi[w] = __shfl_down(lo[w], 1, 64);
+                }
+                if (own) {
+                    hi = v4u{0, 0, 0, 0};
+                    if (d != 0 && i < nspan && (a + 1) * 8 < mend) hi = mv[a + 1];
+                }
+                if (i < nspan) {
+                    const uint32_t cat[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    Vec16<T> mk;
+                    switch (d >> 1) {                        // uniform over the wave: a branch, not a select per lane
+#define RT_PICK(O)                                                                                                              \
+    _Pragma("unroll") for (int w = 0; w < 4; w++)                                                                              \
+        mk.u[w] = (d & 1) ? __builtin_amdgcn_alignbyte(cat[w + O + 1 < 8 ? w + O + 1 : 7], cat[w + O], 2) : cat[w + O];
+                        case 0: RT_PICK(0) break;
+                        case 1: RT_PICK(1) break;
+                        case 2: RT_PICK(2) break;
+                        default: RT_PICK(3) break;
+#undef RT_PICK
+                    }
+#pragma unroll
+                    for (int q = 0; q < 8; q++)
+                        if (column(i, q) < cols) v[k].e[q] = Ar<T>::add(v[k].e[q], mk.e[q]);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < NV; k++) {
+                const uint32_t i = lane + k * LANES;
+                if (i < nspan)
+#pragma unroll
+                    for (int q = 0; q < 8; q++) {
+                        const uint32_t c = column(i, q);
+                        if (c < cols) v[k].e[q] = Ar<T>::add(v[k].e[q], mr[p.mlast ? c : 0]);
+                    }
+            }
+        }
+    }
+    float e[NV][8];
+    float m = 0.0f;
+    if (MODE == 1) {
+        m = -__builtin_huge_valf();
+#pragma unroll
+        for (int k = 0; k < NV; k++) {
+            const uint32_t i = lane + k * LANES;
+            if (i < nspan)
+#pragma unroll
+                for (int q = 0; q < 8; q++)
+                    if (column(i, q) < cols) m = fmaxf(m, Ar<T>::widen(v[k].e[q]));
+        }
+        m = row_max<LANES>(m);
+        if (m == -__builtin_huge_valf()) m = 0.0f;
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        const uint32_t i = lane + k * LANES;
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            e[k][q] = 0.0f;
+            if (i < nspan && column(i, q) < cols) {
+                e[k][q] = via32_exp(Ar<T>::widen(v[k].e[q]) - m);
+                s += e[k][q];
+            }
+        }
+    }
+    s = row_sum<LANES>(s);
+    const bool plain = (s >= 1.17549435e-38f) && (s < __builtin_huge_valf());
+    const float rs = 1.0f / s;
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        const uint32_t i = lane + k * LANES;
+        if (i < nspan) {
+            Vec16<T> o;
+#pragma unroll
+            for (int q = 0; q < 8; q++) o.e[q] = Ar<T>::conv(plain ? e[k][q] * rs : e[k][q] / s);
+            if (column(i, 0) < cols && column(i, 7) < cols) {
+                st_stream(yv + i, o.u);
+            } else {
+#pragma unroll
+                for (int q = 0; q < 8; q++) {
+                    const uint32_t c = column(i, q);
+                    if (c < cols) yrow[c] = o.e[q];
+                }
+            }
         }
     }
 }
@@ -1087,6 +1223,39 @@ int launch_via32(rt_device* dev, const void* x, const void* mask, void* y, uint6
         RT_CHECK_LAUNCH("softmax_via32_wave_kernel");
         return RT_OK;
     }
+    // rows that are not whole aligned vectors, in tensors that start on a vector boundary: the span kernel
+    const uint32_t span = (cols + 14) / 8;                   // vectors a row can touch at most
+    if (rt_aligned(x, 16) && rt_aligned(y, 16) && span <= (uint32_t)(BLOCK * 8)) {
+        if (span <= (uint32_t)(WAVE * 8)) {
+            const uint32_t nv = (span + WAVE - 1) / WAVE;
+            const uint64_t blocks = (rows + WAVES - 1) / WAVES;
+            RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax_via_f32: too many rows");
+            const dim3 grid((unsigned)blocks), block(BLOCK);
+#define RT_SV(NVC)                                                                                                                 \
+    hipLaunchKernelGGL((softmax_via32_span_kernel<T, NVC, MODE, MASK, WAVE>), grid, block, 0, dev->stream, (const T*)x, (const T*)mask, \
+                       (T*)y, rows, cols, p)
+            if (nv <= 1) RT_SV(1);
+            else if (nv <= 2) RT_SV(2);
+            else if (nv <= 4) RT_SV(4);
+            else if (nv <= 6) RT_SV(6);
+            else RT_SV(8);
+#undef RT_SV
+        } else {
+            const uint32_t nv = (span + BLOCK - 1) / BLOCK;
+            RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax_via_f32: too many rows");
+            const dim3 grid((unsigned)rows), block(BLOCK);
+#define RT_SV(NVC)                                                                                                                  \
+    hipLaunchKernelGGL((softmax_via32_span_kernel<T, NVC, MODE, MASK, BLOCK>), grid, block, 0, dev->stream, (const T*)x, (const T*)mask, \
+                       (T*)y, rows, cols, p)
+            if (nv <= 3) RT_SV(3);
+            else if (nv <= 4) RT_SV(4);
+            else if (nv <= 6) RT_SV(6);
+            else RT_SV(8);
+#undef RT_SV
+        }
+        RT_CHECK_LAUNCH("softmax_via32_span_kernel");
+        return RT_OK;
+    }
     RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax_via_f32: too many rows");
     hipLaunchKernelGGL((softmax_via32_generic_kernel<T, MODE, MASK>), dim3((unsigned)rows), dim3(BLOCK), 0, dev->stream, (const T*)x,
                        (const T*)mask, (T*)y, rows, cols, p);
@@ -1134,6 +1303,7 @@ extern "C" int rt_softmax_via_f32(rt_device* dev, int io_dt, const void* x, cons
     p.d1 = make_fastdiv(x_shape[1]);
     p.ms[0] = p.ms[1] = p.ms[2] = 0;
     p.mlast = 0;
+    p.mvec = mask && rt_aligned(mask, 16) ? 1u : 0u;
     bool mask_vec_ok = true;
     if (mask) {
         uint64_t st = 1;

@@ -132,7 +132,11 @@ def _attn_case(rng, B, H, S, T, mask_kind, dtype=np.float16):
                                                (2, 2, 33, 77, "per_batch"), (1, 2, 40, 64, "row_scalar"), (1, 8, 512, 1024, "causal"),
                                                (1, 2, 7, 4096, "causal"), (1, 1, 3, 8200, None), (1, 3, 5, 4100, "causal"),
                                                (1, 2, 6, 8192, "causal"), (2, 1, 3, 16384, "per_batch"), (1, 2, 4, 6000, None),
-                                               (1, 1, 2, 16392, None)])
+                                               (1, 1, 2, 16392, None),
+                                               # rows that are not whole vectors (prompts of 1001, 333, 13 tokens): the span kernel
+                                               (1, 4, 1001, 1001, "causal"), (2, 3, 333, 333, "causal4"), (1, 2, 5, 13, "causal"),
+                                               (2, 2, 9, 1004, "per_batch"), (1, 3, 1, 2047, None), (1, 2, 3, 4101, "causal"),
+                                               (1, 2, 2, 9001, None), (1, 1, 3, 1, None), (3, 1, 7, 7, "row_scalar")])
 def test_softmax_via_f32(dev, oracle, B, H, S, T, mask_kind):
     rng = np.random.default_rng(504)
     x, mask = _attn_case(rng, B, H, S, T, mask_kind)
@@ -151,6 +155,9 @@ def test_softmax_via_f32(dev, oracle, B, H, S, T, mask_kind):
     stable = dev.softmax_via_f32(dev.upload(x), dev.upload(mask) if mask is not None else None, mode=_lib.SOFTMAX_STABLE).to_numpy()
     ok, info = close(oracle, stable, want, 1e-3)
     assert ok, ("stable", info)
+    dx = dev.upload(x)                                        # in place: a row's ragged ends share vectors with its neighbours
+    dev.softmax_via_f32(dx, dev.upload(mask) if mask is not None else None, out=dx)
+    assert same_bits(dx.to_numpy(), got)
 
 
 def test_softmax_via_f32_overflow_and_fully_masked_rows(dev, oracle):
