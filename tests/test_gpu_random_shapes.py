@@ -87,7 +87,7 @@ def test_rows_random(dev, oracle, seed):
     rng = np.random.default_rng(920 + seed)
     for _ in range(12):
         rows = int(rng.integers(1, 70))
-        cols = int(rng.choice([1, 2, 7, 8, 33, 64, 255, 256, 520, 1000, 2048, 2056, 4096, 4104, 5000]))
+        cols = int(rng.choice([1, 2, 7, 8, 12, 33, 64, 255, 256, 520, 1000, 1001, 2047, 2048, 2056, 4096, 4104, 5000, 8200]))
         off = int(rng.choice([0, 0, 1, 3, 8]))
         for dtype, tol in ((np.float32, 1e-5), (np.float16, 0.0)):
             x = randn(rng, (rows, cols), dtype, 2.0)
@@ -123,3 +123,17 @@ def test_rows_random(dev, oracle, seed):
                 want = oracle.cast(oracle.softmax(x.astype(np.float32)), np.float16)
                 bad, mx = oracle.count_not_close(got, want, 1e-3, 1e-3)
                 assert bad == 0, ("softmax_via_f32", rows, cols, off, mx)
+                # with the mask, at an element offset of its own (the mask's alignment is independent of the rows')
+                moff = int(rng.choice([0, 0, 5, 8]))
+                mv = BufferView(dev.empty((rows * cols + 16,), 1), moff, (rows, cols)).upload(mask)
+                got = dev.softmax_via_f32(xv, mv).to_numpy()
+                want = oracle.cast(oracle.softmax(oracle.binary("add", x, mask).astype(np.float32)), np.float16)
+                bad, mx = oracle.count_not_close(got, want, 1e-3, 1e-3)
+                assert bad == 0, ("softmax_via_f32 masked", rows, cols, off, moff, mx)
+                # bf16 reference softmax on the same numbers
+                xb = oracle.cast(x.astype(np.float32), np.uint16, dst_bf16=True)
+                bv = BufferView(dev.empty((rows * cols + 16,), 2), off, (rows, cols)).upload(xb)
+                got = dev.softmax(bv).to_numpy()
+                want = oracle.softmax(xb, bf16=True)
+                nan = (want & 0x7fff) > 0x7f80
+                assert np.array_equal(got[~nan], want[~nan]) and (((got & 0x7fff) > 0x7f80) == nan).all(), ("softmax bf16", rows, cols, off)
