@@ -1154,8 +1154,10 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
     return RT_OK;
 }
 
+// (rows that are not whole aligned vectors only: everything else streams.  Eight rows per block: a thousand rows of
+// 1001 columns are 125 blocks, not 16)
 template <typename T> int launch_seq16(rt_device* dev, const void* x, void* y, uint64_t rows, uint32_t cols) {
-    constexpr int RB = 64, TC = 128;
+    constexpr int RB = 8, TC = 512;
     const uint64_t blocks = (rows + RB - 1) / RB;
     RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax: too many rows");
     const bool vec_ok = (cols % 8 == 0) && rt_aligned(x, 16) && rt_aligned(y, 16);
