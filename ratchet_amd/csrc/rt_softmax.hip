@@ -1003,8 +1003,7 @@ __global__ void __launch_bounds__(BLOCK) softmax_via32_generic_kernel(const T* _
 template <typename T, int MODE> int launch_wave(rt_device* dev, const void* x, void* y, uint64_t rows, uint32_t cols) {
     constexpr int VE = 16 / sizeof(T);
     const uint32_t nvec = cols / VE;
-    const bool vec_ok = true;
-    if (vec_ok && nvec <= 32) {
+    if (nvec <= 32) {
         // rows of at most 32 vectors: a group of 2..32 lanes per row (one vector each), so that a wave carries 2..32 rows
         // and as many bytes as with long rows
         const uint32_t lanes = nvec <= 2 ? 2 : nvec <= 4 ? 4 : nvec <= 8 ? 8 : nvec <= 16 ? 16 : 32;
