@@ -1,0 +1,178 @@
+// The libm-level routines of the kernels, in portable C++ so that the same text can be compiled for the host and checked
+// against the C library there (tests/device_math_check.cpp does, with g++): the includer defines
+//   RT_FN     the function qualifiers (`__device__ inline` in the kernels, `static inline` on the host)
+//   RT_TABLE  the qualifiers of a constant table (`__device__ static const` / `static const`)
+//
+// Two libm routines are restated operation by operation so that their float32 results equal, bit for bit, what the
+// x86-64 glibc 2.35 `tanhf` and `expf` return (checked on the CPU over all 2^32 inputs with this same code compiled
+// by g++).  ratchet's CPU executor calls exactly those through Rust's f32::tanh / f32::exp
+// (crates/ratchet-core/src/cpu/unary.rs:46-65, cpu/softmax.rs:30), and GELU's `1 + tanh(..)` cancellation turns a
+// 1-ulp tanh difference into hundreds of ulps, so "close" is not good enough there.
+//   tanhf/expm1f: the classic fdlibm float algorithms (float arithmetic only).
+//   expf: the table-driven double-precision algorithm (2^(k/32) table, degree-3 polynomial), with the
+//         reduction r = fma(InvLn2N, x, -kd) that an FMA build of the routine performs.
+// Everything here must be compiled with -ffp-contract=off: each float operation below is meant to round on its own.
+#ifndef RT_LIBM_H
+#define RT_LIBM_H
+
+#include <math.h>
+#include <stdint.h>
+
+RT_FN uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
+RT_FN float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
+
+// ---- expm1f, fdlibm -------------------------------------------------------------------------------------
+RT_FN float rt_expm1f(float x) {
+    const float one = 1.0f, huge = 1.0e+30f, tiny = 1.0e-30f;
+    const float o_threshold = 8.8721679688e+01f, ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f,
+                invln2 = 1.4426950216e+00f;
+    const float Q1 = -3.3333335072e-02f, Q2 = 1.5873016091e-03f, Q3 = -7.9365076090e-05f, Q4 = 4.0082177293e-06f,
+                Q5 = -2.0109921195e-07f;
+    float y, hi, lo, c = 0.0f, t, e, hxs, hfx, r1;
+    int32_t k;
+    uint32_t hx = f2u(x);
+    const uint32_t xsb = hx & 0x80000000u;
+    hx &= 0x7fffffffu;
+    if (hx >= 0x4195b844u) {                       // |x| >= 27 ln2
+        if (hx >= 0x42b17218u) {                   // |x| >= 88.72
+            if (hx > 0x7f800000u) return x + x;    // NaN
+            if (hx == 0x7f800000u) return xsb == 0 ? x : -1.0f;
+            if (x > o_threshold) return huge * huge;
+        }
+        if (xsb != 0) {
+            if (x + tiny < 0.0f) return tiny - one;
+        }
+    }
+    if (hx > 0x3eb17218u) {                        // |x| > 0.5 ln2
+        if (hx < 0x3F851592u) {                    // |x| < 1.5 ln2
+            if (xsb == 0) { hi = x - ln2_hi; lo = ln2_lo; k = 1; }
+            else { hi = x + ln2_hi; lo = -ln2_lo; k = -1; }
+        } else {
+            k = (int32_t)(invln2 * x + ((xsb == 0) ? 0.5f : -0.5f));
+            t = (float)k;
+            hi = x - t * ln2_hi;
+            lo = t * ln2_lo;
+        }
+        x = hi - lo;
+        c = (hi - x) - lo;
+    } else if (hx < 0x33000000u) {                 // |x| < 2^-25
+        t = huge + x;
+        return x - (t - (huge + x));
+    } else {
+        k = 0;
+    }
+    hfx = 0.5f * x;
+    hxs = x * hfx;
+    r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
+    t = 3.0f - r1 * hfx;
+    e = hxs * ((r1 - t) / (6.0f - x * t));
+    if (k == 0) return x - (x * e - hxs);
+    e = (x * (e - c) - c);
+    e -= hxs;
+    if (k == -1) return 0.5f * (x - e) - 0.5f;
+    if (k == 1) {
+        if (x < -0.25f) return -2.0f * (e - (x + 0.5f));
+        return one + 2.0f * (x - e);
+    }
+    if (k <= -2 || k > 56) {
+        y = one - (e - x);
+        y = u2f(f2u(y) + ((uint32_t)k << 23));
+        return y - one;
+    }
+    if (k < 23) {
+        t = u2f(0x3f800000u - (0x1000000u >> k));  // 1 - 2^-k
+        y = t - (e - x);
+        y = u2f(f2u(y) + ((uint32_t)k << 23));
+    } else {
+        t = u2f((uint32_t)(0x7f - k) << 23);       // 2^-k
+        y = x - (e + t);
+        y += one;
+        y = u2f(f2u(y) + ((uint32_t)k << 23));
+    }
+    return y;
+}
+
+// ---- tanhf, fdlibm --------------------------------------------------------------------------------------
+RT_FN float rt_tanhf(float x) {
+    const float one = 1.0f, two = 2.0f, tiny = 1.0e-30f;
+    float t, z;
+    const int32_t jx = (int32_t)f2u(x);
+    const int32_t ix = jx & 0x7fffffff;
+    if (ix >= 0x7f800000) {
+        if (jx >= 0) return one / x + one;         // tanh(+inf) = 1, NaN stays NaN
+        return one / x - one;
+    }
+    if (ix < 0x41b00000) {                         // |x| < 22
+        if (ix == 0) return x;
+        if (ix < 0x24000000) return x * (one + x); // |x| < 2^-55
+        // one expm1f evaluation for both ranges (lanes of a wave take both, and two inlined copies would both run):
+        // |x| >= 1: t = expm1f(2|x|), z = 1 - 2 / (t + 2); |x| < 1: t = expm1f(-2|x|), z = -t / (t + 2)
+        const bool big = ix >= 0x3f800000;
+        t = rt_expm1f(big ? two * fabsf(x) : -two * fabsf(x));
+        const float q = (big ? two : -t) / (t + two);
+        z = big ? one - q : q;
+    } else {
+        z = one - tiny;
+    }
+    return (jx >= 0) ? z : -z;
+}
+
+// ---- expf, table-driven double algorithm ----------------------------------------------------------------
+// T[i] = bits(2^(i/32)) - (i << 47)
+RT_TABLE uint64_t rt_exp2f_tab[32] = {
+    0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull,
+    0x3fef72b83c7d517bull, 0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull,
+    0x3fef06fe0a31b715ull, 0x3feef1a7373aa9cbull, 0x3feedea64c123422ull, 0x3feece086061892dull,
+    0x3feebfdad5362a27ull, 0x3feeb42b569d4f82ull, 0x3feeab07dd485429ull, 0x3feea47eb03a5585ull,
+    0x3feea09e667f3bcdull, 0x3fee9f75e8ec5f74ull, 0x3feea11473eb0187ull, 0x3feea589994cce13ull,
+    0x3feeace5422aa0dbull, 0x3feeb737b0cdc5e5ull, 0x3feec49182a3f090ull, 0x3feed503b23e255dull,
+    0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull,
+    0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull};
+
+RT_FN float rt_expf(float x) {
+    const double N = 32.0;
+    const double InvLn2N = 0x1.71547652b82fep+0 * N;
+    const double SHIFT = 0x1.8p52;
+    const double C0 = 0x1.c6af84b912394p-5 / N / N / N, C1 = 0x1.ebfce50fac4f3p-3 / N / N, C2 = 0x1.62e42ff0c52d6p-1 / N;
+    const uint32_t abstop = (f2u(x) >> 20) & 0x7ffu;
+    if (abstop >= (0x42b00000u >> 20)) {           // |x| >= 88 or NaN
+        if (f2u(x) == 0xff800000u) return 0.0f;
+        if (abstop >= (0x7f800000u >> 20)) return x + x;
+        if (x > 0x1.62e42ep6f) return __builtin_huge_valf();
+        if (x < -0x1.9fe368p6f) return 0.0f;
+    }
+    const double xd = (double)x;
+    const double z = InvLn2N * xd;
+    double kd = z + SHIFT;
+    const uint64_t ki = __builtin_bit_cast(uint64_t, kd);
+    kd -= SHIFT;
+    const double r = __builtin_fma(InvLn2N, xd, -kd);
+    uint64_t t = rt_exp2f_tab[ki & 31];
+    t += ki << (52 - 5);
+    const double s = __builtin_bit_cast(double, t);
+    const double p = __builtin_fma(C0, r, C1);
+    const double r2 = r * r;
+    double y = __builtin_fma(C2, r, 1.0);
+    y = __builtin_fma(p, r2, y);
+    y = y * s;
+    return (float)y;
+}
+
+// log / sin / cos: evaluated in double and rounded once.  The double routines are accurate to about 1 ulp of
+// double, so the float result is the correctly rounded one except in astronomically rare double-rounding cases;
+// glibc's logf/sinf/cosf are within 1 float ulp of that.
+RT_FN float rt_logf(float x) { return (float)log((double)x); }
+RT_FN float rt_sinf(float x) { return (float)sin((double)x); }
+RT_FN float rt_cosf(float x) { return (float)cos((double)x); }
+
+// bf16 <-> f32 with the rounding of half::bf16::from_f32 (round to nearest even, NaN quieted)
+RT_FN float bf2f(uint16_t b) { return u2f((uint32_t)b << 16); }
+RT_FN uint16_t f2bf(float f) {
+    const uint32_t x = f2u(f);
+    if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x0040u);
+    const uint32_t round_bit = 0x00008000u;
+    if ((x & round_bit) != 0 && (x & (3u * round_bit - 1u)) != 0) return (uint16_t)((x >> 16) + 1);
+    return (uint16_t)(x >> 16);
+}
+
+#endif
