@@ -130,7 +130,7 @@ def test_cast_and_reindex_trials(hdev, oracle):
 
 
 def test_whisper_bias_gelu_layer_norm_graph(hdev, oracle):
-    # BASELINE config 0 as ONE lazy graph: bias add (broadcast fused) -> tanh GELU -> LayerNorm, f32
+    # the reference-runnable benchmark case as ONE lazy graph: bias add (broadcast fused) -> tanh GELU -> LayerNorm, f32
     rng = np.random.default_rng(404)
     x = rng.standard_normal((1, 1500, 384)).astype(np.float32)
     bias = (0.02 * rng.standard_normal(384)).astype(np.float32)

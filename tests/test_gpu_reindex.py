@@ -1,7 +1,7 @@
 """GPU parity: permute / slice / broadcast_to / concat against the CPU oracle (bit-exact), through the C ABI.
 
 Problem spaces follow the reference's own tests (crates/ratchet-core/src/ops/reindex/{permute,slice,broadcast}.rs,
-ops/concat.rs) plus the BASELINE shapes and alignment / odd-size edge cases.
+ops/concat.rs) plus the benchmark shapes and alignment / odd-size edge cases.
 """
 import itertools
 
