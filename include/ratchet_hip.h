@@ -137,6 +137,16 @@ int rt_cache(rt_device* dev, int elem_bytes, void* cache, const uint32_t cache_s
 int rt_index_select(rt_device* dev, int elem_bytes, const void* src, const uint32_t src_shape[4], const int32_t* indices,
                     uint32_t n_indices, int dim, void* dst);
 
+/* IndexSelect from a Q8_0 source (ops/select.rs:107-111,144-161; cpu/mod.rs:86-103 with quant.rs:101-130): the
+ * embedding lookup of a quantized model.  `packed` and `scales` are the two segments of the reference's quantized buffer
+ * (quant.rs:19-49): numel / 4 words of four signed bytes each, then, from the next multiple of 256 bytes on, numel / 32
+ * scales; scale_dt RT_F32 is Q8_0F, RT_F16 is Q8_0H, and dst has that type.  dst[left, i, right] =
+ * int8(src[left, indices[i], right]) * scale[group of 32 of that flat source element], one rounding.  numel must be a
+ * multiple of 32 and the extents after `dim` a multiple of 4, as in the reference; rows for indices outside the source
+ * are zero (the reference's kernel clamps the index, its CPU path panics). */
+int rt_index_select_q8_0(rt_device* dev, int scale_dt, const uint32_t* packed, const void* scales, const uint32_t src_shape[4],
+                         const int32_t* indices, uint32_t n_indices, int dim, void* dst);
+
 /* IndexWrite (ops/index_write.rs:14-111): dst, in place, receives the src_numel elements of src as one flat run that
  * starts at the element write_start addresses (D[offset(write_start) + i] = S[i], :96-104).  A run that would leave dst
  * is rejected (the reference's kernel has no bound). */

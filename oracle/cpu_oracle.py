@@ -46,6 +46,8 @@ def lib():
         L.orc_rope.argtypes = [i, vp, vp, vp, ctypes.c_uint64, f, ctypes.c_uint64]
         L.orc_index_select.argtypes = [i, vp, i, vp, vp, ctypes.c_uint64, i, vp]
         L.orc_index_write.argtypes = [i, vp, i, vp, vp, ctypes.c_uint64, vp]
+        L.orc_q8_0_quantize.argtypes = [i, vp, ctypes.c_uint64, vp, vp]
+        L.orc_q8_0_dequantize.argtypes = [i, vp, vp, ctypes.c_uint64, vp]
         L.orc_softmax.argtypes = [i, vp, vp, sz, sz]
         L.orc_layer_norm.argtypes = [i, vp, vp, vp, vp, sz, sz, f, sz]
         L.orc_rms_norm.argtypes = [i, vp, vp, vp, sz, sz, f, sz]
@@ -197,6 +199,30 @@ def index_select(src, indices, dim):
     _check(lib().orc_index_select(src.dtype.itemsize, _p(src), src.ndim, _p(_u64(src.shape)), _p(indices), indices.shape[0], dim, _p(y)),
            "index_select")
     return y
+
+
+def q8_0_quantize(x):
+    """quantize::<Q8_0F / Q8_0H>(x) by x's dtype (float32 / float16): (words uint32 [numel / 4], scales [numel / 32])"""
+    x = _c(x)
+    fp = 1 if x.dtype == np.float16 else 0
+    words = np.empty(x.size // 4, np.uint32)
+    scales = np.empty(x.size // 32, x.dtype)
+    _check(lib().orc_q8_0_quantize(fp, _p(x), x.size, _p(words), _p(scales)), "q8_0_quantize")
+    return words, scales
+
+
+def q8_0_dequantize(words, scales, shape):
+    """dequantize of a Q8_0F (float32 scales) / Q8_0H (float16 scales) buffer to an array of `shape`"""
+    words, scales = np.ascontiguousarray(words, np.uint32), _c(scales)
+    fp = 1 if scales.dtype == np.float16 else 0
+    y = np.empty(shape, scales.dtype)
+    _check(lib().orc_q8_0_dequantize(fp, _p(words), _p(scales), y.size, _p(y)), "q8_0_dequantize")
+    return y
+
+
+def q8_0_index_select(words, scales, shape, indices, dim):
+    """IndexSelect from a quantized source: dequantize everything, then index_select (cpu/mod.rs:86-103)"""
+    return index_select(q8_0_dequantize(words, scales, shape), indices, dim)
 
 
 def index_write(dst, src, write_start):

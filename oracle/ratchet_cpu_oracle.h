@@ -74,6 +74,14 @@ int orc_index_select(int elem_bytes, const void* src, int rank, const uint64_t* 
 int orc_index_write(int elem_bytes, void* dst, int rank, const uint64_t* dst_shape, const void* src, uint64_t src_numel,
                     const uint64_t* write_start);
 
+/* Q8_0 quantized buffers (crates/ratchet-core/src/quant.rs:19-49 quantize_inner, :101-130 dequantize_inner, with
+ * PACK_SIZE 4, GROUP_SIZE 32, SF 127 from dtype/blocks.rs:180-199).  fp_dt 0 = Q8_0F (f32 scales), 1 = Q8_0H (f16 scales,
+ * every operation rounded to f16).  numel must be a multiple of 32.  words: numel / 4, scales: numel / 32 (the reference
+ * stores them in one buffer, the scales from the next multiple of 256 bytes after the words on).
+ * A quantized IndexSelect is dequantize followed by orc_index_select, as cpu/mod.rs:86-103 does it. */
+int orc_q8_0_quantize(int fp_dt, const void* x, uint64_t numel, uint32_t* words, void* scales);
+int orc_q8_0_dequantize(int fp_dt, const uint32_t* words, const void* scales, uint64_t numel, void* y);
+
 int orc_softmax(int dt, const void* x, void* y, size_t rows, size_t cols);
 /* shape0 = size of the input's first dimension: the reference broadcasts scale/bias with a
  * vector special case that depends on it (pass 1 to get the mathematically intended result) */

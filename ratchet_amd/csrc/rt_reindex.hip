@@ -7,6 +7,7 @@
 // vectors along the destination's last dimension with multiply-shift index math.  A permutation that moves the
 // source's contiguous dimension is transposed in V x V blocks in registers when rows are whole 16-byte vectors, and
 // through an LDS tile otherwise, so both the read and the write side stay coalesced.
+#include "rt_arith.h"
 #include "rt_internal.h"
 
 namespace {
@@ -309,6 +310,39 @@ __global__ void __launch_bounds__(BLOCK) index_select_kernel(const VecT* __restr
     VecT val = {};
     if (idx < p.src_dim) val = src[((uint64_t)left * p.src_dim + idx) * p.rv.d + col];
     st_stream(dst + v, val);
+}
+
+// IndexSelect from a Q8_0 source (the embedding table of a quantized model): four signed bytes per packed word, one scale
+// per 32 consecutive elements of the flat source; a thread expands one word: dst = float(int8) * scale, rounded once to
+// the scale's type (f32 for Q8_0F, f16 for Q8_0H).
+template <typename T>
+__global__ void __launch_bounds__(BLOCK) index_select_q8_kernel(const uint32_t* __restrict__ packed, const T* __restrict__ scales,
+                                                                const int32_t* __restrict__ indices, T* __restrict__ dst, SelectArgs p) {
+    const uint32_t v = blockIdx.x * BLOCK + threadIdx.x;       // destination word index: 4 elements
+    if (v >= p.nvec) return;
+    uint32_t row, col, left, i;
+    fd_divmod(v, p.rv, row, col);
+    fd_divmod(row, p.n_ids, left, i);
+    const uint32_t idx = (uint32_t)indices[i];
+    T out[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) out[j] = Ar<T>::conv(0.0f);
+    if (idx < p.src_dim) {
+        const uint64_t w = ((uint64_t)left * p.src_dim + idx) * p.rv.d + col;          // source word
+        const uint32_t q = packed[w];
+        const float sc = Ar<T>::widen(scales[w >> 3]);
+#pragma unroll
+        for (int j = 0; j < 4; j++) out[j] = Ar<T>::conv((float)(int8_t)(q >> (8 * j)) * sc);
+    }
+    if (sizeof(T) == 4) {
+        v4u o;
+        __builtin_memcpy(&o, out, 16);
+        st_stream(reinterpret_cast<v4u*>(dst) + v, o);
+    } else {
+        v2u o;
+        __builtin_memcpy(&o, out, 8);
+        st_stream(reinterpret_cast<v2u*>(dst) + v, o);
+    }
 }
 
 // IndexWrite: a flat run of src copied into dst from a linear offset (bytes here)
@@ -774,6 +808,46 @@ int rt_index_select(rt_device* dev, int elem_bytes, const void* src, const uint3
     else if (vb == 4) hipLaunchKernelGGL((index_select_kernel<uint32_t>), grid, block, 0, dev->stream, (const uint32_t*)src, indices, (uint32_t*)dst, p);
     else hipLaunchKernelGGL((index_select_kernel<uint16_t>), grid, block, 0, dev->stream, (const uint16_t*)src, indices, (uint16_t*)dst, p);
     RT_CHECK_LAUNCH("index_select_kernel");
+    return RT_OK;
+}
+
+int rt_index_select_q8_0(rt_device* dev, int scale_dt, const uint32_t* packed, const void* scales, const uint32_t src_shape[4],
+                         const int32_t* indices, uint32_t n_indices, int dim, void* dst) {
+    RT_REQUIRE(scale_dt == RT_F32 || scale_dt == RT_F16, RT_ERR_DTYPE, "rt_index_select_q8_0: scale dtype %d is not F32 (Q8_0F) / F16 (Q8_0H)",
+               scale_dt);
+    RT_REQUIRE(dim >= 0 && dim < 4, RT_ERR_ARG, "rt_index_select_q8_0: dim %d out of range", dim);
+    RT_REQUIRE(src_shape, RT_ERR_NULL_POINTER, "rt_index_select_q8_0: NULL shape");
+    RT_REQUIRE(n_indices > 0, RT_ERR_SHAPE, "rt_index_select_q8_0: no indices");
+    uint64_t left = 1, right = 1;
+    for (int a = 0; a < 4; a++) {
+        RT_REQUIRE(src_shape[a] > 0, RT_ERR_SHAPE, "rt_index_select_q8_0: zero extent in dim %d", a);
+        if (a < dim) left *= src_shape[a];
+        if (a > dim) right *= src_shape[a];
+    }
+    const uint64_t numel = left * src_shape[dim] * right;
+    RT_REQUIRE(numel <= RT_MAX_NUMEL, RT_ERR_SIZE, "rt_index_select_q8_0: source too large");
+    // quantize_inner's own conditions (quant.rs:20-21) and the kernel's word granularity (ops/select.rs:144-161)
+    RT_REQUIRE(numel % 32 == 0 && right % 4 == 0, RT_ERR_SHAPE,
+               "rt_index_select_q8_0: %llu elements / runs of %llu: the source must be whole groups of 32 and the runs whole words of 4",
+               (unsigned long long)numel, (unsigned long long)right);
+    RT_REQUIRE(packed && scales && indices && dst, RT_ERR_NULL_POINTER, "rt_index_select_q8_0: NULL operand");
+    const size_t ob = scale_dt == RT_F32 ? 16 : 8;
+    RT_REQUIRE(rt_aligned(packed, 4) && rt_aligned(scales, (size_t)rt_dt_bytes(scale_dt)) && rt_aligned(indices, 4) && rt_aligned(dst, ob),
+               RT_ERR_ALIGN, "rt_index_select_q8_0: misaligned pointer (the destination must be aligned to four elements)");
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    const uint64_t nvec = left * n_indices * (right / 4);
+    RT_REQUIRE(nvec <= 0xffffffffull - BLOCK && left * n_indices <= 0xffffffffull, RT_ERR_SIZE,
+               "rt_index_select_q8_0: output too large for 32-bit word indices");
+    SelectArgs p;
+    p.rv = make_fastdiv((uint32_t)(right / 4));
+    p.n_ids = make_fastdiv(n_indices);
+    p.src_dim = src_shape[dim];
+    p.nvec = (uint32_t)nvec;
+    const dim3 grid(blocks_for(nvec, BLOCK)), block(BLOCK);
+    if (scale_dt == RT_F32) hipLaunchKernelGGL((index_select_q8_kernel<float>), grid, block, 0, dev->stream, packed, (const float*)scales, indices, (float*)dst, p);
+    else hipLaunchKernelGGL((index_select_q8_kernel<half_t>), grid, block, 0, dev->stream, packed, (const half_t*)scales, indices, (half_t*)dst, p);
+    RT_CHECK_LAUNCH("index_select_q8_kernel");
     return RT_OK;
 }
 

@@ -284,6 +284,17 @@ class Device:
                                        dim + (4 - rank), out.ptr))
         return out
 
+    def index_select_q8_0(self, packed, scales, src_shape, indices, dim, out=None):
+        """IndexSelect from a Q8_0 source: packed is the U32 word segment, scales the F32 (Q8_0F) or F16 (Q8_0H) segment of the
+        reference's quantized buffer, src_shape the logical shape; the result has the scales' dtype."""
+        rank = len(src_shape)
+        out_shape = list(src_shape)
+        out_shape[dim] = indices.numel
+        out = out or Buffer(self, out_shape, scales.dt)
+        check(self.lib.rt_index_select_q8_0(self.handle, scales.dt, packed.ptr, scales.ptr, shape4(src_shape), indices.ptr, indices.numel,
+                                            dim + (4 - rank), out.ptr))
+        return out
+
     def index_write(self, dst, src, write_start):
         """dst is modified in place and returned."""
         pad = 4 - len(dst.shape)

@@ -140,6 +140,15 @@ def test_rope_and_index_validation(lib):
     assert lib.rt_index_select(None, 4, SOME, u4(1, 1, 8, 4), SOME, 0, 2, SOME) == 4
     assert lib.rt_index_select(None, 4, SOME, u4(1, 1, 8, 4), None, 3, 2, SOME) == 1
     assert lib.rt_index_select(None, 1, SOME, u4(1, 1, 8, 4), SOME, 3, 2, SOME) == 7
+    # quantized source: whole groups of 32 elements, runs of whole 4-element words (quant.rs:20-21, ops/select.rs:144-161)
+    assert lib.rt_index_select_q8_0(None, _lib.F32, SOME, SOME, u4(1, 1, 8, 32), SOME, 3, 2, SOME) == 8
+    assert lib.rt_index_select_q8_0(None, _lib.F16, SOME, SOME, u4(1, 1, 8, 32), SOME, 3, 2, SOME) == 8
+    assert lib.rt_index_select_q8_0(None, _lib.BF16, SOME, SOME, u4(1, 1, 8, 32), SOME, 3, 2, SOME) == 2
+    assert lib.rt_index_select_q8_0(None, _lib.F32, SOME, SOME, u4(1, 1, 8, 30), SOME, 3, 2, SOME) == 4    # 240 elements: not whole groups
+    assert lib.rt_index_select_q8_0(None, _lib.F32, SOME, SOME, u4(1, 1, 32, 2), SOME, 3, 2, SOME) == 4    # runs of 2 elements
+    assert lib.rt_index_select_q8_0(None, _lib.F32, SOME, None, u4(1, 1, 8, 32), SOME, 3, 2, SOME) == 1
+    assert lib.rt_index_select_q8_0(None, _lib.F32, SOME, SOME, u4(1, 1, 8, 32), SOME, 0, 2, SOME) == 4
+    assert lib.rt_index_select_q8_0(None, _lib.F32, SOME, SOME, u4(1, 1, 8, 32), SOME, 3, 4, SOME) == 7
     assert lib.rt_index_write(None, 4, SOME, u4(1, 1, 3, 2), SOME, 2, u4(0, 0, 2, 0)) == 8
     assert lib.rt_index_write(None, 4, SOME, u4(1, 1, 3, 2), SOME, 3, u4(0, 0, 2, 0)) == 4   # the run would leave dst
     assert lib.rt_index_write(None, 4, SOME, u4(1, 1, 3, 2), SOME, 1, u4(0, 0, 3, 0)) == 4   # write_start outside dst

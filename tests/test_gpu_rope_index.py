@@ -107,6 +107,37 @@ def test_index_select(dev, oracle, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_index_select_from_q8_0_table(dev, oracle, dtype):
+    """The embedding lookup of a quantized model (ops/select.rs:107-111,144-161): rows of a Q8_0F / Q8_0H table, bit for bit
+    what dequantize-then-index_select gives (cpu/mod.rs:86-103); the packed words and the scales are the two segments of the
+    reference's buffer, the scales starting at the next multiple of 256 bytes (quant.rs:8-17,46)."""
+    rng = np.random.default_rng(607)
+    for shape, dim, idx in [((256, 32), 0, [64, 192, 255]),                      # the reference's test shape (ops/select.rs:350-357)
+                            ((51200 // 8, 2560), 0, rng.integers(0, 51200 // 8, 77)),   # an embedding table, prefill-sized gather
+                            ((3, 50, 64), 1, [49, 0, 7, 7]), ((2, 4, 8, 12), 2, [3, 1])]:
+        table = (rng.standard_normal(shape) * 0.05).astype(dtype)
+        words, scales = oracle.q8_0_quantize(table)
+        # one device buffer laid out as the reference lays it out
+        nq = words.nbytes
+        off = (nq + 255) // 256 * 256
+        raw = np.zeros(off + scales.nbytes, np.uint8)
+        raw[:nq] = words.view(np.uint8)
+        raw[off:] = scales.view(np.uint8)
+        buf = dev.upload(raw.view(np.uint32) if raw.nbytes % 4 == 0 else np.concatenate([raw, np.zeros(4 - raw.nbytes % 4, np.uint8)]).view(np.uint32))
+        from ratchet_amd.runtime import BufferView
+        packed = BufferView(buf, 0, (nq // 4,))
+        sc = BufferView(buf, off // 4, (scales.nbytes // 4 if dtype == np.float32 else (scales.nbytes + 3) // 4,))
+        sc.dt = 0 if dtype == np.float32 else 1
+        ids = np.asarray(idx, np.int32)
+        want = oracle.q8_0_index_select(words, scales, shape, ids, dim)
+        got = dev.index_select_q8_0(packed, sc, shape, dev.upload(ids), dim).to_numpy()
+        assert got.dtype == dtype and same_bits(got, want), (shape, dim)
+    # an index outside the table gives a row of zeros
+    got = dev.index_select_q8_0(packed, sc, shape, dev.upload(np.array([1, 99], np.int32)), dim).to_numpy()
+    assert np.all(got[:, :, 1, :] == 0) and same_bits(got[:, :, 0, :], want[:, :, 1, :])
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
 def test_index_write(dev, oracle, dtype):
     rng = np.random.default_rng(604)
     dst = np.array([1, 2, 3, 4, 5, 6], dtype).reshape(3, 2)     # the reference's own test (ops/index_write.rs:203-224)

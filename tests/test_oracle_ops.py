@@ -459,3 +459,62 @@ def test_index_write_reference_case(oracle):
     assert np.array_equal(d, np.array([[0, 1, 2], [3, 0, 0]], np.float16))
     with pytest.raises(ValueError):
         oracle.index_write(d, np.array([1, 2, 3], np.float16), [1, 1])                      # would leave dst
+
+
+# ---- Q8_0 (crates/ratchet-core/src/quant.rs): pins for the quantized IndexSelect's oracle ---------------------------------------
+def _q8_numpy_dequantize(words, scales, shape):
+    """independent model of dequantize_inner: byte j of word i is element 4 i + j (quant.rs:118-127), times its group's scale"""
+    q = np.ascontiguousarray(words, np.uint32).view(np.int8).astype(scales.dtype)      # little endian: byte 0 first
+    return (q * np.repeat(scales, 32)).reshape(shape)
+
+
+def test_q8_0_dequantize_known_answer_and_numpy_model(oracle):
+    # one group of 32 elements by hand: bytes 0x01, 0xff, 0x80, 0x7f = 1, -1, -128, 127 in the first word
+    words = np.zeros(8, np.uint32)
+    words[0] = 0x7F80FF01
+    words[7] = 0x000000FE                                                                # element 28 = -2
+    for dt in (np.float32, np.float16):
+        got = oracle.q8_0_dequantize(words, np.array([0.5], dt), (32,))
+        assert got.dtype == dt
+        assert got[:4].tolist() == [0.5, -0.5, -64.0, 63.5] and got[28] == -1.0 and np.count_nonzero(got) == 5
+    rng = np.random.default_rng(460)
+    words = rng.integers(0, 2 ** 32, size=64 * 64 // 4, dtype=np.uint64).astype(np.uint32)
+    for dt in (np.float32, np.float16):
+        scales = (rng.random(64 * 64 // 32) * 0.05 + 1e-3).astype(dt)
+        got = oracle.q8_0_dequantize(words, scales, (64, 64))
+        assert np.array_equal(got, _q8_numpy_dequantize(words, scales, (64, 64)))         # f16: numpy rounds the product the same way
+
+
+def test_q8_0_quantize_model_and_reflexivity(oracle):
+    """quantize_inner against a numpy model (scale = max|x| / 127 per 32 elements, round half away from zero), and the reference's
+    own check (quant.rs:171-190): dequantize(quantize(x)) is all_close to x at atol = rtol = 0.1 on randn [64, 64]."""
+    rng = np.random.default_rng(461)
+    x = rng.standard_normal((64, 64)).astype(np.float32)
+    x[3, :32] = 0.0                                                                      # an all-zero group: 0 / 0 -> NaN -> 0
+    words, scales = oracle.q8_0_quantize(x)
+    g = x.reshape(-1, 32)
+    d = (np.abs(g).max(axis=1) / np.float32(127)).astype(np.float32)
+    assert np.array_equal(scales, d)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        r = g / d[:, None]
+    q = np.where(np.isnan(r), 0, np.trunc(r + np.copysign(np.float32(0.5), r))).astype(np.int64) & 0xFF
+    model = (q.reshape(-1, 4) << (8 * np.arange(4))).sum(axis=1).astype(np.uint32)
+    assert np.array_equal(words, model)
+    back = oracle.q8_0_dequantize(words, scales, x.shape)
+    bad, mx = oracle.count_not_close(back, x, 0.1, 0.1)
+    assert bad == 0, mx
+    assert np.abs(back - x).max() <= np.abs(x).max() / 127 / 2 * 1.0001                   # half a quantisation step
+    xh = x.astype(np.float16)
+    wh, sh = oracle.q8_0_quantize(xh)
+    assert sh.dtype == np.float16
+    bad, mx = oracle.count_not_close(oracle.q8_0_dequantize(wh, sh, x.shape), xh, 0.1, 0.1)
+    assert bad == 0, mx
+
+
+def test_q8_0_index_select_is_take_of_the_dequantized_table(oracle):
+    rng = np.random.default_rng(462)
+    table = (rng.standard_normal((96, 64)) * 0.1).astype(np.float32)
+    words, scales = oracle.q8_0_quantize(table)
+    idx = np.array([5, 0, 95, 5], np.int32)
+    got = oracle.q8_0_index_select(words, scales, table.shape, idx, 0)
+    assert np.array_equal(got, np.take(_q8_numpy_dequantize(words, scales, table.shape), idx, axis=0))
