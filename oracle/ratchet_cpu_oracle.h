@@ -1,6 +1,6 @@
 /*
  * TEST INFRASTRUCTURE ONLY - CPU restatement of ratchet-core's CPU executor for the
- * memory-bound tensor ops (binary, unary, cast, reindex, concat, softmax, norms).
+ * memory-bound tensor ops (binary, unary, cast, reindex, concat, softmax, norms, cache, rope, index ops, Q8_0 gather).
  *
  * Nothing in the shipped library links, loads or calls this file.  It exists so the
  * parity tests, the smoke check and the benchmark's CPU leg have an independent answer
@@ -21,6 +21,7 @@
  *   cache, index_select, index_write ..... numpy concatenate / take / flat assignment and the reference's own test cases
  *   rope ................................. float64 closed form of the half-rotation RoPE (what the reference's mlx ground
  *                                          truth computes), rotation invariants, offset additivity
+ *   q8_0 quantize / dequantize ........... hand-made words, a numpy byte-view model, the reference's reflexivity check
  *   PARITY UNPINNED: the accumulation type of `Sum for f16` inside `mean` (assumed: f32
  *   accumulation, one rounding; switchable with orc_set_f16_sum_mode) - the `half` crate is
  *   not present in the reference tree and no reference test exercises the f16 CPU path.
