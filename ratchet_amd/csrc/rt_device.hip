@@ -128,6 +128,14 @@ int rt_device_create(int ordinal, rt_device** out) {
         delete dev;
         return rt_fail_hip(e, "hipMalloc(scratch)");
     }
+    e = hipMalloc((void**)&dev->sm_row_sums, RT_SM_ROW_SUMS * sizeof(uint16_t));
+    if (e != hipSuccess) {
+        (void)hipFree(dev->gn_scratch);
+        (void)hipStreamDestroy(dev->stream);
+        delete dev->pool;
+        delete dev;
+        return rt_fail_hip(e, "hipMalloc(row sums)");
+    }
     *out = dev;
     return RT_OK;
 }
@@ -144,6 +152,7 @@ int rt_device_destroy(rt_device* dev) {
             if (dev->unary_lut_via32[t][i]) (void)hipFree(dev->unary_lut_via32[t][i]);
         }
     if (dev->gn_scratch) (void)hipFree(dev->gn_scratch);
+    if (dev->sm_row_sums) (void)hipFree(dev->sm_row_sums);
     // buffers the caller never returned are released with the device, like the parked ones
     for (auto& kv : dev->pool->parked) (void)hipFree(kv.second);
     for (auto& kv : dev->pool->live) (void)hipFree(kv.first);

@@ -8,6 +8,8 @@
 
 #include "../../include/ratchet_hip.h"
 
+constexpr size_t RT_SM_ROW_SUMS = 1u << 19;
+
 struct rt_device {
     int ordinal;
     hipStream_t stream;
@@ -23,6 +25,8 @@ struct rt_device {
     int gated_attr_set[2];
     unsigned gn_lds_attr_set;
     uint64_t sp_attr_set;   // streaming softmax instantiations whose dynamic-LDS limit has been raised on this device
+    // row sums of one launch of the streaming softmax's ragged-row variant (RT_SM_ROW_SUMS 16-bit values, allocated with the device)
+    uint16_t* sm_row_sums;
     // caching allocator behind rt_malloc / rt_free (defined in rt_device.hip)
     struct rt_pool* pool;
     int capturing;          // between rt_capture_begin and rt_capture_end

@@ -310,6 +310,7 @@ template <typename T> int launch_lane16(rt_device* dev, const void* x, void* y, 
 // Global loads run SP_PF steps ahead across group boundaries, so the pipeline never drains.
 // ------------------------------------------------------------------------------------------------------------------
 constexpr int SP_BLOCK = 1024;
+constexpr uint32_t RAGGED_STREAM_MIN_COLS = 192;   // shorter ragged rows: the two-pass tile walker is faster
 constexpr int SP_ROWS = 30;                  // 15 loader waves x 2 rows each; wave 0 only walks
 constexpr int SP_HALF = SP_ROWS / 2;
 constexpr int SP_TC = 512;                   // columns per step: 64 lanes x 8 halves
@@ -401,11 +402,20 @@ template <> struct SpType<bf16_t> {
 // NSTEP > 0: rows of up to NSTEP * 512 columns, exp values parked in registers.  NSTEP == 0: longer rows; the exp values
 // are parked in y instead and read back (by the thread that wrote them) when the row sum is known: 4 bytes of traffic per
 // element and byte of the type instead of 2, any row length.
-template <typename T, int NSTEP, bool FULL, bool MASK>
+//
+// RAGGED (rows that are not whole aligned vectors, e.g. 1001 columns; x and y 16-byte aligned, no mask, parked variant):
+// every row is handled over the span of aligned 16-byte vectors that covers it.  Row r starts `sh` = (r * cols * 2) % 16
+// bytes into its first vector; span elements outside the row belong to the neighbouring rows: they are zeroed after the
+// table lookup (adding +0 leaves the running sum as it is), and a vector that is not entirely inside its row is not
+// stored.  Wave 0 also writes each row's sum to `row_sums`; the elements of those ragged vectors (at most 14 per row) are
+// finished by softmax16_edges_kernel from x, the table and that sum.  An aligned vector that holds one byte of the tensor
+// lies in a mapped page, so the loads are safe at the tensor's ends too.
+template <typename T, int NSTEP, bool FULL, bool MASK, bool RAGGED = false>
 __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16_t* __restrict__ table, const T* x, const T* mask, T* y,
-                                                                    uint64_t rows, uint32_t cols, SpSched sch) {
+                                                                    uint64_t rows, uint32_t cols, SpSched sch, uint16_t* row_sums) {
     typedef SpType<T> ST;
     constexpr bool PARK = NSTEP > 0;
+    static_assert(!RAGGED || (PARK && !FULL && !MASK), "the ragged variant parks in registers, has no full-step shortcut and no mask");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint16_t* lut = reinterpret_cast<uint16_t*>(smem);
     uint16_t (*tile)[SP_TC + SP_PAD] = reinterpret_cast<uint16_t (*)[SP_TC + SP_PAD]>(smem + SP_LUT_BYTES);
@@ -455,6 +465,12 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                 }
             }
             if (lane < SP_ROWS) sums[gpar][lane] = ST::run_bits(run);
+            if (RAGGED) {
+                uint32_t rep, pg;
+                sp_item(sch, blockIdx.x, gridDim.x, it, rep, pg);
+                const uint32_t prow = pg * sch.R + lane;
+                if (lane < sch.R && prow < sch.P) row_sums[rep * sch.P + prow] = ST::run_bits(run);
+            }
             run = ST::zero();
             gpar ^= 1;
         }
@@ -472,7 +488,8 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
     const uint32_t rr = __builtin_amdgcn_readfirstlane(lt >> 6);   // rows rr and rr + 15 of the group: the same for the whole wave
     const uint32_t ccol = (lt & 63) * 8;                     // column of this thread's vectors inside a step
     const uint32_t row_bytes = cols * 2;
-    const uint32_t nbytes = (uint32_t)(rows * row_bytes);    // the launcher keeps this below 2^31
+    // the launcher keeps this below 2^31; the ragged variant's last vector may reach past the tensor's last element
+    const uint32_t nbytes = RAGGED ? (uint32_t)((rows * row_bytes + 15) & ~15ull) : (uint32_t)(rows * row_bytes);
     const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(x), 0, nbytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(y, 0, nbytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t rm =
@@ -484,6 +501,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
     // needed for data): byte offset of rows rr / rr + 15 of item `it` in x / y, or OOB, and the difference between that
     // and the row's offset in the mask (for a row that does not exist the mask offset is arbitrary, which is harmless:
     // the load is range checked, and what is computed from it is never stored).
+    // (RAGGED: xo is the offset of the row's first span vector and mdiff carries sh, the row's start inside that vector)
     auto item_off = [&](uint32_t it, uint32_t (&xo)[2], uint32_t (&mdiff)[2]) {
         uint32_t rep, pg;
         sp_item(sch, blockIdx.x, G, it, rep, pg);
@@ -493,6 +511,11 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
             const uint32_t prow = pg * sch.R + r;            // row inside the period
             const bool ok = it < n_items && r < sch.R && prow < sch.P;
             const uint32_t row = rep * sch.P + prow;
+            if (RAGGED) {
+                xo[h] = __builtin_amdgcn_readfirstlane(ok ? (row * row_bytes) & ~15u : OOB);
+                mdiff[h] = __builtin_amdgcn_readfirstlane((row * row_bytes) & 15u);
+                continue;
+            }
             xo[h] = __builtin_amdgcn_readfirstlane(ok ? row * row_bytes : OOB);
             if (MASK) {
                 uint32_t q, mrow;
@@ -509,6 +532,17 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
         if (past_end(t)) return OOB;
         return row_off + t * (SP_TC * 2) + cbyte;
     };
+    // RAGGED: the same in span coordinates.  The vector at span byte p holds row bytes [sh, sh + row_bytes) ∩ [p, p + 16).
+    auto span_load_off = [&](uint32_t row_off, uint32_t sh, uint32_t t) -> uint32_t {
+        const uint32_t p = t * (SP_TC * 2) + cbyte;
+        return p >= sh + row_bytes ? OOB : row_off + p;
+    };
+    auto span_store_off = [&](uint32_t row_off, uint32_t sh, uint32_t t) -> uint32_t {     // only vectors entirely inside the row
+        const uint32_t p = t * (SP_TC * 2) + cbyte;
+        return (p >= sh && p + 16 <= sh + row_bytes) ? row_off + p : OOB;
+    };
+    auto ld_off = [&](uint32_t row_off, uint32_t sh, uint32_t t) -> uint32_t { return RAGGED ? span_load_off(row_off, sh, t) : step_off(row_off, t); };
+    auto st_off = [&](uint32_t row_off, uint32_t sh, uint32_t t) -> uint32_t { return RAGGED ? span_store_off(row_off, sh, t) : step_off(row_off, t); };
     auto load_x = [&](uint32_t off) -> v4u { return __builtin_amdgcn_raw_buffer_load_b128(rx, off, 0, 2); };   // 2: non-temporal
     auto load_m = [&](uint32_t off) -> v4u { return __builtin_amdgcn_raw_buffer_load_b128(rm, off, 0, 0); };   // re-read by other heads
     auto load_y = [&](uint32_t off) -> v4u { return __builtin_amdgcn_raw_buffer_load_b128(ry, off, 0, 0); };
@@ -557,14 +591,27 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
     };
     // exp of the vector that arrived, in place (zeros past the row end: adding +0 is a no-op; rows past the tensor's end
     // read zeros and their sums are never used)
-    auto exp_in_place = [&](v4u& in, const v4u& m, uint32_t t) {
+    auto exp_in_place = [&](v4u& in, const v4u& m, uint32_t t, uint32_t sh) {
         if (MASK) in = ST::add_vec(in, m);                   // scores + mask in the 16-bit type, as the separate add would round it
 #pragma unroll
         for (int w = 0; w < 4; w++) in[w] = sp_exp_pair(lut, in[w]);
-        if (past_end(t)) in = v4u{0, 0, 0, 0};
+        if (RAGGED) {
+            const uint32_t p = t * (SP_TC * 2) + cbyte, end = sh + row_bytes;
+            if (p >= end) {
+                in = v4u{0, 0, 0, 0};
+            } else if (p < sh || p + 16 > end) {             // one of the row's two ragged vectors: a few lanes per row
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    const uint32_t b0 = p + 4 * w, b1 = b0 + 2;
+                    in[w] &= ((b0 >= sh && b0 < end) ? 0xffffu : 0u) | ((b1 >= sh && b1 < end) ? 0xffff0000u : 0u);
+                }
+            }
+        } else if (past_end(t)) {
+            in = v4u{0, 0, 0, 0};
+        }
     };
 
-    uint32_t cur[2], nxt[2], prev[2] = {OOB, OOB}, pcur[2], pnxt[2];
+    uint32_t cur[2], nxt[2], prev[2] = {OOB, OOB}, pcur[2], pnxt[2], pprev[2] = {0, 0};
     item_off(0, cur, pcur);
     item_off(1, nxt, pnxt);
     uint32_t gpar = 0;
@@ -580,7 +627,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
 #pragma unroll
         for (int k = 0; k < PF; k++) {
 #pragma unroll
-            for (int h = 0; h < 2; h++) pre[k][h] = load_x(step_off(cur[h], k));
+            for (int h = 0; h < 2; h++) pre[k][h] = load_x(ld_off(cur[h], pcur[h], k));
 #pragma unroll
             for (int h = 0; h < 2; h++) store_y(v4u{0, 0, 0, 0}, OOB);
         }
@@ -593,7 +640,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
 #pragma unroll
             for (int t = 0; t < NSTEP; t++) {
 #pragma unroll
-                for (int h = 0; h < 2; h++) exp_in_place(pre[t % PF][h], mpre[h], t);
+                for (int h = 0; h < 2; h++) exp_in_place(pre[t % PF][h], mpre[h], t, pcur[h]);
                 __syncthreads();                             // A: wave 0 has left the previous tile
                 *reinterpret_cast<v4u*>(&tile[rr][ccol]) = pre[t % PF][0];
                 *reinterpret_cast<v4u*>(&tile[rr + SP_HALF][ccol]) = pre[t % PF][1];
@@ -607,12 +654,12 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                 }
 #pragma unroll
                 for (int h = 0; h < 2; h++)
-                    pre[t % PF][h] = (t + PF < NSTEP) ? load_x(step_off(cur[h], t + PF)) : load_x(step_off(nxt[h], t + PF - NSTEP));
+                    pre[t % PF][h] = (t + PF < NSTEP) ? load_x(ld_off(cur[h], pcur[h], t + PF)) : load_x(ld_off(nxt[h], pnxt[h], t + PF - NSTEP));
                 __syncthreads();                             // B: parked for the walk
                 if (t == 0) read_prev_sum(gpar ^ 1);         // published by wave 0 before it reached barrier A
 #pragma unroll
                 for (int h = 0; h < 2; h++) {
-                    store_y(quotients(e[t][h], h), step_off(prev[h], t));   // first group: prev is OOB, the store is dropped
+                    store_y(quotients(e[t][h], h), st_off(prev[h], pprev[h], t));   // first group: prev is OOB, the store is dropped
                     // this group's values come back from the tile, which stays intact until the next barrier A
                     e[t][h] = *reinterpret_cast<const v4u*>(&tile[rr + h * SP_HALF][ccol]);
                 }
@@ -622,8 +669,11 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                 prev[h] = cur[h];
                 cur[h] = nxt[h];
             }
-            pcur[0] = pnxt[0];
-            pcur[1] = pnxt[1];
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                pprev[h] = pcur[h];
+                pcur[h] = pnxt[h];
+            }
             item_off(it + 2, nxt, pnxt);
             gpar ^= 1;
         }
@@ -633,7 +683,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
 #pragma unroll
         for (int t = 0; t < NSTEP; t++)
 #pragma unroll
-            for (int h = 0; h < 2; h++) store_y(quotients(e[t][h], h), step_off(prev[h], t));
+            for (int h = 0; h < 2; h++) store_y(quotients(e[t][h], h), st_off(prev[h], pprev[h], t));
     } else {
         // One flat loop over the steps of all groups, two steps per trip (nsteps is even; a step past the row end moves
         // nothing).  Per step and row: exp values to the tile and to y, x of two steps ahead, the previous group's exp
@@ -662,7 +712,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
             for (int k = 0; k < 2; k++) {
                 const uint32_t t = t0 + k;
 #pragma unroll
-                for (int h = 0; h < 2; h++) exp_in_place(pre[k][h], mpre[h], t);
+                for (int h = 0; h < 2; h++) exp_in_place(pre[k][h], mpre[h], t, 0);
                 __syncthreads();                             // A
                 *reinterpret_cast<v4u*>(&tile[rr][ccol]) = pre[k][0];
                 *reinterpret_cast<v4u*>(&tile[rr + SP_HALF][ccol]) = pre[k][1];
@@ -1061,18 +1111,52 @@ template <typename T, int MODE> int launch_f32_style(rt_device* dev, const void*
 
 // mask == nullptr: plain softmax.  Otherwise the mask has `period` rows of `cols` columns and repeats every `period`
 // rows of x (rows % period == 0).  Returns RT_OK with *done = false when the shape does not fit this kernel.
+// The ragged-row variant's second launch: the elements of a row's first and last span vectors when those vectors are
+// shared with a neighbouring row (at most 7 + 7 per row), from x, the exp table and the row sum the streaming kernel
+// left in row_sums.  Sixteen threads per row: 0..7 the elements of the first span vector, 8..15 those of the last.
+// The quotient is the IEEE division the streaming kernel's short division reproduces.
+template <typename T>
+__global__ void __launch_bounds__(BLOCK) softmax16_edges_kernel(const uint16_t* __restrict__ table, const T* x, T* y,
+                                                                const uint16_t* __restrict__ row_sums, uint64_t rows, uint32_t cols) {
+    const uint64_t gid = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+    const uint64_t row = gid >> 4;
+    if (row >= rows) return;
+    const uint32_t j = (uint32_t)gid & 7u;
+    const bool tail = (gid & 8u) != 0;
+    const uint64_t first = row * cols;
+    const uint32_t shift = (uint32_t)(first & 7);
+    const uint32_t last_vec = (shift + cols - 1) >> 3;       // index of the row's last span vector
+    const bool first_whole = shift == 0 && cols >= 8;
+    const bool last_whole = ((shift + cols) & 7) == 0 && (last_vec > 0 || shift == 0);
+    if (tail ? (last_vec == 0 || last_whole) : first_whole) return;
+    const uint32_t e = (tail ? last_vec * 8 : 0) + j;        // element of the span
+    if (e < shift || e - shift >= cols) return;
+    const uint64_t at = first + (e - shift);
+    const uint16_t xb = __builtin_bit_cast(uint16_t, x[at]);
+    const T ev = __builtin_bit_cast(T, table[xb]);
+    y[at] = Ar<T>::div(ev, __builtin_bit_cast(T, row_sums[row]));
+}
+
 template <typename T>
 int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t period, void* y, uint64_t rows, uint32_t cols, bool* done) {
     *done = false;
     constexpr int TI = sizeof(typename SpType<T>::Run) == 4 ? 1 : 0;         // table and attribute index: 0 f16, 1 bf16
     const uint64_t row_bytes = (uint64_t)cols * 2;
     if (!mask) period = rows;
+    const bool ragged = cols % 8 != 0;                       // rows over their covering aligned vectors, finished by the edges kernel
+    if (ragged && mask) return RT_OK;
     // the kernel addresses a launch with 32-bit byte offsets below 2^31: larger tensors go in chunks of whole periods
     // (whole 30-row groups when nothing repeats)
     uint64_t chunk_rows;
     if (mask) {
         if (period * row_bytes > 0x7fffffffull) return RT_OK;
         chunk_rows = (0x7fffffffull / (period * row_bytes)) * period;
+    } else if (ragged) {
+        // a chunk's row sums must fit the device's buffer, and every chunk must start on a 16-byte boundary (8 rows do)
+        uint64_t max_rows = 0x7fffffe0ull / row_bytes;
+        if (max_rows > RT_SM_ROW_SUMS) max_rows = RT_SM_ROW_SUMS;
+        chunk_rows = rows <= max_rows ? rows : max_rows / 120 * 120;
+        if (chunk_rows == 0) return RT_OK;
     } else {
         chunk_rows = (0x7fffffffull / row_bytes) / SP_ROWS * SP_ROWS;
         if (chunk_rows == 0) return RT_OK;
@@ -1080,8 +1164,9 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
     const uint16_t* table = nullptr;
     int rc = rt_unary_table(dev, TI, RT_EXP, &table);
     if (rc) return rc;
-    const uint32_t nt = (cols + SP_TC - 1) / SP_TC;
-    const bool full = cols % SP_TC == 0 && (nt == 1 || nt == 2 || nt == 4 || nt == 8);
+    const uint32_t nt = (cols + (ragged ? 7 : 0) + SP_TC - 1) / SP_TC;       // a ragged row's span is up to 7 elements longer
+    if (ragged && nt > SP_MAX_STEPS) return RT_OK;
+    const bool full = !ragged && cols % SP_TC == 0 && (nt == 1 || nt == 2 || nt == 4 || nt == 8);
 #define RT_SP(NS, F, M)                                                                                                              \
     do {                                                                                                                             \
         const uint64_t bit = 1ull << (TI * 20 + (NS == 0 ? 4 : NS == 1 ? 0 : NS == 2 ? 1 : NS == 4 ? 2 : 3) * 4 + (F ? 2 : 0) + (M ? 1 : 0)); \
@@ -1091,7 +1176,18 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
             dev->sp_attr_set |= bit;                                                                                                 \
         }                                                                                                                            \
         hipLaunchKernelGGL((softmax16_stream_kernel<T, NS, F, M>), dim3(blocks), dim3(SP_BLOCK), SP_SMEM_BYTES, dev->stream, table,  \
-                           xc, (const T*)mask, yc, n, cols, sch);                                                                    \
+                           xc, (const T*)mask, yc, n, cols, sch, (uint16_t*)nullptr);                                                \
+    } while (0)
+#define RT_SP_RAGGED(NS)                                                                                                             \
+    do {                                                                                                                             \
+        const uint64_t bit = 1ull << (40 + TI * 4 + (NS == 1 ? 0 : NS == 2 ? 1 : NS == 4 ? 2 : 3));                                  \
+        if (!(dev->sp_attr_set & bit)) {                                                                                             \
+            RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(softmax16_stream_kernel<T, NS, false, false, true>),            \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)SP_SMEM_BYTES));                             \
+            dev->sp_attr_set |= bit;                                                                                                 \
+        }                                                                                                                            \
+        hipLaunchKernelGGL((softmax16_stream_kernel<T, NS, false, false, true>), dim3(blocks), dim3(SP_BLOCK), SP_SMEM_BYTES,        \
+                           dev->stream, table, xc, (const T*)nullptr, yc, n, cols, sch, dev->sm_row_sums);                           \
     } while (0)
 #define RT_SP_NS(F, M)                                      \
     do {                                                    \
@@ -1135,6 +1231,18 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
         const uint64_t items = (uint64_t)sch.GP * sch.reps;
         RT_REQUIRE(items <= 0xffffffffull, RT_ERR_SIZE, "rt_softmax: too many row groups");
         const unsigned blocks = (unsigned)(items < (uint64_t)dev->num_cus ? items : (uint64_t)dev->num_cus);   // one resident block per CU
+        if (ragged) {
+            if (nt <= 1) RT_SP_RAGGED(1);
+            else if (nt <= 2) RT_SP_RAGGED(2);
+            else if (nt <= 4) RT_SP_RAGGED(4);
+            else RT_SP_RAGGED(8);
+            RT_CHECK_LAUNCH("softmax16_stream_kernel");
+            const uint64_t eblocks = (n * 16 + BLOCK - 1) / BLOCK;
+            hipLaunchKernelGGL((softmax16_edges_kernel<T>), dim3((unsigned)eblocks), dim3(BLOCK), 0, dev->stream, table, xc, yc,
+                               (const uint16_t*)dev->sm_row_sums, n, cols);
+            RT_CHECK_LAUNCH("softmax16_edges_kernel");
+            continue;
+        }
         if (nt > SP_MAX_STEPS) {                         // long rows: exp values parked in y
             if (mask) RT_SP(0, false, true);
             else RT_SP(0, false, false);
@@ -1148,6 +1256,7 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
         RT_CHECK_LAUNCH("softmax16_stream_kernel");
     }
 #undef RT_SP_NS
+#undef RT_SP_RAGGED
 #undef RT_SP
     *done = true;
     return RT_OK;
@@ -1345,8 +1454,10 @@ extern "C" int rt_softmax(rt_device* dev, int dt, const void* x, void* y, uint64
             // 16-bit types, rows that are whole aligned vectors: one pass; up to 128 columns (and enough rows to fill the chip) a lane per row, up to 4096
             // columns streamed with the row held in registers, longer ones parked in y (also small problems: the per-block table load costs about 5 us, the two-pass walker
             // more); everything else takes the two-pass tile walker
-            if (cols % 8 == 0 && rt_aligned(x, 16) && rt_aligned(y, 16)) {
-                if (cols <= LANE_MAX_COLS && rows >= 32768) return dt == RT_F16 ? launch_lane16<half_t>(dev, x, y, rows, cols) : launch_lane16<bf16_t>(dev, x, y, rows, cols);
+            // (rows that are not whole vectors stream over their covering vectors, with a second small launch for the
+            // shared ones: measured faster than the tile walker from about 200 columns, 12.7 against 34.5 us on [4096, 1001])
+            if (rt_aligned(x, 16) && rt_aligned(y, 16) && (cols % 8 == 0 || cols >= RAGGED_STREAM_MIN_COLS)) {
+                if (cols % 8 == 0 && cols <= LANE_MAX_COLS && rows >= 32768) return dt == RT_F16 ? launch_lane16<half_t>(dev, x, y, rows, cols) : launch_lane16<bf16_t>(dev, x, y, rows, cols);
                 bool done = false;
                 rc = dt == RT_F16 ? launch_stream16<half_t>(dev, x, nullptr, 0, y, rows, cols, &done)
                                   : launch_stream16<bf16_t>(dev, x, nullptr, 0, y, rows, cols, &done);

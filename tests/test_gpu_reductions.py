@@ -178,6 +178,59 @@ def test_softmax_16_bit_long_rows(dev, oracle, shape, kind):
         assert not ((got != want) & ~(isnan(got) & isnan(want))).any(), shape
 
 
+@pytest.mark.parametrize("shape,kind", [((2, 4, 333, 1001), "f16"), ((1, 3, 100, 199), "f16"), ((70, 4089), "f16"), ((7, 4090), "f16"), ((33, 513), "f16"),
+                                        ((1000, 193), "f16"), ((61, 2561), "f16"), ((2, 2, 77, 1001), "bf16"), ((40, 3001), "bf16"), ((900, 250), "bf16")])
+def test_softmax_16_bit_ragged_rows_stream(dev, oracle, shape, kind):
+    """rows of 192 or more columns that are not whole 16-byte vectors (a prompt of 1001 tokens): streamed over the aligned
+    vectors that cover each row, the vectors shared by two rows finished by a second small launch; bit-exact like the
+    aligned rows, out of place and in place.  4089 columns fill the largest register-parked variant, 4090 are past it."""
+    from ratchet_amd.runtime import BufferView
+
+    rng = np.random.default_rng(308)
+    n = shape[-1]
+    xf = (rng.standard_normal(shape) * 2).astype(np.float32)
+    flat = xf.reshape(-1, n)
+    if flat.shape[0] >= 20:
+        _special_rows(flat, n)
+    flat[0, n // 3:] = -np.inf
+    flat[-1, :] = 95.0 if kind == "bf16" else 12.0                   # the last row overflows its sum
+    flat[1, :7] = 11.0                                                # large terms in a row's first (shared) vector
+    flat[2, -7:] = 11.0                                               # and in its last
+    bf = kind == "bf16"
+    x = _bf16(oracle, xf) if bf else xf.astype(np.float16)
+    want = oracle.softmax(x, bf16=bf)
+    isnan = (lambda b: (b & 0x7fff) > 0x7f80) if bf else (lambda b: (b.view(np.uint16) & 0x7fff) > 0x7c00)
+    same = lambda g: not ((g.view(np.uint16) != want.view(np.uint16)) & ~(isnan(g) & isnan(want))).any()
+    dx = dev.upload(x, bf16=bf)
+    assert same(dev.softmax(dx).to_numpy()), shape
+    # into the middle of a larger allocation: the elements next to the first and the last row stay as they were
+    fill = np.full(x.size + 24, 0x1234, np.uint16)
+    big = dev.upload(fill if bf else fill.view(np.float16), bf16=bf)
+    out = BufferView(big, 8, x.shape)
+    dev.softmax(dx, out=out)
+    assert same(out.to_numpy()), shape
+    whole = big.to_numpy().view(np.uint16)
+    assert (whole[:8] == 0x1234).all() and (whole[8 + x.size:] == 0x1234).all()
+    dev.softmax(dx, out=dx)
+    assert same(dx.to_numpy()), shape
+
+
+def test_softmax_f16_ragged_rows_many_rows_in_chunks(dev, oracle):
+    """more rows than one launch of the ragged variant keeps sums for (2^19): the launches split on 16-byte boundaries"""
+    from ratchet_amd.runtime import BufferView
+
+    rng = np.random.default_rng(309)
+    rows, cols = (1 << 19) + 4321, 193
+    x = (rng.standard_normal((rows, cols)) * 2).astype(np.float16)
+    want = oracle.softmax(x)
+    big = dev.empty((rows * cols + 24,), 1)
+    xv = BufferView(big, 8, (rows, cols)).upload(x)                    # 16 bytes into the allocation: still vector aligned
+    got = dev.softmax(xv).to_numpy()
+    assert mismatch_count(got, want) == 0, describe_mismatch(got, want, x)
+    xo = BufferView(big, 3, (1000, cols)).upload(x[:1000])             # off the vector alignment: the tile walker, same results
+    assert same_bits(dev.softmax(xo).to_numpy(), want[:1000])
+
+
 @pytest.mark.parametrize("rows,cols,kind", [(40000, 8, "f16"), (33001, 72, "f16"), (32768 + 5, 128, "f16"), (50000, 24, "bf16"), (32800, 104, "bf16")])
 def test_softmax_16_bit_many_narrow_rows(dev, oracle, rows, cols, kind):
     """tens of thousands of rows of at most 128 columns: the kernel with one lane per row; also in place"""
