@@ -24,20 +24,28 @@ template <typename T> __device__ __forceinline__ float stable_exp(float v) { ret
 // ------------------------------------------------------------------------------------------------------------------
 // Row held in registers by the LANES threads that share it: a wave64 (four rows per block) for rows of up to 512
 // vectors, the whole 256-thread block for rows of up to 2048 vectors (8192 f32 / 16384 16-bit columns).
-// Requires cols % VE == 0, 16-byte aligned rows, cols / VE <= LANES * NV.
+// Requires 16-byte aligned x and y and at most LANES * NV vectors per row; rows of whole vectors, or (SPAN) any length.
 // MODE 0: reference arithmetic for f32 (exp, tree sum, divide).  MODE 1: stable (max subtraction, f32 accumulate) for
 // any T; results are rounded to T once.
 // ------------------------------------------------------------------------------------------------------------------
-template <typename T, int NV, int MODE, int LANES>
-__global__ void __launch_bounds__(BLOCK) softmax_wave_kernel(const T* __restrict__ x, T* __restrict__ y, uint64_t rows,
-                                                             uint32_t cols) {
+template <typename T, int NV, int MODE, int LANES, bool SPAN>
+__global__ void __launch_bounds__(BLOCK) softmax_wave_kernel(const T* x, T* y, uint64_t rows, uint32_t cols) {
     constexpr int VE = 16 / sizeof(T);
     const uint64_t row = (uint64_t)blockIdx.x * (BLOCK / LANES) + (threadIdx.x / LANES);
     if (row >= rows) return;
     const int lane = threadIdx.x & (LANES - 1);
-    const uint32_t nvec = cols / VE;
-    const v4u* xr = reinterpret_cast<const v4u*>(x + row * cols);
-    v4u* yr = reinterpret_cast<v4u*>(y + row * cols);
+    // SPAN (rows that are not whole aligned vectors; x and y 16-byte aligned): the row is handled over the aligned vectors
+    // that cover it.  It starts `shift` elements into the first one; span elements outside the row belong to the
+    // neighbouring rows, are left out of the sums and are not written (the row's two ragged vectors are stored element
+    // by element).  An aligned vector that holds one byte of the tensor lies in a mapped page, so the loads are safe
+    // at the tensor's ends too.
+    const uint64_t first = row * cols;
+    const uint32_t shift = SPAN ? (uint32_t)(first & (VE - 1)) : 0;
+    const uint32_t nvec = SPAN ? (shift + cols + VE - 1) / VE : cols / VE;
+    const v4u* xr = reinterpret_cast<const v4u*>(x) + first / VE;
+    v4u* yr = reinterpret_cast<v4u*>(y) + first / VE;
+    // column of element q of vector i, valid when below cols (elements before the row wrap around)
+    auto inside = [&](uint32_t i, int q) -> bool { return !SPAN || i * VE + (uint32_t)q - shift < cols; };
     Vec16<T> v[NV];
 #pragma unroll
     for (int k = 0; k < NV; k++) {
@@ -45,58 +53,49 @@ __global__ void __launch_bounds__(BLOCK) softmax_wave_kernel(const T* __restrict
         if (i < nvec) v[k].u = ld_stream(xr + i);
     }
     float e[NV][VE];
+    float m = 0.0f;
     if (MODE == 1) {
-        float m = -__builtin_huge_valf();
+        m = -__builtin_huge_valf();
 #pragma unroll
         for (int k = 0; k < NV; k++)
             if (lane + k * LANES < nvec)
 #pragma unroll
-                for (int q = 0; q < VE; q++) m = fmaxf(m, Ar<T>::widen(v[k].e[q]));
+                for (int q = 0; q < VE; q++)
+                    if (inside(lane + k * LANES, q)) m = fmaxf(m, Ar<T>::widen(v[k].e[q]));
         m = row_max<LANES>(m);
         if (m == -__builtin_huge_valf()) m = 0.0f;           // fully masked row: exp(-inf - 0) = 0, 0/0 = NaN as torch does
-        float s = 0.0f;
+    }
+    float s = 0.0f;
 #pragma unroll
-        for (int k = 0; k < NV; k++)
-            if (lane + k * LANES < nvec)
+    for (int k = 0; k < NV; k++)
+        if (lane + k * LANES < nvec)
 #pragma unroll
-                for (int q = 0; q < VE; q++) {
-                    e[k][q] = expf(Ar<T>::widen(v[k].e[q]) - m);
+            for (int q = 0; q < VE; q++) {
+                e[k][q] = 0.0f;
+                if (inside(lane + k * LANES, q)) {
+                    e[k][q] = (MODE == 1) ? expf(Ar<T>::widen(v[k].e[q]) - m) : expf(Ar<T>::widen(v[k].e[q]));
                     s += e[k][q];
                 }
-        s = row_sum<LANES>(s);
-#pragma unroll
-        for (int k = 0; k < NV; k++) {
-            const uint32_t i = lane + k * LANES;
-            if (i < nvec) {
-                Vec16<T> o;
-#pragma unroll
-                for (int q = 0; q < VE; q++) o.e[q] = Ar<T>::conv(e[k][q] / s);
-                st_stream(yr + i, o.u);
             }
-        }
-    } else {
-        float s = 0.0f;
+    s = row_sum<LANES>(s);
+    // MODE 0: e / s as e * (1/s): one correctly rounded reciprocal per row, at most 1 ulp from the quotient (bar: 1e-5).
+    // A zero, subnormal, inf or NaN sum keeps the division so that 0/0, x/inf and inf/inf come out as the reference's do.
+    const bool plain = MODE == 0 && (s >= 1.17549435e-38f) && (s < __builtin_huge_valf());
+    const float rs = 1.0f / s;
 #pragma unroll
-        for (int k = 0; k < NV; k++)
-            if (lane + k * LANES < nvec)
+    for (int k = 0; k < NV; k++) {
+        const uint32_t i = lane + k * LANES;
+        if (i < nvec) {
+            Vec16<T> o;
 #pragma unroll
-                for (int q = 0; q < VE; q++) {
-                    e[k][q] = expf(Ar<T>::widen(v[k].e[q]));
-                    s += e[k][q];
-                }
-        s = row_sum<LANES>(s);
-        // e / s as e * (1/s): one correctly rounded reciprocal per row, at most 1 ulp from the quotient (bar: 1e-5).
-        // A zero, subnormal, inf or NaN sum keeps the division so that 0/0, x/inf and inf/inf come out as the reference's do.
-        const bool plain = (s >= 1.17549435e-38f) && (s < __builtin_huge_valf());
-        const float rs = 1.0f / s;
-#pragma unroll
-        for (int k = 0; k < NV; k++) {
-            const uint32_t i = lane + k * LANES;
-            if (i < nvec) {
-                Vec16<T> o;
-#pragma unroll
-                for (int q = 0; q < VE; q++) o.e[q] = Ar<T>::conv(plain ? e[k][q] * rs : e[k][q] / s);
+            for (int q = 0; q < VE; q++) o.e[q] = Ar<T>::conv(plain ? e[k][q] * rs : e[k][q] / s);
+            if (!SPAN || (inside(i, 0) && inside(i, VE - 1))) {
                 st_stream(yr + i, o.u);
+            } else {
+                T* yrow = y + first;
+#pragma unroll
+                for (int q = 0; q < VE; q++)
+                    if (inside(i, q)) yrow[i * VE + (uint32_t)q - shift] = o.e[q];
             }
         }
     }
@@ -1050,9 +1049,9 @@ __global__ void __launch_bounds__(BLOCK) softmax_via32_generic_kernel(const T* _
     for (uint32_t j = threadIdx.x; j < cols; j += BLOCK) yr[j] = Ar<T>::conv(expf(elem(j) - m) / s);
 }
 
-template <typename T, int MODE> int launch_wave(rt_device* dev, const void* x, void* y, uint64_t rows, uint32_t cols) {
+template <typename T, int MODE, bool SPAN> int launch_wave(rt_device* dev, const void* x, void* y, uint64_t rows, uint32_t cols) {
     constexpr int VE = 16 / sizeof(T);
-    const uint32_t nvec = cols / VE;
+    const uint32_t nvec = SPAN ? (cols + 2 * VE - 2) / VE : cols / VE;       // SPAN: the most vectors a row can touch
     if (nvec <= 32) {
         // rows of at most 32 vectors: a group of 2..32 lanes per row (one vector each), so that a wave carries 2..32 rows
         // and as many bytes as with long rows
@@ -1060,7 +1059,7 @@ template <typename T, int MODE> int launch_wave(rt_device* dev, const void* x, v
         const uint64_t blocks = (rows + BLOCK / lanes - 1) / (BLOCK / lanes);
         RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax: too many rows");
         const dim3 grid((unsigned)blocks), block(BLOCK);
-#define RT_NARROW(L) hipLaunchKernelGGL((softmax_wave_kernel<T, 1, MODE, L>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols)
+#define RT_NARROW(L) hipLaunchKernelGGL((softmax_wave_kernel<T, 1, MODE, L, SPAN>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols)
         if (lanes == 2) RT_NARROW(2);
         else if (lanes == 4) RT_NARROW(4);
         else if (lanes == 8) RT_NARROW(8);
@@ -1075,7 +1074,7 @@ template <typename T, int MODE> int launch_wave(rt_device* dev, const void* x, v
         const uint64_t blocks = (rows + WAVES - 1) / WAVES;
         RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax: too many rows");
         const dim3 grid((unsigned)blocks), block(BLOCK);
-#define RT_SM(NVC) hipLaunchKernelGGL((softmax_wave_kernel<T, NVC, MODE, WAVE>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols)
+#define RT_SM(NVC) hipLaunchKernelGGL((softmax_wave_kernel<T, NVC, MODE, WAVE, SPAN>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols)
         if (nv <= 1) RT_SM(1);
         else if (nv <= 2) RT_SM(2);
         else if (nv <= 3) RT_SM(3);
@@ -1087,7 +1086,7 @@ template <typename T, int MODE> int launch_wave(rt_device* dev, const void* x, v
         const uint32_t nv = (nvec + BLOCK - 1) / BLOCK;
         RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax: too many rows");
         const dim3 grid((unsigned)rows), block(BLOCK);
-#define RT_SM(NVC) hipLaunchKernelGGL((softmax_wave_kernel<T, NVC, MODE, BLOCK>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols)
+#define RT_SM(NVC) hipLaunchKernelGGL((softmax_wave_kernel<T, NVC, MODE, BLOCK, SPAN>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols)
         if (nv <= 3) RT_SM(3);
         else if (nv <= 4) RT_SM(4);
         else if (nv <= 6) RT_SM(6);
@@ -1100,8 +1099,10 @@ template <typename T, int MODE> int launch_wave(rt_device* dev, const void* x, v
 
 template <typename T, int MODE> int launch_f32_style(rt_device* dev, const void* x, void* y, uint64_t rows, uint32_t cols) {
     constexpr int VE = 16 / sizeof(T);
-    const bool vec_ok = (cols % VE == 0) && rt_aligned(x, 16) && rt_aligned(y, 16) && (cols / VE) <= (uint32_t)(BLOCK * 8);
-    if (vec_ok) return launch_wave<T, MODE>(dev, x, y, rows, cols);
+    const bool aligned = rt_aligned(x, 16) && rt_aligned(y, 16);
+    if (aligned && cols % VE == 0 && cols / VE <= (uint32_t)(BLOCK * 8)) return launch_wave<T, MODE, false>(dev, x, y, rows, cols);
+    // rows that are not whole vectors: over the aligned vectors that cover each row
+    if (aligned && (cols + 2 * VE - 2) / VE <= (uint32_t)(BLOCK * 8)) return launch_wave<T, MODE, true>(dev, x, y, rows, cols);
     RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax: too many rows");
     hipLaunchKernelGGL((softmax_generic_kernel<T, MODE>), dim3((unsigned)rows), dim3(BLOCK), 0, dev->stream, (const T*)x, (T*)y, rows,
                        cols);
@@ -1109,8 +1110,6 @@ template <typename T, int MODE> int launch_f32_style(rt_device* dev, const void*
     return RT_OK;
 }
 
-// mask == nullptr: plain softmax.  Otherwise the mask has `period` rows of `cols` columns and repeats every `period`
-// rows of x (rows % period == 0).  Returns RT_OK with *done = false when the shape does not fit this kernel.
 // The ragged-row variant's second launch: the elements of a row's first and last span vectors when those vectors are
 // shared with a neighbouring row (at most 7 + 7 per row), from x, the exp table and the row sum the streaming kernel
 // left in row_sums.  Sixteen threads per row: 0..7 the elements of the first span vector, 8..15 those of the last.
@@ -1137,6 +1136,8 @@ __global__ void __launch_bounds__(BLOCK) softmax16_edges_kernel(const uint16_t* 
     y[at] = Ar<T>::div(ev, __builtin_bit_cast(T, row_sums[row]));
 }
 
+// mask == nullptr: plain softmax.  Otherwise the mask has `period` rows of `cols` columns and repeats every `period`
+// rows of x (rows % period == 0).  Returns RT_OK with *done = false when the shape does not fit this kernel.
 template <typename T>
 int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t period, void* y, uint64_t rows, uint32_t cols, bool* done) {
     *done = false;

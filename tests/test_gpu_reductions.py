@@ -40,6 +40,46 @@ def test_softmax_f32(dev, oracle, shape):
     assert bad == 0, (shape, bad, mx)
 
 
+@pytest.mark.parametrize("shape", [(2, 3, 101, 101), (1, 7, 33), (300, 5), (64, 1), (9, 1499), (5, 2047), (3, 5001), (2, 8190), (2, 8191), (40, 13)])
+def test_softmax_f32_rows_that_are_not_whole_vectors(dev, oracle, shape):
+    """ragged f32 rows run over the aligned vectors that cover them (8190 columns are the most that fit; 8191 take the
+    scalar kernel): same results as for whole vectors, masked and overflowing rows included, and nothing written outside
+    the tensor; reference and stable mode, also for f16 in stable mode"""
+    from ratchet_amd import _lib
+    from ratchet_amd.runtime import BufferView
+
+    rng = np.random.default_rng(310)
+    x = randn(rng, shape, np.float32, 3.0)
+    flat = x.reshape(-1, shape[-1])
+    flat[0, shape[-1] // 2 + 1:] = -np.inf
+    flat[-1, :] = -np.inf                                              # 0 / 0 in the last row
+    if flat.shape[0] > 2:
+        flat[1, 0] = 100.0                                             # overflow in a row's first (shared) vector
+    want = oracle.softmax(x)
+    dx = dev.upload(x)
+    fill = np.full(x.size + 12, 7.25, np.float32)
+    big = dev.upload(fill)
+    out = BufferView(big, 4, x.shape)
+    dev.softmax(dx, out=out)
+    got = out.to_numpy()
+    bad, mx = oracle.count_not_close(got, want, 1e-5, 1e-5)
+    assert bad == 0, (shape, bad, mx)
+    whole = big.to_numpy()
+    assert (whole[:4] == 7.25).all() and (whole[4 + x.size:] == 7.25).all()
+    dev.softmax(dx, out=dx)                                             # in place
+    assert same_bits(dx.to_numpy(), got)
+    x[np.isinf(x) | (x == 100.0)] = -5.0
+    with np.errstate(all="ignore"):
+        ref = F.softmax(torch.from_numpy(x), dim=-1).numpy()
+    got = dev.softmax(dev.upload(x), mode=_lib.SOFTMAX_STABLE).to_numpy()
+    bad, mx = oracle.count_not_close(got, ref, 1e-6, 1e-6)
+    assert bad == 0, ("stable", shape, bad, mx)
+    got = dev.softmax(dev.upload(x.astype(np.float16)), mode=_lib.SOFTMAX_STABLE).to_numpy()
+    ref = F.softmax(torch.from_numpy(x.astype(np.float16).astype(np.float32)), dim=-1).numpy()
+    bad, mx = oracle.count_not_close(got.astype(np.float32), ref, 1e-3, 1e-3)
+    assert bad == 0, ("stable f16", shape, bad, mx)
+
+
 def test_softmax_f32_masks_overflow_in_place(dev, oracle):
     ninf = -np.inf
     x = np.zeros((4, 64), np.float32)
