@@ -61,18 +61,24 @@ template <typename T, int KIND> __device__ __forceinline__ T norm_one(T x, const
     return v;
 }
 
-// cols % VE == 0, rows 16-byte aligned, cols / VE <= 64 * NV
-template <typename T, int NV, int KIND, int LANES>
-__global__ void __launch_bounds__(BLOCK) norm_wave_kernel(const T* __restrict__ x, const T* __restrict__ scale,
-                                                          const T* __restrict__ bias, T* __restrict__ y, uint64_t rows, uint32_t cols,
-                                                          float eps) {
+// x and y 16-byte aligned, at most LANES * NV vectors per row.  Rows of whole vectors (scale and bias 16-byte aligned as
+// well), or SPAN: rows of any length over the aligned vectors that cover them.  A row then starts `shift` elements into
+// its first vector; span elements outside the row belong to the neighbouring rows, stay out of the sums and are not
+// written (the row's two ragged vectors are stored element by element), and scale / bias are read by column.  An
+// aligned vector that holds one byte of the tensor lies in a mapped page, so the loads are safe at the tensor's ends too.
+template <typename T, int NV, int KIND, int LANES, bool SPAN>
+__global__ void __launch_bounds__(BLOCK) norm_wave_kernel(const T* x, const T* __restrict__ scale, const T* __restrict__ bias, T* y,
+                                                          uint64_t rows, uint32_t cols, float eps) {
     constexpr int VE = 16 / sizeof(T);
     const uint64_t row = (uint64_t)blockIdx.x * (BLOCK / LANES) + (threadIdx.x / LANES);
     if (row >= rows) return;
     const int lane = threadIdx.x & (LANES - 1);
-    const uint32_t nvec = cols / VE;
-    const v4u* xr = reinterpret_cast<const v4u*>(x + row * cols);
-    v4u* yr = reinterpret_cast<v4u*>(y + row * cols);
+    const uint64_t first = row * cols;
+    const uint32_t shift = SPAN ? (uint32_t)(first & (VE - 1)) : 0;
+    const uint32_t nvec = SPAN ? (shift + cols + VE - 1) / VE : cols / VE;
+    const v4u* xr = reinterpret_cast<const v4u*>(x) + first / VE;
+    v4u* yr = reinterpret_cast<v4u*>(y) + first / VE;
+    auto inside = [&](uint32_t i, int q) -> bool { return !SPAN || i * VE + (uint32_t)q - shift < cols; };
     Vec16<T> v[NV];
 #pragma unroll
     for (int k = 0; k < NV; k++) {
@@ -84,11 +90,12 @@ __global__ void __launch_bounds__(BLOCK) norm_wave_kernel(const T* __restrict__ 
     for (int k = 0; k < NV; k++)
         if (lane + k * LANES < nvec)
 #pragma unroll
-            for (int q = 0; q < VE; q++) {
-                const T e = v[k].e[q];
-                if (KIND == NORM_LAYER) sx += Ar<T>::widen(e);
-                sq += Ar<T>::widen(Ar<T>::mul(e, e));
-            }
+            for (int q = 0; q < VE; q++)
+                if (inside(lane + k * LANES, q)) {
+                    const T e = v[k].e[q];
+                    if (KIND == NORM_LAYER) sx += Ar<T>::widen(e);
+                    sq += Ar<T>::widen(Ar<T>::mul(e, e));
+                }
     if (KIND == NORM_LAYER) sx = row_sum<LANES>(sx);
     sq = row_sum<LANES>(sq);
     const RowStats<T> st = finish_stats<T, KIND>(sx, sq, cols, eps);
@@ -99,11 +106,31 @@ __global__ void __launch_bounds__(BLOCK) norm_wave_kernel(const T* __restrict__ 
         const uint32_t i = lane + k * LANES;
         if (i < nvec) {
             Vec16<T> s, b, o;
-            s.u = sv[i];
-            if (KIND == NORM_LAYER && bias) b.u = bv[i];
+            if (!SPAN) {
+                s.u = sv[i];
+                if (KIND == NORM_LAYER && bias) b.u = bv[i];
 #pragma unroll
-            for (int q = 0; q < VE; q++) o.e[q] = norm_one<T, KIND>(v[k].e[q], st, s.e[q], b.e[q], bias != nullptr);
-            st_stream(yr + i, o.u);
+                for (int q = 0; q < VE; q++) o.e[q] = norm_one<T, KIND>(v[k].e[q], st, s.e[q], b.e[q], bias != nullptr);
+                st_stream(yr + i, o.u);
+            } else if (inside(i, 0) && inside(i, VE - 1)) {
+                // a vector inside the row: its scale / bias elements are 16 contiguous bytes at element alignment
+                const uint32_t c0 = i * VE - shift;
+                __builtin_memcpy(&s.u, scale + c0, 16);
+                if (KIND == NORM_LAYER && bias) __builtin_memcpy(&b.u, bias + c0, 16);
+#pragma unroll
+                for (int q = 0; q < VE; q++) o.e[q] = norm_one<T, KIND>(v[k].e[q], st, s.e[q], b.e[q], bias != nullptr);
+                st_stream(yr + i, o.u);
+            } else {
+                T* yrow = y + first;
+#pragma unroll
+                for (int q = 0; q < VE; q++) {
+                    const uint32_t c = i * VE + (uint32_t)q - shift;
+                    if (c < cols) {
+                        const T bq = (KIND == NORM_LAYER && bias) ? bias[c] : Ar<T>::conv(0.0f);
+                        yrow[c] = norm_one<T, KIND>(v[k].e[q], st, scale[c], bq, bias != nullptr);
+                    }
+                }
+            }
         }
     }
 }
@@ -571,12 +598,30 @@ __global__ void __launch_bounds__(BLOCK) gn_apply_kernel(const T* __restrict__ x
     }
 }
 
+template <typename T, int KIND, bool SPAN>
+int launch_norm_wave(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint64_t rows, uint32_t cols, float eps);
+
 template <typename T, int KIND>
 int launch_norm(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint64_t rows, uint32_t cols, float eps) {
     constexpr int VE = 16 / sizeof(T);
-    const uint32_t nvec = cols / VE;
-    const bool vec_ok = (cols % VE == 0) && rt_aligned(x, 16) && rt_aligned(y, 16) && rt_aligned(scale, 16) &&
-                        (!bias || rt_aligned(bias, 16)) && nvec <= (uint32_t)(BLOCK * 8);
+    const bool io_aligned = rt_aligned(x, 16) && rt_aligned(y, 16);
+    if (io_aligned && cols % VE == 0 && rt_aligned(scale, 16) && (!bias || rt_aligned(bias, 16)) && cols / VE <= (uint32_t)(BLOCK * 8))
+        return launch_norm_wave<T, KIND, false>(dev, x, scale, bias, y, rows, cols, eps);
+    // rows that are not whole vectors (or scale / bias off their alignment): over the aligned vectors that cover each row
+    if (io_aligned && (cols + 2 * VE - 2) / VE <= (uint32_t)(BLOCK * 8))
+        return launch_norm_wave<T, KIND, true>(dev, x, scale, bias, y, rows, cols, eps);
+    RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
+    hipLaunchKernelGGL((norm_generic_kernel<T, KIND>), dim3((unsigned)rows), dim3(BLOCK), 0, dev->stream, (const T*)x, (const T*)scale,
+                       (const T*)bias, (T*)y, rows, cols, eps);
+    RT_CHECK_LAUNCH("norm_generic_kernel");
+    return RT_OK;
+}
+
+template <typename T, int KIND, bool SPAN>
+int launch_norm_wave(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint64_t rows, uint32_t cols, float eps) {
+    constexpr int VE = 16 / sizeof(T);
+    const uint32_t nvec = SPAN ? (cols + 2 * VE - 2) / VE : cols / VE;       // SPAN: the most vectors a row can touch
+    const bool vec_ok = true;
     if (vec_ok && nvec <= 32) {
         // rows of at most 32 vectors: a group of 2..32 lanes per row (one vector each), so that a wave carries 2..32 rows
         // and as many bytes as with long rows
@@ -584,7 +629,7 @@ int launch_norm(rt_device* dev, const void* x, const void* scale, const void* bi
         const uint64_t blocks = (rows + BLOCK / lanes - 1) / (BLOCK / lanes);
         RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
         const dim3 grid((unsigned)blocks), block(BLOCK);
-#define RT_NARROW(L) hipLaunchKernelGGL((norm_wave_kernel<T, 1, KIND, L>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, (T*)y, rows, cols, eps)
+#define RT_NARROW(L) hipLaunchKernelGGL((norm_wave_kernel<T, 1, KIND, L, SPAN>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, (T*)y, rows, cols, eps)
         if (lanes == 2) RT_NARROW(2);
         else if (lanes == 4) RT_NARROW(4);
         else if (lanes == 8) RT_NARROW(8);
@@ -600,7 +645,7 @@ int launch_norm(rt_device* dev, const void* x, const void* scale, const void* bi
         RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
         const dim3 grid((unsigned)blocks), block(BLOCK);
 #define RT_NORM(NVC)                                                                                                                 \
-    hipLaunchKernelGGL((norm_wave_kernel<T, NVC, KIND, WAVE>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, \
+    hipLaunchKernelGGL((norm_wave_kernel<T, NVC, KIND, WAVE, SPAN>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, \
                        (T*)y, rows, cols, eps)
         if (nv <= 1) RT_NORM(1);
         else if (nv <= 2) RT_NORM(2);
@@ -618,7 +663,7 @@ int launch_norm(rt_device* dev, const void* x, const void* scale, const void* bi
         RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
         const dim3 grid((unsigned)rows), block(BLOCK);
 #define RT_NORM(NVC)                                                                                                                  \
-    hipLaunchKernelGGL((norm_wave_kernel<T, NVC, KIND, BLOCK>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, \
+    hipLaunchKernelGGL((norm_wave_kernel<T, NVC, KIND, BLOCK, SPAN>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, \
                        (T*)y, rows, cols, eps)
         if (nv <= 3) RT_NORM(3);
         else if (nv <= 4) RT_NORM(4);
@@ -628,11 +673,7 @@ int launch_norm(rt_device* dev, const void* x, const void* scale, const void* bi
         RT_CHECK_LAUNCH("norm_wave_kernel");
         return RT_OK;
     }
-    RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
-    hipLaunchKernelGGL((norm_generic_kernel<T, KIND>), dim3((unsigned)rows), dim3(BLOCK), 0, dev->stream, (const T*)x, (const T*)scale,
-                       (const T*)bias, (T*)y, rows, cols, eps);
-    RT_CHECK_LAUNCH("norm_generic_kernel");
-    return RT_OK;
+    return rt_fail(RT_ERR_SIZE, "norm: row too long for the register-resident kernel");      // not reached: the caller checks the length
 }
 
 // 16-bit reference arithmetic, many rows of at most 128 columns (whole aligned vectors): one lane per row.  A block's

@@ -360,6 +360,36 @@ def test_rms_norm_f32(dev, oracle, shape):
     assert bad == 0, (shape, bad, mx)
 
 
+@pytest.mark.parametrize("shape", [(3, 101, 101), (7, 33), (300, 5), (64, 1), (9, 1499), (5, 2047), (3, 5001), (2, 8190), (2, 8191), (4000, 13)])
+def test_norms_f32_rows_that_are_not_whole_vectors(dev, oracle, shape):
+    """ragged f32 rows run over the aligned vectors that cover them (8191 columns take the scalar kernel): results inside the
+    f32 bar, nothing written outside the tensor; also with scale / bias 4 bytes off their vector alignment on whole-vector rows"""
+    from ratchet_amd.runtime import BufferView
+
+    rng = np.random.default_rng(311)
+    cols = shape[-1]
+    x = randn(rng, shape, np.float32, 1.5)
+    w, b = randn(rng, (cols,), np.float32), randn(rng, (cols,), np.float32)
+    dx, dw, db = dev.upload(x), dev.upload(w), dev.upload(b)
+    for name, want, run in (("layer", oracle.layer_norm(x, w, b, 1e-5, intended=True), lambda o: dev.layer_norm(dx, dw, db, 1e-5, out=o)),
+                            ("layer, no bias", oracle.layer_norm(x, w, None, 1e-5, intended=True), lambda o: dev.layer_norm(dx, dw, None, 1e-5, out=o)),
+                            ("rms", oracle.rms_norm(x, w, 1e-5, intended=True), lambda o: dev.rms_norm(dx, dw, 1e-5, out=o))):
+        big = dev.upload(np.full(x.size + 12, 7.25, np.float32))
+        out = BufferView(big, 4, x.shape)
+        run(out)
+        bad, mx = oracle.count_not_close(out.to_numpy(), want, 1e-5, 1e-5)
+        assert bad == 0 or cols == 1, (name, shape, bad, mx)
+        whole = big.to_numpy()
+        assert (whole[:4] == 7.25).all() and (whole[4 + x.size:] == 7.25).all(), (name, shape)
+    x = randn(rng, (37, 512), np.float32, 1.5)
+    w, b = randn(rng, (512,), np.float32), randn(rng, (512,), np.float32)
+    wv = BufferView(dev.empty((516,), 0), 1, (512,)).upload(w)
+    bv = BufferView(dev.empty((516,), 0), 3, (512,)).upload(b)
+    got = dev.layer_norm(dev.upload(x), wv, bv, 1e-5).to_numpy()
+    bad, mx = oracle.count_not_close(got, oracle.layer_norm(x, w, b, 1e-5, intended=True), 1e-5, 1e-5)
+    assert bad == 0, (bad, mx)
+
+
 @pytest.mark.parametrize("shape", [(2, 64, 2560), (1, 33, 3072), (1, 9, 384), (1, 7, 100), (1, 3, 4104), (16, 128, 256), (1, 5, 1)])
 def test_norms_f16(dev, oracle, shape):
     rng = np.random.default_rng(312)
