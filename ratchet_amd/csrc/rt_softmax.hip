@@ -408,7 +408,8 @@ template <> struct SpType<bf16_t> {
 // table lookup (adding +0 leaves the running sum as it is), and a vector that is not entirely inside its row is not
 // stored.  Wave 0 also writes each row's sum to `row_sums`; the elements of those ragged vectors (at most 14 per row) are
 // finished by softmax16_edges_kernel from x, the table and that sum.  An aligned vector that holds one byte of the tensor
-// lies in a mapped page, so the loads are safe at the tensor's ends too.
+// lies in a mapped page, so the loads are safe at the tensor's ends too.  A row's span can be one vector longer than
+// NSTEP steps hold (2047 columns starting 14 bytes into a vector): wave 0 reads that vector itself and adds it last.
 template <typename T, int NSTEP, bool FULL, bool MASK, bool RAGGED = false>
 __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16_t* __restrict__ table, const T* x, const T* mask, T* y,
                                                                     uint64_t rows, uint32_t cols, SpSched sch, uint16_t* row_sums) {
@@ -442,6 +443,24 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
         typename ST::Run run = ST::zero();
         uint32_t gpar = 0;
         for (uint32_t it = 0; it < n_items; it++) {
+            // RAGGED: a row that starts sh bytes into its first vector can reach up to 14 bytes past its last step.  That
+            // one vector is fetched here, at the start of the group, and added after the group's last step.
+            uint32_t my_row = 0, tail_end = 0;               // tail_end: bytes of the row inside the extra vector, 0 = none
+            bool my_ok = false;
+            v4u tailv = {0, 0, 0, 0};
+            if (RAGGED) {
+                uint32_t rep, pg;
+                sp_item(sch, blockIdx.x, gridDim.x, it, rep, pg);
+                const uint32_t prow = pg * sch.R + lane;
+                my_ok = lane < sch.R && prow < sch.P;
+                my_row = rep * sch.P + prow;
+                const uint32_t off = my_row * (cols * 2);
+                const uint32_t end = (off & 15u) + cols * 2; // one past the row's last byte, in span coordinates
+                if (my_ok && end > nsteps * (SP_TC * 2)) {
+                    tail_end = end - nsteps * (SP_TC * 2);
+                    tailv = *reinterpret_cast<const v4u*>(reinterpret_cast<const char*>(x) + (off & ~15u) + nsteps * (SP_TC * 2));
+                }
+            }
 #pragma unroll 1
             for (uint32_t t = 0; t < nsteps; t++) {
                 __syncthreads();                             // A
@@ -463,13 +482,15 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                     c1 = n1;
                 }
             }
-            if (lane < SP_ROWS) sums[gpar][lane] = ST::run_bits(run);
-            if (RAGGED) {
-                uint32_t rep, pg;
-                sp_item(sch, blockIdx.x, gridDim.x, it, rep, pg);
-                const uint32_t prow = pg * sch.R + lane;
-                if (lane < sch.R && prow < sch.P) row_sums[rep * sch.P + prow] = ST::run_bits(run);
+            if (RAGGED && tail_end) {
+#pragma unroll
+                for (int w = 0; w < 4; w++) {                // elements past the row's end count as +0
+                    const uint32_t keep = ((uint32_t)(4 * w) < tail_end ? 0xffffu : 0u) | ((uint32_t)(4 * w + 2) < tail_end ? 0xffff0000u : 0u);
+                    ST::add_pair(run, sp_exp_pair(lut, tailv[w]) & keep);
+                }
             }
+            if (lane < SP_ROWS) sums[gpar][lane] = ST::run_bits(run);
+            if (RAGGED && my_ok) row_sums[my_row] = ST::run_bits(run);
             run = ST::zero();
             gpar ^= 1;
         }
@@ -594,19 +615,32 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
         if (MASK) in = ST::add_vec(in, m);                   // scores + mask in the 16-bit type, as the separate add would round it
 #pragma unroll
         for (int w = 0; w < 4; w++) in[w] = sp_exp_pair(lut, in[w]);
-        if (RAGGED) {
-            const uint32_t p = t * (SP_TC * 2) + cbyte, end = sh + row_bytes;
-            if (p >= end) {
-                in = v4u{0, 0, 0, 0};
-            } else if (p < sh || p + 16 > end) {             // one of the row's two ragged vectors: a few lanes per row
-#pragma unroll
-                for (int w = 0; w < 4; w++) {
-                    const uint32_t b0 = p + 4 * w, b1 = b0 + 2;
-                    in[w] &= ((b0 >= sh && b0 < end) ? 0xffffu : 0u) | ((b1 >= sh && b1 < end) ? 0xffff0000u : 0u);
-                }
+        if (RAGGED ? t * (SP_TC * 2) + cbyte >= sh + row_bytes : past_end(t)) in = v4u{0, 0, 0, 0};
+    };
+    // RAGGED: the neighbours' elements in a row's first and last vector are zeroed in the tile, after the vector has been
+    // written there (on the LDS copy, so that the data registers of the main path stay untouched: masking them in a branch
+    // cost 50 vector registers).  Which step and lane hold those two vectors is the same for the whole wave (sh lives in a
+    // scalar register), so every test below is a scalar branch except the one that picks the lane, and the zeros go out
+    // as at most three aligned writes of 8, 4 and 2 bytes.
+    auto zero_outside = [&](uint32_t t, uint32_t sh, uint32_t trow_idx) {
+        unsigned char* trb = reinterpret_cast<unsigned char*>(&tile[trow_idx][0]);
+        if (t == 0 && sh != 0 && cbyte == 0) {               // bytes [0, sh) of the span belong to the row before
+            if (sh & 8) *reinterpret_cast<uint64_t*>(trb) = 0;
+            if (sh & 4) *reinterpret_cast<uint32_t*>(trb + (sh & 8)) = 0;
+            if (sh & 2) *reinterpret_cast<uint16_t*>(trb + (sh & 12)) = 0;
+        }
+        const uint32_t end = sh + row_bytes, pe = end & ~15u;        // the vector at span byte pe holds the row's end
+        if ((end & 15u) != 0 && t == pe / (SP_TC * 2) && cbyte == (pe & (SP_TC * 2 - 1))) {
+            uint32_t at = (pe & (SP_TC * 2 - 1)) + (end & 15u);      // bytes [at, next vector) belong to the row after
+            if (at & 2) {
+                *reinterpret_cast<uint16_t*>(trb + at) = 0;
+                at += 2;
             }
-        } else if (past_end(t)) {
-            in = v4u{0, 0, 0, 0};
+            if (at & 4) {
+                *reinterpret_cast<uint32_t*>(trb + at) = 0;
+                at += 4;
+            }
+            if (at & 8) *reinterpret_cast<uint64_t*>(trb + at) = 0;
         }
     };
 
@@ -643,6 +677,10 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                 __syncthreads();                             // A: wave 0 has left the previous tile
                 *reinterpret_cast<v4u*>(&tile[rr][ccol]) = pre[t % PF][0];
                 *reinterpret_cast<v4u*>(&tile[rr + SP_HALF][ccol]) = pre[t % PF][1];
+                if (RAGGED) {
+                    zero_outside(t, pcur[0], rr);
+                    zero_outside(t, pcur[1], rr + SP_HALF);
+                }
                 // the registers are free again: next loads, PF steps ahead, possibly in the block's next group
                 // (loads return in order: the mask of the next step goes first, so that waiting for it does not wait for x
                 // of the step after)
@@ -1165,8 +1203,8 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
     const uint16_t* table = nullptr;
     int rc = rt_unary_table(dev, TI, RT_EXP, &table);
     if (rc) return rc;
-    const uint32_t nt = (cols + (ragged ? 7 : 0) + SP_TC - 1) / SP_TC;       // a ragged row's span is up to 7 elements longer
-    if (ragged && nt > SP_MAX_STEPS) return RT_OK;
+    const uint32_t nt = (cols + SP_TC - 1) / SP_TC;
+    if (ragged && nt > SP_MAX_STEPS) return RT_OK;           // (a ragged row's one vector past its last step is the walker's)
     const bool full = !ragged && cols % SP_TC == 0 && (nt == 1 || nt == 2 || nt == 4 || nt == 8);
 #define RT_SP(NS, F, M)                                                                                                              \
     do {                                                                                                                             \

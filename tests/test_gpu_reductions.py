@@ -218,12 +218,13 @@ def test_softmax_16_bit_long_rows(dev, oracle, shape, kind):
         assert not ((got != want) & ~(isnan(got) & isnan(want))).any(), shape
 
 
-@pytest.mark.parametrize("shape,kind", [((2, 4, 333, 1001), "f16"), ((1, 3, 100, 199), "f16"), ((70, 4089), "f16"), ((7, 4090), "f16"), ((33, 513), "f16"),
-                                        ((1000, 193), "f16"), ((61, 2561), "f16"), ((2, 2, 77, 1001), "bf16"), ((40, 3001), "bf16"), ((900, 250), "bf16")])
+@pytest.mark.parametrize("shape,kind", [((2, 4, 333, 1001), "f16"), ((1, 3, 100, 199), "f16"), ((70, 4095), "f16"), ((7, 4097), "f16"), ((50, 2047), "f16"), ((90, 511), "f16"), ((45, 1535), "f16"), ((33, 3071), "f16"), ((33, 513), "f16"),
+                                        ((1000, 193), "f16"), ((61, 2561), "f16"), ((2, 2, 77, 1001), "bf16"), ((40, 3001), "bf16"), ((31, 1535), "bf16"), ((900, 250), "bf16")])
 def test_softmax_16_bit_ragged_rows_stream(dev, oracle, shape, kind):
     """rows of 192 or more columns that are not whole 16-byte vectors (a prompt of 1001 tokens): streamed over the aligned
     vectors that cover each row, the vectors shared by two rows finished by a second small launch; bit-exact like the
-    aligned rows, out of place and in place.  4089 columns fill the largest register-parked variant, 4090 are past it."""
+    aligned rows, out of place and in place.  4095 columns fill the largest register-parked variant, 4097 are past it; rows
+    of 511, 1535, 2047, 4095 columns can reach one vector past their last 512-column step."""
     from ratchet_amd.runtime import BufferView
 
     rng = np.random.default_rng(308)
