@@ -415,7 +415,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                                                                     uint64_t rows, uint32_t cols, SpSched sch, uint16_t* row_sums) {
     typedef SpType<T> ST;
     constexpr bool PARK = NSTEP > 0;
-    static_assert(!RAGGED || (PARK && !FULL && !MASK), "the ragged variant parks in registers, has no full-step shortcut and no mask");
+    static_assert(!RAGGED || (PARK && !FULL), "the ragged variant parks in registers and has no full-step shortcut");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint16_t* lut = reinterpret_cast<uint16_t*>(smem);
     uint16_t (*tile)[SP_TC + SP_PAD] = reinterpret_cast<uint16_t (*)[SP_TC + SP_PAD]>(smem + SP_LUT_BYTES);
@@ -513,7 +513,8 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
     const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(x), 0, nbytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(y, 0, nbytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t rm =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(MASK ? mask : x), 0, MASK ? sch.PM * row_bytes : nbytes, 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(MASK ? mask : x), 0,
+                                          MASK ? (RAGGED ? (sch.PM * row_bytes + 15) & ~15u : sch.PM * row_bytes) : nbytes, 0x00020000);
     constexpr uint32_t OOB = 0x80000000u;                    // >= nbytes, and stays so after adding a column offset
     const uint32_t G = gridDim.x;
 
@@ -522,7 +523,9 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
     // and the row's offset in the mask (for a row that does not exist the mask offset is arbitrary, which is harmless:
     // the load is range checked, and what is computed from it is never stored).
     // (RAGGED: xo is the offset of the row's first span vector and mdiff carries sh, the row's start inside that vector)
-    auto item_off = [&](uint32_t it, uint32_t (&xo)[2], uint32_t (&mdiff)[2]) {
+    // (RAGGED with MASK: mq is the mask byte that lines up with the row's span origin, mask row offset minus sh; it is only
+    // element aligned, and negative for the mask's first row when sh > 0)
+    auto item_off = [&](uint32_t it, uint32_t (&xo)[2], uint32_t (&mdiff)[2], uint32_t (&mq)[2]) {
         uint32_t rep, pg;
         sp_item(sch, blockIdx.x, G, it, rep, pg);
 #pragma unroll
@@ -531,9 +534,15 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
             const uint32_t prow = pg * sch.R + r;            // row inside the period
             const bool ok = it < n_items && r < sch.R && prow < sch.P;
             const uint32_t row = rep * sch.P + prow;
+            mq[h] = 0;
             if (RAGGED) {
                 xo[h] = __builtin_amdgcn_readfirstlane(ok ? (row * row_bytes) & ~15u : OOB);
                 mdiff[h] = __builtin_amdgcn_readfirstlane((row * row_bytes) & 15u);
+                if (MASK) {
+                    uint32_t q, mrow;
+                    fd_divmod(row, sch.pm_div, q, mrow);
+                    mq[h] = __builtin_amdgcn_readfirstlane(mrow * row_bytes - ((row * row_bytes) & 15u));
+                }
                 continue;
             }
             xo[h] = __builtin_amdgcn_readfirstlane(ok ? row * row_bytes : OOB);
@@ -563,6 +572,40 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
     };
     auto ld_off = [&](uint32_t row_off, uint32_t sh, uint32_t t) -> uint32_t { return RAGGED ? span_load_off(row_off, sh, t) : step_off(row_off, t); };
     auto st_off = [&](uint32_t row_off, uint32_t sh, uint32_t t) -> uint32_t { return RAGGED ? span_store_off(row_off, sh, t) : step_off(row_off, t); };
+    // RAGGED with MASK: the sixteen mask bytes for the vector at span byte p start at mask byte mq + p, which is only
+    // element aligned: they straddle the aligned mask vectors at (mq & ~15) + p and 16 bytes on, (mq & 15) bytes into the
+    // first.  A lane loads the first; the second is its right neighbour's first (one wave shift), except for lane 63,
+    // which loads its own.  An offset before the mask's start wraps to a huge one and is dropped like any other.
+    auto mask_lo_off = [&](uint32_t mq, uint32_t sh, uint32_t t) -> uint32_t {
+        const uint32_t p = t * (SP_TC * 2) + cbyte;
+        return p >= sh + row_bytes + 16 ? OOB : (mq & ~15u) + p;      // also the lane after the row's last vector: it feeds its left neighbour
+    };
+    auto mask_hi_off = [&](uint32_t mq, uint32_t sh, uint32_t t) -> uint32_t {
+        const uint32_t p = t * (SP_TC * 2) + cbyte;
+        return (cbyte != 63 * 16 || p >= sh + row_bytes) ? OOB : (mq & ~15u) + p + 16;
+    };
+    auto mask_funnel = [&](const v4u& lo, const v4u& hi_own, uint32_t mq) -> v4u {
+        const uint32_t d = mq & 15u;                         // the same for the whole wave: branches, not selects
+        uint32_t cat[8];
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            cat[w] = lo[w];
+            // lane i takes lane i + 1's value; lane 63 keeps the vector it loaded itself
+            cat[w + 4] = (uint32_t)__builtin_amdgcn_update_dpp((int)hi_own[w], (int)lo[w], 0x130, 0xf, 0xf, false);
+        }
+        v4u out;
+        switch (d >> 2) {
+#define RT_PICK(O)                                                                                                              \
+    _Pragma("unroll") for (int w = 0; w < 4; w++)                                                                              \
+        out[w] = (d & 2) ? __builtin_amdgcn_alignbyte(cat[w + O + 1 < 8 ? w + O + 1 : 7], cat[w + O], 2) : cat[w + O];
+            case 0: RT_PICK(0) break;
+            case 1: RT_PICK(1) break;
+            case 2: RT_PICK(2) break;
+            default: RT_PICK(3) break;
+#undef RT_PICK
+        }
+        return out;
+    };
     auto load_x = [&](uint32_t off) -> v4u { return __builtin_amdgcn_raw_buffer_load_b128(rx, off, 0, 2); };   // 2: non-temporal
     auto load_m = [&](uint32_t off) -> v4u { return __builtin_amdgcn_raw_buffer_load_b128(rm, off, 0, 0); };   // re-read by other heads
     auto load_y = [&](uint32_t off) -> v4u { return __builtin_amdgcn_raw_buffer_load_b128(ry, off, 0, 0); };
@@ -644,15 +687,16 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
         }
     };
 
-    uint32_t cur[2], nxt[2], prev[2] = {OOB, OOB}, pcur[2], pnxt[2], pprev[2] = {0, 0};
-    item_off(0, cur, pcur);
-    item_off(1, nxt, pnxt);
+    uint32_t cur[2], nxt[2], prev[2] = {OOB, OOB}, pcur[2], pnxt[2], pprev[2] = {0, 0}, mcur[2], mnxt[2];
+    item_off(0, cur, pcur, mcur);
+    item_off(1, nxt, pnxt, mnxt);
     uint32_t gpar = 0;
 
     if constexpr (PARK) {
         constexpr int PF = NSTEP < SP_PF ? NSTEP : SP_PF;    // steps of x in flight per thread
         v4u e[NSTEP][2];                                     // exp values of the group in flight, 8 halves per vector
         v4u pre[PF][2], mpre[2];                             // x: PF steps in flight; mask: one (L2 hits: a short distance is enough)
+        v4u mhi[2];                                          // RAGGED: lane 63's second mask vector
 #pragma unroll
         for (int t = 0; t < NSTEP; t++) e[t][0] = e[t][1] = v4u{0, 0, 0, 0};
         // The pending memory operations at the top of the group loop are the same on entry as after a group (two loads, two
@@ -664,16 +708,24 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
 #pragma unroll
             for (int h = 0; h < 2; h++) store_y(v4u{0, 0, 0, 0}, OOB);
         }
-        if (MASK) {
+        if (MASK && !RAGGED) {
 #pragma unroll
             for (int h = 0; h < 2; h++) mpre[h] = load_m(step_off(cur[h] - pcur[h], 0));
+        }
+        if (MASK && RAGGED) {
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                mpre[h] = load_m(mask_lo_off(mcur[h], pcur[h], 0));
+                mhi[h] = load_m(mask_hi_off(mcur[h], pcur[h], 0));
+            }
         }
 
         for (uint32_t it = 0; it < n_items; it++) {
 #pragma unroll
             for (int t = 0; t < NSTEP; t++) {
 #pragma unroll
-                for (int h = 0; h < 2; h++) exp_in_place(pre[t % PF][h], mpre[h], t, pcur[h]);
+                for (int h = 0; h < 2; h++)
+                    exp_in_place(pre[t % PF][h], (MASK && RAGGED) ? mask_funnel(mpre[h], mhi[h], mcur[h]) : mpre[h], t, pcur[h]);
                 __syncthreads();                             // A: wave 0 has left the previous tile
                 *reinterpret_cast<v4u*>(&tile[rr][ccol]) = pre[t % PF][0];
                 *reinterpret_cast<v4u*>(&tile[rr + SP_HALF][ccol]) = pre[t % PF][1];
@@ -684,10 +736,17 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                 // the registers are free again: next loads, PF steps ahead, possibly in the block's next group
                 // (loads return in order: the mask of the next step goes first, so that waiting for it does not wait for x
                 // of the step after)
-                if (MASK) {
+                if (MASK && !RAGGED) {
 #pragma unroll
                     for (int h = 0; h < 2; h++)
                         mpre[h] = (t + 1 < NSTEP) ? load_m(step_off(cur[h] - pcur[h], t + 1)) : load_m(step_off(nxt[h] - pnxt[h], 0));
+                }
+                if (MASK && RAGGED) {
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        mpre[h] = (t + 1 < NSTEP) ? load_m(mask_lo_off(mcur[h], pcur[h], t + 1)) : load_m(mask_lo_off(mnxt[h], pnxt[h], 0));
+                        mhi[h] = (t + 1 < NSTEP) ? load_m(mask_hi_off(mcur[h], pcur[h], t + 1)) : load_m(mask_hi_off(mnxt[h], pnxt[h], 0));
+                    }
                 }
 #pragma unroll
                 for (int h = 0; h < 2; h++)
@@ -710,8 +769,9 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
             for (int h = 0; h < 2; h++) {
                 pprev[h] = pcur[h];
                 pcur[h] = pnxt[h];
+                mcur[h] = mnxt[h];
             }
-            item_off(it + 2, nxt, pnxt);
+            item_off(it + 2, nxt, pnxt, mnxt);
             gpar ^= 1;
         }
         // drain: outputs of the block's last group
@@ -782,7 +842,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                 }
                 pcur[0] = pnxt[0];
                 pcur[1] = pnxt[1];
-                item_off(trip / (nsteps / 2) + 2, nxt, pnxt);
+                item_off(trip / (nsteps / 2) + 2, nxt, pnxt, mnxt);
                 gpar ^= 1;
             }
         }
@@ -1149,12 +1209,13 @@ template <typename T, int MODE> int launch_f32_style(rt_device* dev, const void*
 }
 
 // The ragged-row variant's second launch: the elements of a row's first and last span vectors when those vectors are
-// shared with a neighbouring row (at most 7 + 7 per row), from x, the exp table and the row sum the streaming kernel
+// shared with a neighbouring row (at most 7 + 7 per row), from x (plus the mask), the exp table and the row sum the streaming kernel
 // left in row_sums.  Sixteen threads per row: 0..7 the elements of the first span vector, 8..15 those of the last.
 // The quotient is the IEEE division the streaming kernel's short division reproduces.
 template <typename T>
-__global__ void __launch_bounds__(BLOCK) softmax16_edges_kernel(const uint16_t* __restrict__ table, const T* x, T* y,
-                                                                const uint16_t* __restrict__ row_sums, uint64_t rows, uint32_t cols) {
+__global__ void __launch_bounds__(BLOCK) softmax16_edges_kernel(const uint16_t* __restrict__ table, const T* x, const T* __restrict__ mask,
+                                                                uint32_t mask_rows, T* y, const uint16_t* __restrict__ row_sums,
+                                                                uint64_t rows, uint32_t cols) {
     const uint64_t gid = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
     const uint64_t row = gid >> 4;
     if (row >= rows) return;
@@ -1169,7 +1230,9 @@ __global__ void __launch_bounds__(BLOCK) softmax16_edges_kernel(const uint16_t* 
     const uint32_t e = (tail ? last_vec * 8 : 0) + j;        // element of the span
     if (e < shift || e - shift >= cols) return;
     const uint64_t at = first + (e - shift);
-    const uint16_t xb = __builtin_bit_cast(uint16_t, x[at]);
+    T xv = x[at];
+    if (mask) xv = Ar<T>::add(xv, mask[(row % mask_rows) * cols + (e - shift)]);     // row r takes mask row r % mask_rows
+    const uint16_t xb = __builtin_bit_cast(uint16_t, xv);
     const T ev = __builtin_bit_cast(T, table[xb]);
     y[at] = Ar<T>::div(ev, __builtin_bit_cast(T, row_sums[row]));
 }
@@ -1183,7 +1246,8 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
     const uint64_t row_bytes = (uint64_t)cols * 2;
     if (!mask) period = rows;
     const bool ragged = cols % 8 != 0;                       // rows over their covering aligned vectors, finished by the edges kernel
-    if (ragged && mask) return RT_OK;
+    // with a mask: in one launch only, a mask on a 16-byte boundary, and steps that hold every row's whole span
+    if (ragged && mask && (!rt_aligned(mask, 16) || rows * row_bytes > 0x7fffffe0ull || rows > RT_SM_ROW_SUMS)) return RT_OK;
     // the kernel addresses a launch with 32-bit byte offsets below 2^31: larger tensors go in chunks of whole periods
     // (whole 30-row groups when nothing repeats)
     uint64_t chunk_rows;
@@ -1203,8 +1267,9 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
     const uint16_t* table = nullptr;
     int rc = rt_unary_table(dev, TI, RT_EXP, &table);
     if (rc) return rc;
-    const uint32_t nt = (cols + SP_TC - 1) / SP_TC;
-    if (ragged && nt > SP_MAX_STEPS) return RT_OK;           // (a ragged row's one vector past its last step is the walker's)
+    // (a ragged row's one vector past its last step is the walker's, which knows no mask: with one, the steps cover it)
+    const uint32_t nt = (cols + (ragged && mask ? 7 : 0) + SP_TC - 1) / SP_TC;
+    if (ragged && nt > SP_MAX_STEPS) return RT_OK;
     const bool full = !ragged && cols % SP_TC == 0 && (nt == 1 || nt == 2 || nt == 4 || nt == 8);
 #define RT_SP(NS, F, M)                                                                                                              \
     do {                                                                                                                             \
@@ -1217,16 +1282,23 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
         hipLaunchKernelGGL((softmax16_stream_kernel<T, NS, F, M>), dim3(blocks), dim3(SP_BLOCK), SP_SMEM_BYTES, dev->stream, table,  \
                            xc, (const T*)mask, yc, n, cols, sch, (uint16_t*)nullptr);                                                \
     } while (0)
-#define RT_SP_RAGGED(NS)                                                                                                             \
+#define RT_SP_RAGGED(NS, M)                                                                                                          \
     do {                                                                                                                             \
-        const uint64_t bit = 1ull << (40 + TI * 4 + (NS == 1 ? 0 : NS == 2 ? 1 : NS == 4 ? 2 : 3));                                  \
+        const uint64_t bit = 1ull << (40 + (M ? 8 : 0) + TI * 4 + (NS == 1 ? 0 : NS == 2 ? 1 : NS == 4 ? 2 : 3));                    \
         if (!(dev->sp_attr_set & bit)) {                                                                                             \
-            RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(softmax16_stream_kernel<T, NS, false, false, true>),            \
+            RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(softmax16_stream_kernel<T, NS, false, M, true>),                \
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)SP_SMEM_BYTES));                             \
             dev->sp_attr_set |= bit;                                                                                                 \
         }                                                                                                                            \
-        hipLaunchKernelGGL((softmax16_stream_kernel<T, NS, false, false, true>), dim3(blocks), dim3(SP_BLOCK), SP_SMEM_BYTES,        \
-                           dev->stream, table, xc, (const T*)nullptr, yc, n, cols, sch, dev->sm_row_sums);                           \
+        hipLaunchKernelGGL((softmax16_stream_kernel<T, NS, false, M, true>), dim3(blocks), dim3(SP_BLOCK), SP_SMEM_BYTES,            \
+                           dev->stream, table, xc, (const T*)mask, yc, n, cols, sch, dev->sm_row_sums);                              \
+    } while (0)
+#define RT_SP_RAGGED_NS(M)                                  \
+    do {                                                    \
+        if (nt <= 1) RT_SP_RAGGED(1, M);                    \
+        else if (nt <= 2) RT_SP_RAGGED(2, M);               \
+        else if (nt <= 4) RT_SP_RAGGED(4, M);               \
+        else RT_SP_RAGGED(8, M);                            \
     } while (0)
 #define RT_SP_NS(F, M)                                      \
     do {                                                    \
@@ -1271,14 +1343,12 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
         RT_REQUIRE(items <= 0xffffffffull, RT_ERR_SIZE, "rt_softmax: too many row groups");
         const unsigned blocks = (unsigned)(items < (uint64_t)dev->num_cus ? items : (uint64_t)dev->num_cus);   // one resident block per CU
         if (ragged) {
-            if (nt <= 1) RT_SP_RAGGED(1);
-            else if (nt <= 2) RT_SP_RAGGED(2);
-            else if (nt <= 4) RT_SP_RAGGED(4);
-            else RT_SP_RAGGED(8);
+            if (mask) RT_SP_RAGGED_NS(true);
+            else RT_SP_RAGGED_NS(false);
             RT_CHECK_LAUNCH("softmax16_stream_kernel");
             const uint64_t eblocks = (n * 16 + BLOCK - 1) / BLOCK;
-            hipLaunchKernelGGL((softmax16_edges_kernel<T>), dim3((unsigned)eblocks), dim3(BLOCK), 0, dev->stream, table, xc, yc,
-                               (const uint16_t*)dev->sm_row_sums, n, cols);
+            hipLaunchKernelGGL((softmax16_edges_kernel<T>), dim3((unsigned)eblocks), dim3(BLOCK), 0, dev->stream, table, xc, (const T*)mask,
+                               sch.PM, yc, (const uint16_t*)dev->sm_row_sums, n, cols);
             RT_CHECK_LAUNCH("softmax16_edges_kernel");
             continue;
         }
@@ -1295,6 +1365,7 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
         RT_CHECK_LAUNCH("softmax16_stream_kernel");
     }
 #undef RT_SP_NS
+#undef RT_SP_RAGGED_NS
 #undef RT_SP_RAGGED
 #undef RT_SP
     *done = true;
@@ -1537,8 +1608,9 @@ extern "C" int rt_softmax_masked(rt_device* dev, int dt, const void* x, const ui
         if (mask_shape[i] != x_shape[i]) whole = false;
         period *= x_shape[i];
     }
-    if (dt != RT_F32 && mode == RT_SOFTMAX_REFERENCE && whole && cols % 8 == 0 && rt_aligned(x, 16) && rt_aligned(y, 16) &&
-        rt_aligned(mask, 16)) {
+    // (rows that are not whole vectors: from RAGGED_STREAM_MIN_COLS columns, like the plain softmax)
+    if (dt != RT_F32 && mode == RT_SOFTMAX_REFERENCE && whole && (cols % 8 == 0 || cols >= RAGGED_STREAM_MIN_COLS) && rt_aligned(x, 16) &&
+        rt_aligned(y, 16) && rt_aligned(mask, 16)) {
         bool done = false;
         rc = dt == RT_F16 ? launch_stream16<half_t>(dev, x, mask, period, y, rows, cols, &done)
                           : launch_stream16<bf16_t>(dev, x, mask, period, y, rows, cols, &done);

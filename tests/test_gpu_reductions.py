@@ -488,6 +488,41 @@ def test_softmax_masked_equals_add_then_softmax(dev, oracle, shape, mshape):
     assert same_bits(dx.to_numpy(), got)
 
 
+@pytest.mark.parametrize("shape,mshape,kind", [((1, 4, 333, 1001), (333, 1001), "f16"), ((2, 3, 77, 199), (1, 1, 77, 199), "f16"),
+                                               ((1, 2, 50, 2047), (50, 2047), "f16"), ((2, 2, 40, 511), (2, 1, 40, 511), "f16"),
+                                               ((1, 8, 9, 193), (1, 1, 1, 193), "f16"), ((1, 2, 30, 4089), (30, 4089), "f16"),
+                                               ((1, 2, 30, 4095), (30, 4095), "f16"), ((1, 3, 1001, 1001), (1, 3, 1001, 1001), "f16"),
+                                               ((1, 4, 250, 1003), (250, 1003), "bf16"), ((2, 2, 31, 1535), (1, 1, 31, 1535), "bf16")])
+def test_softmax_masked_rows_that_are_not_whole_vectors(dev, oracle, shape, mshape, kind):
+    """the one-launch masked softmax on ragged rows (a prompt of 1001 tokens): the mask row that belongs to a row of scores
+    has an alignment of its own, so every mask vector is assembled from two aligned ones; the bits of add-then-softmax.
+    4089 columns are the most that fit the registers with a mask (4095 take two launches)."""
+    rng = np.random.default_rng(323)
+    bf = kind == "bf16"
+    S, T = mshape[-2], mshape[-1]
+    xf = (rng.standard_normal(shape) * 2).astype(np.float32)
+    mf = np.zeros(mshape, np.float32)
+    m2 = mf.reshape(-1, S, T)
+    if S > 1:
+        m2[:] = np.triu(np.full((S, T), -np.inf, np.float32), k=1 + max(T - S, 0))
+        m2[:, S // 2, :] = rng.standard_normal(T).astype(np.float32)
+        m2[:, S - 1, :] = 3 * rng.standard_normal(T).astype(np.float32)
+        m2[:, 0, :9] = rng.standard_normal(9).astype(np.float32)   # finite values in the first elements of the mask (the vector before them does not exist)
+    else:
+        m2[:] = 3 * rng.standard_normal(T).astype(np.float32)
+    x = _bf16(oracle, xf) if bf else xf.astype(np.float16)
+    mask = _bf16(oracle, mf) if bf else mf.astype(np.float16)
+    full_mask = np.ascontiguousarray(np.broadcast_to(mask.reshape((1,) * (4 - mask.ndim) + mask.shape), shape))
+    want = oracle.softmax(oracle.binary("add", x, full_mask, bf16=bf), bf16=bf)
+    isnan = (lambda b: (b & 0x7fff) > 0x7f80) if bf else (lambda b: (b.view(np.uint16) & 0x7fff) > 0x7c00)
+    same = lambda g: not ((g.view(np.uint16) != want.view(np.uint16)) & ~(isnan(g) & isnan(want))).any()
+    dx, dm = dev.upload(x, bf16=bf), dev.upload(mask, bf16=bf)
+    got = dev.softmax_masked(dx, dm).to_numpy()
+    assert same(got), (shape, mshape, kind, int(((got.view(np.uint16) != want.view(np.uint16)) & ~(isnan(got) & isnan(want))).sum()))
+    dev.softmax_masked(dx, dm, out=dx)                                 # in place
+    assert same(dx.to_numpy()), (shape, mshape, kind)
+
+
 @pytest.mark.parametrize("shape,mshape,kind", [((1, 4, 50, 8192), (50, 8192), "f16"), ((2, 2, 33, 4200), (1, 1, 33, 4200), "f16"),
                                                ((1, 8, 128, 512), (128, 512), "bf16"), ((1, 3, 40, 6000), (40, 6000), "bf16")])
 def test_softmax_masked_long_rows_and_bf16(dev, oracle, shape, mshape, kind):
