@@ -181,7 +181,7 @@ int rt_group_norm(rt_device* dev, int dt, const void* x, const void* scale, cons
 /* scores.add(mask).softmax(last dim) in the tensors' own arithmetic (the 16-bit sum is rounded as the separate add
  * rounds it, then Softmax's contract applies), result bit-identical to rt_binary_bcast(RT_ADD) followed by rt_softmax
  * but the sum never reaches memory when the shape allows (f16 or bf16, reference mode, x / y / mask on 16-byte
- * boundaries, rows of whole 16-byte vectors or of 192 to 4089 columns of any length, a mask that covers whole trailing
+ * boundaries, rows of whole 16-byte vectors or of 192 to 4095 columns of any length, a mask that covers whole trailing
  * dims and repeats over the leading ones).  Each mask extent is 1 or the scores' extent; y may be x.
  * Binary: ops/binary.rs:27-119 via tensor.rs:249-280; Softmax: ops/softmax.rs:17-73, cpu/softmax.rs:22-42. */
 int rt_softmax_masked(rt_device* dev, int dt, const void* x, const uint32_t x_shape[4], const void* mask,

@@ -447,7 +447,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
             // one vector is fetched here, at the start of the group, and added after the group's last step.
             uint32_t my_row = 0, tail_end = 0;               // tail_end: bytes of the row inside the extra vector, 0 = none
             bool my_ok = false;
-            v4u tailv = {0, 0, 0, 0};
+            v4u tailv = {0, 0, 0, 0}, tailm = {0, 0, 0, 0};
             if (RAGGED) {
                 uint32_t rep, pg;
                 sp_item(sch, blockIdx.x, gridDim.x, it, rep, pg);
@@ -459,6 +459,14 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                 if (my_ok && end > nsteps * (SP_TC * 2)) {
                     tail_end = end - nsteps * (SP_TC * 2);
                     tailv = *reinterpret_cast<const v4u*>(reinterpret_cast<const char*>(x) + (off & ~15u) + nsteps * (SP_TC * 2));
+                    if (MASK) {                              // its mask elements, one by one (the mask row has its own alignment)
+                        uint32_t q, mrow;
+                        fd_divmod(my_row, sch.pm_div, q, mrow);
+                        const uint16_t* mp = reinterpret_cast<const uint16_t*>(mask) + (uint64_t)mrow * cols + (nsteps * (SP_TC * 2) - (off & 15u)) / 2;
+#pragma unroll
+                        for (int e = 0; e < 7; e++)
+                            if ((uint32_t)(2 * e) < tail_end) tailm[e >> 1] |= (uint32_t)mp[e] << (16 * (e & 1));
+                    }
                 }
             }
 #pragma unroll 1
@@ -483,6 +491,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                 }
             }
             if (RAGGED && tail_end) {
+                if (MASK) tailv = ST::add_vec(tailv, tailm);
 #pragma unroll
                 for (int w = 0; w < 4; w++) {                // elements past the row's end count as +0
                     const uint32_t keep = ((uint32_t)(4 * w) < tail_end ? 0xffffu : 0u) | ((uint32_t)(4 * w + 2) < tail_end ? 0xffff0000u : 0u);
@@ -1246,7 +1255,7 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
     const uint64_t row_bytes = (uint64_t)cols * 2;
     if (!mask) period = rows;
     const bool ragged = cols % 8 != 0;                       // rows over their covering aligned vectors, finished by the edges kernel
-    // with a mask: in one launch only, a mask on a 16-byte boundary, and steps that hold every row's whole span
+    // with a mask: in one launch only, and a mask on a 16-byte boundary
     if (ragged && mask && (!rt_aligned(mask, 16) || rows * row_bytes > 0x7fffffe0ull || rows > RT_SM_ROW_SUMS)) return RT_OK;
     // the kernel addresses a launch with 32-bit byte offsets below 2^31: larger tensors go in chunks of whole periods
     // (whole 30-row groups when nothing repeats)
@@ -1267,9 +1276,8 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
     const uint16_t* table = nullptr;
     int rc = rt_unary_table(dev, TI, RT_EXP, &table);
     if (rc) return rc;
-    // (a ragged row's one vector past its last step is the walker's, which knows no mask: with one, the steps cover it)
-    const uint32_t nt = (cols + (ragged && mask ? 7 : 0) + SP_TC - 1) / SP_TC;
-    if (ragged && nt > SP_MAX_STEPS) return RT_OK;
+    const uint32_t nt = (cols + SP_TC - 1) / SP_TC;
+    if (ragged && nt > SP_MAX_STEPS) return RT_OK;           // (a ragged row's one vector past its last step is the walker's)
     const bool full = !ragged && cols % SP_TC == 0 && (nt == 1 || nt == 2 || nt == 4 || nt == 8);
 #define RT_SP(NS, F, M)                                                                                                              \
     do {                                                                                                                             \
