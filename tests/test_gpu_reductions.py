@@ -135,16 +135,17 @@ def test_softmax_f16_streaming_kernel(dev, oracle, shape):
     assert same_bits(dx.to_numpy(), want)
 
 
-def test_softmax_f16_streaming_kernel_beyond_2_gib(dev, oracle):
+@pytest.mark.parametrize("rows,n,split", [(262140 + 47, 4096, 262140), (262200 + 131, 4095, 262200)])
+def test_softmax_f16_streaming_kernel_beyond_2_gib(dev, oracle, rows, n, split):
     # the kernel addresses a launch with 32-bit byte offsets below 2^31, so a larger tensor is split into row chunks
-    # (262 140 rows of 4096 f16 each); rows on both sides of the split and at the end are compared with the oracle
-    rows, n = 262140 + 47, 4096
+    # (262 140 rows of 4096 f16 each; 262 200 rows of 4095, a multiple of 120 so that the second chunk starts on a 16-byte
+    # boundary); rows on both sides of the split and at the end are compared with the oracle
     rng = np.random.default_rng(304)
     block = randn(rng, (1021, n), np.float16, 2.0)
     block[::3, 1000:] = -np.inf
     x = np.tile(block, (rows // 1021 + 1, 1))[:rows]
     got = dev.softmax(dev.upload(x)).to_numpy()
-    for lo, hi in ((0, 64), (262100, rows)):
+    for lo, hi in ((0, 64), (split - 40, rows)):
         want = oracle.softmax(x[lo:hi])
         assert mismatch_count(got[lo:hi], want) == 0, (lo, hi)
     # every row equals the result of its source row in the repeated block
