@@ -29,6 +29,7 @@ constexpr int BLOCK = 256;
 constexpr int WAVES = BLOCK / WAVE;
 
 enum { NORM_LAYER = 0, NORM_RMS = 1 };
+constexpr int NORM_WIDE_BLOCK = 1024;                   // threads per row for f32 rows that do not fit 256 threads' registers
 
 // per-row statistics in T arithmetic, given f32 sums
 template <typename T> struct RowStats {
@@ -67,10 +68,12 @@ template <typename T, int KIND> __device__ __forceinline__ T norm_one(T x, const
 // written (the row's two ragged vectors are stored element by element), and scale / bias are read by column.  An
 // aligned vector that holds one byte of the tensor lies in a mapped page, so the loads are safe at the tensor's ends too.
 template <typename T, int NV, int KIND, int LANES, bool SPAN>
-__global__ void __launch_bounds__(BLOCK) norm_wave_kernel(const T* x, const T* __restrict__ scale, const T* __restrict__ bias, T* y,
-                                                          uint64_t rows, uint32_t cols, float eps) {
+__global__ void __launch_bounds__(LANES > BLOCK ? LANES : BLOCK) norm_wave_kernel(const T* x, const T* __restrict__ scale,
+                                                                                  const T* __restrict__ bias, T* y, uint64_t rows,
+                                                                                  uint32_t cols, float eps) {
     constexpr int VE = 16 / sizeof(T);
-    const uint64_t row = (uint64_t)blockIdx.x * (BLOCK / LANES) + (threadIdx.x / LANES);
+    constexpr int THREADS = LANES > BLOCK ? LANES : BLOCK;   // rows beyond 2048 vectors: one 1024-thread block per row
+    const uint64_t row = (uint64_t)blockIdx.x * (THREADS / LANES) + (threadIdx.x / LANES);
     if (row >= rows) return;
     const int lane = threadIdx.x & (LANES - 1);
     const uint64_t first = row * cols;
@@ -605,10 +608,11 @@ template <typename T, int KIND>
 int launch_norm(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint64_t rows, uint32_t cols, float eps) {
     constexpr int VE = 16 / sizeof(T);
     const bool io_aligned = rt_aligned(x, 16) && rt_aligned(y, 16);
-    if (io_aligned && cols % VE == 0 && rt_aligned(scale, 16) && (!bias || rt_aligned(bias, 16)) && cols / VE <= (uint32_t)(BLOCK * 8))
+    constexpr uint32_t MAX_VEC = NORM_WIDE_BLOCK * 16;       // 65536 f32 columns
+    if (io_aligned && cols % VE == 0 && rt_aligned(scale, 16) && (!bias || rt_aligned(bias, 16)) && cols / VE <= MAX_VEC)
         return launch_norm_wave<T, KIND, false>(dev, x, scale, bias, y, rows, cols, eps);
     // rows that are not whole vectors (or scale / bias off their alignment): over the aligned vectors that cover each row
-    if (io_aligned && (cols + 2 * VE - 2) / VE <= (uint32_t)(BLOCK * 8))
+    if (io_aligned && (cols + 2 * VE - 2) / VE <= MAX_VEC)
         return launch_norm_wave<T, KIND, true>(dev, x, scale, bias, y, rows, cols, eps);
     RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
     hipLaunchKernelGGL((norm_generic_kernel<T, KIND>), dim3((unsigned)rows), dim3(BLOCK), 0, dev->stream, (const T*)x, (const T*)scale,
@@ -621,8 +625,7 @@ template <typename T, int KIND, bool SPAN>
 int launch_norm_wave(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint64_t rows, uint32_t cols, float eps) {
     constexpr int VE = 16 / sizeof(T);
     const uint32_t nvec = SPAN ? (cols + 2 * VE - 2) / VE : cols / VE;       // SPAN: the most vectors a row can touch
-    const bool vec_ok = true;
-    if (vec_ok && nvec <= 32) {
+    if (nvec <= 32) {
         // rows of at most 32 vectors: a group of 2..32 lanes per row (one vector each), so that a wave carries 2..32 rows
         // and as many bytes as with long rows
         const uint32_t lanes = nvec <= 2 ? 2 : nvec <= 4 ? 4 : nvec <= 8 ? 8 : nvec <= 16 ? 16 : 32;
@@ -639,7 +642,7 @@ int launch_norm_wave(rt_device* dev, const void* x, const void* scale, const voi
         RT_CHECK_LAUNCH("norm_wave_kernel");
         return RT_OK;
     }
-    if (vec_ok && nvec <= (uint32_t)(WAVE * 8)) {
+    if (nvec <= (uint32_t)(WAVE * 8)) {
         const uint32_t nv = (nvec + WAVE - 1) / WAVE;
         const uint64_t blocks = (rows + WAVES - 1) / WAVES;
         RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
@@ -658,9 +661,9 @@ int launch_norm_wave(rt_device* dev, const void* x, const void* scale, const voi
         RT_CHECK_LAUNCH("norm_wave_kernel");
         return RT_OK;
     }
-    if (vec_ok) {                                            // longer rows: the 256 threads of a block share one row
+    RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
+    if (nvec <= (uint32_t)(BLOCK * 8)) {                     // longer rows: the 256 threads of a block share one row
         const uint32_t nv = (nvec + BLOCK - 1) / BLOCK;
-        RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
         const dim3 grid((unsigned)rows), block(BLOCK);
 #define RT_NORM(NVC)                                                                                                                  \
     hipLaunchKernelGGL((norm_wave_kernel<T, NVC, KIND, BLOCK, SPAN>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, \
@@ -670,10 +673,20 @@ int launch_norm_wave(rt_device* dev, const void* x, const void* scale, const voi
         else if (nv <= 6) RT_NORM(6);
         else RT_NORM(8);
 #undef RT_NORM
-        RT_CHECK_LAUNCH("norm_wave_kernel");
-        return RT_OK;
+    } else {                                                 // up to 65536 f32 columns (the caller has checked): 1024 threads share one row
+        const uint32_t nv = (nvec + NORM_WIDE_BLOCK - 1) / NORM_WIDE_BLOCK;
+        const dim3 grid((unsigned)rows), block(NORM_WIDE_BLOCK);
+#define RT_NORM(NVC)                                                                                                                  \
+    hipLaunchKernelGGL((norm_wave_kernel<T, NVC, KIND, NORM_WIDE_BLOCK, SPAN>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, \
+                       (const T*)bias, (T*)y, rows, cols, eps)
+        if (nv <= 4) RT_NORM(4);
+        else if (nv <= 8) RT_NORM(8);
+        else if (nv <= 13) RT_NORM(13);
+        else RT_NORM(16);
+#undef RT_NORM
     }
-    return rt_fail(RT_ERR_SIZE, "norm: row too long for the register-resident kernel");      // not reached: the caller checks the length
+    RT_CHECK_LAUNCH("norm_wave_kernel");
+    return RT_OK;
 }
 
 // 16-bit reference arithmetic, many rows of at most 128 columns (whole aligned vectors): one lane per row.  A block's

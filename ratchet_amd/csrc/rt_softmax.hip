@@ -21,17 +21,21 @@ constexpr int WAVES = BLOCK / WAVE;
 
 template <typename T> __device__ __forceinline__ float stable_exp(float v) { return expf(v); }
 
+constexpr int WIDE_BLOCK = 1024;                        // threads per row for rows that do not fit 256 threads' registers
+
 // ------------------------------------------------------------------------------------------------------------------
 // Row held in registers by the LANES threads that share it: a wave64 (four rows per block) for rows of up to 512
-// vectors, the whole 256-thread block for rows of up to 2048 vectors (8192 f32 / 16384 16-bit columns).
+// vectors, the whole 256-thread block for rows of up to 2048 vectors (8192 f32 / 16384 16-bit columns), a 1024-thread
+// block for rows of up to 16384 vectors (65536 f32 columns: vocabulary-sized rows).
 // Requires 16-byte aligned x and y and at most LANES * NV vectors per row; rows of whole vectors, or (SPAN) any length.
 // MODE 0: reference arithmetic for f32 (exp, tree sum, divide).  MODE 1: stable (max subtraction, f32 accumulate) for
 // any T; results are rounded to T once.
 // ------------------------------------------------------------------------------------------------------------------
 template <typename T, int NV, int MODE, int LANES, bool SPAN>
-__global__ void __launch_bounds__(BLOCK) softmax_wave_kernel(const T* x, T* y, uint64_t rows, uint32_t cols) {
+__global__ void __launch_bounds__(LANES > BLOCK ? LANES : BLOCK) softmax_wave_kernel(const T* x, T* y, uint64_t rows, uint32_t cols) {
     constexpr int VE = 16 / sizeof(T);
-    const uint64_t row = (uint64_t)blockIdx.x * (BLOCK / LANES) + (threadIdx.x / LANES);
+    constexpr int THREADS = LANES > BLOCK ? LANES : BLOCK;   // rows beyond 2048 vectors: one 1024-thread block per row
+    const uint64_t row = (uint64_t)blockIdx.x * (THREADS / LANES) + (threadIdx.x / LANES);
     if (row >= rows) return;
     const int lane = threadIdx.x & (LANES - 1);
     // SPAN (rows that are not whole aligned vectors; x and y 16-byte aligned): the row is handled over the aligned vectors
@@ -1189,7 +1193,7 @@ template <typename T, int MODE, bool SPAN> int launch_wave(rt_device* dev, const
         else if (nv <= 6) RT_SM(6);
         else RT_SM(8);
 #undef RT_SM
-    } else {
+    } else if (nvec <= (uint32_t)(BLOCK * 8)) {
         const uint32_t nv = (nvec + BLOCK - 1) / BLOCK;
         RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax: too many rows");
         const dim3 grid((unsigned)rows), block(BLOCK);
@@ -1199,6 +1203,18 @@ template <typename T, int MODE, bool SPAN> int launch_wave(rt_device* dev, const
         else if (nv <= 6) RT_SM(6);
         else RT_SM(8);
 #undef RT_SM
+    } else {
+        const uint32_t nv = (nvec + WIDE_BLOCK - 1) / WIDE_BLOCK;
+        RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax: too many rows");
+        const dim3 grid((unsigned)rows), block(WIDE_BLOCK);
+#define RT_SM(NVC) hipLaunchKernelGGL((softmax_wave_kernel<T, NVC, MODE, WIDE_BLOCK, SPAN>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols)
+        if (nv <= 4) RT_SM(4);
+        else if (nv <= 8) RT_SM(8);
+        else if constexpr (sizeof(T) == 4) {                 // (16-bit rows hold 8 values per vector: 8 vectors are the registers' limit)
+            if (nv <= 13) RT_SM(13);
+            else RT_SM(16);
+        }
+#undef RT_SM
     }
     RT_CHECK_LAUNCH("softmax_wave_kernel");
     return RT_OK;
@@ -1207,9 +1223,10 @@ template <typename T, int MODE, bool SPAN> int launch_wave(rt_device* dev, const
 template <typename T, int MODE> int launch_f32_style(rt_device* dev, const void* x, void* y, uint64_t rows, uint32_t cols) {
     constexpr int VE = 16 / sizeof(T);
     const bool aligned = rt_aligned(x, 16) && rt_aligned(y, 16);
-    if (aligned && cols % VE == 0 && cols / VE <= (uint32_t)(BLOCK * 8)) return launch_wave<T, MODE, false>(dev, x, y, rows, cols);
+    constexpr uint32_t MAX_VEC = WIDE_BLOCK * (sizeof(T) == 4 ? 16 : 8);     // 65536 columns
+    if (aligned && cols % VE == 0 && cols / VE <= MAX_VEC) return launch_wave<T, MODE, false>(dev, x, y, rows, cols);
     // rows that are not whole vectors: over the aligned vectors that cover each row
-    if (aligned && (cols + 2 * VE - 2) / VE <= (uint32_t)(BLOCK * 8)) return launch_wave<T, MODE, true>(dev, x, y, rows, cols);
+    if (aligned && (cols + 2 * VE - 2) / VE <= MAX_VEC) return launch_wave<T, MODE, true>(dev, x, y, rows, cols);
     RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax: too many rows");
     hipLaunchKernelGGL((softmax_generic_kernel<T, MODE>), dim3((unsigned)rows), dim3(BLOCK), 0, dev->stream, (const T*)x, (T*)y, rows,
                        cols);
