@@ -127,3 +127,36 @@ def test_reindex_random_large(dev, oracle, seed):
                 want = oracle.unary(op, x)
                 bad, mx = oracle.count_not_close(got, want, 1e-3, 1e-3)
                 assert bad == 0, (op, shape, mx)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_ragged_rows_masked_softmax_random(dev, oracle, seed):
+    """16-bit softmax with and without a mask on rows that are not whole vectors: every mask broadcast pattern, mask periods on
+    both sides of the 240 rows where groups stop running across periods, masks at 16-byte offsets inside an allocation"""
+    from ratchet_amd.runtime import BufferView
+    rng = np.random.default_rng(11000 + seed)
+    b, h = int(rng.integers(1, 3)), int(rng.integers(1, 7))
+    s = int(rng.choice([1, 2, 7, 30, 31, 100, 239, 240, 241, 500]))
+    t = int(rng.choice([193, 199, 255, 257, 511, 513, 1001, 1023, 1535, 2047, 2049, 3001, 4095, int(rng.integers(192, 4096))]))
+    shape = (b, h, s, t)
+    bf = bool(rng.integers(0, 2))
+    xf = (rng.standard_normal(shape) * 2).astype(np.float32)
+    x = oracle.cast(xf, np.uint16, dst_bf16=True) if bf else xf.astype(np.float16)
+    dx = dev.upload(x, bf16=bf)
+    isnan = (lambda v: (v & 0x7fff) > 0x7f80) if bf else (lambda v: (v.view(np.uint16) & 0x7fff) > 0x7c00)
+    for mshape in ((1, 1, s, t), (b, 1, s, t), (b, h, s, t), (1, 1, 1, t)):
+        mf = rng.standard_normal(mshape).astype(np.float32)
+        mf[rng.random(mshape) < 0.3] = -np.inf
+        mask = oracle.cast(mf, np.uint16, dst_bf16=True) if bf else mf.astype(np.float16)
+        full = np.ascontiguousarray(np.broadcast_to(mask, shape))
+        want = oracle.softmax(oracle.binary("add", x, full, bf16=bf), bf16=bf)
+        moff = int(rng.choice([0, 8, 16]))
+        mbuf = dev.empty((mask.size + 24,), 2 if bf else 1)
+        mv = BufferView(mbuf, moff, mshape).upload(mask)
+        got = dev.softmax_masked(dx, mv).to_numpy()
+        bad = (got.view(np.uint16) != want.view(np.uint16)) & ~(isnan(got) & isnan(want))
+        assert not bad.any(), (shape, mshape, moff, int(bad.sum()), np.argwhere(bad)[:5])
+    want = oracle.softmax(x, bf16=bf)
+    got = dev.softmax(dx).to_numpy()
+    bad = (got.view(np.uint16) != want.view(np.uint16)) & ~(isnan(got) & isnan(want))
+    assert not bad.any(), (shape, "plain", int(bad.sum()))
