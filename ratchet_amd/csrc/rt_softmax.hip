@@ -1295,10 +1295,10 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
     if (rc) return rc;
     const uint32_t nt = (cols + SP_TC - 1) / SP_TC;
     if (ragged && nt > SP_MAX_STEPS) return RT_OK;           // (a ragged row's one vector past its last step is the walker's)
-    const bool full = !ragged && cols % SP_TC == 0 && (nt == 1 || nt == 2 || nt == 4 || nt == 8);
+    const bool full = !ragged && cols % SP_TC == 0 && (nt == 1 || nt == 2 || nt == 4 || nt == 6 || nt == 8);
 #define RT_SP(NS, F, M)                                                                                                              \
     do {                                                                                                                             \
-        const uint64_t bit = 1ull << (TI * 20 + (NS == 0 ? 4 : NS == 1 ? 0 : NS == 2 ? 1 : NS == 4 ? 2 : 3) * 4 + (F ? 2 : 0) + (M ? 1 : 0)); \
+        const uint64_t bit = 1ull << (TI * 24 + (NS == 0 ? 4 : NS == 1 ? 0 : NS == 2 ? 1 : NS == 4 ? 2 : NS == 6 ? 5 : 3) * 4 + (F ? 2 : 0) + (M ? 1 : 0)); \
         if (!(dev->sp_attr_set & bit)) {               /* the LDS opt-in is per function and per device */                           \
             RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(softmax16_stream_kernel<T, NS, F, M>),                          \
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)SP_SMEM_BYTES));                             \
@@ -1309,11 +1309,11 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
     } while (0)
 #define RT_SP_RAGGED(NS, M)                                                                                                          \
     do {                                                                                                                             \
-        const uint64_t bit = 1ull << (40 + (M ? 8 : 0) + TI * 4 + (NS == 1 ? 0 : NS == 2 ? 1 : NS == 4 ? 2 : 3));                    \
-        if (!(dev->sp_attr_set & bit)) {                                                                                             \
+        const uint64_t bit = 1ull << ((M ? 16 : 0) + TI * 8 + (NS == 1 ? 0 : NS == 2 ? 1 : NS == 4 ? 2 : NS == 6 ? 4 : 3));          \
+        if (!(dev->sp_ragged_attr_set & bit)) {                                                                                      \
             RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(softmax16_stream_kernel<T, NS, false, M, true>),                \
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)SP_SMEM_BYTES));                             \
-            dev->sp_attr_set |= bit;                                                                                                 \
+            dev->sp_ragged_attr_set |= bit;                                                                                              \
         }                                                                                                                            \
         hipLaunchKernelGGL((softmax16_stream_kernel<T, NS, false, M, true>), dim3(blocks), dim3(SP_BLOCK), SP_SMEM_BYTES,            \
                            dev->stream, table, xc, (const T*)mask, yc, n, cols, sch, dev->sm_row_sums);                              \
@@ -1323,6 +1323,7 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
         if (nt <= 1) RT_SP_RAGGED(1, M);                    \
         else if (nt <= 2) RT_SP_RAGGED(2, M);               \
         else if (nt <= 4) RT_SP_RAGGED(4, M);               \
+        else if (nt <= 6) RT_SP_RAGGED(6, M);               \
         else RT_SP_RAGGED(8, M);                            \
     } while (0)
 #define RT_SP_NS(F, M)                                      \
@@ -1330,6 +1331,7 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
         if (nt <= 1) RT_SP(1, F, M);                        \
         else if (nt <= 2) RT_SP(2, F, M);                   \
         else if (nt <= 4) RT_SP(4, F, M);                   \
+        else if (nt <= 6) RT_SP(6, F, M);                   \
         else RT_SP(8, F, M);                                \
     } while (0)
     for (uint64_t row0 = 0; row0 < rows; row0 += chunk_rows) {
