@@ -706,7 +706,10 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
     uint32_t gpar = 0;
 
     if constexpr (PARK) {
-        constexpr int PF = NSTEP < SP_PF ? NSTEP : SP_PF;    // steps of x in flight per thread
+        // steps of x in flight per thread: two, or the whole row when the step count is odd (the slot of step t is t % PF in
+        // every group, so PF has to divide the step count)
+        constexpr int PF = NSTEP % SP_PF == 0 ? SP_PF : NSTEP;
+        static_assert(NSTEP % PF == 0 && PF <= 5, "prefetch slots must tile the steps of a row");
         v4u e[NSTEP][2];                                     // exp values of the group in flight, 8 halves per vector
         v4u pre[PF][2], mpre[2];                             // x: PF steps in flight; mask: one (L2 hits: a short distance is enough)
         v4u mhi[2];                                          // RAGGED: lane 63's second mask vector
@@ -1295,10 +1298,10 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
     if (rc) return rc;
     const uint32_t nt = (cols + SP_TC - 1) / SP_TC;
     if (ragged && nt > SP_MAX_STEPS) return RT_OK;           // (a ragged row's one vector past its last step is the walker's)
-    const bool full = !ragged && cols % SP_TC == 0 && (nt == 1 || nt == 2 || nt == 4 || nt == 6 || nt == 8);
+    const bool full = !ragged && cols % SP_TC == 0 && nt != 7 && nt <= 8;
 #define RT_SP(NS, F, M)                                                                                                              \
     do {                                                                                                                             \
-        const uint64_t bit = 1ull << (TI * 24 + (NS == 0 ? 4 : NS == 1 ? 0 : NS == 2 ? 1 : NS == 4 ? 2 : NS == 6 ? 5 : 3) * 4 + (F ? 2 : 0) + (M ? 1 : 0)); \
+        const uint64_t bit = 1ull << (TI * 32 + (NS == 0 ? 4 : NS == 1 ? 0 : NS == 2 ? 1 : NS == 4 ? 2 : NS == 6 ? 5 : NS == 3 ? 6 : NS == 5 ? 7 : 3) * 4 + (F ? 2 : 0) + (M ? 1 : 0)); \
         if (!(dev->sp_attr_set & bit)) {               /* the LDS opt-in is per function and per device */                           \
             RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(softmax16_stream_kernel<T, NS, F, M>),                          \
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)SP_SMEM_BYTES));                             \
@@ -1309,7 +1312,7 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
     } while (0)
 #define RT_SP_RAGGED(NS, M)                                                                                                          \
     do {                                                                                                                             \
-        const uint64_t bit = 1ull << ((M ? 16 : 0) + TI * 8 + (NS == 1 ? 0 : NS == 2 ? 1 : NS == 4 ? 2 : NS == 6 ? 4 : 3));          \
+        const uint64_t bit = 1ull << ((M ? 16 : 0) + TI * 8 + (NS == 1 ? 0 : NS == 2 ? 1 : NS == 4 ? 2 : NS == 6 ? 4 : NS == 3 ? 5 : NS == 5 ? 6 : 3)); \
         if (!(dev->sp_ragged_attr_set & bit)) {                                                                                      \
             RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(softmax16_stream_kernel<T, NS, false, M, true>),                \
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)SP_SMEM_BYTES));                             \
@@ -1322,7 +1325,9 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
     do {                                                    \
         if (nt <= 1) RT_SP_RAGGED(1, M);                    \
         else if (nt <= 2) RT_SP_RAGGED(2, M);               \
+        else if (nt <= 3) RT_SP_RAGGED(3, M);               \
         else if (nt <= 4) RT_SP_RAGGED(4, M);               \
+        else if (nt <= 5) RT_SP_RAGGED(5, M);               \
         else if (nt <= 6) RT_SP_RAGGED(6, M);               \
         else RT_SP_RAGGED(8, M);                            \
     } while (0)
@@ -1330,7 +1335,9 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
     do {                                                    \
         if (nt <= 1) RT_SP(1, F, M);                        \
         else if (nt <= 2) RT_SP(2, F, M);                   \
+        else if (nt <= 3) RT_SP(3, F, M);                   \
         else if (nt <= 4) RT_SP(4, F, M);                   \
+        else if (nt <= 5) RT_SP(5, F, M);                   \
         else if (nt <= 6) RT_SP(6, F, M);                   \
         else RT_SP(8, F, M);                                \
     } while (0)
