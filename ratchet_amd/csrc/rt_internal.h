@@ -96,6 +96,12 @@ int rt_enter(rt_device* dev);
 // built on first use by running the exact unary kernel over all bit patterns (blocks until the table is ready).
 int rt_unary_table(rt_device* dev, int type_index, int op, const uint16_t** out);
 
+// The streaming 16-bit softmax (rt_softmax_stream_f16.hip / rt_softmax_stream_bf16.hip).  mask == nullptr: plain softmax;
+// otherwise the mask has `period` rows of `cols` columns and repeats every `period` rows of x.  Returns RT_OK with
+// *done = false when the shape does not fit the kernel (the caller then takes another path).
+int rt_softmax_stream_f16(rt_device* dev, const void* x, const void* mask, uint64_t period, void* y, uint64_t rows, uint32_t cols, bool* done);
+int rt_softmax_stream_bf16(rt_device* dev, const void* x, const void* mask, uint64_t period, void* y, uint64_t rows, uint32_t cols, bool* done);
+
 // ---------------------------------------------------------------------------------------------------------
 // u32 division by a launch-time constant: q = (n * m) >> (32 + s), exact for all n < 2^32 (round-up method)
 // ---------------------------------------------------------------------------------------------------------
