@@ -362,11 +362,8 @@ __global__ void __launch_bounds__(BLOCK) norm_seq16_kernel(const T* __restrict__
 // and raises its issue priority; the four loader waves fetch one 16-byte vector per thread per tile two tiles ahead,
 // widen x and T(x*x) to f32 and park them in double-buffered LDS tiles; one barrier per tile.  The kernel runs at the
 // speed of the dependent v_add_f32 chain (about 3 ns per column on this chip).
-// KEEP > 0 (rows of at most KEEP tiles): a loader thread keeps the vectors it fetched (one per tile, 4 registers each) and
-// produces the outputs from them once the row statistics are known, so x is read once; KEEP == 0 reads the row again.
 constexpr int NP_BLOCK = 320;
-constexpr int NP_KEEP = 16;                  // 4096 columns
-template <typename T, int KIND, int KEEP>
+template <typename T, int KIND>
 __global__ void __launch_bounds__(NP_BLOCK) norm_pipe16_kernel(const T* __restrict__ x, const T* __restrict__ scale,
                                                                const T* __restrict__ bias, T* __restrict__ y, uint64_t rows, uint32_t cols,
                                                                float eps) {
@@ -462,66 +459,6 @@ __global__ void __launch_bounds__(NP_BLOCK) norm_pipe16_kernel(const T* __restri
         __syncthreads();
     };
 
-    if constexpr (KEEP > 0) {
-        v4u kept[KEEP];
-#pragma unroll
-        for (int t = 0; t < KEEP; t++) kept[t] = v4u{0, 0, 0, 0};
-        issue(0, kept[0]);
-        if (KEEP > 1) issue(1, kept[KEEP > 1 ? 1 : 0]);
-#pragma unroll
-        for (int t = 0; t < KEEP; t++) {
-            if ((uint32_t)t < ntiles) {                                         // the same for every thread: the barriers stay matched
-                const uint32_t buf = t & 1;
-                const uint32_t col = t * TC + cv * 8;
-                if (rvalid) {
-                    float sq[8], xv[8];
-                    if (col < cols) {
-                        Vec16<T> in;
-                        in.u = kept[t];
-#pragma unroll
-                        for (int q = 0; q < 8; q++) {
-                            sq[q] = Ar<T>::widen(Ar<T>::mul(in.e[q], in.e[q]));
-                            xv[q] = Ar<T>::widen(in.e[q]);
-                        }
-                    } else {
-#pragma unroll
-                        for (int q = 0; q < 8; q++) sq[q] = xv[q] = 0.0f;
-                    }
-                    float4* d0 = reinterpret_cast<float4*>(&tile[buf][0][r][cv * 8]);
-                    d0[0] = make_float4(sq[0], sq[1], sq[2], sq[3]);
-                    d0[1] = make_float4(sq[4], sq[5], sq[6], sq[7]);
-                    if (KIND == NORM_LAYER) {
-                        float4* d1 = reinterpret_cast<float4*>(&tile[buf][NSUM - 1][r][cv * 8]);
-                        d1[0] = make_float4(xv[0], xv[1], xv[2], xv[3]);
-                        d1[1] = make_float4(xv[4], xv[5], xv[6], xv[7]);
-                    }
-                }
-                if (t + 2 < KEEP) issue(t + 2, kept[t + 2 < KEEP ? t + 2 : 0]);
-                __syncthreads();
-            }
-        }
-        __syncthreads();                                                        // sums published (wave 0 finishes the stats)
-        __syncthreads();                                                        // row statistics published
-        if (!rvalid) return;
-        RowStats<T> st;
-        st.mu = s_mu[r];
-        st.r = s_r[r];
-        T* yrow = y + (row0 + r) * cols;
-#pragma unroll
-        for (int t = 0; t < KEEP; t++) {
-            const uint32_t c = t * (TC / 8) + cv;                               // vector index within the row
-            if (c * 8 < cols) {
-                Vec16<T> in, sc, bi, out;
-                in.u = kept[t];
-                sc.u = reinterpret_cast<const v4u*>(scale)[c];
-                if (KIND == NORM_LAYER && bias) bi.u = reinterpret_cast<const v4u*>(bias)[c];
-#pragma unroll
-                for (int q = 0; q < 8; q++) out.e[q] = norm_one<T, KIND>(in.e[q], st, sc.e[q], bi.e[q], bias != nullptr);
-                st_stream(reinterpret_cast<v4u*>(yrow) + c, out.u);
-            }
-        }
-        return;
-    }
     issue(0, pre0);
     issue(1, pre1);
     for (uint32_t t = 0; t < ntiles; t += 2) {
@@ -839,13 +776,8 @@ int launch_norm16(rt_device* dev, const void* x, const void* scale, const void* 
     if (vec_ok) {
         const uint64_t blocks = (rows + 7) / 8;
         RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
-        if (cols <= 256u * NP_KEEP) {
-            hipLaunchKernelGGL((norm_pipe16_kernel<T, KIND, NP_KEEP>), dim3((unsigned)blocks), dim3(NP_BLOCK), 0, dev->stream, (const T*)x,
-                               (const T*)scale, (const T*)bias, (T*)y, rows, cols, eps);
-        } else {
-            hipLaunchKernelGGL((norm_pipe16_kernel<T, KIND, 0>), dim3((unsigned)blocks), dim3(NP_BLOCK), 0, dev->stream, (const T*)x,
-                               (const T*)scale, (const T*)bias, (T*)y, rows, cols, eps);
-        }
+        hipLaunchKernelGGL((norm_pipe16_kernel<T, KIND>), dim3((unsigned)blocks), dim3(NP_BLOCK), 0, dev->stream, (const T*)x, (const T*)scale,
+                           (const T*)bias, (T*)y, rows, cols, eps);
         RT_CHECK_LAUNCH("norm_pipe16_kernel");
         return RT_OK;
     }
