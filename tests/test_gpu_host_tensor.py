@@ -263,6 +263,34 @@ def test_caller_patterns_resolve_in_one_launch(hdev, oracle):
     assert same_bits(fused["glu"][0], want)
 
 
+def test_masked_softmax_on_a_prompt_of_odd_length_is_one_launch(hdev, oracle):
+    """scores.add(mask).softmax(3) in f16 with 1001 tokens (rows that are not whole 16-byte vectors): still folded into
+    one launch, still the bits of the two separate ops; the f32-intermediate attention pattern on the same shape too"""
+    from ratchet_amd import _lib
+    from ratchet_amd.host import set_pattern_fusion
+
+    rng = np.random.default_rng(409)
+    S, H = 1001, 3
+    scores = (2 * rng.standard_normal((1, H, S, S))).astype(np.float16)
+    mask = np.triu(np.full((S, S), -np.inf, np.float16), k=1)
+    full_mask = np.ascontiguousarray(np.broadcast_to(mask, scores.shape))
+    g = T(scores, hdev).add(T(mask, hdev)).softmax(3).resolve()
+    assert g.last_resolve_launches() == 1
+    want = oracle.softmax(oracle.binary("add", scores, full_mask))
+    assert same_bits(g.to_numpy(), want)
+    set_pattern_fusion(False)
+    try:
+        plain = T(scores, hdev).add(T(mask, hdev)).softmax(3).resolve()
+        assert plain.last_resolve_launches() == 2 and same_bits(plain.to_numpy(), want)
+    finally:
+        set_pattern_fusion(True)
+    g32 = T(scores, hdev).add(T(mask, hdev)).full().softmax(3).cast(_lib.F16).resolve()
+    assert g32.last_resolve_launches() == 1
+    want32 = oracle.cast(oracle.softmax(oracle.cast(oracle.binary("add", scores, full_mask), np.float32)), np.float16)
+    ok, info = close(oracle, g32.to_numpy(), want32, 1e-3)
+    assert ok, info
+
+
 def test_pattern_with_a_visible_intermediate_is_not_folded(hdev, oracle):
     from ratchet_amd import _lib
 
