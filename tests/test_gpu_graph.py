@@ -81,6 +81,39 @@ def test_replays_match_eager_execution(dev, oracle):
     assert same_bits(got_ln, ln.to_numpy())
 
 
+def test_replays_of_ragged_row_softmax_match_eager_execution(dev, oracle):
+    """rows that are not whole vectors: the streaming softmax leaves every row's sum in a buffer owned by the device and a second
+    launch finishes the vectors shared by two rows; two such softmaxes (plain and masked) in one graph use that buffer one
+    after the other, replay after replay"""
+    rng = np.random.default_rng(802)
+    a = randn(rng, (1, 4, 333, 1001), np.float16, 2.0)
+    b = randn(rng, (2, 2, 70, 513), np.float16, 2.0)
+    mask = np.triu(np.full((70, 513), -np.inf, np.float16), k=444)
+    f = randn(rng, (3, 50, 1499), np.float32, 2.0)
+    da, db, dm, df = (dev.upload(v) for v in (a, b, mask, f))
+    ya, yb, yf = dev.empty(a.shape, F16), dev.empty(b.shape, F16), dev.empty(f.shape, F32)
+
+    def sequence():
+        dev.softmax(da, out=ya)
+        dev.softmax_masked(db, dm, out=yb)
+        dev.softmax(df, out=yf)
+
+    sequence()
+    want = [o.to_numpy() for o in (ya, yb, yf)]
+    assert same_bits(want[0], oracle.softmax(a))
+    assert same_bits(want[1], oracle.softmax(oracle.binary("add", b, np.ascontiguousarray(np.broadcast_to(mask, b.shape)))))
+    with dev.capture() as cap:
+        sequence()
+    for replay in range(3):
+        for o in (ya, yb, yf):
+            o.zero_()
+        cap.launch()
+        for k, (o, w) in enumerate(zip((ya, yb, yf), want)):
+            assert same_bits(o.to_numpy(), w), (replay, k)
+        dev.softmax(db, out=yb)                                # eager use of the same row-sum buffer between replays
+        dev.sync()
+
+
 def test_calls_that_cannot_be_captured_say_so(dev):
     from ratchet_amd import RatchetError
 
