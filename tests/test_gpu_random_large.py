@@ -160,3 +160,87 @@ def test_ragged_rows_masked_softmax_random(dev, oracle, seed):
     got = dev.softmax(dx).to_numpy()
     bad = (got.view(np.uint16) != want.view(np.uint16)) & ~(isnan(got) & isnan(want))
     assert not bad.any(), (shape, "plain", int(bad.sum()))
+
+
+@pytest.mark.parametrize("seed", range(9))
+def test_f32_rows_random_large(dev, oracle, seed):
+    """f32 softmax, norms and unaries over thousands of rows, tens of thousands of narrow rows and rows of up to 20000 columns
+    (most of them not whole vectors).  Layer norm is held to 1e-4 here: the reference's one-pass variance amplifies the
+    rounding of the sums by mean^2 / variance, and among a few hundred thousand random short rows some are ill conditioned."""
+    rng = np.random.default_rng(8000 + seed)
+    kind = seed % 3
+    if kind == 0:
+        shape = (int(rng.integers(200, 6000)), int(rng.integers(1, 600)) * 4)
+    elif kind == 1:
+        shape = (int(rng.integers(20000, 70000)), int(rng.integers(1, 40)))
+    else:
+        shape = (int(rng.integers(1, 300)), int(rng.integers(1, 20000)))
+    while np.prod(shape) > 12_000_000:
+        shape = (max(1, shape[0] // 2), shape[1])
+    x = randn(rng, shape, np.float32, 2.0)
+    dx = dev.upload(x)
+    got = dev.softmax(dx).to_numpy()
+    bad, mx = oracle.count_not_close(got, oracle.softmax(x), 1e-5, 1e-5)
+    assert bad == 0, ("softmax", shape, mx)
+    cols = shape[-1]
+    w, b = randn(rng, (cols,), np.float32), randn(rng, (cols,), np.float32)
+    got = dev.layer_norm(dx, dev.upload(w), dev.upload(b), 1e-5).to_numpy()
+    bad, mx = oracle.count_not_close(got, oracle.layer_norm(x, w, b, 1e-5, intended=True), 1e-4, 1e-4)
+    assert bad == 0 or cols < 3, ("ln", shape, mx)
+    got = dev.rms_norm(dx, dev.upload(w), 1e-5).to_numpy()
+    bad, mx = oracle.count_not_close(got, oracle.rms_norm(x, w, 1e-5, intended=True), 1e-5, 1e-5)
+    assert bad == 0, ("rms", shape, mx)
+    for op in ("gelu", "tanh", "exp", "silu", "sigmoid", "sqrt", "neg", "abs", "relu", "log", "sin", "cos", "floor", "ceil"):
+        want = oracle.unary(op, x)
+        got = dev.unary(op, dx).to_numpy()
+        bad, mx = oracle.count_not_close(got, want, 1e-5, 1e-5)
+        assert bad == 0, (op, shape, mx)
+
+@pytest.mark.parametrize("seed", range(8))
+def test_group_norm_and_cache_random(dev, oracle, seed):
+    rng = np.random.default_rng(8100 + seed)
+    for dtype, tol in ((np.float32, 1e-4), (np.float16, 2e-3)):
+        B, G = int(rng.integers(1, 4)), int(rng.choice([1, 2, 4, 8, 32]))
+        cpg, L = int(rng.integers(1, 9)), int(rng.integers(1, 5000))
+        C = G * cpg
+        x = randn(rng, (B, C, L), dtype)
+        w, b = randn(rng, (C,), dtype), randn(rng, (C,), dtype)
+        got = dev.group_norm(dev.upload(x), G, dev.upload(w), dev.upload(b), 1e-5).to_numpy()
+        want = oracle.group_norm(x, G, w, b, 1e-5)
+        bad, mx = oracle.count_not_close(got, want, tol, tol)
+        assert bad == 0, ("gn", B, C, L, G, dtype.__name__, mx)
+        # cache
+        bb, h, T, hd = int(rng.integers(1, 3)), int(rng.integers(1, 9)), int(rng.integers(4, 600)), int(rng.choice([8, 64, 80, 96, 128, 100]))
+        n = int(rng.integers(1, T))
+        off = int(rng.integers(0, T - n + 1))
+        c, s = randn(rng, (bb, h, T, hd), dtype), randn(rng, (bb, h, n, hd), dtype)
+        dc = dev.upload(c)
+        got = dev.cache(dc, dev.upload(s), 2, off).to_numpy()
+        c2 = c.copy()
+        want = oracle.cache(c2, s, 2, off)
+        assert same_bits(got, want) and same_bits(dc.to_numpy(), c2), ("cache", c.shape, n, off)
+
+@pytest.mark.parametrize("seed", range(8))
+def test_binary_broadcast_random_large(dev, oracle, seed):
+    rng = np.random.default_rng(8200 + seed)
+    pool = [1, 2, 3, 5, 8, 12, 32, 50, 64, 80, 128, 200, 256, 1000, 1001, 2560]
+    for _ in range(8):
+        dtype = (np.float32, np.float16)[int(rng.integers(0, 2))]
+        rank = int(rng.integers(1, 5))
+        while True:
+            out = tuple(int(rng.choice(pool)) for _ in range(rank))
+            if np.prod(out) < 8_000_000:
+                break
+        sa = tuple(s if rng.random() < 0.7 else 1 for s in out)
+        sb = tuple(s if (rng.random() < 0.7 or sa[i] == 1) else 1 for i, s in enumerate(out))
+        if rng.random() < 0.3:
+            sb = tuple(sb[int(rng.integers(0, rank)):]) or (1,)
+        try:
+            oshape = np.broadcast_shapes(sa, sb)
+        except ValueError:
+            continue
+        a, b = randn(rng, sa, dtype), randn(rng, sb, dtype)
+        op = ("add", "sub", "mul", "div")[int(rng.integers(0, 4))]
+        want = oracle.binary(op, np.ascontiguousarray(np.broadcast_to(a, oshape)), np.ascontiguousarray(np.broadcast_to(b, oshape)))
+        got = dev.binary(op, dev.upload(a), dev.upload(b)).to_numpy()
+        assert got.shape == tuple(oshape) and same_bits(got, want), (op, sa, sb)
