@@ -16,7 +16,11 @@
  *   binary, cast, reindex, concat ........ numpy / IEEE-754 closed forms, bit-exact
  *   unary f32 ............................ torch / float64 evaluation at the reference's tolerances
  *   unary f16 ............................ exhaustive (65536 inputs) against a numpy float16 model
- *   softmax, layer_norm, rms_norm ........ torch at the reference's own tolerances + invariants
+ *   softmax, layer_norm, rms_norm ........ torch at the reference's own tolerances + invariants; the f16 and bf16 paths
+ *                                          bit for bit against step-wise numpy models (float16 / bit-rounded bfloat16
+ *                                          arithmetic, left-to-right float32 sums, libm expf), with variants that drop a
+ *                                          rounding point or reorder a step shown to disagree
+ *   unary bf16 (gelu, silu, sigmoid, exp, tanh)  all 65536 inputs, bit for bit, against the same kind of model
  *   group_norm ........................... torch F.group_norm (the reference CPU path is a no-op)
  *   cache, index_select, index_write ..... numpy concatenate / take / flat assignment and the reference's own test cases
  *   rope ................................. float64 closed form of the half-rotation RoPE (what the reference's mlx ground
