@@ -29,6 +29,7 @@ constexpr int BLOCK = 256;
 constexpr int WAVES = BLOCK / WAVE;
 
 enum { NORM_LAYER = 0, NORM_RMS = 1 };
+
 constexpr int NORM_WIDE_BLOCK = 1024;                   // threads per row for f32 rows that do not fit 256 threads' registers
 
 // per-row statistics in T arithmetic, given f32 sums
@@ -877,6 +878,69 @@ __global__ void __launch_bounds__(GN_LDS_BLOCK) gn_lds_kernel(const T* __restric
     }
 }
 
+// Fewer (batch, group) pairs than half the CUs (32 groups of 96 KB on 256 CUs): `slices` blocks per group, all in one
+// launch and without any wait between blocks.  Every block of a group loads the WHOLE group into registers (thread t holds
+// vectors t, t + 1024, ...; NV of them) and reduces it to the same mean and variance in the same order, so the blocks of
+// a group agree bit for bit without exchanging anything; each then normalises and stores only its own run of
+// nvec / slices vectors.  The repeated reads of a group hit the L2 of the XCD its blocks share (see the block -> (group,
+// slice) map in launch_gn), so HBM still sees the group once.  Same definitions as gn_lds_kernel.
+template <typename T, int NV>
+__global__ void __launch_bounds__(GN_LDS_BLOCK) gn_reg_kernel(const T* __restrict__ x, const T* __restrict__ scale, const T* __restrict__ bias,
+                                                              T* __restrict__ y, uint32_t glen, uint32_t cpg, uint32_t groups, FastDiv L,
+                                                              float eps, uint32_t slices, uint32_t per_xcd) {
+    constexpr int VE = 16 / sizeof(T);
+    // blocks are handed to the 8 XCDs round robin: pair index p runs over the (group, slice) pairs of one XCD first
+    const uint32_t p = per_xcd ? (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3) : blockIdx.x;
+    const uint32_t grp = p / slices, slice = p - grp * slices, g = grp % groups;
+    const v4u* xs = reinterpret_cast<const v4u*>(x + (uint64_t)grp * glen);
+    v4u* ys = reinterpret_cast<v4u*>(y + (uint64_t)grp * glen);
+    const uint32_t nvec = glen / VE;
+    Vec16<T> v[NV];
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        const uint32_t i = threadIdx.x + k * GN_LDS_BLOCK;
+        v[k].u = v4u{0u, 0u, 0u, 0u};
+        if (i < nvec) v[k].u = xs[i];
+    }
+    float acc = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+#pragma unroll
+        for (int q = 0; q < VE; q++) acc += Ar<T>::widen(v[k].e[q]);         // vectors past the group hold zeros
+    }
+    const float mean = row_sum<GN_LDS_BLOCK>(acc) / (float)glen;
+    float m2 = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        if (threadIdx.x + k * GN_LDS_BLOCK < nvec) {
+#pragma unroll
+            for (int q = 0; q < VE; q++) {
+                const float d = Ar<T>::widen(v[k].e[q]) - mean;
+                m2 += d * d;
+            }
+        }
+    }
+    const float var = row_sum<GN_LDS_BLOCK>(m2) / (float)glen;
+    const float rstd = 1.0f / __builtin_sqrtf(var + eps);
+    const uint32_t lo = (uint32_t)(((uint64_t)nvec * slice) / slices), hi = (uint32_t)(((uint64_t)nvec * (slice + 1)) / slices);
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        const uint32_t i = threadIdx.x + k * GN_LDS_BLOCK;
+        if (i >= lo && i < hi) {
+            const uint32_t c = g * cpg + fd_div(i * VE, L);                  // L % VE == 0: one channel per vector
+            const float w = scale ? Ar<T>::widen(scale[c]) : 1.0f;
+            const float b = bias ? Ar<T>::widen(bias[c]) : 0.0f;
+            Vec16<T> o;
+#pragma unroll
+            for (int q = 0; q < VE; q++) {
+                const float t = (Ar<T>::widen(v[k].e[q]) - mean) * rstd;
+                o.e[q] = Ar<T>::conv(t * w + b);
+            }
+            st_stream(ys + i, o.u);
+        }
+    }
+}
+
 // Many slices per group (few, very large groups): the partials of a group are combined once, by one block, into a
 // single (mean, M2, count) triple that the apply kernel then reads as if the group had one slice.
 __global__ void __launch_bounds__(BLOCK) gn_combine_kernel(const float* __restrict__ part, float* __restrict__ out, uint32_t splits) {
@@ -926,6 +990,31 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
     if (splits < 1) splits = 1;
     constexpr int VEMAX = 16 / sizeof(T);
     const bool vec = (L % VEMAX == 0) && rt_aligned(x, 16) && rt_aligned(y, 16);       // then glen % VEMAX == 0 too
+    if (vec && (size_t)glen * sizeof(T) <= GN_LDS_MAX_BYTES && 2u * bg <= (uint32_t)dev->num_cus) {
+        // few groups: several blocks per group, each reducing the whole group and writing one slice of it
+        uint32_t slices = (uint32_t)dev->num_cus / bg;
+        if (slices > 32) slices = 32;
+        const uint32_t nvec = glen / VEMAX;
+        if (slices > nvec) slices = nvec;
+        const uint32_t blocks = bg * slices;
+        // with a block count that the 8 XCDs share evenly, block b (on XCD b % 8) takes pair (b % 8) * blocks / 8 + b / 8, which
+        // puts the slices of a group on one XCD (all of them when bg is a multiple of 8)
+        const uint32_t per_xcd = blocks % 8 == 0 ? blocks / 8 : 0;
+        const uint32_t nv = (nvec + GN_LDS_BLOCK - 1) / GN_LDS_BLOCK;
+        const dim3 grid(blocks), block(GN_LDS_BLOCK);
+#define RT_GN_REG(NVC)                                                                                                                      \
+    hipLaunchKernelGGL((gn_reg_kernel<T, NVC>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, (T*)y, glen, cpg, \
+                       groups, make_fastdiv(L), eps, slices, per_xcd)
+        if (nv <= 1) RT_GN_REG(1);
+        else if (nv <= 2) RT_GN_REG(2);
+        else if (nv <= 3) RT_GN_REG(3);
+        else if (nv <= 4) RT_GN_REG(4);
+        else if (nv <= 6) RT_GN_REG(6);
+        else RT_GN_REG(9);
+#undef RT_GN_REG
+        RT_CHECK_LAUNCH("gn_reg_kernel");
+        return RT_OK;
+    }
     if (vec && (size_t)glen * sizeof(T) <= GN_LDS_MAX_BYTES && bg <= 2u * (uint32_t)dev->num_cus) {
         const int ti = sizeof(T) == 4 ? 0 : (std::is_same<T, half_t>::value ? 1 : 2);
         if (!(dev->gn_lds_attr_set & (1u << ti))) {
@@ -953,14 +1042,15 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
     }
     const dim3 grid(bg, splits), block(BLOCK);
     const bool separate = splits > FUSED_COMBINE_MAX;
-    const float* stats = separate ? dev->gn_scratch + (size_t)bg * splits * 3 : dev->gn_scratch;
+    float* const part = dev->gn_scratch;
+    const float* stats = separate ? part + (size_t)bg * splits * 3 : part;
     const uint32_t stat_splits = separate ? 1 : splits;
-    if (vec) hipLaunchKernelGGL((gn_stats_kernel<T, VEMAX>), grid, block, 0, dev->stream, (const T*)x, dev->gn_scratch, glen, chunk, splits);
-    else hipLaunchKernelGGL((gn_stats_kernel<T, 1>), grid, block, 0, dev->stream, (const T*)x, dev->gn_scratch, glen, chunk, splits);
+    if (vec) hipLaunchKernelGGL((gn_stats_kernel<T, VEMAX>), grid, block, 0, dev->stream, (const T*)x, part, glen, chunk, splits);
+    else hipLaunchKernelGGL((gn_stats_kernel<T, 1>), grid, block, 0, dev->stream, (const T*)x, part, glen, chunk, splits);
     RT_CHECK_LAUNCH("gn_stats_kernel");
     if (separate) {
-        hipLaunchKernelGGL(gn_combine_kernel, dim3(bg), block, 0, dev->stream, (const float*)dev->gn_scratch,
-                           dev->gn_scratch + (size_t)bg * splits * 3, splits);
+        hipLaunchKernelGGL(gn_combine_kernel, dim3(bg), block, 0, dev->stream, (const float*)part,
+                           part + (size_t)bg * splits * 3, splits);
         RT_CHECK_LAUNCH("gn_combine_kernel");
     }
     if (vec) {
