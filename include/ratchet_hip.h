@@ -178,6 +178,17 @@ int rt_rms_norm(rt_device* dev, int dt, const void* x, const void* scale, void* 
 int rt_group_norm(rt_device* dev, int dt, const void* x, const void* scale, const void* bias, void* y, uint32_t B,
                   uint32_t C, uint32_t L, uint32_t groups, float eps);
 
+/* rt_group_norm for callers that cannot allocate (code recorded into a HIP graph, tight serving loops, harnesses that
+ * forbid hipMalloc).  No counterpart in the reference.  Same arguments, same results bit for bit, but the partial
+ * statistics of groups that are split over several blocks go to a fixed 256 KiB array that lives in the library's code
+ * object (one copy per GPU, held until the process ends) instead of the device's growable buffer, and the call never
+ * reaches hipMalloc / hipFree.  A problem whose partials do not fit (more than about 10 900 (batch, group) pairs that
+ * each exceed 144 KB) returns RT_ERR_SIZE.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU
+ * (two rt_devices with the same ordinal, or a replaying graph next to an eager call) race; calls on one rt_device are
+ * ordered by its stream.  Nothing in the array has to start at zero: each launch writes every partial it reads. */
+int rt_group_norm_static(rt_device* dev, int dt, const void* x, const void* scale, const void* bias, void* y, uint32_t B,
+                         uint32_t C, uint32_t L, uint32_t groups, float eps);
+
 /* scores.add(mask).softmax(last dim) in the tensors' own arithmetic (the 16-bit sum is rounded as the separate add
  * rounds it, then Softmax's contract applies), result bit-identical to rt_binary_bcast(RT_ADD) followed by rt_softmax
  * but the sum never reaches memory when the shape allows (f16 or bf16, reference mode, x / y / mask on 16-byte

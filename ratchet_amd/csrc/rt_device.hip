@@ -136,6 +136,15 @@ int rt_device_create(int ordinal, rt_device** out) {
         delete dev;
         return rt_fail_hip(e, "hipMalloc(row sums)");
     }
+    int rc = rt_norm_device_init(dev);
+    if (rc) {
+        (void)hipFree(dev->sm_row_sums);
+        (void)hipFree(dev->gn_scratch);
+        (void)hipStreamDestroy(dev->stream);
+        delete dev->pool;
+        delete dev;
+        return rc;
+    }
     *out = dev;
     return RT_OK;
 }

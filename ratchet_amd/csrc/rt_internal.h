@@ -17,6 +17,8 @@ struct rt_device {
     // GroupNorm partial statistics: {mean, m2, count} triples, one per (group, split)
     float* gn_scratch;
     size_t gn_scratch_bytes;
+    // this device's copy of the fixed partial-statistics array behind rt_group_norm_static (rt_norm.hip), resolved at create
+    float* gn_static_ptr;
     // 65536-entry 16-bit -> 16-bit lookup tables, built on first use by the exact kernels ([0] = f16, [1] = bf16)
     uint16_t* unary_lut[2][RT_UNARY_COUNT];
     // the same for "widen to f32, f32 op, round once" (the full -> op -> cast caller pattern)
@@ -91,6 +93,9 @@ static const uint64_t RT_MAX_NUMEL = 1ull << 40;
 
 // Makes dev's ordinal current.  Every entry point calls it first.
 int rt_enter(rt_device* dev);
+
+// rt_norm.hip: resolves the device-side address of the fixed GroupNorm scratch array for the current device
+int rt_norm_device_init(rt_device* dev);
 
 // Device pointer to the 65536-entry table out[bits(x)] = bits(op(x)) for a 16-bit type (type_index 0 = f16, 1 = bf16),
 // built on first use by running the exact unary kernel over all bit patterns (blocks until the table is ready).

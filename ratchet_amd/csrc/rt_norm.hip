@@ -30,6 +30,11 @@ constexpr int WAVES = BLOCK / WAVE;
 
 enum { NORM_LAYER = 0, NORM_RMS = 1 };
 
+// Partial statistics for rt_group_norm_static, the entry point that allocates nothing: a fixed array in the code object,
+// one copy per GPU.  In host code the array's name is only a stand-in; rt_norm_device_init asks the runtime where the
+// current device's copy lies and every launch is given that pointer.
+constexpr size_t GN_STATIC_SCRATCH_BYTES = 256 * 1024;
+static __device__ __align__(256) unsigned char gn_static_scratch[GN_STATIC_SCRATCH_BYTES];
 constexpr int NORM_WIDE_BLOCK = 1024;                   // threads per row for f32 rows that do not fit 256 threads' registers
 
 // per-row statistics in T arithmetic, given f32 sums
@@ -977,9 +982,11 @@ __global__ void __launch_bounds__(BLOCK) gn_combine_kernel(const float* __restri
     }
 }
 
+// fixed_scratch == nullptr: partial statistics go to the device's own buffer, grown from the driver when a problem needs
+// more; otherwise to fixed_scratch (GN_STATIC_SCRATCH_BYTES), and a problem that needs more is refused.
 template <typename T>
 int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint32_t bg, uint32_t glen, uint32_t cpg,
-              uint32_t groups, uint32_t L, float eps) {
+              uint32_t groups, uint32_t L, float eps, float* fixed_scratch) {
     // enough blocks to cover the chip, slices of at least 2048 elements; beyond 64 slices per group the partials are
     // combined by a launch of their own instead of by every apply block
     constexpr uint32_t FUSED_COMBINE_MAX = 64;
@@ -1031,7 +1038,11 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
     if (vec) chunk = (chunk + VEMAX - 1) / VEMAX * VEMAX;                               // slices start on vector boundaries
     splits = (glen + chunk - 1) / chunk;
     const size_t need = ((size_t)bg * splits + bg) * 3 * sizeof(float);           // partials, then one combined triple per group
-    if (need > dev->gn_scratch_bytes) {
+    if (fixed_scratch) {
+        RT_REQUIRE(need <= GN_STATIC_SCRATCH_BYTES, RT_ERR_SIZE,
+                   "rt_group_norm_static: %u (batch, group) pairs in %u slices need %zu bytes of partial statistics, the fixed buffer holds %zu",
+                   bg, splits, need, GN_STATIC_SCRATCH_BYTES);
+    } else if (need > dev->gn_scratch_bytes) {
         RT_NO_CAPTURE(dev, "growing the GroupNorm scratch");
         RT_HIP(hipStreamSynchronize(dev->stream));
         RT_HIP(hipFree(dev->gn_scratch));
@@ -1042,7 +1053,7 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
     }
     const dim3 grid(bg, splits), block(BLOCK);
     const bool separate = splits > FUSED_COMBINE_MAX;
-    float* const part = dev->gn_scratch;
+    float* const part = fixed_scratch ? fixed_scratch : dev->gn_scratch;
     const float* stats = separate ? part + (size_t)bg * splits * 3 : part;
     const uint32_t stat_splits = separate ? 1 : splits;
     if (vec) hipLaunchKernelGGL((gn_stats_kernel<T, VEMAX>), grid, block, 0, dev->stream, (const T*)x, part, glen, chunk, splits);
@@ -1123,6 +1134,14 @@ int launch_norm_via32(rt_device* dev, const void* x, const float* scale, const f
 
 }  // namespace
 
+// Called by rt_device_create with the new device current: looks up where THIS device's copy of gn_static_scratch lies.
+int rt_norm_device_init(rt_device* dev) {
+    void* p = nullptr;
+    RT_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(gn_static_scratch)));
+    dev->gn_static_ptr = static_cast<float*>(p);
+    return RT_OK;
+}
+
 extern "C" {
 
 int rt_norm_via_f32(rt_device* dev, int kind, int io_dt, const void* x, const float* scale, const float* bias, void* y, uint64_t rows,
@@ -1155,8 +1174,8 @@ int rt_rms_norm(rt_device* dev, int dt, const void* x, const void* scale, void* 
     return norm_entry(dev, NORM_RMS, dt, x, scale, nullptr, y, rows, cols, eps, "rt_rms_norm");
 }
 
-int rt_group_norm(rt_device* dev, int dt, const void* x, const void* scale, const void* bias, void* y, uint32_t B, uint32_t C, uint32_t L,
-                  uint32_t groups, float eps) {
+static int group_norm_entry(rt_device* dev, int dt, const void* x, const void* scale, const void* bias, void* y, uint32_t B, uint32_t C,
+                            uint32_t L, uint32_t groups, float eps, bool fixed) {
     RT_REQUIRE(rt_is_float_dt(dt), RT_ERR_DTYPE, "rt_group_norm: dtype %d is not F32/F16/BF16", dt);
     RT_REQUIRE(B > 0 && C > 0 && L > 0, RT_ERR_SHAPE, "rt_group_norm: zero extent");
     RT_REQUIRE(groups > 0 && C % groups == 0, RT_ERR_ARG, "rt_group_norm: %u channels do not split into %u groups", C, groups);
@@ -1170,11 +1189,26 @@ int rt_group_norm(rt_device* dev, int dt, const void* x, const void* scale, cons
     int rc = rt_enter(dev);
     if (rc) return rc;
     const uint32_t bg = B * groups;
-    switch (dt) {
-        case RT_F32: return launch_gn<float>(dev, x, scale, bias, y, bg, (uint32_t)glen, C / groups, groups, L, eps);
-        case RT_F16: return launch_gn<half_t>(dev, x, scale, bias, y, bg, (uint32_t)glen, C / groups, groups, L, eps);
-        default: return launch_gn<bf16_t>(dev, x, scale, bias, y, bg, (uint32_t)glen, C / groups, groups, L, eps);
+    float* fixed_scratch = nullptr;
+    if (fixed) {
+        fixed_scratch = dev->gn_static_ptr;
+        RT_REQUIRE(fixed_scratch, RT_ERR_ARG, "rt_group_norm_static: the device's fixed scratch buffer was not resolved at rt_device_create");
     }
+    switch (dt) {
+        case RT_F32: return launch_gn<float>(dev, x, scale, bias, y, bg, (uint32_t)glen, C / groups, groups, L, eps, fixed_scratch);
+        case RT_F16: return launch_gn<half_t>(dev, x, scale, bias, y, bg, (uint32_t)glen, C / groups, groups, L, eps, fixed_scratch);
+        default: return launch_gn<bf16_t>(dev, x, scale, bias, y, bg, (uint32_t)glen, C / groups, groups, L, eps, fixed_scratch);
+    }
+}
+
+int rt_group_norm(rt_device* dev, int dt, const void* x, const void* scale, const void* bias, void* y, uint32_t B, uint32_t C, uint32_t L,
+                  uint32_t groups, float eps) {
+    return group_norm_entry(dev, dt, x, scale, bias, y, B, C, L, groups, eps, false);
+}
+
+int rt_group_norm_static(rt_device* dev, int dt, const void* x, const void* scale, const void* bias, void* y, uint32_t B, uint32_t C,
+                         uint32_t L, uint32_t groups, float eps) {
+    return group_norm_entry(dev, dt, x, scale, bias, y, B, C, L, groups, eps, true);
 }
 
 }  // extern "C"

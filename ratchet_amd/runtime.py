@@ -361,10 +361,12 @@ class Device:
                                             up_row_stride or cols, out.ptr, rows, cols))
         return out
 
-    def group_norm(self, x, groups, scale, bias, eps=1e-5, out=None):
+    def group_norm(self, x, groups, scale, bias, eps=1e-5, out=None, static_scratch=False):
+        """static_scratch=True calls rt_group_norm_static, which never allocates (pass `out`, or the Buffer made here does)."""
         B, C = x.shape[0], x.shape[1]
         L = x.numel // (B * C)
         out = out or Buffer(self, x.shape, x.dt)
-        check(self.lib.rt_group_norm(self.handle, x.dt, x.ptr, scale.ptr if scale is not None else None,
-                                     bias.ptr if bias is not None else None, out.ptr, B, C, L, groups, eps))
+        fn = self.lib.rt_group_norm_static if static_scratch else self.lib.rt_group_norm
+        check(fn(self.handle, x.dt, x.ptr, scale.ptr if scale is not None else None,
+                 bias.ptr if bias is not None else None, out.ptr, B, C, L, groups, eps))
         return out
