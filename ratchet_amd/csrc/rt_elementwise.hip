@@ -70,7 +70,6 @@ struct BcastArgs {
     FastDiv d2, d1;
     uint32_t as[4], bs[4];
     uint32_t nvec;     // total vectors
-    uint32_t a_once, b_once;   // operand is read exactly once (no broadcast dim): stream it past the caches
     // XCD-aware block order for a large operand repeated over the leading dims (an [S,S] mask under H heads): hardware
     // block b runs on XCD b % 8, so the `reps` blocks that need the same 4 KiB slab of that operand are given to one
     // XCD back to back and its L2 fetches the slab once.  An XCD walks 2^chunk_log2 of its slabs per repeat before it
@@ -84,7 +83,10 @@ struct BcastArgs {
 constexpr int BC_UNROLL = 2;
 constexpr uint32_t XCDS = 8;
 
-template <typename T, int OP, int VE>
+// ONCE: bit 0 / bit 1 set when a / b has no broadcast dim, so each of its elements is read exactly once and its loads
+// carry the non-temporal hint.  (A compile-time choice: with `once ? ld_stream(q) : *q` on a run-time flag the compiler
+// merges the two loads into one ordinary load, and a 1 GiB operand then floods L2 and the memory-side cache.)
+template <typename T, int OP, int VE, int ONCE>
 __global__ void __launch_bounds__(BLOCK) binary_bcast_kernel(const T* __restrict__ a, const T* __restrict__ b,
                                                              T* __restrict__ y, BcastArgs p) {
     uint32_t blk = blockIdx.x;
@@ -111,9 +113,13 @@ __global__ void __launch_bounds__(BLOCK) binary_bcast_kernel(const T* __restrict
         if (VE > 1 && p.as[3] == 1) {
             Vec16<T> t16;
             const v4u* q = reinterpret_cast<const v4u*>(a + ao);
-            t16.u = p.a_once ? ld_stream(q) : *q;
+            t16.u = (ONCE & 1) ? ld_stream(q) : *q;
 #pragma unroll
             for (int e = 0; e < VE; e++) ra[e] = t16.e[e];
+        } else if (p.as[3] == 0) {
+            const T one = a[ao];                                  // broadcast along the last dim: one load, splatted
+#pragma unroll
+            for (int e = 0; e < VE; e++) ra[e] = one;
         } else {
 #pragma unroll
             for (int e = 0; e < VE; e++) ra[e] = a[ao + (uint64_t)e * p.as[3]];
@@ -121,9 +127,13 @@ __global__ void __launch_bounds__(BLOCK) binary_bcast_kernel(const T* __restrict
         if (VE > 1 && p.bs[3] == 1) {
             Vec16<T> t16;
             const v4u* q = reinterpret_cast<const v4u*>(b + bo);
-            t16.u = p.b_once ? ld_stream(q) : *q;
+            t16.u = (ONCE & 2) ? ld_stream(q) : *q;
 #pragma unroll
             for (int e = 0; e < VE; e++) rb[e] = t16.e[e];
+        } else if (p.bs[3] == 0) {
+            const T one = b[bo];                                  // broadcast along the last dim: one load, splatted
+#pragma unroll
+            for (int e = 0; e < VE; e++) rb[e] = one;
         } else {
 #pragma unroll
             for (int e = 0; e < VE; e++) rb[e] = b[bo + (uint64_t)e * p.bs[3]];
@@ -193,6 +203,7 @@ __global__ void __launch_bounds__(BLOCK) unary_scalar_kernel(const T* x, T* y, u
 // costs less than the memory traffic.
 constexpr int LUT_BLOCK = 1024;
 constexpr int LUT_UNROLL = 4;
+constexpr int LUT_TILE = LUT_BLOCK * LUT_UNROLL;   // vectors per tile
 constexpr size_t LUT_BYTES = 65536 * sizeof(uint16_t);
 
 __global__ void iota16_kernel(uint16_t* p) {
@@ -200,9 +211,31 @@ __global__ void iota16_kernel(uint16_t* p) {
     if (i < 65536) p[i] = (uint16_t)i;
 }
 
+// one 32-bit word = two elements through the table
+__device__ __forceinline__ uint32_t lut_pair(const uint16_t* lut, uint32_t w) {
+    const uint32_t lo = lut[w & 0xffffu];
+    const uint32_t hi = lut[w >> 16];
+    return lo | (hi << 16);
+}
+
+// The tensor is cut into tiles of LUT_TILE vectors (64 KiB of input); block b takes tiles b, b + gridDim.x, ...  The loads
+// of a block's next tile are issued before the lookups of the current one (and those of its first tile before the
+// table copy), so the HBM reads run underneath the LDS phase instead of after it: with every wave of the chip released
+// by the same barrier, a loop that loads, looks up and stores in turn alternates between a memory-bound and an
+// LDS-bound phase and pays for both.
 __global__ void __launch_bounds__(LUT_BLOCK) unary_lut_kernel(const uint16_t* __restrict__ table, const uint16_t* __restrict__ x,
                                                               uint16_t* y, uint64_t numel) {
     extern __shared__ __attribute__((aligned(16))) uint16_t lut[];
+    const uint64_t nvec = numel / 8;
+    const uint64_t tiles = nvec / LUT_TILE;
+    const v4u* xv = reinterpret_cast<const v4u*>(x);
+    v4u* yv = reinterpret_cast<v4u*>(y);
+    uint64_t t = blockIdx.x;
+    v4u cur[LUT_UNROLL];
+    if (t < tiles) {
+#pragma unroll
+        for (int k = 0; k < LUT_UNROLL; k++) cur[k] = ld_stream(xv + t * LUT_TILE + k * LUT_BLOCK + threadIdx.x);
+    }
     {
         const v4u* src = reinterpret_cast<const v4u*>(table);
         v4u* dst = reinterpret_cast<v4u*>(lut);
@@ -210,33 +243,36 @@ __global__ void __launch_bounds__(LUT_BLOCK) unary_lut_kernel(const uint16_t* __
         for (int i = 0; i < (int)(LUT_BYTES / 16 / LUT_BLOCK); i++) dst[i * LUT_BLOCK + threadIdx.x] = src[i * LUT_BLOCK + threadIdx.x];
     }
     __syncthreads();
-    const uint64_t nvec = numel / 8;
-    const v4u* xv = reinterpret_cast<const v4u*>(x);
-    v4u* yv = reinterpret_cast<v4u*>(y);
-    const uint64_t stride = (uint64_t)gridDim.x * (LUT_BLOCK * LUT_UNROLL);
-    for (uint64_t base = (uint64_t)blockIdx.x * (LUT_BLOCK * LUT_UNROLL) + threadIdx.x; base < nvec; base += stride) {
-        v4u in[LUT_UNROLL];
+    while (t < tiles) {
+        const uint64_t tn = t + gridDim.x;
+        v4u nxt[LUT_UNROLL];
 #pragma unroll
-        for (int k = 0; k < LUT_UNROLL; k++) {
-            const uint64_t i = base + (uint64_t)k * LUT_BLOCK;
-            if (i < nvec) in[k] = ld_stream(xv + i);
+        for (int k = 0; k < LUT_UNROLL; k++) nxt[k] = cur[k];
+        if (tn < tiles) {
+#pragma unroll
+            for (int k = 0; k < LUT_UNROLL; k++) nxt[k] = ld_stream(xv + tn * LUT_TILE + k * LUT_BLOCK + threadIdx.x);
         }
 #pragma unroll
         for (int k = 0; k < LUT_UNROLL; k++) {
-            const uint64_t i = base + (uint64_t)k * LUT_BLOCK;
-            if (i < nvec) {
-                v4u out;
+            v4u out;
 #pragma unroll
-                for (int w = 0; w < 4; w++) {
-                    const uint32_t lo = lut[in[k][w] & 0xffffu];
-                    const uint32_t hi = lut[in[k][w] >> 16];
-                    out[w] = lo | (hi << 16);
-                }
-                st_stream(yv + i, out);
-            }
+            for (int w = 0; w < 4; w++) out[w] = lut_pair(lut, cur[k][w]);
+            st_stream(yv + t * LUT_TILE + k * LUT_BLOCK + threadIdx.x, out);
         }
+#pragma unroll
+        for (int k = 0; k < LUT_UNROLL; k++) cur[k] = nxt[k];
+        t = tn;
     }
-    if (blockIdx.x == 0) {
+    // what is left after the whole tiles: fewer than LUT_TILE vectors and fewer than 8 elements, taken by the block
+    // that would have had the next tile
+    if (blockIdx.x == tiles % gridDim.x) {
+        for (uint64_t i = tiles * LUT_TILE + threadIdx.x; i < nvec; i += LUT_BLOCK) {
+            const v4u in = ld_stream(xv + i);
+            v4u out;
+#pragma unroll
+            for (int w = 0; w < 4; w++) out[w] = lut_pair(lut, in[w]);
+            st_stream(yv + i, out);
+        }
         const uint64_t i = nvec * 8 + threadIdx.x;
         if (i < numel) y[i] = lut[x[i]];
     }
@@ -495,7 +531,7 @@ template <typename T, bool VIA32 = false> int unary_via_lut(rt_device* dev, int 
                                    (int)LUT_BYTES));
         dev->lut_attr_set = 1;
     }
-    uint64_t blocks = (numel / 8 + LUT_BLOCK * LUT_UNROLL - 1) / (LUT_BLOCK * LUT_UNROLL);
+    uint64_t blocks = (numel / 8 + LUT_TILE - 1) / LUT_TILE;
     if (blocks > (uint64_t)dev->num_cus) blocks = dev->num_cus;          // one resident block per CU (128 KiB of LDS each)
     if (blocks < 1) blocks = 1;
     hipLaunchKernelGGL(unary_lut_kernel, dim3((unsigned)blocks), dim3(LUT_BLOCK), LUT_BYTES, dev->stream,
@@ -646,10 +682,10 @@ int launch_bcast(rt_device* dev, const void* a, const uint32_t a_shape[4], const
     p.d2 = make_fastdiv(y_shape[2]);
     p.d1 = make_fastdiv(y_shape[1]);
     p.nvec = (uint32_t)nvec;
-    p.a_once = p.b_once = 1;
+    bool a_once = true, b_once = true;                             // read exactly once (no broadcast dim): streamed past the caches
     for (int i = 0; i < 4; i++) {
-        if (a_shape[i] != y_shape[i]) p.a_once = 0;
-        if (b_shape[i] != y_shape[i]) p.b_once = 0;
+        if (a_shape[i] != y_shape[i]) a_once = false;
+        if (b_shape[i] != y_shape[i]) b_once = false;
     }
     const unsigned blocks = blocks_for(nvec, BLOCK * BC_UNROLL);
     // one operand full-size, the other equal to y's trailing dims and repeated over the leading ones, too large to
@@ -657,8 +693,8 @@ int launch_bcast(rt_device* dev, const void* a, const uint32_t a_shape[4], const
     p.slabs = 0;
     p.chunk_log2 = 0;
     p.reps = make_fastdiv(1);
-    if (p.a_once != p.b_once) {
-        const uint32_t* rs = p.a_once ? b_shape : a_shape;
+    if (a_once != b_once) {
+        const uint32_t* rs = a_once ? b_shape : a_shape;
         int lead = 0;
         while (lead < 4 && rs[lead] == 1) lead++;
         bool prefix = lead > 0 && lead < 4;
@@ -678,13 +714,14 @@ int launch_bcast(rt_device* dev, const void* a, const uint32_t a_shape[4], const
             p.chunk_log2 = per_xcd % 64 == 0 ? 6 : per_xcd % 4 == 0 ? 2 : 0;
         }
     }
-    if (ve == VEMAX) {
-        hipLaunchKernelGGL((binary_bcast_kernel<T, OP, VEMAX>), dim3(blocks), dim3(BLOCK), 0, dev->stream, (const T*)a,
-                           (const T*)b, (T*)y, p);
-    } else {
-        hipLaunchKernelGGL((binary_bcast_kernel<T, OP, 1>), dim3(blocks), dim3(BLOCK), 0, dev->stream, (const T*)a,
-                           (const T*)b, (T*)y, p);
-    }
+#define RT_BCAST(VEC, ONCE) \
+    hipLaunchKernelGGL((binary_bcast_kernel<T, OP, VEC, ONCE>), dim3(blocks), dim3(BLOCK), 0, dev->stream, (const T*)a, (const T*)b, (T*)y, p)
+    if (ve != VEMAX) RT_BCAST(1, 0);                              // scalar accesses
+    else if (a_once && b_once) RT_BCAST(VEMAX, 3);
+    else if (a_once) RT_BCAST(VEMAX, 1);
+    else if (b_once) RT_BCAST(VEMAX, 2);
+    else RT_BCAST(VEMAX, 0);
+#undef RT_BCAST
     RT_CHECK_LAUNCH("binary_bcast_kernel");
     return RT_OK;
 }

@@ -2,8 +2,8 @@
 //
 // Arithmetic contract (REFERENCE mode) = crates/ratchet-core/src/cpu/softmax.rs:22-42: e_j = exp(x_j) with no max
 // subtraction, stored in the element type; sum accumulated over j ascending in the element type; y_j = e_j / sum.
-//   f32: the row lives in registers (one wave64 per row, 16-byte loads), one exp per element (the device library's
-//        1-ulp expf; the 1e-5 bar leaves room for that), the sum is a wave butterfly instead of a sequential fold
+//   f32: the row lives in registers (one wave64 per row, 16-byte loads), one exp per element (v_exp_f32 on
+//        x * log2 e, see ref_exp_f32; the 1e-5 bar leaves room for that), the sum is a wave butterfly instead of a sequential fold
 //        (differs from the reference by float rounding order only), one IEEE division per element.
 //        HBM traffic: one read, one write.
 //   f16/bf16: the sequential 16-bit accumulation is order dependent (terms below half an ulp of the running sum
@@ -20,6 +20,12 @@ constexpr int BLOCK = 256;
 constexpr int WAVES = BLOCK / WAVE;
 
 template <typename T> __device__ __forceinline__ float stable_exp(float v) { return expf(v); }
+
+// e^v of the f32 reference mode in the register-resident kernel: one v_exp_f32 (1 ulp) on v * log2(e).  The rounding of
+// that product, half an ulp of |v| * 1.44, is the error: 3.3e-7 relative for |v| < 11, 6.6e-7 below 22, 2.6e-6 at the
+// overflow threshold (bar: 1e-5).  -inf gives 0, +inf and anything from 88.73 up give inf, NaN stays NaN, as with expf;
+// the library expf costs about four times the instructions, which at 27 M elements is most of the memory time.
+__device__ __forceinline__ float ref_exp_f32(float v) { return __builtin_amdgcn_exp2f(v * 1.44269504088896341f); }
 
 constexpr int WIDE_BLOCK = 1024;                        // threads per row for rows that do not fit 256 threads' registers
 
@@ -77,12 +83,12 @@ __global__ void __launch_bounds__(LANES > BLOCK ? LANES : BLOCK) softmax_wave_ke
             for (int q = 0; q < VE; q++) {
                 e[k][q] = 0.0f;
                 if (inside(lane + k * LANES, q)) {
-                    e[k][q] = (MODE == 1) ? expf(Ar<T>::widen(v[k].e[q]) - m) : expf(Ar<T>::widen(v[k].e[q]));
+                    e[k][q] = (MODE == 1) ? expf(Ar<T>::widen(v[k].e[q]) - m) : ref_exp_f32(Ar<T>::widen(v[k].e[q]));
                     s += e[k][q];
                 }
             }
     s = row_sum<LANES>(s);
-    // MODE 0: e / s as e * (1/s): one correctly rounded reciprocal per row, at most 1 ulp from the quotient (bar: 1e-5).
+    // MODE 0: e / s as e * (1/s) with one correctly rounded reciprocal per row and a Newton step per element.
     // A zero, subnormal, inf or NaN sum keeps the division so that 0/0, x/inf and inf/inf come out as the reference's do.
     const bool plain = MODE == 0 && (s >= 1.17549435e-38f) && (s < __builtin_huge_valf());
     const float rs = 1.0f / s;
@@ -92,7 +98,10 @@ __global__ void __launch_bounds__(LANES > BLOCK ? LANES : BLOCK) softmax_wave_ke
         if (i < nvec) {
             Vec16<T> o;
 #pragma unroll
-            for (int q = 0; q < VE; q++) o.e[q] = Ar<T>::conv(plain ? e[k][q] * rs : e[k][q] / s);
+            for (int q = 0; q < VE; q++) {
+                const float p0 = e[k][q] * rs;               // one Newton step on e * (1/s): the correctly rounded quotient for normal sums
+                o.e[q] = Ar<T>::conv(plain ? __builtin_fmaf(__builtin_fmaf(-s, p0, e[k][q]), rs, p0) : e[k][q] / s);
+            }
             if (!SPAN || (inside(i, 0) && inside(i, VE - 1))) {
                 st_stream(yr + i, o.u);
             } else {
