@@ -26,6 +26,7 @@ struct rt_device {
     int lut_attr_set;
     int gated_attr_set[2];
     unsigned gn_lds_attr_set;
+    unsigned np_attr_set;   // 16-bit norm instantiations (LDS-resident rows) whose dynamic-LDS limit has been raised on this device
     uint64_t sp_attr_set;   // streaming softmax instantiations whose dynamic-LDS limit has been raised on this device
     uint64_t sp_ragged_attr_set;   // the same for the ragged-row variants
     // row sums of one launch of the streaming softmax's ragged-row variant (RT_SM_ROW_SUMS 16-bit values, allocated with the device)

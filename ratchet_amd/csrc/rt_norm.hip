@@ -368,8 +368,15 @@ __global__ void __launch_bounds__(BLOCK) norm_seq16_kernel(const T* __restrict__
 // and raises its issue priority; the four loader waves fetch one 16-byte vector per thread per tile two tiles ahead,
 // widen x and T(x*x) to f32 and park them in double-buffered LDS tiles; one barrier per tile.  The kernel runs at the
 // speed of the dependent v_add_f32 chain (about 3 ns per column on this chip).
+// KEEP (launches whose blocks are all resident at once, rows of at most NP_KEEP_MAX_COLS columns): the walk of every row
+// of the tensor then ends at the same moment and nothing can hide what comes after it, so the output pass must be
+// nothing but stores: each loader thread also parks the raw vectors it loaded in dynamic LDS, scale and bias are staged
+// there once at the start, and after the statistics the block reads LDS, normalises and streams the result out,
+// instead of fetching x a second time through a loop of dependent load / store pairs.
 constexpr int NP_BLOCK = 320;
-template <typename T, int KIND>
+constexpr uint32_t NP_KEEP_MAX_COLS = 4096;
+constexpr size_t NP_KEEP_BYTES_PER_TILE = 256 * 16 + 2 * 32 * 16;   // the block's x vectors, one scale and one bias vector per column group
+template <typename T, int KIND, bool KEEP>
 __global__ void __launch_bounds__(NP_BLOCK) norm_pipe16_kernel(const T* __restrict__ x, const T* __restrict__ scale,
                                                                const T* __restrict__ bias, T* __restrict__ y, uint64_t rows, uint32_t cols,
                                                                float eps) {
@@ -378,6 +385,7 @@ __global__ void __launch_bounds__(NP_BLOCK) norm_pipe16_kernel(const T* __restri
     __shared__ __attribute__((aligned(16))) float tile[2][NSUM][RB][TC + PAD];   // [.][0] = squares, [.][1] = values
     __shared__ float sums[NSUM][RB];
     __shared__ T s_mu[RB], s_r[RB];
+    extern __shared__ __attribute__((aligned(16))) v4u np_keep[];               // KEEP: [ntiles][256] x, [ntiles][32] scale, [ntiles][32] bias
     const uint64_t row0 = (uint64_t)blockIdx.x * RB;
     const uint32_t nrows = (rows - row0 < (uint64_t)RB) ? (uint32_t)(rows - row0) : (uint32_t)RB;
     const uint32_t ntiles = (cols + TC - 1) / TC;
@@ -429,6 +437,9 @@ __global__ void __launch_bounds__(NP_BLOCK) norm_pipe16_kernel(const T* __restri
     const bool rvalid = r < nrows;
     const T* xrow = x + (row0 + (rvalid ? r : 0)) * cols;
     v4u pre0 = {0, 0, 0, 0}, pre1 = {0, 0, 0, 0};
+    v4u* keep_x = np_keep;
+    v4u* keep_scale = np_keep + ntiles * 256;
+    v4u* keep_bias = keep_scale + ntiles * 32;
 
     auto issue = [&](uint32_t t, v4u& dst) {
         const uint32_t col = t * TC + cv * 8;
@@ -442,6 +453,7 @@ __global__ void __launch_bounds__(NP_BLOCK) norm_pipe16_kernel(const T* __restri
             if (col < cols) {
                 Vec16<T> in;
                 in.u = __builtin_bit_cast(v4u, reg);
+                if (KEEP) keep_x[t * 256 + lt] = in.u;                          // read back by this same thread after the walk
 #pragma unroll
                 for (int q = 0; q < 8; q++) {
                     sq[q] = Ar<T>::widen(Ar<T>::mul(in.e[q], in.e[q]));
@@ -467,6 +479,14 @@ __global__ void __launch_bounds__(NP_BLOCK) norm_pipe16_kernel(const T* __restri
 
     issue(0, pre0);
     issue(1, pre1);
+    if (KEEP) {
+        // scale and bias, once per block, in flight together with the first two tiles; the barriers of the walk make
+        // them visible long before the output pass
+        for (uint32_t c = lt; c < cols / 8; c += 256) {
+            keep_scale[c] = reinterpret_cast<const v4u*>(scale)[c];
+            if (KIND == NORM_LAYER && bias) keep_bias[c] = reinterpret_cast<const v4u*>(bias)[c];
+        }
+    }
     for (uint32_t t = 0; t < ntiles; t += 2) {
         step(t, pre0);
         if (t + 1 < ntiles) step(t + 1, pre1);
@@ -479,6 +499,19 @@ __global__ void __launch_bounds__(NP_BLOCK) norm_pipe16_kernel(const T* __restri
     st.r = s_r[r];
     T* yrow = y + (row0 + r) * cols;
     const uint32_t cvec = cols / 8;
+    if (KEEP) {
+#pragma unroll 2
+        for (uint32_t c = cv, t = 0; c < cvec; c += 32, t++) {
+            Vec16<T> in, sc, bi, out;
+            in.u = keep_x[t * 256 + lt];
+            sc.u = keep_scale[c];
+            if (KIND == NORM_LAYER && bias) bi.u = keep_bias[c];
+#pragma unroll
+            for (int q = 0; q < 8; q++) out.e[q] = norm_one<T, KIND>(in.e[q], st, sc.e[q], bi.e[q], bias != nullptr);
+            st_stream(reinterpret_cast<v4u*>(yrow) + c, out.u);
+        }
+        return;
+    }
     for (uint32_t c = cv; c < cvec; c += 32) {
         Vec16<T> in, sc, bi, out;
         in.u = ld_stream(reinterpret_cast<const v4u*>(xrow) + c);
@@ -782,8 +815,25 @@ int launch_norm16(rt_device* dev, const void* x, const void* scale, const void* 
     if (vec_ok) {
         const uint64_t blocks = (rows + 7) / 8;
         RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");
-        hipLaunchKernelGGL((norm_pipe16_kernel<T, KIND>), dim3((unsigned)blocks), dim3(NP_BLOCK), 0, dev->stream, (const T*)x, (const T*)scale,
-                           (const T*)bias, (T*)y, rows, cols, eps);
+        // all blocks resident at once (the latency-bound case): the output pass comes from LDS
+        const uint32_t ntiles = (cols + 255) / 256;
+        const size_t keep_bytes = (size_t)ntiles * NP_KEEP_BYTES_PER_TILE;
+        const size_t static_bytes = (KIND == NORM_LAYER ? 2 : 1) * 2 * 8 * 260 * sizeof(float) + 256;
+        const size_t per_cu = (160 * 1024) / (static_bytes + keep_bytes);
+        if (cols <= NP_KEEP_MAX_COLS && blocks <= (uint64_t)dev->num_cus * per_cu) {
+            const int ti = (std::is_same<T, half_t>::value ? 0 : 2) + (KIND == NORM_LAYER ? 0 : 1);
+            if (!(dev->np_attr_set & (1u << ti))) {
+                RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(norm_pipe16_kernel<T, KIND, true>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)((NP_KEEP_MAX_COLS / 256) * NP_KEEP_BYTES_PER_TILE)));
+                dev->np_attr_set |= 1u << ti;
+            }
+            hipLaunchKernelGGL((norm_pipe16_kernel<T, KIND, true>), dim3((unsigned)blocks), dim3(NP_BLOCK), keep_bytes, dev->stream, (const T*)x,
+                               (const T*)scale, (const T*)bias, (T*)y, rows, cols, eps);
+        } else {
+            hipLaunchKernelGGL((norm_pipe16_kernel<T, KIND, false>), dim3((unsigned)blocks), dim3(NP_BLOCK), 0, dev->stream, (const T*)x,
+                               (const T*)scale, (const T*)bias, (T*)y, rows, cols, eps);
+        }
         RT_CHECK_LAUNCH("norm_pipe16_kernel");
         return RT_OK;
     }
