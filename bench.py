@@ -26,10 +26,27 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBPS = 8000.0
-# HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same script (KiB counters scaled by
-# what a 1 GiB copy kernel reads on them, x2.000 and x1.000); bench.py cannot collect counters itself
-PMC_TRAFFIC_BYTES = {"softmax16_stream_kernel": int((1050201.0 + 1048126.2) * 1024),
-                     "binary_bcast_kernel": int((1081372.1 + 1047819.4) * 1024)}
+# rocprofv3 summaries of this same script (bench.py cannot run the profiler on itself): per launch of the step, in step
+# order, the kernel's own duration from a --kernel-trace run and the HBM-side bytes from two --pmc runs (FETCH_SIZE,
+# WRITE_SIZE).  Read at run time; a missing file or row gives null, never a stale literal.
+PROFILE_KERNEL_TRACE = os.path.join("profiles", "bench_step_kernel_trace.txt")
+PROFILE_HBM_TRAFFIC = os.path.join("profiles", "bench_step_hbm_traffic_pmc.txt")
+
+
+def read_step_rows(rel_path):
+    """{position in the step (1-based): fields after the position} of the `step_op` lines of a profile summary."""
+    rows = {}
+    try:
+        with open(os.path.join(ROOT, rel_path)) as f:
+            for line in f:
+                if line.startswith("step_op"):
+                    fields = [x.strip() for x in line[len("step_op"):].split("|")]
+                    rows[int(fields[0])] = fields[1:]
+    except (OSError, ValueError):
+        return {}
+    return rows
+
+
 F32, F16 = 0, 1
 
 
@@ -370,8 +387,9 @@ def download_rows(dev, buf, nrows, row_elems, np_dtype):
     return out
 
 
-def check_and_time_cpu(dev, op, oracle):
-    """Parity of the timed output buffer against the oracle; returns (ok, cpu_seconds, cpu_bytes)."""
+def check_and_time_cpu(dev, op, oracle, check=True):
+    """Parity of the timed output buffer against the oracle; returns (ok, cpu_seconds, cpu_bytes).  check=False only
+    times the oracle (the second, loop-only CPU figure) and leaves the device buffers alone."""
     c = op.cpu_sample
     kind = c["kind"]
     np_dt = {"f32": np.float32, "f16": np.float16, "f16->f32": np.float32, "f32->f16": np.float16}[op.dtype]
@@ -387,17 +405,23 @@ def check_and_time_cpu(dev, op, oracle):
     if kind == "exact":
         want = timed(lambda: c["run"](oracle))
         b_cpu = c["bytes"]
+        if not check:
+            return True, t_cpu, b_cpu
         got = c["out"].to_numpy()
         ok = np.array_equal(got.view(np.uint8), np.ascontiguousarray(want).view(np.uint8))
     elif kind == "close":
         want = timed(lambda: c["run"](oracle))
         b_cpu = c["bytes"]
+        if not check:
+            return True, t_cpu, b_cpu
         bad, _ = oracle.count_not_close(c["out"].to_numpy(), want, c["tol"], c["tol"])
         ok = bad == 0
     elif kind == "softmax":
         x = c["x"].reshape(-1, c["x"].shape[-1])[: c["rows"]]
         want = timed(lambda: oracle.softmax(x))
         b_cpu = 2 * x.nbytes
+        if not check:
+            return True, t_cpu, b_cpu
         got = download_rows(dev, c["out"], c["rows"], x.shape[-1], np_dt)
         bad, _ = oracle.count_not_close(got, want, c["tol"], c["tol"])
         ok = bad == 0
@@ -405,6 +429,8 @@ def check_and_time_cpu(dev, op, oracle):
         x = c["x"].reshape(-1, c["x"].shape[-1])[: c["rows"]]
         want = timed(lambda: c["fn"](oracle, x))
         b_cpu = 2 * x.nbytes
+        if not check:
+            return True, t_cpu, b_cpu
         got = download_rows(dev, c["out"], c["rows"], x.shape[-1], np_dt)
         bad, _ = oracle.count_not_close(got, want, c["tol"], c["tol"])
         ok = bad == 0
@@ -415,6 +441,8 @@ def check_and_time_cpu(dev, op, oracle):
         del inp
         want = want.reshape(n, -1)
         b_cpu = int(n * c["bytes_per_row"])
+        if not check:
+            return True, t_cpu, b_cpu
         got = download_rows(dev, c["out"], n, want.shape[-1], np_dt)
         if c["tol"] == 0.0:
             ok = np.array_equal(got.view(np.uint16), want.view(np.uint16)) or bool(
@@ -527,7 +555,7 @@ def main():
     value = total_bytes / (ms_per_step * 1e-3) / 1e9
 
     oracle = None
-    parity_ok, cpu_t, cpu_b = True, 0.0, 0
+    parity_ok, cpu_t, cpu_b, loop_t = True, 0.0, 0, 0.0
     per_op_cpu = {}
     if not (args.no_check and args.no_cpu):
         from oracle import cpu_oracle as oracle          # the checker / CPU baseline only; never on the measured path
@@ -542,19 +570,45 @@ def main():
             cpu_t += t
             cpu_b += b
             per_op_cpu[id(o)] = (t, b)
+        # second CPU figure: the op's loop alone, without the reference's to_vec / store copies around it
+        loop_t = 0.0
+        if not args.no_cpu:
+            oracle.set_reference_copies(False)
+            for o in ops:
+                loop_t += check_and_time_cpu(dev, o, oracle, check=False)[1]
+            oracle.set_reference_copies(True)
 
     ceiling = copy_ceiling(dev) if not args.ops else None      # after the parity check: it overwrites an output buffer
     patterns = one_pass_patterns(dev, seed, oracle if not args.no_check else None) if not (args.ops or args.no_patterns) else None
     decode = decode_step(dev, seed) if not (args.ops or args.no_patterns) else None
 
+    # the kernels' own durations and HBM-side bytes, from the committed rocprofv3 summaries (whole step only: rows are by position)
+    kt_rows = read_step_rows(PROFILE_KERNEL_TRACE) if not args.ops else {}
+    pmc_rows = read_step_rows(PROFILE_HBM_TRAFFIC) if not args.ops else {}
+
+    def kernel_us(pos):
+        try:
+            return float(kt_rows[pos][2])
+        except (KeyError, IndexError, ValueError):
+            return None
+
+    def traffic_bytes(pos):
+        try:
+            return int((float(pmc_rows[pos][2]) + float(pmc_rows[pos][3])) * 1024)
+        except (KeyError, IndexError, ValueError):
+            return None
+
     rows = []
-    for o in ops:
+    for pos, o in enumerate(ops, 1):
         med = float(np.median(o.us))
         gbps = o.alg_bytes / (med * 1e-6) / 1e9
         t, b = per_op_cpu.get(id(o), (0.0, 0))
         rows.append({"cfg": o.cfg, "op": o.name, "dtype": o.dtype, "shape": o.shapes, "alg_MB": round(o.alg_bytes / 1e6, 3),
                      "us": round(med, 2), "us_mean": round(float(np.mean(o.us)), 2), "GBps": round(gbps, 1),
                      "frac_hbm": round(gbps / PEAK_HBM_GBPS, 4),
+                     # the kernel alone (rocprofv3 --kernel-trace of this script, profiles/): `us` adds the two events and the launch gap
+                     "kernel_us": kernel_us(pos),
+                     "kernel_frac_hbm": None if not kernel_us(pos) else round(o.alg_bytes / (kernel_us(pos) * 1e-6) / 1e9 / PEAK_HBM_GBPS, 4),
                      "cpu_GBps": round(b / t / 1e9, 4) if t > 0 else None})
 
     dom_avg_us = float(np.mean(dom_us))
@@ -572,12 +626,15 @@ def main():
         "roofline": {"bound": "hbm", "kernel": dom.kernel or dom.name, "op": f"cfg{dom.cfg} {dom.name}",
                      "achieved": round(dom_gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(dom_gbps / PEAK_HBM_GBPS, 4),
                      "avg_launch_us": round(dom_avg_us, 2), "algorithmic_bytes": dom.alg_bytes,
-                     # FETCH_SIZE + WRITE_SIZE per launch, scaled by a 1 GiB copy kernel (profiles/bench_step_hbm_traffic_pmc.txt)
-                     "traffic": PMC_TRAFFIC_BYTES.get(dom.kernel)},
+                     # FETCH_SIZE + WRITE_SIZE per launch, scaled by a 1 GiB copy kernel; null when the summary lacks the row
+                     "traffic": traffic_bytes(ops.index(dom) + 1), "traffic_source": PROFILE_HBM_TRAFFIC,
+                     "kernel_us_source": PROFILE_KERNEL_TRACE},
         "cpu_baseline": None if args.no_cpu or cpu_t == 0 else {
             "value": round(cpu_b / cpu_t / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": "every op of the step on one host core with the reference's to_vec/store copies, whole tensors "
                       "(%.1f MB algorithmic, %.1f s)" % (cpu_b / 1e6, cpu_t),
+            # the same ops timed without those copies: what the reference's loops alone cost
+            "loop_only": None if loop_t == 0 else {"value": round(cpu_b / loop_t / 1e9, 4), "unit": "GB/s", "seconds": round(loop_t, 2)},
             "host_cpus": os.cpu_count()},
         "hbm_copy_ceiling": ceiling,
         "one_pass_patterns": patterns,

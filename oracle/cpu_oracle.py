@@ -10,7 +10,8 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "libratchet_cpu_oracle.so")
+# RATCHET_ORACLE_LIB names another build of the same library (the sanitizer build, oracle/_asan/, in tests/test_sanitizers.py)
+_LIB_PATH = os.environ.get("RATCHET_ORACLE_LIB") or os.path.join(_HERE, "libratchet_cpu_oracle.so")
 
 F32, F16, BF16, I32, U32 = 0, 1, 2, 3, 4
 ADD, SUB, MUL, DIV = 0, 1, 2, 3

@@ -57,11 +57,24 @@ def _compile(src, force):
     return obj
 
 
-def build_host(force=False):
+def build_host(force=False, sanitize=False):
     """libratchet_host.so: the C++ mirror of ratchet's lazy Tensor API (host code only, g++), linked against
-    libratchet_hip.so in the same directory."""
+    libratchet_hip.so in the same directory.  sanitize=True builds the same sources with AddressSanitizer and
+    UndefinedBehaviorSanitizer into csrc/build/asan/ instead (CPU only; loaded by tests/test_sanitizers.py)."""
     srcs = sorted(glob.glob(os.path.join(HOST_DIR, "*.cpp")))
     deps = srcs + glob.glob(os.path.join(HOST_DIR, "*.hpp")) + headers() + [LIB_PATH]
+    if sanitize:
+        out_dir = os.path.join(OBJ_DIR, "asan")
+        os.makedirs(out_dir, exist_ok=True)
+        out = os.path.join(out_dir, "libratchet_host.so")
+        if force or _newer(out, deps):
+            cmd = [os.environ.get("CXX", "g++"), "-O1", "-g", "-std=c++17", "-fPIC", "-shared", "-fsanitize=address,undefined",
+                   "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer", "-o", out] + srcs + [
+                "-L" + HERE, "-lratchet_hip", "-Wl,-rpath," + HERE]
+            r = subprocess.run(cmd, capture_output=True, text=True)
+            if r.returncode != 0:
+                raise RuntimeError("sanitizer build of the host library failed:\n%s\n%s" % (" ".join(cmd), r.stderr[-8000:]))
+        return out
     if force or _newer(HOST_LIB_PATH, deps):
         cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-o", HOST_LIB_PATH] + srcs + [
             "-L" + HERE, "-lratchet_hip", "-Wl,-rpath,$ORIGIN"]

@@ -67,6 +67,11 @@ extern "C" {
 
 const char* rt_last_error(void) { return g_err; }
 
+int rt_debug_hip_status(int hip_error, const char* what) {
+    if (hip_error == 0) return RT_OK;
+    return rt_fail_hip((hipError_t)hip_error, what ? what : "injected");
+}
+
 const char* rt_status_name(int status) {
     switch (status) {
         case RT_OK: return "RT_OK";

@@ -15,7 +15,8 @@ import numpy as np
 from . import _lib
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-HOST_LIB_PATH = os.path.join(HERE, "libratchet_host.so")
+# RATCHET_HOST_LIB names another build of the same library (the sanitizer build of tests/test_sanitizers.py)
+HOST_LIB_PATH = os.environ.get("RATCHET_HOST_LIB") or os.path.join(HERE, "libratchet_host.so")
 
 _NP_TO_DT = {np.dtype(np.float32): _lib.F32, np.dtype(np.float16): _lib.F16, np.dtype(np.int32): _lib.I32,
              np.dtype(np.uint32): _lib.U32}

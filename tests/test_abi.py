@@ -40,6 +40,23 @@ def test_status_names(lib):
     assert lib.rt_status_name(-2).decode() == "HIP_ERROR"
 
 
+def test_hip_errors_map_to_negative_status_with_the_runtime_s_name(lib):
+    """every entry point turns a failed HIP call into -hipError_t and a message that names the call and the runtime's
+    own error string; injected here through the test hook, since nothing fails on demand without a GPU"""
+    lib.rt_debug_hip_status.argtypes = [ctypes.c_int, ctypes.c_char_p]
+    assert lib.rt_debug_hip_status(0, b"nothing") == 0
+    for code, name in ((1, b"hipErrorInvalidValue"), (2, b"hipErrorOutOfMemory"), (100, b"hipErrorNoDevice"), (101, b"hipErrorInvalidDevice"),
+                       (700, b"hipErrorIllegalAddress"), (719, b"hipErrorLaunchFailure")):
+        rc = lib.rt_debug_hip_status(code, b"hipFakeCall(args)")
+        assert rc == -code
+        msg = lib.rt_last_error()
+        assert msg.startswith(b"hipFakeCall(args): ") and name in msg, msg
+        assert lib.rt_status_name(rc).decode() == "HIP_ERROR"
+    # an argument error reported afterwards replaces the message (the HIP failure is not sticky in the library)
+    assert lib.rt_device_create(-1, ctypes.byref(ctypes.c_void_p())) == 7           # RT_ERR_ARG
+    assert b"negative ordinal" in lib.rt_last_error()
+
+
 def test_no_device_is_reported_not_hidden(lib):
     n = ctypes.c_int(-1)
     rc = lib.rt_device_count(ctypes.byref(n))

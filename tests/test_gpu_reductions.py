@@ -445,6 +445,32 @@ def test_layer_norm_variance_form_matches_reference(dev, oracle):
     assert np.nanmax(np.abs(got - want)) < np.nanmax(np.abs(two_pass - want)) or np.allclose(two_pass, want, atol=1e-4)
 
 
+# Three rows of five columns whose mean is far from zero next to their spread (mean 2.6-2.9, sigma 0.16-0.17), found by a
+# search over random rows.  The reference's one-pass variance E[x^2] - mu^2 (cpu/norm.rs:116-122) amplifies the rounding of
+# its two sums by mu^2 / var, so on these rows the reference formula itself lands about 3e-5 (in the all_close rule's
+# units) from the float64 result whatever the summation order: the 1e-5 bar cannot be met against the true value there,
+# and the bar of the reference's own test (1e-4, ops/norm/mod.rs:467) is the one that applies.
+OFFSET_ROWS_BITS = [[0x40231C58, 0x4031057B, 0x4012EEA4, 0x40278F96, 0x402C5483],
+                    [0x4039B87D, 0x403248EC, 0x402E5EA2, 0x40310982, 0x404CA049],
+                    [0x403C178E, 0x4033E167, 0x401D0871, 0x402F6B91, 0x40287424]]
+
+
+def test_layer_norm_f32_known_answer_rows_with_an_offset(dev, oracle):
+    x = np.array(OFFSET_ROWS_BITS, dtype=np.uint32).view(np.float32)
+    w, b = np.ones(5, np.float32), np.zeros(5, np.float32)
+    x64 = x.astype(np.float64)
+    exact = ((x64 - x64.mean(1, keepdims=True)) / np.sqrt(x64.var(1, keepdims=True) + 1e-5)).astype(np.float32)
+    want = oracle.layer_norm(x, w, b, 1e-5, intended=True)
+    bad5, _ = oracle.count_not_close(want, exact, 1e-5, 1e-5)
+    assert bad5 > 0                                                    # the formula, not a kernel: the oracle itself misses 1e-5 here
+    bad4, mx = oracle.count_not_close(want, exact, 1e-4, 1e-4)
+    assert bad4 == 0, mx
+    got = dev.layer_norm(dev.upload(x), dev.upload(w), dev.upload(b), 1e-5).to_numpy()
+    for name, ref in (("float64 result", exact), ("oracle", want)):
+        bad, mx = oracle.count_not_close(got, ref, 1e-4, 1e-4)
+        assert bad == 0, (name, bad, mx)
+
+
 @pytest.mark.parametrize("B,C,L,G", [(1, 3, 1, 1), (2, 8, 5, 4), (1, 6, 7, 6), (3, 4, 9, 1), (1, 64, 3000, 32), (2, 32, 17, 8),
                                      (1, 512, 3000, 32),          # the benchmark shape: 32 groups of 96 KB, staged in LDS, one launch
                                      (9, 128, 40, 64),            # 576 groups: more than two per CU, the two-launch streaming path
