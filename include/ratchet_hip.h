@@ -79,6 +79,9 @@ int rt_free(rt_device* dev, void* dptr);                     /* last drop of a P
  * (hits) or passed to hipMalloc (misses); any out pointer may be NULL. */
 int rt_pool_trim(rt_device* dev);
 int rt_pool_stats(rt_device* dev, uint64_t* live_bytes, uint64_t* parked_bytes, uint64_t* hits, uint64_t* misses);
+/* the most bytes that were handed out at one time since the last reset (reset != 0 restarts the mark at what is handed
+ * out now): what a graph executor checks its activation memory plan against (allocator.rs:266-271 logs the same total) */
+int rt_pool_peak(rt_device* dev, uint64_t* peak_live_bytes, int reset);
 int rt_memset0(rt_device* dev, void* dptr, size_t bytes);    /* GPUBuffer::zeros (gpu_buffer.rs:29-37) */
 int rt_h2d(rt_device* dev, void* dptr, const void* host, size_t bytes);   /* GPUBuffer::from_bytes (:49-59), blocking */
 int rt_d2h(rt_device* dev, void* host, const void* dptr, size_t bytes);   /* GPUBuffer::to_cpu (:199-218), blocking */

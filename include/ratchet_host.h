@@ -28,6 +28,7 @@ rth_device* rth_device_request(int ordinal);                          /* Device:
 void rth_device_release(rth_device* dev);
 /* {bytes handed out, bytes parked in the pool, requests served by the pool, requests passed to the driver} (rt_pool_stats) */
 int rth_pool_stats(rth_device* dev, uint64_t out[4]);
+int rth_pool_peak(rth_device* dev, uint64_t* peak_live_bytes, int reset);   /* rt_pool_peak of the device */
 
 /* Tensor::from_data + to(device) (tensor.rs:553-571,874-892); dt codes as in ratchet_hip.h */
 rth_tensor* rth_from_host(rth_device* dev, const void* data, int rank, const uint64_t* shape, int dt);
@@ -64,6 +65,13 @@ int rth_resolve(rth_tensor* t);                                        /* Tensor
 int rth_to_host(const rth_tensor* t, void* out);                       /* to(&Device::CPU) (tensor.rs:957-975) */
 long rth_last_resolve_launches(const rth_tensor* t);                   /* kernels launched by the last rth_resolve(t) */
 int rth_execution_order(const rth_tensor* t, uint64_t* ids, int cap);  /* ids in execution order; returns the count */
+/* The memory plan rth_resolve(t) would follow (BufferAllocator::greedy_by_size with in-place leasing,
+ * gpu/buffer_allocator/allocator.rs:141-271), without allocating or launching anything: the sizes of the shared objects,
+ * and per launch, in execution order, four values {tensor id, bytes, object, source}: object is an index into
+ * object_bytes, -1 for an allocation of its own (t itself and tensors still visible outside the graph) or -2 when the
+ * op runs in place in a buffer that exists already; source is the tensor whose allocation the result lives in.
+ * Returns the number of launches (entries beyond entry_cap are not written), -1 on error. */
+int rth_memory_plan(const rth_tensor* t, uint64_t* object_bytes, int object_cap, int* n_objects, int64_t* entries, int entry_cap);
 uint64_t rth_id(const rth_tensor* t);
 
 #ifdef __cplusplus

@@ -1,6 +1,7 @@
 // Implementation of the C++ host mirror (see ratchet.hpp).  Host code only: it talks to the GPU through the C ABI of
 // libratchet_hip.so and contains no arithmetic on tensor data.
 #include "ratchet.hpp"
+#include "planner.hpp"
 
 #include <algorithm>
 #include <atomic>
@@ -633,7 +634,7 @@ struct Resolver {
     static void run_fused(Node* n, const FusedPlan& plan, size_t& launches) {
         rt_device* dev = n->device.raw();
         const int dt = (int)n->dt;
-        n->storage = std::make_shared<Buffer>(n->device, n->shape.numel() * size_of(n->dt));
+        if (!n->storage) n->storage = std::make_shared<Buffer>(n->device, n->shape.numel() * size_of(n->dt));
         const size_t cols = n->shape[n->shape.rank() - 1];
         const uint64_t rows = n->shape.numel() / cols;
         switch (plan.what) {
@@ -682,16 +683,12 @@ struct Resolver {
         rt_device* dev = n->device.raw();
         const int dt = (int)n->dt;
         auto src = [&](size_t i) -> Node* { return Node::of(n->srcs[i]); };
-        auto out_buffer = [&]() { n->storage = std::make_shared<Buffer>(n->device, n->shape.numel() * size_of(n->dt)); };
-        // tensor.rs:823-824: supports_inplace() && Arc::strong_count(srcs[0]) == 1 (and here: nobody else shares the buffer)
-        auto take_src0_if_unshared = [&]() {
-            Node* s0 = src(0);
-            if (Node::holders(n->srcs[0]) == 1 && s0->storage.use_count() == 1 && s0->shape == n->shape && s0->dt == n->dt) {
-                n->storage = s0->storage;
-                return true;
-            }
-            return false;
+        // resolve() has given the node its output buffer already (the source's own when the op runs in place, a shared
+        // object of the memory plan, or an allocation of its own)
+        auto out_buffer = [&]() {
+            if (!n->storage) n->storage = std::make_shared<Buffer>(n->device, n->shape.numel() * size_of(n->dt));
         };
+        auto take_src0_if_unshared = [&]() { return (bool)n->storage; };
         switch (n->kind) {
             case Kind::Const: throw Error("Unresolved", "constant tensor " + std::to_string(n->id) + " has no storage (placeholder)");
             case Kind::View: n->storage = src(0)->storage; return;
@@ -842,8 +839,28 @@ struct Resolver {
         }
     }
 
-    static void resolve(Node* root) {
-        size_t launches = 0;
+    // Everything resolve() decides before the first launch: which nodes run, which are folded into a neighbour, what
+    // each launch reads, and the memory plan.
+    struct Prepared {
+        std::vector<Node*> order;                                  // needed nodes, execution order
+        std::unordered_set<Node*> skip;
+        std::unordered_map<Node*, FusedPlan> fused;
+        std::vector<planner::Step> steps;                          // one per launch
+        std::vector<Node*> step_node;
+        std::vector<std::vector<Node*>> step_reads;                // the nodes behind Step::reads
+        std::unordered_map<Node*, size_t> step_of;
+        std::vector<std::vector<Node*>> release_at;                // per index into order: nodes whose storage handle is dropped after it
+        planner::Plan plan;
+    };
+
+    // the node whose buffer is read when `t` is an operand: through views (which alias their source)
+    static Node* base_of(Node* n) {
+        while (n->kind == Kind::View && !n->storage) n = Node::of(n->srcs[0]);
+        return n;
+    }
+
+    static Prepared prepare(Node* root) {
+        Prepared P;
         const std::vector<Node*> full_order = execution_order(root);
         // only what the root still needs: nothing below a tensor that already has its storage (tensor.rs:783 skips those;
         // their own inputs may have given their buffers back, see below)
@@ -857,12 +874,12 @@ struct Resolver {
                 for (const Tensor& s : n->srcs) todo.push_back(Node::of(s));
             }
         }
-        std::vector<Node*> order;
+        std::vector<Node*>& order = P.order;
         for (Node* n : full_order)
             if (needed.count(n)) order.push_back(n);
-        std::unordered_set<Node*> skip;
+        std::unordered_set<Node*>& skip = P.skip;
         // caller patterns, consumers first so that the longest sequence wins (the gated multiply contains a unary one)
-        std::unordered_map<Node*, FusedPlan> fused;
+        std::unordered_map<Node*, FusedPlan>& fused = P.fused;
         if (g_fuse_patterns) {
             for (auto it = order.rbegin(); it != order.rend(); ++it) {
                 Node* n = *it;
@@ -881,10 +898,8 @@ struct Resolver {
                 for (const Tensor& s : n->srcs)
                     if (fusable_broadcast(s)) skip.insert(Node::of(s));
 
-        // Liveness, the job of the reference's allocation planner (gpu/buffer_allocator/allocator.rs:141-271): an
-        // intermediate that nobody outside this graph can see gives its buffer back to the device's pool right after the
-        // last launch that reads it, so a long graph holds a few live buffers instead of one per node.  Launches run in
-        // stream order, which makes the hand-over safe without waiting.
+        // Liveness: an intermediate that nobody outside this graph can see drops its handle on its buffer right after the
+        // last launch that reads it.  Launches run in stream order, which makes the hand-over safe without waiting.
         std::unordered_map<Node*, size_t> index_of, edges, last_use;
         std::unordered_map<Node*, Node*> consumer;                 // of a skipped node: the one node that absorbs it
         for (size_t i = 0; i < order.size(); i++) index_of[order[i]] = i;
@@ -899,7 +914,7 @@ struct Resolver {
             while (skip.count(n)) n = consumer.at(n);
             return index_of.at(n);
         };
-        std::vector<std::vector<Node*>> release_at(order.size());
+        P.release_at.resize(order.size());
         for (Node* n : order) {
             if (n->storage) continue;
             for (const Tensor& s : n->srcs) {
@@ -909,31 +924,117 @@ struct Resolver {
                 if (it == last_use.end() || it->second < at) last_use[src] = at;
             }
         }
+        // every holder of the node is an edge of this graph: no user handle, no other graph
+        auto hidden = [&](Node* n, const Tensor& handle) { return n != root && !n->srcs.empty() && (size_t)Node::holders(handle) == edges[n]; };
+        std::unordered_set<Node*> hidden_nodes;
         for (Node* n : order) {
             if (n->storage) continue;
             for (const Tensor& s : n->srcs) {
                 Node* src = Node::of(s);
-                // every holder of the node is an edge of this graph: no user handle, no other graph
-                if (src != root && !src->srcs.empty() && (size_t)Node::holders(s) == edges[src] && last_use.count(src)) {
-                    release_at[last_use[src]].push_back(src);
-                    last_use.erase(src);
+                if (hidden(src, s)) {
+                    hidden_nodes.insert(src);
+                    if (last_use.count(src)) {
+                        P.release_at[last_use[src]].push_back(src);
+                        last_use.erase(src);
+                    }
                 }
             }
         }
 
-        for (size_t i = 0; i < order.size(); i++) {
-            Node* n = order[i];
-            if (!n->storage && !skip.count(n)) {                   // else: already resolved or fused away
-                auto f = fused.find(n);
-                if (f != fused.end()) run_fused(n, f->second, launches);
-                else run(n, launches);
+        // The launches and what each reads, for the memory plan (gpu/buffer_allocator/allocator.rs:141-271).
+        auto launches_here = [&](Node* n) { return !n->storage && !skip.count(n) && n->kind != Kind::View && !n->srcs.empty(); };
+        for (Node* n : order) {
+            if (!launches_here(n)) continue;
+            planner::Step st;
+            st.id = n->id;
+            st.bytes = n->shape.numel() * size_of(n->dt);
+            st.pinned = !hidden_nodes.count(n);
+            std::vector<Node*> reads;
+            std::vector<Node*> todo;
+            for (auto it = n->srcs.rbegin(); it != n->srcs.rend(); ++it) todo.push_back(Node::of(*it));
+            while (!todo.empty()) {                                // operands in bind order, through folded-away nodes and views
+                Node* m = todo.back();
+                todo.pop_back();
+                if (!m->storage && (skip.count(m) || m->kind == Kind::View)) {
+                    for (auto it = m->srcs.rbegin(); it != m->srcs.rend(); ++it) todo.push_back(Node::of(*it));
+                    continue;
+                }
+                if (std::find(reads.begin(), reads.end(), m) == reads.end()) reads.push_back(m);
             }
-            for (Node* dead : release_at[i]) dead->storage.reset();
+            // tensor.rs:823-824: supports_inplace() && Arc::strong_count(srcs[0]) == 1 (here also: same size, and nobody
+            // else shares a buffer that exists already); IndexWrite's result is its destination (ops/index_write.rs:40-50)
+            if (!fused.count(n)) {
+                const Tensor& s0T = n->srcs[0];
+                Node* s0 = Node::of(s0T);
+                bool in_place = false;
+                if (n->kind == Kind::IndexWrite) {
+                    in_place = true;
+                } else if (n->kind == Kind::Unary || n->kind == Kind::Softmax || n->kind == Kind::RoPE ||
+                           (n->kind == Kind::Binary && !fusable_broadcast(n->srcs[0]) && !fusable_broadcast(n->srcs[1]))) {
+                    in_place = Node::holders(s0T) == 1 && s0->shape == n->shape && s0->dt == n->dt && s0->kind != Kind::View &&
+                               (s0->storage ? s0->storage.use_count() == 1 : true);
+                }
+                if (in_place) st.inplace = (int)(std::find(reads.begin(), reads.end(), base_of(s0)) - reads.begin());
+            }
+            for (Node* r : reads) st.reads.push_back(r->id);
+            P.step_of[n] = P.steps.size();
+            P.steps.push_back(st);
+            P.step_node.push_back(n);
+            P.step_reads.push_back(reads);
+        }
+        P.plan = planner::greedy_by_size(P.steps);
+        return P;
+    }
+
+    static void resolve(Node* root) {
+        size_t launches = 0;
+        Prepared P = prepare(root);
+        // shared objects come from the device's pool when their first tenant is produced and go back after their last reader
+        std::vector<std::shared_ptr<Buffer>> objects(P.plan.object_bytes.size());
+        for (size_t i = 0; i < P.order.size(); i++) {
+            Node* n = P.order[i];
+            auto st = P.step_of.find(n);
+            if (st != P.step_of.end()) {
+                const planner::Step& step = P.steps[st->second];
+                const int obj = P.plan.object_of.at(n->id);
+                if (step.inplace >= 0) {
+                    n->storage = P.step_reads[st->second][(size_t)step.inplace]->storage;
+                } else if (obj >= 0) {
+                    if (!objects[(size_t)obj]) objects[(size_t)obj] = std::make_shared<Buffer>(n->device, P.plan.object_bytes[(size_t)obj]);
+                    n->storage = objects[(size_t)obj];
+                } else {
+                    n->storage = std::make_shared<Buffer>(n->device, step.bytes);
+                }
+                auto f = P.fused.find(n);
+                if (f != P.fused.end()) run_fused(n, f->second, launches);
+                else run(n, launches);
+                for (size_t o = 0; o < objects.size(); o++)
+                    if (objects[o] && P.plan.object_last_use[o] == st->second) objects[o].reset();
+            } else if (!n->storage && !P.skip.count(n)) {
+                run(n, launches);                                  // a view (no launch) or a constant without storage (throws)
+            }
+            for (Node* dead : P.release_at[i]) dead->storage.reset();
         }
         check_rt(rt_sync(root->device.raw()), "rt_sync");      // resolve returns after completion (tensor.rs:855-856)
         root->last_launches = launches;
     }
 };
+
+MemoryPlan Tensor::memory_plan() const {
+    if (!node_) throw Error("NullTensor", "memory_plan on an empty tensor");
+    Resolver::Prepared P = Resolver::prepare(node_.get());
+    MemoryPlan out;
+    out.object_bytes = P.plan.object_bytes;
+    for (size_t i = 0; i < P.steps.size(); i++) {
+        MemoryPlan::Entry e;
+        e.id = P.steps[i].id;
+        e.bytes = P.steps[i].bytes;
+        e.object = P.plan.object_of.at(e.id);
+        e.source = P.plan.source_of.at(e.id);
+        out.entries.push_back(e);
+    }
+    return out;
+}
 
 Tensor Tensor::resolve() const {
     if (!node_) throw Error("NullTensor", "resolve on an empty tensor");

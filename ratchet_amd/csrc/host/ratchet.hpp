@@ -98,6 +98,20 @@ bool pattern_fusion();
 class Tensor;
 struct Node;                                                  // LazyOp + operands (op.rs:14-31)
 
+// What resolve() would allocate for the intermediates of a graph (gpu/buffer_allocator/allocator.rs:208-271, see
+// planner.hpp): one entry per launch, in execution order.
+struct MemoryPlan {
+    struct Entry {
+        uint64_t id = 0;          // the tensor the launch produces
+        size_t bytes = 0;
+        int object = -1;          // index into object_bytes; -1: an allocation of its own (the resolved tensor, tensors
+                                  // visible outside the graph); -2: works in place in a buffer that exists already
+        uint64_t source = 0;      // the tensor whose allocation it lives in (itself unless it runs in place)
+    };
+    std::vector<size_t> object_bytes;
+    std::vector<Entry> entries;
+};
+
 class Tensor {
   public:
     Tensor() {}
@@ -166,6 +180,9 @@ class Tensor {
     void to_host(void* out) const;
     // number of kernel launches the last resolve() of this tensor issued (for tests)
     size_t last_resolve_launches() const;
+
+    // the memory plan resolve() would follow; works on placeholder graphs (nothing is allocated or launched)
+    MemoryPlan memory_plan() const;
 
     // unit-test hook for the topological order (tensor.rs:696-740): ids in execution order
     std::vector<uint64_t> execution_order_ids() const;

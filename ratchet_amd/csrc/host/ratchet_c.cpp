@@ -54,6 +54,8 @@ int rth_pool_stats(rth_device* dev, uint64_t out[4]) {
     return rt_pool_stats(dev->dev.raw(), &out[0], &out[1], &out[2], &out[3]);
 }
 
+int rth_pool_peak(rth_device* dev, uint64_t* peak_live_bytes, int reset) { return rt_pool_peak(dev->dev.raw(), peak_live_bytes, reset); }
+
 rth_tensor* rth_from_host(rth_device* dev, const void* data, int rank, const uint64_t* shape, int dt) {
     return build([&] { return Tensor::from_host(data, make_shape(rank, shape), (DType)dt, dev->dev); });
 }
@@ -167,6 +169,23 @@ int rth_execution_order(const rth_tensor* t, uint64_t* ids, int cap) {
     const std::vector<uint64_t> v = t->t.execution_order_ids();
     for (int i = 0; i < cap && i < (int)v.size(); i++) ids[i] = v[i];
     return (int)v.size();
+}
+int rth_memory_plan(const rth_tensor* t, uint64_t* object_bytes, int object_cap, int* n_objects, int64_t* entries, int entry_cap) {
+    try {
+        const MemoryPlan p = t->t.memory_plan();
+        if (n_objects) *n_objects = (int)p.object_bytes.size();
+        for (int i = 0; i < object_cap && i < (int)p.object_bytes.size(); i++) object_bytes[i] = p.object_bytes[i];
+        for (int i = 0; i < entry_cap && i < (int)p.entries.size(); i++) {
+            entries[4 * i + 0] = (int64_t)p.entries[i].id;
+            entries[4 * i + 1] = (int64_t)p.entries[i].bytes;
+            entries[4 * i + 2] = p.entries[i].object;
+            entries[4 * i + 3] = (int64_t)p.entries[i].source;
+        }
+        return (int)p.entries.size();
+    } catch (const std::exception& e) {
+        capture(e);
+        return -1;
+    }
 }
 
 }  // extern "C"

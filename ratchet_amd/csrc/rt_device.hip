@@ -21,6 +21,7 @@ struct rt_pool {
     std::multimap<size_t, void*> parked;            // block size -> block, free for reuse
     std::unordered_map<void*, size_t> live;         // blocks handed out by rt_malloc
     size_t parked_bytes = 0;
+    size_t live_bytes = 0, peak_live_bytes = 0;     // handed out now / the most that was handed out at once since the last reset
     uint64_t hits = 0, misses = 0;
 };
 
@@ -214,6 +215,8 @@ int rt_malloc(rt_device* dev, size_t bytes, void** dptr) {
     if (it != pool->parked.end() && it->first <= sz + sz / 4) {
         *dptr = it->second;
         pool->live.emplace(it->second, it->first);
+        pool->live_bytes += it->first;
+        if (pool->live_bytes > pool->peak_live_bytes) pool->peak_live_bytes = pool->live_bytes;
         pool->parked_bytes -= it->first;
         pool->parked.erase(it);
         pool->hits++;
@@ -234,6 +237,8 @@ int rt_malloc(rt_device* dev, size_t bytes, void** dptr) {
         return rt_fail_hip(e, "hipMalloc");
     }
     pool->live.emplace(*dptr, sz);
+    pool->live_bytes += sz;
+    if (pool->live_bytes > pool->peak_live_bytes) pool->peak_live_bytes = pool->live_bytes;
     pool->misses++;
     return RT_OK;
 }
@@ -248,6 +253,7 @@ int rt_free(rt_device* dev, void* dptr) {
     RT_REQUIRE(it != pool->live.end(), RT_ERR_ARG, "rt_free: %p was not allocated by rt_malloc on this device (or was freed twice)", dptr);
     pool->parked.emplace(it->second, dptr);
     pool->parked_bytes += it->second;
+    pool->live_bytes -= it->second;
     pool->live.erase(it);
     return RT_OK;
 }
@@ -280,6 +286,15 @@ int rt_pool_stats(rt_device* dev, uint64_t* live_bytes, uint64_t* parked_bytes, 
     if (parked_bytes) *parked_bytes = pool->parked_bytes;
     if (hits) *hits = pool->hits;
     if (misses) *misses = pool->misses;
+    return RT_OK;
+}
+
+int rt_pool_peak(rt_device* dev, uint64_t* peak_live_bytes, int reset) {
+    RT_REQUIRE(dev, RT_ERR_NULL_DEVICE, "rt_device is NULL");
+    rt_pool* pool = dev->pool;
+    std::lock_guard<std::mutex> lock(pool->mu);
+    if (peak_live_bytes) *peak_live_bytes = pool->peak_live_bytes;
+    if (reset) pool->peak_live_bytes = pool->live_bytes;
     return RT_OK;
 }
 

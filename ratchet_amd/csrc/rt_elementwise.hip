@@ -583,7 +583,9 @@ int launch_gated(rt_device* dev, int op, const void* gate, uint64_t gs, const vo
     p.gs = gs;
     p.us = us;
     const bool vec = cols % 8 == 0 && gs % 8 == 0 && us % 8 == 0 && rt_aligned(gate, 16) && rt_aligned(up, 16) && rt_aligned(y, 16);
-    if (vec && numel >= RT_LUT_MIN_NUMEL) {
+    // (while a graph is being captured a table that does not exist yet cannot be built: the computing kernel below gives
+    // the same bits)
+    if (vec && numel >= RT_LUT_MIN_NUMEL && (!dev->capturing || dev->unary_lut_via32[ti][op])) {
         int rc = build_unary_table<T, true>(dev, ti, op);
         if (rc) return rc;
         if (!dev->gated_attr_set[ti]) {
@@ -807,9 +809,11 @@ int rt_unary(rt_device* dev, int op, int dt, const void* x, void* y, uint64_t nu
     RT_REQUIRE(rt_aligned(x, eb) && rt_aligned(y, eb), RT_ERR_ALIGN, "rt_unary: misaligned pointer");
     int rc = rt_enter(dev);
     if (rc) return rc;
-    // large 16-bit tensors: table lookup (bit-identical to computing, see unary_lut_kernel)
-    const bool lut = dt != RT_F32 && numel >= RT_LUT_MIN_NUMEL && lut_worthwhile(op) && rt_aligned(x, 16) && rt_aligned(y, 16);
-    // in between: the table read in place (while a graph is being captured only if the table exists already)
+    // large 16-bit tensors: table lookup (bit-identical to computing, see unary_lut_kernel); while a graph is being
+    // captured only if the table exists already (building it synchronises), otherwise the computing kernel runs
+    const bool have_table = dt != RT_F32 && (!dev->capturing || dev->unary_lut[dt == RT_BF16 ? 1 : 0][op]);
+    const bool lut = have_table && numel >= RT_LUT_MIN_NUMEL && lut_worthwhile(op) && rt_aligned(x, 16) && rt_aligned(y, 16);
+    // in between: the table read in place
     const bool gather = dt != RT_F32 && !lut && numel >= RT_GATHER_MIN_NUMEL && lut_worthwhile(op) && rt_aligned(x, 16) && rt_aligned(y, 16) &&
                         (!dev->capturing || dev->unary_lut[dt == RT_BF16 ? 1 : 0][op]);
     switch (dt) {
@@ -832,9 +836,9 @@ int rt_unary_via_f32(rt_device* dev, int op, int io_dt, const void* x, void* y, 
     RT_REQUIRE(rt_aligned(x, 2) && rt_aligned(y, 2), RT_ERR_ALIGN, "rt_unary_via_f32: misaligned pointer");
     int rc = rt_enter(dev);
     if (rc) return rc;
-    const bool lut = numel >= RT_LUT_MIN_NUMEL && lut_worthwhile(op) && rt_aligned(x, 16) && rt_aligned(y, 16);
-    const bool gather = !lut && numel >= RT_GATHER_MIN_NUMEL && lut_worthwhile(op) && rt_aligned(x, 16) && rt_aligned(y, 16) &&
-                        (!dev->capturing || dev->unary_lut_via32[io_dt == RT_BF16 ? 1 : 0][op]);
+    const bool have_table = !dev->capturing || dev->unary_lut_via32[io_dt == RT_BF16 ? 1 : 0][op];
+    const bool lut = have_table && numel >= RT_LUT_MIN_NUMEL && lut_worthwhile(op) && rt_aligned(x, 16) && rt_aligned(y, 16);
+    const bool gather = !lut && have_table && numel >= RT_GATHER_MIN_NUMEL && lut_worthwhile(op) && rt_aligned(x, 16) && rt_aligned(y, 16);
     if (io_dt == RT_F16)
         return lut ? unary_via_lut<half_t, true>(dev, op, x, y, numel)
                    : gather ? unary_via_table_gather<half_t, true>(dev, op, x, y, numel) : dispatch_unary<half_t, true>(dev, op, x, y, numel);

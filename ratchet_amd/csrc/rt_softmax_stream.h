@@ -659,6 +659,9 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
         chunk_rows = (0x7fffffffull / row_bytes) / SP_ROWS * SP_ROWS;
         if (chunk_rows == 0) return RT_OK;
     }
+    // the exp table is built on first use, which synchronises: while a graph is being captured a missing table sends the
+    // caller to the two-pass kernel instead (same bits)
+    if (dev->capturing && !dev->unary_lut[TI][RT_EXP]) return RT_OK;
     const uint16_t* table = nullptr;
     int rc = rt_unary_table(dev, TI, RT_EXP, &table);
     if (rc) return rc;

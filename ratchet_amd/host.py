@@ -66,12 +66,16 @@ def load():
         fn = getattr(H, name)
         fn.argtypes = args
         fn.restype = i
+    H.rth_memory_plan.argtypes = [vp, u64p, i, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int64), i]
+    H.rth_memory_plan.restype = i
     H.rth_last_resolve_launches.argtypes = [vp]
     H.rth_last_resolve_launches.restype = ctypes.c_long
     H.rth_id.argtypes = [vp]
     H.rth_id.restype = ctypes.c_uint64
     H.rth_pool_stats.argtypes = [vp, u64p]
     H.rth_pool_stats.restype = i
+    H.rth_pool_peak.argtypes = [vp, u64p, i]
+    H.rth_pool_peak.restype = i
     H.rth_set_pattern_fusion.argtypes = [i]
     H.rth_set_pattern_fusion.restype = None
     _h = H
@@ -106,6 +110,13 @@ class HostDevice:
         if self.H.rth_pool_stats(self.handle, out) != 0:
             _raise()
         return tuple(int(v) for v in out)
+
+    def pool_peak(self, reset=False):
+        """the most bytes handed out at one time since the last reset"""
+        out = (ctypes.c_uint64 * 1)()
+        if self.H.rth_pool_peak(self.handle, out, int(bool(reset))) != 0:
+            _raise()
+        return int(out[0])
 
     def close(self):
         if self.handle:
@@ -247,6 +258,19 @@ class Tensor:
 
     def last_resolve_launches(self):
         return int(self.H.rth_last_resolve_launches(self.handle))
+
+    def memory_plan(self):
+        """(object_bytes, entries) of the plan resolve() would follow; entries are dicts id / bytes / object / source in
+        execution order (object -1: own allocation, -2: in place in a buffer that exists already)"""
+        nobj = ctypes.c_int(0)
+        n = self.H.rth_memory_plan(self.handle, None, 0, ctypes.byref(nobj), None, 0)
+        if n < 0:
+            _raise()
+        objs = (ctypes.c_uint64 * max(nobj.value, 1))()
+        ent = (ctypes.c_int64 * max(4 * n, 1))()
+        self.H.rth_memory_plan(self.handle, objs, nobj.value, ctypes.byref(nobj), ent, n)
+        entries = [dict(id=int(ent[4 * k]), bytes=int(ent[4 * k + 1]), object=int(ent[4 * k + 2]), source=int(ent[4 * k + 3])) for k in range(n)]
+        return [int(objs[k]) for k in range(nobj.value)], entries
 
     def execution_order(self):
         n = self.H.rth_execution_order(self.handle, _u64([0]), 0)

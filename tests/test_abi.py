@@ -34,6 +34,28 @@ def test_header_and_library_agree(lib):
     assert sorted(_lib.EXPORTS) == declared
 
 
+def test_rust_binding_in_integration_md_lists_the_header_s_entry_points():
+    """INTEGRATION.md shows the `extern "C"` block a ratchet maintainer would put into the -sys crate; it has to name every
+    entry point ratchet_hip.h declares, no other, each with as many arguments as the C declaration has"""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    header = open(os.path.join(root, "include", "ratchet_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    c_decls = {m.group(1): m.group(2) for m in re.finditer(r"\b(rt_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", header)}
+    doc = open(os.path.join(root, "INTEGRATION.md")).read()
+    block = doc[doc.index('extern "C" {'):]
+    block = block[:block.index("\n}\n")]
+    block = re.sub(r"//[^\n]*", "", block)
+    rust_decls = {m.group(1): m.group(2) for m in re.finditer(r"pub fn (rt_[a-z0-9_]+)\s*\((.*?)\)\s*->", block, flags=re.S)}
+    assert sorted(rust_decls) == sorted(c_decls)
+
+    def count(args, void_word):
+        args = args.strip()
+        return 0 if args in ("", void_word) else args.count(",") + 1
+
+    for name in c_decls:
+        assert count(rust_decls[name], "") == count(c_decls[name], "void"), name
+
+
 def test_status_names(lib):
     for code, name in _lib.STATUS_NAMES.items():
         assert lib.rt_status_name(code).decode() == name
