@@ -226,6 +226,44 @@ def copy_ceiling(dev):
             "frac_of_peak": round(2 * src.nbytes / ms / 1e6 / PEAK_HBM_GBPS, 4)}
 
 
+def copy_reference(dev, ops, steps):
+    """The floor under every row of the per-op table: the step once more, every op replaced by a plain copy kernel that
+    moves the same number of bytes (half read, half written) through fresh regions of two 1 GiB buffers, timed exactly
+    like the per-op pass (HIP events around each launch, the launches of a step back to back).  What a row's `us` exceeds
+    its copy by is the op's own cost; what the copy itself falls short of the roofline by (a launch and the cache
+    write-back and invalidation at a kernel boundary cost about 4 us whatever the kernel does) no kernel design recovers.
+    Also times a 16-byte fill launched right after a large kernel: that boundary cost alone."""
+    import ctypes
+
+    from ratchet_amd import _lib
+
+    src, dst = ops_extra["copy_pair"]
+    ev = [(dev.event(), dev.event()) for _ in ops]
+    floor_ev = (dev.event(), dev.event())
+    us = [[] for _ in ops]
+    floor_us = []
+    tiny = dev.empty((4,), F32)
+    off = 0
+    for _ in range(steps):
+        for o, (e0, e1) in zip(ops, ev):
+            half = min((o.alg_bytes // 2) & ~15, src.nbytes)       # (the mask add moves 16 MB more per side than the buffers hold)
+            if off + half > src.nbytes:
+                off = 0
+            assert off + half <= src.nbytes and off + half <= dst.nbytes
+            e0.record()
+            _lib.check(dev.lib.rt_cast(dev.handle, F16, F16, ctypes.c_void_p(src.ptr.value + off), ctypes.c_void_p(dst.ptr.value + off), half // 2))
+            e1.record()
+            off += half
+        floor_ev[0].record()
+        tiny.zero_()
+        floor_ev[1].record()
+        dev.sync()
+        for k, (e0, e1) in enumerate(ev):
+            us[k].append(e0.elapsed_ms(e1) * 1e3)
+        floor_us.append(floor_ev[0].elapsed_ms(floor_ev[1]) * 1e3)
+    return [float(np.median(u)) for u in us], float(np.median(floor_us))
+
+
 def one_pass_patterns(dev, seed, oracle):
     """The models wrap 16-bit norms, softmax and activations in full() ... cast(dt); the library has one-pass entry points
     for those sequences.  Reported beside the step (never part of `value`): time of the one-pass launch and of the op
@@ -579,6 +617,7 @@ def main():
             oracle.set_reference_copies(True)
 
     ceiling = copy_ceiling(dev) if not args.ops else None      # after the parity check: it overwrites an output buffer
+    copy_us, boundary_us = copy_reference(dev, ops, args.steps) if not args.ops else ([None] * len(ops), None)
     patterns = one_pass_patterns(dev, seed, oracle if not args.no_check else None) if not (args.ops or args.no_patterns) else None
     decode = decode_step(dev, seed) if not (args.ops or args.no_patterns) else None
 
@@ -606,6 +645,9 @@ def main():
         rows.append({"cfg": o.cfg, "op": o.name, "dtype": o.dtype, "shape": o.shapes, "alg_MB": round(o.alg_bytes / 1e6, 3),
                      "us": round(med, 2), "us_mean": round(float(np.mean(o.us)), 2), "GBps": round(gbps, 1),
                      "frac_hbm": round(gbps / PEAK_HBM_GBPS, 4),
+                     # a plain copy kernel moving the same bytes, timed the same way in the same place of the step
+                     "copy_us": None if copy_us[pos - 1] is None else round(copy_us[pos - 1], 2),
+                     "frac_of_copy": None if copy_us[pos - 1] is None else round(copy_us[pos - 1] / med, 4),
                      # the kernel alone (rocprofv3 --kernel-trace of this script, profiles/): `us` adds the two events and the launch gap
                      "kernel_us": kernel_us(pos),
                      "kernel_frac_hbm": None if not kernel_us(pos) else round(o.alg_bytes / (kernel_us(pos) * 1e-6) / 1e9 / PEAK_HBM_GBPS, 4),
@@ -637,6 +679,8 @@ def main():
             "loop_only": None if loop_t == 0 else {"value": round(cpu_b / loop_t / 1e9, 4), "unit": "GB/s", "seconds": round(loop_t, 2)},
             "host_cpus": os.cpu_count()},
         "hbm_copy_ceiling": ceiling,
+        # a 16-byte fill launched right behind a 21 MB permute, HIP events around it: what one more kernel boundary costs
+        "kernel_boundary_us": None if boundary_us is None else round(boundary_us, 2),
         "one_pass_patterns": patterns,
         "decode_step": decode,
         "parity_ok": bool(parity_ok) if not args.no_check else None,
