@@ -264,3 +264,43 @@ def test_storage_pool_reuses_blocks_in_stream_order(oracle):
         assert d.lib.rt_free(d.handle, ctypes.c_void_p(0x1000)) == 7      # not a block of this pool
     finally:
         d.close()
+
+
+@pytest.mark.parametrize("n", [(1 << 21), (1 << 21) + 8, 5 * 32768 * 64 + 32768 * 7 + 8 * 100 + 5, 32768 * 300 - 1])
+def test_unary_table_path_tiles_and_remainders(dev, oracle, n):
+    """the table kernel walks whole 64 KiB tiles with the next tile's loads in flight and hands the rest (fewer vectors
+    than a tile, fewer elements than a vector) to one block: every element once, none beyond the end"""
+    rng = np.random.default_rng(123)
+    x = rng.integers(0, 65536, n).astype(np.uint16).view(np.float16)
+    want = oracle.unary("silu", x)
+    big = dev.upload(np.full(n + 24, 7.25, np.float16))
+    from ratchet_amd.runtime import BufferView
+
+    out = BufferView(big, 8, (n,))
+    dev.unary("silu", dev.upload(x), out=out)
+    got = out.to_numpy()
+    assert np.all((got.view(np.uint16) == want.view(np.uint16)) | (np.isnan(got) & np.isnan(want)))
+    whole = big.to_numpy()
+    assert (whole[:8] == 7.25).all() and (whole[8 + n:] == 7.25).all()
+
+
+@pytest.mark.parametrize("a_shape,b_shape", [((1, 4, 256, 512), (1, 1, 256, 512)), ((1, 1, 256, 512), (1, 4, 256, 512)), ((1, 4, 256, 1), (1, 1, 1, 512)),
+                                             ((2, 3, 64, 40), (2, 3, 64, 40)), ((1, 4, 256, 512), (512,)), ((3, 5, 7, 9), (1, 5, 1, 9))])
+def test_broadcast_binary_streaming_variants(dev, oracle, a_shape, b_shape):
+    """each side of rt_binary_bcast is streamed past the caches when it has no broadcast dim and cached when it repeats:
+    the four instantiations (and the scalar one for odd rows) give the same bits as the oracle on materialised operands"""
+    from ratchet_amd import _lib
+    from ratchet_amd._lib import check
+    from ratchet_amd.runtime import shape4
+
+    rng = np.random.default_rng(124)
+    a, b = randn(rng, a_shape, np.float16), randn(rng, b_shape, np.float16)
+    shape = np.broadcast_shapes(a_shape, b_shape)
+    for op in ("add", "mul", "div"):
+        want = oracle.binary(op, np.ascontiguousarray(np.broadcast_to(a, shape)), np.ascontiguousarray(np.broadcast_to(b, shape)))
+        da, db = dev.upload(a), dev.upload(b)
+        out = dev.empty(shape, da.dt)
+        # through rt_binary_bcast also when the shapes are equal (both sides streamed)
+        check(dev.lib.rt_binary_bcast(dev.handle, _lib.BINARY_OPS.index(op), da.dt, da.ptr, shape4(a_shape), db.ptr, shape4(b_shape), out.ptr,
+                                      shape4(shape)))
+        assert same_bits(out.to_numpy(), want), (op, a_shape, b_shape)

@@ -418,6 +418,24 @@ def test_norms_f16(dev, oracle, shape):
     assert mismatch_count(got, want) == 0, mismatch_count(got, want)
 
 
+@pytest.mark.parametrize("rows,cols,kind", [(13, 2560, "f16"), (2048, 4096, "f16"), (2051, 3072, "bf16"), (5, 8, "bf16"), (300, 264, "f16"),   # all blocks resident: output pass from LDS
+                                            (40000, 256, "f16"), (9000, 1536, "bf16"), (64, 4104, "f16")])                              # more blocks than fit, rows too long: x re-read
+def test_norms_16_bit_both_output_passes(dev, oracle, rows, cols, kind):
+    """the 16-bit reference norms keep the raw rows, scale and bias in LDS for the output pass when every block of the
+    launch is resident at once, and re-read x otherwise: same bits either way, with and without bias, ragged last block"""
+    rng = np.random.default_rng(315)
+    bf = kind == "bf16"
+    conv = (lambda a: _bf16(oracle, a)) if bf else (lambda a: np.asarray(a, np.float32).astype(np.float16))
+    x = conv(rng.standard_normal((rows, cols)) * 1.5 + 0.25)
+    w = conv(1 + 0.02 * rng.standard_normal(cols))
+    b = conv(0.02 * rng.standard_normal(cols))
+    dx, dw, db = dev.upload(x, bf16=bf), dev.upload(w, bf16=bf), dev.upload(b, bf16=bf)
+    for name, want, got in (("layer", oracle.layer_norm(x, w, b, 1e-5, bf16=bf, intended=True), dev.layer_norm(dx, dw, db, 1e-5).to_numpy()),
+                            ("layer, no bias", oracle.layer_norm(x, w, None, 1e-5, bf16=bf, intended=True), dev.layer_norm(dx, dw, None, 1e-5).to_numpy()),
+                            ("rms", oracle.rms_norm(x, w, 1e-5, bf16=bf, intended=True), dev.rms_norm(dx, dw, 1e-5).to_numpy())):
+        assert np.array_equal(np.asarray(got).view(np.uint16), np.asarray(want).view(np.uint16)), (name, rows, cols, kind)
+
+
 @pytest.mark.parametrize("rows,cols,kind", [(20000, 8, "f16"), (16384 + 3, 64, "f16"), (17000, 128, "f16"), (30000, 24, "bf16"), (16500, 120, "bf16")])
 def test_norms_16_bit_many_narrow_rows(dev, oracle, rows, cols, kind):
     """tens of thousands of rows of at most 128 columns take a kernel with one lane per row; same bits as the walkers"""
