@@ -20,12 +20,30 @@ struct GatherArgs {
     uint64_t base;           // source offset of dst[0,0,0,0], in vectors (elements for the splat kernel)
     uint64_t s[4];           // source strides per destination dim, in vectors (elements for the splat kernel)
     uint32_t nvec;           // destination vectors
+    // Block order for a swap of two outer dims with short rows (K/V heads: [S, H, 80] -> [H, S, 80] in f16, 160-byte
+    // rows): the source rows of neighbouring heads share 128-byte lines, and in destination order those heads are
+    // 40 blocks apart, on another XCD, so every shared line is fetched twice (FETCH_SIZE 1.6x the tensor).  Hardware
+    // block b runs on XCD b % 8; with rm_h > 0 an XCD's consecutive blocks take the same rows of rm_h consecutive
+    // heads (rm_j blocks per head, a multiple of 8), and the second head finds the line in that XCD's L2.
+    FastDiv rm_h;
+    uint32_t rm_j;
 };
+
+__device__ __forceinline__ uint32_t gather_block(const GatherArgs& p) {
+    uint32_t blk = blockIdx.x;
+    if (p.rm_j) {
+        const uint32_t xcd = blk & 7u;
+        uint32_t jj, h;
+        fd_divmod(blk >> 3, p.rm_h, jj, h);
+        blk = h * p.rm_j + jj * 8u + xcd;
+    }
+    return blk;
+}
 
 // one VecT per thread-iteration; source contiguous along the destination's last dim (s[3] == 1)
 template <typename VecT>
 __global__ void __launch_bounds__(BLOCK) gather_vec_kernel(const VecT* __restrict__ x, VecT* __restrict__ y, GatherArgs p) {
-    const uint32_t base = blockIdx.x * (BLOCK * UNROLL) + threadIdx.x;
+    const uint32_t base = gather_block(p) * (BLOCK * UNROLL) + threadIdx.x;
     VecT r[UNROLL];
 #pragma unroll
     for (int k = 0; k < UNROLL; k++) {
@@ -423,6 +441,20 @@ int launch_gather(rt_device* dev, int eb, const void* x, void* y, const uint32_t
     p.d1 = make_fastdiv(dst_shape[1]);
     p.nvec = (uint32_t)nvec;
     const unsigned blocks = blocks_for(nvec, BLOCK * UNROLL);
+    p.rm_h = make_fastdiv(1);
+    p.rm_j = 0;
+    if (!splat && dst_shape[1] > 1 && dst_shape[2] > 1 && S[1] != 0 && S[1] < S[2] && (row_bytes % 128) != 0) {
+        // dim 1 lies closer together in the source than dim 2 and the rows do not fill whole lines
+        const uint64_t slice_vec = (uint64_t)dst_shape[2] * dst_shape[3] / per;
+        const uint64_t heads = (uint64_t)dst_shape[0] * dst_shape[1];
+        if (slice_vec % (BLOCK * UNROLL) == 0) {
+            const uint64_t j = slice_vec / (BLOCK * UNROLL);
+            if (j % 8 == 0 && j * heads == blocks) {
+                p.rm_h = make_fastdiv((uint32_t)heads);
+                p.rm_j = (uint32_t)j;
+            }
+        }
+    }
     if (splat) {
         p.base = base_elems;
         for (int i = 0; i < 4; i++) p.s[i] = S[i];
