@@ -311,6 +311,13 @@ struct MaskArgs {
     uint32_t ms[3];          // mask row strides in elements over dims 0..2 (0 where the mask extent is 1)
     uint32_t mlast;          // 1: the mask has a full last dim, 0: one value per row
     uint32_t mvec;           // the mask starts on a 16-byte boundary (the span kernel may read it in aligned vectors)
+    // Block order of the one-wave-per-row kernel for a large mask that repeats over the leading dims (an [S, T] mask
+    // under B * H heads): hardware block b runs on XCD b % 8, so the `reps` blocks that need the same four mask rows go
+    // to one XCD back to back and its L2 fetches them once; an XCD takes 2^chunk_log2 of its row blocks per repeat
+    // before it moves to the next repeat (as in the broadcast add, rt_elementwise.hip).  slabs (blocks per repeat) == 0:
+    // plain order.
+    FastDiv reps;
+    uint32_t slabs, chunk_log2;
 };
 
 template <typename T> __device__ __forceinline__ uint64_t mask_row_offset(uint64_t row, const MaskArgs& p) {
@@ -329,7 +336,14 @@ __device__ __forceinline__ float via32_exp(float v) { return __builtin_amdgcn_ex
 template <typename T, int NV, int MODE, bool MASK, int LANES>
 __global__ void __launch_bounds__(BLOCK) softmax_via32_wave_kernel(const T* __restrict__ x, const T* __restrict__ mask,
                                                                    T* __restrict__ y, uint64_t rows, uint32_t cols, MaskArgs p) {
-    const uint64_t row = (uint64_t)blockIdx.x * (BLOCK / LANES) + (threadIdx.x / LANES);
+    uint32_t blk = blockIdx.x;
+    if (MASK && LANES == WAVE && p.slabs) {
+        uint32_t rep, chunk;
+        const uint32_t idx = blk >> 3;
+        fd_divmod(idx >> p.chunk_log2, p.reps, chunk, rep);
+        blk = rep * p.slabs + ((chunk << p.chunk_log2) + (idx & ((1u << p.chunk_log2) - 1))) * 8u + (blk & 7u);
+    }
+    const uint64_t row = (uint64_t)blk * (BLOCK / LANES) + (threadIdx.x / LANES);
     if (row >= rows) return;
     const int lane = threadIdx.x & (LANES - 1);
     const uint32_t nvec = cols / 8;
@@ -807,6 +821,9 @@ extern "C" int rt_softmax_via_f32(rt_device* dev, int io_dt, const void* x, cons
     p.ms[0] = p.ms[1] = p.ms[2] = 0;
     p.mlast = 0;
     p.mvec = mask && rt_aligned(mask, 16) ? 1u : 0u;
+    p.reps = make_fastdiv(1);
+    p.slabs = 0;
+    p.chunk_log2 = 0;
     bool mask_vec_ok = true;
     if (mask) {
         uint64_t st = 1;
@@ -818,6 +835,26 @@ extern "C" int rt_softmax_via_f32(rt_device* dev, int io_dt, const void* x, cons
             st *= mask_shape[i];
         }
         mask_vec_ok = !p.mlast || (rt_aligned(mask, 16) && cols % 8 == 0);
+        // a mask of whole trailing dims, at least 1 MiB, repeated over the leading ones, whose period is whole groups of
+        // eight 4-row blocks: the XCD-aware block order (used by the one-wave-per-row kernel only)
+        int lead = 0;
+        while (lead < 3 && mask_shape[lead] == 1) lead++;
+        bool whole = p.mlast && lead > 0;
+        uint64_t period = 1, reps = 1;
+        for (int i = 0; i < 3; i++) {
+            if (i < lead) reps *= x_shape[i];
+            else {
+                period *= x_shape[i];
+                if (mask_shape[i] != x_shape[i]) whole = false;
+            }
+        }
+        if (whole && reps > 1 && reps <= 0xffffffffull && period * cols * 2 >= (1u << 20) && period % (WAVES * 8) == 0 &&
+            rows / WAVES <= 0xffffffffull) {
+            p.reps = make_fastdiv((uint32_t)reps);
+            p.slabs = (uint32_t)(period / WAVES);
+            const uint32_t per_xcd = p.slabs / 8;
+            p.chunk_log2 = per_xcd % 64 == 0 ? 6 : per_xcd % 4 == 0 ? 2 : 0;
+        }
     }
     if (io_dt == RT_F16) return dispatch_via32<half_t>(dev, x, mask, y, rows, cols, p, mask_vec_ok, mode);
     return dispatch_via32<bf16_t>(dev, x, mask, y, rows, cols, p, mask_vec_ok, mode);
