@@ -134,7 +134,7 @@ def _attn_case(rng, B, H, S, T, mask_kind, dtype=np.float16):
                                                (1, 2, 6, 8192, "causal"), (2, 1, 3, 16384, "per_batch"), (1, 2, 4, 6000, None),
                                                (1, 1, 2, 16392, None),
                                                # masks of 1 MiB and more under several heads: the XCD-aware block order (chunks of 64, 4, 1)
-                                               (3, 2, 2048, 512, "causal"), (1, 3, 160, 4096, "causal"),
+                                               (2, 2, 2048, 2048, "causal"), (1, 3, 160, 4096, "causal"),
                                                # rows that are not whole vectors (prompts of 1001, 333, 13 tokens): the span kernel
                                                (1, 4, 1001, 1001, "causal"), (2, 3, 333, 333, "causal4"), (1, 2, 5, 13, "causal"),
                                                (2, 2, 9, 1004, "per_batch"), (1, 3, 1, 2047, None), (1, 2, 3, 4101, "causal"),
