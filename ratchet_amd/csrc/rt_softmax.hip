@@ -311,13 +311,13 @@ struct MaskArgs {
     uint32_t ms[3];          // mask row strides in elements over dims 0..2 (0 where the mask extent is 1)
     uint32_t mlast;          // 1: the mask has a full last dim, 0: one value per row
     uint32_t mvec;           // the mask starts on a 16-byte boundary (the span kernel may read it in aligned vectors)
-    // Block order of the one-wave-per-row kernel for a large mask that repeats over the leading dims (an [S, T] mask
-    // under B * H heads): hardware block b runs on XCD b % 8, so the `reps` blocks that need the same four mask rows go
-    // to one XCD back to back and its L2 fetches them once; an XCD takes 2^chunk_log2 of its row blocks per repeat
-    // before it moves to the next repeat (as in the broadcast add, rt_elementwise.hip).  slabs (blocks per repeat) == 0:
-    // plain order.
+    // Block order of the kernels with whole rows per block (four with a wave per row, one with a block per row) for a
+    // large mask that repeats over the leading dims (an [S, T] mask under B * H heads): hardware block b runs on XCD
+    // b % 8, so the `reps` blocks that need the same mask rows go to one XCD back to back and its L2 fetches them once;
+    // an XCD takes a chunk of its row blocks (64 when they divide, else 4, else 1) per repeat before it moves to the
+    // next repeat (as in the broadcast add, rt_elementwise.hip).  period (mask rows, a multiple of 32) == 0: plain order.
     FastDiv reps;
-    uint32_t slabs, chunk_log2;
+    uint32_t period;
 };
 
 template <typename T> __device__ __forceinline__ uint64_t mask_row_offset(uint64_t row, const MaskArgs& p) {
@@ -337,11 +337,14 @@ template <typename T, int NV, int MODE, bool MASK, int LANES>
 __global__ void __launch_bounds__(BLOCK) softmax_via32_wave_kernel(const T* __restrict__ x, const T* __restrict__ mask,
                                                                    T* __restrict__ y, uint64_t rows, uint32_t cols, MaskArgs p) {
     uint32_t blk = blockIdx.x;
-    if (MASK && LANES == WAVE && p.slabs) {
+    if (MASK && (LANES == WAVE || LANES == BLOCK) && p.period) {
+        const uint32_t slabs = p.period / (BLOCK / LANES);               // blocks per repeat, a multiple of 8
+        const uint32_t per_xcd = slabs >> 3;
+        const uint32_t cl = per_xcd % 64 == 0 ? 6 : per_xcd % 4 == 0 ? 2 : 0;
         uint32_t rep, chunk;
         const uint32_t idx = blk >> 3;
-        fd_divmod(idx >> p.chunk_log2, p.reps, chunk, rep);
-        blk = rep * p.slabs + ((chunk << p.chunk_log2) + (idx & ((1u << p.chunk_log2) - 1))) * 8u + (blk & 7u);
+        fd_divmod(idx >> cl, p.reps, chunk, rep);
+        blk = rep * slabs + ((chunk << cl) + (idx & ((1u << cl) - 1))) * 8u + (blk & 7u);
     }
     const uint64_t row = (uint64_t)blk * (BLOCK / LANES) + (threadIdx.x / LANES);
     if (row >= rows) return;
@@ -615,7 +618,14 @@ template <typename T, int MODE, bool SPAN> int launch_wave(rt_device* dev, const
         RT_CHECK_LAUNCH("softmax_wave_kernel");
         return RT_OK;
     }
-    if (nvec <= (uint32_t)(WAVE * 8)) {
+    // One wave per row up to 320 vectors (five loads per lane) in reference mode; beyond that the block shares the row,
+    // so that a thread has two or three loads and stores of its own: a kernel tends to move more bytes per second the
+    // fewer accesses each thread issues before it ends.  Measured cold, wave / block per row: [1,6,1500,1500] f32 (375
+    // vectors) 23.2 / 21.7 us (21.8 / 20.0 by the profiler inside the benchmark step), [8192,2048] f32 25.3 / 24.7 us;
+    // [4096,1280] f32 (320 vectors) 8.2 / 10.4 us the other way, and the stable mode on 16-bit rows loses with the block
+    // ([65536,2560] f16 145 / 173 us), so it keeps the wave up to 512 vectors.
+    constexpr uint32_t WAVE_ROW_MAX = MODE == 0 ? WAVE * 5 : WAVE * 8;
+    if (nvec <= WAVE_ROW_MAX) {
         const uint32_t nv = (nvec + WAVE - 1) / WAVE;
         const uint64_t blocks = (rows + WAVES - 1) / WAVES;
         RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax: too many rows");
@@ -708,7 +718,9 @@ int launch_via32(rt_device* dev, const void* x, const void* mask, void* y, uint6
         RT_CHECK_LAUNCH("softmax_via32_wave_kernel");
         return RT_OK;
     }
-    if (vec_ok && nvec <= (uint32_t)(WAVE * 8)) {
+    // (beyond 320 vectors the block shares the row in reference mode, as in launch_wave: [32768,4096] f16 90.3 -> 85.1 us,
+    // with a [4096,4096] mask under 32 heads 365 -> 346 us)
+    if (vec_ok && nvec <= (uint32_t)(MODE == 0 ? WAVE * 5 : WAVE * 8)) {
         const uint32_t nv = (nvec + WAVE - 1) / WAVE;
         const uint64_t blocks = (rows + WAVES - 1) / WAVES;
         RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax_via_f32: too many rows");
@@ -822,8 +834,7 @@ extern "C" int rt_softmax_via_f32(rt_device* dev, int io_dt, const void* x, cons
     p.mlast = 0;
     p.mvec = mask && rt_aligned(mask, 16) ? 1u : 0u;
     p.reps = make_fastdiv(1);
-    p.slabs = 0;
-    p.chunk_log2 = 0;
+    p.period = 0;
     bool mask_vec_ok = true;
     if (mask) {
         uint64_t st = 1;
@@ -849,11 +860,9 @@ extern "C" int rt_softmax_via_f32(rt_device* dev, int io_dt, const void* x, cons
             }
         }
         if (whole && reps > 1 && reps <= 0xffffffffull && period * cols * 2 >= (1u << 20) && period % (WAVES * 8) == 0 &&
-            rows / WAVES <= 0xffffffffull) {
+            rows <= 0x7fffffffull) {
             p.reps = make_fastdiv((uint32_t)reps);
-            p.slabs = (uint32_t)(period / WAVES);
-            const uint32_t per_xcd = p.slabs / 8;
-            p.chunk_log2 = per_xcd % 64 == 0 ? 6 : per_xcd % 4 == 0 ? 2 : 0;
+            p.period = (uint32_t)period;
         }
     }
     if (io_dt == RT_F16) return dispatch_via32<half_t>(dev, x, mask, y, rows, cols, p, mask_vec_ok, mode);
