@@ -97,6 +97,8 @@ __global__ void __launch_bounds__(BLOCK) binary_bcast_kernel(const T* __restrict
         blk = rep * p.slabs + ((chunk << p.chunk_log2) + (idx & ((1u << p.chunk_log2) - 1))) * XCDS + (blk % XCDS);
     }
     const uint32_t base = blk * (BLOCK * BC_UNROLL) + threadIdx.x;
+    // every load of the thread's BC_UNROLL vectors is issued before the first store
+    T ra[BC_UNROLL][VE], rb[BC_UNROLL][VE];
 #pragma unroll
     for (int k = 0; k < BC_UNROLL; k++) {
         const uint32_t v = base + k * BLOCK;
@@ -109,45 +111,47 @@ __global__ void __launch_bounds__(BLOCK) binary_bcast_kernel(const T* __restrict
                             (uint64_t)col * VE * p.as[3];
         const uint64_t bo = (uint64_t)i0 * p.bs[0] + (uint64_t)i1 * p.bs[1] + (uint64_t)i2 * p.bs[2] +
                             (uint64_t)col * VE * p.bs[3];
-        T ra[VE], rb[VE], r[VE];
         if (VE > 1 && p.as[3] == 1) {
             Vec16<T> t16;
             const v4u* q = reinterpret_cast<const v4u*>(a + ao);
             t16.u = (ONCE & 1) ? ld_stream(q) : *q;
 #pragma unroll
-            for (int e = 0; e < VE; e++) ra[e] = t16.e[e];
+            for (int e = 0; e < VE; e++) ra[k][e] = t16.e[e];
         } else if (p.as[3] == 0) {
             const T one = a[ao];                                  // broadcast along the last dim: one load, splatted
 #pragma unroll
-            for (int e = 0; e < VE; e++) ra[e] = one;
+            for (int e = 0; e < VE; e++) ra[k][e] = one;
         } else {
 #pragma unroll
-            for (int e = 0; e < VE; e++) ra[e] = a[ao + (uint64_t)e * p.as[3]];
+            for (int e = 0; e < VE; e++) ra[k][e] = a[ao + (uint64_t)e * p.as[3]];
         }
         if (VE > 1 && p.bs[3] == 1) {
             Vec16<T> t16;
             const v4u* q = reinterpret_cast<const v4u*>(b + bo);
             t16.u = (ONCE & 2) ? ld_stream(q) : *q;
 #pragma unroll
-            for (int e = 0; e < VE; e++) rb[e] = t16.e[e];
+            for (int e = 0; e < VE; e++) rb[k][e] = t16.e[e];
         } else if (p.bs[3] == 0) {
             const T one = b[bo];                                  // broadcast along the last dim: one load, splatted
 #pragma unroll
-            for (int e = 0; e < VE; e++) rb[e] = one;
+            for (int e = 0; e < VE; e++) rb[k][e] = one;
         } else {
 #pragma unroll
-            for (int e = 0; e < VE; e++) rb[e] = b[bo + (uint64_t)e * p.bs[3]];
+            for (int e = 0; e < VE; e++) rb[k][e] = b[bo + (uint64_t)e * p.bs[3]];
         }
+    }
 #pragma unroll
-        for (int e = 0; e < VE; e++) r[e] = ar_binary<OP, T>(ra[e], rb[e]);
+    for (int k = 0; k < BC_UNROLL; k++) {
+        const uint32_t v = base + k * BLOCK;
+        if (v >= p.nvec) break;
         const uint64_t yo = (uint64_t)v * VE;
         if (VE > 1) {
             Vec16<T> t16;
 #pragma unroll
-            for (int e = 0; e < VE; e++) t16.e[e] = r[e];
+            for (int e = 0; e < VE; e++) t16.e[e] = ar_binary<OP, T>(ra[k][e], rb[k][e]);
             st_stream(reinterpret_cast<v4u*>(y + yo), t16.u);
         } else {
-            y[yo] = r[0];
+            y[yo] = ar_binary<OP, T>(ra[k][0], rb[k][0]);
         }
     }
 }
