@@ -35,8 +35,9 @@ def test_header_and_library_agree(lib):
 
 
 def test_rust_binding_in_integration_md_lists_the_header_s_entry_points():
-    """INTEGRATION.md shows the `extern "C"` block a ratchet maintainer would put into the -sys crate; it has to name every
-    entry point ratchet_hip.h declares, no other, each with as many arguments as the C declaration has"""
+    """the integration guide at the repository root shows the `extern "C"` block a ratchet maintainer would put into the
+    -sys crate; it has to name every entry point ratchet_hip.h declares, no other, each with as many arguments as the C
+    declaration has"""
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     header = open(os.path.join(root, "include", "ratchet_hip.h")).read()
     header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
