@@ -414,6 +414,64 @@ def decode_step(dev, seed):
             "note": "eager = nine calls through ctypes on the device's stream; replay = one hipGraphLaunch of the captured sequence"}
 
 
+def host_graph_step(seed):
+    """The same decode-layer ops as a lazy graph through the host mirror of the reference's Tensor API: built, planned and
+    resolved every step, as the reference's models do, against one dispatch of the graph compiled once (Executable)."""
+    from ratchet_amd import host
+
+    np16, np32 = np.float16, np.float32
+    H, D, N, T = 32, 80, 2560, 2047
+    hd = host.HostDevice(0)
+    up = lambda a: host.Tensor.from_numpy(a, hd)
+    table, ids = up(normal(seed, 951, (4096, N), 1.0, np16)), up(np.array([1234], np.int32))
+    w32, b32 = up(normal(seed, 952, (N,), 0.02, np32, mean=1.0)), up(normal(seed, 953, (N,), 0.02, np32))
+    kc, knew = up(np.zeros((1, H, 2048, D), np16)), up(normal(seed, 955, (1, H, 1, D), 1.0, np16))
+    scores = up(normal(seed, 957, (1, H, 1, T + 1), 2.0, np16))
+    ff = up(normal(seed, 958, (1, 4 * N), 1.0, np16))
+
+    def build():
+        x = table.index_select(ids, 0)                                               # embedding row
+        h = x.full().layer_norm(w32, b32, 1e-5).cast(F16)                            # one launch (caller pattern)
+        k = knew.full().rope(32, 10000.0, T).cast(F16)                               # rotary in f32, as the CPU op has it
+        return [x.add(h),                                                            # residual
+                kc.cache(k, 2, T),                                                   # KV append
+                scores.full().softmax(3).cast(F16),                                  # attention weights, one launch
+                ff.full().gelu().cast(F16)]                                          # MLP activation, one launch
+
+    def resolve_all():
+        for r in build():
+            r.resolve()
+
+    roots = build()
+    exes = [r.compile() for r in roots]
+    launches = sum(e.launches for e in exes)
+
+    def dispatch_all():
+        for e in exes[:-1]:
+            e.dispatch(wait=False)
+        exes[-1].dispatch()
+
+    def timed(fn, n=100):
+        fn()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        return (time.perf_counter() - t0) / n * 1e6
+
+    resolve_us, dispatch_us = timed(resolve_all), timed(dispatch_all)
+    held = sum(e.held_bytes for e in exes)
+    for e in exes:
+        e.close()
+    del roots
+    hd.close()
+    return {"graphs": "index_select + layer_norm(via f32) + add, cache(cast(rope(full))), softmax(via f32), gelu(via f32) at Phi-2 decode shapes",
+            "launches": launches, "build_plan_resolve_us": round(resolve_us, 1), "executable_dispatch_us": round(dispatch_us, 1),
+            "executable_held_bytes": held,
+            "note": "resolve = graph building, pattern matching, memory plan, launches and a wait per graph, through ctypes; "
+                    "dispatch = the launch list each compiled graph keeps, on the buffers of its memory plan (one hipGraphLaunch from "
+                    "eight launches on, call by call below that), one wait"}
+
+
 def download_rows(dev, buf, nrows, row_elems, np_dtype):
     """first nrows rows (row_elems each) of a device buffer"""
     import ctypes
@@ -620,6 +678,7 @@ def main():
     copy_us, boundary_us = copy_reference(dev, ops, args.steps) if not args.ops else ([None] * len(ops), None)
     patterns = one_pass_patterns(dev, seed, oracle if not args.no_check else None) if not (args.ops or args.no_patterns) else None
     decode = decode_step(dev, seed) if not (args.ops or args.no_patterns) else None
+    host_step = host_graph_step(seed) if not (args.ops or args.no_patterns) else None
 
     # the kernels' own durations and HBM-side bytes, from the committed rocprofv3 summaries (whole step only: rows are by position)
     kt_rows = read_step_rows(PROFILE_KERNEL_TRACE) if not args.ops else {}
@@ -683,6 +742,7 @@ def main():
         "kernel_boundary_us": None if boundary_us is None else round(boundary_us, 2),
         "one_pass_patterns": patterns,
         "decode_step": decode,
+        "host_graph_step": host_step,
         "parity_ok": bool(parity_ok) if not args.no_check else None,
         "ops": rows,
         "wall_s": round(wall, 3), "setup_s": round(t_setup, 2),

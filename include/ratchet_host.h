@@ -20,6 +20,7 @@ extern "C" {
 
 typedef struct rth_device rth_device;
 typedef struct rth_tensor rth_tensor;
+typedef struct rth_executable rth_executable;
 
 const char* rth_last_error(void);
 const char* rth_last_error_kind(void);
@@ -73,6 +74,20 @@ int rth_execution_order(const rth_tensor* t, uint64_t* ids, int cap);  /* ids in
  * Returns the number of launches (entries beyond entry_cap are not written), -1 on error. */
 int rth_memory_plan(const rth_tensor* t, uint64_t* object_bytes, int object_cap, int* n_objects, int64_t* entries, int entry_cap);
 uint64_t rth_id(const rth_tensor* t);
+
+/* The compiled form of a graph: what the reference's Executable is to a command buffer (executable.rs:13-59), this is
+ * to a HIP graph.  rth_compile resolves t (it runs the graph once) and records the same launches, on buffers assigned
+ * once by the memory plan, for replay; rth_executable_dispatch replays them with one submission (fewer than eight
+ * launches: call by call, which costs less than a graph launch; wait != 0: returns after completion, like rth_resolve).  Shapes, offsets and buffer addresses are fixed at compile time: new input data
+ * goes into the graph's constant tensors with rth_update_from_host, results are read from t with rth_to_host.  The
+ * executable keeps every buffer of the graph alive; release it with rth_executable_release.  NULL on error. */
+rth_executable* rth_compile(rth_tensor* t);
+int rth_executable_dispatch(rth_executable* exe, int wait);
+long rth_executable_launches(const rth_executable* exe);              /* kernels per dispatch */
+uint64_t rth_executable_held_bytes(const rth_executable* exe);        /* device memory of the intermediates it keeps */
+void rth_executable_release(rth_executable* exe);
+/* overwrite the contents of a tensor that has storage (numel * element size bytes are read from data) */
+int rth_update_from_host(rth_tensor* t, const void* data);
 
 #ifdef __cplusplus
 }

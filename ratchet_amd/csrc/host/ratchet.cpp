@@ -492,7 +492,35 @@ struct FusedPlan {
     uint64_t x_off = 0, up_off = 0, x_stride = 0, up_stride = 0;   // GatedMul views, in elements
 };
 
+// Everything resolve() decides before the first launch: which nodes run, which are folded into a neighbour, what
+// each launch reads, and the memory plan.
+struct PreparedGraph {
+    std::vector<Node*> order;                                  // needed nodes, execution order
+    std::unordered_set<Node*> skip;
+    std::unordered_map<Node*, FusedPlan> fused;
+    std::vector<planner::Step> steps;                          // one per launch
+    std::vector<Node*> step_node;
+    std::vector<std::vector<Node*>> step_reads;                // the nodes behind Step::reads
+    std::unordered_map<Node*, size_t> step_of;
+    std::vector<std::vector<Node*>> release_at;                // per index into order: nodes whose storage handle is dropped after it
+    planner::Plan plan;
+};
+
+struct Executable::Inner {
+    Device device;
+    rt_graph* graph = nullptr;                // the recorded launches; null for a short list, which is re-issued call by call
+    size_t launches = 0;
+    size_t held = 0;
+    PreparedGraph prepared;                   // the launch list and what each launch reads
+    std::vector<std::shared_ptr<Buffer>> storage;   // per entry of prepared.order: the buffer the node had after the first run
+    std::shared_ptr<Node> root;               // keeps the graph's nodes, and with them its constants' storage
+    ~Inner() {
+        if (graph) rt_graph_destroy(graph);
+    }
+};
+
 struct Resolver {
+    typedef PreparedGraph Prepared;
     // a Broadcast node nobody else holds, not yet materialised, feeding a Binary: fused into the binary kernel
     static bool fusable_broadcast(const Tensor& operand) {
         Node* b = Node::of(operand);
@@ -839,27 +867,15 @@ struct Resolver {
         }
     }
 
-    // Everything resolve() decides before the first launch: which nodes run, which are folded into a neighbour, what
-    // each launch reads, and the memory plan.
-    struct Prepared {
-        std::vector<Node*> order;                                  // needed nodes, execution order
-        std::unordered_set<Node*> skip;
-        std::unordered_map<Node*, FusedPlan> fused;
-        std::vector<planner::Step> steps;                          // one per launch
-        std::vector<Node*> step_node;
-        std::vector<std::vector<Node*>> step_reads;                // the nodes behind Step::reads
-        std::unordered_map<Node*, size_t> step_of;
-        std::vector<std::vector<Node*>> release_at;                // per index into order: nodes whose storage handle is dropped after it
-        planner::Plan plan;
-    };
-
     // the node whose buffer is read when `t` is an operand: through views (which alias their source)
     static Node* base_of(Node* n) {
         while (n->kind == Kind::View && !n->storage) n = Node::of(n->srcs[0]);
         return n;
     }
 
-    static Prepared prepare(Node* root) {
+    // for_replay: the launches will run more than once (Executable), so nothing may work in place in a buffer that holds
+    // an input of the graph
+    static Prepared prepare(Node* root, bool for_replay = false) {
         Prepared P;
         const std::vector<Node*> full_order = execution_order(root);
         // only what the root still needs: nothing below a tensor that already has its storage (tensor.rs:783 skips those;
@@ -943,6 +959,7 @@ struct Resolver {
 
         // The launches and what each reads, for the memory plan (gpu/buffer_allocator/allocator.rs:141-271).
         auto launches_here = [&](Node* n) { return !n->storage && !skip.count(n) && n->kind != Kind::View && !n->srcs.empty(); };
+        std::unordered_set<Node*> in_input;                        // results that live in a buffer which existed before this graph
         for (Node* n : order) {
             if (!launches_here(n)) continue;
             planner::Step st;
@@ -973,8 +990,12 @@ struct Resolver {
                            (n->kind == Kind::Binary && !fusable_broadcast(n->srcs[0]) && !fusable_broadcast(n->srcs[1]))) {
                     in_place = Node::holders(s0T) == 1 && s0->shape == n->shape && s0->dt == n->dt && s0->kind != Kind::View &&
                                (s0->storage ? s0->storage.use_count() == 1 : true);
+                    if (for_replay && (s0->storage || in_input.count(s0))) in_place = false;
                 }
-                if (in_place) st.inplace = (int)(std::find(reads.begin(), reads.end(), base_of(s0)) - reads.begin());
+                if (in_place) {
+                    st.inplace = (int)(std::find(reads.begin(), reads.end(), base_of(s0)) - reads.begin());
+                    if (base_of(s0)->storage || in_input.count(base_of(s0))) in_input.insert(n);
+                }
             }
             for (Node* r : reads) st.reads.push_back(r->id);
             P.step_of[n] = P.steps.size();
@@ -1018,7 +1039,123 @@ struct Resolver {
         check_rt(rt_sync(root->device.raw()), "rt_sync");      // resolve returns after completion (tensor.rs:855-856)
         root->last_launches = launches;
     }
+
+    // Issues the launches of a compiled graph once more on the buffers of its first run: the nodes get their buffers back
+    // for the duration of the call (hidden intermediates drop theirs after resolve, the executable keeps them).
+    static void replay(Executable::Inner& in) {
+        const Prepared& P = in.prepared;
+        std::vector<size_t> lent;
+        for (size_t i = 0; i < P.order.size(); i++)
+            if (!P.order[i]->storage && in.storage[i]) {
+                P.order[i]->storage = in.storage[i];
+                lent.push_back(i);
+            }
+        auto give_back = [&] {
+            for (size_t i : lent) P.order[i]->storage.reset();
+        };
+        try {
+            size_t launches = 0;
+            for (Node* n : P.order) {
+                if (!P.step_of.count(n)) continue;
+                auto f = P.fused.find(n);
+                if (f != P.fused.end()) run_fused(n, f->second, launches);
+                else run(n, launches);
+            }
+        } catch (...) {
+            give_back();
+            throw;
+        }
+        give_back();
+    }
+
+    // A shorter launch list is re-issued call by call: measured on this stack, a graph launch costs 32-35 us up to its
+    // completion whatever it holds, a list of n small kernels issued one by one about 10 + 3 n us.
+    static constexpr size_t GRAPH_MIN_LAUNCHES = 8;
+
+    // resolve() that keeps its buffers and its launch list.  The first run is a plain one (it also builds the lookup
+    // tables and grows the scratch the kernels want, which a capture cannot); a list of GRAPH_MIN_LAUNCHES or more is then
+    // issued again on the same buffers while the device's stream is capturing.  Every buffer is assigned before the first
+    // launch and none is handed back between launches: the plan's shared objects are safe to share because a replay
+    // keeps the launch order.
+    static Executable compile(const std::shared_ptr<Node>& root_ref) {
+        Node* root = root_ref.get();
+        auto inner = std::make_shared<Executable::Inner>();
+        inner->prepared = prepare(root, true);
+        const Prepared& P = inner->prepared;
+        for (Node* n : P.order)
+            if (n->srcs.empty() && !n->storage)
+                throw Error("Unresolved", "constant tensor " + std::to_string(n->id) + " has no storage (placeholder)");
+        inner->device = root->device;
+        inner->root = root_ref;
+        std::vector<std::shared_ptr<Buffer>> objects(P.plan.object_bytes.size());
+        for (size_t o = 0; o < objects.size(); o++) {
+            objects[o] = std::make_shared<Buffer>(root->device, P.plan.object_bytes[o]);
+            inner->held += P.plan.object_bytes[o];
+        }
+        rt_device* dev = root->device.raw();
+        size_t launches = 0;
+        for (Node* n : P.order) {
+            auto st = P.step_of.find(n);
+            if (st != P.step_of.end()) {
+                const planner::Step& step = P.steps[st->second];
+                const int obj = P.plan.object_of.at(n->id);
+                if (step.inplace >= 0) {
+                    n->storage = P.step_reads[st->second][(size_t)step.inplace]->storage;
+                } else if (obj >= 0) {
+                    n->storage = objects[(size_t)obj];
+                } else {
+                    n->storage = std::make_shared<Buffer>(n->device, step.bytes);
+                    inner->held += step.bytes;
+                }
+                auto f = P.fused.find(n);
+                if (f != P.fused.end()) run_fused(n, f->second, launches);
+                else run(n, launches);
+            } else if (!n->storage && !P.skip.count(n)) {
+                run(n, launches);                                  // a view (no launch)
+            }
+        }
+        check_rt(rt_sync(dev), "rt_sync");
+        inner->launches = launches;
+        root->last_launches = launches;
+        // the executable now owns what the launches touch; the nodes look as they do after resolve()
+        for (Node* n : P.order) inner->storage.push_back(n->storage);
+        for (const std::vector<Node*>& dead_list : P.release_at)
+            for (Node* dead : dead_list) dead->storage.reset();
+        if (launches >= GRAPH_MIN_LAUNCHES) {
+            check_rt(rt_capture_begin(dev), "rt_capture_begin");
+            try {
+                replay(*inner);
+            } catch (...) {                                        // leave the device usable: close the capture, drop what it recorded
+                rt_graph* g = nullptr;
+                if (rt_capture_end(dev, &g) == RT_OK && g) rt_graph_destroy(g);
+                throw;
+            }
+            check_rt(rt_capture_end(dev, &inner->graph), "rt_capture_end");
+        }
+        Executable exe;
+        exe.inner_ = inner;
+        return exe;
+    }
 };
+
+void Executable::dispatch(bool wait) const {
+    if (!inner_) throw Error("NullExecutable", "dispatch on an empty executable");
+    if (inner_->graph) check_rt(rt_graph_launch(inner_->device.raw(), inner_->graph), "rt_graph_launch");
+    else if (inner_->launches) Resolver::replay(*inner_);
+    if (wait) check_rt(rt_sync(inner_->device.raw()), "rt_sync");
+}
+size_t Executable::launches() const { return inner_ ? inner_->launches : 0; }
+size_t Executable::held_bytes() const { return inner_ ? inner_->held : 0; }
+
+Executable Tensor::compile() const {
+    if (!node_) throw Error("NullTensor", "compile on an empty tensor");
+    return Resolver::compile(node_);
+}
+
+void Tensor::update_from_host(const void* data) const {
+    if (!resolved()) throw Error("Unresolved", "update_from_host needs a tensor that has storage");
+    check_rt(rt_h2d(node_->device.raw(), node_->storage->ptr, data, numel() * size_of(dt())), "rt_h2d");
+}
 
 MemoryPlan Tensor::memory_plan() const {
     if (!node_) throw Error("NullTensor", "memory_plan on an empty tensor");

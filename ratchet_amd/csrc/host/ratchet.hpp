@@ -112,6 +112,27 @@ struct MemoryPlan {
     std::vector<Entry> entries;
 };
 
+// The compiled form of a graph: the reference's Executable is the ordered list of compiled ops that dispatch() encodes
+// into one command buffer and submits once (executable.rs:13-59, built by resolve_gpu, tensor.rs:795-859).  Here the
+// list is a HIP graph over buffers assigned once by the memory plan: dispatch() is one graph launch, whatever the number
+// of kernels (a list of fewer than eight launches is re-issued call by call instead, which is cheaper than a graph
+// launch: no graph building, pattern matching, planning or allocation either way).  Shapes, offsets (cache, rope, index_write) and buffer addresses are fixed at compile(); new input data
+// goes into the graph's constant tensors with Tensor::update_from_host, and the output tensor's buffer is rewritten by
+// every dispatch.  The executable keeps every buffer of the graph alive, intermediates included.
+class Executable {
+  public:
+    Executable() {}
+    // replays all launches of the graph in order; wait = return after completion, as resolve() does (tensor.rs:855-856)
+    void dispatch(bool wait = true) const;
+    size_t launches() const;                                  // kernels per dispatch
+    size_t held_bytes() const;                                // device memory of the intermediates this executable keeps
+
+  private:
+    struct Inner;
+    std::shared_ptr<Inner> inner_;
+    friend struct Resolver;
+};
+
 class Tensor {
   public:
     Tensor() {}
@@ -176,8 +197,14 @@ class Tensor {
 
     // tensor.rs:861-863: runs every unresolved node this tensor depends on; returns after completion
     Tensor resolve() const;
+    // resolve() that also keeps the launch list: runs the graph once (so this tensor is resolved on return), then records
+    // the same launches on the same buffers into an Executable.  An op is not run in place in a buffer that existed
+    // before the call (a replay would apply it to its own result); cache and index_write still update their destination.
+    Executable compile() const;
     // to(&Device::CPU) + to_vec (tensor.rs:957-975): blocking download of the resolved tensor
     void to_host(void* out) const;
+    // overwrite the contents of a resolved tensor (numel * size_of(dt) bytes), e.g. an input of a compiled graph
+    void update_from_host(const void* data) const;
     // number of kernel launches the last resolve() of this tensor issued (for tests)
     size_t last_resolve_launches() const;
 

@@ -15,6 +15,9 @@ struct rth_device {
 struct rth_tensor {
     Tensor t;
 };
+struct rth_executable {
+    Executable exe;
+};
 
 static thread_local std::string g_msg, g_kind;
 
@@ -185,6 +188,36 @@ int rth_memory_plan(const rth_tensor* t, uint64_t* object_bytes, int object_cap,
     } catch (const std::exception& e) {
         capture(e);
         return -1;
+    }
+}
+
+rth_executable* rth_compile(rth_tensor* t) {
+    try {
+        return new rth_executable{t->t.compile()};
+    } catch (const std::exception& e) {
+        capture(e);
+        return nullptr;
+    }
+}
+int rth_executable_dispatch(rth_executable* exe, int wait) {
+    try {
+        exe->exe.dispatch(wait != 0);
+        return 0;
+    } catch (const std::exception& e) {
+        capture(e);
+        return 1;
+    }
+}
+long rth_executable_launches(const rth_executable* exe) { return (long)exe->exe.launches(); }
+uint64_t rth_executable_held_bytes(const rth_executable* exe) { return (uint64_t)exe->exe.held_bytes(); }
+void rth_executable_release(rth_executable* exe) { delete exe; }
+int rth_update_from_host(rth_tensor* t, const void* data) {
+    try {
+        t->t.update_from_host(data);
+        return 0;
+    } catch (const std::exception& e) {
+        capture(e);
+        return 1;
     }
 }
 

@@ -78,6 +78,18 @@ def load():
     H.rth_pool_peak.restype = i
     H.rth_set_pattern_fusion.argtypes = [i]
     H.rth_set_pattern_fusion.restype = None
+    H.rth_compile.argtypes = [vp]
+    H.rth_compile.restype = vp
+    H.rth_executable_dispatch.argtypes = [vp, i]
+    H.rth_executable_dispatch.restype = i
+    H.rth_executable_launches.argtypes = [vp]
+    H.rth_executable_launches.restype = ctypes.c_long
+    H.rth_executable_held_bytes.argtypes = [vp]
+    H.rth_executable_held_bytes.restype = ctypes.c_uint64
+    H.rth_executable_release.argtypes = [vp]
+    H.rth_executable_release.restype = None
+    H.rth_update_from_host.argtypes = [vp, vp]
+    H.rth_update_from_host.restype = i
     _h = H
     return H
 
@@ -122,6 +134,38 @@ class HostDevice:
         if self.handle:
             self.H.rth_device_release(self.handle)
             self.handle = None
+
+
+class Executable:
+    """The recorded launch list of a compiled graph (the reference's Executable, executable.rs:13-59, as a HIP graph)."""
+
+    def __init__(self, handle):
+        self.H = load()
+        self.handle = handle
+
+    def dispatch(self, wait=True):
+        if self.H.rth_executable_dispatch(self.handle, int(bool(wait))) != 0:
+            _raise()
+        return self
+
+    @property
+    def launches(self):
+        return int(self.H.rth_executable_launches(self.handle))
+
+    @property
+    def held_bytes(self):
+        return int(self.H.rth_executable_held_bytes(self.handle))
+
+    def close(self):
+        if self.handle:
+            self.H.rth_executable_release(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 class Tensor:
@@ -258,6 +302,22 @@ class Tensor:
 
     def last_resolve_launches(self):
         return int(self.H.rth_last_resolve_launches(self.handle))
+
+    def compile(self):
+        """resolve() that also records its launches: returns the Executable that replays them with one graph launch"""
+        h = self.H.rth_compile(self.handle)
+        if not h:
+            _raise()
+        return Executable(h)
+
+    def update(self, a):
+        """overwrite the contents of a tensor that has storage (an input of a compiled graph) with array `a`"""
+        a = np.ascontiguousarray(a)
+        if a.nbytes != int(np.prod(self.shape, dtype=np.int64)) * np.dtype(_DT_TO_NP[self.dt]).itemsize:
+            raise ValueError("update: the array does not have the tensor's size")
+        if self.H.rth_update_from_host(self.handle, a.ctypes.data_as(ctypes.c_void_p)) != 0:
+            _raise()
+        return self
 
     def memory_plan(self):
         """(object_bytes, entries) of the plan resolve() would follow; entries are dicts id / bytes / object / source in

@@ -191,3 +191,10 @@ def test_placeholders_cannot_be_resolved():
     with pytest.raises(HostError) as e:
         P(2, 3).gelu().resolve()
     assert e.value.kind == "Unresolved"
+
+
+def test_placeholders_cannot_be_compiled():
+    # compile() is resolve() plus a recording of its launches: the same precondition, checked before anything is allocated
+    with pytest.raises(HostError) as e:
+        P(2, 3).gelu().tanh().compile()
+    assert e.value.kind == "Unresolved"
