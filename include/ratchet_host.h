@@ -33,6 +33,12 @@ int rth_pool_peak(rth_device* dev, uint64_t* peak_live_bytes, int reset);   /* r
 
 /* Tensor::from_data + to(device) (tensor.rs:553-571,874-892); dt codes as in ratchet_hip.h */
 rth_tensor* rth_from_host(rth_device* dev, const void* data, int rank, const uint64_t* shape, int dt);
+/* Tensor::from_quantized (tensor.rs:618-628): dt 5 = Q8_0F, 6 = Q8_0H (codes that continue ratchet_hip.h's); data is the
+ * quantized buffer as the reference lays it out (quant.rs:19-49: numel signed bytes packed four to a word, padded to 256
+ * bytes, then numel / 32 scales of f32 / f16, padded to 256 bytes: rth_storage_bytes in all).  Such a tensor can only be
+ * the source of rth_index_select (ops/select.rs:107-111), whose result has the scales' type. */
+rth_tensor* rth_from_quantized(rth_device* dev, const void* data, int rank, const uint64_t* shape, int dt);
+uint64_t rth_storage_bytes(int rank, const uint64_t* shape, int dt);
 /* shape-only constant without storage: graph building and its errors can be exercised without a GPU; cannot be resolved */
 rth_tensor* rth_placeholder(int rank, const uint64_t* shape, int dt);
 void rth_release(rth_tensor* t);

@@ -14,14 +14,24 @@
 namespace ratchet {
 
 // ------------------------------------------------------------------------------------------------------------ basics
-size_t size_of(DType dt) { return (dt == DType::F16 || dt == DType::BF16) ? 2 : 4; }
+size_t size_of(DType dt) { return is_quantized(dt) ? 0 : (dt == DType::F16 || dt == DType::BF16) ? 2 : 4; }
 bool is_float(DType dt) { return dt == DType::F32 || dt == DType::F16 || dt == DType::BF16; }
+bool is_quantized(DType dt) { return dt == DType::Q8_0F || dt == DType::Q8_0H; }
+DType activation_dt(DType dt) { return dt == DType::Q8_0F ? DType::F32 : dt == DType::Q8_0H ? DType::F16 : dt; }
+static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+size_t storage_bytes(const Shape& shape, DType dt) {
+    const size_t n = shape.numel();
+    if (!is_quantized(dt)) return n * size_of(dt);
+    return align256(n) + align256(n / 32 * size_of(activation_dt(dt)));
+}
 const char* as_str(DType dt) {
     switch (dt) {
         case DType::F32: return "F32";
         case DType::F16: return "F16";
         case DType::BF16: return "BF16";
         case DType::I32: return "I32";
+        case DType::Q8_0F: return "Q8_0F";
+        case DType::Q8_0H: return "Q8_0H";
         default: return "U32";
     }
 }
@@ -138,6 +148,10 @@ static std::shared_ptr<Node> new_node(Kind k, const Shape& shape, DType dt, cons
 static void require_same_device(const Tensor& a, const Tensor& b) {
     if (!(a.device() == b.device())) throw Error("DeviceMismatch", "operands live on different devices");
 }
+// every op but index_select computes on plain element types
+static void require_plain(const Tensor& t, const char* who) {
+    if (is_quantized(t.dt())) throw Error("UnsupportedDType", std::string(who) + " on a quantized tensor (" + as_str(t.dt()) + ")");
+}
 static void require_rank4(const Shape& s, const char* who) {
     if (s.rank() == 0 || s.rank() > 4) throw Error("RankMismatch", std::string(who) + ": rank " + std::to_string(s.rank()) + " (1..4 supported)");
 }
@@ -174,8 +188,20 @@ const char* Tensor::op_name() const {
     }
 }
 
+Tensor Tensor::from_quantized(const void* data, const Shape& shape, DType dt, const Device& device) {
+    require_rank4(shape, "from_quantized");
+    if (!is_quantized(dt)) throw Error("UnsupportedDType", std::string("from_quantized takes a quantized type, got ") + as_str(dt));
+    if (shape.numel() % 32 != 0) throw Error("ShapeMismatch", "a Q8_0 tensor holds whole groups of 32 elements (quant.rs:20-21)");
+    auto n = new_node(Kind::Const, shape, dt, device);
+    const size_t bytes = storage_bytes(shape, dt);
+    n->storage = std::make_shared<Buffer>(device, bytes);
+    check_rt(rt_h2d(device.raw(), n->storage->ptr, data, bytes), "rt_h2d");
+    return Tensor(n);
+}
+
 Tensor Tensor::from_host(const void* data, const Shape& shape, DType dt, const Device& device) {
     require_rank4(shape, "from_host");
+    if (is_quantized(dt)) throw Error("UnsupportedDType", "quantized data comes in through from_quantized");
     auto n = new_node(Kind::Const, shape, dt, device);
     const size_t bytes = shape.numel() * size_of(dt);
     n->storage = std::make_shared<Buffer>(device, bytes);
@@ -184,6 +210,7 @@ Tensor Tensor::from_host(const void* data, const Shape& shape, DType dt, const D
 }
 Tensor Tensor::zeros(const Shape& shape, DType dt, const Device& device) {
     require_rank4(shape, "zeros");
+    if (is_quantized(dt)) throw Error("UnsupportedDType", as_str(dt));
     auto n = new_node(Kind::Const, shape, dt, device);
     const size_t bytes = shape.numel() * size_of(dt);
     n->storage = std::make_shared<Buffer>(device, bytes);
@@ -287,6 +314,7 @@ Tensor Tensor::softmax(size_t dim, SoftmaxMode mode) const {
 }
 
 Tensor Tensor::slice(const std::vector<std::pair<size_t, size_t>>& ranges) const {
+    require_plain(*this, "slice");
     if (ranges.size() != rank()) throw Error("RankMismatch", "slice needs one range per dimension");
     std::vector<size_t> out;
     for (size_t i = 0; i < ranges.size(); i++) {
@@ -303,6 +331,7 @@ Tensor Tensor::slice(const std::vector<std::pair<size_t, size_t>>& ranges) const
 }
 
 Tensor Tensor::view(const Shape& shape_) const {
+    require_plain(*this, "view");
     if (shape_.rank() != rank()) throw Error("RankMismatch", "view keeps the rank (View::check_shapes)");
     if (shape_.numel() != numel()) throw Error("ShapeMismatch", "view keeps the element count");
     auto n = new_node(Kind::View, shape_, dt(), device());
@@ -315,6 +344,7 @@ Tensor Tensor::cat(const std::vector<Tensor>& tensors, size_t dim) {
     if (tensors.size() < 2 || tensors.size() > 8) throw Error("ConcatArity", std::to_string(tensors.size()) + " inputs (2..8 supported)");
     const Tensor& first = tensors[0];
     require_rank4(first.shape(), "cat");
+    require_plain(first, "cat");
     if (dim >= first.rank()) throw Error("DimOutOfRange", "cat dim " + std::to_string(dim));
     size_t stacked = 0;
     for (const Tensor& t : tensors) {
@@ -336,6 +366,7 @@ Tensor Tensor::cat(const std::vector<Tensor>& tensors, size_t dim) {
 // Cache guards: ops/cache.rs:124-133
 Tensor Tensor::cache(const Tensor& source, size_t dim, size_t offset) const {
     require_same_device(*this, source);
+    require_plain(*this, "cache");
     if (rank() < 3 || rank() > 4) throw Error("RankMismatch", "cache needs rank 3 or 4");
     if (source.rank() != rank()) throw Error("RankMismatch", "cache and source must have one rank");
     if (dt() != source.dt()) throw Error("DTypeMismatch", std::string("expected ") + as_str(dt()) + ", got " + as_str(source.dt()));
@@ -375,10 +406,12 @@ Tensor Tensor::index_select(const Tensor& indices, size_t dim) const {
     if (indices.rank() != 1) throw Error("RankMismatch", "index_select indices must have rank 1, got " + std::to_string(indices.rank()));
     if (indices.dt() != DType::I32) throw Error("DTypeMismatch", std::string("expected I32, got ") + as_str(indices.dt()));
     if (dim >= rank()) throw Error("DimOutOfRange", "index_select dim " + std::to_string(dim));
-    if (size_of(dt()) != 2 && size_of(dt()) != 4) throw Error("UnsupportedDType", as_str(dt()));
+    // a Q8_0 table: whole words of four elements along the row, as the reference's kernel reads them (ops/select.rs:144-161)
+    if (is_quantized(dt()) && (dim != 0 || shape()[1] % 4 != 0))
+        throw Error("ShapeMismatch", "index_select from a quantized table takes rows (dim 0) of a multiple of 4 columns");
     Shape out = shape();
     out[dim] = indices.shape()[0];
-    auto n = new_node(Kind::IndexSelect, out, dt(), device());
+    auto n = new_node(Kind::IndexSelect, out, activation_dt(dt()), device());      // compute_view, ops/select.rs:48-60
     n->dim = dim;
     n->srcs = {*this, indices};
     return Tensor(n);
@@ -387,6 +420,7 @@ Tensor Tensor::index_select(const Tensor& indices, size_t dim) const {
 // IndexWrite has no guards in the reference (ops/index_write.rs:29-33); the run it writes must stay inside dst
 Tensor Tensor::index_write(const Tensor& src, const std::vector<size_t>& write_start) const {
     require_same_device(*this, src);
+    require_plain(*this, "index_write");
     require_rank4(shape(), "index_write");
     if (dt() != src.dt()) throw Error("DTypeMismatch", std::string("expected ") + as_str(dt()) + ", got " + as_str(src.dt()));
     if (write_start.size() != rank()) throw Error("RankMismatch", "write_start must have one entry per dimension");
@@ -403,6 +437,7 @@ Tensor Tensor::index_write(const Tensor& src, const std::vector<size_t>& write_s
 }
 
 Tensor Tensor::permute(const std::vector<size_t>& dims) const {
+    require_plain(*this, "permute");
     if (dims.size() != rank()) throw Error("RankMismatch", "permute needs one index per dimension");    // Permute::check_shapes
     std::vector<bool> seen(rank(), false);
     std::vector<size_t> out(rank());
@@ -419,6 +454,7 @@ Tensor Tensor::permute(const std::vector<size_t>& dims) const {
 }
 
 Tensor Tensor::broadcast_to(const Shape& to) const {
+    require_plain(*this, "broadcast_to");
     require_rank4(to, "broadcast_to");
     if (rank() > to.rank())
         throw Error("InvalidBroadcast", "source has more dimensions than the target: " + shape().to_string() + " -> " + to.to_string());
@@ -823,6 +859,15 @@ struct Resolver {
                 uint32_t ss[4];
                 shape4(src(0)->shape, ss);
                 out_buffer();
+                if (is_quantized(src(0)->dt)) {
+                    const char* base = static_cast<const char*>(src(0)->storage->ptr);
+                    check_rt(rt_index_select_q8_0(dev, dt, reinterpret_cast<const uint32_t*>(base), base + align256(src(0)->shape.numel()), ss,
+                                                  static_cast<const int32_t*>(src(1)->storage->ptr), (uint32_t)src(1)->shape[0],
+                                                  (int)(n->dim + 4 - n->shape.rank()), n->storage->ptr),
+                             "rt_index_select_q8_0");
+                    launches++;
+                    return;
+                }
                 check_rt(rt_index_select(dev, (int)size_of(n->dt), src(0)->storage->ptr, ss, static_cast<const int32_t*>(src(1)->storage->ptr),
                                          (uint32_t)src(1)->shape[0], (int)(n->dim + 4 - n->shape.rank()), n->storage->ptr),
                          "rt_index_select");
@@ -1154,7 +1199,7 @@ Executable Tensor::compile() const {
 
 void Tensor::update_from_host(const void* data) const {
     if (!resolved()) throw Error("Unresolved", "update_from_host needs a tensor that has storage");
-    check_rt(rt_h2d(node_->device.raw(), node_->storage->ptr, data, numel() * size_of(dt())), "rt_h2d");
+    check_rt(rt_h2d(node_->device.raw(), node_->storage->ptr, data, storage_bytes(shape(), dt())), "rt_h2d");
 }
 
 MemoryPlan Tensor::memory_plan() const {
@@ -1181,7 +1226,7 @@ Tensor Tensor::resolve() const {
 
 void Tensor::to_host(void* out) const {
     if (!resolved()) throw Error("Unresolved", "to_host needs a resolved tensor (call resolve() first)");
-    check_rt(rt_d2h(node_->device.raw(), out, node_->storage->ptr, numel() * size_of(dt())), "rt_d2h");
+    check_rt(rt_d2h(node_->device.raw(), out, node_->storage->ptr, storage_bytes(shape(), dt())), "rt_d2h");
 }
 
 }  // namespace ratchet

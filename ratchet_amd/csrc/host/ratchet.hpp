@@ -30,10 +30,13 @@ struct Error : std::runtime_error {
     Error(const std::string& k, const std::string& msg) : std::runtime_error(k + ": " + msg), kind(k) {}
 };
 
-// dtype/mod.rs:12-23 (the quantized types are off this path)
-enum class DType { F32 = 0, F16 = 1, BF16 = 2, I32 = 3, U32 = 4 };
-size_t size_of(DType dt);
+// dtype/mod.rs:12-23.  Of the quantized types only Q8_0 is here, and only as the source of index_select (the embedding
+// table of a quantized model, ops/select.rs:107-111): every other op rejects it.
+enum class DType { F32 = 0, F16 = 1, BF16 = 2, I32 = 3, U32 = 4, Q8_0F = 5, Q8_0H = 6 };
+size_t size_of(DType dt);                                     // bytes per element; 0 for a quantized type
 bool is_float(DType dt);
+bool is_quantized(DType dt);
+DType activation_dt(DType dt);                                // dtype/mod.rs:99-107: what a quantized tensor dequantizes to
 const char* as_str(DType dt);
 
 // shape.rs: rank <= 4 on every path here
@@ -58,6 +61,9 @@ class Shape {
     std::vector<size_t> dims_;
 };
 std::vector<ptrdiff_t> contiguous_strides(const Shape& s);    // Strides::from(&Shape), strides.rs:85-96
+// bytes of a tensor's storage: numel * size_of, or for Q8_0 the two segments of dtype/blocks.rs:73-81 (numel signed
+// bytes, then numel / 32 scales of the activation type, each segment rounded up to 256 bytes)
+size_t storage_bytes(const Shape& shape, DType dt);
 
 enum class BinaryOp { Add = 0, Sub, Mul, Div };
 enum class UnaryOp { Gelu = 0, Tanh, Exp, Log, Sin, Cos, Abs, Sqrt, Relu, Floor, Ceil, Neg, Silu, Sigmoid };
@@ -138,6 +144,9 @@ class Tensor {
     Tensor() {}
     // Tensor::from_data + to(device): upload `numel * size_of(dt)` bytes (tensor.rs:553-571, 874-892)
     static Tensor from_host(const void* data, const Shape& shape, DType dt, const Device& device);
+    // Tensor::from_quantized (tensor.rs:618-628): `data` is the quantized buffer as quantize() lays it out (quant.rs:19-49),
+    // storage_bytes(shape, dt) bytes; numel must be a multiple of 32
+    static Tensor from_quantized(const void* data, const Shape& shape, DType dt, const Device& device);
     static Tensor zeros(const Shape& shape, DType dt, const Device& device);
     // A constant without storage or device: lets graph building (shape/dtype rules, errors, execution order) run on a
     // machine without a GPU.  resolve() on a graph that contains one fails.

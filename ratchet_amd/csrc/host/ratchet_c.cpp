@@ -62,6 +62,10 @@ int rth_pool_peak(rth_device* dev, uint64_t* peak_live_bytes, int reset) { retur
 rth_tensor* rth_from_host(rth_device* dev, const void* data, int rank, const uint64_t* shape, int dt) {
     return build([&] { return Tensor::from_host(data, make_shape(rank, shape), (DType)dt, dev->dev); });
 }
+rth_tensor* rth_from_quantized(rth_device* dev, const void* data, int rank, const uint64_t* shape, int dt) {
+    return build([&] { return Tensor::from_quantized(data, make_shape(rank, shape), (DType)dt, dev->dev); });
+}
+uint64_t rth_storage_bytes(int rank, const uint64_t* shape, int dt) { return (uint64_t)storage_bytes(make_shape(rank, shape), (DType)dt); }
 rth_tensor* rth_placeholder(int rank, const uint64_t* shape, int dt) {
     return build([&] { return Tensor::placeholder(make_shape(rank, shape), (DType)dt); });
 }

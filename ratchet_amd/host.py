@@ -22,6 +22,8 @@ _NP_TO_DT = {np.dtype(np.float32): _lib.F32, np.dtype(np.float16): _lib.F16, np.
              np.dtype(np.uint32): _lib.U32}
 _DT_TO_NP = {_lib.F32: np.float32, _lib.F16: np.float16, _lib.BF16: np.uint16, _lib.I32: np.int32, _lib.U32: np.uint32}
 
+Q8_0F, Q8_0H = 5, 6            # the quantized types of the host mirror (sources of index_select only)
+
 _h = None
 
 
@@ -52,7 +54,7 @@ def load():
     H.rth_release.argtypes = [vp]
     H.rth_release.restype = None
     for name, args in {
-        "rth_from_host": [vp, vp, i, u64p, i], "rth_placeholder": [i, u64p, i], "rth_binary": [vp, vp, i], "rth_unary": [vp, i],
+        "rth_from_host": [vp, vp, i, u64p, i], "rth_from_quantized": [vp, vp, i, u64p, i], "rth_placeholder": [i, u64p, i], "rth_binary": [vp, vp, i], "rth_unary": [vp, i],
         "rth_cast": [vp, i], "rth_layer_norm": [vp, vp, vp, f], "rth_rms_norm": [vp, vp, f], "rth_group_norm": [vp, sz, vp, vp, f],
         "rth_softmax": [vp, sz, i], "rth_slice": [vp, i, u64p, u64p], "rth_view": [vp, i, u64p],
         "rth_cat": [ctypes.POINTER(vp), i, sz], "rth_cache": [vp, vp, sz, sz], "rth_rope": [vp, sz, f, sz], "rth_index_select": [vp, vp, sz],
@@ -78,6 +80,8 @@ def load():
     H.rth_pool_peak.restype = i
     H.rth_set_pattern_fusion.argtypes = [i]
     H.rth_set_pattern_fusion.restype = None
+    H.rth_storage_bytes.argtypes = [i, u64p, i]
+    H.rth_storage_bytes.restype = ctypes.c_uint64
     H.rth_compile.argtypes = [vp]
     H.rth_compile.restype = vp
     H.rth_executable_dispatch.argtypes = [vp, i]
@@ -189,6 +193,22 @@ class Tensor:
         a = np.ascontiguousarray(a)
         dt = _lib.BF16 if bf16 else _NP_TO_DT[a.dtype]
         return Tensor(load().rth_from_host(device.handle, a.ctypes.data_as(ctypes.c_void_p), a.ndim, _u64(a.shape), dt))
+
+    @staticmethod
+    def from_quantized(words, scales, shape, device):
+        """Tensor::from_quantized (tensor.rs:618-628): `words` are the packed signed bytes (uint32, numel / 4 of them),
+        `scales` one f32 (Q8_0F) or f16 (Q8_0H) per group of 32; they are laid out as the reference's quantized buffer is
+        (quant.rs:19-49: each segment padded to 256 bytes)."""
+        words, scales = np.ascontiguousarray(words, np.uint32), np.ascontiguousarray(scales)
+        dt = {np.dtype(np.float32): Q8_0F, np.dtype(np.float16): Q8_0H}[scales.dtype]
+        total = int(load().rth_storage_bytes(len(shape), _u64(shape), dt))
+        buf = np.zeros(total, np.uint8)
+        scale_at = (words.nbytes + 255) & ~255
+        if scale_at + scales.nbytes > total:
+            raise ValueError("from_quantized: words / scales do not match the shape")
+        buf[:words.nbytes] = words.view(np.uint8).ravel()
+        buf[scale_at:scale_at + scales.nbytes] = scales.view(np.uint8).ravel()
+        return Tensor(load().rth_from_quantized(device.handle, buf.ctypes.data_as(ctypes.c_void_p), len(shape), _u64(shape), dt))
 
     @staticmethod
     def placeholder(shape, dt=_lib.F32):

@@ -331,6 +331,29 @@ def test_rope_index_select_index_write_graphs(hdev, oracle):
     assert np.array_equal(dst.to_numpy(), out.to_numpy())                      # in place: the destination's buffer is the result
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_embedding_lookup_from_a_quantized_table(hdev, oracle, dtype):
+    """Tensor::from_quantized + index_select (tensor.rs:618-628, ops/select.rs:48-60,107-111): the result has the scales'
+    type and is, bit for bit, dequantize-then-gather (cpu/mod.rs:86-103); followed by the models' next op on it."""
+    from ratchet_amd.host import Tensor
+
+    rng = np.random.default_rng(409)
+    for shape, idx in (((256, 32), [64, 192, 255]),                              # the reference's test shape (ops/select.rs:350-357)
+                       ((6400, 2560), rng.integers(0, 6400, 77))):               # embedding-table rows, prefill-sized gather
+        table = (rng.standard_normal(shape) * 0.05).astype(dtype)
+        words, scales = oracle.q8_0_quantize(table)
+        ids = np.asarray(idx, np.int32)
+        q = Tensor.from_quantized(words, scales, shape, hdev)
+        y = q.index_select(T(ids, hdev), 0)
+        assert y.shape == (len(ids), shape[1]) and y.dt == (0 if dtype == np.float32 else 1)
+        want = oracle.q8_0_index_select(words, scales, shape, ids, 0)
+        assert same_bits(y.resolve().to_numpy(), want) and y.last_resolve_launches() == 1
+        g = (1 + 0.1 * rng.standard_normal(shape[1])).astype(dtype)
+        z = q.index_select(T(ids, hdev), 0).rms_norm(T(g, hdev), 1e-5).resolve().to_numpy()
+        ok, info = close(oracle, z, oracle.rms_norm(want, g, 1e-5, intended=True), 1e-5 if dtype == np.float32 else 1e-3)
+        assert ok, info
+
+
 def test_intermediates_return_their_buffers_during_resolve(oracle):
     """What the reference's allocation planner achieves (gpu/buffer_allocator/allocator.rs:141-271): a long graph holds a few
     live buffers, not one per node.  Twelve alternating casts of an 8 MiB tensor (Cast never runs in place) need three

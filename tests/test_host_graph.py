@@ -198,3 +198,27 @@ def test_placeholders_cannot_be_compiled():
     with pytest.raises(HostError) as e:
         P(2, 3).gelu().tanh().compile()
     assert e.value.kind == "Unresolved"
+
+
+def test_quantized_tensors_are_sources_of_index_select_only():
+    # dtype/mod.rs:99-107 (activation_dt), ops/select.rs:48-60: the gather's result has the scales' type; nothing else
+    # computes on the packed bytes
+    from ratchet_amd.host import Q8_0F, Q8_0H
+
+    ids = Tensor.placeholder((5,), _lib.I32)
+    for qdt, act in ((Q8_0F, _lib.F32), (Q8_0H, _lib.F16)):
+        q = Tensor.placeholder((64, 32), qdt)
+        y = q.index_select(ids, 0)
+        assert y.shape == (5, 32) and y.dt == act
+        for bad in (lambda: q.gelu(), lambda: q.add(q), lambda: q.full(), lambda: q.softmax(1), lambda: q.permute((1, 0)),
+                    lambda: q.view((32, 64)), lambda: q.slice(((0, 1), (0, 32))), lambda: Tensor.cat([q, q], 0),
+                    lambda: q.broadcast_to((2, 64, 32)), lambda: q.rms_norm(Tensor.placeholder((32,), _lib.F32), 1e-5)):
+            with pytest.raises(HostError) as e:
+                bad()
+            assert e.value.kind in ("UnsupportedDType", "UnsupportedCast", "DTypeMismatch"), e.value.kind
+        with pytest.raises(HostError) as e:
+            q.index_select(ids, 1)                                   # rows only
+        assert e.value.kind == "ShapeMismatch"
+        with pytest.raises(HostError) as e:
+            Tensor.placeholder((64, 30), qdt).index_select(ids, 0)   # whole words of four along the row
+        assert e.value.kind == "ShapeMismatch"
