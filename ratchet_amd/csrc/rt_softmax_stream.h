@@ -44,6 +44,7 @@ constexpr int SP_TC = 512;                   // columns per step: 64 lanes x 8 h
 constexpr int SP_PAD = 8;
 constexpr int SP_PF = 2;                     // steps loaded ahead
 constexpr int SP_MAX_STEPS = 8;              // rows of up to 4096 columns
+constexpr double SP_PACE_BYTES_PER_S = 6.65e12;   // what the paced kernel asks of HBM, all blocks together (measured optimum 6.6-6.7e12)
 constexpr size_t SP_LUT_BYTES = 65536 * sizeof(uint16_t);
 constexpr size_t SP_TILE_BYTES = SP_ROWS * (SP_TC + SP_PAD) * sizeof(uint16_t);
 constexpr size_t SP_SMEM_BYTES = SP_LUT_BYTES + SP_TILE_BYTES + 2 * 32 * sizeof(uint16_t);      // 162 400 of the CU's 163 840 bytes
@@ -55,6 +56,14 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 // exp of two packed f16 bit patterns: two lookups in the full 65536-entry table (NaN, inf and the saturated ends included)
 __device__ __forceinline__ uint32_t sp_exp_pair(const uint16_t* lut, uint32_t p) {
     return (uint32_t)lut[p & 0xffffu] | ((uint32_t)lut[p >> 16] << 16);
+}
+
+// the 100 MHz wall clock (low 32 bits), read as one opaque block so that it does not take part in the scheduling of the
+// code around it
+__device__ __forceinline__ uint32_t sp_clock() {
+    uint64_t t;
+    asm volatile("s_memrealtime %0\n s_waitcnt lgkmcnt(0)" : "=s"(t) :: "memory");
+    return (uint32_t)t;
 }
 
 // Which 30-row groups a block works on.  Rows come in `reps` periods of P rows (P = all rows when nothing repeats; P = the
@@ -70,6 +79,7 @@ struct SpSched {
     FastDiv gp_div;
     FastDiv pm_div;          // rows of the mask: row (rep * P + r) of x takes mask row (rep * P + r) % PM.  PM == P unless the
     uint32_t PM;             // mask is only a few rows tall, where groups that stop at every period would be nearly empty
+    uint32_t pace;           // shortest time between two steps of a block, in ticks of the 100 MHz wall clock; 0: unpaced
 };
 
 __device__ __forceinline__ uint32_t sp_item_count(const SpSched& s, uint32_t b, uint32_t G) {
@@ -143,6 +153,10 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                                                                     uint64_t rows, uint32_t cols, SpSched sch, uint16_t* row_sums) {
     typedef SpType<T> ST;
     constexpr bool PARK = NSTEP > 0;
+    // Only the plain variant holds its steps to a pace (see launch_stream16).  The masked and ragged variants take longer
+    // per step than the pace by themselves, and the mere presence of the pacing code changed their register allocation
+    // and cost the masked one 6 % (390 -> 416 us), so for them it is compiled out.
+    constexpr bool PACED = !MASK && !RAGGED;
     static_assert(!RAGGED || (PARK && !FULL), "the ragged variant parks in registers and has no full-step shortcut");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint16_t* lut = reinterpret_cast<uint16_t*>(smem);
@@ -170,6 +184,9 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
         const v4u* trow = reinterpret_cast<const v4u*>(tile[wr]);
         typename ST::Run run = ST::zero();
         uint32_t gpar = 0;
+        // the blocks take their steps out of phase with each other: block b starts b / grid of a step late
+        uint32_t t_step = 0, free_steps = 0;
+        if constexpr (PACED) t_step = sp_clock() - sch.pace + (uint32_t)(((uint64_t)blockIdx.x * sch.pace) / gridDim.x);
         for (uint32_t it = 0; it < n_items; it++) {
             // RAGGED: a row that starts sh bytes into its first vector can reach up to 14 bytes past its last step.  That
             // one vector is fetched here, at the start of the group, and added after the group's last step.
@@ -199,6 +216,22 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
             }
 #pragma unroll 1
             for (uint32_t t = 0; t < nsteps; t++) {
+                if (PACED && sch.pace) {                     // the walker is the block's clock: see SpSched::pace
+                    if (free_steps) {                        // not looking at the clock; start timing again at the last of them
+                        if (--free_steps == 0) t_step = sp_clock();
+                    } else {
+                        uint32_t el = sp_clock() - t_step;
+                        if (el >= sch.pace + sch.pace / 4) {
+                            free_steps = 4;                  // the steps take longer than the pace by themselves: stay out of the way
+                        } else {
+                            while (el < sch.pace) {
+                                __builtin_amdgcn_s_sleep(1);
+                                el = sp_clock() - t_step;
+                            }
+                            t_step += sch.pace;
+                        }
+                    }
+                }
                 __syncthreads();                             // A
                 __syncthreads();                             // B: tile t is in LDS
                 // 16 values per chunk; the LDS reads of the next chunk are in flight during the 16 dependent adds
@@ -768,10 +801,26 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
             }
         }
         sch.GP = (sch.P + sch.R - 1) / sch.R;
+        sch.pace = 0;                                        // set below, once the grid is known
         sch.gp_div = make_fastdiv(sch.GP);
         const uint64_t items = (uint64_t)sch.GP * sch.reps;
         RT_REQUIRE(items <= 0xffffffffull, RT_ERR_SIZE, "rt_softmax: too many row groups");
         const unsigned blocks = (unsigned)(items < (uint64_t)dev->num_cus ? items : (uint64_t)dev->num_cus);   // one resident block per CU
+        // Pacing.  Left to itself the kernel offers HBM more requests than it sustains, and what it then gets is less than
+        // what it gets when it asks for slightly less: 366 us unpaced against 343 us on [1,32,4096,4096] in the benchmark
+        // step (a plain persistent copy loop shows the same: 5.9 TB/s unpaced, 6.4 TB/s with a sleep of the right length
+        // per iteration, and a write-only loop 4.4 against 6.6 TB/s).  So the walker holds the block's steps to the period
+        // at which all blocks together move SP_PACE_BYTES_PER_S, by the 100 MHz wall clock, and the blocks start out of
+        // phase.  A pace that is too fast gives the unpaced behaviour back (7.0e12: 359 us), one that is too slow costs
+        // in proportion (6.4e12: 355 us).  When the steps are slower than the pace by themselves (dense inputs, whose
+        // table lookups collide in the LDS banks; bf16) the walker stops looking at the clock for a few steps at a time.
+        // A grid that does not fill the chip is not paced.
+        if (blocks == dev->num_cus && !mask && !ragged) {
+            const double rate = SP_PACE_BYTES_PER_S;
+            const double group_bytes = (double)sch.R * cols * 2 * (nt > SP_MAX_STEPS ? 4 : 2);     // in and out (long rows: parked and read back)
+            const double steps = nt > SP_MAX_STEPS ? sch.nsteps : nt == 7 ? 8 : nt;          // the steps the kernel variant takes per group
+            sch.pace = (uint32_t)(group_bytes / steps * blocks / rate * 1e8 + 0.5);
+        }
         if (ragged) {
             if (mask) RT_SP_RAGGED_NS(true);
             else RT_SP_RAGGED_NS(false);
