@@ -120,6 +120,11 @@ int rt_device_create(int ordinal, rt_device** out) {
     dev->pool = new rt_pool();
     dev->ordinal = ordinal;
     dev->num_cus = prop.multiProcessorCount;
+    {
+        int khz = 0;
+        if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, ordinal) != hipSuccess) (void)hipGetLastError();
+        dev->wall_clock_hz = khz > 0 ? khz * 1e3 : 1e8;
+    }
     hipError_t e = hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking);   // default priority
     if (e != hipSuccess) {
         delete dev->pool;

@@ -14,6 +14,7 @@ struct rt_device {
     int ordinal;
     hipStream_t stream;
     int num_cus;
+    double wall_clock_hz;   // rate of the device's constant-frequency wall clock (s_memrealtime), 100 MHz on this chip
     // GroupNorm partial statistics: {mean, m2, count} triples, one per (group, split)
     float* gn_scratch;
     size_t gn_scratch_bytes;

@@ -79,7 +79,7 @@ struct SpSched {
     FastDiv gp_div;
     FastDiv pm_div;          // rows of the mask: row (rep * P + r) of x takes mask row (rep * P + r) % PM.  PM == P unless the
     uint32_t PM;             // mask is only a few rows tall, where groups that stop at every period would be nearly empty
-    uint32_t pace;           // shortest time between two steps of a block, in ticks of the 100 MHz wall clock; 0: unpaced
+    uint32_t pace;           // shortest time between two steps of a block, in ticks of the device's wall clock (100 MHz); 0: unpaced
 };
 
 __device__ __forceinline__ uint32_t sp_item_count(const SpSched& s, uint32_t b, uint32_t G) {
@@ -819,7 +819,7 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
             const double rate = SP_PACE_BYTES_PER_S;
             const double group_bytes = (double)sch.R * cols * 2 * (nt > SP_MAX_STEPS ? 4 : 2);     // in and out (long rows: parked and read back)
             const double steps = nt > SP_MAX_STEPS ? sch.nsteps : nt == 7 ? 8 : nt;          // the steps the kernel variant takes per group
-            sch.pace = (uint32_t)(group_bytes / steps * blocks / rate * 1e8 + 0.5);
+            sch.pace = (uint32_t)(group_bytes / steps * blocks / rate * dev->wall_clock_hz + 0.5);
         }
         if (ragged) {
             if (mask) RT_SP_RAGGED_NS(true);
