@@ -367,7 +367,11 @@ __global__ void __launch_bounds__(BLOCK) norm_seq16_kernel(const T* __restrict__
 // 8 rows per 320-thread block, 256-column tiles.  Wave 0 does nothing but walk (8 lanes for RMSNorm, 16 for LayerNorm)
 // and raises its issue priority; the four loader waves fetch one 16-byte vector per thread per tile two tiles ahead,
 // widen x and T(x*x) to f32 and park them in double-buffered LDS tiles; one barrier per tile.  The kernel runs at the
-// speed of the dependent v_add_f32 chain (about 3 ns per column on this chip).
+// speed of the walk.  A dependent v_add_f32 takes 4.9 cycles (2.0 ns) on this chip, but the walker also has to issue its
+// own LDS reads, one per four values of an f32 tile, which brings a column to about 3 ns.  For f16 the tiles therefore
+// hold the 16-bit values themselves (x, and T(x*x), which is an f16 value too): one LDS read per eight values, and the
+// chain adds them with v_fma_mix_f32 (1.0 * f16 operand + running f32 sum: the same sum, the widening is part of the
+// instruction).  bf16 has no such instruction and keeps the f32 tiles.
 // KEEP (launches whose blocks are all resident at once, rows of at most NP_KEEP_MAX_COLS columns): the walk of every row
 // of the tensor then ends at the same moment and nothing can hide what comes after it, so the output pass must be
 // nothing but stores: each loader thread also parks the raw vectors it loaded in dynamic LDS, scale and bias are staged
@@ -376,13 +380,35 @@ __global__ void __launch_bounds__(BLOCK) norm_seq16_kernel(const T* __restrict__
 constexpr int NP_BLOCK = 320;
 constexpr uint32_t NP_KEEP_MAX_COLS = 4096;
 constexpr size_t NP_KEEP_BYTES_PER_TILE = 256 * 16 + 2 * 32 * 16;   // the block's x vectors, one scale and one bias vector per column group
+typedef _Float16 np_h8 __attribute__((ext_vector_type(8)));
+// run += the 32 f16 values packed in four vectors, left to right: each add is 1.0 * widen(f16) + run in one instruction
+// with one rounding, which is the f32 sum of the widened values.  One asm statement for the whole run of adds: between
+// separate statements the compiler, which cannot see into them, puts wait states that cost more than the adds.
+#define NP_MIX_LO(N) "v_fma_mix_f32 %0, %" #N ", %17, %0 op_sel_hi:[1,0,0]\n"
+#define NP_MIX_HI(N) "v_fma_mix_f32 %0, %" #N ", %17, %0 op_sel:[1,0,0] op_sel_hi:[1,0,0]\n"
+#define NP_MIX(N) NP_MIX_LO(N) NP_MIX_HI(N)
+__device__ __forceinline__ void np_add_f16x32(float& run, const v4u& a, const v4u& b, const v4u& c, const v4u& d) {
+    const float one = 1.0f;
+    asm(NP_MIX(1) NP_MIX(2) NP_MIX(3) NP_MIX(4) NP_MIX(5) NP_MIX(6) NP_MIX(7) NP_MIX(8) NP_MIX(9) NP_MIX(10) NP_MIX(11) NP_MIX(12)
+        NP_MIX(13) NP_MIX(14) NP_MIX(15) NP_MIX(16)
+        : "+v"(run)
+        : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]), "v"(c[0]), "v"(c[1]), "v"(c[2]), "v"(c[3]),
+          "v"(d[0]), "v"(d[1]), "v"(d[2]), "v"(d[3]), "s"(one));
+}
+#undef NP_MIX
+#undef NP_MIX_HI
+#undef NP_MIX_LO
 template <typename T, int KIND, bool KEEP>
 __global__ void __launch_bounds__(NP_BLOCK) norm_pipe16_kernel(const T* __restrict__ x, const T* __restrict__ scale,
                                                                const T* __restrict__ bias, T* __restrict__ y, uint64_t rows, uint32_t cols,
                                                                float eps) {
-    constexpr int RB = 8, TC = 256, PAD = 4;
+    constexpr int RB = 8, TC = 256, PAD = 4, PAD16 = 8;
     constexpr int NSUM = (KIND == NORM_LAYER) ? 2 : 1;
-    __shared__ __attribute__((aligned(16))) float tile[2][NSUM][RB][TC + PAD];   // [.][0] = squares, [.][1] = values
+    constexpr bool H16 = std::is_same<T, half_t>::value;                         // 16-bit tiles and the fma_mix chain
+    // [.][0] = squares, [.][1] = values: f32, or the f16 bit patterns
+    __shared__ __attribute__((aligned(16))) unsigned char tile_raw[H16 ? 2 * NSUM * RB * (TC + PAD16) * 2 : 2 * NSUM * RB * (TC + PAD) * 4];
+    float (*tile)[NSUM][RB][TC + PAD] = reinterpret_cast<float (*)[NSUM][RB][TC + PAD]>(tile_raw);
+    uint16_t (*tile16)[NSUM][RB][TC + PAD16] = reinterpret_cast<uint16_t (*)[NSUM][RB][TC + PAD16]>(tile_raw);
     __shared__ float sums[NSUM][RB];
     __shared__ T s_mu[RB], s_r[RB];
     extern __shared__ __attribute__((aligned(16))) v4u np_keep[];               // KEEP: [ntiles][256] x, [ntiles][32] scale, [ntiles][32] bias
@@ -400,6 +426,23 @@ __global__ void __launch_bounds__(NP_BLOCK) norm_pipe16_kernel(const T* __restri
             __syncthreads();                                                    // tile t is in LDS
             // fixed trip count (tiles are zero padded): LDS reads of the next 32 values are issued before the 32 dependent
             // adds of the current ones
+            if constexpr (H16) {
+                const v4u* trow16 = reinterpret_cast<const v4u*>(tile16[t & 1][wsum][wrow]);
+                v4u cur[4], nxt[4];
+#pragma unroll
+                for (int k = 0; k < 4; k++) cur[k] = trow16[k];
+#pragma unroll
+                for (int c = 0; c < TC / 32; c++) {
+                    if (c + 1 < TC / 32) {
+#pragma unroll
+                        for (int k = 0; k < 4; k++) nxt[k] = trow16[(c + 1) * 4 + k];
+                    }
+                    np_add_f16x32(run, cur[0], cur[1], cur[2], cur[3]);
+#pragma unroll
+                    for (int k = 0; k < 4; k++) cur[k] = nxt[k];
+                }
+                continue;
+            }
             const float4* trow = reinterpret_cast<const float4*>(tile[t & 1][wsum][wrow]);
             float4 cur[8], nxt[8];
 #pragma unroll
@@ -448,7 +491,17 @@ __global__ void __launch_bounds__(NP_BLOCK) norm_pipe16_kernel(const T* __restri
     auto step = [&](uint32_t t, v4u& reg) {
         const uint32_t buf = t & 1;
         const uint32_t col = t * TC + cv * 8;
-        if (rvalid) {
+        if (H16 && rvalid) {
+            v4u sqv = {0, 0, 0, 0}, xvv = {0, 0, 0, 0};                         // past the end of the row: +0.0 terms
+            if (col < cols) {
+                xvv = __builtin_bit_cast(v4u, reg);
+                if (KEEP) keep_x[t * 256 + lt] = xvv;                           // read back by this same thread after the walk
+                const np_h8 h = __builtin_bit_cast(np_h8, xvv);
+                sqv = __builtin_bit_cast(v4u, h * h);                           // T(x*x): eight f16 products, each rounded once
+            }
+            *reinterpret_cast<v4u*>(&tile16[buf][0][r][cv * 8]) = sqv;
+            if (KIND == NORM_LAYER) *reinterpret_cast<v4u*>(&tile16[buf][NSUM - 1][r][cv * 8]) = xvv;
+        } else if (rvalid) {
             float sq[8], xv[8];
             if (col < cols) {
                 Vec16<T> in;
@@ -818,7 +871,7 @@ int launch_norm16(rt_device* dev, const void* x, const void* scale, const void* 
         // all blocks resident at once (the latency-bound case): the output pass comes from LDS
         const uint32_t ntiles = (cols + 255) / 256;
         const size_t keep_bytes = (size_t)ntiles * NP_KEEP_BYTES_PER_TILE;
-        const size_t static_bytes = (KIND == NORM_LAYER ? 2 : 1) * 2 * 8 * 260 * sizeof(float) + 256;
+        const size_t static_bytes = (KIND == NORM_LAYER ? 2 : 1) * 2 * 8 * (std::is_same<T, half_t>::value ? 264 * 2 : 260 * sizeof(float)) + 256;
         const size_t per_cu = (160 * 1024) / (static_bytes + keep_bytes);
         if (cols <= NP_KEEP_MAX_COLS && blocks <= (uint64_t)dev->num_cus * per_cu) {
             const int ti = (std::is_same<T, half_t>::value ? 0 : 2) + (KIND == NORM_LAYER ? 0 : 1);
