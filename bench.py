@@ -691,8 +691,14 @@ def main():
             return None
 
     def traffic_bytes(pos):
+        """fetch + write of the launch at step position `pos`, from the committed counter summary; None when the summary
+        is missing or does not describe this op (its own algorithmic columns disagree with the op's bytes by more than 1 %)"""
         try:
-            return int((float(pmc_rows[pos][2]) + float(pmc_rows[pos][3])) * 1024)
+            r = pmc_rows[pos]
+            alg_kib = float(r[4]) + float(r[5])
+            if abs(alg_kib * 1024 - ops[pos - 1].alg_bytes) > 0.01 * ops[pos - 1].alg_bytes:
+                return None
+            return int((float(r[2]) + float(r[3])) * 1024)
         except (KeyError, IndexError, ValueError):
             return None
 
