@@ -66,6 +66,46 @@ __device__ __forceinline__ uint32_t sp_clock() {
     return (uint32_t)t;
 }
 
+// The block's schedule: a step may not start before `pace` ticks of the wall clock have passed since the one before
+// was allowed to (t_step): a wave that arrives early waits, and a late one goes on at once and the schedule starts
+// again from its arrival, so that a step which was late is not followed by a burst (it is the bursts that overload
+// HBM).  Inputs whose steps are longer than the pace for reasons of their own (dense scores: the table lookups collide
+// in the LDS banks) must not be held at all, because their short steps would be delayed and their long ones not made up
+// for: the wave keeps a running average of the time between its steps (`avg`, a quarter of each new value), and while
+// that is above 1.2 paces it only keeps time.  Everything is in scalar registers and in one asm statement: written as
+// C++ the loop changed the register allocation and instruction order of the whole kernel, loader waves included.
+__device__ __forceinline__ void sp_pace_step(uint32_t& t_step, uint32_t& t_last, uint32_t& avg, uint32_t pace, uint32_t slow) {
+    asm volatile(
+        "s_memrealtime s[96:97]\n"
+        "s_waitcnt lgkmcnt(0)\n"
+        "s_sub_u32 s98, s96, %1\n"              // time since the previous step
+        "s_mov_b32 %1, s96\n"
+        "s_sub_u32 s98, s98, %2\n"
+        "s_ashr_i32 s98, s98, 2\n"
+        "s_add_u32 %2, %2, s98\n"               // avg += (dt - avg) / 4
+        "s_cmp_ge_i32 %2, %4\n"
+        "s_cbranch_scc1 2f\n"                   // steps are slow by themselves: only keep time
+        "s_sub_u32 s98, s96, %0\n"              // ticks since the last permitted start
+        "s_cmp_ge_i32 s98, %3\n"
+        "s_cbranch_scc1 2f\n"                   // late or on time
+        "1:\n"
+        "s_sleep 1\n"                           // early: wait for the step's time
+        "s_memrealtime s[96:97]\n"
+        "s_waitcnt lgkmcnt(0)\n"
+        "s_sub_u32 s98, s96, %0\n"
+        "s_cmp_ge_i32 s98, %3\n"
+        "s_cbranch_scc0 1b\n"
+        "s_add_u32 %0, %0, %3\n"                // started exactly on schedule
+        "s_mov_b32 %1, s96\n"
+        "s_branch 3f\n"
+        "2:\n"
+        "s_mov_b32 %0, s96\n"                   // the schedule starts again from this arrival
+        "3:\n"
+        : "+s"(t_step), "+s"(t_last), "+s"(avg)
+        : "s"(pace), "s"(slow)
+        : "s96", "s97", "s98", "scc", "memory");
+}
+
 // Which 30-row groups a block works on.  Rows come in `reps` periods of P rows (P = all rows when nothing repeats; P = the
 // rows one mask covers when a mask is added, e.g. S rows per head for an [S, T] mask under B * H heads); a period holds
 // GP = ceil(P / 30) groups, none of which straddles two periods.  Item w = block + i * grid -> (rep, group) = (w / GP, w % GP):
@@ -80,6 +120,7 @@ struct SpSched {
     FastDiv pm_div;          // rows of the mask: row (rep * P + r) of x takes mask row (rep * P + r) % PM.  PM == P unless the
     uint32_t PM;             // mask is only a few rows tall, where groups that stop at every period would be nearly empty
     uint32_t pace;           // shortest time between two steps of a block, in ticks of the device's wall clock (100 MHz); 0: unpaced
+    uint32_t phase_fx;       // pace / grid in 16.16 fixed point: block b takes its steps b * pace / grid ticks after block 0
 };
 
 __device__ __forceinline__ uint32_t sp_item_count(const SpSched& s, uint32_t b, uint32_t G) {
@@ -185,8 +226,12 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
         typename ST::Run run = ST::zero();
         uint32_t gpar = 0;
         // the blocks take their steps out of phase with each other: block b starts b / grid of a step late
-        uint32_t t_step = 0, free_steps = 0;
-        if constexpr (PACED) t_step = sp_clock() - sch.pace + (uint32_t)(((uint64_t)blockIdx.x * sch.pace) / gridDim.x);
+        uint32_t t_step = 0, t_last = 0, t_avg = sch.pace, t_slow = sch.pace + sch.pace / 5;
+        if constexpr (PACED) {
+            t_last = __builtin_amdgcn_readfirstlane(sp_clock());
+            t_step = t_last - sch.pace + ((blockIdx.x * sch.phase_fx) >> 16);
+            t_last -= sch.pace;
+        }
         for (uint32_t it = 0; it < n_items; it++) {
             // RAGGED: a row that starts sh bytes into its first vector can reach up to 14 bytes past its last step.  That
             // one vector is fetched here, at the start of the group, and added after the group's last step.
@@ -216,22 +261,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
             }
 #pragma unroll 1
             for (uint32_t t = 0; t < nsteps; t++) {
-                if (PACED && sch.pace) {                     // the walker is the block's clock: see SpSched::pace
-                    if (free_steps) {                        // not looking at the clock; start timing again at the last of them
-                        if (--free_steps == 0) t_step = sp_clock();
-                    } else {
-                        uint32_t el = sp_clock() - t_step;
-                        if (el >= sch.pace + sch.pace / 4) {
-                            free_steps = 4;                  // the steps take longer than the pace by themselves: stay out of the way
-                        } else {
-                            while (el < sch.pace) {
-                                __builtin_amdgcn_s_sleep(1);
-                                el = sp_clock() - t_step;
-                            }
-                            t_step += sch.pace;
-                        }
-                    }
-                }
+                if (PACED && sch.pace) sp_pace_step(t_step, t_last, t_avg, sch.pace, t_slow);   // the walker is the block's clock
                 __syncthreads();                             // A
                 __syncthreads();                             // B: tile t is in LDS
                 // 16 values per chunk; the LDS reads of the next chunk are in flight during the 16 dependent adds
@@ -801,25 +831,25 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
             }
         }
         sch.GP = (sch.P + sch.R - 1) / sch.R;
-        sch.pace = 0;                                        // set below, once the grid is known
+        sch.pace = sch.phase_fx = 0;                         // set below, once the grid is known
         sch.gp_div = make_fastdiv(sch.GP);
         const uint64_t items = (uint64_t)sch.GP * sch.reps;
         RT_REQUIRE(items <= 0xffffffffull, RT_ERR_SIZE, "rt_softmax: too many row groups");
         const unsigned blocks = (unsigned)(items < (uint64_t)dev->num_cus ? items : (uint64_t)dev->num_cus);   // one resident block per CU
         // Pacing.  Left to itself the kernel offers HBM more requests than it sustains, and what it then gets is less than
-        // what it gets when it asks for slightly less: 366 us unpaced against 343 us on [1,32,4096,4096] in the benchmark
-        // step (a plain persistent copy loop shows the same: 5.9 TB/s unpaced, 6.4 TB/s with a sleep of the right length
-        // per iteration, and a write-only loop 4.4 against 6.6 TB/s).  So the walker holds the block's steps to the period
-        // at which all blocks together move SP_PACE_BYTES_PER_S, by the 100 MHz wall clock, and the blocks start out of
-        // phase.  A pace that is too fast gives the unpaced behaviour back (7.0e12: 359 us), one that is too slow costs
-        // in proportion (6.4e12: 355 us).  When the steps are slower than the pace by themselves (dense inputs, whose
-        // table lookups collide in the LDS banks; bf16) the walker stops looking at the clock for a few steps at a time.
-        // A grid that does not fill the chip is not paced.
+        // what it gets when it asks for slightly less: 366 us unpaced against 345-350 us on [1,32,4096,4096] in the
+        // benchmark step (a plain persistent copy loop shows the same: 5.9 TB/s unpaced, 6.4 TB/s with a sleep of the
+        // right length per iteration, and a write-only loop 4.4 against 6.6 TB/s).  So the walker holds the block's
+        // steps to the period at which all blocks together move SP_PACE_BYTES_PER_S, by the device's wall clock, and the
+        // blocks start out of phase (sp_pace_step).  A pace that is too fast gives the unpaced behaviour back (7.0e12:
+        // 359 us), one that is too slow costs in proportion (6.4e12: 355 us).  Only the plain variant on a grid that
+        // fills the chip is paced.
         if (blocks == dev->num_cus && !mask && !ragged) {
             const double rate = SP_PACE_BYTES_PER_S;
             const double group_bytes = (double)sch.R * cols * 2 * (nt > SP_MAX_STEPS ? 4 : 2);     // in and out (long rows: parked and read back)
             const double steps = nt > SP_MAX_STEPS ? sch.nsteps : nt == 7 ? 8 : nt;          // the steps the kernel variant takes per group
             sch.pace = (uint32_t)(group_bytes / steps * blocks / rate * dev->wall_clock_hz + 0.5);
+            sch.phase_fx = (sch.pace << 16) / blocks;
         }
         if (ragged) {
             if (mask) RT_SP_RAGGED_NS(true);
