@@ -150,31 +150,53 @@ template <> struct SpType<half_t> {
         return __builtin_bit_cast(v4u, __builtin_bit_cast(h16x8, a) + __builtin_bit_cast(h16x8, b));
     }
     static constexpr bool SHORT_DIVISION = true;
+    static constexpr bool CHUNK_ASM = false;                                      // the walker adds pair by pair
 };
 template <> struct SpType<bf16_t> {
     typedef float Run;                                                            // always a bf16 value, held widened
     static __device__ __forceinline__ Run zero() { return 0.0f; }
-    // bf16(a + b): both operands have 16 zero low bits, so a NaN sum has them too and the rounding increment cannot carry
-    // into the exponent; everything else is plain round-to-nearest-even on the bit pattern
+    // two f32 values rounded to bf16 (nearest even) and packed, low half first: one instruction on this chip
+    static __device__ __forceinline__ uint32_t cvt_pk(float lo, float hi) {
+        uint32_t r;
+        asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
+        return r;
+    }
+    // bf16(a + b), held widened: converting into the high half of a word whose low half is bf16(0) = 0 gives the f32
+    // form of the rounded sum directly, so a link of the walker's chain is two dependent instructions
     static __device__ __forceinline__ float add_round(float a, float b) {
-        const uint32_t x = f2u(a + b);
-        return u2f((x + 0x7fffu + ((x >> 16) & 1u)) & 0xffff0000u);
+        const float s = a + b;
+        uint32_t r;
+        asm("v_cvt_pk_bf16_f32 %0, 0, %1" : "=v"(r) : "v"(s));
+        return u2f(r);
     }
     static __device__ __forceinline__ void add_pair(Run& run, uint32_t w) {
         run = add_round(run, u2f(w << 16));
         run = add_round(run, u2f(w & 0xffff0000u));
     }
+    // sixteen values, left to right, as one asm statement (between separate statements the compiler, which cannot see
+    // into them, puts wait states): per value the operand is moved to the top of a word, added, and the sum rounded
+#define SP_BF_LINK(N)                                                                                               \
+    "v_lshlrev_b32 %1, 16, %" #N "\n v_add_f32 %0, %0, %1\n v_cvt_pk_bf16_f32 %0, 0, %0\n"                           \
+    "v_and_b32 %1, 0xffff0000, %" #N "\n v_add_f32 %0, %0, %1\n v_cvt_pk_bf16_f32 %0, 0, %0\n"
+    static __device__ __forceinline__ void add_chunk(Run& run, const v4u& c0, const v4u& c1) {
+        uint32_t t;
+        asm(SP_BF_LINK(2) SP_BF_LINK(3) SP_BF_LINK(4) SP_BF_LINK(5) SP_BF_LINK(6) SP_BF_LINK(7) SP_BF_LINK(8) SP_BF_LINK(9)
+            : "+v"(run), "=&v"(t)
+            : "v"(c0[0]), "v"(c0[1]), "v"(c0[2]), "v"(c0[3]), "v"(c1[0]), "v"(c1[1]), "v"(c1[2]), "v"(c1[3]));
+    }
+#undef SP_BF_LINK
     static __device__ __forceinline__ uint16_t run_bits(Run run) { return (uint16_t)(f2u(run) >> 16); }
     static __device__ __forceinline__ float widen_bits(uint32_t b) { return u2f(b << 16); }
-    static __device__ __forceinline__ uint32_t round_pair(float q0, float q1) { return (uint32_t)f2bf(q0) | ((uint32_t)f2bf(q1) << 16); }
+    static __device__ __forceinline__ uint32_t round_pair(float q0, float q1) { return cvt_pk(q0, q1); }
     static __device__ __forceinline__ v4u add_vec(const v4u& a, const v4u& b) {
         v4u r;
 #pragma unroll
         for (int w = 0; w < 4; w++)
-            r[w] = (uint32_t)f2bf(u2f(a[w] << 16) + u2f(b[w] << 16)) | ((uint32_t)f2bf(u2f(a[w] & 0xffff0000u) + u2f(b[w] & 0xffff0000u)) << 16);
+            r[w] = cvt_pk(u2f(a[w] << 16) + u2f(b[w] << 16), u2f(a[w] & 0xffff0000u) + u2f(b[w] & 0xffff0000u));
         return r;
     }
     static constexpr bool SHORT_DIVISION = false;                                 // the quotient's range is f32's: always the IEEE division
+    static constexpr bool CHUNK_ASM = true;                                       // the walker adds sixteen values per asm statement (add_chunk)
 };
 
 // NSTEP > 0: rows of up to NSTEP * 512 columns, exp values parked in registers.  NSTEP == 0: longer rows; the exp values
@@ -273,10 +295,14 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                         n0 = trow[(c + 1) * 2];
                         n1 = trow[(c + 1) * 2 + 1];
                     }
+                    if constexpr (ST::CHUNK_ASM) {
+                        ST::add_chunk(run, c0, c1);
+                    } else {
 #pragma unroll
-                    for (int w = 0; w < 4; w++) ST::add_pair(run, c0[w]);
+                        for (int w = 0; w < 4; w++) ST::add_pair(run, c0[w]);
 #pragma unroll
-                    for (int w = 0; w < 4; w++) ST::add_pair(run, c1[w]);
+                        for (int w = 0; w < 4; w++) ST::add_pair(run, c1[w]);
+                    }
                     c0 = n0;
                     c1 = n1;
                 }
