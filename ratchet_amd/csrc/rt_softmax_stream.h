@@ -23,8 +23,9 @@ constexpr int BLOCK = 256;
 //        (162 400 of the CU's 163 840 bytes), so exp is one ds_read_u16 per element with the bit pattern as the index:
 //        no range clamping, no NaN special case.
 //   sum: per 512-column step the exp values also go to an LDS tile; lanes 0..29 of wave 0 each walk one row of the
-//        tile left to right with dependent v_add_f16 (3 ns each on this chip, 1.5 us per step; bf16: add, round on the
-//        bit pattern, 12 ns).  The tile is single
+//        tile left to right with dependent v_add_f16 (3 ns each on this chip with the LDS reads the wave issues in
+//        between, 1.5 us per step; bf16: v_add_f32 and v_cvt_pk_bf16_f32 into the high half of a word, two dependent
+//        instructions and one that moves the operand into place, 5 ns).  The tile is single
 //        buffered with two barriers per step: the loaders look up step t+1 into registers and divide / store the
 //        previous group's step t while wave 0 walks step t, and only the short LDS write of the tile sits between the
 //        barriers with wave 0 idle.  A step is 30 KiB in and 30 KiB out of HBM per CU, about 2 us at a CU's share of
