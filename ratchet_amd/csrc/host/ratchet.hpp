@@ -124,7 +124,8 @@ struct MemoryPlan {
 // of kernels (a list of fewer than eight launches is re-issued call by call instead, which is cheaper than a graph
 // launch: no graph building, pattern matching, planning or allocation either way).  Shapes, offsets (cache, rope, index_write) and buffer addresses are fixed at compile(); new input data
 // goes into the graph's constant tensors with Tensor::update_from_host, and the output tensor's buffer is rewritten by
-// every dispatch.  The executable keeps every buffer of the graph alive, intermediates included.
+// every dispatch.  The executable keeps every buffer of the graph alive, intermediates included.  Like the tensors it is
+// for one thread at a time (a call-by-call dispatch lends the graph's nodes their buffers for its duration).
 class Executable {
   public:
     Executable() {}
