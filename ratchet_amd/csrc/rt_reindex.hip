@@ -13,7 +13,7 @@
 namespace {
 
 constexpr int BLOCK = 256;
-constexpr int UNROLL = 2;                 // vectors per thread: two before the first store (four were slower on the 21 MB concat and permute: 9.4 -> 7.7 us, 7.3 -> 6.5 us; one gained nothing more)
+constexpr int UNROLL = 2;                 // vectors per thread where more than one pays (concat, splat, repeated source dims): two before the first store (four were slower on the 21 MB concat: 9.4 -> 7.7 us)
 
 struct GatherArgs {
     FastDiv d3, d2, d1;      // destination extents, d3 in vectors
@@ -41,12 +41,17 @@ __device__ __forceinline__ uint32_t gather_block(const GatherArgs& p) {
 }
 
 // one VecT per thread-iteration; source contiguous along the destination's last dim (s[3] == 1)
-template <typename VecT>
+// U vectors per thread: one for a large tensor whose destination vectors each have a source vector of their own
+// (permute, slice: a wave that stores once and ends leaves HBM a more even stream; [32,4096,32,128] f16 heads swap
+// 389 -> 347 us, 134 MB 37 -> 35 us), UNROLL for small ones (21 MB: 6.5 us against 6.9) and when a source dim is
+// repeated (broadcast_to [1,1,4096,4096] -> [1,32,..]: 224 us against 250)
+constexpr uint64_t GATHER_ONE_FROM_BYTES = 48ull << 20;
+template <typename VecT, int U>
 __global__ void __launch_bounds__(BLOCK) gather_vec_kernel(const VecT* __restrict__ x, VecT* __restrict__ y, GatherArgs p) {
-    const uint32_t base = gather_block(p) * (BLOCK * UNROLL) + threadIdx.x;
-    VecT r[UNROLL];
+    const uint32_t base = gather_block(p) * (BLOCK * U) + threadIdx.x;
+    VecT r[U];
 #pragma unroll
-    for (int k = 0; k < UNROLL; k++) {
+    for (int k = 0; k < U; k++) {
         const uint32_t v = base + k * BLOCK;
         if (v < p.nvec) {
             uint32_t row, i3, t, i2, i1, i0;
@@ -57,7 +62,7 @@ __global__ void __launch_bounds__(BLOCK) gather_vec_kernel(const VecT* __restric
         }
     }
 #pragma unroll
-    for (int k = 0; k < UNROLL; k++) {
+    for (int k = 0; k < U; k++) {
         const uint32_t v = base + k * BLOCK;
         if (v < p.nvec) st_stream(y + v, r[k]);
     }
@@ -440,15 +445,19 @@ int launch_gather(rt_device* dev, int eb, const void* x, void* y, const uint32_t
     p.d2 = make_fastdiv(dst_shape[2]);
     p.d1 = make_fastdiv(dst_shape[1]);
     p.nvec = (uint32_t)nvec;
-    const unsigned blocks = blocks_for(nvec, BLOCK * UNROLL);
+    // vectors per thread of the vector kernel: see gather_vec_kernel
+    bool repeats = false;
+    for (int i = 0; i < 4; i++) repeats = repeats || (dst_shape[i] > 1 && S[i] == 0);
+    const int per_thread = (splat || repeats || n * (uint64_t)eb < GATHER_ONE_FROM_BYTES) ? UNROLL : 1;
+    const unsigned blocks = blocks_for(nvec, (uint64_t)BLOCK * per_thread);
     p.rm_h = make_fastdiv(1);
     p.rm_j = 0;
     if (!splat && dst_shape[1] > 1 && dst_shape[2] > 1 && S[1] != 0 && S[1] < S[2] && (row_bytes % 128) != 0) {
         // dim 1 lies closer together in the source than dim 2 and the rows do not fill whole lines
         const uint64_t slice_vec = (uint64_t)dst_shape[2] * dst_shape[3] / per;
         const uint64_t heads = (uint64_t)dst_shape[0] * dst_shape[1];
-        if (slice_vec % (BLOCK * UNROLL) == 0) {
-            const uint64_t j = slice_vec / (BLOCK * UNROLL);
+        if (slice_vec % (BLOCK * per_thread) == 0) {
+            const uint64_t j = slice_vec / (BLOCK * per_thread);
             if (j % 8 == 0 && j * heads == blocks) {
                 p.rm_h = make_fastdiv((uint32_t)heads);
                 p.rm_j = (uint32_t)j;
@@ -476,7 +485,13 @@ int launch_gather(rt_device* dev, int eb, const void* x, void* y, const uint32_t
         p.base = base_elems / per;
         for (int i = 0; i < 3; i++) p.s[i] = (dst_shape[i] > 1) ? S[i] / per : 0;
         p.s[3] = (per > 1 || dst_shape[3] == 1) ? (dst_shape[3] == 1 ? 0 : 1) : S[3];
-#define RT_GATHER(VT) hipLaunchKernelGGL((gather_vec_kernel<VT>), dim3(blocks), dim3(BLOCK), 0, dev->stream, (const VT*)x, (VT*)y, p)
+#define RT_GATHER(VT)                                                                                                                  \
+    do {                                                                                                                               \
+        if (per_thread == 1)                                                                                                           \
+            hipLaunchKernelGGL((gather_vec_kernel<VT, 1>), dim3(blocks), dim3(BLOCK), 0, dev->stream, (const VT*)x, (VT*)y, p);       \
+        else                                                                                                                           \
+            hipLaunchKernelGGL((gather_vec_kernel<VT, UNROLL>), dim3(blocks), dim3(BLOCK), 0, dev->stream, (const VT*)x, (VT*)y, p);  \
+    } while (0)
         if (vb == 16) RT_GATHER(v4u);
         else if (vb == 8) RT_GATHER(v2u);
         else if (vb == 4) RT_GATHER(uint32_t);
