@@ -128,3 +128,24 @@ def test_reindex_stress_round_trips(dev, oracle):
     gn = dev.group_norm(dev.upload(gx), 32, dev.upload(gw), dev.upload(gb), 1e-5).to_numpy()
     bad, mx = oracle.count_not_close(gn, oracle.group_norm(gx, 32, gw, gb, 1e-5), 1e-3, 1e-3)
     assert bad == 0, mx
+
+
+def test_casts_and_gathers_beyond_the_one_access_per_thread_thresholds(dev, oracle):
+    """From 2^23 elements a cast, and from 48 MB a permute / slice without repeated source dims, run one access per
+    thread instead of four / two: the same results, bit for bit, on sizes just past the switch (with a ragged tail)."""
+    rng = np.random.default_rng(77)
+    n = (1 << 23) + 5
+    x32 = rng.standard_normal(n).astype(np.float32)
+    got16 = dev.cast(dev.upload(x32), F16).to_numpy()
+    assert same_bits(got16, x32.astype(np.float16))
+    assert same_bits(got16, oracle.cast(x32, np.float16))
+    assert same_bits(dev.cast(dev.upload(got16), F32).to_numpy(), got16.astype(np.float32))
+    # 64 MB head swap and its way back; a slice of it with offsets in every dim
+    q = rng.standard_normal((4, 1024, 64, 128)).astype(np.float16)
+    dq = dev.upload(q)
+    p = dev.permute(dq, (0, 2, 1, 3))
+    assert same_bits(p.to_numpy(), q.transpose(0, 2, 1, 3))
+    assert same_bits(dev.permute(p, (0, 2, 1, 3)).to_numpy(), q)
+    big = rng.standard_normal((5, 1030, 64, 136)).astype(np.float16)
+    got = dev.slice(dev.upload(big), [(1, 5), (3, 1027), (0, 64), (8, 136)]).to_numpy()
+    assert same_bits(got, big[1:5, 3:1027, :, 8:136])
