@@ -3,7 +3,7 @@
 // types every operator and every libm call is "widen to f32, operate, round to nearest even".
 //   f16: + - * use the native v_*_f16 instructions (IEEE, correctly rounded, identical to going through f32);
 //        / and sqrt go through correctly rounded f32 (24 >= 2*11+2 bits, so the second rounding is innocuous).
-//   bf16: everything through f32; the rounding back is the hardware conversion.
+//   bf16: everything through f32.
 // Compile with -ffp-contract=off.
 #ifndef RT_ARITH_H
 #define RT_ARITH_H
@@ -51,9 +51,10 @@ template <> struct Ar<half_t> {
 template <> struct Ar<bf16_t> {
     typedef bf16_t T;
     static constexpr int BYTES = 2;
-    // round to nearest even with the chip's own conversion (v_cvt_pk_bf16_f32): one instruction where the rounding on the
-    // bit pattern (f2bf in rt_libm.h, the host-checkable statement of the same function) takes six; NaN stays NaN
-    static __device__ __forceinline__ T conv(float f) { T r; r.b = __builtin_bit_cast(uint16_t, (__bf16)f); return r; }
+    // (the chip's own conversion, `(__bf16)f` = v_cvt_pk_bf16_f32, gives the same bits in one instruction, but this
+    // compiler fails to select code for it in some kernels ("cannot select v2f32 = bitcast" in the f32-routed unary
+    // kernel) and the kernels that use this are bound by memory, not by these six instructions)
+    static __device__ __forceinline__ T conv(float f) { T r; r.b = f2bf(f); return r; }
     static __device__ __forceinline__ float widen(T a) { return bf2f(a.b); }
     static __device__ __forceinline__ T add(T a, T b) { return conv(widen(a) + widen(b)); }
     static __device__ __forceinline__ T sub(T a, T b) { return conv(widen(a) - widen(b)); }
