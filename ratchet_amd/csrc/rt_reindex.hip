@@ -191,6 +191,54 @@ __global__ void __launch_bounds__(BLOCK) transpose_reg_kernel(const ElemT* __res
     for (int k = 0; k < V; k++) st_stream(reinterpret_cast<v4u*>(dst + (uint64_t)k * p.dq), out[k]);
 }
 
+// The same permutations through LDS with one 16-byte load and one 16-byte store per thread: a 512-thread block moves a
+// patch of 64 (dst dim 3) x 8 vectors (dst dim q) = 8 KiB, whole 128-byte lines on both sides.  A thread loads one
+// vector of a source row and writes its words to the tile (pitch 33 words: the column reads below touch every bank
+// once); then it gathers the V elements of one destination vector from V consecutive tile rows and stores it.  A wave's
+// store covers 8 (f16) or 4 (f32) destination rows with one full run of 128 / 256 bytes each.
+constexpr int TV_BLOCK = 512;
+template <typename ElemT>
+__global__ void __launch_bounds__(TV_BLOCK) transpose_vec_kernel(const ElemT* __restrict__ x, ElemT* __restrict__ y, TransposeArgs p) {
+    constexpr int V = 16 / sizeof(ElemT);            // elements per vector
+    constexpr int TJ = 64, TQW = 32;                 // patch: 64 rows of 32 words (8 vectors)
+    __shared__ uint32_t tile[TJ][TQW + 1];
+    uint32_t oa, obi, bz, byx, by, bx;
+    fd_divmod(blockIdx.x, p.gx, byx, bx);
+    fd_divmod(byx, p.gy, bz, by);
+    fd_divmod(bz, p.ob, oa, obi);
+    const uint64_t src0 = oa * p.sa + obi * p.sb;
+    const uint64_t dst0 = oa * p.da + obi * p.db;
+    const uint32_t q0 = bx * (8 * V), j0 = by * TJ;
+    {
+        const uint32_t r = threadIdx.x >> 3, v = threadIdx.x & 7;
+        const uint32_t j = j0 + r, q = q0 + v * V;
+        if (j < p.n3 && q < p.nq) {
+            const v4u in = ld_stream(reinterpret_cast<const v4u*>(x + src0 + (uint64_t)j * p.s3 + q));
+#pragma unroll
+            for (int w = 0; w < 4; w++) tile[r][v * 4 + w] = in[w];
+        }
+    }
+    __syncthreads();
+    const uint32_t d = threadIdx.x / (TJ / V), tv = threadIdx.x % (TJ / V);      // d: 0..63 (f16) or 0..31 (f32)
+    const uint32_t q = q0 + d, j = j0 + tv * V;
+    if (q < p.nq && j < p.n3) {
+        v4u out;
+        if (sizeof(ElemT) == 4) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) out[k] = tile[tv * 4 + k][d];
+        } else {
+            const uint16_t* t16 = reinterpret_cast<const uint16_t*>(&tile[0][0]);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const uint32_t lo = t16[(tv * 8 + 2 * k) * (2 * (TQW + 1)) + d];
+                const uint32_t hi = t16[(tv * 8 + 2 * k + 1) * (2 * (TQW + 1)) + d];
+                out[k] = lo | (hi << 16);
+            }
+        }
+        st_stream(reinterpret_cast<v4u*>(y + dst0 + (uint64_t)q * p.dq + j), out);
+    }
+}
+
 // concat: input k is [a_dim, bv[k]] vectors, copied into dst rows of dst_sv vectors at column dst_ov[k]
 struct ConcatArgs {
     const void* src[8];
@@ -556,6 +604,42 @@ int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uin
     int others[2], no = 0;
     for (int i = 0; i < 3; i++)
         if (i != q) others[no++] = i;
+    {
+        // The LDS patch kernel where it beats the register transpose below: source rows of 9 to 12 vectors (head dims 80
+        // and 96 in f16), which the register kernel covers with one wave-wide run per row and so stores in runs that
+        // are not whole lines ([1,32,4096,96] f16: 15.8 -> 12.4 us, [1,32,2048,80]: 8.2 -> 7.1 us), and tensors of
+        // 128 MB and more, where one store per thread pays ([8,32,2048,128] f16: 48 -> 45 us).
+        const uint32_t V = 16u / (uint32_t)elem_bytes;
+        const uint32_t row_vecs = dst_shape[q] / V;
+        uint64_t total = (uint64_t)elem_bytes;
+        for (int i = 0; i < 4; i++) total *= dst_shape[i];
+        if (((row_vecs > 8 && row_vecs <= 12) || total >= (128ull << 20)) && dst_shape[q] % V == 0 && dst_shape[3] % V == 0 &&
+            S[3] % V == 0 && S[others[0]] % V == 0 && S[others[1]] % V == 0 && rt_aligned(x, 16) && rt_aligned(y, 16)) {
+            TransposeArgs p;
+            p.nq = dst_shape[q];
+            p.n3 = dst_shape[3];
+            p.s3 = S[3];
+            p.dq = dst_strides[q];
+            p.ob = make_fastdiv(dst_shape[others[1]]);
+            p.sa = S[others[0]];
+            p.sb = S[others[1]];
+            p.da = dst_strides[others[0]];
+            p.db = dst_strides[others[1]];
+            const uint64_t gx = (p.nq + 8 * V - 1) / (8 * V), gy = (p.n3 + 63) / 64;
+            const uint64_t blocks = gx * gy * dst_shape[others[0]] * dst_shape[others[1]];
+            RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_permute: %llu tiles exceed the grid limit", (unsigned long long)blocks);
+            p.gx = make_fastdiv((uint32_t)gx);
+            p.gy = make_fastdiv((uint32_t)gy);
+            if (elem_bytes == 4)
+                hipLaunchKernelGGL((transpose_vec_kernel<uint32_t>), dim3((unsigned)blocks), dim3(TV_BLOCK), 0, dev->stream, (const uint32_t*)x,
+                                   (uint32_t*)y, p);
+            else
+                hipLaunchKernelGGL((transpose_vec_kernel<uint16_t>), dim3((unsigned)blocks), dim3(TV_BLOCK), 0, dev->stream, (const uint16_t*)x,
+                                   (uint16_t*)y, p);
+            RT_CHECK_LAUNCH("transpose_vec_kernel");
+            return RT_OK;
+        }
+    }
     {
         // whole aligned 16-byte vectors on both sides: the register transpose
         const uint32_t V = 16u / (uint32_t)elem_bytes;

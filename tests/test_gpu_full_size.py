@@ -149,3 +149,15 @@ def test_casts_and_gathers_beyond_the_one_access_per_thread_thresholds(dev, orac
     big = rng.standard_normal((5, 1030, 64, 136)).astype(np.float16)
     got = dev.slice(dev.upload(big), [(1, 5), (3, 1027), (0, 64), (8, 136)]).to_numpy()
     assert same_bits(got, big[1:5, 3:1027, :, 8:136])
+
+
+def test_large_transpose_takes_the_patch_kernel(dev):
+    """From 128 MB on (and for source rows of 9-12 vectors, covered at small sizes in test_gpu_reindex.py) a permutation
+    that moves the contiguous dim runs through the LDS patch kernel: K^T of eight Phi-2-sized layers at once, and the
+    [B,T,H,D] -> [B,H,D,T] form with a ragged last patch."""
+    rng = np.random.default_rng(78)
+    k = rng.standard_normal((8, 32, 2048, 128)).astype(np.float16)
+    dk = dev.upload(k)
+    assert same_bits(dev.permute(dk, (0, 1, 3, 2)).to_numpy(), k.transpose(0, 1, 3, 2))
+    x = rng.standard_normal((4, 2056, 32, 136)).astype(np.float16)
+    assert same_bits(dev.permute(dev.upload(x), (0, 2, 3, 1)).to_numpy(), x.transpose(0, 2, 3, 1))
