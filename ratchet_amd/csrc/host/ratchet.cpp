@@ -1194,6 +1194,8 @@ size_t Executable::held_bytes() const { return inner_ ? inner_->held : 0; }
 
 Executable Tensor::compile() const {
     if (!node_) throw Error("NullTensor", "compile on an empty tensor");
+    // a tensor that has its storage already has nothing left to run: an executable of it would replay nothing
+    if (node_->storage && !node_->srcs.empty()) throw Error("AlreadyResolved", "compile() wants a tensor that has not been resolved yet");
     return Resolver::compile(node_);
 }
 

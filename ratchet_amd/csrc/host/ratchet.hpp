@@ -210,6 +210,7 @@ class Tensor {
     // resolve() that also keeps the launch list: runs the graph once (so this tensor is resolved on return), then records
     // the same launches on the same buffers into an Executable.  An op is not run in place in a buffer that existed
     // before the call (a replay would apply it to its own result); cache and index_write still update their destination.
+    // A tensor that is resolved already cannot be compiled (there is nothing left to record).
     Executable compile() const;
     // to(&Device::CPU) + to_vec (tensor.rs:957-975): blocking download of the resolved tensor
     void to_host(void* out) const;
