@@ -112,7 +112,9 @@ __device__ __forceinline__ void sp_pace_step(uint32_t& t_step, uint32_t& t_last,
 // GP = ceil(P / 30) groups, none of which straddles two periods.  Item w = block + i * grid -> (rep, group) = (w / GP, w % GP):
 // the blocks running at one time work on one contiguous window of x.  (An order that put all heads of one mask slab on one
 // XCD, as the broadcast add does, was measured slower here, 461 against 441 us on [1,32,4096,4096]: thirty-two streams
-// 32 MiB apart collide in the memory channels, and the mask re-reads it saves are served by the Infinity Cache anyway.)
+// 32 MiB apart collide in the memory channels, and the mask re-reads it saves are served by the Infinity Cache anyway.
+// Orders in between, where the 32 blocks of an XCD work on the same 32 / h groups of h periods at one time so that the
+// mask rows they share stay in that XCD's L2, change nothing for h = 1, 2 and lose for h = 4 (+1 %), 8 (+9 %), 32 (+4 %).)
 struct SpSched {
     uint32_t P, GP, reps;
     uint32_t R;              // rows per group actually used (<= SP_ROWS): chosen so that the groups fill whole rounds of the grid
