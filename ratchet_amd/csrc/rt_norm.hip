@@ -422,27 +422,40 @@ __global__ void __launch_bounds__(NP_BLOCK) norm_pipe16_kernel(const T* __restri
         const uint32_t wrow = threadIdx.x % RB, wsum = (threadIdx.x / RB) % NSUM;   // lanes beyond NSUM*RB shadow and never publish
         const bool publish = (threadIdx.x < NSUM * RB) && (wrow < nrows);
         float run = 0.0f;
-        for (uint32_t t = 0; t < ntiles; t++) {
-            __syncthreads();                                                    // tile t is in LDS
-            // fixed trip count (tiles are zero padded): LDS reads of the next 32 values are issued before the 32 dependent
-            // adds of the current ones
-            if constexpr (H16) {
-                const v4u* trow16 = reinterpret_cast<const v4u*>(tile16[t & 1][wsum][wrow]);
-                v4u cur[4], nxt[4];
+        if constexpr (H16) {
+            // The barrier that says "tile t + 1 is in LDS" is taken before the last 32 adds of tile t, whose operands are in
+            // registers by then (the loaders may overwrite tile t after it): the first LDS reads of the next tile are in
+            // flight during those adds, so the chain never waits for LDS at a tile's start.
+            __syncthreads();                                                    // tile 0 is in LDS
+            v4u cur[4], nxt[4];
+            {
+                const v4u* first = reinterpret_cast<const v4u*>(tile16[0][wsum][wrow]);
 #pragma unroll
-                for (int k = 0; k < 4; k++) cur[k] = trow16[k];
+                for (int k = 0; k < 4; k++) cur[k] = first[k];
+            }
+            for (uint32_t t = 0; t < ntiles; t++) {
+                const v4u* trow16 = reinterpret_cast<const v4u*>(tile16[t & 1][wsum][wrow]);
+                const v4u* trow16n = reinterpret_cast<const v4u*>(tile16[(t + 1) & 1][wsum][wrow]);
 #pragma unroll
                 for (int c = 0; c < TC / 32; c++) {
                     if (c + 1 < TC / 32) {
 #pragma unroll
                         for (int k = 0; k < 4; k++) nxt[k] = trow16[(c + 1) * 4 + k];
+                    } else if (t + 1 < ntiles) {
+                        __syncthreads();                                        // tile t + 1 is in LDS
+#pragma unroll
+                        for (int k = 0; k < 4; k++) nxt[k] = trow16n[k];
                     }
                     np_add_f16x32(run, cur[0], cur[1], cur[2], cur[3]);
 #pragma unroll
                     for (int k = 0; k < 4; k++) cur[k] = nxt[k];
                 }
-                continue;
             }
+        }
+        for (uint32_t t = 0; !H16 && t < ntiles; t++) {
+            __syncthreads();                                                    // tile t is in LDS
+            // fixed trip count (tiles are zero padded): LDS reads of the next 32 values are issued before the 32 dependent
+            // adds of the current ones
             const float4* trow = reinterpret_cast<const float4*>(tile[t & 1][wsum][wrow]);
             float4 cur[8], nxt[8];
 #pragma unroll
