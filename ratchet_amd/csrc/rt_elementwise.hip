@@ -81,12 +81,13 @@ struct BcastArgs {
 };
 
 constexpr int BC_UNROLL = 2;
+constexpr uint64_t BC_ONE_FROM_VECS = 1ull << 26;
 constexpr uint32_t XCDS = 8;
 
 // ONCE: bit 0 / bit 1 set when a / b has no broadcast dim, so each of its elements is read exactly once and its loads
 // carry the non-temporal hint.  (A compile-time choice: with `once ? ld_stream(q) : *q` on a run-time flag the compiler
 // merges the two loads into one ordinary load, and a 1 GiB operand then floods L2 and the memory-side cache.)
-template <typename T, int OP, int VE, int ONCE>
+template <typename T, int OP, int VE, int ONCE, int U = BC_UNROLL>
 __global__ void __launch_bounds__(BLOCK) binary_bcast_kernel(const T* __restrict__ a, const T* __restrict__ b,
                                                              T* __restrict__ y, BcastArgs p) {
     uint32_t blk = blockIdx.x;
@@ -96,11 +97,12 @@ __global__ void __launch_bounds__(BLOCK) binary_bcast_kernel(const T* __restrict
         fd_divmod(idx >> p.chunk_log2, p.reps, chunk, rep);
         blk = rep * p.slabs + ((chunk << p.chunk_log2) + (idx & ((1u << p.chunk_log2) - 1))) * XCDS + (blk % XCDS);
     }
-    const uint32_t base = blk * (BLOCK * BC_UNROLL) + threadIdx.x;
-    // every load of the thread's BC_UNROLL vectors is issued before the first store
-    T ra[BC_UNROLL][VE], rb[BC_UNROLL][VE];
+    const uint32_t base = blk * (BLOCK * U) + threadIdx.x;
+    if (U == 1 && base >= p.nvec) return;
+    // every load of the thread's U vectors is issued before the first store
+    T ra[U][VE], rb[U][VE];
 #pragma unroll
-    for (int k = 0; k < BC_UNROLL; k++) {
+    for (int k = 0; k < U; k++) {
         const uint32_t v = base + k * BLOCK;
         if (v >= p.nvec) break;
         uint32_t row, col, i0, i1, i2, t;
@@ -141,7 +143,7 @@ __global__ void __launch_bounds__(BLOCK) binary_bcast_kernel(const T* __restrict
         }
     }
 #pragma unroll
-    for (int k = 0; k < BC_UNROLL; k++) {
+    for (int k = 0; k < U; k++) {
         const uint32_t v = base + k * BLOCK;
         if (v >= p.nvec) break;
         const uint64_t yo = (uint64_t)v * VE;
@@ -149,7 +151,10 @@ __global__ void __launch_bounds__(BLOCK) binary_bcast_kernel(const T* __restrict
             Vec16<T> t16;
 #pragma unroll
             for (int e = 0; e < VE; e++) t16.e[e] = ar_binary<OP, T>(ra[k][e], rb[k][e]);
-            st_stream(reinterpret_cast<v4u*>(y + yo), t16.u);
+            // U == 1: the compiler drops the non-temporal hint of the builtin when the kernel has a single store (and the
+            // lines an ordinary 1 GiB store leaves in the caches cost the kernels behind it more than this one gains)
+            if (U == 1) asm volatile("global_store_dwordx4 %0, %1, off nt" ::"v"(reinterpret_cast<v4u*>(y + yo)), "v"(t16.u) : "memory");
+            else st_stream(reinterpret_cast<v4u*>(y + yo), t16.u);
         } else {
             y[yo] = ar_binary<OP, T>(ra[k][0], rb[k][0]);
         }
@@ -700,7 +705,11 @@ int launch_bcast(rt_device* dev, const void* a, const uint32_t a_shape[4], const
         if (a_shape[i] != y_shape[i]) a_once = false;
         if (b_shape[i] != y_shape[i]) b_once = false;
     }
-    const unsigned blocks = blocks_for(nvec, BLOCK * BC_UNROLL);
+    // one access per thread for a full-size operand of 1 GiB or more plus a broadcast one (measured on the [1,32,4096,4096]
+    // scores + [4096,4096] mask inside the benchmark step: 343-345 us against 346-351 us with two); below that, and for
+    // the other operand patterns, the two are level
+    const int unroll = (a_once != b_once && ve == VEMAX && nvec >= BC_ONE_FROM_VECS) ? 1 : BC_UNROLL;
+    const unsigned blocks = blocks_for(nvec, BLOCK * unroll);
     // one operand full-size, the other equal to y's trailing dims and repeated over the leading ones, too large to
     // stay in an XCD's L2 by itself (>= 1 MiB) and made of whole groups of 8 slabs
     p.slabs = 0;
@@ -719,18 +728,23 @@ int launch_bcast(rt_device* dev, const void* a, const uint32_t a_shape[4], const
                 if (rs[i] != y_shape[i]) prefix = false;
             }
         }
-        const uint64_t per_block = (uint64_t)BLOCK * BC_UNROLL * ve;
+        const uint64_t per_block = (uint64_t)BLOCK * unroll * ve;
         if (prefix && reps > 1 && inner * sizeof(T) >= (1u << 20) && inner % (per_block * XCDS) == 0) {
             p.reps = make_fastdiv((uint32_t)reps);
             p.slabs = (uint32_t)(inner / per_block);
             const uint32_t per_xcd = p.slabs / XCDS;
             p.chunk_log2 = per_xcd % 64 == 0 ? 6 : per_xcd % 4 == 0 ? 2 : 0;
+            if (unroll == 1 && per_xcd % 128 == 0) p.chunk_log2 = 7;
         }
     }
+#define RT_BCAST1(VEC, ONCE) \
+    hipLaunchKernelGGL((binary_bcast_kernel<T, OP, VEC, ONCE, 1>), dim3(blocks), dim3(BLOCK), 0, dev->stream, (const T*)a, (const T*)b, (T*)y, p)
 #define RT_BCAST(VEC, ONCE) \
     hipLaunchKernelGGL((binary_bcast_kernel<T, OP, VEC, ONCE>), dim3(blocks), dim3(BLOCK), 0, dev->stream, (const T*)a, (const T*)b, (T*)y, p)
     if (ve != VEMAX) RT_BCAST(1, 0);                              // scalar accesses
     else if (a_once && b_once) RT_BCAST(VEMAX, 3);
+    else if (a_once && unroll == 1) RT_BCAST1(VEMAX, 1);
+    else if (b_once && unroll == 1) RT_BCAST1(VEMAX, 2);
     else if (a_once) RT_BCAST(VEMAX, 1);
     else if (b_once) RT_BCAST(VEMAX, 2);
     else RT_BCAST(VEMAX, 0);

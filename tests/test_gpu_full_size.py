@@ -69,6 +69,14 @@ def test_phi3_attention_tail_at_full_size(dev, oracle):
     for h in range(H):
         _lib.check(dev.lib.rt_d2d(dev.handle, scores.ptr.value + h * head.nbytes, dh.ptr, head.nbytes))
     masked = dev.binary("add", scores, dev.upload(mask))
+    # the add itself (from 1 GiB the broadcast kernel makes one access per thread), and the same size with a row operand
+    mk = masked.to_numpy()
+    assert all(same_bits(mk[0, h, 1000:1064], head[1000:1064] + mask[1000:1064]) for h in (0, 17, 31))
+    del mk
+    row = rng.standard_normal(S).astype(np.float16)
+    biased = dev.binary("add", scores, dev.upload(row)).to_numpy()
+    assert all(same_bits(biased[0, h, -64:], head[-64:] + row) for h in (0, 9, 31))
+    del biased
     soft = dev.softmax(masked)
     out = soft.to_numpy()
     # every head holds the same data, so every head must hold the same result, bit for bit (catches any grid / chunk mapping slip)
