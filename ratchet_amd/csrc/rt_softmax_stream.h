@@ -73,7 +73,8 @@ __device__ __forceinline__ uint32_t sp_clock() {
 // HBM).  Inputs whose steps are longer than the pace for reasons of their own (dense scores: the table lookups collide
 // in the LDS banks) must not be held at all, because their short steps would be delayed and their long ones not made up
 // for: the wave keeps a running average of the time between its steps (`avg`, a quarter of each new value), and while
-// that is above 1.2 paces it only keeps time.  Everything is in scalar registers and in one asm statement: written as
+// that is above 1.2 paces it only keeps time.  A wait ends after 4096 looks at the clock at the latest (a step is a few
+// hundred ticks, a look takes several), so the kernel finishes whatever the clock does.  Everything is in scalar registers and in one asm statement: written as
 // C++ the loop changed the register allocation and instruction order of the whole kernel, loader waves included.
 __device__ __forceinline__ void sp_pace_step(uint32_t& t_step, uint32_t& t_last, uint32_t& avg, uint32_t pace, uint32_t slow) {
     asm volatile(
@@ -89,10 +90,14 @@ __device__ __forceinline__ void sp_pace_step(uint32_t& t_step, uint32_t& t_last,
         "s_sub_u32 s98, s96, %0\n"              // ticks since the last permitted start
         "s_cmp_ge_i32 s98, %3\n"
         "s_cbranch_scc1 2f\n"                   // late or on time
+        "s_movk_i32 s99, 0x1000\n"
         "1:\n"
         "s_sleep 1\n"                           // early: wait for the step's time
         "s_memrealtime s[96:97]\n"
         "s_waitcnt lgkmcnt(0)\n"
+        "s_sub_u32 s99, s99, 1\n"
+        "s_cmp_eq_u32 s99, 0\n"
+        "s_cbranch_scc1 2f\n"                   // 4096 looks at a clock that does not get there: stop waiting for it
         "s_sub_u32 s98, s96, %0\n"
         "s_cmp_ge_i32 s98, %3\n"
         "s_cbranch_scc0 1b\n"
@@ -104,7 +109,7 @@ __device__ __forceinline__ void sp_pace_step(uint32_t& t_step, uint32_t& t_last,
         "3:\n"
         : "+s"(t_step), "+s"(t_last), "+s"(avg)
         : "s"(pace), "s"(slow)
-        : "s96", "s97", "s98", "scc", "memory");
+        : "s96", "s97", "s98", "s99", "scc", "memory");
 }
 
 // Which 30-row groups a block works on.  Rows come in `reps` periods of P rows (P = all rows when nothing repeats; P = the
