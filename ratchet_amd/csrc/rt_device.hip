@@ -73,6 +73,13 @@ int rt_debug_hip_status(int hip_error, const char* what) {
     return rt_fail_hip((hipError_t)hip_error, what ? what : "injected");
 }
 
+int rt_debug_softmax_pace(rt_device* dev, uint32_t ticks) {
+    if (!dev) return rt_fail(RT_ERR_NULL_DEVICE, "rt_device is NULL");
+    RT_REQUIRE(ticks < (1u << 30), RT_ERR_ARG, "rt_debug_softmax_pace: %u ticks out of range", ticks);
+    dev->debug_softmax_pace = ticks;
+    return RT_OK;
+}
+
 const char* rt_status_name(int status) {
     switch (status) {
         case RT_OK: return "RT_OK";
@@ -124,6 +131,7 @@ int rt_device_create(int ordinal, rt_device** out) {
         int khz = 0;
         if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, ordinal) != hipSuccess) (void)hipGetLastError();
         dev->wall_clock_hz = khz > 0 ? khz * 1e3 : 1e8;
+        dev->debug_softmax_pace = 0;
     }
     hipError_t e = hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking);   // default priority
     if (e != hipSuccess) {

@@ -15,6 +15,7 @@ struct rt_device {
     hipStream_t stream;
     int num_cus;
     double wall_clock_hz;   // rate of the device's constant-frequency wall clock (s_memrealtime), 100 MHz on this chip
+    uint32_t debug_softmax_pace;   // test hook (rt_debug_softmax_pace): replaces the computed pace of the streaming softmax, 0 = none
     // GroupNorm partial statistics: {mean, m2, count} triples, one per (group, split)
     float* gn_scratch;
     size_t gn_scratch_bytes;

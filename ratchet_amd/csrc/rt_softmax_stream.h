@@ -883,7 +883,8 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
             const double group_bytes = (double)sch.R * cols * 2 * (nt > SP_MAX_STEPS ? 4 : 2);     // in and out (long rows: parked and read back)
             const double steps = nt > SP_MAX_STEPS ? sch.nsteps : nt == 7 ? 8 : nt;          // the steps the kernel variant takes per group
             sch.pace = (uint32_t)(group_bytes / steps * blocks / rate * dev->wall_clock_hz + 0.5);
-            sch.phase_fx = (sch.pace << 16) / blocks;
+            if (dev->debug_softmax_pace) sch.pace = dev->debug_softmax_pace;
+            sch.phase_fx = sch.pace > 0xffffu ? 0 : (sch.pace << 16) / blocks;
         }
         if (ragged) {
             if (mask) RT_SP_RAGGED_NS(true);

@@ -136,6 +136,40 @@ def test_softmax_f16_streaming_kernel(dev, oracle, shape):
     assert same_bits(dx.to_numpy(), want)
 
 
+def test_softmax_streaming_kernel_leaves_a_wait_that_its_clock_never_ends(dev, oracle):
+    """The paced kernel's walker waves wait for the device's wall clock; every such wait is bounded (4096 looks).  With the
+    pace set far beyond what a step takes, each wait runs into that bound: the kernel must finish, every wave leaving it
+    normally, with the bits of the run at the computed pace (which are the oracle's)."""
+    from ratchet_amd import _lib
+
+    rng = np.random.default_rng(310)
+    x = randn(rng, (1, 8192, 4096), np.float16, 2.0)                   # 304 groups of 27 rows: a grid that fills the chip, so paced
+    dx, dy = dev.upload(x), dev.empty(x.shape, _lib.F16)
+
+    def timed_ms():
+        e0, e1 = dev.event(), dev.event()
+        e0.record()
+        dev.softmax(dx, out=dy)
+        e1.record()
+        return e0.elapsed_ms(e1)
+
+    timed_ms()
+    usual = timed_ms()
+    want = dy.to_numpy()
+    assert mismatch_count(want[0, :64], oracle.softmax(x[0, :64])) == 0
+    _lib.check(dev.lib.rt_debug_softmax_pace(dev.handle, 1 << 28))     # 2.7 s a step, if anything waited for it
+    try:
+        held = timed_ms()
+        got = dy.to_numpy()
+    finally:
+        _lib.check(dev.lib.rt_debug_softmax_pace(dev.handle, 0))
+    assert mismatch_count(got, want) == 0
+    # 16 steps a block, each held for 4096 looks at the clock and no longer: milliseconds, not the 43 s of the pace asked for
+    assert 20 * usual < held < 2000.0, (usual, held)
+    again = dev.softmax(dx).to_numpy()                                 # and the computed pace is back
+    assert mismatch_count(again, want) == 0
+
+
 @pytest.mark.parametrize("rows,n,split", [(262140 + 47, 4096, 262140), (262200 + 131, 4095, 262200)])
 def test_softmax_f16_streaming_kernel_beyond_2_gib(dev, oracle, rows, n, split):
     # the kernel addresses a launch with 32-bit byte offsets below 2^31, so a larger tensor is split into row chunks
