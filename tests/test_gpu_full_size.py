@@ -169,3 +169,73 @@ def test_large_transpose_takes_the_patch_kernel(dev):
     assert same_bits(dev.permute(dk, (0, 1, 3, 2)).to_numpy(), k.transpose(0, 1, 3, 2))
     x = rng.standard_normal((4, 2056, 32, 136)).astype(np.float16)
     assert same_bits(dev.permute(dev.upload(x), (0, 2, 3, 1)).to_numpy(), x.transpose(0, 2, 3, 1))
+
+
+def test_ops_across_the_4_gib_boundary(dev, oracle):
+    """Tensors of 2^31 + 2^20 + 24 f16 elements (4.3 GB): element 2^31 lies at byte 2^32, where a 32-bit byte offset or
+    element index would wrap.  The tensor repeats a 2^24-element pattern, so any window of it is known without holding
+    4 GB on the host; the windows checked sit at the start, across the boundary and at the ragged end."""
+    from ratchet_amd import _lib
+    from ratchet_amd.runtime import BufferView
+
+    P = 1 << 24
+    n = (1 << 31) + (1 << 20) + 24
+    rng = np.random.default_rng(707)
+    pat = (2 * rng.standard_normal(P)).astype(np.float16)
+    pat[:8] = [0.0, -0.0, np.inf, -np.inf, np.nan, 65504.0, 6e-8, -6e-8]
+    x = dev.empty((n,), F16)
+    dp = dev.upload(pat)
+    for k in range(0, n, P):
+        _lib.check(dev.lib.rt_d2d(dev.handle, x.ptr.value + 2 * k, dp.ptr, 2 * min(P, n - k)))
+    windows = [(0, 64), ((1 << 31) - 40, (1 << 31) + 40), (n - 56, n)]
+
+    def expect(lo, hi):
+        return pat[np.arange(lo, hi) % P]
+
+    def window(buf, lo, hi):
+        return BufferView(buf, lo, (hi - lo,)).to_numpy()
+
+    y = dev.binary("add", x, x)
+    for lo, hi in windows:
+        assert same_bits(window(y, lo, hi), oracle.binary("add", expect(lo, hi), expect(lo, hi))), ("add", lo)
+    dev.unary("gelu", x, out=y)                                        # the table kernel
+    for lo, hi in windows:
+        assert same_bits(window(y, lo, hi), oracle.unary("gelu", expect(lo, hi))), ("gelu", lo)
+    dev.unary("neg", x, out=y)                                         # the computing kernel
+    for lo, hi in windows:
+        assert same_bits(window(y, lo, hi), oracle.unary("neg", expect(lo, hi))), ("neg", lo)
+    del y
+    wide = dev.cast(x, F32)
+    for lo, hi in windows:
+        assert same_bits(window(wide, lo, hi), expect(lo, hi).astype(np.float32)), ("cast", lo)
+    del wide
+    # the last rows of the aligned part as a slice: source offsets beyond 2^32 bytes
+    cols = 4096
+    rows = ((1 << 31) + (1 << 20)) // cols
+    tail = dev.slice(BufferView(x, 0, (1, 1, rows, cols)), [(0, 1), (0, 1), (rows - 300, rows), (0, cols)]).to_numpy()
+    assert same_bits(tail.reshape(-1), expect((rows - 300) * cols, rows * cols))
+    # row ops over the same bytes as [rows, 4096]: the rows on either side of byte 2^32 and the last ones
+    xr = BufferView(x, 0, (rows, cols))
+    at = [(1 << 31) // cols - 1, (1 << 31) // cols + 1, rows - 3, rows - 2, rows - 1]
+    want_rows = np.stack([expect(r * cols, (r + 1) * cols) for r in at])
+    g = (1 + 0.02 * rng.standard_normal(cols)).astype(np.float16)
+    b = (0.02 * rng.standard_normal(cols)).astype(np.float16)
+
+    def rows_of(buf):
+        return np.stack([window(buf, r * cols, (r + 1) * cols) for r in at])
+
+    out = dev.layer_norm(xr, dev.upload(g), dev.upload(b), 1e-5)
+    assert same_bits(rows_of(out), oracle.layer_norm(want_rows, g, b, 1e-5, intended=True))
+    dev.rms_norm(xr, dev.upload(g), 1e-5, out=out)
+    assert same_bits(rows_of(out), oracle.rms_norm(want_rows, g, 1e-5, intended=True))
+    dev.softmax(xr, out=out)                                           # split into launches of less than 2 GiB
+    assert same_bits(rows_of(out), oracle.softmax(want_rows))
+    dev.softmax_via_f32(xr, out=out)
+    want = oracle.cast(oracle.softmax(oracle.cast(want_rows, np.float32)), np.float16)
+    bad, mx = oracle.count_not_close(rows_of(out), want, 1e-3, 1e-3)
+    assert bad == 0, mx
+    g32 = g.astype(np.float32)
+    dev.norm_via_f32("rms", xr, dev.upload(g32), None, 1e-5, out=out)
+    want = oracle.cast(oracle.rms_norm(oracle.cast(want_rows, np.float32), g32, 1e-5, intended=True), np.float16)
+    bad, mx = oracle.count_not_close(rows_of(out), want, 1e-3, 1e-3)
+    assert bad == 0, mx
