@@ -239,3 +239,34 @@ def test_ops_across_the_4_gib_boundary(dev, oracle):
     want = oracle.cast(oracle.rms_norm(oracle.cast(want_rows, np.float32), g32, 1e-5, intended=True), np.float16)
     bad, mx = oracle.count_not_close(rows_of(out), want, 1e-3, 1e-3)
     assert bad == 0, mx
+
+
+def test_reindex_across_the_4_gib_boundary(dev):
+    """Permutes of a 4.3 GB f16 tensor (a repeated 2^24-element pattern): moving heads in front of the sequence (vector
+    gather) and transposing the last two dims (LDS patches); windows of the result on either side of byte 2^32."""
+    from ratchet_amd import _lib
+    from ratchet_amd.runtime import BufferView
+
+    P = 1 << 24
+    n = (1 << 31) + (1 << 20)
+    pat = np.random.default_rng(708).integers(0, 1 << 16, P, dtype=np.uint16).view(np.float16)     # any bits: nothing is computed
+    x = dev.empty((n,), F16)
+    dp = dev.upload(pat)
+    for k in range(0, n, P):
+        _lib.check(dev.lib.rt_d2d(dev.handle, x.ptr.value + 2 * k, dp.ptr, 2 * min(P, n - k)))
+
+    def src(idx):
+        return pat[np.asarray(idx, dtype=np.int64) % P]
+
+    # [1, S, 32, 128] -> [1, 32, S, 128]: out[h, s, :] = in[s, h, :]
+    S, H, D = n // (32 * 128), 32, 128
+    y = dev.permute(BufferView(x, 0, (1, S, H, D)), (0, 2, 1, 3))
+    for h, s in ((0, 0), (15, S // 2), (16, (1 << 31) // (H * D) - 1), (16, (1 << 31) // (H * D)), (31, S - 1)):
+        got = BufferView(y, (h * S + s) * D, (D,)).to_numpy()
+        assert same_bits(got, src((s * H + h) * D + np.arange(D))), (h, s)
+    # [1, 2049, 4096, 256] -> [1, 2049, 256, 4096]: slab 2048 starts at byte 2^32
+    A, R, C = n // (4096 * 256), 4096, 256
+    dev.permute(BufferView(x, 0, (1, A, R, C)), (0, 1, 3, 2), out=BufferView(y, 0, (1, A, C, R)))
+    for a, c in ((0, 0), (2047, 255), (2048, 0), (2048, 129), (A - 1, 255)):
+        got = BufferView(y, (a * C + c) * R, (R,)).to_numpy()
+        assert same_bits(got, src((a * R + np.arange(R)) * C + c)), (a, c)
