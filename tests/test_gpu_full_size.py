@@ -270,3 +270,50 @@ def test_reindex_across_the_4_gib_boundary(dev):
     for a, c in ((0, 0), (2047, 255), (2048, 0), (2048, 129), (A - 1, 255)):
         got = BufferView(y, (a * C + c) * R, (R,)).to_numpy()
         assert same_bits(got, src((a * R + np.arange(R)) * C + c)), (a, c)
+
+
+def test_concat_cache_and_broadcast_across_the_4_gib_boundary(dev, oracle):
+    """A 4.3 GB KV-cache-shaped tensor [1, 16, 32784, 4096] f16 built by concat from two halves, appended to through the
+    cache op, and added to a row vector: windows of the results in the first head and in the last (beyond byte 2^32)."""
+    from ratchet_amd import _lib
+    from ratchet_amd.runtime import BufferView
+
+    P = 1 << 24
+    Hd, R, C = 16, 16392, 4096
+    half = Hd * R * C                                                  # 2.1 GB each
+    rng = np.random.default_rng(709)
+    pat = rng.standard_normal(P).astype(np.float16)
+    x = dev.empty((2 * half,), F16)
+    dp = dev.upload(pat)
+    for k in range(0, 2 * half, P):
+        _lib.check(dev.lib.rt_d2d(dev.handle, x.ptr.value + 2 * k, dp.ptr, 2 * min(P, 2 * half - k)))
+
+    def src(idx):
+        return pat[np.asarray(idx, dtype=np.int64) % P]
+
+    a, b = BufferView(x, 0, (1, Hd, R, C)), BufferView(x, half, (1, Hd, R, C))
+    cat = dev.concat([a, b], 2)                                        # [1, 16, 32784, 4096]
+    cols = np.arange(C)
+
+    def cat_row(h, r):                                                 # what row r of head h of `cat` holds
+        return src((h * R + r) * C + cols) if r < R else src(half + (h * R + r - R) * C + cols)
+
+    def row_of(buf, h, r, rows_per_head=2 * R):
+        return BufferView(buf, (h * rows_per_head + r) * C, (C,)).to_numpy()
+
+    probes = [(0, 0), (0, R - 1), (0, R), (7, 2 * R - 1), (8, 0), (15, R - 1), (15, R), (15, 2 * R - 1)]
+    for h, r in probes:
+        assert same_bits(row_of(cat, h, r), cat_row(h, r)), ("concat", h, r)
+    # append 8 new rows per head at row 32776 of the cache: dst = cat(cache[:32776], new), and the cache holds them too
+    new = rng.standard_normal((1, Hd, 8, C)).astype(np.float16)
+    dst = dev.cache(cat, dev.upload(new), 2, 2 * R - 8)
+    for h, r in probes:
+        want = new[0, h, r - (2 * R - 8)] if r >= 2 * R - 8 else cat_row(h, r)
+        assert same_bits(row_of(dst, h, r), want), ("cache dst", h, r)
+        assert same_bits(row_of(cat, h, r), want), ("cache", h, r)
+    # the whole tensor plus a row vector
+    row = rng.standard_normal(C).astype(np.float16)
+    dev.binary("add", cat, dev.upload(row), out=dst)
+    for h, r in probes:
+        base = new[0, h, r - (2 * R - 8)] if r >= 2 * R - 8 else cat_row(h, r)
+        assert same_bits(row_of(dst, h, r), oracle.binary("add", base, row)), ("add", h, r)
