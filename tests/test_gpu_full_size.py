@@ -317,3 +317,40 @@ def test_concat_cache_and_broadcast_across_the_4_gib_boundary(dev, oracle):
     for h, r in probes:
         base = new[0, h, r - (2 * R - 8)] if r >= 2 * R - 8 else cat_row(h, r)
         assert same_bits(row_of(dst, h, r), oracle.binary("add", base, row)), ("add", h, r)
+
+
+def test_rope_and_index_select_across_the_4_gib_boundary(dev, oracle):
+    """RoPE on a 4.3 GB f32 tensor [1, 32, 349600, 96] and an embedding lookup from a 4.3 GB f16 table: positions and
+    rows whose bytes lie beyond 2^32."""
+    from ratchet_amd import _lib
+    from ratchet_amd.runtime import BufferView
+
+    P = 1 << 22
+    H, S, D = 32, 349600, 96
+    n = H * S * D                                                      # 1.07e9 f32 elements
+    rng = np.random.default_rng(710)
+    pat = rng.standard_normal(P).astype(np.float32)
+    x = dev.empty((1, H, S, D), F32)
+    dp = dev.upload(pat)
+    for k in range(0, n, P):
+        _lib.check(dev.lib.rt_d2d(dev.handle, x.ptr.value + 4 * k, dp.ptr, 4 * min(P, n - k)))
+    y = dev.rope(x, 64, 10000.0, 3)                                    # rotate 64 of the 96 columns, positions from 3
+    for h, s0 in ((0, 0), (15, S - 16), (16, 0), (31, S - 16)):
+        first = (h * S + s0) * D
+        win = pat[(first + np.arange(16 * D)) % P].reshape(1, 1, 16, D)
+        got = BufferView(y, first, (1, 1, 16, D)).to_numpy()
+        want = oracle.rope(win, 64, 10000.0, 3 + s0)
+        bad, mx = oracle.count_not_close(got, want, 1e-5, 1e-5)
+        assert bad == 0, (h, s0, mx)
+    del y, x
+    # embedding lookup: table [524544, 4096] f16
+    V, C = 524544, 4096
+    pat16 = rng.integers(0, 1 << 16, 1 << 24, dtype=np.uint16).view(np.float16)
+    table = dev.empty((V, C), F16)
+    dp = dev.upload(pat16)
+    for k in range(0, V * C, 1 << 24):
+        _lib.check(dev.lib.rt_d2d(dev.handle, table.ptr.value + 2 * k, dp.ptr, 2 * min(1 << 24, V * C - k)))
+    ids = np.array([0, 524287, 524288, V - 1, 17, 524400, V - 2, 300000], np.int32)
+    emb = dev.index_select(table, dev.upload(ids), 0).to_numpy()
+    for i, r in enumerate(ids):
+        assert same_bits(emb[i], pat16[(int(r) * C + np.arange(C)) % (1 << 24)]), r
