@@ -354,3 +354,36 @@ def test_rope_and_index_select_across_the_4_gib_boundary(dev, oracle):
     emb = dev.index_select(table, dev.upload(ids), 0).to_numpy()
     for i, r in enumerate(ids):
         assert same_bits(emb[i], pat16[(int(r) * C + np.arange(C)) % (1 << 24)]), r
+
+
+def test_group_norm_across_the_4_gib_boundary(dev, oracle):
+    """GroupNorm on a 4.3 GB f16 tensor [8, 512, 524544] with 32 groups (16 MB each, so every group is split over many
+    blocks): the first group, the two on either side of byte 2^32 and the last one, against torch's definition in f64."""
+    from ratchet_amd import _lib
+    from ratchet_amd.runtime import BufferView
+
+    P = 1 << 24
+    B, C, L, G = 8, 512, 524544, 32
+    n = B * C * L
+    rng = np.random.default_rng(711)
+    pat = (0.5 + rng.standard_normal(P)).astype(np.float16)
+    x = dev.empty((B, C, L), F16)
+    dp = dev.upload(pat)
+    for k in range(0, n, P):
+        _lib.check(dev.lib.rt_d2d(dev.handle, x.ptr.value + 2 * k, dp.ptr, 2 * min(P, n - k)))
+    w = (1 + 0.1 * rng.standard_normal(C)).astype(np.float16)
+    bi = (0.1 * rng.standard_normal(C)).astype(np.float16)
+    y = dev.group_norm(x, G, dev.upload(w), dev.upload(bi), 1e-5)
+    glen, cpg = (C // G) * L, C // G
+    for pair in (0, (1 << 31) // glen - 1, (1 << 31) // glen, B * G - 1):
+        first = pair * glen
+        grp = pat[(first + np.arange(glen, dtype=np.int64)) % P].astype(np.float64)
+        mu, var = grp.mean(), grp.var()
+        g = pair % G
+        for ch, l0 in ((0, 0), (cpg - 1, L - 64)):                     # 64 elements at the start and at the end of the group
+            c = g * cpg + ch
+            got = BufferView(y, first + ch * L + l0, (64,)).to_numpy()
+            xs = grp[ch * L + l0: ch * L + l0 + 64]
+            want = ((xs - mu) / np.sqrt(var + 1e-5) * float(w[c]) + float(bi[c])).astype(np.float16)
+            bad, mx = oracle.count_not_close(got, want, 1e-3, 1e-3)
+            assert bad == 0, (pair, ch, mx)
