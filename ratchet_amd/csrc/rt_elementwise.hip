@@ -74,7 +74,9 @@ struct BcastArgs {
     // block b runs on XCD b % 8, so the `reps` blocks that need the same 4 KiB slab of that operand are given to one
     // XCD back to back and its L2 fetches the slab once.  An XCD walks 2^chunk_log2 of its slabs per repeat before it
     // moves to the next repeat (measured on [1,32,4096,4096] + [4096,4096]: 64 slabs 363 us, 4 slabs 366 us, 1 slab
-    // 376 us, 16 slabs 416 us, identity order 404 us).  slabs == 0: identity order.
+    // 376 us, 16 slabs 416 us, identity order 404 us; with one vector per thread, where a slab is 4 KiB: 128 slabs
+    // 342 us, 256 slabs 349 us, 512 slabs 356 us, 64 slabs 382 us, 32 slabs 422 us, 1024 slabs 445 us: 512 KiB of the
+    // repeated operand per XCD either way).  slabs == 0: identity order.
     FastDiv reps;
     uint32_t slabs;    // blocks per repeat
     uint32_t chunk_log2;
