@@ -12,6 +12,19 @@
 //   expf: the table-driven double-precision algorithm (2^(k/32) table, degree-3 polynomial), with the
 //         reduction r = fma(InvLn2N, x, -kd) that an FMA build of the routine performs.
 // Everything here must be compiled with -ffp-contract=off: each float operation below is meant to round on its own.
+//
+// Provenance.  The routines below are restatements of published algorithms, with their published constants (a result
+// that must equal the C library's bit for bit cannot use others); no file of either library was copied.
+//   rt_expm1f, rt_tanhf: the float versions of FreeBSD's msun / Sun's fdlibm `s_expm1f.c` and `s_tanhf.c`, as glibc
+//     ships them.  fdlibm's notice, which asks to be kept with the algorithm:
+//       Copyright (C) 1993 by Sun Microsystems, Inc. All rights reserved.
+//       Developed at SunPro, a Sun Microsystems, Inc. business.
+//       Permission to use, copy, modify, and distribute this software is freely granted, provided that this notice
+//       is preserved.
+//   rt_expf: the single-precision exp of Arm's optimized-routines (`math/expf.c`, `math/exp2f_data.c`; Copyright (c)
+//     2017-2018 Arm Limited, SPDX-License-Identifier: MIT), which glibc 2.27 and later use for `expf`: the 32-entry
+//     table follows from its defining formula (the comment above it), the three polynomial coefficients and the
+//     reduction constants are the published ones.
 #ifndef RT_LIBM_H
 #define RT_LIBM_H
 
