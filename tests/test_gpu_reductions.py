@@ -154,7 +154,7 @@ def test_softmax_streaming_kernel_leaves_a_wait_that_its_clock_never_ends(dev, o
         return e0.elapsed_ms(e1)
 
     timed_ms()
-    usual = timed_ms()
+    usual = min(timed_ms() for _ in range(3))
     want = dy.to_numpy()
     assert mismatch_count(want[0, :64], oracle.softmax(x[0, :64])) == 0
     _lib.check(dev.lib.rt_debug_softmax_pace(dev.handle, 1 << 28))     # 2.7 s a step, if anything waited for it
@@ -165,7 +165,7 @@ def test_softmax_streaming_kernel_leaves_a_wait_that_its_clock_never_ends(dev, o
         _lib.check(dev.lib.rt_debug_softmax_pace(dev.handle, 0))
     assert mismatch_count(got, want) == 0
     # 16 steps a block, each held for 4096 looks at the clock and no longer: milliseconds, not the 43 s of the pace asked for
-    assert 10 * usual < held < 2000.0, (usual, held)
+    assert max(5 * usual, 0.5) < held < 2000.0, (usual, held)
     again = dev.softmax(dx).to_numpy()                                 # and the computed pace is back
     assert mismatch_count(again, want) == 0
 
