@@ -387,3 +387,47 @@ def test_group_norm_across_the_4_gib_boundary(dev, oracle):
             want = ((xs - mu) / np.sqrt(var + 1e-5) * float(w[c]) + float(bi[c])).astype(np.float16)
             bad, mx = oracle.count_not_close(got, want, 1e-3, 1e-3)
             assert bad == 0, (pair, ch, mx)
+
+
+def test_f32_rows_broadcast_and_index_write_across_the_4_gib_boundary(dev, oracle):
+    """f32 softmax and norms on [716800, 1500] (4.3 GB; rows of 6000 bytes, so most rows start off a 128-byte line), a
+    broadcast to 4.3 GB and an index_write into the far end of a 4.3 GB destination."""
+    from ratchet_amd import _lib
+    from ratchet_amd.runtime import BufferView
+
+    P = 1 << 22
+    rows, cols = 716800, 1500
+    n = rows * cols
+    rng = np.random.default_rng(712)
+    pat = rng.standard_normal(P).astype(np.float32)
+    x = dev.empty((rows, cols), F32)
+    dp = dev.upload(pat)
+    for k in range(0, n, P):
+        _lib.check(dev.lib.rt_d2d(dev.handle, x.ptr.value + 4 * k, dp.ptr, 4 * min(P, n - k)))
+    at = [0, (1 << 32) // (4 * cols) - 1, (1 << 32) // (4 * cols), (1 << 32) // (4 * cols) + 1, rows - 2, rows - 1]
+    want_rows = np.stack([pat[(r * cols + np.arange(cols, dtype=np.int64)) % P] for r in at])
+
+    def rows_of(buf):
+        return np.stack([BufferView(buf, r * cols, (cols,)).to_numpy() for r in at])
+
+    g = (1 + 0.02 * rng.standard_normal(cols)).astype(np.float32)
+    b = (0.02 * rng.standard_normal(cols)).astype(np.float32)
+    out = dev.softmax(x)
+    bad, mx = oracle.count_not_close(rows_of(out), oracle.softmax(want_rows), 1e-5, 1e-5)
+    assert bad == 0, mx
+    dev.layer_norm(x, dev.upload(g), dev.upload(b), 1e-5, out=out)
+    bad, mx = oracle.count_not_close(rows_of(out), oracle.layer_norm(want_rows, g, b, 1e-5, intended=True), 1e-5, 1e-5)
+    assert bad == 0, mx
+    dev.rms_norm(x, dev.upload(g), 1e-5, out=out)
+    bad, mx = oracle.count_not_close(rows_of(out), oracle.rms_norm(want_rows, g, 1e-5, intended=True), 1e-5, 1e-5)
+    assert bad == 0, mx
+    del out
+    # broadcast [1, 1, 1500] over 716800 rows, then overwrite two rows at the far end through index_write
+    row = rng.standard_normal((1, 1, cols)).astype(np.float32)
+    big = dev.broadcast_to(dev.upload(row), (1, rows, cols))
+    for r in at:
+        assert same_bits(BufferView(big, r * cols, (cols,)).to_numpy(), row[0, 0]), r
+    patch = rng.standard_normal((1, 2, cols)).astype(np.float32)
+    dev.index_write(big, dev.upload(patch), (0, rows - 2, 0))
+    assert same_bits(BufferView(big, (rows - 2) * cols, (2 * cols,)).to_numpy(), patch.reshape(-1))
+    assert same_bits(BufferView(big, (rows - 3) * cols, (cols,)).to_numpy(), row[0, 0])
