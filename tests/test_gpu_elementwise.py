@@ -304,3 +304,29 @@ def test_broadcast_binary_streaming_variants(dev, oracle, a_shape, b_shape):
         check(dev.lib.rt_binary_bcast(dev.handle, _lib.BINARY_OPS.index(op), da.dt, da.ptr, shape4(a_shape), db.ptr, shape4(b_shape), out.ptr,
                                       shape4(shape)))
         assert same_bits(out.to_numpy(), want), (op, a_shape, b_shape)
+
+
+def test_empty_tensors_are_no_ops(dev):
+    """An op over no elements (or no rows) succeeds, launches nothing and leaves its output as it was; ops whose shape
+    arguments hold a zero extent are refused with RT_ERR_SHAPE before anything runs (checked without a GPU in test_abi)."""
+    import ctypes
+    from ratchet_amd import _lib
+
+    L, h = dev.lib, dev.handle
+    keep = np.arange(64, dtype=np.float32)
+    a, y = dev.upload(keep), dev.upload(keep)
+    u4 = lambda *s: (ctypes.c_uint32 * 4)(*s)
+    calls = [
+        L.rt_binary(h, _lib.BINARY_OPS.index("add"), _lib.F32, a.ptr, a.ptr, y.ptr, 0),
+        L.rt_unary(h, _lib.UNARY_OPS.index("gelu"), _lib.F32, a.ptr, y.ptr, 0),
+        L.rt_unary_via_f32(h, _lib.UNARY_OPS.index("gelu"), _lib.F16, a.ptr, y.ptr, 0),
+        L.rt_cast(h, _lib.F32, _lib.F16, a.ptr, y.ptr, 0),
+        L.rt_softmax(h, _lib.F32, a.ptr, y.ptr, 0, 8, 0),
+        L.rt_layer_norm(h, _lib.F32, a.ptr, a.ptr, a.ptr, y.ptr, 0, 8, 1e-5),
+        L.rt_rms_norm(h, _lib.F32, a.ptr, a.ptr, y.ptr, 0, 8, 1e-5),
+        L.rt_norm_via_f32(h, 0, _lib.F16, a.ptr, a.ptr, a.ptr, y.ptr, 0, 8, 1e-5),
+        L.rt_gated_mul_via_f32(h, _lib.UNARY_OPS.index("silu"), _lib.F16, a.ptr, 8, a.ptr, 8, y.ptr, 0, 8),
+        L.rt_index_write(h, 4, y.ptr, u4(1, 1, 8, 8), a.ptr, 0, u4(0, 0, 0, 0)),
+    ]
+    assert calls == [0] * len(calls), calls
+    assert same_bits(y.to_numpy(), keep)
