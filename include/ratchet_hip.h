@@ -65,15 +65,6 @@ int rt_device_destroy(rt_device* dev);
 int rt_sync(rt_device* dev);                                 /* device.poll(Wait) (tensor.rs:855-856) */
 const char* rt_last_error(void);                             /* message for the last non-zero status, thread-local */
 const char* rt_status_name(int status);
-/* Test hook, no counterpart in the reference: maps a HIP error code the way every entry point maps a failed HIP call
- * (status = -code, rt_last_error() = "<what>: <hipGetErrorString> (<hipGetErrorName>)", the runtime's sticky error
- * cleared), so that the mapping can be checked without a failing GPU.  hip_error 0 returns RT_OK and leaves the message. */
-int rt_debug_hip_status(int hip_error, const char* what);
-/* Test hook, no counterpart in the reference: the streaming 16-bit softmax holds its blocks to a pace by the device's
- * wall clock; `ticks` (of that clock, < 2^30) replaces the pace the launcher computes, 0 restores it.  With a pace far
- * beyond what a step takes every wait runs into its own bound (4096 looks at the clock) and the kernel must still
- * finish with the same results: that is what the test checks, with every wave leaving the kernel normally. */
-int rt_debug_softmax_pace(rt_device* dev, uint32_t ticks);
 int rt_malloc(rt_device* dev, size_t bytes, void** dptr);    /* BufferPool::get_or_create (buffer_pool.rs:68-116): sizes
                                                                 are rounded up to 4 B, minimum 16 B (:82-93) */
 int rt_free(rt_device* dev, void* dptr);                     /* last drop of a PooledGPUBuffer */

@@ -985,20 +985,35 @@ struct Resolver {
                 if (it == last_use.end() || it->second < at) last_use[src] = at;
             }
         }
-        // every holder of the node is an edge of this graph: no user handle, no other graph
-        auto hidden = [&](Node* n, const Tensor& handle) { return n != root && !n->srcs.empty() && (size_t)Node::holders(handle) == edges[n]; };
-        std::unordered_set<Node*> hidden_nodes;
+        // every holder of the node is an edge of this graph: no user handle, no other graph.  A view aliases its source's
+        // buffer, so a source is only hidden when every view of it is hidden too (a view kept by the caller, or the root
+        // being a view, keeps the buffer below it visible); consumers come after their sources in `order`, so the walk
+        // goes backwards and a view's own answer is known before its source asks.
+        std::unordered_map<Node*, const Tensor*> handle_of;        // (a pointer: a copy would be one more holder)
+        std::unordered_map<Node*, std::vector<Node*>> views_of;
         for (Node* n : order) {
             if (n->storage) continue;
             for (const Tensor& s : n->srcs) {
-                Node* src = Node::of(s);
-                if (hidden(src, s)) {
-                    hidden_nodes.insert(src);
-                    if (last_use.count(src)) {
-                        P.release_at[last_use[src]].push_back(src);
-                        last_use.erase(src);
-                    }
-                }
+                handle_of.emplace(Node::of(s), &s);
+                if (n->kind == Kind::View) views_of[Node::of(s)].push_back(n);
+            }
+        }
+        std::unordered_set<Node*> hidden_nodes;
+        for (auto it = order.rbegin(); it != order.rend(); ++it) {
+            Node* src = *it;
+            auto h = handle_of.find(src);
+            if (h == handle_of.end()) continue;                    // nobody in this graph reads it
+            bool hidden = src != root && !src->srcs.empty() && (size_t)Node::holders(*h->second) == edges[src];
+            if (hidden) {
+                auto v = views_of.find(src);
+                if (v != views_of.end())
+                    for (Node* view : v->second) hidden = hidden && hidden_nodes.count(view);
+            }
+            if (!hidden) continue;
+            hidden_nodes.insert(src);
+            if (last_use.count(src)) {
+                P.release_at[last_use[src]].push_back(src);
+                last_use.erase(src);
             }
         }
 

@@ -7,6 +7,7 @@
 #include <stddef.h>
 
 #include "../../include/ratchet_hip.h"
+#include "../../include/ratchet_hip_debug.h"
 
 constexpr size_t RT_SM_ROW_SUMS = 1u << 19;
 

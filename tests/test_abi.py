@@ -1,4 +1,4 @@
-"""CPU-only checks of the C ABI: the library loads without a GPU, exports every symbol include/ratchet_hip.h declares, and
+"""CPU-only checks of the C ABI: the library loads without a GPU, exports every symbol the headers under include/ declare, and
 rejects bad arguments before touching HIP (so these paths are testable here; no compute call needs a device).
 
 Error behaviour mirrors the reference's guards: Permute duplicate dims (ops/reindex/permute.rs:49-52), Broadcast shape
@@ -25,36 +25,56 @@ def u4(*v):
     return (ctypes.c_uint32 * 4)(*v)
 
 
-def test_header_and_library_agree(lib):
-    header = open(os.path.join(ROOT, "include", "ratchet_hip.h")).read()
-    declared = sorted(set(re.findall(r"^(?:int|const char\*)\s+(rt_[a-z0-9_]+)\(", header, flags=re.M)))
-    assert declared, "no declarations parsed"
-    for name in declared:
-        assert hasattr(lib, name), f"{name} is declared in ratchet_hip.h but not exported"
-    assert sorted(_lib.EXPORTS) == declared
+HEADERS = ("ratchet_hip.h", "ratchet_hip_debug.h")     # the seam a -sys crate binds, and the library's test hooks
 
 
-def test_rust_binding_in_integration_md_lists_the_header_s_entry_points():
-    """the integration guide at the repository root shows the `extern "C"` block a ratchet maintainer would put into the
-    -sys crate; it has to name every entry point ratchet_hip.h declares, no other, each with as many arguments as the C
-    declaration has"""
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    header = open(os.path.join(root, "include", "ratchet_hip.h")).read()
+def c_declarations(name):
+    """{entry point: argument list} of one header under include/, comments removed"""
+    header = open(os.path.join(ROOT, "include", name)).read()
     header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
-    c_decls = {m.group(1): m.group(2) for m in re.finditer(r"\b(rt_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", header)}
-    doc = open(os.path.join(root, "INTEGRATION.md")).read()
-    block = doc[doc.index('extern "C" {'):]
-    block = block[:block.index("\n}\n")]
-    block = re.sub(r"//[^\n]*", "", block)
-    rust_decls = {m.group(1): m.group(2) for m in re.finditer(r"pub fn (rt_[a-z0-9_]+)\s*\((.*?)\)\s*->", block, flags=re.S)}
-    assert sorted(rust_decls) == sorted(c_decls)
+    return {m.group(1): m.group(2) for m in re.finditer(r"\b(rt_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", header)}
+
+
+def test_headers_and_library_agree(lib):
+    declared = []
+    for h in HEADERS:
+        names = sorted(c_declarations(h))
+        assert names, f"no declarations parsed in {h}"
+        declared += names
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared under include/ but not exported"
+    assert sorted(_lib.EXPORTS) == sorted(declared)
+    # the product header holds no test hook, the debug header nothing else
+    assert not [n for n in c_declarations("ratchet_hip.h") if n.startswith("rt_debug_")]
+    assert all(n.startswith("rt_debug_") for n in c_declarations("ratchet_hip_debug.h"))
+
+
+def test_rust_bindings_in_integration_md_list_the_headers_entry_points():
+    """the integration guide at the repository root shows the `extern "C"` blocks a ratchet maintainer would put into the
+    -sys crate: the first has to name every entry point ratchet_hip.h declares, no other, each with as many arguments as
+    the C declaration has; the second (behind a feature) does the same for ratchet_hip_debug.h"""
+    doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    blocks = []
+    at = 0
+    while True:
+        at = doc.find('extern "C" {', at)
+        if at < 0:
+            break
+        end = doc.index("\n}\n", at)
+        blocks.append(re.sub(r"//[^\n]*", "", doc[at:end]))
+        at = end
+    assert len(blocks) == len(HEADERS)
 
     def count(args, void_word):
         args = args.strip()
         return 0 if args in ("", void_word) else args.count(",") + 1
 
-    for name in c_decls:
-        assert count(rust_decls[name], "") == count(c_decls[name], "void"), name
+    for h, block in zip(HEADERS, blocks):
+        c_decls = c_declarations(h)
+        rust_decls = {m.group(1): m.group(2) for m in re.finditer(r"pub fn (rt_[a-z0-9_]+)\s*\((.*?)\)\s*->", block, flags=re.S)}
+        assert sorted(rust_decls) == sorted(c_decls), h
+        for name in c_decls:
+            assert count(rust_decls[name], "") == count(c_decls[name], "void"), name
 
 
 def test_status_names(lib):

@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 
 from gpu_util import same_bits
+from ratchet_amd._lib import F16, F32
 
 pytestmark = pytest.mark.gpu
 
@@ -172,3 +173,29 @@ def test_dispatch_allocates_nothing_and_holds_what_the_plan_says(hdev):
         with pytest.raises(HostError) as e:
             done.compile()
         assert e.value.kind == "AlreadyResolved"
+
+
+def test_a_view_the_caller_keeps_still_shows_its_data_after_later_launches_reused_buffers(hdev, oracle):
+    # exp(x) is only held by a view; the casts behind the view are the tenants that a shared object would go to next
+    rng = np.random.default_rng(905)
+    x = rng.standard_normal((64, 1024)).astype(np.float32)
+    want_view = oracle.unary("exp", x)
+    for mode in ("resolve", "compile"):
+        a = T(x, hdev).exp()
+        v = a.view((64, 1024))
+        del a
+        e = v.cast(F16).cast(F32).cast(F16).cast(F32).neg()
+        exe = None
+        if mode == "resolve":
+            e.resolve()
+        else:
+            exe = e.compile()
+            exe.dispatch()
+        assert same_bits(v.to_numpy(), want_view), mode
+        # a second graph built on the kept view reads exp(x), not the last tenant's data
+        got = v.neg().resolve().to_numpy()
+        assert same_bits(got, oracle.unary("neg", want_view)), mode
+        want = oracle.unary("neg", oracle.cast(oracle.cast(oracle.cast(oracle.cast(want_view, np.float16), np.float32), np.float16), np.float32))
+        assert same_bits(e.to_numpy(), want), mode
+        if exe:
+            exe.close()

@@ -64,6 +64,60 @@ def test_a_tensor_the_caller_still_holds_is_never_shared():
     assert sorted(objects) == [2 * KB, 4 * KB]
 
 
+def test_a_kept_view_pins_the_tensor_it_aliases():
+    """a view shares its source's buffer: while the caller holds the view, the source must not be housed in an object
+    that later launches reuse, although every holder of the source itself is an edge of the graph"""
+    x = P(1024)
+    a = x.exp()
+    v = a.view((1024,))
+    aid = a.id
+    del a
+    e = v.cast(F16).cast(F32).cast(F16).cast(F32)
+    objects, entries = e.memory_plan()
+    by_id = {t["id"]: t for t in entries}
+    assert by_id[aid]["object"] == -1                                  # own allocation: v keeps showing exp(x)
+    # dropped, the same view hides nothing: exp's buffer joins the shared objects again
+    x = P(1024)
+    a = x.exp()
+    aid = a.id
+    e = a.view((1024,)).cast(F16).cast(F32).cast(F16).cast(F32)
+    del a
+    objects, entries = e.memory_plan()
+    assert {t["id"]: t for t in entries}[aid]["object"] >= 0
+
+
+def test_a_view_read_by_a_second_unresolved_graph_pins_its_source():
+    x = P(1024)
+    a = x.exp()
+    v = a.view((1024,))
+    aid = a.id
+    del a
+    other = v.neg()                                                    # a second graph, not resolved yet, reads the view
+    e = v.cast(F16).cast(F32).cast(F16).cast(F32)
+    objects, entries = e.memory_plan()
+    assert {t["id"]: t for t in entries}[aid]["object"] == -1
+    # a view of a view: the chain is followed down to the buffer's owner
+    x = P(1024)
+    a = x.exp()
+    aid = a.id
+    vv = a.view((1024,)).view((1024,))
+    del a
+    e = vv.cast(F16).cast(F32).cast(F16).cast(F32)
+    objects, entries = e.memory_plan()
+    assert {t["id"]: t for t in entries}[aid]["object"] == -1
+    del other
+
+
+def test_the_root_being_a_view_pins_its_source():
+    x = P(1024)
+    a = x.exp().cast(F16).cast(F32)
+    aid = a.id
+    root = a.view((1024,))
+    del a
+    objects, entries = root.memory_plan()
+    assert {t["id"]: t for t in entries}[aid]["object"] == -1
+
+
 def test_diamond_keeps_the_shared_operand_alive_to_its_last_reader():
     """a feeds both branches: its interval runs to the add at the end, so nothing else may use its object"""
     x = P(2048)
