@@ -31,6 +31,9 @@ PEAK_HBM_GBPS = 8000.0
 # WRITE_SIZE).  Read at run time; a missing file or row gives null, never a stale literal.
 PROFILE_KERNEL_TRACE = os.path.join("profiles", "bench_step_kernel_trace.txt")
 PROFILE_HBM_TRAFFIC = os.path.join("profiles", "bench_step_hbm_traffic_pmc.txt")
+# algorithmic bytes of the 17 ops of the step, in step order (what build_workload's rows carry; checked against them in main)
+STEP_ALG_BYTES = [108000000, 4608000, 4608000, 31457280, 20981760, 83886080, 31457280, 31457280, 50337792, 134217728, 201326592,
+                  2181038080, 2147483648, 20971520, 6146048, 268570624, 20971520]
 
 
 def read_step_rows(rel_path):
@@ -45,6 +48,29 @@ def read_step_rows(rel_path):
     except (OSError, ValueError):
         return {}
     return rows
+
+
+def profile_head(rel_path):
+    """the `git_head:` line of a profile summary: the commit whose kernels it describes"""
+    try:
+        with open(os.path.join(ROOT, rel_path)) as f:
+            for line in f:
+                if line.startswith("git_head:"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return None
+
+
+def git_head():
+    """commit of the tree this script runs from, when it is a git checkout (the GPU box receives the tree without .git)"""
+    try:
+        head = open(os.path.join(ROOT, ".git", "HEAD")).read().strip()
+        if head.startswith("ref:"):
+            return open(os.path.join(ROOT, ".git", head.split(" ", 1)[1])).read().strip()[:12]
+        return head[:12]
+    except OSError:
+        return None
 
 
 F32, F16 = 0, 1
@@ -62,15 +88,22 @@ def normal(seed, stream, shape, std, dtype, mean=0.0):
 
 
 class Op:
-    """One benchmark row: device buffers, a launch closure, algorithmic bytes, and a CPU check/baseline closure."""
+    """One benchmark row: device buffers, a launch closure, algorithmic bytes, and a CPU check/baseline closure.
+    `call(ins, out)` enqueues the op on the buffers it is given; `ins` / `out` are the buffers of the step (set 0).
+    `rotating` lists which inputs get copies of their own in the sets of the event-free pass (the large operands; scale,
+    bias and other small vectors are shared)."""
 
-    def __init__(self, cfg, name, dtype, shapes, alg_bytes, launch, cpu_sample, kernel=None):
+    def __init__(self, cfg, name, dtype, shapes, alg_bytes, call, ins, out, cpu_sample, kernel, rotating=None):
         self.cfg, self.name, self.dtype, self.shapes = cfg, name, dtype, shapes
         self.alg_bytes = int(alg_bytes)
-        self.launch = launch
-        self.cpu_sample = cpu_sample        # () -> (want, got_fn, tol, sample_alg_bytes, run_fn)
-        self.kernel = kernel
+        self.call, self.ins, self.out = call, list(ins), out
+        self.rotating = list(range(len(ins))) if rotating is None else list(rotating)
+        self.cpu_sample = cpu_sample        # dict: how to check the output buffer of set 0 and what to time on the CPU
+        self.kernel = kernel                # substring of the kernel's name in a rocprofv3 trace
         self.us = []
+
+    def launch(self):
+        self.call(self.ins, self.out)
 
 
 def build_workload(dev, seed):
@@ -91,19 +124,19 @@ def build_workload(dev, seed):
     scores1 = normal(seed, nxt(), (1, 6, 1500, 1500), 3.0, np32)
     d_scores1 = up(scores1)
     d_soft1 = dev.empty(scores1.shape, F32)
-    ops.append(Op(1, "softmax", "f32", "[1,6,1500,1500]", 2 * scores1.nbytes, lambda: dev.softmax(d_scores1, out=d_soft1),
-                  dict(kind="softmax", x=scores1, out=d_soft1, rows=9000, tol=1e-5), kernel="softmax_wave_kernel"))
+    ops.append(Op(1, "softmax", "f32", "[1,6,1500,1500]", 2 * scores1.nbytes, lambda i, o: dev.softmax(i[0], out=o), [d_scores1], d_soft1,
+                  dict(kind="softmax", x=scores1, out=d_soft1, rows=9000, tol=1e-5), "softmax_wave_kernel"))
     q1 = normal(seed, nxt(), (1, 1500, 6, 64), 1.0, np32)
     d_q1 = up(q1)
     d_q1p = dev.empty((1, 6, 1500, 64), F32)
     d_q1b = dev.empty((1, 1500, 6, 64), F32)
     q1p = np.ascontiguousarray(q1.transpose(0, 2, 1, 3))
     ops.append(Op(1, "permute[0,2,1,3]", "f32", "[1,1500,6,64]->[1,6,1500,64]", 2 * q1.nbytes,
-                  lambda: dev.permute(d_q1, (0, 2, 1, 3), out=d_q1p),
-                  dict(kind="exact", out=d_q1p, run=lambda o: o.permute(q1, (0, 2, 1, 3)), bytes=2 * q1.nbytes)))
+                  lambda i, o: dev.permute(i[0], (0, 2, 1, 3), out=o), [d_q1], d_q1p,
+                  dict(kind="exact", out=d_q1p, run=lambda o: o.permute(q1, (0, 2, 1, 3)), bytes=2 * q1.nbytes), "gather_vec_kernel"))
     ops.append(Op(1, "permute back", "f32", "[1,6,1500,64]->[1,1500,6,64]", 2 * q1.nbytes,
-                  lambda: dev.permute(d_q1p, (0, 2, 1, 3), out=d_q1b),
-                  dict(kind="exact", out=d_q1b, run=lambda o: o.permute(q1p, (0, 2, 1, 3)), bytes=2 * q1.nbytes)))
+                  lambda i, o: dev.permute(i[0], (0, 2, 1, 3), out=o), [d_q1p], d_q1b,
+                  dict(kind="exact", out=d_q1b, run=lambda o: o.permute(q1p, (0, 2, 1, 3)), bytes=2 * q1.nbytes), "gather_vec_kernel"))
 
     # ------------------------------------------------------------------ cfg 2: Phi-2 prefill elementwise block, f16
     x2 = normal(seed, nxt(), (1, 2048, 2560), 1.0, np16)
@@ -115,18 +148,18 @@ def build_workload(dev, seed):
     d_res2, d_ln2, d_gelu2 = dev.empty(x2.shape, F16), dev.empty(x2.shape, F16), dev.empty(h2.shape, F16)
     d_x2f32, d_x2f16 = dev.empty(x2.shape, F32), dev.empty(x2.shape, F16)
     x2_f32 = x2.astype(np32)
-    ops.append(Op(2, "residual add", "f16", "[1,2048,2560]x2", 3 * x2.nbytes, lambda: dev.binary("add", d_x2, d_a2, out=d_res2),
-                  dict(kind="exact", out=d_res2, run=lambda o: o.binary("add", x2, a2), bytes=3 * x2.nbytes)))
+    ops.append(Op(2, "residual add", "f16", "[1,2048,2560]x2", 3 * x2.nbytes, lambda i, o: dev.binary("add", i[0], i[1], out=o), [d_x2, d_a2], d_res2,
+                  dict(kind="exact", out=d_res2, run=lambda o: o.binary("add", x2, a2), bytes=3 * x2.nbytes), "binary_vec_kernel"))
     ops.append(Op(2, "layer_norm", "f16", "2048x2560", 2 * x2.nbytes + g2.nbytes + b2.nbytes,
-                  lambda: dev.layer_norm(d_x2, d_g2, d_b2, 1e-5, out=d_ln2),
+                  lambda i, o: dev.layer_norm(i[0], i[1], i[2], 1e-5, out=o), [d_x2, d_g2, d_b2], d_ln2,
                   dict(kind="rows", out=d_ln2, x=x2, rows=2048, tol=1e-3, fn=lambda o, xs: o.layer_norm(xs, g2, b2, 1e-5, intended=True)),
-                  kernel="norm_pipe16_kernel"))
-    ops.append(Op(2, "gelu", "f16", "[1,2048,10240]", 2 * h2.nbytes, lambda: dev.unary("gelu", d_h2, out=d_gelu2),
-                  dict(kind="rows", out=d_gelu2, x=h2, rows=2048, tol=1e-3, fn=lambda o, xs: o.unary("gelu", xs)), kernel="unary_lut_kernel"))
-    ops.append(Op(2, "cast f16->f32", "f16->f32", "[1,2048,2560]", x2.nbytes * 3, lambda: dev.cast(d_x2, F32, out=d_x2f32),
-                  dict(kind="exact", out=d_x2f32, run=lambda o: o.cast(x2, np32), bytes=3 * x2.nbytes)))
-    ops.append(Op(2, "cast f32->f16", "f32->f16", "[1,2048,2560]", x2.nbytes * 3, lambda: dev.cast(d_x2f32, F16, out=d_x2f16),
-                  dict(kind="exact", out=d_x2f16, run=lambda o: o.cast(x2_f32, np16), bytes=3 * x2.nbytes)))
+                  "norm_pipe16_kernel", rotating=[0]))
+    ops.append(Op(2, "gelu", "f16", "[1,2048,10240]", 2 * h2.nbytes, lambda i, o: dev.unary("gelu", i[0], out=o), [d_h2], d_gelu2,
+                  dict(kind="rows", out=d_gelu2, x=h2, rows=2048, tol=1e-3, fn=lambda o, xs: o.unary("gelu", xs)), "unary_lut_kernel"))
+    ops.append(Op(2, "cast f16->f32", "f16->f32", "[1,2048,2560]", x2.nbytes * 3, lambda i, o: dev.cast(i[0], F32, out=o), [d_x2], d_x2f32,
+                  dict(kind="exact", out=d_x2f32, run=lambda o: o.cast(x2, np32), bytes=3 * x2.nbytes), "cast_vec_kernel"))
+    ops.append(Op(2, "cast f32->f16", "f32->f16", "[1,2048,2560]", x2.nbytes * 3, lambda i, o: dev.cast(i[0], F16, out=o), [d_x2f32], d_x2f16,
+                  dict(kind="exact", out=d_x2f16, run=lambda o: o.cast(x2_f32, np16), bytes=3 * x2.nbytes), "cast_vec_kernel"))
 
     # ------------------------------------------------------------------ cfg 3: Phi-3-mini prefill, f16
     x3 = normal(seed, nxt(), (1, 4096, 3072), 1.0, np16)
@@ -135,16 +168,17 @@ def build_workload(dev, seed):
     up3 = normal(seed, nxt(), (1, 4096, 8192), 1.0, np16)
     d_x3, d_g3, d_gate3, d_up3 = up(x3), up(g3), up(gate3), up(up3)
     d_rms3, d_silu3, d_swiglu3 = dev.empty(x3.shape, F16), dev.empty(gate3.shape, F16), dev.empty(gate3.shape, F16)
-    ops.append(Op(3, "rms_norm", "f16", "4096x3072", 2 * x3.nbytes + g3.nbytes, lambda: dev.rms_norm(d_x3, d_g3, 1e-5, out=d_rms3),
+    ops.append(Op(3, "rms_norm", "f16", "4096x3072", 2 * x3.nbytes + g3.nbytes, lambda i, o: dev.rms_norm(i[0], i[1], 1e-5, out=o), [d_x3, d_g3], d_rms3,
                   dict(kind="rows", out=d_rms3, x=x3, rows=4096, tol=1e-3, fn=lambda o, xs: o.rms_norm(xs, g3, 1e-5, intended=True)),
-                  kernel="norm_pipe16_kernel"))
-    ops.append(Op(3, "silu(gate)", "f16", "[1,4096,8192]", 2 * gate3.nbytes, lambda: dev.unary("silu", d_gate3, out=d_silu3),
-                  dict(kind="rows", out=d_silu3, x=gate3, rows=4096, tol=1e-3, fn=lambda o, xs: o.unary("silu", xs)), kernel="unary_lut_kernel"))
-    ops.append(Op(3, "mul silu(gate)*up", "f16", "[1,4096,8192]x2", 3 * gate3.nbytes, lambda: dev.binary("mul", d_up3, d_silu3, out=d_swiglu3),
+                  "norm_pipe16_kernel", rotating=[0]))
+    ops.append(Op(3, "silu(gate)", "f16", "[1,4096,8192]", 2 * gate3.nbytes, lambda i, o: dev.unary("silu", i[0], out=o), [d_gate3], d_silu3,
+                  dict(kind="rows", out=d_silu3, x=gate3, rows=4096, tol=1e-3, fn=lambda o, xs: o.unary("silu", xs)), "unary_lut_kernel"))
+    ops.append(Op(3, "mul silu(gate)*up", "f16", "[1,4096,8192]x2", 3 * gate3.nbytes, lambda i, o: dev.binary("mul", i[0], i[1], out=o),
+                  [d_up3, d_silu3], d_swiglu3,
                   dict(kind="rows2", out=d_swiglu3, rows=4096,
                        prep=lambda o, n: (up3.reshape(4096, 8192)[:n], o.unary("silu", gate3.reshape(4096, 8192)[:n])),
                        fn=lambda o, inp: o.binary("mul", inp[0], inp[1]),
-                       tol=0.0, bytes_per_row=3 * 8192 * 2)))
+                       tol=0.0, bytes_per_row=3 * 8192 * 2), "binary_vec_kernel"))
     # scores [1,32,4096,4096]: one head of N(0,2) generated on the host, replicated over the 32 heads on the device
     S, H = 4096, 32
     head = normal(seed, nxt(), (S, S), 2.0, np16)
@@ -157,14 +191,14 @@ def build_workload(dev, seed):
     d_soft3 = dev.empty((1, H, S, S), F16)
     nb = H * head.nbytes
     ops.append(Op(3, "scores + causal mask (broadcast fused)", "f16", "[1,32,4096,4096]+[4096,4096]", 2 * nb + mask.nbytes,
-                  lambda: dev.binary("add", d_scores3, d_mask, out=d_masked3),
+                  lambda i, o: dev.binary("add", i[0], i[1], out=o), [d_scores3, d_mask], d_masked3,
                   dict(kind="rows2", out=d_masked3, rows=H * S, tol=0.0, bytes_per_row=2 * S * 2 + S * 2 / H,     # the mask counts once, as in the op's own bytes
                        prep=lambda o, n: (np.tile(head, (n // S, 1)), np.tile(mask, (n // S, 1))),
-                       fn=lambda o, inp: o.binary("add", inp[0], inp[1])), kernel="binary_bcast_kernel"))
-    ops.append(Op(3, "softmax (causal)", "f16", "131072x4096", 2 * nb, lambda: dev.softmax(d_masked3, out=d_soft3),
+                       fn=lambda o, inp: o.binary("add", inp[0], inp[1])), "binary_bcast_kernel"))
+    ops.append(Op(3, "softmax (causal)", "f16", "131072x4096", 2 * nb, lambda i, o: dev.softmax(i[0], out=o), [d_masked3], d_soft3,
                   dict(kind="rows2", out=d_soft3, rows=H * S, tol=0.0, bytes_per_row=2 * S * 2,
                        prep=lambda o, n: np.tile(o.binary("add", head, mask), (n // S, 1)),
-                       fn=lambda o, inp: o.softmax(inp)), kernel="softmax16_stream_kernel"))
+                       fn=lambda o, inp: o.softmax(inp)), "softmax16_stream_kernel"))
 
     # ------------------------------------------------------------------ cfg 4: broadcast / reindex stress, f16
     kv_a = normal(seed, nxt(), (1, 32, 1984, 80), 1.0, np16)
@@ -172,34 +206,37 @@ def build_workload(dev, seed):
     d_kva, d_kvb = up(kv_a), up(kv_b)
     d_kv = dev.empty((1, 32, 2048, 80), F16)
     ops.append(Op(4, "concat dim 2", "f16", "[1,32,1984,80]+[1,32,64,80]", 2 * (kv_a.nbytes + kv_b.nbytes),
-                  lambda: dev.concat([d_kva, d_kvb], 2, out=d_kv),
-                  dict(kind="exact", out=d_kv, run=lambda o: o.concat([kv_a, kv_b], 2), bytes=2 * (kv_a.nbytes + kv_b.nbytes))))
+                  lambda i, o: dev.concat([i[0], i[1]], 2, out=o), [d_kva, d_kvb], d_kv,
+                  dict(kind="exact", out=d_kv, run=lambda o: o.concat([kv_a, kv_b], 2), bytes=2 * (kv_a.nbytes + kv_b.nbytes)), "concat_kernel"))
     gx = normal(seed, nxt(), (1, 512, 3000), 1.0, np16)
     gw = normal(seed, nxt(), (512,), 0.02, np16, mean=1.0)
     gb = normal(seed, nxt(), (512,), 0.02, np16)
     d_gx, d_gw, d_gb = up(gx), up(gw), up(gb)
     d_gn = dev.empty(gx.shape, F16)
     ops.append(Op(4, "group_norm G=32", "f16", "[1,512,3000]", 2 * gx.nbytes + gw.nbytes + gb.nbytes,
-                  lambda: dev.group_norm(d_gx, 32, d_gw, d_gb, 1e-5, out=d_gn),
-                  dict(kind="close", out=d_gn, tol=1e-3, run=lambda o: o.group_norm(gx, 32, gw, gb, 1e-5), bytes=2 * gx.nbytes)))
+                  lambda i, o: dev.group_norm(i[0], 32, i[1], i[2], 1e-5, out=o), [d_gx, d_gw, d_gb], d_gn,
+                  dict(kind="close", out=d_gn, tol=1e-3, run=lambda o: o.group_norm(gx, 32, gw, gb, 1e-5), bytes=2 * gx.nbytes),
+                  "gn_reg_kernel", rotating=[0]))
     ma = normal(seed, nxt(), (1, 32, 2048, 1), 1.0, np16)
     mb = normal(seed, nxt(), (1, 1, 1, 2048), 1.0, np16)
     d_ma, d_mb = up(ma), up(mb)
     d_mm = dev.empty((1, 32, 2048, 2048), F16)
     ops.append(Op(4, "mul two-sided broadcast (fused)", "f16", "[1,32,2048,1]x[1,1,1,2048]", ma.nbytes + mb.nbytes + d_mm.nbytes,
-                  lambda: dev.binary("mul", d_ma, d_mb, out=d_mm),
+                  lambda i, o: dev.binary("mul", i[0], i[1], out=o), [d_ma, d_mb], d_mm,
                   dict(kind="rows2", out=d_mm, rows=65536, tol=0.0, bytes_per_row=2048 * 2,
                        prep=lambda o, n: n,         # the reference's CPU path materialises both broadcasts: that stays inside the timed region
                        fn=lambda o, n: o.binary("mul", np.ascontiguousarray(np.broadcast_to(ma.reshape(-1, 1)[:n], (n, 2048))),
-                                                np.ascontiguousarray(np.broadcast_to(mb.reshape(1, 2048), (n, 2048)))))))
+                                                np.ascontiguousarray(np.broadcast_to(mb.reshape(1, 2048), (n, 2048))))),
+                  "binary_bcast_kernel"))
     p4 = normal(seed, nxt(), (1, 2048, 32, 80), 1.0, np16)
     d_p4 = up(p4)
     d_p4o = dev.empty((1, 32, 2048, 80), F16)
     ops.append(Op(4, "permute[0,2,1,3]", "f16", "[1,2048,32,80]->[1,32,2048,80]", 2 * p4.nbytes,
-                  lambda: dev.permute(d_p4, (0, 2, 1, 3), out=d_p4o),
-                  dict(kind="exact", out=d_p4o, run=lambda o: o.permute(p4, (0, 2, 1, 3)), bytes=2 * p4.nbytes)))
+                  lambda i, o: dev.permute(i[0], (0, 2, 1, 3), out=o), [d_p4], d_p4o,
+                  dict(kind="exact", out=d_p4o, run=lambda o: o.permute(p4, (0, 2, 1, 3)), bytes=2 * p4.nbytes), "gather_vec_kernel"))
     ops_extra["copy_pair"] = (d_scores3, d_masked3)
     ops_extra["attn"] = (d_scores3, d_mask, d_masked3, d_soft3)
+    ops_extra["head"] = (head, mask)
     return ops
 
 
@@ -472,6 +509,190 @@ def host_graph_step(seed):
                     "eight launches on, call by call below that), one wait"}
 
 
+def rotating_sets(dev, op, min_bytes=768e6, max_sets=192):
+    """[(ins, out), ...]: the op's own buffers plus copies of its large operands and outputs, enough of them that going
+    round the sets moves more than `min_bytes` (three Infinity Caches) before a buffer comes up again"""
+    from ratchet_amd import _lib
+
+    k = int(min(max_sets, max(1, -(-int(min_bytes) // op.alg_bytes))))
+    sets = [(op.ins, op.out)]
+    for _ in range(k - 1):
+        ins = list(op.ins)
+        for j in op.rotating:
+            b = dev.empty(op.ins[j].shape, op.ins[j].dt)
+            _lib.check(dev.lib.rt_d2d(dev.handle, b.ptr, op.ins[j].ptr, b.nbytes))
+            ins[j] = b
+        sets.append((ins, dev.empty(op.out.shape, op.out.dt)))
+    return sets
+
+
+def time_without_events(dev, op, min_launches=24):
+    """us per launch with nothing between the launches: the op issued back to back over its rotating sets (cold operands
+    every time), one pair of events around the whole run.  What `us` of the per-op pass has on top of this is the two
+    events and the completion signal each of them forces."""
+    sets = rotating_sets(dev, op)
+    n = max(min_launches, 2 * len(sets)) if op.alg_bytes < 768e6 else 6
+    for k in range(min(len(sets), 4)):
+        op.call(*sets[k])
+    dev.sync()
+    best = None
+    for _ in range(3):
+        e0, e1 = dev.event(), dev.event()
+        e0.record()
+        for k in range(n):
+            op.call(*sets[k % len(sets)])
+        e1.record()
+        t = e0.elapsed_ms(e1) * 1e3 / n
+        best = t if best is None else min(best, t)
+    del sets
+    return best, n
+
+
+def extra_rows(dev, seed, oracle):
+    """Rows reported beside the step, never part of `value`: inputs the step does not show.  (a) the f16 streaming softmax
+    on dense N(0,2) scores [1,32,4096,4096] (no mask, so no run of -inf: the table lookups of a wave fall into different
+    LDS banks); (b) BASELINE config 0, the reference's own CPU-runnable case, as three launches on [1,1500,384] f32:
+    bias add (broadcast fused), tanh GELU, LayerNorm.  Each with the copy of the same bytes timed the same way."""
+    import ctypes
+
+    from ratchet_amd import _lib
+
+    np16, np32 = np.float16, np.float32
+    rows = []
+    src, dst = ops_extra["copy_pair"]
+
+    def copy_us(nbytes, n=12):
+        half = (nbytes // 2) & ~15
+        ts = []
+        for k in range(n):
+            off = (k * half) % (src.nbytes - half) & ~255
+            e0, e1 = dev.event(), dev.event()
+            e0.record()
+            _lib.check(dev.lib.rt_cast(dev.handle, F16, F16, ctypes.c_void_p(src.ptr.value + off), ctypes.c_void_p(dst.ptr.value + off), half // 2))
+            e1.record()
+            ts.append(e0.elapsed_ms(e1) * 1e3)
+        return float(np.median(ts[2:]))
+
+    def timed(fn, n=12):
+        ts = []
+        for _ in range(n):
+            e0, e1 = dev.event(), dev.event()
+            e0.record()
+            fn()
+            e1.record()
+            ts.append(e0.elapsed_ms(e1) * 1e3)
+        return float(np.median(ts[2:]))
+
+    def add(name, shape, dtype, alg, us, ok, note=None):
+        c = copy_us(alg)
+        r = {"row": name, "shape": shape, "dtype": dtype, "alg_MB": round(alg / 1e6, 3), "us": round(us, 2), "GBps": round(alg / us / 1e3, 1),
+             "frac_hbm": round(alg / us / 1e3 / PEAK_HBM_GBPS, 4), "copy_us": round(c, 2), "frac_of_copy": round(c / us, 4), "parity_ok": ok}
+        if note:
+            r["note"] = note
+        rows.append(r)
+
+    # (a) dense scores: the score head itself, replicated over the heads, no mask added
+    scores, _mask, masked, soft = ops_extra["attn"]
+    head, _ = ops_extra["head"]
+    us = timed(lambda: dev.softmax(scores, out=soft), n=8)
+    ok = None
+    if oracle is not None:
+        want = oracle.softmax(head[:256])
+        got = download_rows(dev, soft, 256, head.shape[1], np16)
+        ok = bool(np.all((got.view(np.uint16) == want.view(np.uint16)) | (np.isnan(got) & np.isnan(want))))
+    add("softmax, dense scores (no mask)", "131072x4096", "f16", 2 * scores.nbytes, us, ok,
+        "launched back to back on a cold input; the causal row of the step reads what the mask add has just written")
+    # the causal input in the same position (back to back, input not just written), for comparison with the step's row
+    us = timed(lambda: dev.softmax(masked, out=soft), n=8)
+    add("softmax, causal scores, launched back to back", "131072x4096", "f16", 2 * scores.nbytes, us, None)
+
+    # (b) config 0
+    x = normal(seed, 801, (1, 1500, 384), 1.0, np32)
+    bias = normal(seed, 802, (384,), 0.02, np32)
+    g = normal(seed, 803, (384,), 0.02, np32, mean=1.0)
+    b = normal(seed, 804, (384,), 0.02, np32)
+    dx, dbias, dg, db = dev.upload(x), dev.upload(bias), dev.upload(g), dev.upload(b)
+    y1, y2, y3 = dev.empty(x.shape, F32), dev.empty(x.shape, F32), dev.empty(x.shape, F32)
+    h1 = h2 = h3 = None
+    if oracle is not None:
+        h1 = oracle.binary("add", x, np.ascontiguousarray(np.broadcast_to(bias, x.shape)))
+        h2 = oracle.unary("gelu", h1)
+        h3 = oracle.layer_norm(h2, g, b, 1e-5)
+    t1 = timed(lambda: dev.binary("add", dx, dbias, out=y1))
+    t2 = timed(lambda: dev.unary("gelu", y1, out=y2))
+    t3 = timed(lambda: dev.layer_norm(y2, dg, db, 1e-5, out=y3))
+    ok1 = ok2 = ok3 = None
+    if oracle is not None:
+        ok1 = bool(np.array_equal(y1.to_numpy().view(np.uint32), h1.view(np.uint32)))
+        ok2 = oracle.count_not_close(y2.to_numpy(), h2, 1e-5, 1e-5)[0] == 0
+        ok3 = oracle.count_not_close(y3.to_numpy(), h3, 1e-5, 1e-5)[0] == 0
+    note0 = "4.6 MB: the operands stay in the caches between repetitions (cache-warm, unlike the rows of the step)"
+    add("cfg0 bias add (broadcast fused)", "[1,1500,384]+[384]", "f32", 2 * x.nbytes + bias.nbytes, t1, ok1, note0)
+    add("cfg0 gelu (tanh approx)", "[1,1500,384]", "f32", 2 * x.nbytes, t2, ok2, note0)
+    add("cfg0 layer_norm", "1500x384", "f32", 2 * x.nbytes + g.nbytes + b.nbytes, t3, ok3, note0)
+    return rows
+
+
+def profile_targets(dev, seed, names, reps):
+    """For rocprofv3: launches each named target `reps` times back to back and nothing else, so that a kernel trace or a
+    counter run of this script shows those launches alone.  No events, no checks, no JSON line.
+      softmax_masked  rt_softmax_masked on causal [1,32,4096,4096] f16 scores + the [4096,4096] mask (config 3 as written)
+      softmax_causal  rt_softmax on the same scores with the mask already added (the step's launch, on its own)
+      softmax_dense   rt_softmax on dense N(0,2) scores of that shape (no -inf: the table lookups of a wave differ)
+      copy_1gib       the plain copy kernel on 1 GiB (the counters' calibration and the copy ceiling)
+      copy_reference  one plain copy per op of the step (half the op's algorithmic bytes read, half written, fresh regions
+                      of two 1 GiB buffers), then a 21 MB copy + 16-byte fill and a 2 MB copy + 16-byte fill: per repetition
+                      19 copy launches and 2 fills, in that order"""
+    from ratchet_amd import _lib
+
+    S, H = 4096, 32
+    head = normal(seed, 112, (S, S), 2.0, np.float16)          # stream 112: the score head of build_workload
+    mask = np.triu(np.full((S, S), -np.inf, np.float16), k=1)
+    d_head, d_mask = dev.upload(head), dev.upload(mask)
+    x = dev.empty((1, H, S, S), F16)
+    for h in range(H):
+        _lib.check(dev.lib.rt_d2d(dev.handle, x.ptr.value + h * head.nbytes, d_head.ptr, head.nbytes))
+    y = dev.empty((1, H, S, S), F16)
+    masked = None
+    for name in names:
+        if name == "softmax_masked":
+            fn = lambda: dev.softmax_masked(x, d_mask, out=y)
+        elif name == "softmax_dense":
+            fn = lambda: dev.softmax(x, out=y)
+        elif name == "softmax_causal":
+            if masked is None:
+                masked = dev.empty((1, H, S, S), F16)
+                dev.binary("add", x, d_mask, out=masked)
+            fn = lambda: dev.softmax(masked, out=y)
+        elif name == "copy_1gib":
+            fn = lambda: _lib.check(dev.lib.rt_cast(dev.handle, F16, F16, x.ptr, y.ptr, x.numel))
+        elif name == "copy_reference":
+            # the copy pass of the bench (one copy per op of the step, same bytes, back to back), without its events; behind
+            # it the boundary probes: a 16-byte fill behind a 21 MB copy and behind a 2 MB copy
+            import ctypes
+
+            tiny = dev.empty((4,), F32)
+            off = [0]
+
+            def copies():
+                for nbytes in STEP_ALG_BYTES + [20971520, 2097152]:
+                    half = min((nbytes // 2) & ~15, x.nbytes)
+                    if off[0] + half > x.nbytes:
+                        off[0] = 0
+                    _lib.check(dev.lib.rt_cast(dev.handle, F16, F16, ctypes.c_void_p(x.ptr.value + off[0]), ctypes.c_void_p(y.ptr.value + off[0]), half // 2))
+                    off[0] += half
+                    if nbytes in (20971520, 2097152):
+                        tiny.zero_()
+
+            fn = copies
+        else:
+            raise SystemExit("bench.py --profile: unknown target %r" % name)
+        for _ in range(reps):
+            fn()
+        dev.sync()
+        print("profiled", name, reps, flush=True)
+
+
 def download_rows(dev, buf, nrows, row_elems, np_dtype):
     """first nrows rows (row_elems each) of a device buffer"""
     import ctypes
@@ -558,6 +779,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline timing")
     ap.add_argument("--no-check", action="store_true", help="skip the parity check of the timed buffers")
     ap.add_argument("--no-patterns", action="store_true", help="skip the one-pass caller-pattern timings reported beside the step")
+    ap.add_argument("--no-rotate", action="store_true", help="skip the event-free per-op pass over rotating cold buffers (it allocates about 12 GB)")
+    ap.add_argument("--profile", type=str, default=None, help="comma-separated targets to launch alone under rocprofv3 (see profile_targets)")
+    ap.add_argument("--reps", type=int, default=6, help="launches per --profile target")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (every op is row/element parallel; there is no multi-GPU path). "
@@ -568,11 +792,17 @@ def main():
 
     seed = int(os.environ.get("RATCHET_SEED", "0"))
     dev = Device(0)
+    if args.profile:
+        profile_targets(dev, seed, args.profile.split(","), args.reps)
+        dev.close()
+        return
     t_setup = time.perf_counter()
     ops = build_workload(dev, seed)
     if args.ops:
         rx = re.compile(args.ops)
         ops = [o for o in ops if rx.search(f"cfg{o.cfg} {o.name}")]
+    elif [o.alg_bytes for o in ops] != STEP_ALG_BYTES:
+        raise SystemExit("bench.py: STEP_ALG_BYTES is out of step with build_workload")
     dev.sync()
     t_setup = time.perf_counter() - t_setup
 
@@ -585,7 +815,11 @@ def main():
 
     # per-op pass (not the timed region): HIP events around every launch, one synchronisation per step.  These give the
     # per-op table; the events and the per-step wait cost about 6 us per op, which is why `value` is not taken here.
+    # A 16-byte fill goes ahead of the first op of every step, so that it does not start on a queue the wait has drained
+    # (the first row would otherwise carry the cost of waking the queue, about 3 us, which no other row has).
+    tiny = dev.empty((4,), F32)
     for _ in range(args.steps):
+        tiny.zero_()
         for o, (e0, e1) in zip(ops, ev):
             e0.record()
             o.launch()
@@ -674,6 +908,12 @@ def main():
                 loop_t += check_and_time_cpu(dev, o, oracle, check=False)[1]
             oracle.set_reference_copies(True)
 
+    # the per-op figure that carries no events (after the parity check: the rotating sets are made from the same inputs)
+    no_events = {}
+    if not args.no_rotate:
+        for o in ops:
+            no_events[id(o)] = time_without_events(dev, o)
+    extras = extra_rows(dev, seed, oracle if not args.no_check else None) if not (args.ops or args.no_patterns) else None
     ceiling = copy_ceiling(dev) if not args.ops else None      # after the parity check: it overwrites an output buffer
     copy_us, boundary_us = copy_reference(dev, ops, args.steps) if not args.ops else ([None] * len(ops), None)
     patterns = one_pass_patterns(dev, seed, oracle if not args.no_check else None) if not (args.ops or args.no_patterns) else None
@@ -685,10 +925,17 @@ def main():
     pmc_rows = read_step_rows(PROFILE_HBM_TRAFFIC) if not args.ops else {}
 
     def kernel_us(pos):
+        """the kernel's own average duration at step position `pos` from the committed trace summary; None when the
+        summary is missing, when the row's kernel is not the one this op launches, or when the figure exceeds what the
+        events measured around the launch in this run (then the summary describes another build of the kernel)"""
         try:
-            return float(kt_rows[pos][2])
+            name, us = kt_rows[pos][1], float(kt_rows[pos][2])
         except (KeyError, IndexError, ValueError):
             return None
+        o = ops[pos - 1]
+        if not o.kernel or o.kernel not in name or us > float(np.median(o.us)):
+            return None
+        return us
 
     def traffic_bytes(pos):
         """fetch + write of the launch at step position `pos`, from the committed counter summary; None when the summary
@@ -711,6 +958,9 @@ def main():
                      "us": round(med, 2), "us_mean": round(float(np.mean(o.us)), 2), "GBps": round(gbps, 1),
                      "frac_hbm": round(gbps / PEAK_HBM_GBPS, 4),
                      # a plain copy kernel moving the same bytes, timed the same way in the same place of the step
+                     # launched back to back over rotating cold buffers, no events in between (one pair around `launches` of them)
+                     "us_no_events": None if id(o) not in no_events else round(no_events[id(o)][0], 2),
+                     "frac_hbm_no_events": None if id(o) not in no_events else round(o.alg_bytes / no_events[id(o)][0] / 1e3 / PEAK_HBM_GBPS, 4),
                      "copy_us": None if copy_us[pos - 1] is None else round(copy_us[pos - 1], 2),
                      "frac_of_copy": None if copy_us[pos - 1] is None else round(copy_us[pos - 1] / med, 4),
                      # the kernel alone (rocprofv3 --kernel-trace of this script, profiles/): `us` adds the two events and the launch gap
@@ -735,7 +985,10 @@ def main():
                      "avg_launch_us": round(dom_avg_us, 2), "algorithmic_bytes": dom.alg_bytes,
                      # FETCH_SIZE + WRITE_SIZE per launch, scaled by a 1 GiB copy kernel; null when the summary lacks the row
                      "traffic": traffic_bytes(ops.index(dom) + 1), "traffic_source": PROFILE_HBM_TRAFFIC,
-                     "kernel_us_source": PROFILE_KERNEL_TRACE},
+                     "kernel_us_source": PROFILE_KERNEL_TRACE,
+                     # the commit the two summaries were taken at (their `git_head:` line) and the commit of this run
+                     "profiles_git_head": {"kernel_trace": profile_head(PROFILE_KERNEL_TRACE), "hbm_traffic": profile_head(PROFILE_HBM_TRAFFIC)},
+                     "git_head": git_head()},
         "cpu_baseline": None if args.no_cpu or cpu_t == 0 else {
             "value": round(cpu_b / cpu_t / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": "every op of the step on one host core with the reference's to_vec/store copies, whole tensors "
@@ -746,6 +999,7 @@ def main():
         "hbm_copy_ceiling": ceiling,
         # a 16-byte fill launched right behind a 21 MB permute, HIP events around it: what one more kernel boundary costs
         "kernel_boundary_us": None if boundary_us is None else round(boundary_us, 2),
+        "extra_rows": extras,
         "one_pass_patterns": patterns,
         "decode_step": decode,
         "host_graph_step": host_step,

@@ -147,7 +147,12 @@ int rt_device_create(int ordinal, rt_device** out) {
         delete dev;
         return rt_fail_hip(e, "hipMalloc(scratch)");
     }
-    e = hipMalloc((void**)&dev->sm_row_sums, RT_SM_ROW_SUMS * sizeof(uint16_t));
+    e = hipMalloc((void**)&dev->sm_row_sums, RT_SM_ROW_SUMS * sizeof(uint16_t) + (RT_SM_TILES_HEAD + RT_SM_MASK_TILES) * sizeof(uint32_t));
+    if (e == hipSuccess) {
+        dev->sm_mask_tiles = reinterpret_cast<uint32_t*>(dev->sm_row_sums + RT_SM_ROW_SUMS);
+        e = hipMemset(dev->sm_mask_tiles, 0xff, RT_SM_TILES_HEAD * sizeof(uint32_t));
+        if (e != hipSuccess) (void)hipFree(dev->sm_row_sums);
+    }
     if (e != hipSuccess) {
         (void)hipFree(dev->gn_scratch);
         (void)hipStreamDestroy(dev->stream);

@@ -10,6 +10,8 @@
 #include "../../include/ratchet_hip_debug.h"
 
 constexpr size_t RT_SM_ROW_SUMS = 1u << 19;
+constexpr size_t RT_SM_MASK_TILES = 1u << 18;   // 512-column tiles of a mask that the streaming softmax can classify per launch
+constexpr size_t RT_SM_TILES_HEAD = 16;         // entries in front of them that always read "load this tile"
 
 struct rt_device {
     int ordinal;
@@ -32,8 +34,13 @@ struct rt_device {
     unsigned np_attr_set;   // 16-bit norm instantiations (LDS-resident rows) whose dynamic-LDS limit has been raised on this device
     uint64_t sp_attr_set;   // streaming softmax instantiations whose dynamic-LDS limit has been raised on this device
     uint64_t sp_ragged_attr_set;   // the same for the ragged-row variants
+    uint32_t sp_pair_attr_set;     // the same for the variants that take one mask row for two heads
     // row sums of one launch of the streaming softmax's ragged-row variant (RT_SM_ROW_SUMS 16-bit values, allocated with the device)
     uint16_t* sm_row_sums;
+    // one word per 512-column tile of the mask of a masked streaming softmax (behind the row sums, in the same allocation): the
+    // tile's value twice when all its elements are equal, 0xffffffff when the tile has to be loaded; the first RT_SM_TILES_HEAD
+    // words always hold 0xffffffff
+    uint32_t* sm_mask_tiles;
     // caching allocator behind rt_malloc / rt_free (defined in rt_device.hip)
     struct rt_pool* pool;
     int capturing;          // between rt_capture_begin and rt_capture_end

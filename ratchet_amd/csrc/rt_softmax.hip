@@ -25,7 +25,16 @@ template <typename T> __device__ __forceinline__ float stable_exp(float v) { ret
 // that product, half an ulp of |v| * 1.44, is the error: 3.3e-7 relative for |v| < 11, 6.6e-7 below 22, 2.6e-6 at the
 // overflow threshold (bar: 1e-5).  -inf gives 0, +inf and anything from 88.73 up give inf, NaN stays NaN, as with expf;
 // the library expf costs about four times the instructions, which at 27 M elements is most of the memory time.
-__device__ __forceinline__ float ref_exp_f32(float v) { return __builtin_amdgcn_exp2f(v * 1.44269504088896341f); }
+// v_exp_f32 returns 0 where the result would be subnormal (v below about -87.3), where expf and the reference's CPU code
+// return the subnormal: a row whose entries all lie there would sum to 0 and come out as 0 / 0.  Below 2^-126 the
+// exponent is therefore raised by 64 before the instruction and the result scaled back by 2^-64, which is exact but for
+// the one rounding into the subnormal grid that expf has too.
+__device__ __forceinline__ float ref_exp_f32(float v) {
+    const float p = v * 1.44269504088896341f;
+    const bool tiny = p < -126.0f;
+    const float e = __builtin_amdgcn_exp2f(p + (tiny ? 64.0f : 0.0f));
+    return e * (tiny ? 0x1p-64f : 1.0f);
+}
 
 constexpr int WIDE_BLOCK = 1024;                        // threads per row for rows that do not fit 256 threads' registers
 

@@ -127,12 +127,14 @@ struct SpSched {
     FastDiv gp_div;
     FastDiv pm_div;          // rows of the mask: row (rep * P + r) of x takes mask row (rep * P + r) % PM.  PM == P unless the
     uint32_t PM;             // mask is only a few rows tall, where groups that stop at every period would be nearly empty
+    uint32_t tile_stride;    // words per mask row in the table of tile classes (the steps of a row); 0: no table, every tile is loaded
+    uint32_t item_reps;      // periods in units of items: reps, or ceil(reps / 2) when a loader wave's two rows are one row of two periods
     uint32_t pace;           // shortest time between two steps of a block, in ticks of the device's wall clock (100 MHz); 0: unpaced
     uint32_t phase_fx;       // pace / grid in 16.16 fixed point: block b takes its steps b * pace / grid ticks after block 0
 };
 
 __device__ __forceinline__ uint32_t sp_item_count(const SpSched& s, uint32_t b, uint32_t G) {
-    const uint32_t total = s.GP * s.reps;
+    const uint32_t total = s.GP * s.item_reps;
     return b < total ? (total - b + G - 1) / G : 0;
 }
 __device__ __forceinline__ void sp_item(const SpSched& s, uint32_t b, uint32_t G, uint32_t it, uint32_t& rep, uint32_t& pg) {
@@ -159,6 +161,7 @@ template <> struct SpType<half_t> {
     }
     static constexpr bool SHORT_DIVISION = true;
     static constexpr bool CHUNK_ASM = false;                                      // the walker adds pair by pair
+    static constexpr uint32_t NEG_INF_PAIR = 0xfc00fc00u;                         // two -inf
 };
 template <> struct SpType<bf16_t> {
     typedef float Run;                                                            // always a bf16 value, held widened
@@ -203,6 +206,7 @@ template <> struct SpType<bf16_t> {
             r[w] = cvt_pk(u2f(a[w] << 16) + u2f(b[w] << 16), u2f(a[w] & 0xffff0000u) + u2f(b[w] & 0xffff0000u));
         return r;
     }
+    static constexpr uint32_t NEG_INF_PAIR = 0xff80ff80u;
     static constexpr bool SHORT_DIVISION = false;                                 // the quotient's range is f32's: always the IEEE division
     static constexpr bool CHUNK_ASM = true;                                       // the walker adds sixteen values per asm statement (add_chunk)
 };
@@ -219,16 +223,21 @@ template <> struct SpType<bf16_t> {
 // finished by softmax16_edges_kernel from x, the table and that sum.  An aligned vector that holds one byte of the tensor
 // lies in a mapped page, so the loads are safe at the tensor's ends too.  A row's span can be one vector longer than
 // NSTEP steps hold (2047 columns starting 14 bytes into a vector): wave 0 reads that vector itself and adds it last.
-template <typename T, int NSTEP, bool FULL, bool MASK, bool RAGGED = false>
+template <typename T, int NSTEP, bool FULL, int MASK, bool RAGGED = false>
 __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16_t* __restrict__ table, const T* x, const T* mask, T* y,
-                                                                    uint64_t rows, uint32_t cols, SpSched sch, uint16_t* row_sums) {
+                                                                    uint64_t rows, uint32_t cols, SpSched sch, uint16_t* row_sums,
+                                                                    const uint32_t* __restrict__ tiles) {
     typedef SpType<T> ST;
     constexpr bool PARK = NSTEP > 0;
     // Only the plain variant holds its steps to a pace (see launch_stream16).  The masked and ragged variants take longer
     // per step than the pace by themselves, and the mere presence of the pacing code changed their register allocation
     // and cost the masked one 6 % (390 -> 416 us), so for them it is compiled out.
     constexpr bool PACED = !MASK && !RAGGED;
+    // MASK == 2: the two rows of a loader wave are the same row of two neighbouring periods (two heads under one [S, T]
+    // mask), so one mask vector serves both and the register of the second holds the mask of the step after next
+    constexpr bool PAIR = MASK == 2;
     static_assert(!RAGGED || (PARK && !FULL), "the ragged variant parks in registers and has no full-step shortcut");
+    static_assert(!PAIR || (PARK && !RAGGED && NSTEP % 2 == 0), "the paired variant parks in registers and alternates two mask slots");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     uint16_t* lut = reinterpret_cast<uint16_t*>(smem);
     uint16_t (*tile)[SP_TC + SP_PAD] = reinterpret_cast<uint16_t (*)[SP_TC + SP_PAD]>(smem + SP_LUT_BYTES);
@@ -359,15 +368,37 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
     // (RAGGED: xo is the offset of the row's first span vector and mdiff carries sh, the row's start inside that vector)
     // (RAGGED with MASK: mq is the mask byte that lines up with the row's span origin, mask row offset minus sh; it is only
     // element aligned, and negative for the mask's first row when sh > 0)
+    // With a mask, register-parked rows of whole vectors: the classes of the NSTEP tiles of each of the wave's mask rows
+    // (one row when paired), in scalar registers (see mask_tiles_kernel)
+    constexpr bool TILES = MASK && PARK && !RAGGED;
+    constexpr int NCLS = TILES ? NSTEP : 1, NCROW = PAIR ? 1 : 2;
+    auto item_tiles = [&](uint32_t it, uint32_t (&cw)[NCROW][NCLS]) {
+        if constexpr (TILES) {
+            uint32_t rep, pg;
+            sp_item(sch, blockIdx.x, G, it, rep, pg);
+#pragma unroll
+            for (int h = 0; h < NCROW; h++) {
+                const uint32_t r = PAIR ? rr : rr + h * SP_HALF;
+                const uint32_t prow = pg * sch.R + r;
+                const bool ok = it < n_items && r < sch.R && prow < sch.P && sch.tile_stride != 0;
+                uint32_t q, mrow;
+                fd_divmod((PAIR ? rep * 2 : rep) * sch.P + prow, sch.pm_div, q, mrow);
+                const uint32_t base = __builtin_amdgcn_readfirstlane(ok ? (uint32_t)RT_SM_TILES_HEAD + mrow * sch.tile_stride : 0u);
+#pragma unroll
+                for (int t = 0; t < NCLS; t++) cw[h][t] = __builtin_amdgcn_readfirstlane(tiles[base + t]);
+            }
+        }
+    };
     auto item_off = [&](uint32_t it, uint32_t (&xo)[2], uint32_t (&mdiff)[2], uint32_t (&mq)[2]) {
         uint32_t rep, pg;
         sp_item(sch, blockIdx.x, G, it, rep, pg);
 #pragma unroll
         for (int h = 0; h < 2; h++) {
-            const uint32_t r = rr + h * SP_HALF;
+            const uint32_t r = PAIR ? rr : rr + h * SP_HALF;
             const uint32_t prow = pg * sch.R + r;            // row inside the period
-            const bool ok = it < n_items && r < sch.R && prow < sch.P;
-            const uint32_t row = rep * sch.P + prow;
+            const uint32_t per = PAIR ? rep * 2 + h : rep;
+            const bool ok = it < n_items && r < sch.R && prow < sch.P && per < sch.reps;
+            const uint32_t row = per * sch.P + prow;
             mq[h] = 0;
             if (RAGGED) {
                 xo[h] = __builtin_amdgcn_readfirstlane(ok ? (row * row_bytes) & ~15u : OOB);
@@ -442,6 +473,18 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
     };
     auto load_x = [&](uint32_t off) -> v4u { return __builtin_amdgcn_raw_buffer_load_b128(rx, off, 0, 2); };   // 2: non-temporal
     auto load_m = [&](uint32_t off) -> v4u { return __builtin_amdgcn_raw_buffer_load_b128(rm, off, 0, 0); };   // re-read by other heads
+    // A mask tile whose elements are all equal is not loaded (the offset goes outside the buffer, which costs no memory
+    // access and returns zeros) and its value is put in place of those zeros when the vector is used; cw is the tile's
+    // class word
+    constexpr uint32_t TILE_MIXED = 0xffffffffu;
+    auto load_m_tile = [&](uint32_t off, uint32_t cw) -> v4u {
+        const uint32_t skip = __builtin_amdgcn_readfirstlane(cw != TILE_MIXED ? OOB : 0u);
+        return load_m(off | skip);
+    };
+    auto tile_value = [&](const v4u& loaded, uint32_t cw) -> v4u {
+        const uint32_t fill = __builtin_amdgcn_readfirstlane(cw != TILE_MIXED ? cw : 0u);
+        return v4u{loaded[0] | fill, loaded[1] | fill, loaded[2] | fill, loaded[3] | fill};
+    };
     auto load_y = [&](uint32_t off) -> v4u { return __builtin_amdgcn_raw_buffer_load_b128(ry, off, 0, 0); };
     auto store_y = [&](const v4u& v, uint32_t off) { __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, 2); };      // results: non-temporal
     auto store_park = [&](const v4u& v, uint32_t off) { __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, 0); };   // read back soon
@@ -488,10 +531,18 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
     };
     // exp of the vector that arrived, in place (zeros past the row end: adding +0 is a no-op; rows past the tensor's end
     // read zeros and their sums are never used)
+    // A wave whose 512 values of this step are all -inf (the part of a row that a causal mask covers) takes exp(-inf) for
+    // all of them without the eight table reads per lane; the test is wave-wide, so the branch is a scalar one.
+    const uint32_t exp_ninf = __builtin_amdgcn_readfirstlane((uint32_t)lut[ST::NEG_INF_PAIR & 0xffffu] * 0x10001u);
     auto exp_in_place = [&](v4u& in, const v4u& m, uint32_t t, uint32_t sh) {
         if (MASK) in = ST::add_vec(in, m);                   // scores + mask in the 16-bit type, as the separate add would round it
+        const bool mine = ((in[0] ^ ST::NEG_INF_PAIR) | (in[1] ^ ST::NEG_INF_PAIR) | (in[2] ^ ST::NEG_INF_PAIR) | (in[3] ^ ST::NEG_INF_PAIR)) == 0;
+        if (__builtin_amdgcn_ballot_w64(!mine) == 0) {
+            in = v4u{exp_ninf, exp_ninf, exp_ninf, exp_ninf};
+        } else {
 #pragma unroll
-        for (int w = 0; w < 4; w++) in[w] = sp_exp_pair(lut, in[w]);
+            for (int w = 0; w < 4; w++) in[w] = sp_exp_pair(lut, in[w]);
+        }
         if (RAGGED ? t * (SP_TC * 2) + cbyte >= sh + row_bytes : past_end(t)) in = v4u{0, 0, 0, 0};
     };
     // RAGGED: the neighbours' elements in a row's first and last vector are zeroed in the tile, after the vector has been
@@ -522,8 +573,11 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
     };
 
     uint32_t cur[2], nxt[2], prev[2] = {OOB, OOB}, pcur[2], pnxt[2], pprev[2] = {0, 0}, mcur[2], mnxt[2];
+    uint32_t ccur[NCROW][NCLS], cnxt[NCROW][NCLS];
     item_off(0, cur, pcur, mcur);
     item_off(1, nxt, pnxt, mnxt);
+    item_tiles(0, ccur);
+    item_tiles(1, cnxt);
     uint32_t gpar = 0;
 
     if constexpr (PARK) {
@@ -545,9 +599,11 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
 #pragma unroll
             for (int h = 0; h < 2; h++) store_y(v4u{0, 0, 0, 0}, OOB);
         }
-        if (MASK && !RAGGED) {
+        if (MASK && !RAGGED) {                               // PAIR: the mask of steps 0 and 1 (NSTEP is even, so 1 exists)
 #pragma unroll
-            for (int h = 0; h < 2; h++) mpre[h] = load_m(step_off(cur[h] - pcur[h], 0));
+            for (int h = 0; h < 2; h++)
+                mpre[h] = PAIR ? load_m_tile(step_off(cur[0] - pcur[0], h), ccur[0][TILES ? h : 0])
+                               : load_m_tile(step_off(cur[h] - pcur[h], 0), ccur[PAIR ? 0 : h][0]);
         }
         if (MASK && RAGGED) {
 #pragma unroll
@@ -562,7 +618,12 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
             for (int t = 0; t < NSTEP; t++) {
 #pragma unroll
                 for (int h = 0; h < 2; h++)
-                    exp_in_place(pre[t % PF][h], (MASK && RAGGED) ? mask_funnel(mpre[h], mhi[h], mcur[h]) : mpre[h], t, pcur[h]);
+                    exp_in_place(pre[t % PF][h],
+                                 (MASK && RAGGED) ? mask_funnel(mpre[h], mhi[h], mcur[h])
+                                 : PAIR           ? tile_value(mpre[t % 2], ccur[0][TILES ? t : 0])
+                                 : TILES          ? tile_value(mpre[h], ccur[PAIR ? 0 : h][TILES ? t : 0])
+                                                  : mpre[h],
+                                 t, pcur[h]);
                 __syncthreads();                             // A: wave 0 has left the previous tile
                 *reinterpret_cast<v4u*>(&tile[rr][ccol]) = pre[t % PF][0];
                 *reinterpret_cast<v4u*>(&tile[rr + SP_HALF][ccol]) = pre[t % PF][1];
@@ -573,11 +634,15 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                 // the registers are free again: next loads, PF steps ahead, possibly in the block's next group
                 // (loads return in order: the mask of the next step goes first, so that waiting for it does not wait for x
                 // of the step after)
-                if (MASK && !RAGGED) {
+                if (MASK && !RAGGED && !PAIR) {
 #pragma unroll
                     for (int h = 0; h < 2; h++)
-                        mpre[h] = (t + 1 < NSTEP) ? load_m(step_off(cur[h] - pcur[h], t + 1)) : load_m(step_off(nxt[h] - pnxt[h], 0));
+                        mpre[h] = (t + 1 < NSTEP) ? load_m_tile(step_off(cur[h] - pcur[h], t + 1), ccur[PAIR ? 0 : h][TILES && t + 1 < NSTEP ? t + 1 : 0])
+                                                  : load_m_tile(step_off(nxt[h] - pnxt[h], 0), cnxt[PAIR ? 0 : h][0]);
                 }
+                if (PAIR)                                    // this step's slot is free: the mask of two steps ahead
+                    mpre[t % 2] = (t + 2 < NSTEP) ? load_m_tile(step_off(cur[0] - pcur[0], t + 2), ccur[0][PAIR && t + 2 < NSTEP ? t + 2 : 0])
+                                                  : load_m_tile(step_off(nxt[0] - pnxt[0], t + 2 - NSTEP), cnxt[0][PAIR && t + 2 >= NSTEP ? t + 2 - NSTEP : 0]);
                 if (MASK && RAGGED) {
 #pragma unroll
                     for (int h = 0; h < 2; h++) {
@@ -609,6 +674,11 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                 mcur[h] = mnxt[h];
             }
             item_off(it + 2, nxt, pnxt, mnxt);
+#pragma unroll
+            for (int h = 0; h < NCROW; h++)
+#pragma unroll
+                for (int t = 0; t < NCLS; t++) ccur[h][t] = cnxt[h][t];
+            item_tiles(it + 2, cnxt);
             gpar ^= 1;
         }
         // drain: outputs of the block's last group
@@ -729,6 +799,41 @@ __global__ void __launch_bounds__(BLOCK) softmax16_edges_kernel(const uint16_t* 
     y[at] = Ar<T>::div(ev, __builtin_bit_cast(T, row_sums[row]));
 }
 
+// The class of every 512-column tile of a mask, for the masked variants of the streaming kernel that park in registers:
+// a tile whose elements all have the same bits v gets the word v | v << 16 (what the kernel puts in place of the loads it
+// then leaves out: under a causal mask seven tiles of eight hold nothing but 0 or nothing but -inf), any other tile, and
+// a tile of 0xffff, gets 0xffffffff.  cols % 8 == 0; a row's last tile may be short.  A wave takes MT_PER_WAVE tiles with
+// all their loads in flight at once.
+constexpr int MT_PER_WAVE = 8;
+template <typename T>
+__global__ void __launch_bounds__(BLOCK) mask_tiles_kernel(const T* __restrict__ mask, uint32_t mask_rows, uint32_t cols, uint32_t nt,
+                                                           uint32_t* __restrict__ tiles) {
+    const uint32_t wave = blockIdx.x * (BLOCK / 64) + threadIdx.x / 64;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t ntiles = mask_rows * nt;
+    const uint16_t* m16 = reinterpret_cast<const uint16_t*>(mask);
+    v4u v[MT_PER_WAVE];
+    bool have[MT_PER_WAVE];
+#pragma unroll
+    for (int k = 0; k < MT_PER_WAVE; k++) {
+        const uint32_t tile = wave * MT_PER_WAVE + k;
+        const uint32_t row = tile / nt, t = tile - row * nt;
+        const uint32_t col = t * SP_TC + lane * 8;
+        have[k] = tile < ntiles && col < cols;
+        v[k] = v4u{0, 0, 0, 0};
+        if (have[k]) v[k] = *reinterpret_cast<const v4u*>(m16 + (uint64_t)row * cols + col);
+    }
+#pragma unroll
+    for (int k = 0; k < MT_PER_WAVE; k++) {
+        const uint32_t tile = wave * MT_PER_WAVE + k;
+        if (tile >= ntiles) break;                           // the same for the whole wave
+        const uint32_t first = (__builtin_amdgcn_readfirstlane(v[k][0]) & 0xffffu) * 0x10001u;     // lane 0 holds the tile's first element
+        const bool same = !have[k] || ((v[k][0] ^ first) | (v[k][1] ^ first) | (v[k][2] ^ first) | (v[k][3] ^ first)) == 0;
+        const bool uniform = __builtin_amdgcn_ballot_w64(!same) == 0 && first != 0xffffffffu;
+        if (lane == 0) tiles[RT_SM_TILES_HEAD + tile] = uniform ? first : 0xffffffffu;
+    }
+}
+
 // mask == nullptr: plain softmax.  Otherwise the mask has `period` rows of `cols` columns and repeats every `period`
 // rows of x (rows % period == 0).  Returns RT_OK with *done = false when the shape does not fit this kernel.
 template <typename T>
@@ -774,7 +879,25 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
             dev->sp_attr_set |= bit;                                                                                                 \
         }                                                                                                                            \
         hipLaunchKernelGGL((softmax16_stream_kernel<T, NS, F, M>), dim3(blocks), dim3(SP_BLOCK), SP_SMEM_BYTES, dev->stream, table,  \
-                           xc, (const T*)mask, yc, n, cols, sch, (uint16_t*)nullptr);                                                \
+                           xc, (const T*)mask, yc, n, cols, sch, (uint16_t*)nullptr, (const uint32_t*)dev->sm_mask_tiles);          \
+    } while (0)
+#define RT_SP_PAIR(NS, F)                                                                                                            \
+    do {                                                                                                                             \
+        const uint32_t bit = 1u << (TI * 8 + (NS / 2 - 1) * 2 + (F ? 1 : 0));                                                        \
+        if (!(dev->sp_pair_attr_set & bit)) {                                                                                        \
+            RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(softmax16_stream_kernel<T, NS, F, 2>),                          \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)SP_SMEM_BYTES));                             \
+            dev->sp_pair_attr_set |= bit;                                                                                            \
+        }                                                                                                                            \
+        hipLaunchKernelGGL((softmax16_stream_kernel<T, NS, F, 2>), dim3(blocks), dim3(SP_BLOCK), SP_SMEM_BYTES, dev->stream, table,  \
+                           xc, (const T*)mask, yc, n, cols, sch, (uint16_t*)nullptr, (const uint32_t*)dev->sm_mask_tiles);          \
+    } while (0)
+#define RT_SP_PAIR_NS(F)                                    \
+    do {                                                    \
+        if (nt <= 2) RT_SP_PAIR(2, F);                      \
+        else if (nt <= 4) RT_SP_PAIR(4, F);                 \
+        else if (nt <= 6) RT_SP_PAIR(6, F);                 \
+        else RT_SP_PAIR(8, F);                              \
     } while (0)
 #define RT_SP_RAGGED(NS, M)                                                                                                          \
     do {                                                                                                                             \
@@ -785,7 +908,7 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
             dev->sp_ragged_attr_set |= bit;                                                                                              \
         }                                                                                                                            \
         hipLaunchKernelGGL((softmax16_stream_kernel<T, NS, false, M, true>), dim3(blocks), dim3(SP_BLOCK), SP_SMEM_BYTES,            \
-                           dev->stream, table, xc, (const T*)mask, yc, n, cols, sch, dev->sm_row_sums);                              \
+                           dev->stream, table, xc, (const T*)mask, yc, n, cols, sch, dev->sm_row_sums, (const uint32_t*)nullptr);                              \
     } while (0)
 #define RT_SP_RAGGED_NS(M)                                  \
     do {                                                    \
@@ -818,6 +941,10 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
         sch.P = (uint32_t)(mask && period >= 8 * SP_ROWS ? period : n);
         sch.reps = (uint32_t)(n / sch.P);
         sch.nsteps = (nt + 1) & ~1u;
+        // one mask row for two heads: rows of an even number of steps under a mask that repeats every P rows
+        const bool pair = mask && !ragged && nt <= SP_MAX_STEPS && (nt % 2 == 0 || nt == 7) && sch.PM == sch.P && sch.reps >= 2;
+        sch.item_reps = pair ? (sch.reps + 1) / 2 : sch.reps;
+        const uint32_t rmax = pair ? SP_HALF : SP_ROWS, rmul = pair ? 2 : 1;
         // rows per group: every block runs ceil(groups / grid) rounds of 8-or-fewer steps whatever the group holds, so
         // 4370 groups of 30 rows on 256 CUs cost 18 rounds where 17.07 are needed; 27-row groups make 19 full rounds.
         // A step takes the longer of the walk (1.5 us whatever the group holds) and the group's memory time (2 KiB per
@@ -831,20 +958,20 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
         // the cheapest size by the count alone, 26 rows and 158 groups, 224 us; 114 against 121 us on [1,32,2048,2048]).
         {
             auto cost_of = [&](uint32_t R) -> uint64_t {
-                const uint64_t groups = (uint64_t)((sch.P + R - 1) / R) * sch.reps;
+                const uint64_t groups = (uint64_t)((sch.P + R - 1) / R) * sch.item_reps;
                 const uint64_t rounds = (groups + dev->num_cus - 1) / dev->num_cus;
-                return rounds * (R + 1 > 18 ? R + 1 : 18);
+                return rounds * (R * rmul + 1 > 18 ? R * rmul + 1 : 18);
             };
             uint64_t best = ~0ull;
-            sch.R = SP_ROWS;
-            for (uint32_t R = SP_ROWS; R >= 1; R--) {
+            sch.R = rmax;
+            for (uint32_t R = rmax; R >= 1; R--) {
                 const uint64_t cost = cost_of(R);
                 if (cost <= best) {
                     best = cost;
                     sch.R = R;
                 }
             }
-            if (mask && sch.reps > 1) {
+            if (mask && sch.reps > 1 && !pair) {
                 auto xcds_of = [&](uint32_t R) -> uint32_t {
                     const uint32_t g = ((sch.P + R - 1) / R) % 8;
                     return g == 0 ? 1 : (g % 4 == 0) ? 2 : (g % 2 == 0) ? 4 : 8;
@@ -867,7 +994,7 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
         sch.GP = (sch.P + sch.R - 1) / sch.R;
         sch.pace = sch.phase_fx = 0;                         // set below, once the grid is known
         sch.gp_div = make_fastdiv(sch.GP);
-        const uint64_t items = (uint64_t)sch.GP * sch.reps;
+        const uint64_t items = (uint64_t)sch.GP * sch.item_reps;
         RT_REQUIRE(items <= 0xffffffffull, RT_ERR_SIZE, "rt_softmax: too many row groups");
         const unsigned blocks = (unsigned)(items < (uint64_t)dev->num_cus ? items : (uint64_t)dev->num_cus);   // one resident block per CU
         // Pacing.  Left to itself the kernel offers HBM more requests than it sustains, and what it then gets is less than
@@ -880,11 +1007,21 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
         // fills the chip is paced.
         if (blocks == dev->num_cus && !mask && !ragged) {
             const double rate = SP_PACE_BYTES_PER_S;
-            const double group_bytes = (double)sch.R * cols * 2 * (nt > SP_MAX_STEPS ? 4 : 2);     // in and out (long rows: parked and read back)
+            const double group_bytes = (double)sch.R * rmul * cols * 2 * (nt > SP_MAX_STEPS ? 4 : 2);     // in and out (long rows: parked and read back)
             const double steps = nt > SP_MAX_STEPS ? sch.nsteps : nt == 7 ? 8 : nt;          // the steps the kernel variant takes per group
             sch.pace = (uint32_t)(group_bytes / steps * blocks / rate * dev->wall_clock_hz + 0.5);
             if (dev->debug_softmax_pace) sch.pace = dev->debug_softmax_pace;
             sch.phase_fx = sch.pace > 0xffffu ? 0 : (sch.pace << 16) / blocks;
+        }
+        // the classes of the mask's tiles, for the variants that use them (a table of at most RT_SM_MASK_TILES words)
+        sch.tile_stride = 0;
+        if (mask && !ragged && nt <= SP_MAX_STEPS && (uint64_t)sch.PM * nt <= RT_SM_MASK_TILES && rt_aligned(mask, 16)) {
+            const uint32_t ntiles = sch.PM * nt;
+            const uint32_t per_block = (BLOCK / 64) * MT_PER_WAVE;
+            hipLaunchKernelGGL((mask_tiles_kernel<T>), dim3((ntiles + per_block - 1) / per_block), dim3(BLOCK), 0, dev->stream, (const T*)mask,
+                               sch.PM, cols, nt, dev->sm_mask_tiles);
+            RT_CHECK_LAUNCH("mask_tiles_kernel");
+            sch.tile_stride = nt;
         }
         if (ragged) {
             if (mask) RT_SP_RAGGED_NS(true);
@@ -899,6 +1036,9 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
         if (nt > SP_MAX_STEPS) {                         // long rows: exp values parked in y
             if (mask) RT_SP(0, false, true);
             else RT_SP(0, false, false);
+        } else if (pair) {
+            if (full) RT_SP_PAIR_NS(true);
+            else RT_SP_PAIR_NS(false);
         } else if (mask) {
             if (full) RT_SP_NS(true, true);
             else RT_SP_NS(false, true);
@@ -909,6 +1049,8 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
         RT_CHECK_LAUNCH("softmax16_stream_kernel");
     }
 #undef RT_SP_NS
+#undef RT_SP_PAIR_NS
+#undef RT_SP_PAIR
 #undef RT_SP_RAGGED_NS
 #undef RT_SP_RAGGED
 #undef RT_SP

@@ -97,6 +97,36 @@ def test_softmax_f32_masks_overflow_in_place(dev, oracle):
     assert np.isnan(got[2, 0]) and np.all(got[2, 1:] == 0) and np.all(np.isnan(got[3]))
 
 
+@pytest.mark.parametrize("cols", [64, 1500, 3000, 5001])
+def test_softmax_f32_rows_whose_exponentials_are_subnormal(dev, oracle, cols):
+    """known answers: every entry of a row at -95 (or -100) has a subnormal exponential, the row sums to a subnormal or tiny
+    normal number and every probability is 1 / cols, as expf gives it on the CPU; an exp that flushes subnormals to zero
+    returns 0 / 0 = NaN here.  Mixed rows around the threshold (-87.34) are compared with the oracle."""
+    x = np.empty((6, cols), np.float32)
+    x[0], x[1] = -95.0, -100.0
+    rng = np.random.default_rng(cols)
+    x[2] = -87.0 - 3.0 * rng.random(cols, dtype=np.float32)            # straddles the first subnormal result
+    x[3] = -95.0 - 5.0 * rng.random(cols, dtype=np.float32)            # all subnormal: 3930 down to 26 units of 2^-149
+    x[4] = -103.0 - 2.0 * rng.random(cols, dtype=np.float32)           # some round to zero
+    x[5] = -95.0
+    x[5, 0] = -90.0
+    want = oracle.softmax(x)
+    assert np.isfinite(want[:4]).all() and abs(want[0, 0] * cols - 1.0) < 1e-5
+    got = dev.softmax(dev.upload(x)).to_numpy()
+    assert np.isfinite(got[:4]).all() and np.isfinite(got[5]).all()
+    # the subnormal grid is coarse: an exponential of a few units of 2^-149 carries a relative error of its own, in the
+    # oracle and in the kernel alike, so rows 3 and 4 are held to the spacing of that grid instead of 1e-5
+    bad, mx = oracle.count_not_close(got[[0, 1, 2, 5]], want[[0, 1, 2, 5]], 1e-5, 1e-5)
+    assert bad == 0, (cols, bad, mx)
+    assert np.allclose(got[0], 1.0 / cols, rtol=1e-5) and np.allclose(got[1], 1.0 / cols, rtol=1e-5)
+    with np.errstate(all="ignore"):
+        e3 = np.exp(x[3].astype(np.float64))
+        ref3 = e3 / e3.sum()
+    assert np.max(np.abs(got[3] - ref3) / ref3) < 0.05                 # half a unit of 2^-149 against values of 26 and more
+    both_nan = np.isnan(got[4]) & np.isnan(want[4])
+    assert (np.isfinite(got[4]) | both_nan).all()
+
+
 @pytest.mark.parametrize("shape", [(3, 64, 256), (1, 7, 33), (2, 1, 1), (1, 70, 1000), (1, 65, 4096), (1, 3, 4100), (1, 129, 8)])
 def test_softmax_f16_reference_sequence(dev, oracle, shape):
     rng = np.random.default_rng(301)
