@@ -646,8 +646,9 @@ def extra_rows(dev, seed, oracle):
 
 
 def profile_targets(dev, seed, names, reps):
-    """For rocprofv3: launches each named target `reps` times back to back and nothing else, so that a kernel trace or a
-    counter run of this script shows those launches alone.  No events, no checks, no JSON line.
+    """For rocprofv3: launches each named target back to back and nothing else, so that a kernel trace or a counter run of
+    this script shows those launches alone: a second of them to bring the clocks up, then the `reps` that a summary reads
+    (the last `reps` dispatches of the target's kernel).  No events, no checks, no JSON line.
       softmax_masked  rt_softmax_masked on causal [1,32,4096,4096] f16 scores + the [4096,4096] mask (config 3 as written)
       softmax_causal  rt_softmax on the same scores with the mask already added (the step's launch, on its own)
       softmax_dense   rt_softmax on dense N(0,2) scores of that shape (no -inf: the table lookups of a wave differ)
@@ -687,18 +688,19 @@ def profile_targets(dev, seed, names, reps):
             off = [0]
 
             def copies():
-                for nbytes in STEP_ALG_BYTES + [20971520, 2097152]:
+                for k, nbytes in enumerate(STEP_ALG_BYTES + [20971520, 2097152]):
                     half = min((nbytes // 2) & ~15, x.nbytes)
                     if off[0] + half > x.nbytes:
                         off[0] = 0
                     _lib.check(dev.lib.rt_cast(dev.handle, F16, F16, ctypes.c_void_p(x.ptr.value + off[0]), ctypes.c_void_p(y.ptr.value + off[0]), half // 2))
                     off[0] += half
-                    if nbytes in (20971520, 2097152):
+                    if k >= len(STEP_ALG_BYTES):             # the two probes
                         tiny.zero_()
 
             fn = copies
         else:
             raise SystemExit("bench.py --profile: unknown target %r" % name)
+        warm_up(dev, fn, 1.0)                                # clocks up before the launches a summary reads: the last `reps`
         for _ in range(reps):
             fn()
         dev.sync()

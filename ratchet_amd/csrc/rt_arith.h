@@ -51,10 +51,17 @@ template <> struct Ar<half_t> {
 template <> struct Ar<bf16_t> {
     typedef bf16_t T;
     static constexpr int BYTES = 2;
-    // (the chip's own conversion, `(__bf16)f` = v_cvt_pk_bf16_f32, gives the same bits in one instruction, but this
-    // compiler fails to select code for it in some kernels ("cannot select v2f32 = bitcast" in the f32-routed unary
-    // kernel) and the kernels that use this are bound by memory, not by these six instructions)
-    static __device__ __forceinline__ T conv(float f) { T r; r.b = f2bf(f); return r; }
+    // The chip's own conversion (round to nearest even, NaN quieted), one instruction, written as an instruction: through
+    // `(__bf16)f` this compiler fails to select code for it in some kernels ("cannot select v2f32 = bitcast" in the
+    // f32-routed unary kernel).  The second operand's half of the result is not used.  On the bit pattern the same
+    // rounding is six instructions, and the 16-bit norms spend four conversions on every element.
+    static __device__ __forceinline__ T conv(float f) {
+        uint32_t r;
+        asm("v_cvt_pk_bf16_f32 %0, %1, 0" : "=v"(r) : "v"(f));
+        T out;
+        out.b = (uint16_t)r;
+        return out;
+    }
     static __device__ __forceinline__ float widen(T a) { return bf2f(a.b); }
     static __device__ __forceinline__ T add(T a, T b) { return conv(widen(a) + widen(b)); }
     static __device__ __forceinline__ T sub(T a, T b) { return conv(widen(a) - widen(b)); }

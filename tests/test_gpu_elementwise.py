@@ -180,6 +180,15 @@ def test_cast(dev, oracle):
     assert np.array_equal(gb, oracle.cast(y, np.uint16, dst_bf16=True))
     back = dev.cast(dev.upload(gb, bf16=True), _lib.F32).to_numpy()
     assert same_bits(back, oracle.cast(gb, np.float32, src_bf16=True))
+    # f32 -> bf16 over random bit patterns (NaNs with payloads, infinities, subnormals) and around every tie: the kernels
+    # round with the chip's conversion instruction, the oracle on the bit pattern as half::bf16::from_f32 does
+    hi = rng.integers(0, 2**16, size=200_000, dtype=np.uint64).astype(np.uint32) << 16
+    around = np.concatenate([hi | 0x7fff, hi | 0x8000, hi | 0x8001, hi | 0xffff, hi])
+    z = np.concatenate([rand.view(np.uint32), around]).view(np.float32)
+    gz = dev.cast(dev.upload(z), _lib.BF16).to_numpy()
+    wz = oracle.cast(z, np.uint16, dst_bf16=True)
+    bad = np.flatnonzero(gz != wz)
+    assert bad.size == 0, (bad.size, [hex(v) for v in z.view(np.uint32)[bad[:5]]], [hex(v) for v in gz[bad[:5]]], [hex(v) for v in wz[bad[:5]]])
     # f32 <-> i32/u32: bit reinterpretation, as the reference does (cpu/mod.rs:116-125)
     gi = dev.cast(dev.upload(y), _lib.I32).to_numpy()
     assert np.array_equal(gi, y.view(np.int32))
