@@ -35,6 +35,7 @@ struct rt_device {
     uint64_t sp_attr_set;   // streaming softmax instantiations whose dynamic-LDS limit has been raised on this device
     uint64_t sp_ragged_attr_set;   // the same for the ragged-row variants
     uint32_t sp_pair_attr_set;     // the same for the variants that take one mask row for two heads
+    uint16_t rp_resident[2][9];    // wave-per-row RMSNorm: blocks of an instantiation ([f16, bf16][vectors per lane]) that one CU holds; 0 = not asked yet
     // row sums of one launch of the streaming softmax's ragged-row variant (RT_SM_ROW_SUMS 16-bit values, allocated with the device)
     uint16_t* sm_row_sums;
     // one word per 512-column tile of the mask of a masked streaming softmax (behind the row sums, in the same allocation): the

@@ -838,6 +838,269 @@ __global__ void __launch_bounds__(BLOCK) norm16_lane_kernel(const T* x, const T*
     for (uint32_t i = threadIdx.x; i < nvec; i += BLOCK) st_stream(yb + i, stage[(i / NV) * (NV + 1) + i % NV]);
 }
 
+// ------------------------------------------------------------------------------------------------------------------
+// RMSNorm in the 16-bit types, one wave per row, with the reference's row sum replayed exactly but not sequentially.
+//
+// The reference adds T(x*x) left to right in f32 (cpu/norm.rs:72-89, half's Sum): s <- fl(s + a_j), a_j >= 0.  While s
+// stays inside one binade, [2^e, 2^(e+1)), s is 2^e + k * ulp with an integer k, and what one add does to k depends on s
+// only through the parity of k (round to nearest even: the parity decides ties).  A run of adds that stays inside the
+// binade is therefore a function k -> k + c[k & 1] of two constants, and such functions compose.  Both constants come
+// out of the floating-point adder itself: the run is added up twice, from 2^e and from 2^e + ulp, and c[p] is the
+// distance the p-th sum has moved, read off the bit patterns.
+//
+// Lane i of the wave owns the contiguous run of 8 * V elements i * 8V .. (the row is turned through LDS so that it does).
+//   1. approximate sums of the runs and their prefix over the lanes say in which binade each run starts and ends;
+//   2. a lane whose run starts and ends in one binade, with a margin for what the approximation can be off by, is
+//      `clean`: its two sums give its pair (c[0], c[1]);
+//   3. a segmented scan composes the pairs of neighbouring clean lanes;
+//   4. the lanes that are not clean (the first, those in which the sum crosses a power of two: about seven per row,
+//      and any lane the margins do not clear) are taken in order: the composed function of the clean stretch before
+//      such a lane is applied to the running value t, then every lane adds its own run to t left to right and the
+//      result of the lane in question is kept.
+// Nothing rests on the approximation: before a pair is applied, t must lie in the binade the pair was made for, and
+// the result must still lie in it; if either fails the row is done again with every lane treated as not clean, which
+// is the plain left-to-right sum, 64 runs one after the other.  bf16 takes the same path with widened operands.
+// ------------------------------------------------------------------------------------------------------------------
+constexpr int RP_BLOCK = 256;                                // four rows per block; the waves never meet
+template <typename T> struct RpChain;
+template <> struct RpChain<half_t> {
+    // a <- fl(a + h) and b <- fl(b + h) for the eight halves of a vector, left to right: 1.0 * widen(h) + sum in one
+    // instruction with one rounding
+#define RP_MIX2(N)                                                              \
+    "v_fma_mix_f32 %0, %" #N ", %6, %0 op_sel_hi:[1,0,0]\n"                      \
+    "v_fma_mix_f32 %1, %" #N ", %6, %1 op_sel_hi:[1,0,0]\n"                      \
+    "v_fma_mix_f32 %0, %" #N ", %6, %0 op_sel:[1,0,0] op_sel_hi:[1,0,0]\n"       \
+    "v_fma_mix_f32 %1, %" #N ", %6, %1 op_sel:[1,0,0] op_sel_hi:[1,0,0]\n"
+    static __device__ __forceinline__ void add2(float& a, float& b, const v4u& v) {
+        const float one = 1.0f;
+        asm(RP_MIX2(2) RP_MIX2(3) RP_MIX2(4) RP_MIX2(5) : "+v"(a), "+v"(b) : "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]), "s"(one));
+    }
+#undef RP_MIX2
+#define RP_MIX1(N)                                                              \
+    "v_fma_mix_f32 %0, %" #N ", %5, %0 op_sel_hi:[1,0,0]\n"                      \
+    "v_fma_mix_f32 %0, %" #N ", %5, %0 op_sel:[1,0,0] op_sel_hi:[1,0,0]\n"
+    static __device__ __forceinline__ void add1(float& a, const v4u& v) {
+        const float one = 1.0f;
+        asm(RP_MIX1(1) RP_MIX1(2) RP_MIX1(3) RP_MIX1(4) : "+v"(a) : "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]), "s"(one));
+    }
+#undef RP_MIX1
+    // the sum of the eight halves added to acc, in any order and with any rounding: only the binade is taken from it
+    // (v_dot2_f32_f16 with a pair of ones; written as instructions: through the builtin this compiler fed all four the
+    // vector's first word)
+    static __device__ __forceinline__ float rough(const v4u& v, float acc) {
+        const uint32_t ones = 0x3c003c00u;
+        asm("v_dot2_f32_f16 %0, %1, %5, %0\n"
+            "v_dot2_f32_f16 %0, %2, %5, %0\n"
+            "v_dot2_f32_f16 %0, %3, %5, %0\n"
+            "v_dot2_f32_f16 %0, %4, %5, %0\n"
+            : "+v"(acc)
+            : "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]), "v"(ones));
+        return acc;
+    }
+    static __device__ __forceinline__ v4u square(const v4u& x) {                 // T(x*x): eight f16 products, each rounded once
+        const np_h8 h = __builtin_bit_cast(np_h8, x);
+        return __builtin_bit_cast(v4u, h * h);
+    }
+};
+template <> struct RpChain<bf16_t> {
+    static __device__ __forceinline__ void add2(float& a, float& b, const v4u& v) {
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float lo = u2f(v[w] << 16), hi = u2f(v[w] & 0xffff0000u);
+            a += lo; b += lo; a += hi; b += hi;
+        }
+    }
+    static __device__ __forceinline__ void add1(float& a, const v4u& v) {
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            a += u2f(v[w] << 16);
+            a += u2f(v[w] & 0xffff0000u);
+        }
+    }
+    static __device__ __forceinline__ float rough(const v4u& v, float acc) {
+#pragma unroll
+        for (int w = 0; w < 4; w++) acc += u2f(v[w] << 16) + u2f(v[w] & 0xffff0000u);
+        return acc;
+    }
+    static __device__ __forceinline__ v4u square(const v4u& x) {
+        Vec16<bf16_t> in, out;
+        in.u = x;
+#pragma unroll
+        for (int q = 0; q < 8; q++) out.e[q] = Ar<bf16_t>::mul(in.e[q], in.e[q]);
+        return out.u;
+    }
+};
+
+template <typename T, int V>
+__global__ void __launch_bounds__(RP_BLOCK) rms16_par_kernel(const T* __restrict__ x, const T* __restrict__ scale, T* __restrict__ y, uint64_t rows,
+                                                             uint32_t cols, float eps) {
+    typedef RpChain<T> C;
+    extern __shared__ __attribute__((aligned(16))) v4u rp_lds[];             // [4 waves][V * 64] vectors of squares
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint64_t first = (uint64_t)blockIdx.x * (RP_BLOCK / 64) + wave, stride = (uint64_t)gridDim.x * (RP_BLOCK / 64);
+    if (first >= rows) return;                                               // a whole wave; the block never synchronises
+    v4u* mine = rp_lds + wave * (V * 64);
+    const uint32_t nvec = cols / 8;
+    // the row as it lies in memory: vector j * 64 + lane (zeros past its end: +0 terms change no sum).  A wave takes rows
+    // first, first + stride, ...; the loads of the next one are in flight while it works on this one (past the last
+    // row they fetch the last row once more, so that no branch stands between the loads and what waits for them)
+    auto fetch = [&](uint64_t r, v4u (&dst)[V]) {
+        const v4u* src = reinterpret_cast<const v4u*>(x + r * cols);
+#pragma unroll
+        for (int j = 0; j < V; j++) {
+            const uint32_t i = j * 64 + lane;
+            dst[j] = v4u{0, 0, 0, 0};
+            if (i < nvec) dst[j] = ld_stream(src + i);
+        }
+    };
+    v4u ahead[V];
+    fetch(first, ahead);
+    for (uint64_t row = first; row < rows; row += stride) {
+    v4u xr[V];
+#pragma unroll
+    for (int j = 0; j < V; j++) xr[j] = ahead[j];
+    fetch(row + stride < rows ? row + stride : rows - 1, ahead);
+    v4u* yrow = reinterpret_cast<v4u*>(y + row * cols);
+#pragma unroll
+    for (int j = 0; j < V; j++) mine[j * 64 + lane] = C::square(xr[j]);
+    // turned: lane i holds the run of vectors i * V .. i * V + V - 1.  The wave wrote them itself and LDS keeps a wave's
+    // order, but other lanes wrote what this lane reads: the fence keeps the compiler from moving a read above a write
+    // that, seen from one lane alone, goes to another address.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    v4u run[V];
+#pragma unroll
+    for (int v = 0; v < V; v++) run[v] = mine[lane * V + v];
+
+    // 1. approximate sum of the run, inclusive prefix over the lanes
+    float rough = 0.0f;
+#pragma unroll
+    for (int v = 0; v < V; v++) rough = C::rough(run[v], rough);
+    float upto = rough;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const float t = __shfl_up(upto, o, 64);
+        if (lane >= (uint32_t)o) upto += t;
+    }
+    float before = __shfl_up(upto, 1, 64);
+    if (lane == 0) before = 0.0f;
+    // 2. clean: the run starts and ends in the binade of `before`, even if both figures are off by 2^-10 of themselves
+    const uint32_t e = (f2u(before) >> 23) & 0xffu;
+    const uint32_t base = e << 23;                                           // bit pattern of 2^e
+    bool clean = lane != 0 && e >= 1 && e < 254 && ((f2u(before * (1.0f - 0x1p-10f)) >> 23) & 0xffu) == e &&
+                 ((f2u(upto * (1.0f + 0x1p-10f)) >> 23) & 0xffu) == e;
+    float s0 = u2f(base), s1 = u2f(base + 1);
+#pragma unroll
+    for (int v = 0; v < V; v++) C::add2(s0, s1, run[v]);
+    uint32_t c0 = f2u(s0) - base, c1 = f2u(s1) - (base + 1);
+    clean = clean && c0 < (1u << 23) && c1 + 1 < (1u << 23);                 // both sums stayed in the binade
+    // the pairs of a stretch of clean lanes are composed as counts of one and the same ulp: a clean lane behind a clean
+    // lane of another binade (which the margins make all but impossible) starts over as a lane that is not clean
+    {
+        const uint32_t pbase = __shfl_up(base, 1, 64);
+        const uint32_t pclean = __shfl_up((uint32_t)clean, 1, 64);
+        if (lane != 0 && pclean && pbase != base) clean = false;
+    }
+    if (!clean) c0 = c1 = 0;
+
+    // 3. segmented scan: (c0, c1) of lane i becomes the composition of the clean lanes from the start of its stretch up to
+    // i; a lane that is not clean, and the lane behind one, start a stretch.  left then right: p -> l[p] + r[(p + l[p]) & 1]
+    const uint64_t dirty_mask = __builtin_amdgcn_ballot_w64(!clean);
+    uint32_t head = (uint32_t)((dirty_mask >> lane) & 1u) | (lane ? (uint32_t)((dirty_mask >> (lane - 1)) & 1u) : 1u);
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const uint32_t l0 = __shfl_up(c0, o, 64), l1 = __shfl_up(c1, o, 64), lh = __shfl_up(head, o, 64);
+        if (lane >= (uint32_t)o && !head) {
+            const uint32_t n0 = l0 + ((l0 & 1u) ? c1 : c0);
+            const uint32_t n1 = l1 + (((l1 + 1u) & 1u) ? c1 : c0);
+            c0 = n0;
+            c1 = n1;
+            head = lh;
+        }
+    }
+
+    // 4. the lanes that are not clean, in order, with the clean stretches between them
+    uint32_t tb = 0;                                                         // bit pattern of the running sum, the same in every lane
+    uint64_t todo = dirty_mask;
+    bool redo = false;
+    for (;;) {
+        int prev = -1;
+        bool failed = false;
+        // applies the composed pair of lane `last` (the end of a clean stretch) to the running sum
+        auto stretch = [&](int last) {
+            const uint32_t f0 = __builtin_amdgcn_readlane(c0, last), f1 = __builtin_amdgcn_readlane(c1, last);
+            const uint32_t eb = __builtin_amdgcn_readlane(base, last);
+            const uint32_t k = tb - eb;                                      // t = 2^e + k ulp, if t lies in that binade
+            const uint32_t k2 = k + ((k & 1u) ? f1 : f0);
+            if ((tb & 0x7f800000u) != eb || k2 >= (1u << 23)) failed = true;
+            tb = eb + k2;
+        };
+        while (todo) {
+            const int d = __builtin_ctzll(todo);
+            todo &= todo - 1;
+            if (!redo && d - 1 > prev) stretch(d - 1);
+            float t = u2f(tb);
+#pragma unroll
+            for (int v = 0; v < V; v++) C::add1(t, run[v]);
+            tb = __builtin_amdgcn_readlane(f2u(t), d);
+            prev = d;
+        }
+        if (!redo && prev < 63) stretch(63);
+        if (!failed || redo) break;
+        redo = true;                                                         // the plain sum: every lane's run, one after the other
+        todo = ~0ull;
+        tb = 0;
+    }
+
+    const RowStats<T> st = finish_stats<T, NORM_RMS>(0.0f, u2f(tb), cols, eps);
+#pragma unroll
+    for (int j = 0; j < V; j++) {
+        const uint32_t i = j * 64 + lane;
+        if (i < nvec) {
+            Vec16<T> in, sc, out;
+            in.u = xr[j];
+            sc.u = reinterpret_cast<const v4u*>(scale)[i];
+#pragma unroll
+            for (int q = 0; q < 8; q++) out.e[q] = norm_one<T, NORM_RMS>(in.e[q], st, sc.e[q], sc.e[q], false);
+            st_stream(yrow + i, out.u);
+        }
+    }
+    // the next row's squares go to the same LDS buffer: every lane has read its run by now (the run is in registers)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+}
+
+template <typename T>
+int launch_rms16_par(rt_device* dev, const void* x, const void* scale, void* y, uint64_t rows, uint32_t cols, float eps) {
+    // as many blocks as the chip holds at one time (what the runtime says for the instantiation's registers and LDS,
+    // asked once per device), each wave taking every grid-th row
+    const uint32_t v = (cols + 511) / 512;
+    constexpr int TI = std::is_same<T, half_t>::value ? 0 : 1;
+    uint64_t blocks = (rows + RP_BLOCK / 64 - 1) / (RP_BLOCK / 64);
+#define RT_RP(VC)                                                                                                                    \
+    case VC:                                                                                                                         \
+        if (!dev->rp_resident[TI][VC]) {                                                                                             \
+            int per_cu = 0;                                                                                                          \
+            RT_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, rms16_par_kernel<T, VC>, RP_BLOCK,                          \
+                                                                (size_t)(RP_BLOCK / 64) * VC * 64 * 16));                            \
+            dev->rp_resident[TI][VC] = (uint16_t)(per_cu < 1 ? 1 : per_cu);                                                          \
+        }                                                                                                                            \
+        if (blocks > (uint64_t)dev->rp_resident[TI][VC] * dev->num_cus) blocks = (uint64_t)dev->rp_resident[TI][VC] * dev->num_cus;  \
+        hipLaunchKernelGGL((rms16_par_kernel<T, VC>), dim3((unsigned)blocks), dim3(RP_BLOCK), (size_t)(RP_BLOCK / 64) * VC * 64 * 16, \
+                           dev->stream, (const T*)x, (const T*)scale, (T*)y, rows, cols, eps);                                       \
+        break
+    switch (v) {
+        RT_RP(1); RT_RP(2); RT_RP(3); RT_RP(4); RT_RP(5); RT_RP(6); RT_RP(7); RT_RP(8);
+        default: return rt_fail(RT_ERR_ARG, "norm: internal: %u columns in the wave-per-row RMSNorm", cols);
+    }
+#undef RT_RP
+    RT_CHECK_LAUNCH("rms16_par_kernel");
+    return RT_OK;
+}
+
 template <typename T, int KIND>
 int launch_norm16_lane(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint64_t rows, uint32_t cols, float eps) {
     const uint64_t blocks = (rows + BLOCK - 1) / BLOCK;
@@ -878,6 +1141,16 @@ template <typename T, int KIND>
 int launch_norm16(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint64_t rows, uint32_t cols, float eps) {
     const bool vec_ok = (cols % 8 == 0) && rt_aligned(x, 16) && rt_aligned(y, 16) && rt_aligned(scale, 16) && (!bias || rt_aligned(bias, 16));
     if (vec_ok && cols <= 128 && rows >= 16384) return launch_norm16_lane<T, KIND>(dev, x, scale, bias, y, rows, cols, eps);
+    // RMSNorm rows of 256 to 4096 columns, as many rows as the chip holds waves at one time: the row sum replayed by the
+    // whole wave.  It issues about twice the instructions of the walk below, which wins back as soon as the rows come in
+    // more than one round ([8192,3072]: 27 against 22 us; [4096,3072]: 13.1 against 14.2 us, [1024,4096]: 11.9 against 14.5).
+    // RMSNorm rows of 256 to 4096 columns, as many of them as the walk below takes in one round (8 rows a block, two
+    // blocks a CU): the row sum replayed by a whole wave per row.  That kernel issues about twice the instructions of
+    // the walk and a row takes a wave about 2.5 us, so it pays where the walk's latency is what the launch costs
+    // ([4096,3072] f16: 12.5 against 14.2 us, [2048,2560] 8.8 against 10.6, [1024,4096] 9.2 against 14.5) and loses
+    // where rows come in several rounds ([8192,3072] 25.5 against 22.1 us, [65536,512] 43 against 25).
+    if (vec_ok && KIND == NORM_RMS && cols >= 256 && cols <= 4096 && rows <= 16ull * (uint64_t)dev->num_cus)
+        return launch_rms16_par<T>(dev, x, scale, y, rows, cols, eps);
     if (vec_ok) {
         const uint64_t blocks = (rows + 7) / 8;
         RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "norm: too many rows");

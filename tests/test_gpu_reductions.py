@@ -500,6 +500,45 @@ def test_norms_16_bit_both_output_passes(dev, oracle, rows, cols, kind):
         assert np.array_equal(np.asarray(got).view(np.uint16), np.asarray(want).view(np.uint16)), (name, rows, cols, kind)
 
 
+@pytest.mark.parametrize("cols", [256, 512, 1000, 1536, 2560, 3072, 4096])
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+def test_rms_norm_16_bit_row_sums_replayed_in_parallel(dev, oracle, cols, kind):
+    """Rows of 256 to 4096 columns take a kernel that replays the reference's left-to-right f32 sum of T(x*x) with the 64
+    lanes of a wave (pairs of sums per lane, composed across lanes) instead of walking it; the output must not differ in
+    one bit from the walk.  Rows that stress what the kernel decides by: sums that land exactly on powers of two, ranges
+    of 2^30 inside a row, heavy tails, squares that overflow the element type, NaN, rows of zeros, single large terms."""
+    rng = np.random.default_rng(316 + cols)
+    bf = kind == "bf16"
+    conv = (lambda a: _bf16(oracle, a)) if bf else (lambda a: np.asarray(a, np.float32).astype(np.float16))
+    rows = []
+    rows += [rng.standard_normal(cols) * s for s in (1.0, 1.0, 1.0, 0.01, 0.3, 3.0, 20.0, 100.0)]
+    rows += [np.ones(cols), np.full(cols, 0.5), np.full(cols, 2.0), np.full(cols, 0.0078125), np.zeros(cols)]
+    rows += [np.concatenate([np.full(cols // 2, 2.5e-4), np.full(cols - cols // 2, 100.0)])]          # tiny terms, then large ones
+    rows += [np.concatenate([np.full(cols // 2, 100.0), np.full(cols - cols // 2, 2.5e-4)])]          # large sum, then terms below its ulp
+    rows += [np.clip(rng.standard_cauchy(cols), -200, 200)]
+    one_big = rng.standard_normal(cols) * 0.1
+    one_big[cols // 3] = 250.0
+    rows += [one_big]
+    overflow = rng.standard_normal(cols)
+    overflow[cols // 2] = 300.0                                                                     # the square is inf in f16
+    rows += [overflow]
+    with_nan = rng.standard_normal(cols)
+    with_nan[7] = np.nan
+    rows += [with_nan]
+    rows += [np.abs(rng.standard_normal(cols)) * 2.0 ** rng.integers(-12, 6, cols)]                   # every term its own binade
+    rows += [np.arange(cols) % 7 * 0.125, np.linspace(0, 8, cols), np.linspace(8, 0, cols)]
+    rows += [rng.standard_normal(cols) for _ in range(40)]
+    x = conv(np.stack(rows))
+    w = conv(1 + 0.02 * rng.standard_normal(cols))
+    want = oracle.rms_norm(x, w, 1e-5, bf16=bf, intended=True)
+    got = dev.rms_norm(dev.upload(x, bf16=bf), dev.upload(w, bf16=bf), 1e-5).to_numpy()
+    g, t = np.asarray(got).view(np.uint16), np.asarray(want).view(np.uint16)
+    nan = (lambda a: (a & 0x7f80) == 0x7f80) if bf else (lambda a: (a & 0x7c00) == 0x7c00)
+    same = (g == t) | (nan(g) & nan(t) & ((g & (0x7f if bf else 0x3ff)) != 0) & ((t & (0x7f if bf else 0x3ff)) != 0))
+    bad_rows = np.flatnonzero(~same.all(axis=1))
+    assert bad_rows.size == 0, (kind, cols, bad_rows[:10].tolist())
+
+
 @pytest.mark.parametrize("rows,cols,kind", [(20000, 8, "f16"), (16384 + 3, 64, "f16"), (17000, 128, "f16"), (30000, 24, "bf16"), (16500, 120, "bf16")])
 def test_norms_16_bit_many_narrow_rows(dev, oracle, rows, cols, kind):
     """tens of thousands of rows of at most 128 columns take a kernel with one lane per row; same bits as the walkers"""

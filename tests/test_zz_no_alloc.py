@@ -69,3 +69,36 @@ def test_static_scratch_group_norm_refuses_what_does_not_fit(dev):
     assert e.value.status == 6 and "fixed buffer" in str(e.value)      # RT_ERR_SIZE
     dev.group_norm(x, 2, None, None, 1e-5, out=y)                      # the growable entry point takes it
     dev.sync()
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_static_scratch_group_norm_records_into_a_graph_and_replays(dev, oracle, dtype):
+    """While a device is capturing, every call that would allocate from the driver or wait for the device is refused
+    (RT_ERR_CAPTURE), and hipMalloc itself is illegal: a capture of rt_group_norm_static that ends cleanly shows that the
+    entry point stays away from the driver, which the pool's counters cannot (the growable scratch of rt_group_norm is
+    grown with hipMalloc directly).  The shape splits every group over slices and needs more partials (98 304 bytes)
+    than nothing, so the fixed array is really used.  Replays, with eager work between them, reproduce the eager bits."""
+    from ratchet_amd.runtime import Buffer
+
+    rng = np.random.default_rng(901)
+    shape, groups = (2, 64, 32768), 8
+    x = randn(rng, shape, dtype)
+    w, b = randn(rng, shape[1], dtype), randn(rng, shape[1], dtype)
+    dx, dw, db = dev.upload(x), dev.upload(w), dev.upload(b)
+    eager, replayed = Buffer(dev, shape, dx.dt), Buffer(dev, shape, dx.dt)
+    dev.group_norm(dx, groups, dw, db, 1e-5, out=eager, static_scratch=True)
+    before = dev.pool_stats()
+    with dev.capture() as g:
+        dev.group_norm(dx, groups, dw, db, 1e-5, out=replayed, static_scratch=True)
+    assert dev.pool_stats() == before
+    want = eager.to_numpy()
+    for k in range(3):
+        replayed.zero_()
+        g.launch()
+        assert same_bits(replayed.to_numpy(), want), k
+        # the program's own eager work between the replays: another problem through the same fixed array
+        other = Buffer(dev, (1, 12, 40000), dx.dt)
+        dev.group_norm(dev.upload(randn(rng, (1, 12, 40000), dtype)), 4, None, None, 1e-5, out=other, static_scratch=True)
+        dev.sync()
+    bad, mx = oracle.count_not_close(want, oracle.group_norm(x, groups, w, b, 1e-5), 1e-3 if dtype == np.float16 else 1e-5, 1e-3 if dtype == np.float16 else 1e-5)
+    assert bad == 0, (bad, mx)
