@@ -653,6 +653,7 @@ def profile_targets(dev, seed, names, reps):
       softmax_causal  rt_softmax on the same scores with the mask already added (the step's launch, on its own)
       softmax_dense   rt_softmax on dense N(0,2) scores of that shape (no -inf: the table lookups of a wave differ)
       copy_1gib       the plain copy kernel on 1 GiB (the counters' calibration and the copy ceiling)
+      bf16_layer_norm, bf16_rms_norm, f16_rms_norm   the 16-bit reference norms on [4096,3072], cold operands every launch
       copy_reference  one plain copy per op of the step (half the op's algorithmic bytes read, half written, fresh regions
                       of two 1 GiB buffers), then a 21 MB copy + 16-byte fill and a 2 MB copy + 16-byte fill: per repetition
                       19 copy launches and 2 fills, in that order"""
@@ -679,6 +680,35 @@ def profile_targets(dev, seed, names, reps):
             fn = lambda: dev.softmax(masked, out=y)
         elif name == "copy_1gib":
             fn = lambda: _lib.check(dev.lib.rt_cast(dev.handle, F16, F16, x.ptr, y.ptr, x.numel))
+        elif name in ("bf16_layer_norm", "bf16_rms_norm", "f16_rms_norm"):
+            # the 16-bit reference norms on [4096,3072], over twelve sets of buffers in turn (cold operands every launch)
+            bf = name.startswith("bf16")
+            rows_n, cols_n = 4096, 3072
+            f32 = normal(seed, 950, (rows_n, cols_n), 1.0, np.float32)
+            if bf:                                               # round to nearest even on the bit pattern
+                u = f32.view(np.uint32)
+                host = ((u + 0x7fff + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+                g = ((np.float32(1.0) + normal(seed, 951, (cols_n,), 0.02, np.float32)).view(np.uint32) >> 16).astype(np.uint16)
+            else:
+                host = f32.astype(np.float16)
+                g = (np.float32(1.0) + normal(seed, 951, (cols_n,), 0.02, np.float32)).astype(np.float16)
+            dt = 2 if bf else F16
+            dg = dev.upload(g, bf16=bf)
+            sets_n = []
+            for _ in range(12):
+                a = dev.upload(host, bf16=bf)
+                sets_n.append((a, dev.empty((rows_n, cols_n), dt)))
+            turn = [0]
+
+            def norm_launch():
+                a, o = sets_n[turn[0] % len(sets_n)]
+                turn[0] += 1
+                if name.endswith("layer_norm"):
+                    dev.layer_norm(a, dg, dg, 1e-5, out=o)
+                else:
+                    dev.rms_norm(a, dg, 1e-5, out=o)
+
+            fn = norm_launch
         elif name == "copy_reference":
             # the copy pass of the bench (one copy per op of the step, same bytes, back to back), without its events; behind
             # it the boundary probes: a 16-byte fill behind a 21 MB copy and behind a 2 MB copy
