@@ -62,6 +62,13 @@ def profile_head(rel_path):
     return None
 
 
+def library_built_from():
+    """the commit the loaded library was linked from, as the build recorded it beside the objects"""
+    from ratchet_amd import build as hip_build
+
+    return hip_build.built_from()
+
+
 def git_head():
     """commit of the tree this script runs from, when it is a git checkout (the GPU box receives the tree without .git)"""
     try:
@@ -170,7 +177,7 @@ def build_workload(dev, seed):
     d_rms3, d_silu3, d_swiglu3 = dev.empty(x3.shape, F16), dev.empty(gate3.shape, F16), dev.empty(gate3.shape, F16)
     ops.append(Op(3, "rms_norm", "f16", "4096x3072", 2 * x3.nbytes + g3.nbytes, lambda i, o: dev.rms_norm(i[0], i[1], 1e-5, out=o), [d_x3, d_g3], d_rms3,
                   dict(kind="rows", out=d_rms3, x=x3, rows=4096, tol=1e-3, fn=lambda o, xs: o.rms_norm(xs, g3, 1e-5, intended=True)),
-                  "norm_pipe16_kernel", rotating=[0]))
+                  "rms16_par_kernel", rotating=[0]))
     ops.append(Op(3, "silu(gate)", "f16", "[1,4096,8192]", 2 * gate3.nbytes, lambda i, o: dev.unary("silu", i[0], out=o), [d_gate3], d_silu3,
                   dict(kind="rows", out=d_silu3, x=gate3, rows=4096, tol=1e-3, fn=lambda o, xs: o.unary("silu", xs)), "unary_lut_kernel"))
     ops.append(Op(3, "mul silu(gate)*up", "f16", "[1,4096,8192]x2", 3 * gate3.nbytes, lambda i, o: dev.binary("mul", i[0], i[1], out=o),
@@ -1032,7 +1039,7 @@ def main():
                      "kernel_us_source": PROFILE_KERNEL_TRACE,
                      # the commit the two summaries were taken at (their `git_head:` line) and the commit of this run
                      "profiles_git_head": {"kernel_trace": profile_head(PROFILE_KERNEL_TRACE), "hbm_traffic": profile_head(PROFILE_HBM_TRAFFIC)},
-                     "git_head": git_head()},
+                     "git_head": git_head(), "library_built_from": library_built_from()},
         "cpu_baseline": None if args.no_cpu or cpu_t == 0 else {
             "value": round(cpu_b / cpu_t / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": "every op of the step on one host core with the reference's to_vec/store copies, whole tensors "

@@ -86,6 +86,34 @@ def build_host(force=False, sanitize=False):
     return HOST_LIB_PATH
 
 
+STAMP_PATH = os.path.join(OBJ_DIR, "built_from.txt")
+
+
+def _stamp():
+    """Record beside the objects which commit the library was linked from (and whether the kernel sources differed from
+    it), so that a run on a machine that received the tree without its history can still say what it measured."""
+    root = os.path.dirname(HERE)
+    try:
+        head = subprocess.run(["git", "-C", root, "rev-parse", "--short=12", "HEAD"], capture_output=True, text=True, timeout=20)
+        dirty = subprocess.run(["git", "-C", root, "status", "--porcelain", "--", "ratchet_amd/csrc", "include"],
+                               capture_output=True, text=True, timeout=20)
+        if head.returncode != 0:
+            return
+        text = head.stdout.strip() + (" + uncommitted changes to the sources" if dirty.stdout.strip() else "")
+    except (OSError, subprocess.SubprocessError):
+        return
+    with open(STAMP_PATH, "w") as f:
+        f.write(text + "\n")
+
+
+def built_from():
+    """what _stamp() wrote at the last link, or None"""
+    try:
+        return open(STAMP_PATH).read().strip() or None
+    except OSError:
+        return None
+
+
 def build(force=False, jobs=4):
     os.makedirs(OBJ_DIR, exist_ok=True)
     with ThreadPoolExecutor(max_workers=jobs) as ex:
@@ -95,6 +123,7 @@ def build(force=False, jobs=4):
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError("link failed:\n%s\n%s" % (" ".join(cmd), r.stderr[-8000:]))
+        _stamp()
     build_host(force)
     return LIB_PATH
 
