@@ -86,7 +86,7 @@ def build_host(force=False, sanitize=False):
     return HOST_LIB_PATH
 
 
-STAMP_PATH = os.path.join(OBJ_DIR, "built_from.txt")
+STAMP_PATH = os.path.join(HERE, "built_from.txt")              # beside the library: it travels with it
 
 
 def _stamp():
