@@ -71,9 +71,14 @@ int rt_free(rt_device* dev, void* dptr);                     /* last drop of a P
 /* rt_malloc / rt_free sit on a per-device pool (the role of gpu/pools/buffer_pool.rs:60-112): a freed block is parked
  * and handed out again to a later request of about its size; since every kernel and copy of a device runs on its one
  * in-order stream, neither call synchronises.  rt_pool_trim returns the parked blocks to the driver (it waits for
- * queued work first); rt_pool_stats reports bytes handed out, bytes parked, and how many requests the pool served
+ * queued work first); rt_pool_begin_pass is the pool's begin_pass (gpu/pools/dynamic_resource_pool.rs:140-190, called
+ * by WgpuDevice::begin_pass, gpu/device.rs:275-277, at the top of every resolve, tensor.rs:800): a block that was
+ * freed before the previous call and has not been handed out since goes back to the driver, so a block survives
+ * one whole pass unused, as the reference's buffers do; when there is no such block the call touches neither the
+ * driver nor the stream, and while the device is capturing it frees nothing; rt_pool_stats reports bytes handed out, bytes parked, and how many requests the pool served
  * (hits) or passed to hipMalloc (misses); any out pointer may be NULL. */
 int rt_pool_trim(rt_device* dev);
+int rt_pool_begin_pass(rt_device* dev);
 int rt_pool_stats(rt_device* dev, uint64_t* live_bytes, uint64_t* parked_bytes, uint64_t* hits, uint64_t* misses);
 /* the most bytes that were handed out at one time since the last reset (reset != 0 restarts the mark at what is handed
  * out now): what a graph executor checks its activation memory plan against (allocator.rs:266-271 logs the same total) */

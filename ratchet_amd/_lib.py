@@ -24,7 +24,7 @@ STATUS_NAMES = {
 
 EXPORTS = [
     "rt_device_count", "rt_device_create", "rt_device_destroy", "rt_sync", "rt_last_error", "rt_status_name", "rt_debug_hip_status", "rt_debug_softmax_pace", "rt_malloc",
-    "rt_free", "rt_pool_trim", "rt_pool_stats", "rt_pool_peak", "rt_capture_begin", "rt_capture_end", "rt_graph_launch", "rt_graph_destroy", "rt_memset0", "rt_h2d", "rt_d2h", "rt_d2d", "rt_event_create", "rt_event_destroy", "rt_event_record",
+    "rt_free", "rt_pool_trim", "rt_pool_begin_pass", "rt_pool_stats", "rt_pool_peak", "rt_capture_begin", "rt_capture_end", "rt_graph_launch", "rt_graph_destroy", "rt_memset0", "rt_h2d", "rt_d2h", "rt_d2d", "rt_event_create", "rt_event_destroy", "rt_event_record",
     "rt_event_elapsed_ms", "rt_binary", "rt_binary_bcast", "rt_unary", "rt_cast", "rt_permute", "rt_slice", "rt_broadcast",
     "rt_concat", "rt_cache", "rt_index_select", "rt_index_select_q8_0", "rt_index_write", "rt_rope", "rt_softmax", "rt_softmax_masked", "rt_layer_norm", "rt_rms_norm", "rt_group_norm", "rt_group_norm_static", "rt_norm_via_f32", "rt_softmax_via_f32", "rt_unary_via_f32", "rt_gated_mul_via_f32",
 ]
@@ -63,6 +63,7 @@ def load():
     L.rt_malloc.argtypes = [vp, sz, pp]
     L.rt_free.argtypes = [vp, vp]
     L.rt_pool_trim.argtypes = [vp]
+    L.rt_pool_begin_pass.argtypes = [vp]
     L.rt_capture_begin.argtypes = [vp]
     L.rt_capture_end.argtypes = [vp, pp]
     L.rt_graph_launch.argtypes = [vp, vp]

@@ -1070,6 +1070,7 @@ struct Resolver {
     static void resolve(Node* root) {
         size_t launches = 0;
         Prepared P = prepare(root);
+        bool pass_begun = false;
         // shared objects come from the device's pool when their first tenant is produced and go back after their last reader
         std::vector<std::shared_ptr<Buffer>> objects(P.plan.object_bytes.size());
         for (size_t i = 0; i < P.order.size(); i++) {
@@ -1078,6 +1079,12 @@ struct Resolver {
             if (st != P.step_of.end()) {
                 const planner::Step& step = P.steps[st->second];
                 const int obj = P.plan.object_of.at(n->id);
+                if (!pass_begun) {
+                    // a resolve is a pass of the storage pool, as in resolve_gpu (tensor.rs:800): blocks that nobody took
+                    // during the last one go back to the driver before this one allocates
+                    check_rt(rt_pool_begin_pass(n->device.raw()), "rt_pool_begin_pass");
+                    pass_begun = true;
+                }
                 if (step.inplace >= 0) {
                     n->storage = P.step_reads[st->second][(size_t)step.inplace]->storage;
                 } else if (obj >= 0) {
@@ -1147,6 +1154,7 @@ struct Resolver {
                 throw Error("Unresolved", "constant tensor " + std::to_string(n->id) + " has no storage (placeholder)");
         inner->device = root->device;
         inner->root = root_ref;
+        check_rt(rt_pool_begin_pass(root->device.raw()), "rt_pool_begin_pass");
         std::vector<std::shared_ptr<Buffer>> objects(P.plan.object_bytes.size());
         for (size_t o = 0; o < objects.size(); o++) {
             objects[o] = std::make_shared<Buffer>(root->device, P.plan.object_bytes[o]);

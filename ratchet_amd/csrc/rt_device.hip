@@ -16,9 +16,14 @@ struct rt_graph {
     int ordinal;
 };
 
+struct rt_parked {
+    void* ptr;
+    uint64_t pass;                                  // the pass (rt_pool_begin_pass count) during which the block was freed
+};
 struct rt_pool {
     std::mutex mu;
-    std::multimap<size_t, void*> parked;            // block size -> block, free for reuse
+    std::multimap<size_t, rt_parked> parked;        // block size -> block, free for reuse
+    uint64_t pass = 0;
     std::unordered_map<void*, size_t> live;         // blocks handed out by rt_malloc
     size_t parked_bytes = 0;
     size_t live_bytes = 0, peak_live_bytes = 0;     // handed out now / the most that was handed out at once since the last reset
@@ -187,7 +192,7 @@ int rt_device_destroy(rt_device* dev) {
     if (dev->gn_scratch) (void)hipFree(dev->gn_scratch);
     if (dev->sm_row_sums) (void)hipFree(dev->sm_row_sums);
     // buffers the caller never returned are released with the device, like the parked ones
-    for (auto& kv : dev->pool->parked) (void)hipFree(kv.second);
+    for (auto& kv : dev->pool->parked) (void)hipFree(kv.second.ptr);
     for (auto& kv : dev->pool->live) (void)hipFree(kv.first);
     delete dev->pool;
     hipError_t e = hipStreamDestroy(dev->stream);
@@ -231,8 +236,8 @@ int rt_malloc(rt_device* dev, size_t bytes, void** dptr) {
     std::lock_guard<std::mutex> lock(pool->mu);
     auto it = pool->parked.lower_bound(sz);
     if (it != pool->parked.end() && it->first <= sz + sz / 4) {
-        *dptr = it->second;
-        pool->live.emplace(it->second, it->first);
+        *dptr = it->second.ptr;
+        pool->live.emplace(it->second.ptr, it->first);
         pool->live_bytes += it->first;
         if (pool->live_bytes > pool->peak_live_bytes) pool->peak_live_bytes = pool->live_bytes;
         pool->parked_bytes -= it->first;
@@ -245,7 +250,7 @@ int rt_malloc(rt_device* dev, size_t bytes, void** dptr) {
     if (e == hipErrorOutOfMemory && !pool->parked.empty()) {   // give the parked blocks back and try once more
         (void)hipGetLastError();
         (void)hipStreamSynchronize(dev->stream);
-        for (auto& kv : pool->parked) (void)hipFree(kv.second);
+        for (auto& kv : pool->parked) (void)hipFree(kv.second.ptr);
         pool->parked.clear();
         pool->parked_bytes = 0;
         e = hipMalloc(dptr, sz);
@@ -269,7 +274,7 @@ int rt_free(rt_device* dev, void* dptr) {
     std::lock_guard<std::mutex> lock(pool->mu);
     auto it = pool->live.find(dptr);
     RT_REQUIRE(it != pool->live.end(), RT_ERR_ARG, "rt_free: %p was not allocated by rt_malloc on this device (or was freed twice)", dptr);
-    pool->parked.emplace(it->second, dptr);
+    pool->parked.emplace(it->second, rt_parked{dptr, pool->pass});
     pool->parked_bytes += it->second;
     pool->live_bytes -= it->second;
     pool->live.erase(it);
@@ -285,11 +290,44 @@ int rt_pool_trim(rt_device* dev) {
     std::lock_guard<std::mutex> lock(pool->mu);
     hipError_t first = hipSuccess;
     for (auto& kv : pool->parked) {
-        hipError_t e = hipFree(kv.second);
+        hipError_t e = hipFree(kv.second.ptr);
         if (e != hipSuccess && first == hipSuccess) first = e;
     }
     pool->parked.clear();
     pool->parked_bytes = 0;
+    if (first != hipSuccess) return rt_fail_hip(first, "hipFree");
+    return RT_OK;
+}
+
+// The reference's pool ages its unused buffers by passes (gpu/pools/dynamic_resource_pool.rs:140-190, called at the top of
+// every resolve: tensor.rs:800, gpu/device.rs:275-277): a buffer released during pass p can be reclaimed during pass
+// p + 1 and is destroyed at the start of pass p + 2 if nobody did.  The same here: a block parked before the previous
+// call of this function, and still parked, goes back to the driver.  A program that repeats its passes reuses every
+// block each time and never gets here with anything to free, so the steady state stays free of hipFree (and of the wait
+// for the stream that has to precede it); one whose sizes drift no longer grows the parked set without bound.  While a
+// device is capturing nothing is freed: the blocks wait for the first pass that begins outside a capture.
+int rt_pool_begin_pass(rt_device* dev) {
+    int rc = rt_enter(dev);
+    if (rc) return rc;
+    rt_pool* pool = dev->pool;
+    std::lock_guard<std::mutex> lock(pool->mu);
+    const uint64_t now = ++pool->pass;                          // blocks freed from here on carry `now`
+    if (dev->capturing) return RT_OK;
+    bool stale = false;
+    for (auto& kv : pool->parked) stale = stale || kv.second.pass + 2 <= now;
+    if (!stale) return RT_OK;
+    RT_HIP(hipStreamSynchronize(dev->stream));                  // queued work may still use a parked block
+    hipError_t first = hipSuccess;
+    for (auto it = pool->parked.begin(); it != pool->parked.end();) {
+        if (it->second.pass + 2 <= now) {
+            hipError_t e = hipFree(it->second.ptr);
+            if (e != hipSuccess && first == hipSuccess) first = e;
+            pool->parked_bytes -= it->first;
+            it = pool->parked.erase(it);
+        } else {
+            ++it;
+        }
+    }
     if (first != hipSuccess) return rt_fail_hip(first, "hipFree");
     return RT_OK;
 }

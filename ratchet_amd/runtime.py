@@ -194,6 +194,11 @@ class Device:
     def pool_trim(self):
         check(self.lib.rt_pool_trim(self.handle))
 
+    def pool_begin_pass(self):
+        """What the reference does at the top of every resolve: blocks freed before the previous call and not reused since
+        go back to the driver."""
+        check(self.lib.rt_pool_begin_pass(self.handle))
+
     # ---- storage
     def empty(self, shape, dt):
         return Buffer(self, shape, dt)

@@ -247,6 +247,7 @@ def test_graph_validation(lib):
 
 def test_pool_validation(lib):
     assert lib.rt_pool_trim(None) == 8
+    assert lib.rt_pool_begin_pass(None) == 8
     assert lib.rt_pool_stats(None, None, None, None, None) == 8
 
 

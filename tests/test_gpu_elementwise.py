@@ -275,6 +275,58 @@ def test_storage_pool_reuses_blocks_in_stream_order(oracle):
         d.close()
 
 
+def test_storage_pool_ages_unused_blocks_by_passes():
+    """rt_pool_begin_pass is the reference's begin_pass (gpu/pools/dynamic_resource_pool.rs:140-190): a block freed during
+    pass p can be taken again during passes p and p + 1 and goes back to the driver at the start of pass p + 2 if nobody
+    did.  With sizes that drift from pass to pass the parked set therefore stays at the last two passes' blocks instead
+    of growing; a program that repeats its sizes keeps hitting the pool and nothing is ever returned."""
+    from ratchet_amd import Device
+
+    d = Device(0)
+    try:
+        MB = 1 << 20
+        d.pool_trim()
+        parked_after = []
+        for k in range(12):                                   # every pass wants a size no earlier pass had
+            d.pool_begin_pass()
+            b = d.empty(((8 + 3 * k) * MB // 4,), 0)
+            c = d.empty(((100 + 20 * k) * MB // 4,), 0)              # apart by more than the pool's size classes (1/16)
+            del b, c
+            parked_after.append(d.pool_stats()[1])
+        # pass k leaves its own two blocks and those of pass k - 1 (sizes are rounded up by at most 1/16)
+        for k in range(1, 12):
+            own = (8 + 3 * k + 100 + 20 * k) * MB
+            before = (8 + 3 * (k - 1) + 100 + 20 * (k - 1)) * MB
+            assert own + before <= parked_after[k] <= (own + before) * 17 // 16, (k, parked_after[k])
+        d.pool_begin_pass()
+        d.pool_begin_pass()
+        assert d.pool_stats()[1] == 0                         # two passes without a taker: everything went back
+        # steady state: the same two sizes every pass are served by the pool, and no block is returned
+        live0, parked0, hits0, misses0 = d.pool_stats()
+        for k in range(6):
+            d.pool_begin_pass()
+            b = d.empty((16 * MB // 4,), 0)
+            c = d.empty((64 * MB // 4,), 0)
+            del b, c
+        live, parked, hits, misses = d.pool_stats()
+        assert misses == misses0 + 2 and hits == hits0 + 10 and parked == 80 * MB
+        # a block in use is not the pool's to return, however many passes go by
+        keep = d.upload(np.arange(1024, dtype=np.float32))
+        for k in range(4):
+            d.pool_begin_pass()
+        assert np.array_equal(keep.to_numpy(), np.arange(1024, dtype=np.float32))
+        # while the device is capturing, a pass returns nothing (hipFree is not allowed there) and does not fail
+        x = d.upload(np.ones(4096, np.float32))
+        y = d.empty((4096,), 0)
+        with d.capture() as g:
+            d.pool_begin_pass()
+            d.unary("neg", x, out=y)
+        g.launch()
+        assert (y.to_numpy() == -1).all()
+    finally:
+        d.close()
+
+
 @pytest.mark.parametrize("n", [(1 << 21), (1 << 21) + 8, 5 * 32768 * 64 + 32768 * 7 + 8 * 100 + 5, 32768 * 300 - 1])
 def test_unary_table_path_tiles_and_remainders(dev, oracle, n):
     """the table kernel walks whole 64 KiB tiles with the next tile's loads in flight and hands the rest (fewer vectors
