@@ -229,10 +229,12 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
                                                                     const uint32_t* __restrict__ tiles) {
     typedef SpType<T> ST;
     constexpr bool PARK = NSTEP > 0;
-    // Only the plain variant holds its steps to a pace (see launch_stream16).  The masked and ragged variants take longer
-    // per step than the pace by themselves, and the mere presence of the pacing code changed their register allocation
-    // and cost the masked one 6 % (390 -> 416 us), so for them it is compiled out.
-    constexpr bool PACED = !MASK && !RAGGED;
+    // The plain variant and the paired masked one hold their steps to a pace (see launch_stream16).  The paired one does
+    // not get faster by it where the output lies well relative to the input in physical memory (372 against 374 us on
+    // [1,32,4096,4096]), but it no longer loses 13 us where it does not: unpaced, its time depends on one bit of the
+    // memory channel hash in which the two buffers' pages agree or differ.  The unpaired masked variant loses at every
+    // pace tried and the ragged ones take longer per step than the pace by themselves, so for them it is compiled out.
+    constexpr bool PACED = MASK != 1 && !RAGGED;
     // MASK == 2: the two rows of a loader wave are the same row of two neighbouring periods (two heads under one [S, T]
     // mask), so one mask vector serves both and the register of the second holds the mask of the step after next
     constexpr bool PAIR = MASK == 2;
@@ -1003,9 +1005,10 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
         // right length per iteration, and a write-only loop 4.4 against 6.6 TB/s).  So the walker holds the block's
         // steps to the period at which all blocks together move SP_PACE_BYTES_PER_S, by the device's wall clock, and the
         // blocks start out of phase (sp_pace_step).  A pace that is too fast gives the unpaced behaviour back (7.0e12:
-        // 359 us), one that is too slow costs in proportion (6.4e12: 355 us).  Only the plain variant on a grid that
-        // fills the chip is paced.
-        if (blocks == dev->num_cus && !mask && !ragged) {
+        // 359 us), one that is too slow costs in proportion (6.4e12: 355 us).  Paced are, on a grid that fills the
+        // chip, the plain variant and the masked one that takes one mask row per pair of heads (at the same rate: 6.4e12
+        // costs that one 3 us, 6.8e12 and 7.0e12 leave 5 us of its dependence on where the buffers lie).
+        if (blocks == dev->num_cus && !ragged && (!mask || pair)) {
             const double rate = SP_PACE_BYTES_PER_S;
             const double group_bytes = (double)sch.R * rmul * cols * 2 * (nt > SP_MAX_STEPS ? 4 : 2);     // in and out (long rows: parked and read back)
             const double steps = nt > SP_MAX_STEPS ? sch.nsteps : nt == 7 ? 8 : nt;          // the steps the kernel variant takes per group
