@@ -376,6 +376,13 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
     constexpr int NCLS = TILES ? NSTEP : 1, NCROW = PAIR ? 1 : 2;
     auto item_tiles = [&](uint32_t it, uint32_t (&cw)[NCROW][NCLS]) {
         if constexpr (TILES) {
+            if (sch.tile_stride == 0) {                      // no table for this launch: every tile is loaded
+#pragma unroll
+                for (int h = 0; h < NCROW; h++)
+#pragma unroll
+                    for (int t = 0; t < NCLS; t++) cw[h][t] = 0xffffffffu;
+                return;
+            }
             uint32_t rep, pg;
             sp_item(sch, blockIdx.x, G, it, rep, pg);
 #pragma unroll
@@ -1016,9 +1023,13 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
             if (dev->debug_softmax_pace) sch.pace = dev->debug_softmax_pace;
             sch.phase_fx = sch.pace > 0xffffu ? 0 : (sch.pace << 16) / blocks;
         }
-        // the classes of the mask's tiles, for the variants that use them (a table of at most RT_SM_MASK_TILES words)
+        // the classes of the mask's tiles, for the variants that use them (a table of at most RT_SM_MASK_TILES words).  Only
+        // for a mask of 16 MiB or more: a smaller one stays in the L2s between its repeats, loading all of it costs
+        // nothing that could be measured ([1,32,2048,2048] and [1,32,2560,2560]: 111 and 188 us either way), and the
+        // pass over the mask is a launch of 3 us ([8,32,512,512] 71 -> 68 us, a decode step's [1,32,1,4096] 29 -> 26 us).
         sch.tile_stride = 0;
-        if (mask && !ragged && nt <= SP_MAX_STEPS && (uint64_t)sch.PM * nt <= RT_SM_MASK_TILES && rt_aligned(mask, 16)) {
+        if (mask && !ragged && nt <= SP_MAX_STEPS && (uint64_t)sch.PM * nt <= RT_SM_MASK_TILES && rt_aligned(mask, 16) &&
+            (uint64_t)sch.PM * cols * sizeof(T) >= (16ull << 20)) {
             const uint32_t ntiles = sch.PM * nt;
             const uint32_t per_block = (BLOCK / 64) * MT_PER_WAVE;
             hipLaunchKernelGGL((mask_tiles_kernel<T>), dim3((ntiles + per_block - 1) / per_block), dim3(BLOCK), 0, dev->stream, (const T*)mask,

@@ -643,6 +643,34 @@ def test_softmax_masked_equals_add_then_softmax(dev, oracle, shape, mshape):
     assert same_bits(dx.to_numpy(), got)
 
 
+@pytest.mark.parametrize("shape,mshape", [((1, 2, 2048, 4096), (2048, 4096)), ((1, 3, 2048, 4096), (2048, 4096)), ((1, 2, 3300, 2560), (3300, 2560)),
+                                          ((2, 1, 2400, 3584), (1, 1, 2400, 3584))])
+def test_softmax_masked_large_masks_whose_uniform_tiles_are_not_loaded(dev, oracle, shape, mshape):
+    """From 16 MiB on, a pass over the mask classifies its 512-column tiles first, and the streaming kernel loads only the
+    tiles whose elements differ (a tile of equal elements is put together from its class word).  Masks here: causal, with
+    a finite row across it, a stretch of rows that are one finite value throughout (uniform tiles that are neither 0 nor
+    -inf), a tile that differs from its neighbours in its last element only, and NaN in one place.  Two and three heads
+    under one mask take one mask row per pair of heads (the odd head out pairs with nothing); 2560 and 3584 columns take
+    five and seven steps a row.  Always the bits of add-then-softmax."""
+    rng = np.random.default_rng(322)
+    x = randn(rng, shape, np.float16, 2.0)
+    S, T = mshape[-2], mshape[-1]
+    m2 = np.triu(np.full((S, T), -np.inf, np.float16), k=1)
+    m2[S // 2, :] = randn(rng, (T,), np.float16)
+    m2[S // 3:S // 3 + 40, :] = np.float16(-2.5)
+    m2[S // 4, 1023] = np.float16(0.125)
+    m2[S // 5, 700] = np.float16(np.nan)
+    mask = np.ascontiguousarray(m2.reshape(mshape))
+    assert mask.nbytes >= 16 << 20
+    full_mask = np.ascontiguousarray(np.broadcast_to(mask.reshape((1,) * (4 - mask.ndim) + mask.shape), shape))
+    want = oracle.softmax(oracle.binary("add", x, full_mask))
+    dx, dm = dev.upload(x), dev.upload(mask)
+    got = dev.softmax_masked(dx, dm).to_numpy()
+    assert mismatch_count(got, want) == 0, (shape, mshape, describe_mismatch(got, want, x))
+    dev.softmax_masked(dx, dm, out=dx)                                 # in place
+    assert same_bits(dx.to_numpy(), got)
+
+
 @pytest.mark.parametrize("shape,mshape,kind", [((1, 4, 333, 1001), (333, 1001), "f16"), ((2, 3, 77, 199), (1, 1, 77, 199), "f16"),
                                                ((1, 2, 50, 2047), (50, 2047), "f16"), ((2, 2, 40, 511), (2, 1, 40, 511), "f16"),
                                                ((1, 8, 9, 193), (1, 1, 1, 193), "f16"), ((1, 2, 30, 4089), (30, 4089), "f16"),
