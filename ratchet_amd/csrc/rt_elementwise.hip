@@ -739,8 +739,8 @@ int launch_bcast(rt_device* dev, const void* a, const uint32_t a_shape[4], const
     // the other operand patterns, the two are level
     const int unroll = (a_once != b_once && ve == VEMAX && nvec >= BC_ONE_FROM_VECS) ? 1 : BC_UNROLL;
     const unsigned blocks = blocks_for(nvec, BLOCK * unroll);
-    // one operand full-size, the other equal to y's trailing dims and repeated over the leading ones, too large to
-    // stay in an XCD's L2 by itself (>= 1 MiB) and made of whole groups of 8 slabs
+    // one operand full-size, the other equal to y's trailing dims and repeated over the leading ones, too large for
+    // the eight L2s to keep between the repeats in the plain order (RT_XCD_ORDER_MIN_BYTES) and made of whole groups of 8 slabs
     p.slabs = 0;
     p.chunk_log2 = 0;
     p.reps = make_fastdiv(1);
@@ -758,7 +758,7 @@ int launch_bcast(rt_device* dev, const void* a, const uint32_t a_shape[4], const
             }
         }
         const uint64_t per_block = (uint64_t)BLOCK * unroll * ve;
-        if (prefix && reps > 1 && inner * sizeof(T) >= (1u << 20) && inner % (per_block * XCDS) == 0) {
+        if (prefix && reps > 1 && inner * sizeof(T) >= RT_XCD_ORDER_MIN_BYTES && inner % (per_block * XCDS) == 0) {
             p.reps = make_fastdiv((uint32_t)reps);
             p.slabs = (uint32_t)(inner / per_block);
             const uint32_t per_xcd = p.slabs / XCDS;

@@ -12,6 +12,14 @@
 constexpr size_t RT_SM_ROW_SUMS = 1u << 19;
 constexpr size_t RT_SM_MASK_TILES = 1u << 18;   // 512-column tiles of a mask that the streaming softmax can classify per launch
 constexpr size_t RT_SM_TILES_HEAD = 16;         // entries in front of them that always read "load this tile"
+// An operand that repeats over the leading dims of the output (an [S, T] mask under B * H heads) is re-read once per
+// repeat.  Hardware block b runs on XCD b % 8, so in the plain block order each of the eight L2s (4 MiB) sees one eighth
+// of that operand and keeps it between the repeats as long as the whole operand is under about 28 MiB; from there on the
+// kernels that re-read such an operand order their blocks so that all repeats of a slab run back to back on one XCD.
+// Below, that order loses to the plain one (it hops between the repeats every few hundred KiB): scores + mask on
+// [1,32,2560,2560] f16 135 against 156 us, [4,32,1024,1024] 87 against 100; above, it is what keeps the re-reads in
+// L2 at all ([1,32,4096,4096] 338 against 440 us, [1,8,6144,6144] 206 against 244).
+constexpr uint64_t RT_XCD_ORDER_MIN_BYTES = 28ull << 20;
 
 struct rt_device {
     int ordinal;

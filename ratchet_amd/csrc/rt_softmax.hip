@@ -312,8 +312,9 @@ constexpr uint32_t RAGGED_STREAM_MIN_COLS = 192;   // shorter ragged rows: the t
 // on 16-bit scores in one pass: the mask (broadcast over batch / heads, optional) is added in the 16-bit type as the
 // separate add would, the sum is widened, the f32 softmax above is applied in registers and the result rounded once.
 // 4 bytes of HBM traffic per element against 26 for the four separate ops (6 + 6 + 8 + 6).
-// (Ordering the blocks so that the heads sharing a mask row run on one XCD, as binary_bcast_kernel does, changed nothing
-// here: 380 us either way on [1,32,4096,4096]; the mask re-reads are served by the Infinity Cache.)
+// A mask too large for the L2s to keep between the heads is read in the block order of binary_bcast_kernel (all heads of a
+// mask slab back to back on one XCD): [1,32,4096,4096] 329 us against 392 us in the plain order; smaller masks take the
+// plain order, which is faster there ([1,32,2560,2560] 141 against 164 us, [1,32,1536,1536] 52 against 62 us).
 // ------------------------------------------------------------------------------------------------------------------
 struct MaskArgs {
     FastDiv d2, d1;          // x extents of dims 2 and 1 (rows = d0 * d1 * d2)
@@ -855,8 +856,9 @@ extern "C" int rt_softmax_via_f32(rt_device* dev, int io_dt, const void* x, cons
             st *= mask_shape[i];
         }
         mask_vec_ok = !p.mlast || (rt_aligned(mask, 16) && cols % 8 == 0);
-        // a mask of whole trailing dims, at least 1 MiB, repeated over the leading ones, whose period is whole groups of
-        // eight 4-row blocks: the XCD-aware block order (used by the one-wave-per-row kernel only)
+        // a mask of whole trailing dims, too large for the L2s to keep between its repeats in the plain order
+        // (RT_XCD_ORDER_MIN_BYTES), repeated over the leading dims, whose period is whole groups of eight 4-row blocks: the
+        // XCD-aware block order (the kernels with whole rows per block)
         int lead = 0;
         while (lead < 3 && mask_shape[lead] == 1) lead++;
         bool whole = p.mlast && lead > 0;
@@ -868,7 +870,7 @@ extern "C" int rt_softmax_via_f32(rt_device* dev, int io_dt, const void* x, cons
                 if (mask_shape[i] != x_shape[i]) whole = false;
             }
         }
-        if (whole && reps > 1 && reps <= 0xffffffffull && period * cols * 2 >= (1u << 20) && period % (WAVES * 8) == 0 &&
+        if (whole && reps > 1 && reps <= 0xffffffffull && period * cols * 2 >= RT_XCD_ORDER_MIN_BYTES && period % (WAVES * 8) == 0 &&
             rows <= 0x7fffffffull) {
             p.reps = make_fastdiv((uint32_t)reps);
             p.period = (uint32_t)period;

@@ -81,10 +81,11 @@ def test_binary_broadcast_fused(dev, oracle, dtype):
     rng = np.random.default_rng(104)
     cases = [((1, 150, 384), (384,)), ((2, 3, 16, 16), (16, 16)), ((1, 4, 64, 1), (1, 1, 1, 64)), ((3, 1, 5), (1, 7, 1)),
              ((5, 7), (1,)), ((1,), (2, 9)), ((2, 3, 4, 10), (2, 1, 4, 1)), ((4, 1, 8), (4, 6, 8)), ((6, 130), (6, 1)),
-             # a >= 1 MiB operand repeated over the leading dims takes the XCD-aware block order (walks of 4, 64 and 1 slabs,
-             # either side repeated)
+             # an operand of 1 to 8 MiB repeated over the leading dims: the L2s keep it between the repeats, plain block order
              ((1, 3, 1024, 512), (1024, 512)), ((1024, 1024), (3, 1024, 1024)), ((5, 136, 4096), (136, 4096)),
-             ((2, 2, 256, 2048), (1, 1, 256, 2048))]
+             ((2, 2, 256, 2048), (1, 1, 256, 2048)),
+             # from 28 MiB on such an operand takes the XCD-aware block order (walks of 64, 4 and 1 slabs, either side repeated)
+             ((2, 4096, 4096), (4096, 4096)), ((3616, 4096), (2, 3616, 4096)), ((1, 2, 3592, 4096), (3592, 4096))]
     for sa, sb in cases:
         a, b = randn(rng, sa, dtype), randn(rng, sb, dtype)
         out_shape = np.broadcast_shapes(sa, sb)

@@ -119,6 +119,8 @@ def _attn_case(rng, B, H, S, T, mask_kind, dtype=np.float16):
         mask = np.triu(np.full((S, T), -np.inf, dtype), k=1 + T - S)
     elif mask_kind == "causal4":
         mask = np.triu(np.full((S, T), -np.inf, dtype), k=1 + T - S).reshape(1, 1, S, T)
+    elif mask_kind == "holes":                                 # finite values with -inf in three places of ten, any S and T
+        mask = np.where(rng.random((S, T)) < 0.3, -np.inf, rng.standard_normal((S, T))).astype(dtype)
     elif mask_kind == "per_batch":
         mask = (rng.standard_normal((B, 1, 1, T)) * 2).astype(dtype)
     elif mask_kind == "row_scalar":
@@ -133,8 +135,11 @@ def _attn_case(rng, B, H, S, T, mask_kind, dtype=np.float16):
                                                (1, 2, 7, 4096, "causal"), (1, 1, 3, 8200, None), (1, 3, 5, 4100, "causal"),
                                                (1, 2, 6, 8192, "causal"), (2, 1, 3, 16384, "per_batch"), (1, 2, 4, 6000, None),
                                                (1, 1, 2, 16392, None),
-                                               # masks of 1 MiB and more under several heads: the XCD-aware block order (chunks of 64, 4, 1)
+                                               # masks of 1 to 8 MiB under several heads (the L2s keep them: plain block order)
                                                (2, 2, 2048, 2048, "causal"), (1, 3, 160, 4096, "causal"),
+                                               # masks of 28 MiB and more: the XCD-aware block order (chunks of 64, 4 and 1 row blocks; wave and block per row)
+                                               (1, 2, 6144, 2560, "holes"), (1, 2, 5888, 2560, "holes"), (1, 2, 5792, 2560, "holes"),
+                                               (1, 2, 3840, 4096, "causal"),
                                                # rows that are not whole vectors (prompts of 1001, 333, 13 tokens): the span kernel
                                                (1, 4, 1001, 1001, "causal"), (2, 3, 333, 333, "causal4"), (1, 2, 5, 13, "causal"),
                                                (2, 2, 9, 1004, "per_batch"), (1, 3, 1, 2047, None), (1, 2, 3, 4101, "causal"),
