@@ -231,6 +231,73 @@ __global__ void __launch_bounds__(BLOCK) norm_via32_wave_kernel(const T* __restr
     }
 }
 
+// RW rows per wave (or per block, LANES == BLOCK): the f32 weights are twice the bytes of a 16-bit row (four times with a
+// bias), and every row fetches them again, behind its reduction, where only the other waves hide the wait
+// ([16384,4096] LayerNorm 52.8 us; without the weight loads 46.1 us; a copy of the same bytes 42.9 us).  With RW rows in
+// registers the weights of a vector are loaded once and applied RW times.  The launcher says where that pays.
+template <typename T, int NV, int KIND, int LANES, int RW>
+__global__ void __launch_bounds__(BLOCK) norm_via32_rows_kernel(const T* __restrict__ x, const float* __restrict__ scale,
+                                                                const float* __restrict__ bias, T* __restrict__ y, uint64_t rows,
+                                                                uint32_t cols, float eps) {
+    const uint64_t row0 = ((uint64_t)blockIdx.x * (BLOCK / LANES) + (threadIdx.x / LANES)) * RW;
+    if (row0 >= rows) return;
+    const int lane = threadIdx.x & (LANES - 1);
+    const uint32_t nvec = cols / 8;
+    Vec16<T> v[RW][NV];
+#pragma unroll
+    for (int r = 0; r < RW; r++) {
+        // a row past the end reads the last row once more (its result is not stored): no branch around the loads
+        const uint64_t row = row0 + r < rows ? row0 + r : rows - 1;
+        const v4u* xr = reinterpret_cast<const v4u*>(x + row * cols);
+#pragma unroll
+        for (int k = 0; k < NV; k++) {
+            const uint32_t i = lane + k * LANES;
+            if (i < nvec) v[r][k].u = ld_stream(xr + i);
+        }
+    }
+    RowStats<float> st[RW];
+#pragma unroll
+    for (int r = 0; r < RW; r++) {
+        float sx = 0.0f, sq = 0.0f;
+#pragma unroll
+        for (int k = 0; k < NV; k++)
+            if (lane + k * LANES < nvec)
+#pragma unroll
+                for (int q = 0; q < 8; q++) {
+                    const float e = Ar<T>::widen(v[r][k].e[q]);
+                    if (KIND == NORM_LAYER) sx += e;
+                    sq += e * e;
+                }
+        if (KIND == NORM_LAYER) sx = row_sum<LANES>(sx);
+        sq = row_sum<LANES>(sq);
+        st[r] = finish_stats<float, KIND>(sx, sq, cols, eps);
+    }
+    const float4* sv = reinterpret_cast<const float4*>(scale);
+    const float4* bv = reinterpret_cast<const float4*>(bias);
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        const uint32_t i = lane + k * LANES;
+        if (i < nvec) {
+            float s[8], b[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            *reinterpret_cast<float4*>(s) = sv[2 * i];
+            *reinterpret_cast<float4*>(s + 4) = sv[2 * i + 1];
+            if (KIND == NORM_LAYER && bias) {
+                *reinterpret_cast<float4*>(b) = bv[2 * i];
+                *reinterpret_cast<float4*>(b + 4) = bv[2 * i + 1];
+            }
+#pragma unroll
+            for (int r = 0; r < RW; r++) {
+                if (row0 + r >= rows) break;
+                Vec16<T> o;
+#pragma unroll
+                for (int q = 0; q < 8; q++)
+                    o.e[q] = Ar<T>::conv(norm_one<float, KIND>(Ar<T>::widen(v[r][k].e[q]), st[r], s[q], b[q], bias != nullptr));
+                st_stream(reinterpret_cast<v4u*>(y + (row0 + r) * cols) + i, o.u);
+            }
+        }
+    }
+}
+
 // any cols / alignment: one block per row, scalar accesses, the row is re-read from cache for the second pass
 template <typename T, int KIND>
 __global__ void __launch_bounds__(BLOCK) norm_via32_generic_kernel(const T* __restrict__ x, const float* __restrict__ scale,
@@ -1488,15 +1555,28 @@ int launch_norm_via32(rt_device* dev, const void* x, const float* scale, const f
     }
     if (vec_ok && nvec <= (uint32_t)(WAVE * 8)) {
         const uint32_t nv = (nvec + WAVE - 1) / WAVE;
-        const uint64_t blocks = (rows + WAVES - 1) / WAVES;
+        // LayerNorm over 16384 rows or more: a wave takes two rows and loads the weights once for both (measured against one
+        // row a wave: [32768,2048] 49.5 against 51.8 us, [16384,3072] 39.2 against 41.9, [65536,512] 25.2 against 27.1; with fewer
+        // rows the chip is not covered often enough for the fatter waves, [8192,4096] 30.5 against 28.8; four rows a wave
+        // win on some shapes and lose on others; RMSNorm, with half the weights, gains nothing at any size)
+        const int rw = KIND == NORM_LAYER && rows >= (uint64_t)dev->num_cus * 64 ? 2 : 1;
+        const uint64_t blocks = ((rows + rw - 1) / rw + WAVES - 1) / WAVES;
         RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_norm_via_f32: too many rows");
         const dim3 grid((unsigned)blocks), block(BLOCK);
-#define RT_NV(NVC) hipLaunchKernelGGL((norm_via32_wave_kernel<T, NVC, KIND, WAVE>), grid, block, 0, dev->stream, (const T*)x, scale, bias, (T*)y, rows, cols, eps)
-        if (nv <= 1) RT_NV(1);
-        else if (nv <= 2) RT_NV(2);
-        else if (nv <= 4) RT_NV(4);
-        else if (nv <= 6) RT_NV(6);
-        else RT_NV(8);
+#define RT_NV(NVC, RWC) hipLaunchKernelGGL((norm_via32_rows_kernel<T, NVC, KIND, WAVE, RWC>), grid, block, 0, dev->stream, (const T*)x, scale, bias, (T*)y, rows, cols, eps)
+#define RT_NV1(NVC) hipLaunchKernelGGL((norm_via32_wave_kernel<T, NVC, KIND, WAVE>), grid, block, 0, dev->stream, (const T*)x, scale, bias, (T*)y, rows, cols, eps)
+#define RT_NV_RW2(NVC)               \
+    do {                             \
+        if (rw == 2) RT_NV(NVC, 2);  \
+        else RT_NV1(NVC);            \
+    } while (0)
+        if (nv <= 1) RT_NV_RW2(1);
+        else if (nv <= 2) RT_NV_RW2(2);
+        else if (nv <= 4) RT_NV_RW2(4);
+        else if (nv <= 6) RT_NV_RW2(6);
+        else RT_NV_RW2(8);
+#undef RT_NV_RW2
+#undef RT_NV1
 #undef RT_NV
         RT_CHECK_LAUNCH("norm_via32_wave_kernel");
         return RT_OK;
@@ -1504,12 +1584,23 @@ int launch_norm_via32(rt_device* dev, const void* x, const float* scale, const f
     if (vec_ok) {
         const uint32_t nv = (nvec + BLOCK - 1) / BLOCK;
         RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "rt_norm_via_f32: too many rows");
-        const dim3 grid((unsigned)rows), block(BLOCK);
-#define RT_NV(NVC) hipLaunchKernelGGL((norm_via32_wave_kernel<T, NVC, KIND, BLOCK>), grid, block, 0, dev->stream, (const T*)x, scale, bias, (T*)y, rows, cols, eps)
-        if (nv <= 3) RT_NV(3);
-        else if (nv <= 4) RT_NV(4);
-        else if (nv <= 6) RT_NV(6);
-        else RT_NV(8);
+        // LayerNorm over 2048 rows or more: a block takes two rows and loads the weights once for both ([2048,8192] 12.7 against
+        // 17.2 us, [8192,5120] 35.5 against 38.5, [16384,8192] 99 against 115; RMSNorm gains nothing)
+        const int rw = KIND == NORM_LAYER && rows >= (uint64_t)dev->num_cus * 8 ? 2 : 1;
+        const dim3 grid((unsigned)((rows + rw - 1) / rw)), block(BLOCK);
+#define RT_NV(NVC, RWC) hipLaunchKernelGGL((norm_via32_rows_kernel<T, NVC, KIND, BLOCK, RWC>), grid, block, 0, dev->stream, (const T*)x, scale, bias, (T*)y, rows, cols, eps)
+#define RT_NV1(NVC) hipLaunchKernelGGL((norm_via32_wave_kernel<T, NVC, KIND, BLOCK>), grid, block, 0, dev->stream, (const T*)x, scale, bias, (T*)y, rows, cols, eps)
+#define RT_NV_RW2(NVC)               \
+    do {                             \
+        if (rw == 2) RT_NV(NVC, 2);  \
+        else RT_NV1(NVC);            \
+    } while (0)
+        if (nv <= 3) RT_NV_RW2(3);
+        else if (nv <= 4) RT_NV_RW2(4);
+        else if (nv <= 6) RT_NV_RW2(6);
+        else RT_NV_RW2(8);
+#undef RT_NV_RW2
+#undef RT_NV1
 #undef RT_NV
         RT_CHECK_LAUNCH("norm_via32_wave_kernel");
         return RT_OK;

@@ -89,7 +89,10 @@ def test_gated_mul_matches_the_op_sequence(dev, oracle, shape, split):
 
 @pytest.mark.parametrize("kind", ["layer", "rms"])
 @pytest.mark.parametrize("rows,cols", [(64, 2560), (100, 3072), (257, 384), (9, 4096), (5, 1000), (3, 77), (2, 8192), (3, 5120), (2, 16384),
-                                       (2, 16392)])
+                                       (2, 16392),
+                                       # enough rows that a LayerNorm wave (a block, beyond 4096 columns) takes two of them and loads the
+                                       # weights once for both; odd row counts leave the last one a row short
+                                       (32771, 512), (16385, 1536), (16385, 3072), (16387, 4096), (2049, 8192), (4099, 5120)])
 def test_norm_via_f32(dev, oracle, kind, rows, cols):
     rng = np.random.default_rng(503)
     x = (randn(rng, (rows, cols), np.float16) * np.float16(3) + np.float16(0.5)).astype(np.float16)
