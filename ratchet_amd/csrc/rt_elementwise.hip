@@ -8,6 +8,7 @@
 
 #include "rt_arith.h"
 #include "rt_internal.h"
+#include "rt_pace.h"
 
 namespace {
 
@@ -237,9 +238,43 @@ __device__ __forceinline__ uint32_t lut_pair(const uint16_t* lut, uint32_t w) {
 // and an LDS-bound phase and pays for both.  One vector per thread and tile (16 KiB tiles, three in flight) measured
 // best inside the benchmark step: GELU on 84 MB 20.4 -> 18.3 us, SiLU on 134 MB 27.6 -> 25.0 us against 64 KiB tiles
 // with one in flight (depths 2 to 5 are level; 32 and 64 KiB tiles at any depth gain on the first only).
+// Large tensors: every wave holds its steps to a period (rt_pace.h); the blocks start out of phase.  pace == 0: unpaced.
+// On 16-bit GELU: 1 GiB 205 -> 173 us (a copy: 163), 512 MiB 100 -> 90 (83), 256 MiB 50 -> 49; on 128 MiB and below the
+// kernel is over before a pace can help and loses 2 us to it, so the unary launcher paces from 32 steps per block on.  The
+// gated multiply (three streams, 48 KiB a step): [32768,8192] 271 -> 252 us (a copy of as many bytes: 247), [16384,11008]
+// 181 -> 172 (167), [16384,8192] 133.5 -> 129.6, but [8192,8192], 32 steps, 66.5 -> 69.2: paced from 64 steps on.
+struct LutPace {
+    uint32_t pace;           // ticks of the wall clock between two steps of a block
+    uint32_t phase_fx;       // pace / grid in 16.16 fixed point
+};
+constexpr uint32_t LUT_PACE_MIN_STEPS = 32, GATED_PACE_MIN_STEPS = 64;
+struct LutClock {
+    uint32_t t_step = 0, t_last = 0, t_avg = 0, t_slow = 0;
+    __device__ __forceinline__ explicit LutClock(const LutPace& pc) {
+        if (pc.pace) {
+            t_avg = pc.pace;
+            t_slow = pc.pace + pc.pace / 5;
+            t_last = __builtin_amdgcn_readfirstlane(rt_pace_clock());
+            t_step = t_last - pc.pace + ((blockIdx.x * pc.phase_fx) >> 16);
+            t_last -= pc.pace;
+        }
+    }
+    __device__ __forceinline__ void step(const LutPace& pc) {
+        if (pc.pace) rt_pace_step(t_step, t_last, t_avg, pc.pace, t_slow);
+    }
+};
+static LutPace lut_pace_for(const rt_device* dev, uint64_t blocks, uint64_t steps_per_block, uint32_t min_steps, double bytes_per_step) {
+    LutPace pc = {0, 0};
+    if (blocks == (uint64_t)dev->num_cus && steps_per_block >= min_steps) {
+        pc.pace = (uint32_t)(bytes_per_step * (double)blocks / RT_PACE_BYTES_PER_S * dev->wall_clock_hz + 0.5);
+        pc.phase_fx = pc.pace > 0xffffu ? 0 : (pc.pace << 16) / (uint32_t)blocks;
+    }
+    return pc;
+}
+
 template <int U, int D>
 __global__ void __launch_bounds__(LUT_BLOCK) unary_lut_kernel(const uint16_t* __restrict__ table, const uint16_t* __restrict__ x,
-                                                                   uint16_t* y, uint64_t numel) {
+                                                                   uint16_t* y, uint64_t numel, LutPace pc) {
     extern __shared__ __attribute__((aligned(16))) uint16_t lut[];
     constexpr int TILE = LUT_BLOCK * U;
     const uint64_t nvec = numel / 8;
@@ -263,10 +298,12 @@ __global__ void __launch_bounds__(LUT_BLOCK) unary_lut_kernel(const uint16_t* __
         for (int i = 0; i < (int)(LUT_BYTES / 16 / LUT_BLOCK); i++) dst[i * LUT_BLOCK + threadIdx.x] = src[i * LUT_BLOCK + threadIdx.x];
     }
     __syncthreads();
+    LutClock clk(pc);
     while (t < tiles) {
 #pragma unroll
         for (int d = 0; d < D; d++) {
             if (t >= tiles) break;
+            clk.step(pc);
             v4u cur[U];
 #pragma unroll
             for (int k = 0; k < U; k++) cur[k] = ring[d][k];
@@ -313,7 +350,7 @@ struct GatedArgs {
 // flight during the lookups of the current one and those of the first steps during the table copy.
 template <typename T>
 __global__ void __launch_bounds__(LUT_BLOCK) gated_lut_kernel(const uint16_t* __restrict__ table, const T* __restrict__ gate,
-                                                              const T* __restrict__ up, T* __restrict__ y, GatedArgs p) {
+                                                              const T* __restrict__ up, T* __restrict__ y, GatedArgs p, LutPace pc) {
     extern __shared__ __attribute__((aligned(16))) uint16_t lut[];
     const uint64_t stride = (uint64_t)gridDim.x * LUT_BLOCK;
     uint64_t v = (uint64_t)blockIdx.x * LUT_BLOCK + threadIdx.x;
@@ -334,25 +371,33 @@ __global__ void __launch_bounds__(LUT_BLOCK) gated_lut_kernel(const uint16_t* __
         for (int i = 0; i < (int)(LUT_BYTES / 16 / LUT_BLOCK); i++) dst[i * LUT_BLOCK + threadIdx.x] = src[i * LUT_BLOCK + threadIdx.x];
     }
     __syncthreads();
-    while (v < p.nvec) {
+    LutClock clk(pc);
+    // the loop runs on the index of the wave's first lane, which is the same for the whole wave (the clock lives in scalar
+    // registers); only the wave that holds the tensor's end has lanes without an element
+    uint64_t v0 = (uint64_t)blockIdx.x * LUT_BLOCK + __builtin_amdgcn_readfirstlane(threadIdx.x & ~63u);
+    while (v0 < p.nvec) {
 #pragma unroll
         for (int d = 0; d < LUT_DEPTH; d++) {
-            if (v >= p.nvec) break;
-            Vec16<T> g, u, o;
-            g.u = rg[d];
-            u.u = ru[d];
-            const uint64_t vn = v + LUT_DEPTH * stride;
-            if (vn < p.nvec) fetch(vn, rg[d], ru[d]);
+            if (v0 >= p.nvec) break;
+            clk.step(pc);
+            if (v < p.nvec) {
+                Vec16<T> g, u, o;
+                g.u = rg[d];
+                u.u = ru[d];
+                const uint64_t vn = v + LUT_DEPTH * stride;
+                if (vn < p.nvec) fetch(vn, rg[d], ru[d]);
 #pragma unroll
-            for (int w = 0; w < 4; w++) {
-                const uint32_t lo = lut[g.u[w] & 0xffffu];
-                const uint32_t hi = lut[g.u[w] >> 16];
-                g.u[w] = lo | (hi << 16);
+                for (int w = 0; w < 4; w++) {
+                    const uint32_t lo = lut[g.u[w] & 0xffffu];
+                    const uint32_t hi = lut[g.u[w] >> 16];
+                    g.u[w] = lo | (hi << 16);
+                }
+#pragma unroll
+                for (int e = 0; e < 8; e++) o.e[e] = Ar<T>::mul(u.e[e], g.e[e]);
+                st_stream(reinterpret_cast<v4u*>(y) + v, o.u);
             }
-#pragma unroll
-            for (int e = 0; e < 8; e++) o.e[e] = Ar<T>::mul(u.e[e], g.e[e]);
-            st_stream(reinterpret_cast<v4u*>(y) + v, o.u);
             v += stride;
+            v0 += stride;
         }
     }
 }
@@ -575,9 +620,10 @@ template <typename T, bool VIA32 = false> int unary_via_lut(rt_device* dev, int 
     uint64_t blocks = (numel / 8 + LUT_TILE - 1) / LUT_TILE;
     if (blocks > (uint64_t)dev->num_cus) blocks = dev->num_cus;          // one resident block per CU (128 KiB of LDS each)
     if (blocks < 1) blocks = 1;
+    const LutPace pc = lut_pace_for(dev, blocks, numel / 8 / LUT_TILE / blocks, LUT_PACE_MIN_STEPS, (double)LUT_TILE * 16 * 2);
     hipLaunchKernelGGL((unary_lut_kernel<LUT_UNROLL, LUT_DEPTH>), dim3((unsigned)blocks), dim3(LUT_BLOCK), LUT_BYTES, dev->stream,
                        (const uint16_t*)(VIA32 ? dev->unary_lut_via32[ti][op] : dev->unary_lut[ti][op]), (const uint16_t*)x,
-                       (uint16_t*)y, numel);
+                       (uint16_t*)y, numel, pc);
     RT_CHECK_LAUNCH("unary_lut_kernel");
     return RT_OK;
 }
@@ -638,8 +684,9 @@ int launch_gated(rt_device* dev, int op, const void* gate, uint64_t gs, const vo
         p.nvec = numel / 8;
         uint64_t blocks = (p.nvec + LUT_BLOCK - 1) / LUT_BLOCK;
         if (blocks > (uint64_t)dev->num_cus) blocks = dev->num_cus;
+        const LutPace pc = lut_pace_for(dev, blocks, p.nvec / LUT_BLOCK / blocks, GATED_PACE_MIN_STEPS, (double)LUT_BLOCK * 16 * 3);
         hipLaunchKernelGGL((gated_lut_kernel<T>), dim3((unsigned)blocks), dim3(LUT_BLOCK), LUT_BYTES, dev->stream,
-                           (const uint16_t*)dev->unary_lut_via32[ti][op], (const T*)gate, (const T*)up, (T*)y, p);
+                           (const uint16_t*)dev->unary_lut_via32[ti][op], (const T*)gate, (const T*)up, (T*)y, p, pc);
         RT_CHECK_LAUNCH("gated_lut_kernel");
         return RT_OK;
     }

@@ -6,6 +6,7 @@
 
 #include "rt_arith.h"
 #include "rt_internal.h"
+#include "rt_pace.h"
 
 namespace {
 
@@ -45,7 +46,6 @@ constexpr int SP_TC = 512;                   // columns per step: 64 lanes x 8 h
 constexpr int SP_PAD = 8;
 constexpr int SP_PF = 2;                     // steps loaded ahead
 constexpr int SP_MAX_STEPS = 8;              // rows of up to 4096 columns
-constexpr double SP_PACE_BYTES_PER_S = 6.65e12;   // what the paced kernel asks of HBM, all blocks together (measured optimum 6.6-6.7e12)
 constexpr size_t SP_LUT_BYTES = 65536 * sizeof(uint16_t);
 constexpr size_t SP_TILE_BYTES = SP_ROWS * (SP_TC + SP_PAD) * sizeof(uint16_t);
 constexpr size_t SP_SMEM_BYTES = SP_LUT_BYTES + SP_TILE_BYTES + 2 * 32 * sizeof(uint16_t);      // 162 400 of the CU's 163 840 bytes
@@ -57,59 +57,6 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 // exp of two packed f16 bit patterns: two lookups in the full 65536-entry table (NaN, inf and the saturated ends included)
 __device__ __forceinline__ uint32_t sp_exp_pair(const uint16_t* lut, uint32_t p) {
     return (uint32_t)lut[p & 0xffffu] | ((uint32_t)lut[p >> 16] << 16);
-}
-
-// the 100 MHz wall clock (low 32 bits), read as one opaque block so that it does not take part in the scheduling of the
-// code around it
-__device__ __forceinline__ uint32_t sp_clock() {
-    uint64_t t;
-    asm volatile("s_memrealtime %0\n s_waitcnt lgkmcnt(0)" : "=s"(t) :: "memory");
-    return (uint32_t)t;
-}
-
-// The block's schedule: a step may not start before `pace` ticks of the wall clock have passed since the one before
-// was allowed to (t_step): a wave that arrives early waits, and a late one goes on at once and the schedule starts
-// again from its arrival, so that a step which was late is not followed by a burst (it is the bursts that overload
-// HBM).  Inputs whose steps are longer than the pace for reasons of their own (dense scores: the table lookups collide
-// in the LDS banks) must not be held at all, because their short steps would be delayed and their long ones not made up
-// for: the wave keeps a running average of the time between its steps (`avg`, a quarter of each new value), and while
-// that is above 1.2 paces it only keeps time.  A wait ends after 4096 looks at the clock at the latest (a step is a few
-// hundred ticks, a look takes several), so the kernel finishes whatever the clock does.  Everything is in scalar registers and in one asm statement: written as
-// C++ the loop changed the register allocation and instruction order of the whole kernel, loader waves included.
-__device__ __forceinline__ void sp_pace_step(uint32_t& t_step, uint32_t& t_last, uint32_t& avg, uint32_t pace, uint32_t slow) {
-    asm volatile(
-        "s_memrealtime s[96:97]\n"
-        "s_waitcnt lgkmcnt(0)\n"
-        "s_sub_u32 s98, s96, %1\n"              // time since the previous step
-        "s_mov_b32 %1, s96\n"
-        "s_sub_u32 s98, s98, %2\n"
-        "s_ashr_i32 s98, s98, 2\n"
-        "s_add_u32 %2, %2, s98\n"               // avg += (dt - avg) / 4
-        "s_cmp_ge_i32 %2, %4\n"
-        "s_cbranch_scc1 2f\n"                   // steps are slow by themselves: only keep time
-        "s_sub_u32 s98, s96, %0\n"              // ticks since the last permitted start
-        "s_cmp_ge_i32 s98, %3\n"
-        "s_cbranch_scc1 2f\n"                   // late or on time
-        "s_movk_i32 s99, 0x1000\n"
-        "1:\n"
-        "s_sleep 1\n"                           // early: wait for the step's time
-        "s_memrealtime s[96:97]\n"
-        "s_waitcnt lgkmcnt(0)\n"
-        "s_sub_u32 s99, s99, 1\n"
-        "s_cmp_eq_u32 s99, 0\n"
-        "s_cbranch_scc1 2f\n"                   // 4096 looks at a clock that does not get there: stop waiting for it
-        "s_sub_u32 s98, s96, %0\n"
-        "s_cmp_ge_i32 s98, %3\n"
-        "s_cbranch_scc0 1b\n"
-        "s_add_u32 %0, %0, %3\n"                // started exactly on schedule
-        "s_mov_b32 %1, s96\n"
-        "s_branch 3f\n"
-        "2:\n"
-        "s_mov_b32 %0, s96\n"                   // the schedule starts again from this arrival
-        "3:\n"
-        : "+s"(t_step), "+s"(t_last), "+s"(avg)
-        : "s"(pace), "s"(slow)
-        : "s96", "s97", "s98", "s99", "scc", "memory");
 }
 
 // Which 30-row groups a block works on.  Rows come in `reps` periods of P rows (P = all rows when nothing repeats; P = the
@@ -269,7 +216,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
         // the blocks take their steps out of phase with each other: block b starts b / grid of a step late
         uint32_t t_step = 0, t_last = 0, t_avg = sch.pace, t_slow = sch.pace + sch.pace / 5;
         if constexpr (PACED) {
-            t_last = __builtin_amdgcn_readfirstlane(sp_clock());
+            t_last = __builtin_amdgcn_readfirstlane(rt_pace_clock());
             t_step = t_last - sch.pace + ((blockIdx.x * sch.phase_fx) >> 16);
             t_last -= sch.pace;
         }
@@ -302,7 +249,7 @@ __global__ void __launch_bounds__(SP_BLOCK) softmax16_stream_kernel(const uint16
             }
 #pragma unroll 1
             for (uint32_t t = 0; t < nsteps; t++) {
-                if (PACED && sch.pace) sp_pace_step(t_step, t_last, t_avg, sch.pace, t_slow);   // the walker is the block's clock
+                if (PACED && sch.pace) rt_pace_step(t_step, t_last, t_avg, sch.pace, t_slow);   // the walker is the block's clock
                 __syncthreads();                             // A
                 __syncthreads();                             // B: tile t is in LDS
                 // 16 values per chunk; the LDS reads of the next chunk are in flight during the 16 dependent adds
@@ -1010,13 +957,13 @@ int launch_stream16(rt_device* dev, const void* x, const void* mask, uint64_t pe
         // what it gets when it asks for slightly less: 366 us unpaced against 345-350 us on [1,32,4096,4096] in the
         // benchmark step (a plain persistent copy loop shows the same: 5.9 TB/s unpaced, 6.4 TB/s with a sleep of the
         // right length per iteration, and a write-only loop 4.4 against 6.6 TB/s).  So the walker holds the block's
-        // steps to the period at which all blocks together move SP_PACE_BYTES_PER_S, by the device's wall clock, and the
+        // steps to the period at which all blocks together move RT_PACE_BYTES_PER_S, by the device's wall clock, and the
         // blocks start out of phase (sp_pace_step).  A pace that is too fast gives the unpaced behaviour back (7.0e12:
         // 359 us), one that is too slow costs in proportion (6.4e12: 355 us).  Paced are, on a grid that fills the
         // chip, the plain variant and the masked one that takes one mask row per pair of heads (at the same rate: 6.4e12
         // costs that one 3 us, 6.8e12 and 7.0e12 leave 5 us of its dependence on where the buffers lie).
         if (blocks == dev->num_cus && !ragged && (!mask || pair)) {
-            const double rate = SP_PACE_BYTES_PER_S;
+            const double rate = RT_PACE_BYTES_PER_S;
             const double group_bytes = (double)sch.R * rmul * cols * 2 * (nt > SP_MAX_STEPS ? 4 : 2);     // in and out (long rows: parked and read back)
             const double steps = nt > SP_MAX_STEPS ? sch.nsteps : nt == 7 ? 8 : nt;          // the steps the kernel variant takes per group
             sch.pace = (uint32_t)(group_bytes / steps * blocks / rate * dev->wall_clock_hz + 0.5);
