@@ -348,7 +348,7 @@ struct GatedArgs {
 
 // Like unary_lut_kernel: one vector of gate and one of up per thread and step, the loads of the next LUT_DEPTH steps in
 // flight during the lookups of the current one and those of the first steps during the table copy.
-template <typename T>
+template <typename T, bool PACED>
 __global__ void __launch_bounds__(LUT_BLOCK) gated_lut_kernel(const uint16_t* __restrict__ table, const T* __restrict__ gate,
                                                               const T* __restrict__ up, T* __restrict__ y, GatedArgs p, LutPace pc) {
     extern __shared__ __attribute__((aligned(16))) uint16_t lut[];
@@ -371,9 +371,33 @@ __global__ void __launch_bounds__(LUT_BLOCK) gated_lut_kernel(const uint16_t* __
         for (int i = 0; i < (int)(LUT_BYTES / 16 / LUT_BLOCK); i++) dst[i * LUT_BLOCK + threadIdx.x] = src[i * LUT_BLOCK + threadIdx.x];
     }
     __syncthreads();
+    if constexpr (!PACED) {
+        while (v < p.nvec) {
+#pragma unroll
+            for (int d = 0; d < LUT_DEPTH; d++) {
+                if (v >= p.nvec) break;
+                Vec16<T> g, u, o;
+                g.u = rg[d];
+                u.u = ru[d];
+                const uint64_t vn = v + LUT_DEPTH * stride;
+                if (vn < p.nvec) fetch(vn, rg[d], ru[d]);
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    const uint32_t lo = lut[g.u[w] & 0xffffu];
+                    const uint32_t hi = lut[g.u[w] >> 16];
+                    g.u[w] = lo | (hi << 16);
+                }
+#pragma unroll
+                for (int e = 0; e < 8; e++) o.e[e] = Ar<T>::mul(u.e[e], g.e[e]);
+                st_stream(reinterpret_cast<v4u*>(y) + v, o.u);
+                v += stride;
+            }
+        }
+        return;
+    }
     LutClock clk(pc);
-    // the loop runs on the index of the wave's first lane, which is the same for the whole wave (the clock lives in scalar
-    // registers); only the wave that holds the tensor's end has lanes without an element
+    // paced: the loop runs on the index of the wave's first lane, which is the same for the whole wave (the clock lives in
+    // scalar registers); only the wave that holds the tensor's end has lanes without an element
     uint64_t v0 = (uint64_t)blockIdx.x * LUT_BLOCK + __builtin_amdgcn_readfirstlane(threadIdx.x & ~63u);
     while (v0 < p.nvec) {
 #pragma unroll
@@ -676,7 +700,9 @@ int launch_gated(rt_device* dev, int op, const void* gate, uint64_t gs, const vo
         int rc = build_unary_table<T, true>(dev, ti, op);
         if (rc) return rc;
         if (!dev->gated_attr_set[ti]) {
-            RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gated_lut_kernel<T>), hipFuncAttributeMaxDynamicSharedMemorySize,
+            RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gated_lut_kernel<T, false>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)LUT_BYTES));
+            RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gated_lut_kernel<T, true>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)LUT_BYTES));
             dev->gated_attr_set[ti] = 1;
         }
@@ -685,8 +711,13 @@ int launch_gated(rt_device* dev, int op, const void* gate, uint64_t gs, const vo
         uint64_t blocks = (p.nvec + LUT_BLOCK - 1) / LUT_BLOCK;
         if (blocks > (uint64_t)dev->num_cus) blocks = dev->num_cus;
         const LutPace pc = lut_pace_for(dev, blocks, p.nvec / LUT_BLOCK / blocks, GATED_PACE_MIN_STEPS, (double)LUT_BLOCK * 16 * 3);
-        hipLaunchKernelGGL((gated_lut_kernel<T>), dim3((unsigned)blocks), dim3(LUT_BLOCK), LUT_BYTES, dev->stream,
-                           (const uint16_t*)dev->unary_lut_via32[ti][op], (const T*)gate, (const T*)up, (T*)y, p, pc);
+        if (pc.pace) {
+            hipLaunchKernelGGL((gated_lut_kernel<T, true>), dim3((unsigned)blocks), dim3(LUT_BLOCK), LUT_BYTES, dev->stream,
+                               (const uint16_t*)dev->unary_lut_via32[ti][op], (const T*)gate, (const T*)up, (T*)y, p, pc);
+        } else {
+            hipLaunchKernelGGL((gated_lut_kernel<T, false>), dim3((unsigned)blocks), dim3(LUT_BLOCK), LUT_BYTES, dev->stream,
+                               (const uint16_t*)dev->unary_lut_via32[ti][op], (const T*)gate, (const T*)up, (T*)y, p, pc);
+        }
         RT_CHECK_LAUNCH("gated_lut_kernel");
         return RT_OK;
     }
