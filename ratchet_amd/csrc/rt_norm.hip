@@ -1281,6 +1281,7 @@ int norm_entry(rt_device* dev, int kind, int dt, const void* x, const void* scal
 // come from LDS.  Same definitions as the two-kernel path (mean, then the variance about that mean, f32 arithmetic).
 constexpr int GN_LDS_BLOCK = 1024;
 constexpr size_t GN_LDS_MAX_BYTES = 144 * 1024;
+constexpr size_t GN_REG_MAX_BYTES = 16 * 1024 * 16;           // what gn_reg_kernel holds without spilling: 16 vectors in each of 1024 threads
 
 template <typename T>
 __global__ void __launch_bounds__(GN_LDS_BLOCK) gn_lds_kernel(const T* __restrict__ x, const T* __restrict__ scale, const T* __restrict__ bias,
@@ -1370,6 +1371,13 @@ __global__ void __launch_bounds__(GN_LDS_BLOCK) gn_reg_kernel(const T* __restric
         for (int q = 0; q < VE; q++) acc += Ar<T>::widen(v[k].e[q]);         // vectors past the group hold zeros
     }
     const float mean = row_sum<GN_LDS_BLOCK>(acc) / (float)glen;
+    // the group stays in registers as it was loaded; the widened values of one pass are not kept for the next (with 16 and
+    // more vectors a thread the compiler otherwise keeps them and spills)
+    auto forget = [&]() {
+#pragma unroll
+        for (int k = 0; k < NV; k++) asm volatile("" : "+v"(v[k].u[0]), "+v"(v[k].u[1]), "+v"(v[k].u[2]), "+v"(v[k].u[3]));
+    };
+    forget();
     float m2 = 0.0f;
 #pragma unroll
     for (int k = 0; k < NV; k++) {
@@ -1382,6 +1390,7 @@ __global__ void __launch_bounds__(GN_LDS_BLOCK) gn_reg_kernel(const T* __restric
         }
     }
     const float var = row_sum<GN_LDS_BLOCK>(m2) / (float)glen;
+    forget();
     const float rstd = 1.0f / __builtin_sqrtf(var + eps);
     const uint32_t lo = (uint32_t)(((uint64_t)nvec * slice) / slices), hi = (uint32_t)(((uint64_t)nvec * (slice + 1)) / slices);
 #pragma unroll
@@ -1453,9 +1462,17 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
     if (splits < 1) splits = 1;
     constexpr int VEMAX = 16 / sizeof(T);
     const bool vec = (L % VEMAX == 0) && rt_aligned(x, 16) && rt_aligned(y, 16);       // then glen % VEMAX == 0 too
-    if (vec && (size_t)glen * sizeof(T) <= GN_LDS_MAX_BYTES && 2u * bg <= (uint32_t)dev->num_cus) {
+    // groups that a 1024-thread block holds in registers (up to 16 vectors a thread, 256 KiB; 20 and 24 spill and were slower
+    // than the three-launch path): few of them (fewer pairs than half the CUs) up to that size, or groups too large for the
+    // LDS kernel below in up to eight rounds of blocks ([8,512,3000] f32, 256 groups of 187 KiB: 33.7 -> 20.3 us; [1,512,3000] f32
+    // 9.1 us, [2,640,4096] f16, 64 groups of 160 KiB, 12.4 us)
+    const bool reg_few = (size_t)glen * sizeof(T) <= GN_REG_MAX_BYTES && 2u * bg <= (uint32_t)dev->num_cus;
+    const bool reg_large = (size_t)glen * sizeof(T) > GN_LDS_MAX_BYTES && (size_t)glen * sizeof(T) <= GN_REG_MAX_BYTES &&
+                           bg <= 8u * (uint32_t)dev->num_cus;
+    if (vec && (reg_few || reg_large)) {
         // few groups: several blocks per group, each reducing the whole group and writing one slice of it
         uint32_t slices = (uint32_t)dev->num_cus / bg;
+        if (slices < 1) slices = 1;
         if (slices > 32) slices = 32;
         const uint32_t nvec = glen / VEMAX;
         if (slices > nvec) slices = nvec;
@@ -1473,7 +1490,9 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
         else if (nv <= 3) RT_GN_REG(3);
         else if (nv <= 4) RT_GN_REG(4);
         else if (nv <= 6) RT_GN_REG(6);
-        else RT_GN_REG(9);
+        else if (nv <= 9) RT_GN_REG(9);
+        else if (nv <= 12) RT_GN_REG(12);
+        else RT_GN_REG(16);
 #undef RT_GN_REG
         RT_CHECK_LAUNCH("gn_reg_kernel");
         return RT_OK;
