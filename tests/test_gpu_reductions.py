@@ -597,7 +597,10 @@ def test_layer_norm_f32_known_answer_rows_with_an_offset(dev, oracle):
                                      (9, 128, 40, 64),            # 576 groups: more than two per CU, the two-launch streaming path
                                      (1, 8, 40000, 2),            # groups larger than LDS
                                      (1, 4, 300000, 1),           # one group of 1.2 M elements: hundreds of slices, combined by a launch of their own
-                                     (2, 16, 24, 4)])
+                                     (2, 16, 24, 4),
+                                     (1, 64, 3000, 4),            # 4 groups of 96 KB (f16) / 187 KB (f32): 32 blocks per group, 6 / 12 vectors a thread
+                                     (2, 256, 4096, 16),          # 32 groups of 128 / 256 KB: up to 16 vectors a thread
+                                     (4, 576, 2040, 72)])         # 288 groups (one block each) of 32 / 64 KB f16/f32
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
 def test_group_norm(dev, oracle, B, C, L, G, dtype):
     rng = np.random.default_rng(320)
@@ -615,6 +618,18 @@ def test_group_norm(dev, oracle, B, C, L, G, dtype):
     assert bad == 0, (bad, mx)
     got = dev.group_norm(dev.upload(x), G, None, None, 1e-5).to_numpy()
     bad, mx = oracle.count_not_close(got, oracle.group_norm(x, G, None, None, 1e-5), tol, tol)
+    assert bad == 0, (bad, mx)
+
+
+def test_group_norm_many_groups_too_large_for_lds(dev, oracle):
+    """288 groups of 160 KB in f32 (more pairs than CUs, groups over what the LDS kernel stages): one block per group with the
+    group in registers, two rounds of blocks; against the oracle"""
+    rng = np.random.default_rng(323)
+    B, C, L, G = 9, 320, 4096, 32
+    x = randn(rng, (B, C, L), np.float32)
+    w, b = randn(rng, C, np.float32), randn(rng, C, np.float32)
+    got = dev.group_norm(dev.upload(x), G, dev.upload(w), dev.upload(b), 1e-5).to_numpy()
+    bad, mx = oracle.count_not_close(got, oracle.group_norm(x, G, w, b, 1e-5), 1e-5, 1e-5)
     assert bad == 0, (bad, mx)
 
 
