@@ -663,7 +663,7 @@ __global__ void __launch_bounds__(NP_BLOCK) norm_pipe16_kernel(const T* __restri
 // apply kernel: same grid; every block combines the group's partials (Chan et al.), then normalises its slice:
 //               y = (x - mean) * rstd * w[c] + b[c], f32 arithmetic, rounded to T once.
 // ------------------------------------------------------------------------------------------------------------------
-// VE = elements per access: 16 / sizeof(T) on the vector path (slices, L and base pointers are multiples of it), 1 otherwise
+// VE = elements per access: 16 / sizeof(T) on the vector path (slices, groups and base pointers are multiples of it), 1 otherwise
 template <typename T, int VE>
 __global__ void __launch_bounds__(BLOCK) gn_stats_kernel(const T* __restrict__ x, float* __restrict__ part, uint32_t glen,
                                                          uint32_t chunk, uint32_t splits) {
@@ -724,6 +724,125 @@ __global__ void __launch_bounds__(BLOCK) gn_stats_kernel(const T* __restrict__ x
     }
 }
 
+// The same partials from a slice that the block's registers hold (NV vectors a thread): the slice is read once, with all
+// its loads in flight together, and the second pass runs on registers ([16,256,4096] f32, slices of 32 KiB: 49.7 -> 33.8 us for the two launches).
+template <typename T, int NV>
+__global__ void __launch_bounds__(BLOCK) gn_stats_reg_kernel(const T* __restrict__ x, float* __restrict__ part, uint32_t glen,
+                                                             uint32_t chunk, uint32_t splits) {
+    constexpr int VE = 16 / sizeof(T);
+    __shared__ float red[WAVES];
+    const uint32_t s = blockIdx.y, grp = blockIdx.x;
+    const uint32_t c0 = s * chunk;
+    const uint32_t c1 = (c0 + chunk < glen) ? c0 + chunk : glen;
+    const v4u* xs = reinterpret_cast<const v4u*>(x + (uint64_t)grp * glen + c0);
+    const uint32_t nvec = (c1 - c0) / VE;
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    Vec16<T> v[NV];
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        const uint32_t i = threadIdx.x + k * BLOCK;
+        v[k].u = v4u{0u, 0u, 0u, 0u};
+        if (i < nvec) v[k].u = xs[i];
+    }
+    float acc = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+#pragma unroll
+        for (int q = 0; q < VE; q++) acc += Ar<T>::widen(v[k].e[q]);             // vectors past the slice hold zeros
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) red[wave] = acc;
+    __syncthreads();
+    float t = 0.0f;
+#pragma unroll
+    for (int w = 0; w < WAVES; w++) t += red[w];
+    const float mean = t / (float)(c1 - c0);
+    float m2 = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        if (threadIdx.x + k * BLOCK < nvec) {
+#pragma unroll
+            for (int q = 0; q < VE; q++) {
+                const float d = Ar<T>::widen(v[k].e[q]) - mean;
+                m2 += d * d;
+            }
+        }
+    }
+    m2 = wave_sum(m2);
+    __syncthreads();
+    if (lane == 0) red[wave] = m2;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float u = 0.0f;
+        for (int w = 0; w < WAVES; w++) u += red[w];
+        float* o = part + ((uint64_t)grp * splits + s) * 3;
+        o[0] = mean;
+        o[1] = u;
+        o[2] = (float)(c1 - c0);
+    }
+}
+
+// y = (x - mean) * rstd * w[c] + b[c] for the VE elements of one vector that starts at element e0 of its group, whose first
+// channel is cbase.  With L a multiple of VE the vector lies in one channel; otherwise the channel is stepped element by
+// element (a vector of [.., 1500] f16 rows crosses into the next channel, with L < VE into several).
+template <typename T>
+__device__ __forceinline__ v4u gn_affine_vec(const Vec16<T>& v, uint32_t e0, uint32_t cbase, FastDiv L, const T* __restrict__ scale,
+                                             const T* __restrict__ bias, float mean, float rstd) {
+    constexpr int VE = 16 / sizeof(T);
+    Vec16<T> o;
+    const uint32_t ch = fd_div(e0, L);
+    uint32_t c = cbase + ch;
+    if (L.d % VE == 0) {
+        const float w = scale ? Ar<T>::widen(scale[c]) : 1.0f;
+        const float b = bias ? Ar<T>::widen(bias[c]) : 0.0f;
+#pragma unroll
+        for (int q = 0; q < VE; q++) {
+            const float t = (Ar<T>::widen(v.e[q]) - mean) * rstd;
+            o.e[q] = Ar<T>::conv(t * w + b);
+        }
+    } else {
+        uint32_t r = e0 - ch * L.d;
+#pragma unroll
+        for (int q = 0; q < VE; q++) {
+            const float w = scale ? Ar<T>::widen(scale[c]) : 1.0f;
+            const float b = bias ? Ar<T>::widen(bias[c]) : 0.0f;
+            const float t = (Ar<T>::widen(v.e[q]) - mean) * rstd;
+            o.e[q] = Ar<T>::conv(t * w + b);
+            if (++r == L.d) {
+                r = 0;
+                c++;
+            }
+        }
+    }
+    return o.u;
+}
+
+// Combines the partials of one group (Chan et al.) in double, by the first wave of the block: lane k takes partial k (the
+// launcher keeps splits <= 64 here), then a tree over the wave, in the same order in every block of the group.
+__device__ __forceinline__ void gn_combine_wave(const float* __restrict__ p, uint32_t splits, float eps, float& s_mean, float& s_rstd) {
+    if (threadIdx.x >= WAVE) return;
+    double n = 0.0, mean = 0.0, m2 = 0.0;
+    if (threadIdx.x < splits) {
+        mean = (double)p[3 * threadIdx.x];
+        m2 = (double)p[3 * threadIdx.x + 1];
+        n = (double)p[3 * threadIdx.x + 2];
+    }
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+        const double nb = __shfl_down(n, off), mb = __shfl_down(mean, off), m2b = __shfl_down(m2, off);
+        if (nb != 0.0) {
+            const double nt = n + nb;
+            const double delta = mb - mean;
+            mean += delta * (nb / nt);
+            m2 += m2b + delta * delta * (n * nb / nt);
+            n = nt;
+        }
+    }
+    if (threadIdx.x == 0) {
+        s_mean = (float)mean;
+        s_rstd = (float)(1.0 / sqrt(m2 / n + (double)eps));
+    }
+}
+
 template <typename T, int VE>
 __global__ void __launch_bounds__(BLOCK) gn_apply_kernel(const T* __restrict__ x, const T* __restrict__ scale,
                                                          const T* __restrict__ bias, T* __restrict__ y,
@@ -731,21 +850,7 @@ __global__ void __launch_bounds__(BLOCK) gn_apply_kernel(const T* __restrict__ x
                                                          uint32_t cpg, uint32_t groups, FastDiv L, float eps) {
     __shared__ float s_mean, s_rstd;
     const uint32_t s = blockIdx.y, grp = blockIdx.x;
-    if (threadIdx.x == 0) {
-        // combine the group's partials (Chan et al.) in double
-        double n = 0.0, mean = 0.0, m2 = 0.0;
-        const float* p = part + (uint64_t)grp * splits * 3;
-        for (uint32_t k = 0; k < splits; k++) {
-            const double nb = (double)p[3 * k + 2], mb = (double)p[3 * k], m2b = (double)p[3 * k + 1];
-            const double nt = n + nb;
-            const double delta = mb - mean;
-            mean += delta * (nb / nt);
-            m2 += m2b + delta * delta * (n * nb / nt);
-            n = nt;
-        }
-        s_mean = (float)mean;
-        s_rstd = (float)(1.0 / sqrt(m2 / n + (double)eps));
-    }
+    gn_combine_wave(part + (uint64_t)grp * splits * 3, splits, eps, s_mean, s_rstd);
     __syncthreads();
     const float meanf = s_mean, rstd = s_rstd;
     const uint32_t g = grp % groups;
@@ -754,21 +859,50 @@ __global__ void __launch_bounds__(BLOCK) gn_apply_kernel(const T* __restrict__ x
     const uint32_t c0 = s * chunk;
     const uint32_t c1 = (c0 + chunk < glen) ? c0 + chunk : glen;
     for (uint32_t i = c0 + threadIdx.x * VE; i < c1; i += BLOCK * VE) {
-        const uint32_t c = g * cpg + fd_div(i, L);                            // with VE > 1, L % VE == 0: one channel per vector
-        const float w = scale ? Ar<T>::widen(scale[c]) : 1.0f;
-        const float b = bias ? Ar<T>::widen(bias[c]) : 0.0f;
         if (VE > 1) {
-            Vec16<T> v, o;
+            Vec16<T> v;
             v.u = *reinterpret_cast<const v4u*>(xs + i);
-#pragma unroll
-            for (int q = 0; q < VE; q++) {
-                const float t = (Ar<T>::widen(v.e[q]) - meanf) * rstd;
-                o.e[q] = Ar<T>::conv(t * w + b);
-            }
-            st_stream(reinterpret_cast<v4u*>(ys + i), o.u);
+            st_stream(reinterpret_cast<v4u*>(ys + i), gn_affine_vec<T>(v, i, g * cpg, L, scale, bias, meanf, rstd));
         } else {
+            const uint32_t c = g * cpg + fd_div(i, L);
+            const float w = scale ? Ar<T>::widen(scale[c]) : 1.0f;
+            const float b = bias ? Ar<T>::widen(bias[c]) : 0.0f;
             const float t = (Ar<T>::widen(xs[i]) - meanf) * rstd;
             ys[i] = Ar<T>::conv(t * w + b);
+        }
+    }
+}
+
+// gn_apply_kernel for slices of up to NV vectors a thread: all loads of the slice are in flight before the first is used
+template <typename T, int NV>
+__global__ void __launch_bounds__(BLOCK) gn_apply_reg_kernel(const T* __restrict__ x, const T* __restrict__ scale,
+                                                             const T* __restrict__ bias, T* __restrict__ y,
+                                                             const float* __restrict__ part, uint32_t glen, uint32_t chunk,
+                                                             uint32_t splits, uint32_t cpg, uint32_t groups, FastDiv L, float eps) {
+    constexpr int VE = 16 / sizeof(T);
+    __shared__ float s_mean, s_rstd;
+    const uint32_t s = blockIdx.y, grp = blockIdx.x;
+    const uint32_t c0 = s * chunk;
+    const uint32_t c1 = (c0 + chunk < glen) ? c0 + chunk : glen;
+    const v4u* xs = reinterpret_cast<const v4u*>(x + (uint64_t)grp * glen + c0);
+    v4u* ys = reinterpret_cast<v4u*>(y + (uint64_t)grp * glen + c0);
+    const uint32_t nvec = (c1 - c0) / VE;
+    Vec16<T> v[NV];
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        const uint32_t i = threadIdx.x + k * BLOCK;
+        v[k].u = v4u{0u, 0u, 0u, 0u};
+        if (i < nvec) v[k].u = ld_stream(xs + i);
+    }
+    gn_combine_wave(part + (uint64_t)grp * splits * 3, splits, eps, s_mean, s_rstd);
+    __syncthreads();
+    const float meanf = s_mean, rstd = s_rstd;
+    const uint32_t g = grp % groups;
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        const uint32_t i = threadIdx.x + k * BLOCK;
+        if (i < nvec) {
+            st_stream(ys + i, gn_affine_vec<T>(v[k], c0 + i * VE, g * cpg, L, scale, bias, meanf, rstd));
         }
     }
 }
@@ -1326,26 +1460,19 @@ __global__ void __launch_bounds__(GN_LDS_BLOCK) gn_lds_kernel(const T* __restric
     const float var = row_sum<GN_LDS_BLOCK>(m2) / (float)glen;
     const float rstd = 1.0f / __builtin_sqrtf(var + eps);
     for (uint32_t i = threadIdx.x; i < nvec; i += GN_LDS_BLOCK) {
-        const uint32_t c = g * cpg + fd_div(i * VE, L);                      // L % VE == 0: one channel per vector
-        const float w = scale ? Ar<T>::widen(scale[c]) : 1.0f;
-        const float b = bias ? Ar<T>::widen(bias[c]) : 0.0f;
-        Vec16<T> v, o;
+        Vec16<T> v;
         v.u = stage[i];
-#pragma unroll
-        for (int q = 0; q < VE; q++) {
-            const float t = (Ar<T>::widen(v.e[q]) - mean) * rstd;
-            o.e[q] = Ar<T>::conv(t * w + b);
-        }
-        st_stream(ys + i, o.u);
+        st_stream(ys + i, gn_affine_vec<T>(v, i * VE, g * cpg, L, scale, bias, mean, rstd));
     }
 }
 
-// Fewer (batch, group) pairs than half the CUs (32 groups of 96 KB on 256 CUs): `slices` blocks per group, all in one
-// launch and without any wait between blocks.  Every block of a group loads the WHOLE group into registers (thread t holds
-// vectors t, t + 1024, ...; NV of them) and reduces it to the same mean and variance in the same order, so the blocks of
-// a group agree bit for bit without exchanging anything; each then normalises and stores only its own run of
-// nvec / slices vectors.  The repeated reads of a group hit the L2 of the XCD its blocks share (see the block -> (group,
-// slice) map in launch_gn), so HBM still sees the group once.  Same definitions as gn_lds_kernel.
+// The group in the registers of 1024-thread blocks (thread t holds vectors t, t + 1024, ...; NV of them), for groups too
+// large for the LDS of gn_lds_kernel (one block per group) and for small problems of few groups (32 groups of 96 KB on 256
+// CUs): there `slices` blocks per group, all in one launch and without any wait between blocks.  Every block of a group
+// loads the WHOLE group and reduces it to the same mean and variance in the same order, so the blocks of a group agree
+// bit for bit without exchanging anything; each then normalises and stores only its own run of nvec / slices vectors.
+// The repeated reads of a group hit the L2 of the XCD its blocks share (see the block -> (group, slice) map in
+// launch_gn), so HBM still sees the group once.  Same definitions as gn_lds_kernel.
 template <typename T, int NV>
 __global__ void __launch_bounds__(GN_LDS_BLOCK) gn_reg_kernel(const T* __restrict__ x, const T* __restrict__ scale, const T* __restrict__ bias,
                                                               T* __restrict__ y, uint32_t glen, uint32_t cpg, uint32_t groups, FastDiv L,
@@ -1397,16 +1524,7 @@ __global__ void __launch_bounds__(GN_LDS_BLOCK) gn_reg_kernel(const T* __restric
     for (int k = 0; k < NV; k++) {
         const uint32_t i = threadIdx.x + k * GN_LDS_BLOCK;
         if (i >= lo && i < hi) {
-            const uint32_t c = g * cpg + fd_div(i * VE, L);                  // L % VE == 0: one channel per vector
-            const float w = scale ? Ar<T>::widen(scale[c]) : 1.0f;
-            const float b = bias ? Ar<T>::widen(bias[c]) : 0.0f;
-            Vec16<T> o;
-#pragma unroll
-            for (int q = 0; q < VE; q++) {
-                const float t = (Ar<T>::widen(v[k].e[q]) - mean) * rstd;
-                o.e[q] = Ar<T>::conv(t * w + b);
-            }
-            st_stream(ys + i, o.u);
+            st_stream(ys + i, gn_affine_vec<T>(v[k], i * VE, g * cpg, L, scale, bias, mean, rstd));
         }
     }
 }
@@ -1455,31 +1573,42 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
     // enough blocks to cover the chip, slices of at least 2048 elements; beyond 64 slices per group the partials are
     // combined by a launch of their own instead of by every apply block
     constexpr uint32_t FUSED_COMBINE_MAX = 64;
+    static_assert(FUSED_COMBINE_MAX <= WAVE, "gn_apply_kernel combines one partial per lane of a wave");
     uint32_t splits = (2048 + bg - 1) / bg;
     const uint32_t max_splits = (glen + 2047) / 2048;
     if (splits > max_splits) splits = max_splits;
     if (splits > 2048) splits = 2048;
     if (splits < 1) splits = 1;
     constexpr int VEMAX = 16 / sizeof(T);
-    const bool vec = (L % VEMAX == 0) && rt_aligned(x, 16) && rt_aligned(y, 16);       // then glen % VEMAX == 0 too
-    // groups that a 1024-thread block holds in registers (up to 16 vectors a thread, 256 KiB; 20 and 24 spill and were slower
-    // than the three-launch path): few of them (fewer pairs than half the CUs) up to that size, or groups too large for the
-    // LDS kernel below in up to eight rounds of blocks ([8,512,3000] f32, 256 groups of 187 KiB: 33.7 -> 20.3 us; [1,512,3000] f32
-    // 9.1 us, [2,640,4096] f16, 64 groups of 160 KiB, 12.4 us)
-    const bool reg_few = (size_t)glen * sizeof(T) <= GN_REG_MAX_BYTES && 2u * bg <= (uint32_t)dev->num_cus;
-    const bool reg_large = (size_t)glen * sizeof(T) > GN_LDS_MAX_BYTES && (size_t)glen * sizeof(T) <= GN_REG_MAX_BYTES &&
-                           bg <= 8u * (uint32_t)dev->num_cus;
+    const bool vec = (glen % VEMAX == 0) && rt_aligned(x, 16) && rt_aligned(y, 16);    // every group starts on a vector boundary
+    // Which path, for vector-aligned groups (measured on 256 CUs; the two or three launches below spread any problem over the
+    // whole chip in small blocks, the one-launch kernels read HBM once but run 1024-thread blocks that hold whole groups):
+    //   small problems (at most 8 MiB) of few groups (at most half as many as CUs) of up to 192 KiB: gn_reg_kernel, several
+    //        blocks per group; one launch where a launch boundary counts (32 groups of 93 KiB f16 between other kernels: 6.6 us
+    //        against 7.0, and 8.4 against 10.7 with events around the op).  On larger ones the launches win: 64 groups of 160
+    //        KiB f16 12.4 us against 9.6, of 187 KiB f32 12.1 against 9.5
+    //   up to 144 KiB, at least 3/8 as many groups as CUs (and at most eight times as many): gn_lds_kernel
+    //        (93 KiB f16 x 96 groups 10.0 us against 11.1, x 256 12.1 against 15.2, 64 KiB x 1024 28.4 against 34.4; 93 KiB
+    //        x 64 and fewer: 9.5 against 8.4; gn_reg_kernel on these sizes was no faster: 93 KiB x 1024 49.1 against 47.0)
+    //   144 to 192 KiB (12 vectors a thread), at least half as many groups as CUs: gn_reg_kernel, one block per group
+    //        (187 KiB f32 x 128 groups 14.5 us against 14.4, x 192 17.2 against 20.8, x 1024 77 against 89; x 64: 12.1 against 9.5)
+    //   192 to 256 KiB (16 vectors a thread; 20 and 24 spill), at least as many groups as CUs: gn_reg_kernel
+    //        (256 KiB f16 x 256 groups 30.9 us against 33.8; x 128: 23.5 against 17.2)
+    //   everything else: the launches below
+    const size_t gbytes = (size_t)glen * sizeof(T);
+    const uint32_t cus = (uint32_t)dev->num_cus;
+    const bool reg_few = 2u * bg <= cus && gbytes <= GN_REG_MAX_BYTES * 3 / 4 && (size_t)bg * gbytes <= ((size_t)8 << 20);
+    const bool reg_large = gbytes > GN_LDS_MAX_BYTES && bg <= 8u * cus &&
+                           ((gbytes <= GN_REG_MAX_BYTES * 3 / 4 && 2u * bg >= cus) || (gbytes <= GN_REG_MAX_BYTES && bg >= cus));
     if (vec && (reg_few || reg_large)) {
-        // few groups: several blocks per group, each reducing the whole group and writing one slice of it
-        uint32_t slices = (uint32_t)dev->num_cus / bg;
-        if (slices < 1) slices = 1;
+        uint32_t slices = reg_few ? cus / bg : 1;
         if (slices > 32) slices = 32;
         const uint32_t nvec = glen / VEMAX;
         if (slices > nvec) slices = nvec;
         const uint32_t blocks = bg * slices;
         // with a block count that the 8 XCDs share evenly, block b (on XCD b % 8) takes pair (b % 8) * blocks / 8 + b / 8, which
         // puts the slices of a group on one XCD (all of them when bg is a multiple of 8)
-        const uint32_t per_xcd = blocks % 8 == 0 ? blocks / 8 : 0;
+        const uint32_t per_xcd = (slices > 1 && blocks % 8 == 0) ? blocks / 8 : 0;
         const uint32_t nv = (nvec + GN_LDS_BLOCK - 1) / GN_LDS_BLOCK;
         const dim3 grid(blocks), block(GN_LDS_BLOCK);
 #define RT_GN_REG(NVC)                                                                                                                      \
@@ -1487,7 +1616,6 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
                        groups, make_fastdiv(L), eps, slices, per_xcd)
         if (nv <= 1) RT_GN_REG(1);
         else if (nv <= 2) RT_GN_REG(2);
-        else if (nv <= 3) RT_GN_REG(3);
         else if (nv <= 4) RT_GN_REG(4);
         else if (nv <= 6) RT_GN_REG(6);
         else if (nv <= 9) RT_GN_REG(9);
@@ -1497,7 +1625,7 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
         RT_CHECK_LAUNCH("gn_reg_kernel");
         return RT_OK;
     }
-    if (vec && (size_t)glen * sizeof(T) <= GN_LDS_MAX_BYTES && bg <= 2u * (uint32_t)dev->num_cus) {
+    if (vec && gbytes <= GN_LDS_MAX_BYTES && 8u * bg >= 3u * cus && bg <= 8u * cus) {
         const int ti = sizeof(T) == 4 ? 0 : (std::is_same<T, half_t>::value ? 1 : 2);
         if (!(dev->gn_lds_attr_set & (1u << ti))) {
             RT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gn_lds_kernel<T>), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1509,9 +1637,20 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
         RT_CHECK_LAUNCH("gn_lds_kernel");
         return RT_OK;
     }
+    // slices of at most 32 KiB stay in the registers of their 256-thread block (8 vectors a thread), in the stats launch and
+    // in the apply launch: more, smaller slices when the rule above leaves them larger
+    constexpr uint32_t GN_SLICE_REG_VEC = 8;
+    constexpr uint32_t slice_reg_elems = GN_SLICE_REG_VEC * BLOCK * VEMAX;
+    if (vec) {
+        const uint32_t want = (glen + slice_reg_elems - 1) / slice_reg_elems;
+        // (only while the partials still fit the fixed buffer of rt_group_norm_static: both entry points slice alike)
+        if (want > splits && want <= 2048 && ((size_t)bg * want + bg) * 3 * sizeof(float) <= GN_STATIC_SCRATCH_BYTES) splits = want;
+    }
     uint32_t chunk = (glen + splits - 1) / splits;
     if (vec) chunk = (chunk + VEMAX - 1) / VEMAX * VEMAX;                               // slices start on vector boundaries
     splits = (glen + chunk - 1) / chunk;
+    const bool slice_reg = vec && chunk <= slice_reg_elems;
+    const uint32_t slice_nv = slice_reg ? (chunk / VEMAX + BLOCK - 1) / BLOCK : 0;
     const size_t need = ((size_t)bg * splits + bg) * 3 * sizeof(float);           // partials, then one combined triple per group
     if (fixed_scratch) {
         RT_REQUIRE(need <= GN_STATIC_SCRATCH_BYTES, RT_ERR_SIZE,
@@ -1531,15 +1670,30 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
     float* const part = fixed_scratch ? fixed_scratch : dev->gn_scratch;
     const float* stats = separate ? part + (size_t)bg * splits * 3 : part;
     const uint32_t stat_splits = separate ? 1 : splits;
-    if (vec) hipLaunchKernelGGL((gn_stats_kernel<T, VEMAX>), grid, block, 0, dev->stream, (const T*)x, part, glen, chunk, splits);
+#define RT_GN_STATS(NVC) \
+    hipLaunchKernelGGL((gn_stats_reg_kernel<T, NVC>), grid, block, 0, dev->stream, (const T*)x, part, glen, chunk, splits)
+    if (slice_reg && slice_nv <= 1) RT_GN_STATS(1);
+    else if (slice_reg && slice_nv <= 2) RT_GN_STATS(2);
+    else if (slice_reg && slice_nv <= 4) RT_GN_STATS(4);
+    else if (slice_reg) RT_GN_STATS(8);
+    else if (vec) hipLaunchKernelGGL((gn_stats_kernel<T, VEMAX>), grid, block, 0, dev->stream, (const T*)x, part, glen, chunk, splits);
     else hipLaunchKernelGGL((gn_stats_kernel<T, 1>), grid, block, 0, dev->stream, (const T*)x, part, glen, chunk, splits);
+#undef RT_GN_STATS
     RT_CHECK_LAUNCH("gn_stats_kernel");
     if (separate) {
         hipLaunchKernelGGL(gn_combine_kernel, dim3(bg), block, 0, dev->stream, (const float*)part,
                            part + (size_t)bg * splits * 3, splits);
         RT_CHECK_LAUNCH("gn_combine_kernel");
     }
-    if (vec) {
+#define RT_GN_APPLY(NVC)                                                                                                                   \
+    hipLaunchKernelGGL((gn_apply_reg_kernel<T, NVC>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, (T*)y, stats, \
+                       glen, chunk, stat_splits, cpg, groups, make_fastdiv(L), eps)
+    if (slice_reg && slice_nv <= 1) RT_GN_APPLY(1);
+    else if (slice_reg && slice_nv <= 2) RT_GN_APPLY(2);
+    else if (slice_reg && slice_nv <= 4) RT_GN_APPLY(4);
+    else if (slice_reg) RT_GN_APPLY(8);
+#undef RT_GN_APPLY
+    else if (vec) {
         hipLaunchKernelGGL((gn_apply_kernel<T, VEMAX>), grid, block, 0, dev->stream, (const T*)x, (const T*)scale, (const T*)bias, (T*)y, stats,
                            glen, chunk, stat_splits, cpg, groups, make_fastdiv(L), eps);
     } else {
