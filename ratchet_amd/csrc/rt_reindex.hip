@@ -239,6 +239,66 @@ __global__ void __launch_bounds__(TV_BLOCK) transpose_vec_kernel(const ElemT* __
     }
 }
 
+// Larger patches of the same scheme for large tensors: TJ source rows (elements along dst dim 3) x TQ elements along the
+// source's contiguous dim, so a block reads TJ runs of TQ * sizeof(ElemT) bytes and writes TQ runs of TJ * sizeof(ElemT)
+// bytes, several vectors per thread, all loads in flight before the tile is written.
+template <typename ElemT, int TJ, int TQ>
+__global__ void __launch_bounds__(TV_BLOCK) transpose_big_kernel(const ElemT* __restrict__ x, ElemT* __restrict__ y, TransposeArgs p) {
+    constexpr int V = 16 / sizeof(ElemT);
+    constexpr int TQW = TQ * (int)sizeof(ElemT) / 4;         // words per tile row
+    constexpr int QV = TQ / V;                               // vectors per source run
+    constexpr int JV = TJ / V;                               // vectors per destination run
+    constexpr int NLD = TJ * QV / TV_BLOCK;                  // vectors per thread
+    static_assert(TJ * QV % TV_BLOCK == 0 && NLD >= 1, "whole vectors per thread");
+    __shared__ uint32_t tile[TJ][TQW + 1];
+    uint32_t oa, obi, bz, byx, by, bx;
+    fd_divmod(blockIdx.x, p.gx, byx, bx);
+    fd_divmod(byx, p.gy, bz, by);
+    fd_divmod(bz, p.ob, oa, obi);
+    const uint64_t src0 = oa * p.sa + obi * p.sb;
+    const uint64_t dst0 = oa * p.da + obi * p.db;
+    const uint32_t q0 = bx * TQ, j0 = by * TJ;
+    v4u in[NLD];
+#pragma unroll
+    for (int k = 0; k < NLD; k++) {
+        const uint32_t t = threadIdx.x + k * TV_BLOCK;
+        const uint32_t r = t / QV, v = t % QV;
+        const uint32_t j = j0 + r, q = q0 + v * V;
+        in[k] = v4u{0u, 0u, 0u, 0u};
+        if (j < p.n3 && q < p.nq) in[k] = ld_stream(reinterpret_cast<const v4u*>(x + src0 + (uint64_t)j * p.s3 + q));
+    }
+#pragma unroll
+    for (int k = 0; k < NLD; k++) {
+        const uint32_t t = threadIdx.x + k * TV_BLOCK;
+        const uint32_t r = t / QV, v = t % QV;
+#pragma unroll
+        for (int w = 0; w < 4; w++) tile[r][v * 4 + w] = in[k][w];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < NLD; k++) {
+        const uint32_t t = threadIdx.x + k * TV_BLOCK;
+        const uint32_t d = t / JV, tv = t % JV;
+        const uint32_t q = q0 + d, j = j0 + tv * V;
+        if (q < p.nq && j < p.n3) {
+            v4u out;
+            if (sizeof(ElemT) == 4) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) out[e] = tile[tv * 4 + e][d];
+            } else {
+                const uint16_t* t16 = reinterpret_cast<const uint16_t*>(&tile[0][0]);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const uint32_t lo = t16[(tv * 8 + 2 * e) * (2 * (TQW + 1)) + d];
+                    const uint32_t hi = t16[(tv * 8 + 2 * e + 1) * (2 * (TQW + 1)) + d];
+                    out[e] = lo | (hi << 16);
+                }
+            }
+            st_stream(reinterpret_cast<v4u*>(y + dst0 + (uint64_t)q * p.dq + j), out);
+        }
+    }
+}
+
 // concat: input k is [a_dim, bv[k]] vectors, copied into dst rows of dst_sv vectors at column dst_ov[k]
 struct ConcatArgs {
     const void* src[8];
@@ -608,7 +668,7 @@ int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uin
         // The LDS patch kernel where it beats the register transpose below: source rows of 9 to 12 vectors (head dims 80
         // and 96 in f16), which the register kernel covers with one wave-wide run per row and so stores in runs that
         // are not whole lines ([1,32,4096,96] f16: 15.8 -> 12.4 us, [1,32,2048,80]: 8.2 -> 7.1 us), and tensors of
-        // 128 MB and more, where one store per thread pays ([8,32,2048,128] f16: 48 -> 45 us).
+        // 128 MB and more, where one store per thread pays ([8,32,2048,128] f16: 48 -> 45 us; 32-bit ones in larger patches).
         const uint32_t V = 16u / (uint32_t)elem_bytes;
         const uint32_t row_vecs = dst_shape[q] / V;
         uint64_t total = (uint64_t)elem_bytes;
@@ -625,6 +685,21 @@ int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uin
             p.sb = S[others[1]];
             p.da = dst_strides[others[0]];
             p.db = dst_strides[others[1]];
+            if (elem_bytes == 4 && total >= (128ull << 20)) {
+                // 32-bit tensors of 128 MB and more: patches of 128 x 64 elements, 256-byte runs in, 512-byte runs out
+                // ([2,4096,4096] 58.6 -> 47.9 us, [1,8192,8192] 137 -> 123 us, [16,2048,2048] 93.9 -> 87.5 us, [3,3000,5120]
+                // 88 -> 79 us; 16-bit tensors gained nothing from patches of 128 x 128, 256 x 64 or 64 x 256)
+                constexpr int TJ = 128, TQ = 64;
+                const uint64_t gx = (p.nq + TQ - 1) / TQ, gy = (p.n3 + TJ - 1) / TJ;
+                const uint64_t blocks = gx * gy * dst_shape[others[0]] * dst_shape[others[1]];
+                RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_permute: %llu tiles exceed the grid limit", (unsigned long long)blocks);
+                p.gx = make_fastdiv((uint32_t)gx);
+                p.gy = make_fastdiv((uint32_t)gy);
+                hipLaunchKernelGGL((transpose_big_kernel<uint32_t, TJ, TQ>), dim3((unsigned)blocks), dim3(TV_BLOCK), 0, dev->stream,
+                                   (const uint32_t*)x, (uint32_t*)y, p);
+                RT_CHECK_LAUNCH("transpose_big_kernel");
+                return RT_OK;
+            }
             const uint64_t gx = (p.nq + 8 * V - 1) / (8 * V), gy = (p.n3 + 63) / 64;
             const uint64_t blocks = gx * gy * dst_shape[others[0]] * dst_shape[others[1]];
             RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_permute: %llu tiles exceed the grid limit", (unsigned long long)blocks);

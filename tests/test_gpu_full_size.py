@@ -169,6 +169,11 @@ def test_large_transpose_takes_the_patch_kernel(dev):
     assert same_bits(dev.permute(dk, (0, 1, 3, 2)).to_numpy(), k.transpose(0, 1, 3, 2))
     x = rng.standard_normal((4, 2056, 32, 136)).astype(np.float16)
     assert same_bits(dev.permute(dev.upload(x), (0, 2, 3, 1)).to_numpy(), x.transpose(0, 2, 3, 1))
+    # 32-bit tensors of that size: patches of 128 x 64 elements, ragged on both sides here (8200 = 64 * 128 + 8, 4100 = 64 * 64 + 4)
+    m = rng.standard_normal((1, 8200, 4100)).astype(np.float32)
+    assert same_bits(dev.permute(dev.upload(m), (0, 2, 1)).to_numpy(), m.transpose(0, 2, 1))
+    h = rng.standard_normal((2, 2056, 32, 260)).astype(np.float32)
+    assert same_bits(dev.permute(dev.upload(h), (0, 2, 3, 1)).to_numpy(), h.transpose(0, 2, 3, 1))
 
 
 def test_ops_across_the_4_gib_boundary(dev, oracle):
