@@ -136,6 +136,56 @@ __global__ void __launch_bounds__(BLOCK) transpose_kernel(const ElemT* __restric
     }
 }
 
+// The same 64 x 64 patch with the widest accesses each side allows: LW elements per load along the source's contiguous
+// dim, SW elements per store along the destination's (each 1, 2, 4 or 8 elements and at most 16 bytes; the launcher
+// checks that every row start and extent on that side is a multiple).  K^T of [B,H,1500,D] in 16 bits, whose destination
+// rows of 1500 elements are whole 8-byte units but not whole 16-byte vectors: 16-byte loads, 8-byte stores.
+template <typename ElemT, int LW, int SW>
+__global__ void __launch_bounds__(BLOCK) transpose_wide_kernel(const ElemT* __restrict__ x, ElemT* __restrict__ y, TransposeArgs p) {
+    constexpr int TQ = 64, TJ = 64;
+    constexpr int PAD = sizeof(ElemT) == 4 ? 1 : 2;
+    __shared__ ElemT tile[TJ][TQ + PAD];
+    uint32_t oa, obi, bz, byx, by, bx;
+    fd_divmod(blockIdx.x, p.gx, byx, bx);
+    fd_divmod(byx, p.gy, bz, by);
+    fd_divmod(bz, p.ob, oa, obi);
+    const uint64_t src0 = oa * p.sa + obi * p.sb;
+    const uint64_t dst0 = oa * p.da + obi * p.db;
+    const uint32_t q0 = bx * TQ, j0 = by * TJ;
+    struct alignas(LW * sizeof(ElemT)) LoadT { ElemT e[LW]; };
+    struct alignas(SW * sizeof(ElemT)) StoreT { ElemT e[SW]; };
+    constexpr int NL = TJ * (TQ / LW) / BLOCK, NS = TQ * (TJ / SW) / BLOCK;
+    static_assert(NL >= 1 && NS >= 1, "at least one access per thread");
+    LoadT in[NL] = {};
+#pragma unroll
+    for (int k = 0; k < NL; k++) {
+        const uint32_t i = threadIdx.x + k * BLOCK;
+        const uint32_t r = i / (TQ / LW), c = (i % (TQ / LW)) * LW;
+        const uint32_t j = j0 + r, q = q0 + c;
+        if (j < p.n3 && q < p.nq) in[k] = *reinterpret_cast<const LoadT*>(x + src0 + (uint64_t)j * p.s3 + q);
+    }
+#pragma unroll
+    for (int k = 0; k < NL; k++) {
+        const uint32_t i = threadIdx.x + k * BLOCK;
+        const uint32_t r = i / (TQ / LW), c = (i % (TQ / LW)) * LW;
+#pragma unroll
+        for (int e = 0; e < LW; e++) tile[r][c + e] = in[k].e[e];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < NS; k++) {
+        const uint32_t i = threadIdx.x + k * BLOCK;
+        const uint32_t r = i / (TJ / SW), c = (i % (TJ / SW)) * SW;
+        const uint32_t q = q0 + r, j = j0 + c;
+        if (q < p.nq && j < p.n3) {
+            StoreT out;
+#pragma unroll
+            for (int e = 0; e < SW; e++) out.e[e] = tile[c + e][r];
+            *reinterpret_cast<StoreT*>(y + dst0 + (uint64_t)q * p.dq + j) = out;
+        }
+    }
+}
+
 // The same permutations when every row on both sides is a whole number of aligned 16-byte vectors (the attention
 // transposes: [B,H,T,D] -> [B,H,D,T], [B,T,H,D] -> [B,H,D,T]): no LDS.  A thread loads V rows of one 16-byte vector
 // (V = 8 halves or 4 words: a V x V block), transposes the block in its registers and stores V vectors.  The 64 lanes of
@@ -718,10 +768,14 @@ int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uin
     {
         // whole aligned 16-byte vectors on both sides: the register transpose
         const uint32_t V = 16u / (uint32_t)elem_bytes;
-        // (when one side is so short that its blocks cannot fill half a wave, the LDS tile below does better)
+        // (when one side is so short that its blocks cannot fill half a wave, the LDS tile below does better; so it does when
+        // the rows of either side are not whole 128-byte lines, where every 128-byte run of the register kernel touches two
+        // lines: [8,1500,1000] f32 34.7 -> 23.3 us, [4,2040,3080] f32 78 -> 54 us, [3,3000,5120] f16 63 -> 44 us, K^T of
+        // [16,6,1500,64] f32 22.1 -> 20.8 us; on whole lines the two are within 5 % of each other)
+        const bool whole_lines = (uint64_t)dst_shape[q] * elem_bytes % 128 == 0 && (uint64_t)dst_shape[3] * elem_bytes % 128 == 0;
         uint32_t qb = dst_shape[q] / V <= 12 ? dst_shape[q] / V : 8, jb = 64 / (qb ? qb : 1);
         if (jb > dst_shape[3] / V) jb = dst_shape[3] / V;
-        if (dst_shape[q] % V == 0 && dst_shape[3] % V == 0 && rt_aligned(x, 16) && rt_aligned(y, 16) && qb * jb >= 32) {
+        if (dst_shape[q] % V == 0 && dst_shape[3] % V == 0 && rt_aligned(x, 16) && rt_aligned(y, 16) && qb * jb >= 32 && whole_lines) {
             TransposeRegArgs r;
             r.nqb = dst_shape[q] / V;
             r.njb = dst_shape[3] / V;
@@ -764,6 +818,45 @@ int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uin
     p.db = dst_strides[others[1]];
     const uint64_t gz = (uint64_t)dst_shape[others[0]] * dst_shape[others[1]];
     const uint32_t tq = p.nq <= 8 ? 8 : p.nq <= 16 ? 16 : p.n3 <= 8 ? 512 : p.n3 <= 16 ? 256 : 64, tj = TILE_ELEMS / tq;
+    if (tq == 64) {
+        // square patches: the widest loads and stores that every row start and extent on each side is a multiple of
+        auto width = [&](uint64_t extent, uint64_t s0, uint64_t s1, uint64_t s2, const void* base) -> int {
+            int w = 16 / elem_bytes;
+            while (w > 1 && (extent % w || s0 % w || s1 % w || s2 % w || !rt_aligned(base, (size_t)w * elem_bytes))) w >>= 1;
+            return w;
+        };
+        const int lw = width(p.nq, p.s3, p.sa, p.sb, x), sw = width(p.n3, p.dq, p.da, p.db, y);
+        if (lw > 1 || sw > 1) {
+            const uint64_t wgx = (p.nq + 63) / 64, wgy = (p.n3 + 63) / 64;
+            const uint64_t wblocks = wgx * wgy * gz;
+            RT_REQUIRE(wblocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_permute: %llu tiles exceed the grid limit", (unsigned long long)wblocks);
+            p.gx = make_fastdiv((uint32_t)wgx);
+            p.gy = make_fastdiv((uint32_t)wgy);
+#define RT_TW(E, LWC, SWC) \
+    hipLaunchKernelGGL((transpose_wide_kernel<E, LWC, SWC>), dim3((unsigned)wblocks), dim3(BLOCK), 0, dev->stream, (const E*)x, (E*)y, p)
+#define RT_TW_S(E, LWC)                   \
+    do {                                  \
+        if (sw == 1) RT_TW(E, LWC, 1);    \
+        else if (sw == 2) RT_TW(E, LWC, 2); \
+        else if (sw == 4 || sizeof(E) == 4) RT_TW(E, LWC, 4); \
+        else RT_TW(E, LWC, (sizeof(E) == 4 ? 4 : 8)); \
+    } while (0)
+#define RT_TW_L(E)                        \
+    do {                                  \
+        if (lw == 1) RT_TW_S(E, 1);       \
+        else if (lw == 2) RT_TW_S(E, 2);  \
+        else if (lw == 4 || sizeof(E) == 4) RT_TW_S(E, 4); \
+        else RT_TW_S(E, (sizeof(E) == 4 ? 4 : 8)); \
+    } while (0)
+            if (elem_bytes == 4) RT_TW_L(uint32_t);
+            else RT_TW_L(uint16_t);
+#undef RT_TW_L
+#undef RT_TW_S
+#undef RT_TW
+            RT_CHECK_LAUNCH("transpose_wide_kernel");
+            return RT_OK;
+        }
+    }
     const uint64_t gx = (p.nq + tq - 1) / tq, gy = (p.n3 + tj - 1) / tj;
     const uint64_t blocks = gx * gy * gz;
     RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_permute: %llu tiles exceed the grid limit", (unsigned long long)blocks);

@@ -56,7 +56,10 @@ def test_permute_transposes_of_whole_vectors(dev, oracle, dtype):
     (K^T in phi2/attn.rs:140, whisper/mha.rs:106, moondream/vision_encoder.rs:58): every order, head dims 64..128,
     extents that leave partial tiles, and a slice-shaped source offset through views of a larger upload."""
     rng = np.random.default_rng(202)
-    for shape in [(2, 3, 40, 80), (1, 6, 1504, 64), (2, 2, 264, 96), (1, 4, 72, 128), (3, 8, 16, 8), (1, 2, 520, 200), (2, 16, 8, 1032)]:
+    # (the last three have rows of whole 128-byte lines on both sides in both types: the register transpose; the others go
+    # through LDS patches in the type whose rows are off the lines)
+    for shape in [(2, 3, 40, 80), (1, 6, 1504, 64), (2, 2, 264, 96), (1, 4, 72, 128), (3, 8, 16, 8), (1, 2, 520, 200), (2, 16, 8, 1032),
+                  (1, 2, 320, 192), (2, 3, 64, 448), (1, 4, 128, 64)]:
         x = randn(rng, shape, dtype)
         dx = dev.upload(x)
         for perm in itertools.permutations(range(4)):
@@ -77,6 +80,31 @@ def test_permute_transposes_of_whole_vectors(dev, oracle, dtype):
     assert np.array_equal(dev.permute(chw, (1, 2, 0)).to_numpy(), img)
     wide = randn(rng, (2, 700, 12), dtype)
     assert np.array_equal(dev.permute(dev.upload(wide), (0, 2, 1)).to_numpy(), np.ascontiguousarray(wide.transpose(0, 2, 1)))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_permute_transposes_with_the_widest_access_each_side_allows(dev, oracle, dtype):
+    """Permutations that move the contiguous dim on shapes whose rows are not whole 16-byte vectors on at least one side:
+    the 64 x 64 patch is loaded and stored in units of 8, 4, 2 or 1 elements, whatever every row start and extent on that
+    side is a multiple of.  K^T at whisper's 1500 frames (whisper/mha.rs:106), extents that leave ragged patches, every
+    order that moves the last dim, and a source that starts off the 16-byte boundary."""
+    rng = np.random.default_rng(203)
+    for shape in [(2, 3, 1500, 64), (1, 2, 70, 66), (1, 3, 1502, 68), (2, 2, 129, 100), (1, 2, 67, 131), (1, 1, 1500, 1028), (2, 2, 36, 252)]:
+        x = randn(rng, shape, dtype)
+        dx = dev.upload(x)
+        for perm in itertools.permutations(range(4)):
+            if perm[3] == 3:
+                continue
+            want = oracle.permute(x, perm)
+            got = dev.permute(dx, perm).to_numpy()
+            assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (shape, perm)
+    from ratchet_amd.runtime import BufferView
+    big = randn(rng, (1 + 4 * 300 * 72,), dtype)
+    dbig = dev.upload(big)
+    for skip in (1, 2, 4):                                             # element offsets: 2..16 bytes off the allocation's alignment
+        view = BufferView(dbig, skip, (3, 300, 72))
+        want = np.ascontiguousarray(big[skip:skip + 3 * 300 * 72].reshape(3, 300, 72).transpose(0, 2, 1))
+        assert np.array_equal(dev.permute(view, (0, 2, 1)).to_numpy().view(np.uint8), want.view(np.uint8)), skip
 
 
 def test_permute_rejects_duplicates(dev):
