@@ -1498,9 +1498,11 @@ __global__ void __launch_bounds__(GN_LDS_BLOCK) gn_reg_kernel(const T* __restric
         for (int q = 0; q < VE; q++) acc += Ar<T>::widen(v[k].e[q]);         // vectors past the group hold zeros
     }
     const float mean = row_sum<GN_LDS_BLOCK>(acc) / (float)glen;
-    // the group stays in registers as it was loaded; the widened values of one pass are not kept for the next (with 16 and
-    // more vectors a thread the compiler otherwise keeps them and spills)
+    // the group stays in registers as it was loaded.  With 16 vectors a thread the widened values of one pass must not be kept
+    // for the next (the compiler otherwise keeps them and spills); with fewer it may keep what fits (32 groups of 93 KiB f16,
+    // 6 vectors a thread: 8.3 us when every pass widens again, 6.3 us when not)
     auto forget = [&]() {
+        if (NV < 16) return;
 #pragma unroll
         for (int k = 0; k < NV; k++) asm volatile("" : "+v"(v[k].u[0]), "+v"(v[k].u[1]), "+v"(v[k].u[2]), "+v"(v[k].u[3]));
     };
@@ -1583,25 +1585,28 @@ int launch_gn(rt_device* dev, const void* x, const void* scale, const void* bias
     const bool vec = (glen % VEMAX == 0) && rt_aligned(x, 16) && rt_aligned(y, 16);    // every group starts on a vector boundary
     // Which path, for vector-aligned groups (measured on 256 CUs; the two or three launches below spread any problem over the
     // whole chip in small blocks, the one-launch kernels read HBM once but run 1024-thread blocks that hold whole groups):
-    //   small problems (at most 8 MiB) of few groups (at most half as many as CUs) of up to 192 KiB: gn_reg_kernel, several
-    //        blocks per group; one launch where a launch boundary counts (32 groups of 93 KiB f16 between other kernels: 6.6 us
-    //        against 7.0, and 8.4 against 10.7 with events around the op).  On larger ones the launches win: 64 groups of 160
-    //        KiB f16 12.4 us against 9.6, of 187 KiB f32 12.1 against 9.5
-    //   up to 144 KiB, at least 3/8 as many groups as CUs (and at most eight times as many): gn_lds_kernel
-    //        (93 KiB f16 x 96 groups 10.0 us against 11.1, x 256 12.1 against 15.2, 64 KiB x 1024 28.4 against 34.4; 93 KiB
-    //        x 64 and fewer: 9.5 against 8.4; gn_reg_kernel on these sizes was no faster: 93 KiB x 1024 49.1 against 47.0)
-    //   144 to 192 KiB (12 vectors a thread), at least half as many groups as CUs: gn_reg_kernel, one block per group
-    //        (187 KiB f32 x 128 groups 14.5 us against 14.4, x 192 17.2 against 20.8, x 1024 77 against 89; x 64: 12.1 against 9.5)
-    //   192 to 256 KiB (16 vectors a thread; 20 and 24 spill), at least as many groups as CUs: gn_reg_kernel
-    //        (256 KiB f16 x 256 groups 30.9 us against 33.8; x 128: 23.5 against 17.2)
+    //   few groups (at most half as many as CUs) of up to 9 vectors a thread (144 KiB; 12 vectors, 192 KiB, in f32):
+    //        gn_reg_kernel, several blocks per group (32 groups of 93 KiB f16 6.3 us against 6.9 for the launches, 96 groups
+    //        7.5 against 10.2 for gn_lds_kernel, 128 groups of 187 KiB f32 12.0 against 13.0 with one block per group).  16-bit
+    //        groups beyond 9 vectors a thread widen to more registers than a thread has: 64 groups of 160 KiB f16 13.3 us
+    //        against 9.6 for the launches
+    //   up to 144 KiB, more groups than that (and at most eight times as many as CUs): gn_lds_kernel
+    //        (93 KiB f16 x 256 groups 12.1 us against 15.2 for the launches, 64 KiB x 1024 28.4 against 34.4; gn_reg_kernel
+    //        on these is within 8 % either way, except 47 KiB f16 x 2048: 53.6 against 42.3)
+    //   f32 groups of 144 to 192 KiB, at least half as many groups as CUs, and of up to 256 KiB (16 vectors a thread; 20 and
+    //        24 spill), at least as many groups as CUs: gn_reg_kernel, one block per group (187 KiB x 256 groups 20.0 us
+    //        against 25.3 for the launches, 256 KiB x 256 27.3 against 32.9, x 1024 107 against 125; 256 KiB x 128: 16.5
+    //        against 16.4).  In 16 bits the launches are as fast or faster on these (160 KiB x 128 groups 13.3 us against
+    //        16.9, 256 KiB x 512 64.2 against 65.8)
     //   everything else: the launches below
     const size_t gbytes = (size_t)glen * sizeof(T);
     const uint32_t cus = (uint32_t)dev->num_cus;
-    const bool reg_few = 2u * bg <= cus && gbytes <= GN_REG_MAX_BYTES * 3 / 4 && (size_t)bg * gbytes <= ((size_t)8 << 20);
-    const bool reg_large = gbytes > GN_LDS_MAX_BYTES && bg <= 8u * cus &&
+    const uint32_t nv_group = (glen / VEMAX + GN_LDS_BLOCK - 1) / GN_LDS_BLOCK;          // vectors a thread of gn_reg_kernel would hold
+    const bool reg_few = 2u * bg <= cus && (nv_group <= 9 || (sizeof(T) == 4 && nv_group <= 12));
+    const bool reg_large = sizeof(T) == 4 && gbytes > GN_LDS_MAX_BYTES && bg <= 8u * cus &&
                            ((gbytes <= GN_REG_MAX_BYTES * 3 / 4 && 2u * bg >= cus) || (gbytes <= GN_REG_MAX_BYTES && bg >= cus));
     if (vec && (reg_few || reg_large)) {
-        uint32_t slices = reg_few ? cus / bg : 1;
+        uint32_t slices = reg_few && bg <= cus ? cus / bg : 1;
         if (slices > 32) slices = 32;
         const uint32_t nvec = glen / VEMAX;
         if (slices > nvec) slices = nvec;

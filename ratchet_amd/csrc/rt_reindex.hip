@@ -43,9 +43,10 @@ __device__ __forceinline__ uint32_t gather_block(const GatherArgs& p) {
 // one VecT per thread-iteration; source contiguous along the destination's last dim (s[3] == 1)
 // U vectors per thread: one for a large tensor whose destination vectors each have a source vector of their own
 // (permute, slice: a wave that stores once and ends leaves HBM a more even stream; [32,4096,32,128] f16 heads swap
-// 389 -> 347 us, 134 MB 37 -> 35 us), UNROLL for small ones (21 MB: 6.5 us against 6.9) and when a source dim is
+// 389 -> 347 us, 134 MB 37 -> 35 us, [1,4096,32,128] f16, 34 MB, 15.5 -> 14.2 us, [1,2048,32,128] f16, 17 MB, 8.4 -> 7.8 us),
+// UNROLL for small ones (10 MB: 6.5 us against 6.9) and when a source dim is
 // repeated (broadcast_to [1,1,4096,4096] -> [1,32,..]: 224 us against 250)
-constexpr uint64_t GATHER_ONE_FROM_BYTES = 48ull << 20;
+constexpr uint64_t GATHER_ONE_FROM_BYTES = 16ull << 20;
 template <typename VecT, int U>
 __global__ void __launch_bounds__(BLOCK) gather_vec_kernel(const VecT* __restrict__ x, VecT* __restrict__ y, GatherArgs p) {
     const uint32_t base = gather_block(p) * (BLOCK * U) + threadIdx.x;

@@ -593,23 +593,24 @@ def test_layer_norm_f32_known_answer_rows_with_an_offset(dev, oracle):
 
 
 @pytest.mark.parametrize("B,C,L,G", [(1, 3, 1, 1), (2, 8, 5, 4), (1, 6, 7, 6), (3, 4, 9, 1), (1, 64, 3000, 32), (2, 32, 17, 8),
-                                     (1, 512, 3000, 32),          # the benchmark shape: 32 groups of 96 KB, fewer than 3/8 of the CUs: slices over the chip, two launches
+                                     (1, 512, 3000, 32),          # the benchmark shape: 32 groups of 96 KB: eight blocks per group, each with the group in registers
                                      (9, 128, 40, 64),            # 576 groups of 80 elements, each staged in LDS by a block
                                      (1, 8, 40000, 2),            # groups larger than LDS
                                      (1, 4, 300000, 1),           # one group of 1.2 M elements: hundreds of slices, combined by a launch of their own
                                      (2, 16, 24, 4),
-                                     (1, 64, 3000, 4),            # 4 groups of 96 KB (f16) / 187 KB (f32)
-                                     (2, 256, 4096, 16),          # 32 groups of 128 / 256 KB
+                                     (1, 64, 3000, 4),            # 4 groups of 96 KB (f16) / 187 KB (f32): 32 blocks per group, 6 / 12 vectors a thread
+                                     (2, 256, 4096, 16),          # 32 groups of 128 (registers) / 256 KB (slices over the chip, two launches)
                                      (4, 576, 2040, 72),          # 288 groups of 32 / 64 KB f16/f32 staged in LDS
                                      (8, 512, 1504, 32),          # 256 groups of 47 KB (LDS) / 94 KB (LDS)
-                                     (4, 1024, 2496, 32),         # 128 groups of 156 KB f16 (12 vectors a thread in registers) / 312 KB f32 (slices)
+                                     (4, 1024, 2496, 32),         # 128 groups of 156 KB f16 / 312 KB f32: slices over the chip
                                      (16, 512, 4096, 32),         # 512 groups of 128 KB f16 (LDS) / 256 KB f32 (16 vectors a thread in registers)
                                      # rows that are not whole vectors (a 16-byte vector crosses into the next channel), groups that are:
                                      (2, 64, 1500, 4),            # f16 rows of 1500: slices in registers
                                      (16, 256, 100, 16),          # 256 groups in LDS, f16 rows of 100
                                      (12, 64, 3, 8),              # 96 groups in LDS, rows shorter than a vector: several channels in one
                                      (1, 256, 1, 8),              # rows of one element
-                                     (4, 1024, 2500, 32)])        # 128 groups of 156 KB f16 in registers, rows of 2500
+                                     (4, 1024, 2500, 32),         # 128 groups of 156 KB f16 in slices, rows of 2500
+                                     (4, 608, 2500, 32)])         # 128 groups of 93 KB f16 / 186 KB f32 in registers (two blocks / one block per group), rows of 2500
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
 def test_group_norm(dev, oracle, B, C, L, G, dtype):
     rng = np.random.default_rng(320)
