@@ -74,7 +74,8 @@ template <> struct Ar<bf16_t> {
 
 // libm-style calls: always through f32 (num_traits::Float on the half types widens)
 template <typename T> __device__ __forceinline__ T ar_tanh(T a) { return Ar<T>::conv(rt_tanhf(Ar<T>::widen(a))); }
-template <typename T> __device__ __forceinline__ T ar_exp(T a) { return Ar<T>::conv(rt_expf(Ar<T>::widen(a))); }
+// (tab: the table of rt_expf_tab, where a kernel has staged a copy of it)
+template <typename T> __device__ __forceinline__ T ar_exp(T a, const uint64_t* tab = rt_exp2f_tab) { return Ar<T>::conv(rt_expf_tab(Ar<T>::widen(a), tab)); }
 template <typename T> __device__ __forceinline__ T ar_log(T a) { return Ar<T>::conv(rt_logf(Ar<T>::widen(a))); }
 template <typename T> __device__ __forceinline__ T ar_sin(T a) { return Ar<T>::conv(rt_sinf(Ar<T>::widen(a))); }
 template <typename T> __device__ __forceinline__ T ar_cos(T a) { return Ar<T>::conv(rt_cosf(Ar<T>::widen(a))); }
@@ -91,20 +92,21 @@ template <typename T> __device__ __forceinline__ T ar_gelu(T x) {
     return A::mul(A::mul(A::conv(0.5f), x), A::add(A::conv(1.0f), t));
 }
 // cpu/unary.rs:64: x / (1 + exp(-x))
-template <typename T> __device__ __forceinline__ T ar_silu(T x) {
+template <typename T> __device__ __forceinline__ T ar_silu(T x, const uint64_t* tab = rt_exp2f_tab) {
     typedef Ar<T> A;
-    return A::div(x, A::add(A::conv(1.0f), ar_exp<T>(A::neg(x))));
+    return A::div(x, A::add(A::conv(1.0f), ar_exp<T>(A::neg(x), tab)));
 }
 // cpu/unary.rs:65: 1 / (1 + exp(-x))
-template <typename T> __device__ __forceinline__ T ar_sigmoid(T x) {
+template <typename T> __device__ __forceinline__ T ar_sigmoid(T x, const uint64_t* tab = rt_exp2f_tab) {
     typedef Ar<T> A;
-    return A::div(A::conv(1.0f), A::add(A::conv(1.0f), ar_exp<T>(A::neg(x))));
+    return A::div(A::conv(1.0f), A::add(A::conv(1.0f), ar_exp<T>(A::neg(x), tab)));
 }
 
-template <int OP, typename T> __device__ __forceinline__ T ar_unary(T x) {
+constexpr bool ar_unary_uses_exp(int op) { return op == RT_EXP || op == RT_SILU || op == RT_SIGMOID; }
+template <int OP, typename T> __device__ __forceinline__ T ar_unary(T x, const uint64_t* tab = rt_exp2f_tab) {
     if (OP == RT_GELU) return ar_gelu<T>(x);
     if (OP == RT_TANH) return ar_tanh<T>(x);
-    if (OP == RT_EXP) return ar_exp<T>(x);
+    if (OP == RT_EXP) return ar_exp<T>(x, tab);
     if (OP == RT_LOG) return ar_log<T>(x);
     if (OP == RT_SIN) return ar_sin<T>(x);
     if (OP == RT_COS) return ar_cos<T>(x);
@@ -114,8 +116,8 @@ template <int OP, typename T> __device__ __forceinline__ T ar_unary(T x) {
     if (OP == RT_FLOOR) return ar_floor<T>(x);
     if (OP == RT_CEIL) return ar_ceil<T>(x);
     if (OP == RT_NEG) return Ar<T>::neg(x);
-    if (OP == RT_SILU) return ar_silu<T>(x);
-    return ar_sigmoid<T>(x);
+    if (OP == RT_SILU) return ar_silu<T>(x, tab);
+    return ar_sigmoid<T>(x, tab);
 }
 
 template <int OP, typename T> __device__ __forceinline__ T ar_binary(T a, T b) {

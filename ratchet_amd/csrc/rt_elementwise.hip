@@ -166,9 +166,9 @@ __global__ void __launch_bounds__(BLOCK) binary_bcast_kernel(const T* __restrict
 
 // ------------------------------------------------------------------------------------------------ unary
 // VIA32: the caller pattern x.full().<op>().cast(dt) on a 16-bit tensor in one pass: widen, the f32 op, one rounding
-template <typename T, int OP, bool VIA32> __device__ __forceinline__ T apply_unary(T v) {
-    if (VIA32) return Ar<T>::conv(ar_unary<OP, float>(Ar<T>::widen(v)));
-    return ar_unary<OP, T>(v);
+template <typename T, int OP, bool VIA32> __device__ __forceinline__ T apply_unary(T v, const uint64_t* tab = rt_exp2f_tab) {
+    if (VIA32) return Ar<T>::conv(ar_unary<OP, float>(Ar<T>::widen(v), tab));
+    return ar_unary<OP, T>(v, tab);
 }
 
 template <typename T, int OP, bool VIA32>
@@ -184,19 +184,28 @@ __global__ void __launch_bounds__(BLOCK) unary_vec_kernel(const T* __restrict__ 
         const uint64_t i = base + (uint64_t)k * BLOCK;
         if (i < nvec) rx[k].u = ld_stream(xv + i);
     }
+    // exp, SiLU and sigmoid look 2^(i/32) up once per element: from a copy of the table in LDS
+    constexpr bool TAB = ar_unary_uses_exp(OP);
+    __shared__ uint64_t exp_tab[TAB ? 32 : 1];
+    const uint64_t* tab = rt_exp2f_tab;
+    if (TAB) {
+        if (threadIdx.x < 32) exp_tab[threadIdx.x] = rt_exp2f_tab[threadIdx.x];
+        __syncthreads();
+        tab = exp_tab;
+    }
 #pragma unroll
     for (int k = 0; k < UNROLL; k++) {
         const uint64_t i = base + (uint64_t)k * BLOCK;
         if (i < nvec) {
             Vec16<T> r;
 #pragma unroll
-            for (int e = 0; e < VE; e++) r.e[e] = apply_unary<T, OP, VIA32>(rx[k].e[e]);
+            for (int e = 0; e < VE; e++) r.e[e] = apply_unary<T, OP, VIA32>(rx[k].e[e], tab);
             st_stream(yv + i, r.u);
         }
     }
     if (blockIdx.x == 0) {
         const uint64_t i = nvec * VE + threadIdx.x;
-        if (i < numel) y[i] = apply_unary<T, OP, VIA32>(x[i]);
+        if (i < numel) y[i] = apply_unary<T, OP, VIA32>(x[i], tab);
     }
 }
 

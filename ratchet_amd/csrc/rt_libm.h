@@ -142,25 +142,23 @@ RT_TABLE uint64_t rt_exp2f_tab[32] = {
     0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull,
     0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull};
 
-RT_FN float rt_expf(float x) {
+// tab: rt_exp2f_tab or a copy of it (a kernel that evaluates many exponentials stages the 256 bytes in LDS: 64 lanes that
+// gather from it cost less there than through the vector memory path; f32 exp on 2^26 elements 5.6 -> 6.35 TB/s)
+RT_FN float rt_expf_tab(float x, const uint64_t* tab) {
     const double N = 32.0;
     const double InvLn2N = 0x1.71547652b82fep+0 * N;
     const double SHIFT = 0x1.8p52;
     const double C0 = 0x1.c6af84b912394p-5 / N / N / N, C1 = 0x1.ebfce50fac4f3p-3 / N / N, C2 = 0x1.62e42ff0c52d6p-1 / N;
-    const uint32_t abstop = (f2u(x) >> 20) & 0x7ffu;
-    if (abstop >= (0x42b00000u >> 20)) {           // |x| >= 88 or NaN
-        if (f2u(x) == 0xff800000u) return 0.0f;
-        if (abstop >= (0x7f800000u >> 20)) return x + x;
-        if (x > 0x1.62e42ep6f) return __builtin_huge_valf();
-        if (x < -0x1.9fe368p6f) return 0.0f;
-    }
+    // The evaluation runs for every input and the special cases are selected afterwards, all without a branch: the table
+    // loads of the elements a thread holds are then issued together instead of each behind its own range test (f32 exp on
+    // 2^26 elements: 4.5 -> 5.6 TB/s).  Inputs out of range (and NaN) produce some double here, never a trap.
     const double xd = (double)x;
     const double z = InvLn2N * xd;
     double kd = z + SHIFT;
     const uint64_t ki = __builtin_bit_cast(uint64_t, kd);
     kd -= SHIFT;
     const double r = __builtin_fma(InvLn2N, xd, -kd);
-    uint64_t t = rt_exp2f_tab[ki & 31];
+    uint64_t t = tab[ki & 31];
     t += ki << (52 - 5);
     const double s = __builtin_bit_cast(double, t);
     const double p = __builtin_fma(C0, r, C1);
@@ -168,8 +166,14 @@ RT_FN float rt_expf(float x) {
     double y = __builtin_fma(C2, r, 1.0);
     y = __builtin_fma(p, r2, y);
     y = y * s;
-    return (float)y;
+    float res = (float)y;
+    res = x < -0x1.9fe368p6f ? 0.0f : res;                     // underflow, -inf
+    res = x > 0x1.62e42ep6f ? __builtin_huge_valf() : res;     // overflow, +inf
+    res = x != x ? x + x : res;                                // NaN
+    return res;
 }
+
+RT_FN float rt_expf(float x) { return rt_expf_tab(x, rt_exp2f_tab); }
 
 // log / sin / cos: evaluated in double and rounded once.  The double routines are accurate to about 1 ulp of
 // double, so the float result is the correctly rounded one except in astronomically rare double-rounding cases;
