@@ -359,21 +359,21 @@ struct ConcatArgs {
     uint32_t dst_sv;
 };
 
-template <typename VecT>
+template <typename VecT, int U>
 __global__ void __launch_bounds__(BLOCK) concat_kernel(VecT* __restrict__ y, ConcatArgs p) {
     const int k = blockIdx.y;
     const VecT* __restrict__ x = reinterpret_cast<const VecT*>(p.src[k]);
     const uint32_t nvec = p.nvec[k];
-    const uint32_t base = blockIdx.x * (BLOCK * UNROLL) + threadIdx.x;
-    if (blockIdx.x * (BLOCK * UNROLL) >= nvec) return;
-    VecT r[UNROLL];
+    const uint32_t base = blockIdx.x * (BLOCK * U) + threadIdx.x;
+    if (blockIdx.x * (BLOCK * U) >= nvec) return;
+    VecT r[U];
 #pragma unroll
-    for (int u = 0; u < UNROLL; u++) {
+    for (int u = 0; u < U; u++) {
         const uint32_t v = base + u * BLOCK;
         if (v < nvec) r[u] = ld_stream(x + v);
     }
 #pragma unroll
-    for (int u = 0; u < UNROLL; u++) {
+    for (int u = 0; u < U; u++) {
         const uint32_t v = base + u * BLOCK;
         if (v < nvec) {
             uint32_t row, col;
@@ -1010,11 +1010,20 @@ int rt_concat(rt_device* dev, int elem_bytes, int n_inputs, const void* const* x
             p.nvec[k] = 0;
         }
     }
-    const dim3 grid(blocks_for(max_nvec, BLOCK * UNROLL), (unsigned)n_inputs);
-    if (vb == 16) hipLaunchKernelGGL((concat_kernel<v4u>), grid, dim3(BLOCK), 0, dev->stream, (v4u*)y, p);
-    else if (vb == 8) hipLaunchKernelGGL((concat_kernel<v2u>), grid, dim3(BLOCK), 0, dev->stream, (v2u*)y, p);
-    else if (vb == 4) hipLaunchKernelGGL((concat_kernel<uint32_t>), grid, dim3(BLOCK), 0, dev->stream, (uint32_t*)y, p);
-    else hipLaunchKernelGGL((concat_kernel<uint16_t>), grid, dim3(BLOCK), 0, dev->stream, (uint16_t*)y, p);
+    // vectors per thread: one for outputs of 64 MiB and more (as in gather_vec_kernel: [1,8192,4096] x 3 f16 71.1 -> 64.0 us,
+    // [1,8192,3072] x 2 36.9 -> 34.3 us), two below ([1,2048,2560] x 2: 8.9 us against 9.3)
+    const bool one = (uint64_t)a_dim * dst_s * elem_bytes >= (64ull << 20);
+    const dim3 grid(blocks_for(max_nvec, BLOCK * (one ? 1 : UNROLL)), (unsigned)n_inputs);
+#define RT_CC(VT)                                                                                                   \
+    do {                                                                                                            \
+        if (one) hipLaunchKernelGGL((concat_kernel<VT, 1>), grid, dim3(BLOCK), 0, dev->stream, (VT*)y, p);          \
+        else hipLaunchKernelGGL((concat_kernel<VT, UNROLL>), grid, dim3(BLOCK), 0, dev->stream, (VT*)y, p);         \
+    } while (0)
+    if (vb == 16) RT_CC(v4u);
+    else if (vb == 8) RT_CC(v2u);
+    else if (vb == 4) RT_CC(uint32_t);
+    else RT_CC(uint16_t);
+#undef RT_CC
     RT_CHECK_LAUNCH("concat_kernel");
     return RT_OK;
 }
