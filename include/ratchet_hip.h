@@ -190,8 +190,8 @@ int rt_group_norm(rt_device* dev, int dt, const void* x, const void* scale, cons
  * forbid hipMalloc).  No counterpart in the reference.  Same arguments, same results bit for bit, but the partial
  * statistics of groups that are split over several blocks go to a fixed 256 KiB array that lives in the library's code
  * object (one copy per GPU, held until the process ends) instead of the device's growable buffer, and the call never
- * reaches hipMalloc / hipFree.  A problem whose partials do not fit (more than about 10 900 (batch, group) pairs that
- * each exceed 144 KB) returns RT_ERR_SIZE.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU
+ * reaches hipMalloc / hipFree.  A problem whose partials do not fit (more than about 10 900 (batch, group) pairs)
+ * returns RT_ERR_SIZE.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU
  * (two rt_devices with the same ordinal, or a replaying graph next to an eager call) race; calls on one rt_device are
  * ordered by its stream.  Nothing in the array has to start at zero: each launch writes every partial it reads. */
 int rt_group_norm_static(rt_device* dev, int dt, const void* x, const void* scale, const void* bias, void* y, uint32_t B,

@@ -1342,9 +1342,6 @@ template <typename T, int KIND>
 int launch_norm16(rt_device* dev, const void* x, const void* scale, const void* bias, void* y, uint64_t rows, uint32_t cols, float eps) {
     const bool vec_ok = (cols % 8 == 0) && rt_aligned(x, 16) && rt_aligned(y, 16) && rt_aligned(scale, 16) && (!bias || rt_aligned(bias, 16));
     if (vec_ok && cols <= 128 && rows >= 16384) return launch_norm16_lane<T, KIND>(dev, x, scale, bias, y, rows, cols, eps);
-    // RMSNorm rows of 256 to 4096 columns, as many rows as the chip holds waves at one time: the row sum replayed by the
-    // whole wave.  It issues about twice the instructions of the walk below, which wins back as soon as the rows come in
-    // more than one round ([8192,3072]: 27 against 22 us; [4096,3072]: 13.1 against 14.2 us, [1024,4096]: 11.9 against 14.5).
     // RMSNorm rows of 256 to 4096 columns, as many of them as the walk below takes in one round (8 rows a block, two
     // blocks a CU): the row sum replayed by a whole wave per row.  That kernel issues about twice the instructions of
     // the walk and a row takes a wave about 2.5 us, so it pays where the walk's latency is what the launch costs
