@@ -155,6 +155,146 @@ __global__ void __launch_bounds__(BLOCK) rope_vec_kernel(const T* x, T* y, RopeV
     }
 }
 
+// The vector kernel with every global access in whole contiguous runs.  A block owns PB consecutive positions and, in each
+// (batch, head) row of its share, the one run of nv = PB * D / VE vectors they occupy: thread (row of the trip, vector of
+// the run) loads its vector, the vectors of the rotated upper half pass through LDS to the thread that holds their
+// partner, which rotates both, and every thread stores the vector it loaded to where it came from in y.  PB is small
+// enough for one sin / cos pair per thread (PB * half <= 256).  rope_vec_kernel, whose waves take one vector slot of many
+// positions, touches 32 to 96 bytes of every line per instruction, and fetches a line again when the next instruction
+// comes for the rest of it (FETCH_SIZE 2.0 x the tensor on [4,32,2048,80] f16, rotary width 32).
+constexpr int RS_U = 4;      // rows of the trip a thread holds
+struct RopeStageArgs {
+    FastDiv rowv_div;        // vectors per position
+    uint32_t S, half, offset, hv, row_v, active_v, PB, nv, rpt;   // active_v: vectors per position that move (all, or 2 * hv in place)
+    uint32_t nbh, bh_chunk;
+    float ln_base;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(BLOCK) rope_stage_kernel(const T* x, T* y, RopeStageArgs a) {
+    constexpr int VE = 16 / sizeof(T);
+    __shared__ v4u stage[RS_U][BLOCK];
+    __shared__ float s_sn[BLOCK], s_cs[BLOCK];
+    const uint32_t p0 = blockIdx.x * a.PB;
+    const uint32_t npos = (a.S - p0 < a.PB) ? a.S - p0 : a.PB;
+    if (threadIdx.x < npos * a.half) {
+        const uint32_t pl = threadIdx.x / a.half, i = threadIdx.x - pl * a.half;
+        const float neg_i = -(float)i;
+        const float inv = rt_expf(neg_i * a.ln_base / (float)a.half);
+        const float theta = (float)(a.offset + p0 + pl) * inv;
+        s_sn[threadIdx.x] = rt_sinf(theta);
+        s_cs[threadIdx.x] = rt_cosf(theta);
+    }
+    __syncthreads();
+    const uint32_t jr = threadIdx.x / a.nv, w = threadIdx.x - jr * a.nv;      // row of the trip, vector of the run
+    uint32_t pl, slot;
+    fd_divmod(w, a.rowv_div, pl, slot);
+    const bool mine = jr < a.rpt && pl < npos && slot < a.active_v;
+    const bool rot = mine && slot < a.hv, upper = mine && slot >= a.hv && slot < 2 * a.hv;
+    float sn[VE], cs[VE];
+#pragma unroll
+    for (int e = 0; e < VE; e++) {
+        sn[e] = rot ? s_sn[pl * a.half + slot * VE + e] : 0.0f;
+        cs[e] = rot ? s_cs[pl * a.half + slot * VE + e] : 0.0f;
+    }
+    const uint32_t bh0 = blockIdx.y * a.bh_chunk;
+    const uint32_t bh1 = (bh0 + a.bh_chunk < a.nbh) ? bh0 + a.bh_chunk : a.nbh;
+    const v4u* xv = reinterpret_cast<const v4u*>(x);
+    v4u* yv = reinterpret_cast<v4u*>(y);
+    const uint64_t row_stride = (uint64_t)a.S * a.row_v;
+    // a thread without a vector of its own loads the block's first one instead (the loads below carry no condition, so the
+    // four of a trip are in flight together and stay in registers) and stores nothing
+    const uint64_t at_w = (uint64_t)p0 * a.row_v + (mine ? w : 0);
+    for (uint32_t b = bh0; b < bh1; b += RS_U * a.rpt) {
+        v4u r[RS_U];
+#pragma unroll
+        for (int u = 0; u < RS_U; u++) {
+            const uint32_t bh = b + u * a.rpt + (mine ? jr : 0);
+            r[u] = xv[(uint64_t)(bh < bh1 ? bh : bh1 - 1) * row_stride + at_w];     // cached loads: neighbouring runs share their edge lines
+        }
+        if (upper) {
+#pragma unroll
+            for (int u = 0; u < RS_U; u++) stage[u][threadIdx.x] = r[u];
+        }
+        __syncthreads();
+        if (rot) {
+#pragma unroll
+            for (int u = 0; u < RS_U; u++) {
+                Vec16<T> lo, hi;
+                lo.u = r[u];
+                hi.u = stage[u][threadIdx.x + a.hv];
+#pragma unroll
+                for (int e = 0; e < VE; e++) {
+                    const float x1 = Ar<T>::widen(lo.e[e]), x2 = Ar<T>::widen(hi.e[e]);
+                    const float r1 = x1 * cs[e] - x2 * sn[e];
+                    const float r2 = x1 * sn[e] + x2 * cs[e];
+                    lo.e[e] = Ar<T>::conv(r1);
+                    hi.e[e] = Ar<T>::conv(r2);
+                }
+                r[u] = lo.u;
+                stage[u][threadIdx.x + a.hv] = hi.u;
+            }
+        }
+        __syncthreads();
+        if (upper) {
+#pragma unroll
+            for (int u = 0; u < RS_U; u++) r[u] = stage[u][threadIdx.x];
+        }
+        if (mine) {
+#pragma unroll
+            for (int u = 0; u < RS_U; u++) {
+                const uint32_t bh = b + u * a.rpt + jr;
+                if (bh < bh1) st_stream(yv + (uint64_t)bh * row_stride + at_w, r[u]);
+            }
+        }
+        // (the next trip writes stage[.][own index] only after this thread has read it, and reads a partner's entry only
+        // behind the next barrier)
+    }
+}
+
+template <typename T> int launch_rope_stage(rt_device* dev, const void* x, void* y, const uint32_t shape[4], uint32_t dim, uint32_t offset, float ln_base) {
+    constexpr uint32_t VE = 16 / sizeof(T);
+    RopeStageArgs a;
+    a.S = shape[2];
+    a.half = dim / 2;
+    a.offset = offset;
+    a.hv = a.half / VE;
+    a.row_v = shape[3] / VE;
+    a.active_v = (x == y) ? 2 * a.hv : a.row_v;              // in place: the pass-through columns stay where they are
+    a.rowv_div = make_fastdiv(a.row_v);
+    a.nbh = shape[0] * shape[1];
+    a.ln_base = ln_base;
+    // positions per block: at most one sin / cos pair per thread, and the run (times the rows of a trip) fills the block best
+    uint32_t pb_max = BLOCK / a.half;
+    if (pb_max > BLOCK / a.row_v) pb_max = BLOCK / a.row_v;
+    if (pb_max > a.S) pb_max = a.S;
+    uint32_t best = 1, best_fill = 0;
+    for (uint32_t pb = 1; pb <= pb_max; pb++) {
+        const uint32_t nv = pb * a.row_v, fill = (BLOCK / nv) * nv;
+        if (fill >= best_fill) {
+            best_fill = fill;
+            best = pb;
+        }
+    }
+    a.PB = best;
+    a.nv = a.PB * a.row_v;
+    a.rpt = BLOCK / a.nv;
+    const uint64_t blocks_x = ((uint64_t)a.S + a.PB - 1) / a.PB;
+    RT_REQUIRE(blocks_x <= 0x7fffffffull, RT_ERR_SIZE, "rt_rope: seq_len too large");
+    // batch * heads is split over blockIdx.y until about four blocks per CU exist, but not below one trip per block
+    uint64_t chunks = ((uint64_t)dev->num_cus * 4 + blocks_x - 1) / blocks_x;
+    const uint64_t per_trip = (uint64_t)RS_U * a.rpt;
+    const uint64_t max_chunks = (a.nbh + per_trip - 1) / per_trip;
+    if (chunks > max_chunks) chunks = max_chunks;
+    if (chunks > 65535) chunks = 65535;
+    if (chunks < 1) chunks = 1;
+    a.bh_chunk = (uint32_t)((a.nbh + chunks - 1) / chunks);
+    chunks = (a.nbh + a.bh_chunk - 1) / a.bh_chunk;
+    hipLaunchKernelGGL((rope_stage_kernel<T>), dim3((unsigned)blocks_x, (unsigned)chunks), dim3(BLOCK), 0, dev->stream, (const T*)x, (T*)y, a);
+    RT_CHECK_LAUNCH("rope_stage_kernel");
+    return RT_OK;
+}
+
 template <typename T> int launch_rope_vec(rt_device* dev, const void* x, void* y, const uint32_t shape[4], uint32_t dim, uint32_t offset, float ln_base) {
     constexpr uint32_t VE = 16 / sizeof(T), ITEMS = BLOCK / VE;
     RopeVecArgs a;
@@ -224,6 +364,17 @@ extern "C" int rt_rope(rt_device* dev, int dt, const void* x, void* y, const uin
     a.nbh = shape[0] * shape[1];
     const uint32_t ve = 16u / (uint32_t)eb;
     if ((dim / 2) % ve == 0 && shape[3] % ve == 0 && rt_aligned(x, 16) && rt_aligned(y, 16)) {
+        // rows that are not whole 256-byte units (head dims 64 to 96 in 16 bits, 80 in f32): the kernel whose accesses are
+        // whole contiguous runs ([4,32,2048,80] f16, rotary width 32: 42.6 -> 22.1 us, [1,32,2048,80] 10.5 -> 7.0 us,
+        // [4,32,4096,96] f16 61.4 -> 45.0 us, [4,32,4096,64] f16 30.1 -> 26.2 us; on rows of 256 and 512 bytes the slot
+        // kernel's pieces are whole lines already and it is 2-8 % faster: [4,32,4096,128] f16 47.5 against 48.5 us)
+        if (dim / 2 <= (uint32_t)BLOCK && shape[3] / ve <= (uint32_t)BLOCK && ((uint64_t)shape[3] * eb) % 256 != 0) {
+            switch (dt) {
+                case RT_F32: return launch_rope_stage<float>(dev, x, y, shape, dim, offset, logf(base));
+                case RT_F16: return launch_rope_stage<half_t>(dev, x, y, shape, dim, offset, logf(base));
+                default: return launch_rope_stage<bf16_t>(dev, x, y, shape, dim, offset, logf(base));
+            }
+        }
         switch (dt) {
             case RT_F32: return launch_rope_vec<float>(dev, x, y, shape, dim, offset, logf(base));
             case RT_F16: return launch_rope_vec<half_t>(dev, x, y, shape, dim, offset, logf(base));

@@ -17,7 +17,8 @@ def dev():
 
 
 @pytest.mark.parametrize("shape,dim,offset", [((1, 2, 5, 16), 16, 0), ((2, 3, 7, 32), 16, 5), ((1, 32, 128, 96), 96, 0), ((1, 32, 1, 96), 96, 4095),
-                                              ((1, 4, 1, 80), 32, 1023), ((2, 1, 300, 128), 64, 17), ((1, 32, 512, 80), 32, 0)])
+                                              ((1, 4, 1, 80), 32, 1023), ((2, 1, 300, 128), 64, 17), ((1, 32, 512, 80), 32, 0),
+                                              ((3, 37, 131, 80), 32, 5), ((2, 9, 77, 96), 64, 1), ((5, 7, 50, 72), 72, 0)])   # rows off 256-byte units: whole runs per block, ragged trips and positions
 def test_rope_f32(dev, oracle, shape, dim, offset):
     rng = np.random.default_rng(601)
     x = rng.standard_normal(shape).astype(np.float32)
@@ -43,7 +44,7 @@ def test_rope_16bit_is_widen_rotate_round(dev, oracle):
 
 
 @pytest.mark.parametrize("shape,dim,offset", [((2, 5, 33, 80), 32, 3), ((1, 3, 9, 80), 40, 0), ((3, 7, 4, 128), 128, 100), ((1, 1, 70, 64), 48, 9),
-                                              ((1, 19, 1, 96), 96, 2047), ((1, 2, 6, 24), 24, 1)])
+                                              ((1, 19, 1, 96), 96, 2047), ((1, 2, 6, 24), 24, 1), ((3, 37, 131, 80), 32, 5), ((2, 40, 77, 64), 64, 1), ((1, 70, 50, 96), 64, 0)])
 def test_rope_16bit_layouts(dev, oracle, shape, dim, offset):
     """f16 / bf16 in the vector layout (half the rotated width a multiple of 8) and outside it (dim 40, 24), odd
     batch * heads counts, with and without pass-through columns, out of place and in place"""
