@@ -141,9 +141,13 @@ __global__ void __launch_bounds__(BLOCK) transpose_kernel(const ElemT* __restric
 // dim, SW elements per store along the destination's (each 1, 2, 4 or 8 elements and at most 16 bytes; the launcher
 // checks that every row start and extent on that side is a multiple).  K^T of [B,H,1500,D] in 16 bits, whose destination
 // rows of 1500 elements are whole 8-byte units but not whole 16-byte vectors: 16-byte loads, 8-byte stores.
-template <typename ElemT, int LW, int SW>
+// TQ other than 64 (80, 96, 128): the patch covers the whole of a short source row (head dims 72 to 128, K^T of
+// [B,H,S,80] and [B,H,S,96]), where patches of 64 leave a second, mostly empty one (80 = 64 + 16: two patches for the
+// work of 1.25); the 64 source rows of such a patch are one contiguous run.
+template <typename ElemT, int LW, int SW, int TQ = 64>
 __global__ void __launch_bounds__(BLOCK) transpose_wide_kernel(const ElemT* __restrict__ x, ElemT* __restrict__ y, TransposeArgs p) {
-    constexpr int TQ = 64, TJ = 64;
+    constexpr int TJ = 64;
+    static_assert(TQ % LW == 0 && TJ % SW == 0, "whole accesses per patch row");
     constexpr int PAD = sizeof(ElemT) == 4 ? 1 : 2;
     __shared__ ElemT tile[TJ][TQ + PAD];
     uint32_t oa, obi, bz, byx, by, bx;
@@ -155,22 +159,24 @@ __global__ void __launch_bounds__(BLOCK) transpose_wide_kernel(const ElemT* __re
     const uint32_t q0 = bx * TQ, j0 = by * TJ;
     struct alignas(LW * sizeof(ElemT)) LoadT { ElemT e[LW]; };
     struct alignas(SW * sizeof(ElemT)) StoreT { ElemT e[SW]; };
-    constexpr int NL = TJ * (TQ / LW) / BLOCK, NS = TQ * (TJ / SW) / BLOCK;
-    static_assert(NL >= 1 && NS >= 1, "at least one access per thread");
+    constexpr int LOADS = TJ * (TQ / LW), STORES = TQ * (TJ / SW);              // accesses per patch
+    constexpr int NL = (LOADS + BLOCK - 1) / BLOCK, NS = (STORES + BLOCK - 1) / BLOCK;
     LoadT in[NL] = {};
 #pragma unroll
     for (int k = 0; k < NL; k++) {
         const uint32_t i = threadIdx.x + k * BLOCK;
         const uint32_t r = i / (TQ / LW), c = (i % (TQ / LW)) * LW;
         const uint32_t j = j0 + r, q = q0 + c;
-        if (j < p.n3 && q < p.nq) in[k] = *reinterpret_cast<const LoadT*>(x + src0 + (uint64_t)j * p.s3 + q);
+        if ((LOADS % BLOCK == 0 || i < LOADS) && j < p.n3 && q < p.nq) in[k] = *reinterpret_cast<const LoadT*>(x + src0 + (uint64_t)j * p.s3 + q);
     }
 #pragma unroll
     for (int k = 0; k < NL; k++) {
         const uint32_t i = threadIdx.x + k * BLOCK;
         const uint32_t r = i / (TQ / LW), c = (i % (TQ / LW)) * LW;
+        if (LOADS % BLOCK == 0 || i < LOADS) {
 #pragma unroll
-        for (int e = 0; e < LW; e++) tile[r][c + e] = in[k].e[e];
+            for (int e = 0; e < LW; e++) tile[r][c + e] = in[k].e[e];
+        }
     }
     __syncthreads();
 #pragma unroll
@@ -178,7 +184,7 @@ __global__ void __launch_bounds__(BLOCK) transpose_wide_kernel(const ElemT* __re
         const uint32_t i = threadIdx.x + k * BLOCK;
         const uint32_t r = i / (TJ / SW), c = (i % (TJ / SW)) * SW;
         const uint32_t q = q0 + r, j = j0 + c;
-        if (q < p.nq && j < p.n3) {
+        if ((STORES % BLOCK == 0 || i < STORES) && q < p.nq && j < p.n3) {
             StoreT out;
 #pragma unroll
             for (int e = 0; e < SW; e++) out.e[e] = tile[c + e][r];
@@ -716,15 +722,15 @@ int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uin
     for (int i = 0; i < 3; i++)
         if (i != q) others[no++] = i;
     {
-        // The LDS patch kernel where it beats the register transpose below: source rows of 9 to 12 vectors (head dims 80
-        // and 96 in f16), which the register kernel covers with one wave-wide run per row and so stores in runs that
-        // are not whole lines ([1,32,4096,96] f16: 15.8 -> 12.4 us, [1,32,2048,80]: 8.2 -> 7.1 us), and tensors of
-        // 128 MB and more, where one store per thread pays ([8,32,2048,128] f16: 48 -> 45 us; 32-bit ones in larger patches).
+        // The LDS patch kernel where it beats the register transpose below: tensors of 128 MB and more, where one store per
+        // thread pays ([8,32,2048,128] f16: 48 -> 45 us; 32-bit ones in larger patches).  (Source rows of 65 to 128 elements
+        // that are not 64 or 128 long, head dims 80 and 96, go to transpose_wide_kernel in one patch across the row: K^T of
+        // [4,32,2048,80] f16 21.6 -> 17.7 us, of [4,32,4096,96] f16 45.2 -> 37.8 us, against 64-wide patches of this kernel.)
         const uint32_t V = 16u / (uint32_t)elem_bytes;
-        const uint32_t row_vecs = dst_shape[q] / V;
         uint64_t total = (uint64_t)elem_bytes;
         for (int i = 0; i < 4; i++) total *= dst_shape[i];
-        if (((row_vecs > 8 && row_vecs <= 12) || total >= (128ull << 20)) && dst_shape[q] % V == 0 && dst_shape[3] % V == 0 &&
+        const bool short_row = dst_shape[q] > 64 && dst_shape[q] <= 128 && dst_shape[q] % 64 != 0;    // one patch of transpose_wide_kernel across it
+        if (total >= (128ull << 20) && !short_row && dst_shape[q] % V == 0 && dst_shape[3] % V == 0 &&
             S[3] % V == 0 && S[others[0]] % V == 0 && S[others[1]] % V == 0 && rt_aligned(x, 16) && rt_aligned(y, 16)) {
             TransposeArgs p;
             p.nq = dst_shape[q];
@@ -828,7 +834,10 @@ int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uin
         };
         const int lw = width(p.nq, p.s3, p.sa, p.sb, x), sw = width(p.n3, p.dq, p.da, p.db, y);
         if (lw > 1 || sw > 1) {
-            const uint64_t wgx = (p.nq + 63) / 64, wgy = (p.n3 + 63) / 64;
+            // a source row of 65 to 128 elements in whole vectors: one patch across it
+            const int lw_max = 16 / elem_bytes;
+            const uint32_t wtq = (lw == lw_max && p.nq > 64 && p.nq <= 128 && p.nq % 64 != 0) ? (p.nq <= 80 ? 80 : p.nq <= 96 ? 96 : 128) : 64;
+            const uint64_t wgx = (p.nq + wtq - 1) / wtq, wgy = (p.n3 + 63) / 64;
             const uint64_t wblocks = wgx * wgy * gz;
             RT_REQUIRE(wblocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_permute: %llu tiles exceed the grid limit", (unsigned long long)wblocks);
             p.gx = make_fastdiv((uint32_t)wgx);
@@ -849,8 +858,27 @@ int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uin
         else if (lw == 4 || sizeof(E) == 4) RT_TW_S(E, 4); \
         else RT_TW_S(E, (sizeof(E) == 4 ? 4 : 8)); \
     } while (0)
-            if (elem_bytes == 4) RT_TW_L(uint32_t);
+#define RT_TW_Q(E, TQC)                                                                                                       \
+    do {                                                                                                                      \
+        constexpr int LWM = 16 / (int)sizeof(E);                                                                              \
+        if (sw == 1) hipLaunchKernelGGL((transpose_wide_kernel<E, LWM, 1, TQC>), dim3((unsigned)wblocks), dim3(BLOCK), 0, dev->stream, (const E*)x, (E*)y, p); \
+        else if (sw == 2) hipLaunchKernelGGL((transpose_wide_kernel<E, LWM, 2, TQC>), dim3((unsigned)wblocks), dim3(BLOCK), 0, dev->stream, (const E*)x, (E*)y, p); \
+        else if (sw == 4 || sizeof(E) == 4) hipLaunchKernelGGL((transpose_wide_kernel<E, LWM, 4, TQC>), dim3((unsigned)wblocks), dim3(BLOCK), 0, dev->stream, (const E*)x, (E*)y, p); \
+        else hipLaunchKernelGGL((transpose_wide_kernel<E, LWM, LWM, TQC>), dim3((unsigned)wblocks), dim3(BLOCK), 0, dev->stream, (const E*)x, (E*)y, p); \
+    } while (0)
+#define RT_TW_QS(E)                          \
+    do {                                     \
+        if (wtq == 80) RT_TW_Q(E, 80);       \
+        else if (wtq == 96) RT_TW_Q(E, 96);  \
+        else RT_TW_Q(E, 128);                \
+    } while (0)
+            if (wtq != 64) {
+                if (elem_bytes == 4) RT_TW_QS(uint32_t);
+                else RT_TW_QS(uint16_t);
+            } else if (elem_bytes == 4) RT_TW_L(uint32_t);
             else RT_TW_L(uint16_t);
+#undef RT_TW_QS
+#undef RT_TW_Q
 #undef RT_TW_L
 #undef RT_TW_S
 #undef RT_TW

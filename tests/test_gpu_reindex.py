@@ -89,7 +89,9 @@ def test_permute_transposes_with_the_widest_access_each_side_allows(dev, oracle,
     side is a multiple of.  K^T at whisper's 1500 frames (whisper/mha.rs:106), extents that leave ragged patches, every
     order that moves the last dim, and a source that starts off the 16-byte boundary."""
     rng = np.random.default_rng(203)
-    for shape in [(2, 3, 1500, 64), (1, 2, 70, 66), (1, 3, 1502, 68), (2, 2, 129, 100), (1, 2, 67, 131), (1, 1, 1500, 1028), (2, 2, 36, 252)]:
+    # (the last four: source rows of 65 to 128 elements in whole vectors take one patch across the row, 80, 96 or 128 wide)
+    for shape in [(2, 3, 1500, 64), (1, 2, 70, 66), (1, 3, 1502, 68), (2, 2, 129, 100), (1, 2, 67, 131), (1, 1, 1500, 1028), (2, 2, 36, 252),
+                  (2, 3, 37, 80), (1, 3, 200, 104), (1, 2, 70, 120), (2, 2, 150, 72)]:
         x = randn(rng, shape, dtype)
         dx = dev.upload(x)
         for perm in itertools.permutations(range(4)):
