@@ -830,6 +830,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline timing")
     ap.add_argument("--no-check", action="store_true", help="skip the parity check of the timed buffers")
     ap.add_argument("--no-patterns", action="store_true", help="skip the one-pass caller-pattern timings reported beside the step")
+    ap.add_argument("--no-decode-graphs", action="store_true",
+                    help="skip the two launch-bound decode sequences (they replay HIP graphs, which a kernel trace of the patterns does not need)")
     ap.add_argument("--no-rotate", action="store_true", help="skip the event-free per-op pass over rotating cold buffers (it allocates about 12 GB)")
     ap.add_argument("--profile", type=str, default=None, help="comma-separated targets to launch alone under rocprofv3 (see profile_targets)")
     ap.add_argument("--reps", type=int, default=6, help="launches per --profile target")
@@ -968,8 +970,8 @@ def main():
     ceiling = copy_ceiling(dev) if not args.ops else None      # after the parity check: it overwrites an output buffer
     copy_us, boundary_us = copy_reference(dev, ops, args.steps) if not args.ops else ([None] * len(ops), None)
     patterns = one_pass_patterns(dev, seed, oracle if not args.no_check else None) if not (args.ops or args.no_patterns) else None
-    decode = decode_step(dev, seed) if not (args.ops or args.no_patterns) else None
-    host_step = host_graph_step(seed) if not (args.ops or args.no_patterns) else None
+    decode = decode_step(dev, seed) if not (args.ops or args.no_patterns or args.no_decode_graphs) else None
+    host_step = host_graph_step(seed) if not (args.ops or args.no_patterns or args.no_decode_graphs) else None
 
     # the kernels' own durations and HBM-side bytes, from the committed rocprofv3 summaries (whole step only: rows are by position)
     kt_rows = read_step_rows(PROFILE_KERNEL_TRACE) if not args.ops else {}
