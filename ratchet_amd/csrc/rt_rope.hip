@@ -373,7 +373,7 @@ extern "C" int rt_rope(rt_device* dev, int dt, const void* x, void* y, const uin
     if ((dim / 2) % ve == 0 && shape[3] % ve == 0 && rt_aligned(x, 16) && rt_aligned(y, 16)) {
         // rows that are not whole 256-byte units (head dims 64 to 96 in 16 bits, 80 in f32): the kernel whose accesses are
         // whole contiguous runs ([4,32,2048,80] f16, rotary width 32: 42.6 -> 22.1 us, [1,32,2048,80] 10.5 -> 7.0 us,
-        // [4,32,4096,96] f16 61.4 -> 45.0 us, [4,32,4096,64] f16 30.1 -> 26.2 us; on rows of 256 and 512 bytes the slot
+        // [4,32,4096,96] f16 61.4 -> 40.0 us, [4,32,4096,64] f16 30.1 -> 26.2 us; on rows of 256 and 512 bytes the slot
         // kernel's pieces are whole lines already and it is 2-8 % faster: [4,32,4096,128] f16 47.5 against 48.5 us)
         if (dim / 2 <= (uint32_t)BLOCK && shape[3] / ve <= (uint32_t)BLOCK && ((uint64_t)shape[3] * eb) % 256 != 0) {
             switch (dt) {
