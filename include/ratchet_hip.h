@@ -199,9 +199,10 @@ int rt_group_norm_static(rt_device* dev, int dt, const void* x, const void* scal
 
 /* scores.add(mask).softmax(last dim) in the tensors' own arithmetic (the 16-bit sum is rounded as the separate add
  * rounds it, then Softmax's contract applies), result bit-identical to rt_binary_bcast(RT_ADD) followed by rt_softmax
- * but the sum never reaches memory when the shape allows (f16 or bf16, reference mode, x / y / mask on 16-byte
- * boundaries, rows of whole 16-byte vectors or of 192 to 4095 columns of any length, a mask that covers whole trailing
- * dims and repeats over the leading ones).  Each mask extent is 1 or the scores' extent; y may be x.
+ * but the sum never reaches memory when the shape allows (x / y / mask on 16-byte boundaries, a mask that covers whole
+ * trailing dims and repeats over the leading ones; f16 or bf16 in reference mode: rows of whole 16-byte vectors or of
+ * 192 to 4095 columns of any length; f32, and the stable mode of any type: rows of whole 16-byte vectors up to 65536
+ * columns).  Each mask extent is 1 or the scores' extent; y may be x.
  * Binary: ops/binary.rs:27-119 via tensor.rs:249-280; Softmax: ops/softmax.rs:17-73, cpu/softmax.rs:22-42. */
 int rt_softmax_masked(rt_device* dev, int dt, const void* x, const uint32_t x_shape[4], const void* mask,
                       const uint32_t mask_shape[4], void* y, int mode);

@@ -47,7 +47,8 @@ constexpr int WIDE_BLOCK = 1024;                        // threads per row for r
 // any T; results are rounded to T once.
 // ------------------------------------------------------------------------------------------------------------------
 template <typename T, int NV, int MODE, int LANES, bool SPAN>
-__global__ void __launch_bounds__(LANES > BLOCK ? LANES : BLOCK) softmax_wave_kernel(const T* x, T* y, uint64_t rows, uint32_t cols) {
+__global__ void __launch_bounds__(LANES > BLOCK ? LANES : BLOCK) softmax_wave_kernel(const T* x, T* y, uint64_t rows, uint32_t cols,
+                                                                                       const T* mask, uint64_t period) {
     constexpr int VE = 16 / sizeof(T);
     constexpr int THREADS = LANES > BLOCK ? LANES : BLOCK;   // rows beyond 2048 vectors: one 1024-thread block per row
     const uint64_t row = (uint64_t)blockIdx.x * (THREADS / LANES) + (threadIdx.x / LANES);
@@ -70,6 +71,21 @@ __global__ void __launch_bounds__(LANES > BLOCK ? LANES : BLOCK) softmax_wave_ke
     for (int k = 0; k < NV; k++) {
         const uint32_t i = lane + k * LANES;
         if (i < nvec) v[k].u = ld_stream(xr + i);
+    }
+    // mask (rows of whole vectors only): row r of x takes mask row r % period, added in T as the separate add would, so
+    // that the result has the bits of add-then-softmax.  Plain loads: a mask row is read once per leading index.
+    if (!SPAN && mask) {
+        const v4u* mr = reinterpret_cast<const v4u*>(mask) + (row % period) * nvec;
+#pragma unroll
+        for (int k = 0; k < NV; k++) {
+            const uint32_t i = lane + k * LANES;
+            if (i < nvec) {
+                Vec16<T> mv;
+                mv.u = mr[i];
+#pragma unroll
+                for (int q = 0; q < VE; q++) v[k].e[q] = Ar<T>::add(v[k].e[q], mv.e[q]);
+            }
+        }
     }
     float e[NV][VE];
     float m = 0.0f;
@@ -608,7 +624,8 @@ __global__ void __launch_bounds__(BLOCK) softmax_via32_generic_kernel(const T* _
     for (uint32_t j = threadIdx.x; j < cols; j += BLOCK) yr[j] = Ar<T>::conv(expf(elem(j) - m) / s);
 }
 
-template <typename T, int MODE, bool SPAN> int launch_wave(rt_device* dev, const void* x, void* y, uint64_t rows, uint32_t cols) {
+template <typename T, int MODE, bool SPAN>
+int launch_wave(rt_device* dev, const void* x, void* y, uint64_t rows, uint32_t cols, const void* mask = nullptr, uint64_t period = 1) {
     constexpr int VE = 16 / sizeof(T);
     const uint32_t nvec = SPAN ? (cols + 2 * VE - 2) / VE : cols / VE;       // SPAN: the most vectors a row can touch
     if (nvec <= 32) {
@@ -618,7 +635,7 @@ template <typename T, int MODE, bool SPAN> int launch_wave(rt_device* dev, const
         const uint64_t blocks = (rows + BLOCK / lanes - 1) / (BLOCK / lanes);
         RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax: too many rows");
         const dim3 grid((unsigned)blocks), block(BLOCK);
-#define RT_NARROW(L) hipLaunchKernelGGL((softmax_wave_kernel<T, 1, MODE, L, SPAN>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols)
+#define RT_NARROW(L) hipLaunchKernelGGL((softmax_wave_kernel<T, 1, MODE, L, SPAN>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols, (const T*)mask, period)
         if (lanes == 2) RT_NARROW(2);
         else if (lanes == 4) RT_NARROW(4);
         else if (lanes == 8) RT_NARROW(8);
@@ -640,7 +657,7 @@ template <typename T, int MODE, bool SPAN> int launch_wave(rt_device* dev, const
         const uint64_t blocks = (rows + WAVES - 1) / WAVES;
         RT_REQUIRE(blocks <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax: too many rows");
         const dim3 grid((unsigned)blocks), block(BLOCK);
-#define RT_SM(NVC) hipLaunchKernelGGL((softmax_wave_kernel<T, NVC, MODE, WAVE, SPAN>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols)
+#define RT_SM(NVC) hipLaunchKernelGGL((softmax_wave_kernel<T, NVC, MODE, WAVE, SPAN>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols, (const T*)mask, period)
         if (nv <= 1) RT_SM(1);
         else if (nv <= 2) RT_SM(2);
         else if (nv <= 3) RT_SM(3);
@@ -652,7 +669,7 @@ template <typename T, int MODE, bool SPAN> int launch_wave(rt_device* dev, const
         const uint32_t nv = (nvec + BLOCK - 1) / BLOCK;
         RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax: too many rows");
         const dim3 grid((unsigned)rows), block(BLOCK);
-#define RT_SM(NVC) hipLaunchKernelGGL((softmax_wave_kernel<T, NVC, MODE, BLOCK, SPAN>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols)
+#define RT_SM(NVC) hipLaunchKernelGGL((softmax_wave_kernel<T, NVC, MODE, BLOCK, SPAN>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols, (const T*)mask, period)
         if (nv <= 3) RT_SM(3);
         else if (nv <= 4) RT_SM(4);
         else if (nv <= 6) RT_SM(6);
@@ -662,7 +679,7 @@ template <typename T, int MODE, bool SPAN> int launch_wave(rt_device* dev, const
         const uint32_t nv = (nvec + WIDE_BLOCK - 1) / WIDE_BLOCK;
         RT_REQUIRE(rows <= 0x7fffffffull, RT_ERR_SIZE, "rt_softmax: too many rows");
         const dim3 grid((unsigned)rows), block(WIDE_BLOCK);
-#define RT_SM(NVC) hipLaunchKernelGGL((softmax_wave_kernel<T, NVC, MODE, WIDE_BLOCK, SPAN>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols)
+#define RT_SM(NVC) hipLaunchKernelGGL((softmax_wave_kernel<T, NVC, MODE, WIDE_BLOCK, SPAN>), grid, block, 0, dev->stream, (const T*)x, (T*)y, rows, cols, (const T*)mask, period)
         if (nv <= 4) RT_SM(4);
         else if (nv <= 8) RT_SM(8);
         else if constexpr (sizeof(T) == 4) {                 // (16-bit rows hold 8 values per vector: 8 vectors are the registers' limit)
@@ -939,7 +956,7 @@ extern "C" int rt_softmax_masked(rt_device* dev, int dt, const void* x, const ui
     if (rc) return rc;
     const uint32_t cols = x_shape[3];
     const uint64_t rows = n / cols;
-    // one pass: f16, reference arithmetic, a mask that covers whole trailing dims and repeats over the leading ones
+    // one pass: 16-bit types, reference arithmetic, a mask that covers whole trailing dims and repeats over the leading ones
     int lead = 0;
     while (lead < 3 && mask_shape[lead] == 1) lead++;
     bool whole = mask_shape[3] == cols;
@@ -955,6 +972,21 @@ extern "C" int rt_softmax_masked(rt_device* dev, int dt, const void* x, const ui
         rc = dt == RT_F16 ? rt_softmax_stream_f16(dev, x, mask, period, y, rows, cols, &done)
                           : rt_softmax_stream_bf16(dev, x, mask, period, y, rows, cols, &done);
         if (rc || done) return rc;
+    }
+    // f32, and the stable mode of any type: the row-in-registers kernel adds the mask as it loads (rows of whole vectors)
+    if ((dt == RT_F32 || mode == RT_SOFTMAX_STABLE) && whole && rt_aligned(x, 16) && rt_aligned(y, 16) && rt_aligned(mask, 16)) {
+        const uint32_t ve = 16 / (uint32_t)eb;
+        const uint32_t max_vec = (uint32_t)WIDE_BLOCK * (eb == 4 ? 16 : 8);
+        if (cols % ve == 0 && cols / ve <= max_vec) {
+            if (mode == RT_SOFTMAX_STABLE) {
+                switch (dt) {
+                    case RT_F32: return launch_wave<float, 1, false>(dev, x, y, rows, cols, mask, period);
+                    case RT_F16: return launch_wave<half_t, 1, false>(dev, x, y, rows, cols, mask, period);
+                    default: return launch_wave<bf16_t, 1, false>(dev, x, y, rows, cols, mask, period);
+                }
+            }
+            return launch_wave<float, 0, false>(dev, x, y, rows, cols, mask, period);
+        }
     }
     // otherwise the two ops, the sum parked in y
     rc = rt_binary_bcast(dev, RT_ADD, dt, x, x_shape, mask, mask_shape, y, x_shape);

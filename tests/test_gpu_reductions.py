@@ -772,6 +772,42 @@ def test_softmax_masked_long_rows_and_bf16(dev, oracle, shape, mshape, kind):
     assert np.array_equal(dx.to_numpy().view(np.uint16), got.view(np.uint16))
 
 
+@pytest.mark.parametrize("shape,mshape", [((2, 3, 33, 200), (33, 200)), ((1, 4, 100, 36), (100, 36)), ((2, 2, 64, 1500), (1, 1, 64, 1500)),
+                                          ((1, 3, 20, 5120), (20, 5120)), ((2, 2, 3, 40000), (2, 1, 3, 40000)), ((1, 2, 50, 64), (1, 1, 1, 64)),
+                                          ((1, 2, 17, 202), (17, 202))])
+@pytest.mark.parametrize("np_dt,stable", [(np.float32, False), (np.float32, True), (np.float16, True), ("bf16", True)])
+def test_softmax_masked_in_the_row_kernel_has_the_bits_of_add_then_softmax(dev, oracle, shape, mshape, np_dt, stable):
+    """f32 scores, and the stable mode of every type: rows of whole vectors take one launch that adds the mask as it loads
+    (each of the kernel's row widths: a few lanes, a wave, a block, a 1024-thread block); the last shape's rows are not
+    whole vectors and take the two ops.  Bits of the two separate ops either way; f32 reference mode against the oracle."""
+    from ratchet_amd import _lib
+
+    rng = np.random.default_rng(326)
+    bf = np_dt == "bf16"
+    S, T = mshape[-2], mshape[-1]
+    x32 = randn(rng, shape, np.float32, 2.0)
+    m32 = np.zeros(mshape, np.float32)
+    m2 = m32.reshape(-1, S, T)
+    m2[:] = np.triu(np.full((S, T), -np.inf, np.float32), k=1 + max(T - S, 0)) if S > 1 else randn(rng, (T,), np.float32) * np.float32(3)
+    m2[..., S // 2, :] = randn(rng, (T,), np.float32)                 # a finite row too: the add must round as the separate op does
+    if bf:
+        x, mask = _bf16(oracle, x32), _bf16(oracle, m32)
+        dx, dm = dev.upload(x, bf16=True), dev.upload(mask, bf16=True)
+    else:
+        x, mask = x32.astype(np_dt), m32.astype(np_dt)
+        dx, dm = dev.upload(x), dev.upload(mask)
+    mode = _lib.SOFTMAX_STABLE if stable else _lib.SOFTMAX_REFERENCE
+    got = dev.softmax_masked(dx, dm, mode=mode).to_numpy()
+    two = dev.softmax(dev.binary("add", dx, dm), mode=mode).to_numpy()
+    assert same_bits(got, two), (shape, mshape, np_dt, stable)
+    if np_dt == np.float32 and not stable:
+        full = np.ascontiguousarray(np.broadcast_to(mask.reshape((1,) * (4 - mask.ndim) + mask.shape), shape))
+        bad, mx = oracle.count_not_close(got, oracle.softmax(oracle.binary("add", x, full)), 1e-5, 1e-5)
+        assert bad == 0, mx
+    dev.softmax_masked(dx, dm, out=dx, mode=mode)                      # in place
+    assert same_bits(dx.to_numpy(), got)
+
+
 def test_softmax_masked_other_types_and_modes(dev, oracle):
     from ratchet_amd import _lib, RatchetError
 
