@@ -43,6 +43,7 @@ struct rt_device {
     uint64_t sp_attr_set;   // streaming softmax instantiations whose dynamic-LDS limit has been raised on this device
     uint64_t sp_ragged_attr_set;   // the same for the ragged-row variants
     uint32_t sp_pair_attr_set;     // the same for the variants that take one mask row for two heads
+    unsigned ry_attr_set;          // the same for the one-wave-per-row softmax (rt_softmax_replay.hip)
     uint16_t rp_resident[2][9];    // wave-per-row RMSNorm: blocks of an instantiation ([f16, bf16][vectors per lane]) that one CU holds; 0 = not asked yet
     // row sums of one launch of the streaming softmax's ragged-row variant (RT_SM_ROW_SUMS 16-bit values, allocated with the device)
     uint16_t* sm_row_sums;
@@ -126,6 +127,9 @@ int rt_unary_table(rt_device* dev, int type_index, int op, const uint16_t** out)
 // *done = false when the shape does not fit the kernel (the caller then takes another path).
 int rt_softmax_stream_f16(rt_device* dev, const void* x, const void* mask, uint64_t period, void* y, uint64_t rows, uint32_t cols, bool* done);
 int rt_softmax_stream_bf16(rt_device* dev, const void* x, const void* mask, uint64_t period, void* y, uint64_t rows, uint32_t cols, bool* done);
+
+// The f16 reference softmax for a few long rows, one wave per row (rt_softmax_replay.hip); arguments as above
+int rt_softmax_replay_f16(rt_device* dev, const void* x, const void* mask, uint64_t period, void* y, uint64_t rows, uint32_t cols, bool* done);
 
 // ---------------------------------------------------------------------------------------------------------
 // u32 division by a launch-time constant: q = (n * m) >> (32 + s), exact for all n < 2^32 (round-up method)

@@ -926,6 +926,10 @@ extern "C" int rt_softmax(rt_device* dev, int dt, const void* x, void* y, uint64
             if (rt_aligned(x, 16) && rt_aligned(y, 16) && (cols % 8 == 0 || cols >= RAGGED_STREAM_MIN_COLS)) {
                 if (cols % 8 == 0 && cols <= LANE_MAX_COLS && rows >= 32768) return dt == RT_F16 ? launch_lane16<half_t>(dev, x, y, rows, cols) : launch_lane16<bf16_t>(dev, x, y, rows, cols);
                 bool done = false;
+                if (dt == RT_F16) {                          // a few long rows (a decode step): one wave per row
+                    rc = rt_softmax_replay_f16(dev, x, nullptr, 0, y, rows, cols, &done);
+                    if (rc || done) return rc;
+                }
                 rc = dt == RT_F16 ? rt_softmax_stream_f16(dev, x, nullptr, 0, y, rows, cols, &done)
                                   : rt_softmax_stream_bf16(dev, x, nullptr, 0, y, rows, cols, &done);
                 if (rc || done) return rc;
@@ -969,6 +973,10 @@ extern "C" int rt_softmax_masked(rt_device* dev, int dt, const void* x, const ui
     if (dt != RT_F32 && mode == RT_SOFTMAX_REFERENCE && whole && (cols % 8 == 0 || cols >= RAGGED_STREAM_MIN_COLS) && rt_aligned(x, 16) &&
         rt_aligned(y, 16) && rt_aligned(mask, 16)) {
         bool done = false;
+        if (dt == RT_F16) {
+            rc = rt_softmax_replay_f16(dev, x, mask, period, y, rows, cols, &done);
+            if (rc || done) return rc;
+        }
         rc = dt == RT_F16 ? rt_softmax_stream_f16(dev, x, mask, period, y, rows, cols, &done)
                           : rt_softmax_stream_bf16(dev, x, mask, period, y, rows, cols, &done);
         if (rc || done) return rc;

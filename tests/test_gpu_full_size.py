@@ -37,6 +37,28 @@ def test_whisper_scores_softmax_rows_sum_to_one_and_permute_round_trip(dev, orac
     assert same_bits(dev.permute(p, (0, 2, 1, 3)).to_numpy(), q)
 
 
+def test_f32_causal_softmax_at_a_2048_token_prompt(dev, oracle):
+    """scores.add(mask).softmax(3) on f32 scores [1,32,2048,2048]: the one-launch path against the two ops (bits), the
+    mask's zeros, row sums, and a slab of rows against the oracle"""
+    rng = np.random.default_rng(702)
+    H, S = 32, 2048
+    scores = (2 * rng.standard_normal((1, H, S, S))).astype(np.float32)
+    mask = np.triu(np.full((S, S), -np.inf, np.float32), k=1)
+    dx, dm = dev.upload(scores), dev.upload(mask)
+    dy = dev.softmax_masked(dx, dm)
+    y = dy.to_numpy()
+    two = dev.softmax(dev.binary("add", dx, dm))
+    assert same_bits(y, two.to_numpy())
+    del two
+    upper = np.triu(np.ones((S, S), bool), k=1)
+    assert not y[0, :, upper].any()                                    # masked entries are exactly zero in every head
+    assert np.abs(y.sum(axis=-1, dtype=np.float64) - 1).max() < 1e-5
+    sl = slice(1000, 1032)
+    want = oracle.softmax(oracle.binary("add", scores[0, 17, sl], mask[sl]))
+    bad, mx = oracle.count_not_close(y[0, 17, sl], want, 1e-5, 1e-5)
+    assert bad == 0, mx
+
+
 def test_phi2_block_identities(dev, oracle):
     rng = np.random.default_rng(702)
     x = rng.standard_normal((1, 2048, 2560)).astype(np.float16)

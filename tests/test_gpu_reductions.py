@@ -772,6 +772,54 @@ def test_softmax_masked_long_rows_and_bf16(dev, oracle, shape, mshape, kind):
     assert np.array_equal(dx.to_numpy().view(np.uint16), got.view(np.uint16))
 
 
+@pytest.mark.parametrize("cols", [1536, 2048, 2056, 2560, 4096, 5000 // 8 * 8, 8192])
+@pytest.mark.parametrize("masked", [False, True])
+def test_softmax_f16_few_long_rows_sums_replayed_in_parallel(dev, oracle, cols, masked):
+    """A few rows of 2048 to 8192 columns in f16 (a decode step's scores) take a kernel that replays the reference's
+    left-to-right f16 sum of the exp values with the 64 lanes of a wave instead of walking it; not one bit may differ from the
+    step-wise model.  Rows that stress what the kernel decides by: sums that stop growing (terms below half an ulp),
+    sums that land on powers of two, tiny terms before and after large ones, overflow to inf, NaN, rows of -inf, a causal
+    tail, every term in a binade of its own."""
+    rng = np.random.default_rng(327 + cols)
+    rows = [rng.standard_normal(cols) * s for s in (0.5, 1.0, 2.0, 3.0, 5.0)]
+    rows += [np.zeros(cols), np.full(cols, -np.inf), np.full(cols, np.log(0.5)), np.full(cols, -8.0), np.full(cols, 3.0), np.full(cols, -17.5)]
+    rows += [np.concatenate([np.full(cols // 2, -10.0), np.full(cols - cols // 2, 5.0)])]             # tiny terms, then large ones
+    rows += [np.concatenate([np.full(cols // 2, 5.0), np.full(cols - cols // 2, -10.0)])]             # large sum, then terms below its ulp
+    one_inf = rng.standard_normal(cols)
+    one_inf[cols // 3] = 12.0                                                                        # exp overflows f16
+    rows += [one_inf]
+    late_big = rng.standard_normal(cols) - 4.0
+    late_big[-5] = 10.0
+    rows += [late_big]
+    with_nan = rng.standard_normal(cols)
+    with_nan[cols // 2 + 3] = np.nan
+    rows += [with_nan]
+    causal = rng.standard_normal(cols) * 2.0
+    causal[cols // 4:] = -np.inf
+    rows += [causal]
+    rows += [rng.uniform(-16.0, 10.0, cols), np.linspace(-10, 10, cols), np.linspace(10, -10, cols), np.arange(cols) % 7 * 0.5 - 2.0]
+    rows += [rng.standard_normal(cols) * 2.0 + m for m in (-6.0, -3.0, 0.0, 1.0) for _ in range(10)]
+    x = np.stack(rows).astype(np.float16)
+    dx = dev.upload(x)
+    if masked:
+        mask = np.zeros((1, cols), np.float16)
+        mask[0, cols - cols // 5:] = -np.inf
+        mask[0, ::3] = rng.standard_normal(len(mask[0, ::3])).astype(np.float16)                     # finite terms: the add rounds in f16
+        want = oracle.softmax(oracle.binary("add", x, np.ascontiguousarray(np.broadcast_to(mask, x.shape))))
+        got = dev.softmax_masked(dx, dev.upload(mask)).to_numpy()
+    else:
+        want = oracle.softmax(x)
+        got = dev.softmax(dx).to_numpy()
+    g, t = got.view(np.uint16), want.view(np.uint16)
+    nan = lambda a: ((a & 0x7c00) == 0x7c00) & ((a & 0x3ff) != 0)
+    same = (g == t) | (nan(g) & nan(t))
+    bad_rows = np.flatnonzero(~same.all(axis=1))
+    assert bad_rows.size == 0, (cols, masked, bad_rows[:10].tolist())
+    if not masked:
+        dev.softmax(dx, out=dx)                                                                      # in place
+        assert same_bits(dx.to_numpy(), got)
+
+
 @pytest.mark.parametrize("shape,mshape", [((2, 3, 33, 200), (33, 200)), ((1, 4, 100, 36), (100, 36)), ((2, 2, 64, 1500), (1, 1, 64, 1500)),
                                           ((1, 3, 20, 5120), (20, 5120)), ((2, 2, 3, 40000), (2, 1, 3, 40000)), ((1, 2, 50, 64), (1, 1, 1, 64)),
                                           ((1, 2, 17, 202), (17, 202))])
