@@ -30,6 +30,7 @@
 namespace {
 
 constexpr int RY_BLOCK = 256;                                // four rows per block; the waves never meet
+constexpr int RY_G = 2;                                      // lanes per step of the ordered pass
 constexpr int RY_K = 3;                                      // binades a lane prepares for
 constexpr uint32_t RY_NO_PAIR = 0x7fff7fffu;                 // in place of a pair: added to any f16 bit pattern, either half leaves the binade
 typedef _Float16 ry_h2 __attribute__((ext_vector_type(2)));
@@ -178,41 +179,57 @@ __global__ void __launch_bounds__(RY_BLOCK) softmax16_replay_kernel(const uint16
     // lane's pair for the binade tb lies in is used when it exists and the result stays in the binade (the sum never
     // decreases, so every sum in between does too); otherwise every lane adds its own run to tb left to right and the
     // result of the lane whose turn it is, is kept.
-    // (One wave issues an instruction every four to five cycles, scalar ones too, and 64 lanes come one after the
-    // other: the usual case, a pair for the guessed binade itself, is tried first and takes fifteen instructions.)
-    const uint32_t guess = etop >= 1 && etop <= 30 ? (uint32_t)etop << 10 : 0xffffffffu;     // the guessed binade as a bit pattern
-    const uint32_t g0 = pair[0] & 0xffffu, g1 = pair[0] >> 16;
+    // c[0] in bits 0-9, c[1] in bits 10-19, the guessed exponent field from bit 20 (127, which no f16 has, without a pair)
+    const uint32_t packed = pair[0] != RY_NO_PAIR ? ((pair[0] & 0x3ffu) | ((pair[0] >> 16) << 10) | ((uint32_t)etop << 20)) : (127u << 20);
     uint32_t tb = 0;
-    // (what lane i + 1 contributes is fetched while lane i is decided: a value on its way from a vector register to the
-    // scalar unit is not waited for then)
-    uint32_t gn = __builtin_amdgcn_readlane(guess, 0), c0n = __builtin_amdgcn_readlane(g0, 0), c1n = __builtin_amdgcn_readlane(g1, 0);
-#pragma nounroll
-    for (int i = 0; i < 64; i++) {
-        const uint32_t gi = gn, c0 = c0n, c1 = c1n;
-        const int nx = i < 63 ? i + 1 : 63;
-        gn = __builtin_amdgcn_readlane(guess, nx);
-        c0n = __builtin_amdgcn_readlane(g0, nx);
-        c1n = __builtin_amdgcn_readlane(g1, nx);
-        if ((tb & 0xfc00u) == gi) {
-            const uint32_t next = tb + ((tb & 1u) ? c1 : c0);                // the low bit of tb is the parity of k
-            if (((next ^ tb) & 0xfc00u) == 0) {                              // still in the binade (never so without a pair)
-                tb = next;
-                continue;
-            }
-        }
+    // one lane: its pair for the binade tb lies in, else its run for real
+    auto one_lane = [&](int i) {
         const int k = __builtin_amdgcn_readlane(etop, i) - (int)(tb >> 10);  // exponent field of tb; 31 for inf and NaN
-        if (k == 1 || k == 2) {
-            const uint32_t p = k == 1 ? __builtin_amdgcn_readlane(pair[1], i) : __builtin_amdgcn_readlane(pair[2], i);
+        if (k >= 0 && k <= 2) {
+            const uint32_t p = k == 0 ? __builtin_amdgcn_readlane(pair[0], i)
+                                      : k == 1 ? __builtin_amdgcn_readlane(pair[1], i) : __builtin_amdgcn_readlane(pair[2], i);
             const uint32_t next = tb + ((tb & 1u) ? (p >> 16) : (p & 0xffffu));
             if (((next ^ tb) & 0xfc00u) == 0) {
                 tb = next;
-                continue;
+                return;
             }
         }
         uint32_t t = tb;
 #pragma unroll
         for (int v = 0; v < V; v++) ry_chain(t, run[v]);
         tb = __builtin_amdgcn_readlane(t, i) & 0xffffu;
+    };
+    // RY_G lanes at a time without a branch in between, for the usual case that each has a pair for the guessed binade
+    // itself and the sum stays in it; a lane's guess and pair travel to the scalar unit as one word, fetched while the
+    // group before is decided.  (By the device's clock, on [32, 2048]: table and loads 1.4 us, lookups 1.0 us, the pairs
+    // 0.7 us, this pass 4 us, of which the groups that fall back to one_lane are more than half, quotients and stores
+    // 0.6 us.)
+    uint32_t dn[RY_G];
+#pragma unroll
+    for (int j = 0; j < RY_G; j++) dn[j] = __builtin_amdgcn_readlane(packed, j);
+#pragma nounroll
+    for (int i = 0; i < 64; i += RY_G) {
+        uint32_t d[RY_G];
+        const int nx = i + RY_G < 64 ? i + RY_G : 64 - RY_G;
+#pragma unroll
+        for (int j = 0; j < RY_G; j++) {
+            d[j] = dn[j];
+            dn[j] = __builtin_amdgcn_readlane(packed, nx + j);
+        }
+        uint32_t t = tb, bad = 0;
+#pragma unroll
+        for (int j = 0; j < RY_G; j++) {
+            const uint32_t c = (t & 1u) ? ((d[j] >> 10) & 0x3ffu) : (d[j] & 0x3ffu);       // the low bit of t is the parity of k
+            const uint32_t next = t + c;
+            bad |= ((t >> 10) ^ (d[j] >> 20)) | ((next ^ t) & 0xfc00u);      // not the guessed binade (or no pair for it), or the sum leaves it
+            t = next;
+        }
+        if (bad == 0) {
+            tb = t;
+            continue;
+        }
+#pragma nounroll
+        for (int j = 0; j < RY_G; j++) one_lane(i + j);
     }
 
     const float s = (float)bits_h((uint16_t)tb);
@@ -229,9 +246,9 @@ __global__ void __launch_bounds__(RY_BLOCK) softmax16_replay_kernel(const uint16
 
 // Few long rows of whole vectors in f16: at most two rows per CU (one wave each, so that no wave waits for another),
 // 2048 to 8192 columns.  Measured against the streaming kernel, whose walker lane takes a row's 512-column steps one
-// after the other: [32, 2048] 13.3 -> 11.3 us, [32, 4096] 22.6 -> 14.1 us, [32, 8192] 48.6 -> 17.5 us, [256, 4096]
-// 22.9 -> 15.8 us, [512, 4096] 23.0 -> 17.6 us; rows of 1024 columns lose (8.8 -> 10 us: the 64 lanes of the ordered
-// pass cost 6 us whatever the row length), and from four rows per CU the streaming kernel's overlap wins.
+// after the other: [32, 2048] 13.3 -> 10.1 us, [32, 4096] 22.6 -> 12.5 us, [32, 8192] 48.6 -> 19.5 us, [256, 2048]
+// 13.5 -> 11.0 us, [256, 4096] 22.9 -> 14.3 us; rows of 1024 columns lose (8.8 -> 10 us: the ordered pass costs 4 us
+// whatever the row length), and from four rows per CU the streaming kernel's overlap wins.
 // Returns RT_OK with *done = false when the shape does not fit.
 int rt_softmax_replay_f16(rt_device* dev, const void* x, const void* mask, uint64_t period, void* y, uint64_t rows, uint32_t cols, bool* done) {
     *done = false;
