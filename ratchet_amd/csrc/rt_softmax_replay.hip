@@ -182,13 +182,17 @@ __global__ void __launch_bounds__(RY_BLOCK) softmax16_replay_kernel(const uint16
     // c[0] in bits 0-9, c[1] in bits 10-19, the guessed exponent field from bit 20 (127, which no f16 has, without a pair)
     const uint32_t packed = pair[0] != RY_NO_PAIR ? ((pair[0] & 0x3ffu) | ((pair[0] >> 16) << 10) | ((uint32_t)etop << 20)) : (127u << 20);
     uint32_t tb = 0;
-    // one lane: its pair for the binade tb lies in, else its run for real
-    auto one_lane = [&](int i) {
-        const int k = __builtin_amdgcn_readlane(etop, i) - (int)(tb >> 10);  // exponent field of tb; 31 for inf and NaN
+    // one lane, d its packed word: its pair for the binade tb lies in, else its run for real
+    auto one_lane = [&](int i, uint32_t d) {
+        const int k = (int)(d >> 20) - (int)(tb >> 10);                      // exponent field of tb; 31 for inf and NaN
         if (k >= 0 && k <= 2) {
-            const uint32_t p = k == 0 ? __builtin_amdgcn_readlane(pair[0], i)
-                                      : k == 1 ? __builtin_amdgcn_readlane(pair[1], i) : __builtin_amdgcn_readlane(pair[2], i);
-            const uint32_t next = tb + ((tb & 1u) ? (p >> 16) : (p & 0xffffu));
+            uint32_t c0 = d & 0x3ffu, c1 = (d >> 10) & 0x3ffu;
+            if (k != 0) {
+                const uint32_t p = k == 1 ? __builtin_amdgcn_readlane(pair[1], i) : __builtin_amdgcn_readlane(pair[2], i);
+                c0 = p & 0xffffu;
+                c1 = p >> 16;
+            }
+            const uint32_t next = tb + ((tb & 1u) ? c1 : c0);
             if (((next ^ tb) & 0xfc00u) == 0) {
                 tb = next;
                 return;
@@ -228,8 +232,8 @@ __global__ void __launch_bounds__(RY_BLOCK) softmax16_replay_kernel(const uint16
             tb = t;
             continue;
         }
-#pragma nounroll
-        for (int j = 0; j < RY_G; j++) one_lane(i + j);
+#pragma unroll
+        for (int j = 0; j < RY_G; j++) one_lane(i + j, d[j]);
     }
 
     const float s = (float)bits_h((uint16_t)tb);
@@ -246,8 +250,8 @@ __global__ void __launch_bounds__(RY_BLOCK) softmax16_replay_kernel(const uint16
 
 // Few long rows of whole vectors in f16: at most two rows per CU (one wave each, so that no wave waits for another),
 // 2048 to 8192 columns.  Measured against the streaming kernel, whose walker lane takes a row's 512-column steps one
-// after the other: [32, 2048] 13.3 -> 10.1 us, [32, 4096] 22.6 -> 12.5 us, [32, 8192] 48.6 -> 19.5 us, [256, 2048]
-// 13.5 -> 11.0 us, [256, 4096] 22.9 -> 14.3 us; rows of 1024 columns lose (8.8 -> 10 us: the ordered pass costs 4 us
+// after the other: [32, 2048] 13.3 -> 9.4 us, [32, 4096] 22.6 -> 12.0 us, [32, 8192] 48.6 -> 20 us, [256, 2048]
+// 13.5 -> 10.4 us, [256, 4096] 22.9 -> 14.3 us; rows of 1024 columns lose (8.8 -> 10 us: the ordered pass costs 4 us
 // whatever the row length), and from four rows per CU the streaming kernel's overlap wins.
 // Returns RT_OK with *done = false when the shape does not fit.
 int rt_softmax_replay_f16(rt_device* dev, const void* x, const void* mask, uint64_t period, void* y, uint64_t rows, uint32_t cols, bool* done) {
