@@ -114,6 +114,38 @@ def test_replays_of_ragged_row_softmax_match_eager_execution(dev, oracle):
         dev.sync()
 
 
+def test_replays_of_a_decode_step_softmax_match_eager_execution(dev, oracle):
+    """[B * H, T] f16 scores of a decode step (one wave per row, the row sum replayed from per-lane pairs), plain and with
+    a [1, T] mask, and the masked f32 row kernel, captured and replayed"""
+    rng = np.random.default_rng(803)
+    a = randn(rng, (1, 32, 1, 2304), np.float16, 2.0)
+    m = np.zeros((1, 1, 1, 2304), np.float16)
+    m[..., 2000:] = -np.inf
+    f = randn(rng, (1, 8, 1, 2304), np.float32, 2.0)
+    da, dm, df, dmf = dev.upload(a), dev.upload(m), dev.upload(f), dev.upload(m.astype(np.float32))
+    ya, yb, yf = dev.empty(a.shape, F16), dev.empty(a.shape, F16), dev.empty(f.shape, F32)
+
+    def sequence():
+        dev.softmax(da, out=ya)
+        dev.softmax_masked(da, dm, out=yb)
+        dev.softmax_masked(df, dmf, out=yf)
+
+    sequence()
+    want = [o.to_numpy() for o in (ya, yb, yf)]
+    assert same_bits(want[0], oracle.softmax(a))
+    assert same_bits(want[1], oracle.softmax(oracle.binary("add", a, np.ascontiguousarray(np.broadcast_to(m, a.shape)))))
+    with dev.capture() as cap:
+        sequence()
+    for replay in range(3):
+        for o in (ya, yb, yf):
+            o.zero_()
+        cap.launch()
+        for k, (o, w) in enumerate(zip((ya, yb, yf), want)):
+            assert same_bits(o.to_numpy(), w), (replay, k)
+        dev.softmax(da, out=yb)
+        dev.sync()
+
+
 def test_calls_that_cannot_be_captured_say_so(dev):
     from ratchet_amd import RatchetError
 
