@@ -732,7 +732,11 @@ int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uin
         uint64_t total = (uint64_t)elem_bytes;
         for (int i = 0; i < 4; i++) total *= dst_shape[i];
         const bool short_row = dst_shape[q] > 64 && dst_shape[q] <= 128 && dst_shape[q] % 64 != 0;    // one patch of transpose_wide_kernel across it
-        if (total >= (128ull << 20) && !short_row && dst_shape[q] % V == 0 && dst_shape[3] % V == 0 &&
+        // (16-bit rows that are not whole 128-byte lines on both sides: transpose_wide_kernel below, whose patches this
+        // kernel's 128-byte runs, each across two lines there, do not beat: [1,8200,8200] f16 154 -> 97 us, [4,4104,4104]
+        // 128 -> 87 us, [1,8192,8200] 82 -> 61 us; 32-bit ones gain nothing from it)
+        const bool lines16 = elem_bytes == 4 || ((uint64_t)dst_shape[q] * elem_bytes % 128 == 0 && (uint64_t)dst_shape[3] * elem_bytes % 128 == 0);
+        if (total >= (128ull << 20) && !short_row && lines16 && dst_shape[q] % V == 0 && dst_shape[3] % V == 0 &&
             S[3] % V == 0 && S[others[0]] % V == 0 && S[others[1]] % V == 0 && rt_aligned(x, 16) && rt_aligned(y, 16)) {
             TransposeArgs p;
             p.nq = dst_shape[q];
