@@ -569,7 +569,8 @@ def extra_rows(dev, seed, oracle):
     """Rows reported beside the step, never part of `value`: inputs the step does not show.  (a) the f16 streaming softmax
     on dense N(0,2) scores [1,32,4096,4096] (no mask, so no run of -inf: the table lookups of a wave fall into different
     LDS banks); (b) BASELINE config 0, the reference's own CPU-runnable case, as three launches on [1,1500,384] f32:
-    bias add (broadcast fused), tanh GELU, LayerNorm.  Each with the copy of the same bytes timed the same way."""
+    bias add (broadcast fused), tanh GELU, LayerNorm; (c) the f16 softmax of a decode step's [1,32,1,2048] scores.  Each
+    with the copy of the same bytes timed the same way."""
     import ctypes
 
     from ratchet_amd import _lib
@@ -649,6 +650,18 @@ def extra_rows(dev, seed, oracle):
     add("cfg0 bias add (broadcast fused)", "[1,1500,384]+[384]", "f32", 2 * x.nbytes + bias.nbytes, t1, ok1, note0)
     add("cfg0 gelu (tanh approx)", "[1,1500,384]", "f32", 2 * x.nbytes, t2, ok2, note0)
     add("cfg0 layer_norm", "1500x384", "f32", 2 * x.nbytes + g.nbytes + b.nbytes, t3, ok3, note0)
+
+    # (c) a decode step's scores in f16: [B * H, T] = [32, 2048], one wave per row (the row sum replayed, not walked)
+    sc = normal(seed, 805, (1, 32, 1, 2048), 2.0, np16)
+    dsc, ysc = dev.upload(sc), dev.empty(sc.shape, F16)
+    t4 = timed(lambda: dev.softmax(dsc, out=ysc))
+    ok4 = None
+    if oracle is not None:
+        want = oracle.softmax(sc)
+        got = ysc.to_numpy()
+        ok4 = bool(np.all((got.view(np.uint16) == want.view(np.uint16)) | (np.isnan(got) & np.isnan(want))))
+    add("softmax, decode scores (32 rows)", "[1,32,1,2048]", "f16", 2 * sc.nbytes, t4, ok4,
+        "0.26 MB: bound by the row's sequential f16 sum and the launch, not by memory")
     return rows
 
 
