@@ -674,6 +674,7 @@ def profile_targets(dev, seed, names, reps):
       softmax_dense   rt_softmax on dense N(0,2) scores of that shape (no -inf: the table lookups of a wave differ)
       copy_1gib       the plain copy kernel on 1 GiB (the counters' calibration and the copy ceiling)
       bf16_layer_norm, bf16_rms_norm, f16_rms_norm   the 16-bit reference norms on [4096,3072], cold operands every launch
+      decode_softmax_2048, _4096, _8192   rt_softmax on a decode step's f16 scores [1,32,1,T]
       copy_reference  one plain copy per op of the step (half the op's algorithmic bytes read, half written, fresh regions
                       of two 1 GiB buffers), then a 21 MB copy + 16-byte fill and a 2 MB copy + 16-byte fill: per repetition
                       19 copy launches and 2 fills, in that order"""
@@ -729,6 +730,12 @@ def profile_targets(dev, seed, names, reps):
                     dev.rms_norm(a, dg, 1e-5, out=o)
 
             fn = norm_launch
+        elif name.startswith("decode_softmax_"):
+            # a decode step's f16 scores [1,32,1,T], T from the name (2048, 4096, 8192): one wave per row
+            T = int(name.rsplit("_", 1)[1])
+            dsc = dev.upload(normal(seed, 805, (1, H, 1, T), 2.0, np.float16))
+            ysc = dev.empty((1, H, 1, T), F16)
+            fn = lambda dsc=dsc, ysc=ysc: dev.softmax(dsc, out=ysc)
         elif name == "copy_reference":
             # the copy pass of the bench (one copy per op of the step, same bytes, back to back), without its events; behind
             # it the boundary probes: a 16-byte fill behind a 21 MB copy and behind a 2 MB copy
