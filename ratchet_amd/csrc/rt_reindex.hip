@@ -137,6 +137,118 @@ __global__ void __launch_bounds__(BLOCK) transpose_kernel(const ElemT* __restric
     }
 }
 
+// A short contiguous dim that changes sides: [.., J, C] -> [.., C, J] (interleaved channels to planes, TO_PLANES) and
+// back, C = 2 .. 16 ([B,H,W,3] <-> [B,3,H,W]).  The interleaved side of a tile of PJ positions is one contiguous run of
+// PJ * C elements, moved with 16-byte accesses; the planar side is C runs of PJ elements, 16-byte accesses too; in
+// between the tile lies in LDS as [position][channel] with an odd pitch (C, or C + 1 for an even C: with the pitch of
+// 4 or 16 channels every lane of the strided side would meet the same bank) and is read (or written) with that stride.
+// The launcher checks that every run starts on a 16-byte boundary and is a whole number of vectors (J a multiple of the
+// vector length, strides of the outer dims and of the planes too); PJ * C <= CH_TILE.
+constexpr int CH_TILE = 4096;
+struct ChannelArgs {
+    uint32_t C, J, PJ;
+    uint32_t P;              // LDS pitch: C | 1
+    FastDiv cdiv;            // C
+    FastDiv gj;              // tiles along J (blockIdx.x = (oa * ob + obi) * gj + tile)
+    FastDiv ob;              // extent of the inner of the two outer dims
+    uint64_t ia, ib;         // strides of the outer dims on the interleaved side
+    uint64_t pa, pb, plane;  // strides of the outer dims and of a plane on the planar side
+};
+
+template <typename ElemT, bool TO_PLANES>
+__global__ void __launch_bounds__(BLOCK) channels_kernel(const ElemT* __restrict__ x, ElemT* __restrict__ y, ChannelArgs p) {
+    constexpr int VE = 16 / (int)sizeof(ElemT);
+    constexpr int NV = CH_TILE / VE / BLOCK;                 // vectors per thread at most: 4 (32-bit), 2 (16-bit)
+    __shared__ __attribute__((aligned(16))) ElemT tile[CH_TILE + CH_TILE / 4];       // PJ <= CH_TILE / 4 whenever C is even
+    uint32_t z, tl, oa, obi;
+    fd_divmod(blockIdx.x, p.gj, z, tl);
+    fd_divmod(z, p.ob, oa, obi);
+    const uint32_t j0 = tl * p.PJ;
+    const uint32_t nj = p.J - j0 < p.PJ ? p.J - j0 : p.PJ;   // a multiple of VE
+    const uint32_t nflat = nj * p.C / VE, nvp = nj / VE;     // vectors of the interleaved run, of one plane's run
+    const uint32_t nplanar = nvp * p.C;
+    const uint64_t inter0 = oa * p.ia + obi * p.ib + (uint64_t)j0 * p.C;
+    const uint64_t planar0 = oa * p.pa + obi * p.pb + j0;
+    // the VE elements of vector i of the interleaved run <-> LDS: they are consecutive channels, wrapping to the next position
+    auto flat_to_lds = [&](uint32_t i, const Vec16<ElemT>& v) {
+        uint32_t j, c;
+        fd_divmod(i * VE, p.cdiv, j, c);
+        uint32_t at = j * p.P + c;
+#pragma unroll
+        for (int e = 0; e < VE; e++) {
+            tile[at] = v.e[e];
+            const bool wrap = ++c == p.C;
+            at += wrap ? 1 + p.P - p.C : 1;
+            c = wrap ? 0 : c;
+        }
+    };
+    auto lds_to_flat = [&](uint32_t i) -> Vec16<ElemT> {
+        Vec16<ElemT> v;
+        uint32_t j, c;
+        fd_divmod(i * VE, p.cdiv, j, c);
+        uint32_t at = j * p.P + c;
+#pragma unroll
+        for (int e = 0; e < VE; e++) {
+            v.e[e] = tile[at];
+            const bool wrap = ++c == p.C;
+            at += wrap ? 1 + p.P - p.C : 1;
+            c = wrap ? 0 : c;
+        }
+        return v;
+    };
+    if (TO_PLANES) {
+        const v4u* src = reinterpret_cast<const v4u*>(x + inter0);
+        Vec16<ElemT> in[NV];
+#pragma unroll
+        for (int k = 0; k < NV; k++) {
+            const uint32_t i = threadIdx.x + k * BLOCK;
+            in[k].u = ld_stream(src + (i < nflat ? i : 0));
+        }
+#pragma unroll
+        for (int k = 0; k < NV; k++) {
+            const uint32_t i = threadIdx.x + k * BLOCK;
+            if (i < nflat) flat_to_lds(i, in[k]);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < NV; k++) {
+            const uint32_t i = threadIdx.x + k * BLOCK;
+            if (i < nplanar) {
+                const uint32_t c = i / nvp, t = i - c * nvp;
+                Vec16<ElemT> out;
+#pragma unroll
+                for (int e = 0; e < VE; e++) out.e[e] = tile[(t * VE + e) * p.P + c];
+                st_stream(reinterpret_cast<v4u*>(y + planar0 + (uint64_t)c * p.plane) + t, out.u);
+            }
+        }
+    } else {
+        Vec16<ElemT> in[NV];
+#pragma unroll
+        for (int k = 0; k < NV; k++) {
+            const uint32_t i = threadIdx.x + k * BLOCK;
+            const uint32_t ii = i < nplanar ? i : 0;
+            const uint32_t c = ii / nvp, t = ii - c * nvp;
+            in[k].u = ld_stream(reinterpret_cast<const v4u*>(x + planar0 + (uint64_t)c * p.plane) + t);
+        }
+#pragma unroll
+        for (int k = 0; k < NV; k++) {
+            const uint32_t i = threadIdx.x + k * BLOCK;
+            if (i < nplanar) {
+                const uint32_t c = i / nvp, t = i - c * nvp;
+#pragma unroll
+                for (int e = 0; e < VE; e++) tile[(t * VE + e) * p.P + c] = in[k].e[e];
+            }
+        }
+        __syncthreads();
+        v4u* dst = reinterpret_cast<v4u*>(y + inter0);
+#pragma unroll
+        for (int k = 0; k < NV; k++) {
+            const uint32_t i = threadIdx.x + k * BLOCK;
+            if (i < nflat) st_stream(dst + i, lds_to_flat(i).u);
+        }
+    }
+}
+
 // The same 64 x 64 patch with the widest accesses each side allows: LW elements per load along the source's contiguous
 // dim, SW elements per store along the destination's (each 1, 2, 4 or 8 elements and at most 16 bytes; the launcher
 // checks that every row start and extent on that side is a multiple).  K^T of [B,H,1500,D] in 16 bits, whose destination
@@ -723,6 +835,68 @@ int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uin
     int others[2], no = 0;
     for (int i = 0; i < 3; i++)
         if (i != q) others[no++] = i;
+    {
+        // a short contiguous dim that changes sides (channels): [.., J, C] -> [.., C, J] or back, in 16-byte accesses on both
+        // sides.  [4,1024,1024,5] -> [4,5,1024,1024] f32 took 33 us with the scalar accesses of the LDS-tile kernel.
+        const uint32_t VE = 16u / (uint32_t)elem_bytes;
+        ChannelArgs c;
+        bool fits = false, to_planes = false;
+        uint32_t ea = 1, eb_ = 1;
+        if (dst_shape[q] >= 2 && dst_shape[q] <= 16 && S[3] == dst_shape[q]) {
+            // interleaved source: dst dim q is the channel, dst dim 3 (with dst dim 2 merged in when it continues the run) is J
+            to_planes = true;
+            c.C = dst_shape[q];
+            uint64_t J = dst_shape[3];
+            const bool merged = q != 2 && S[2] == S[3] * dst_shape[3];
+            if (merged) J *= dst_shape[2];
+            ea = dst_shape[others[0]];
+            eb_ = merged ? 1 : dst_shape[others[1]];
+            c.ia = S[others[0]];
+            c.ib = merged ? 0 : S[others[1]];
+            c.pa = dst_strides[others[0]];
+            c.pb = merged ? 0 : dst_strides[others[1]];
+            c.plane = dst_strides[q];
+            fits = J <= 0xffffffffull;
+            c.J = (uint32_t)J;
+        } else if (q == 2 && dst_shape[3] >= 2 && dst_shape[3] <= 16) {
+            // interleaved destination: dst dim 3 is the channel, dst dim 2 (with dst dim 1 merged in) is J
+            c.C = dst_shape[3];
+            uint64_t J = dst_shape[2];
+            const bool merged = S[1] == dst_shape[2];
+            if (merged) J *= dst_shape[1];
+            ea = dst_shape[0];
+            eb_ = merged ? 1 : dst_shape[1];
+            c.ia = dst_strides[0];
+            c.ib = merged ? 0 : dst_strides[1];
+            c.pa = S[0];
+            c.pb = merged ? 0 : S[1];
+            c.plane = S[3];
+            fits = J <= 0xffffffffull;
+            c.J = (uint32_t)J;
+        }
+        if (fits && c.J % VE == 0 && c.ia % VE == 0 && c.ib % VE == 0 && c.pa % VE == 0 && c.pb % VE == 0 && c.plane % VE == 0 &&
+            rt_aligned(x, 16) && rt_aligned(y, 16)) {
+            c.PJ = c.C <= 4 ? 1024 : c.C <= 8 ? 512 : 256;   // PJ * C <= CH_TILE
+            c.P = c.C | 1u;
+            c.cdiv = make_fastdiv(c.C);
+            const uint64_t gj = ((uint64_t)c.J + c.PJ - 1) / c.PJ;
+            const uint64_t blocks = gj * ea * eb_;
+            if (blocks <= 0x7fffffffull) {
+                c.gj = make_fastdiv((uint32_t)gj);
+                c.ob = make_fastdiv(eb_);
+                const dim3 grid((unsigned)blocks), block(BLOCK);
+                if (elem_bytes == 4) {
+                    if (to_planes) hipLaunchKernelGGL((channels_kernel<uint32_t, true>), grid, block, 0, dev->stream, (const uint32_t*)x, (uint32_t*)y, c);
+                    else hipLaunchKernelGGL((channels_kernel<uint32_t, false>), grid, block, 0, dev->stream, (const uint32_t*)x, (uint32_t*)y, c);
+                } else {
+                    if (to_planes) hipLaunchKernelGGL((channels_kernel<uint16_t, true>), grid, block, 0, dev->stream, (const uint16_t*)x, (uint16_t*)y, c);
+                    else hipLaunchKernelGGL((channels_kernel<uint16_t, false>), grid, block, 0, dev->stream, (const uint16_t*)x, (uint16_t*)y, c);
+                }
+                RT_CHECK_LAUNCH("channels_kernel");
+                return RT_OK;
+            }
+        }
+    }
     {
         // The LDS patch kernel where it beats the register transpose below: tensors of 128 MB and more, where one store per
         // thread pays ([8,32,2048,128] f16: 48 -> 45 us; 32-bit ones in larger patches).  (Source rows of 65 to 128 elements

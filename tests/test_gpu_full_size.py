@@ -196,6 +196,12 @@ def test_large_transpose_takes_the_patch_kernel(dev):
     assert same_bits(dev.permute(dev.upload(m), (0, 2, 1)).to_numpy(), m.transpose(0, 2, 1))
     h = rng.standard_normal((2, 2056, 32, 260)).astype(np.float32)
     assert same_bits(dev.permute(dev.upload(h), (0, 2, 3, 1)).to_numpy(), h.transpose(0, 2, 3, 1))
+    # channels to planes and back at image-batch size (a contiguous dim of 5 that changes sides; H and W merge into one run)
+    img = rng.standard_normal((4, 1024, 1024, 5)).astype(np.float16)
+    planes = dev.permute(dev.upload(img), (0, 3, 1, 2))
+    assert same_bits(planes.to_numpy(), img.transpose(0, 3, 1, 2))
+    assert same_bits(dev.permute(planes, (0, 2, 3, 1)).to_numpy(), img)
+    del planes
     # 16-bit tensors of that size whose rows are not whole 128-byte lines stay with the 64 x 64 patches in the widest units
     m16 = rng.standard_normal((1, 8200, 8200)).astype(np.float16)
     assert same_bits(dev.permute(dev.upload(m16), (0, 2, 1)).to_numpy(), m16.transpose(0, 2, 1))

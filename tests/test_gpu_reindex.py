@@ -8,7 +8,7 @@ import itertools
 import numpy as np
 import pytest
 
-from gpu_util import randn
+from gpu_util import randn, same_bits
 
 pytestmark = pytest.mark.gpu
 
@@ -249,3 +249,19 @@ def test_cache_rejects_overflow(dev):
     with pytest.raises(RatchetError) as e:
         dev.cache(c, s, 2, 3)
     assert e.value.status == 4
+
+
+@pytest.mark.parametrize("shape,perm", [((2, 37, 64, 3), (0, 3, 1, 2)), ((1, 33, 40, 5), (0, 3, 1, 2)), ((3, 5, 24, 2), (0, 3, 1, 2)),
+                                        ((2, 8, 32, 16), (0, 3, 1, 2)), ((2, 3, 40, 4), (0, 1, 3, 2)), ((1, 1, 5000, 3), (0, 1, 3, 2)),
+                                        ((2, 3, 16, 40), (0, 2, 3, 1)), ((1, 5, 33, 40), (0, 2, 3, 1)), ((2, 16, 8, 32), (0, 2, 3, 1)),
+                                        ((2, 3, 4, 40), (0, 1, 3, 2)), ((1, 1, 3, 5000), (0, 1, 3, 2)), ((1, 2, 1031, 8, ), (0, 3, 1, 2)),
+                                        ((1, 7, 9, 3), (0, 3, 1, 2)), ((1, 3, 7, 9), (0, 2, 3, 1)), ((1, 300, 300, 3), (0, 3, 1, 2))])
+@pytest.mark.parametrize("np_dt", [np.float32, np.float16])
+def test_permute_channels_to_planes_and_back(dev, shape, perm, np_dt):
+    """[.., J, C] <-> [.., C, J] with 2 to 16 channels (images: [B,H,W,3] <-> [B,3,H,W]): the interleaved side moves as one
+    contiguous run per tile, the planar side as C runs, both in 16-byte accesses; with and without the neighbouring dim
+    merged into J, tiles that end early, and extents that are not whole vectors (which keep the element-wise tile kernel)"""
+    rng = np.random.default_rng(95)
+    x = rng.standard_normal(shape).astype(np_dt)
+    got = dev.permute(dev.upload(x), perm).to_numpy()
+    assert same_bits(got, np.ascontiguousarray(x.transpose(perm))), (shape, perm)
