@@ -101,12 +101,23 @@ constexpr int TILE_ELEMS = 4096;
 struct TransposeArgs {
     uint32_t nq, n3;         // extents of dst dim q and dst dim 3
     uint64_t s3;             // source stride (elements) of the dim that becomes dst dim 3
+    // dst dim 3 may stand for two dst dims merged (the destination is contiguous across them, the source is not): index j
+    // of it lies at (j / inner) * s2 + (j % inner) * s3 in the source.  Plain: inner = 1, s2 = s3.  (tr_row; the kernels
+    // that take whole-vector rows use s3 alone and are not launched on a merged dim.)
+    FastDiv inner;
+    uint64_t s2;
     uint64_t dq;             // destination stride (elements) of dim q
     FastDiv gx, gy;          // tile counts along dst dim q and dst dim 3 (blockIdx.x = (z * gy + ty) * gx + tx)
     FastDiv ob;              // extent of the second "other" dim (other dims = (oa, ob), ob fastest)
     uint64_t sa, sb;         // source strides of the other dims
     uint64_t da, db;         // destination strides of the other dims
 };
+
+__device__ __forceinline__ uint64_t tr_row(const TransposeArgs& p, uint32_t j) {
+    uint32_t hi, lo;
+    fd_divmod(j, p.inner, hi, lo);
+    return (uint64_t)hi * p.s2 + (uint64_t)lo * p.s3;
+}
 
 template <typename ElemT, int TQ>
 __global__ void __launch_bounds__(BLOCK) transpose_kernel(const ElemT* __restrict__ x, ElemT* __restrict__ y, TransposeArgs p) {
@@ -125,7 +136,7 @@ __global__ void __launch_bounds__(BLOCK) transpose_kernel(const ElemT* __restric
     for (uint32_t i = threadIdx.x; i < TILE_ELEMS; i += BLOCK) {
         const uint32_t r = i / TQ, c = i % TQ;
         const uint32_t j = j0 + r, q = q0 + c;
-        if (j < p.n3 && q < p.nq) tile[r][c] = x[src0 + (uint64_t)j * p.s3 + q];
+        if (j < p.n3 && q < p.nq) tile[r][c] = x[src0 + tr_row(p, j) + q];
     }
     __syncthreads();
     // write: rows = dst dim q, columns = dst dim 3 (contiguous in the destination)
@@ -279,7 +290,7 @@ __global__ void __launch_bounds__(BLOCK) transpose_wide_kernel(const ElemT* __re
         const uint32_t i = threadIdx.x + k * BLOCK;
         const uint32_t r = i / (TQ / LW), c = (i % (TQ / LW)) * LW;
         const uint32_t j = j0 + r, q = q0 + c;
-        if ((LOADS % BLOCK == 0 || i < LOADS) && j < p.n3 && q < p.nq) in[k] = *reinterpret_cast<const LoadT*>(x + src0 + (uint64_t)j * p.s3 + q);
+        if ((LOADS % BLOCK == 0 || i < LOADS) && j < p.n3 && q < p.nq) in[k] = *reinterpret_cast<const LoadT*>(x + src0 + tr_row(p, j) + q);
     }
 #pragma unroll
     for (int k = 0; k < NL; k++) {
@@ -897,6 +908,26 @@ int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uin
             }
         }
     }
+    // A short dst dim 3 (fewer than 64 elements) behind a dst dim 2 that is not the source's contiguous one: the two are
+    // one contiguous run in the destination, so they are transposed against dim q as one dim whose source offset has two
+    // levels ([8,32,512,80] -> perm (1,3,2,0) = [32,80,512,8]: rows of 8 elements became rows of 4096; 56 -> 11 us in f16, the reversal (3,2,1,0) of that shape 61 -> 12 us).
+    bool merged23 = false;
+    uint32_t inner23 = 1;
+    uint64_t s_outer23 = 0;
+    if (q != 2 && dst_shape[3] < 64 && dst_shape[2] > 1 && (uint64_t)dst_shape[2] * dst_shape[3] <= 0xffffffffull) {
+        merged23 = true;
+        inner23 = dst_shape[3];
+        s_outer23 = S[2];
+        const uint32_t d0 = dst_shape[0], d1 = dst_shape[1], d23 = dst_shape[2] * dst_shape[3];
+        const uint64_t s0 = S[0], s1 = S[1], s3 = S[3];
+        dst_shape[0] = 1; dst_shape[1] = d0; dst_shape[2] = d1; dst_shape[3] = d23;
+        S[0] = 0; S[1] = s0; S[2] = s1; S[3] = s3;
+        q += 1;
+        contiguous_strides(dst_shape, dst_strides);
+        no = 0;
+        for (int i = 0; i < 3; i++)
+            if (i != q) others[no++] = i;
+    }
     {
         // The LDS patch kernel where it beats the register transpose below: tensors of 128 MB and more, where one store per
         // thread pays ([8,32,2048,128] f16: 48 -> 45 us; 32-bit ones in larger patches).  (Source rows of 65 to 128 elements
@@ -910,9 +941,11 @@ int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uin
         // kernel's 128-byte runs, each across two lines there, do not beat: [1,8200,8200] f16 154 -> 97 us, [4,4104,4104]
         // 128 -> 87 us, [1,8192,8200] 82 -> 61 us; 32-bit ones gain nothing from it)
         const bool lines16 = elem_bytes == 4 || ((uint64_t)dst_shape[q] * elem_bytes % 128 == 0 && (uint64_t)dst_shape[3] * elem_bytes % 128 == 0);
-        if (total >= (128ull << 20) && !short_row && lines16 && dst_shape[q] % V == 0 && dst_shape[3] % V == 0 &&
+        if (!merged23 && total >= (128ull << 20) && !short_row && lines16 && dst_shape[q] % V == 0 && dst_shape[3] % V == 0 &&
             S[3] % V == 0 && S[others[0]] % V == 0 && S[others[1]] % V == 0 && rt_aligned(x, 16) && rt_aligned(y, 16)) {
             TransposeArgs p;
+            p.inner = make_fastdiv(1);
+            p.s2 = S[3];
             p.nq = dst_shape[q];
             p.n3 = dst_shape[3];
             p.s3 = S[3];
@@ -962,7 +995,7 @@ int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uin
         const bool whole_lines = (uint64_t)dst_shape[q] * elem_bytes % 128 == 0 && (uint64_t)dst_shape[3] * elem_bytes % 128 == 0;
         uint32_t qb = dst_shape[q] / V <= 12 ? dst_shape[q] / V : 8, jb = 64 / (qb ? qb : 1);
         if (jb > dst_shape[3] / V) jb = dst_shape[3] / V;
-        if (dst_shape[q] % V == 0 && dst_shape[3] % V == 0 && rt_aligned(x, 16) && rt_aligned(y, 16) && qb * jb >= 32 && whole_lines) {
+        if (!merged23 && dst_shape[q] % V == 0 && dst_shape[3] % V == 0 && rt_aligned(x, 16) && rt_aligned(y, 16) && qb * jb >= 32 && whole_lines) {
             TransposeRegArgs r;
             r.nqb = dst_shape[q] / V;
             r.njb = dst_shape[3] / V;
@@ -997,6 +1030,8 @@ int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uin
     p.nq = dst_shape[q];
     p.n3 = dst_shape[3];
     p.s3 = S[3];
+    p.inner = make_fastdiv(inner23);
+    p.s2 = merged23 ? s_outer23 : S[3];
     p.dq = dst_strides[q];
     p.ob = make_fastdiv(dst_shape[others[1]]);
     p.sa = S[others[0]];
@@ -1012,7 +1047,9 @@ int rt_permute(rt_device* dev, int elem_bytes, const void* x, void* y, const uin
             while (w > 1 && (extent % w || s0 % w || s1 % w || s2 % w || !rt_aligned(base, (size_t)w * elem_bytes))) w >>= 1;
             return w;
         };
-        const int lw = width(p.nq, p.s3, p.sa, p.sb, x), sw = width(p.n3, p.dq, p.da, p.db, y);
+        int lw = width(p.nq, p.s3, p.sa, p.sb, x);
+        while (lw > 1 && p.s2 % lw) lw >>= 1;
+        const int sw = width(p.n3, p.dq, p.da, p.db, y);
         if (lw > 1 || sw > 1) {
             // a source row of 65 to 128 elements in whole vectors: one patch across it
             const int lw_max = 16 / elem_bytes;

@@ -265,3 +265,16 @@ def test_permute_channels_to_planes_and_back(dev, shape, perm, np_dt):
     x = rng.standard_normal(shape).astype(np_dt)
     got = dev.permute(dev.upload(x), perm).to_numpy()
     assert same_bits(got, np.ascontiguousarray(x.transpose(perm))), (shape, perm)
+
+
+@pytest.mark.parametrize("shape", [(4, 6, 40, 24), (2, 3, 70, 5), (8, 16, 64, 80), (3, 33, 9, 130)])
+@pytest.mark.parametrize("np_dt", [np.float32, np.float16])
+def test_permute_every_order_of_four_dims(dev, shape, np_dt):
+    """all 24 orders, among them those that end in a short dim behind one that is not the source's contiguous dim (the two
+    are transposed as one merged dim whose source offset has two levels)"""
+    rng = np.random.default_rng(96)
+    x = rng.standard_normal(shape).astype(np_dt)
+    dx = dev.upload(x)
+    for perm in itertools.permutations(range(4)):
+        got = dev.permute(dx, perm).to_numpy()
+        assert same_bits(got, np.ascontiguousarray(x.transpose(perm))), (shape, perm)
