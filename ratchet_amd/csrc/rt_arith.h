@@ -76,7 +76,10 @@ template <> struct Ar<bf16_t> {
 template <typename T> __device__ __forceinline__ T ar_tanh(T a) { return Ar<T>::conv(rt_tanhf(Ar<T>::widen(a))); }
 // (tab: the table of rt_expf_tab, where a kernel has staged a copy of it)
 template <typename T> __device__ __forceinline__ T ar_exp(T a, const uint64_t* tab = rt_exp2f_tab) { return Ar<T>::conv(rt_expf_tab(Ar<T>::widen(a), tab)); }
-template <typename T> __device__ __forceinline__ T ar_log(T a) { return Ar<T>::conv(rt_logf(Ar<T>::widen(a))); }
+// (tab: the 32 words of rt_logf_tab, wherever the caller keeps them)
+template <typename T> __device__ __forceinline__ T ar_log(T a, const uint64_t* tab = nullptr) {
+    return Ar<T>::conv(tab ? rt_logf_tab_at(Ar<T>::widen(a), reinterpret_cast<const double*>(tab)) : rt_logf(Ar<T>::widen(a)));
+}
 template <typename T> __device__ __forceinline__ T ar_sin(T a) { return Ar<T>::conv(rt_sinf(Ar<T>::widen(a))); }
 template <typename T> __device__ __forceinline__ T ar_cos(T a) { return Ar<T>::conv(rt_cosf(Ar<T>::widen(a))); }
 template <typename T> __device__ __forceinline__ T ar_sqrt(T a) { return Ar<T>::conv(__builtin_sqrtf(Ar<T>::widen(a))); }
@@ -103,11 +106,12 @@ template <typename T> __device__ __forceinline__ T ar_sigmoid(T x, const uint64_
 }
 
 constexpr bool ar_unary_uses_exp(int op) { return op == RT_EXP || op == RT_SILU || op == RT_SIGMOID; }
+constexpr bool ar_unary_uses_log(int op) { return op == RT_LOG; }
 template <int OP, typename T> __device__ __forceinline__ T ar_unary(T x, const uint64_t* tab = rt_exp2f_tab) {
     if (OP == RT_GELU) return ar_gelu<T>(x);
     if (OP == RT_TANH) return ar_tanh<T>(x);
     if (OP == RT_EXP) return ar_exp<T>(x, tab);
-    if (OP == RT_LOG) return ar_log<T>(x);
+    if (OP == RT_LOG) return ar_log<T>(x, tab == rt_exp2f_tab ? nullptr : tab);
     if (OP == RT_SIN) return ar_sin<T>(x);
     if (OP == RT_COS) return ar_cos<T>(x);
     if (OP == RT_ABS) return Ar<T>::abs(x);

@@ -184,12 +184,13 @@ __global__ void __launch_bounds__(BLOCK) unary_vec_kernel(const T* __restrict__ 
         const uint64_t i = base + (uint64_t)k * BLOCK;
         if (i < nvec) rx[k].u = ld_stream(xv + i);
     }
-    // exp, SiLU and sigmoid look 2^(i/32) up once per element: from a copy of the table in LDS
-    constexpr bool TAB = ar_unary_uses_exp(OP);
+    // exp, SiLU and sigmoid look 2^(i/32) up once per element, log its (1/c, log c): from a copy of the table in LDS
+    constexpr bool TAB = ar_unary_uses_exp(OP) || ar_unary_uses_log(OP);
     __shared__ uint64_t exp_tab[TAB ? 32 : 1];
     const uint64_t* tab = rt_exp2f_tab;
     if (TAB) {
-        if (threadIdx.x < 32) exp_tab[threadIdx.x] = rt_exp2f_tab[threadIdx.x];
+        if (threadIdx.x < 32)
+            exp_tab[threadIdx.x] = ar_unary_uses_log(OP) ? __builtin_bit_cast(uint64_t, rt_logf_tab[threadIdx.x]) : rt_exp2f_tab[threadIdx.x];
         __syncthreads();
         tab = exp_tab;
     }

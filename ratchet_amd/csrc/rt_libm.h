@@ -208,10 +208,47 @@ RT_FN float rt_expf_tab(float x, const uint64_t* tab) {
 
 RT_FN float rt_expf(float x) { return rt_expf_tab(x, rt_exp2f_tab); }
 
-// log / sin / cos: evaluated in double and rounded once.  The double routines are accurate to about 1 ulp of
-// double, so the float result is the correctly rounded one except in astronomically rare double-rounding cases;
-// glibc's logf/sinf/cosf are within 1 float ulp of that.
-RT_FN float rt_logf(float x) { return (float)log((double)x); }
+// logf as glibc computes it (sysdeps/ieee754/flt-32/e_logf.c, the algorithm of ARM's optimized routines): x = 2^k * z
+// with z in [0x1.66p-1, 0x1.66p0), c = the centre of the sixteenth of that interval z lies in, with 1/c and log(c) from
+// a table; log(x) = log1p(z/c - 1) + log(c) + k ln 2, a cubic in r = z/c - 1, all in double, rounded once.  Without a
+// branch: the evaluation runs for every input (a subnormal one scaled by 2^23 first) and the special cases are
+// selected afterwards.  Equal to this machine's logf on all 2^32 inputs (tests/device_math_check.cpp).
+RT_TABLE double rt_logf_tab[32] = {
+    0x1.661ec79f8f3bep+0, -0x1.57bf7808caadep-2, 0x1.571ed4aaf883dp+0, -0x1.2bef0a7c06ddbp-2, 0x1.49539f0f010bp+0,  -0x1.01eae7f513a67p-2,
+    0x1.3c995b0b80385p+0, -0x1.b31d8a68224e9p-3, 0x1.30d190c8864a5p+0, -0x1.6574f0ac07758p-3, 0x1.25e227b0b8eap+0,  -0x1.1aa2bc79c81p-3,
+    0x1.1bb4a4a1a343fp+0, -0x1.a4e76ce8c0e5ep-4, 0x1.12358f08ae5bap+0, -0x1.1973c5a611cccp-4, 0x1.0953f419900a7p+0, -0x1.252f438e10c1ep-5,
+    0x1p+0,               0x0p+0,                0x1.e608cfd9a47acp-1, 0x1.aa5aa5df25984p-5,  0x1.ca4b31f026aap-1,  0x1.c5e53aa362eb4p-4,
+    0x1.b2036576afce6p-1, 0x1.526e57720db08p-3,  0x1.9c2d163a1aa2dp-1, 0x1.bc2860d22477p-3,   0x1.886e6037841edp-1, 0x1.1058bc8a07ee1p-2,
+    0x1.767dcf5534862p-1, 0x1.4043057b6ee09p-2,
+};
+
+RT_FN float rt_logf_tab_at(float x, const double* tab) {
+    const double A0 = -0x1.00ea348b88334p-2, A1 = 0x1.5575b0be00b6ap-2, A2 = -0x1.ffffef20a4123p-2, LN2 = 0x1.62e42fefa39efp-1;
+    uint32_t ix = f2u(x);
+    const bool sub = ix < 0x00800000u;                        // subnormal (or zero, replaced below): scaled up by 2^23
+    const uint32_t scaled = f2u(x * 0x1p23f) - (23u << 23);
+    uint32_t iw = sub ? scaled : ix;
+    const uint32_t tmp = iw - 0x3f330000u;
+    const uint32_t i = (tmp >> 19) & 15u;
+    const int32_t k = (int32_t)tmp >> 23;                     // arithmetic shift
+    const uint32_t iz = iw - (tmp & 0xff800000u);
+    const double invc = tab[2 * i], logc = tab[2 * i + 1];
+    const double z = (double)u2f(iz);
+    const double r = z * invc - 1.0;
+    const double y0 = logc + (double)k * LN2;
+    const double r2 = r * r;
+    double y = A1 * r + A2;
+    y = A0 * r2 + y;
+    y = y * r2 + (y0 + r);
+    float res = (float)y;
+    res = ix == 0x3f800000u ? 0.0f : res;                     // log(1) = +0 exactly
+    res = ix == 0x7f800000u ? x : res;                        // +inf
+    res = (ix & 0x80000000u) != 0 || ix > 0x7f800000u ? (x - x) / 0.0f : res;      // negative or NaN: NaN
+    res = (ix << 1) == 0 ? -__builtin_huge_valf() : res;      // +-0: -inf
+    return res;
+}
+
+RT_FN float rt_logf(float x) { return rt_logf_tab_at(x, rt_logf_tab); }
 RT_FN float rt_sinf(float x) { return (float)sin((double)x); }
 RT_FN float rt_cosf(float x) { return (float)cos((double)x); }
 
