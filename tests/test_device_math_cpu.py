@@ -15,5 +15,7 @@ def test_device_math_matches_the_c_library(tmp_path):
     run = subprocess.run([str(exe), "101"], capture_output=True, text=True)
     assert run.returncode == 0, run.stdout + run.stderr
     fields = run.stdout.split()
-    assert fields[0] == "tanhf" and int(fields[1]) == 0 and int(fields[3]) == 0 and int(fields[5]) == 0 and int(fields[7]) == 0, run.stdout
-    assert int(fields[9]) > 40_000_000
+    counts = dict(zip(fields[0::2], (int(v) for v in fields[1::2])))
+    assert set(counts) == {"tanhf", "expm1f", "expf", "logf", "f2bf", "checked"}, run.stdout
+    assert all(counts[k] == 0 for k in ("tanhf", "expm1f", "expf", "logf", "f2bf")), run.stdout
+    assert counts["checked"] > 40_000_000
