@@ -164,6 +164,52 @@ __global__ void __launch_bounds__(BLOCK) binary_bcast_kernel(const T* __restrict
     }
 }
 
+// Rows that are not whole vectors (a last dim of 1001), one operand of y's own shape and the other broadcast: the output
+// and the full operand are taken as flat arrays in 16-byte vectors, whatever the row length, and only the broadcast
+// operand is read element by element (it is the small one and stays in the caches).  A_FULL: a is the full operand.
+// [4,4096,1001] + [1001] in f16: 33 -> 20 us against the element-wise kernel, + [4,4096,1]: 33 -> 14 us; f32: 5.2 TB/s.
+template <typename T, int OP, bool A_FULL>
+__global__ void __launch_bounds__(BLOCK) binary_flat_kernel(const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ y, BcastArgs p,
+                                                            uint64_t numel) {
+    constexpr int VE = 16 / sizeof(T);
+    const T* full = A_FULL ? a : b;
+    const T* part = A_FULL ? b : a;
+    const uint32_t* ps = A_FULL ? p.bs : p.as;
+    const uint64_t v = (uint64_t)blockIdx.x * BLOCK + threadIdx.x;
+    const uint64_t f0 = v * VE;
+    if (f0 >= numel) return;
+    // position of the vector's first element; p.cv divides by the whole last dim here
+    uint32_t row, col, i0, i1, i2, t;
+    fd_divmod((uint32_t)f0, p.cv, row, col);
+    fd_divmod(row, p.d2, t, i2);
+    fd_divmod(t, p.d1, i0, i1);
+    uint64_t off = (uint64_t)i0 * ps[0] + (uint64_t)i1 * ps[1] + (uint64_t)i2 * ps[2] + (uint64_t)col * ps[3];
+    const uint32_t d3 = p.cv.d;
+    T pv[VE];
+#pragma unroll
+    for (int e = 0; e < VE; e++) {
+        pv[e] = part[off];
+        off += ps[3];
+        if (++col == d3 && e + 1 < VE) {                     // the next element starts a row
+            col = 0;
+            fd_divmod((uint32_t)f0 + e + 1, p.cv, row, t);
+            fd_divmod(row, p.d2, t, i2);
+            fd_divmod(t, p.d1, i0, i1);
+            off = (uint64_t)i0 * ps[0] + (uint64_t)i1 * ps[1] + (uint64_t)i2 * ps[2];
+        }
+    }
+    if (f0 + VE <= numel) {
+        Vec16<T> fv, out;
+        fv.u = ld_stream(reinterpret_cast<const v4u*>(full + f0));
+#pragma unroll
+        for (int e = 0; e < VE; e++) out.e[e] = A_FULL ? ar_binary<OP, T>(fv.e[e], pv[e]) : ar_binary<OP, T>(pv[e], fv.e[e]);
+        st_stream(reinterpret_cast<v4u*>(y + f0), out.u);
+    } else {
+        for (int e = 0; e < VE && f0 + e < numel; e++)       // the tensor's last, partial vector
+            y[f0 + e] = A_FULL ? ar_binary<OP, T>(full[f0 + e], pv[e]) : ar_binary<OP, T>(pv[e], full[f0 + e]);
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ unary
 // VIA32: the caller pattern x.full().<op>().cast(dt) on a 16-bit tensor in one pass: widen, the f32 op, one rounding
 template <typename T, int OP, bool VIA32> __device__ __forceinline__ T apply_unary(T v, const uint64_t* tab = rt_exp2f_tab) {
@@ -825,6 +871,15 @@ int launch_bcast(rt_device* dev, const void* a, const uint32_t a_shape[4], const
     // one access per thread for a full-size operand of 1 GiB or more plus a broadcast one (measured on the [1,32,4096,4096]
     // scores + [4096,4096] mask inside the benchmark step: 343-345 us against 346-351 us with two); below that, and for
     // the other operand patterns, the two are level
+    if (ve == 1 && VEMAX > 1 && a_once != b_once && rt_aligned(y, 16) && rt_aligned(a_once ? a : b, 16) && y_numel <= 0xffffffffull) {
+        // rows that are not whole vectors, one operand of y's shape: flat vectors for it and for y
+        p.cv = make_fastdiv(y_shape[3]);
+        const unsigned fblocks = blocks_for((y_numel + VEMAX - 1) / VEMAX, BLOCK);
+        if (a_once) hipLaunchKernelGGL((binary_flat_kernel<T, OP, true>), dim3(fblocks), dim3(BLOCK), 0, dev->stream, (const T*)a, (const T*)b, (T*)y, p, y_numel);
+        else hipLaunchKernelGGL((binary_flat_kernel<T, OP, false>), dim3(fblocks), dim3(BLOCK), 0, dev->stream, (const T*)a, (const T*)b, (T*)y, p, y_numel);
+        RT_CHECK_LAUNCH("binary_flat_kernel");
+        return RT_OK;
+    }
     const int unroll = (a_once != b_once && ve == VEMAX && nvec >= BC_ONE_FROM_VECS) ? 1 : BC_UNROLL;
     const unsigned blocks = blocks_for(nvec, BLOCK * unroll);
     // one operand full-size, the other equal to y's trailing dims and repeated over the leading ones, too large for

@@ -97,6 +97,30 @@ def test_binary_broadcast_fused(dev, oracle, dtype):
         assert same_bits(got, want), (sa, sb)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
+def test_binary_broadcast_against_rows_that_are_not_whole_vectors(dev, oracle, dtype, op):
+    """one operand of the output's shape, a last dim that is not a multiple of the vector length: the full operand and the output
+    move as flat 16-byte vectors and the broadcast operand element by element; both operand orders, every broadcast pattern,
+    a tensor whose size is not a whole vector, rows shorter than a vector, in place"""
+    rng = np.random.default_rng(105)
+    cases = [((4, 33, 1001), (1001,)), ((1001,), (4, 33, 1001)), ((4, 33, 1001), (4, 33, 1)), ((3, 7, 5, 13), (3, 1, 5, 1)),
+             ((2, 3, 4, 5), (1, 3, 1, 1)), ((1, 3, 1, 1), (2, 3, 4, 5)), ((9, 3), (3,)), ((77, 1), (1,)), ((5, 6, 7), (6, 1)),
+             ((2, 50, 3, 999), (2, 1, 3, 999)), ((64, 3, 31, 31), (1, 3, 1, 1))]
+    for sa, sb in cases:
+        a, b = randn(rng, sa, dtype), randn(rng, sb, dtype)
+        if op == "div":
+            b = np.where(np.abs(b) < 0.1, dtype(0.5), b)
+        out_shape = np.broadcast_shapes(sa, sb)
+        want = oracle.binary(op, np.ascontiguousarray(np.broadcast_to(a, out_shape)), np.ascontiguousarray(np.broadcast_to(b, out_shape)))
+        da, db = dev.upload(a), dev.upload(b)
+        got = dev.binary(op, da, db).to_numpy()
+        assert same_bits(got, want), (op, sa, sb)
+        full = da if tuple(sa) == tuple(out_shape) else db
+        dev.binary(op, da, db, out=full)                                 # in place on the full operand
+        assert same_bits(full.to_numpy(), want), (op, sa, sb, "in place")
+
+
 UNARY = ["gelu", "tanh", "exp", "log", "sin", "cos", "abs", "sqrt", "relu", "floor", "ceil", "neg", "silu", "sigmoid"]
 EXACT32 = {"gelu", "tanh", "exp", "log", "abs", "sqrt", "relu", "floor", "ceil", "neg", "silu", "sigmoid"}
 
