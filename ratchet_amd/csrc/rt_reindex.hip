@@ -679,6 +679,41 @@ inline void contiguous_strides(const uint32_t shape[4], uint64_t out[4]) {
 }
 
 // Launches the gather dst[i] = src[base + sum i_k * S_k] (all in elements) choosing the widest usable vector.
+// Rows that start or end off the vector grid (a slice to columns 3 .. 69): the destination is contiguous, so it is written
+// as flat 16-byte vectors whatever the row length, and only the source is read element by element.  p.d3 divides by the
+// whole last dim, p.s and p.base are in elements here.  [4,32,2048,80] sliced to columns 3 .. 69 in f16: 39.8 -> 21.3 us
+// against element-wise stores, in f32 42.2 -> 27.7 us.
+template <typename ET>
+__global__ void __launch_bounds__(BLOCK) gather_flat_kernel(const ET* __restrict__ x, ET* __restrict__ y, GatherArgs p, uint64_t numel) {
+    constexpr int VE = 16 / (int)sizeof(ET);
+    const uint64_t f0 = ((uint64_t)blockIdx.x * BLOCK + threadIdx.x) * VE;
+    if (f0 >= numel) return;
+    uint32_t row, col, i0, i1, i2, t;
+    fd_divmod((uint32_t)f0, p.d3, row, col);
+    fd_divmod(row, p.d2, t, i2);
+    fd_divmod(t, p.d1, i0, i1);
+    uint64_t off = p.base + (uint64_t)i0 * p.s[0] + (uint64_t)i1 * p.s[1] + (uint64_t)i2 * p.s[2] + (uint64_t)col * p.s[3];
+    const uint32_t d3 = p.d3.d;
+    Vec16<ET> out;
+#pragma unroll
+    for (int e = 0; e < VE; e++) {
+        out.e[e] = (f0 + e < numel) ? x[off] : (ET)0;
+        off += p.s[3];
+        if (++col == d3 && e + 1 < VE) {                     // the next element starts a row
+            col = 0;
+            fd_divmod((uint32_t)f0 + e + 1, p.d3, row, t);
+            fd_divmod(row, p.d2, t, i2);
+            fd_divmod(t, p.d1, i0, i1);
+            off = p.base + (uint64_t)i0 * p.s[0] + (uint64_t)i1 * p.s[1] + (uint64_t)i2 * p.s[2];
+        }
+    }
+    if (f0 + VE <= numel) {
+        st_stream(reinterpret_cast<v4u*>(y + f0), out.u);
+    } else {
+        for (int e = 0; e < VE && f0 + e < numel; e++) y[f0 + e] = out.e[e];
+    }
+}
+
 int launch_gather(rt_device* dev, int eb, const void* x, void* y, const uint32_t dst_shape_in[4], const uint64_t S_in[4],
                   uint64_t base_elems, const char* who) {
     // Drop size-1 dims and merge neighbours that are contiguous on both sides (the destination always is): a slice of
@@ -730,6 +765,24 @@ int launch_gather(rt_device* dev, int eb, const void* x, void* y, const uint32_t
     const uint64_t nvec = n / per;
     RT_REQUIRE(nvec <= 0xffffffffull - (uint64_t)BLOCK * UNROLL, RT_ERR_SIZE, "%s: %llu vectors exceed the 32-bit index space",
                who, (unsigned long long)nvec);
+    if (!splat && contiguous_last && vb == eb && eb < 16 && rt_aligned(y, 16) && n <= 0xfffffff0ull && n * (uint64_t)eb >= (1u << 20)) {
+        // element-wise on both sides otherwise: flat vectors for the destination
+        GatherArgs f;
+        f.d3 = make_fastdiv(dst_shape[3]);
+        f.d2 = make_fastdiv(dst_shape[2]);
+        f.d1 = make_fastdiv(dst_shape[1]);
+        f.base = base_elems;
+        for (int i = 0; i < 4; i++) f.s[i] = dst_shape[i] > 1 ? S[i] : 0;
+        f.nvec = 0;
+        f.rm_h = make_fastdiv(1);
+        f.rm_j = 0;
+        const uint32_t ve = 16u / (uint32_t)eb;
+        const unsigned fblocks = blocks_for((n + ve - 1) / ve, BLOCK);
+        if (eb == 4) hipLaunchKernelGGL((gather_flat_kernel<uint32_t>), dim3(fblocks), dim3(BLOCK), 0, dev->stream, (const uint32_t*)x, (uint32_t*)y, f, n);
+        else hipLaunchKernelGGL((gather_flat_kernel<uint16_t>), dim3(fblocks), dim3(BLOCK), 0, dev->stream, (const uint16_t*)x, (uint16_t*)y, f, n);
+        RT_CHECK_LAUNCH(who);
+        return RT_OK;
+    }
     GatherArgs p;
     p.d3 = make_fastdiv(dst_shape[3] / per);
     p.d2 = make_fastdiv(dst_shape[2]);
