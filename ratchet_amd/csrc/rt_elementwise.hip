@@ -188,7 +188,7 @@ __global__ void __launch_bounds__(BLOCK) binary_flat_kernel(const T* __restrict_
     T pv[VE];
 #pragma unroll
     for (int e = 0; e < VE; e++) {
-        pv[e] = part[off];
+        pv[e] = part[f0 + e < numel ? off : 0];              // (nothing is read past the tensor's last element)
         off += ps[3];
         if (++col == d3 && e + 1 < VE) {                     // the next element starts a row
             col = 0;
@@ -871,7 +871,7 @@ int launch_bcast(rt_device* dev, const void* a, const uint32_t a_shape[4], const
     // one access per thread for a full-size operand of 1 GiB or more plus a broadcast one (measured on the [1,32,4096,4096]
     // scores + [4096,4096] mask inside the benchmark step: 343-345 us against 346-351 us with two); below that, and for
     // the other operand patterns, the two are level
-    if (ve == 1 && VEMAX > 1 && a_once != b_once && rt_aligned(y, 16) && rt_aligned(a_once ? a : b, 16) && y_numel <= 0xffffffffull) {
+    if (ve == 1 && VEMAX > 1 && a_once != b_once && rt_aligned(y, 16) && rt_aligned(a_once ? a : b, 16) && y_numel <= 0xfffffff0ull) {
         // rows that are not whole vectors, one operand of y's shape: flat vectors for it and for y
         p.cv = make_fastdiv(y_shape[3]);
         const unsigned fblocks = blocks_for((y_numel + VEMAX - 1) / VEMAX, BLOCK);

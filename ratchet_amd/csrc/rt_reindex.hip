@@ -697,7 +697,7 @@ __global__ void __launch_bounds__(BLOCK) gather_flat_kernel(const ET* __restrict
     Vec16<ET> out;
 #pragma unroll
     for (int e = 0; e < VE; e++) {
-        out.e[e] = (f0 + e < numel) ? x[off] : (ET)0;
+        out.e[e] = x[f0 + e < numel ? off : p.base];         // (nothing is read past the slice's last element)
         off += p.s[3];
         if (++col == d3 && e + 1 < VE) {                     // the next element starts a row
             col = 0;
