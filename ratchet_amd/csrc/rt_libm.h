@@ -249,8 +249,71 @@ RT_FN float rt_logf_tab_at(float x, const double* tab) {
 }
 
 RT_FN float rt_logf(float x) { return rt_logf_tab_at(x, rt_logf_tab); }
-RT_FN float rt_sinf(float x) { return (float)sin((double)x); }
-RT_FN float rt_cosf(float x) { return (float)cos((double)x); }
+// sinf / cosf as glibc computes them (sysdeps/ieee754/flt-32/s_sinf.c, s_cosf.c, s_sincosf.h: the algorithm of ARM's
+// optimized routines): the argument reduced to [-pi/4, pi/4] in double (one multiply and a rounded quadrant below 120,
+// a 192-bit slice of 4/pi above), a degree-7 sine or degree-8 cosine polynomial in double picked by the quadrant, one
+// rounding to float.
+RT_TABLE uint32_t rt_inv_pio4[24] = {0xa2,       0xa2f9,     0xa2f983,   0xa2f9836e, 0xf9836e4e, 0x836e4e44, 0x6e4e4415, 0x4e441529,
+                                     0x441529fc, 0x1529fc27, 0x29fc2757, 0xfc2757d1, 0x2757d1f5, 0x57d1f534, 0xd1f534dd, 0xf534ddc0,
+                                     0x34ddc0db, 0xddc0db62, 0xc0db6295, 0xdb629599, 0x6295993c, 0x95993c43, 0x993c4390, 0x3c439041};
+
+// the polynomial of quadrant n on the reduced x (x2 = x * x): sine for even n, cosine for odd n; neg: quadrants 2 and 3,
+// whose cosine coefficients carry the other sign (the same as negating the value: every step is symmetric in the sign).
+// Both are evaluated and one is selected: the lanes of a wave lie in different quadrants.
+RT_FN float rt_sincosf_poly(double x, double x2, int n, bool neg) {
+    const double S1 = -0x1.555545995a603p-3, S2 = 0x1.1107605230bc4p-7, S3 = -0x1.994eb3774cf24p-13;
+    const double C0 = 0x1p0, C1 = -0x1.ffffffd0c621cp-2, C2 = 0x1.55553e1068f19p-5, C3 = -0x1.6c087e89a359dp-10, C4 = 0x1.99343027bf8c3p-16;
+    const double x3 = x * x2;
+    const double s1 = S2 + x2 * S3;
+    const double x7 = x3 * x2;
+    const double s = x + x3 * S1;
+    const double sinv = s + x7 * s1;
+    const double x4 = x2 * x2;
+    const double c2 = C3 + x2 * C4;
+    const double c1 = C0 + x2 * C1;
+    const double x6 = x4 * x2;
+    const double c = c1 + x4 * C2;
+    const double cosv = c + x6 * c2;
+    return (float)((n & 1) ? (neg ? -cosv : cosv) : sinv);
+}
+
+// COS: 0 sine, 1 cosine.  The reduction below 120 runs for every input (with 0 in place of larger ones) and covers
+// |y| < pi/4 too (quadrant 0, x unchanged); only the slice-of-4/pi reduction of larger arguments sits behind a branch.
+template <int COS> RT_FN float rt_sincosf(float y) {
+    const uint32_t xi = f2u(y);
+    const uint32_t top = (xi >> 20) & 0x7ffu;
+    const bool large = top >= 0x42fu;                         // |y| >= 120, inf, NaN
+    double x = large ? 0.0 : (double)y;
+    const double r = x * 0x1.45F306DC9C883p+23;               // quadrant from x * (2/pi) * 2^24, rounded
+    int n = ((int32_t)r + 0x800000) >> 24;
+    x = __builtin_fma(-(double)n, 0x1.921FB54442D18p0, x);     // one rounding, as the C library's build for FMA hardware does it
+    int sign = 0;
+    if (large && top < 0x7f8u) {
+        const uint32_t* arr = &rt_inv_pio4[(xi >> 26) & 15];
+        const int shift = (int)((xi >> 23) & 7);
+        uint32_t m = (xi & 0xffffffu) | 0x800000u;
+        m <<= shift;
+        uint64_t res0 = (uint64_t)(uint32_t)(m * arr[0]);
+        const uint64_t res1 = (uint64_t)m * arr[4];
+        const uint64_t res2 = (uint64_t)m * arr[8];
+        res0 = (res2 >> 32) | (res0 << 32);
+        res0 += res1;
+        const uint64_t q = (res0 + (1ull << 61)) >> 62;
+        res0 -= q << 62;
+        x = (double)(int64_t)res0 * 0x1.921FB54442D18p-62;
+        n = (int)q;
+        sign = (int)(xi >> 31);
+    }
+    const int ns = n + sign;
+    const double s = ((ns & 3) == 1 || (ns & 3) == 2) ? -1.0 : 1.0;          // sign of sine in quadrants 0..3: + - - +
+    float res = rt_sincosf_poly(x * s, x * x, n ^ COS, (ns & 2) != 0);
+    res = top < 0x398u ? (COS ? 1.0f : y) : res;              // |y| < 2^-12
+    res = top >= 0x7f8u ? (y - y) / 0.0f : res;               // inf, NaN
+    return res;
+}
+
+RT_FN float rt_sinf(float x) { return rt_sincosf<0>(x); }
+RT_FN float rt_cosf(float x) { return rt_sincosf<1>(x); }
 
 // bf16 <-> f32 with the rounding of half::bf16::from_f32 (round to nearest even, NaN quieted)
 RT_FN float bf2f(uint16_t b) { return u2f((uint32_t)b << 16); }

@@ -1,9 +1,9 @@
 // Host check of the kernels' libm-level routines: ratchet_amd/csrc/rt_libm.h compiled as plain C++ (the very text the
-// kernels compile for the GPU) against this machine's C library, which is what the reference's f32::tanh / f32::exp / f32::ln
+// kernels compile for the GPU) against this machine's C library, which is what the reference's f32::tanh / f32::exp / f32::ln / f32::sin / f32::cos
 // resolve to (crates/ratchet-core/src/cpu/unary.rs:46-65, cpu/softmax.rs:30).  Bit equality is required (any NaN equals
 // any NaN).  Inputs: every `stride`-th float bit pattern over the whole 2^32 range (stride 1 = exhaustive), every value
 // that a 16-bit input can widen to, and the breakpoints of the algorithms.  Build: g++ -O2 -ffp-contract=off.
-// Usage: device_math_check [stride]   -> prints "tanhf <n> expm1f <n> expf <n> logf <n> f2bf <n> checked <m>", exit code 0 iff all n are 0.
+// Usage: device_math_check [stride]   -> prints "tanhf <n> expm1f <n> expf <n> logf <n> sinf <n> cosf <n> f2bf <n> checked <m>", exit code 0 iff all n are 0.
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
@@ -26,13 +26,15 @@ static inline uint16_t bf16_reference(float f) {
 }
 
 struct Counts {
-    unsigned long long tanh_bad = 0, expm1_bad = 0, exp_bad = 0, log_bad = 0, bf_bad = 0, checked = 0;
+    unsigned long long tanh_bad = 0, expm1_bad = 0, exp_bad = 0, log_bad = 0, sin_bad = 0, cos_bad = 0, bf_bad = 0, checked = 0;
     void one(uint32_t bits) {
         const float x = u2f(bits);
         if (!same(rt_tanhf(x), tanhf(x))) tanh_bad++;
         if (!same(rt_expm1f(x), expm1f(x))) expm1_bad++;
         if (!same(rt_expf(x), expf(x))) exp_bad++;
         if (!same(rt_logf(x), logf(x))) log_bad++;
+        if (!same(rt_sinf(x), sinf(x))) sin_bad++;
+        if (!same(rt_cosf(x), cosf(x))) cos_bad++;
         if (f2bf(x) != bf16_reference(x)) bf_bad++;
         checked++;
     }
@@ -61,6 +63,7 @@ int main(int argc, char** argv) {
             c.one(mk + (uint32_t)d);
             c.one((mk + (uint32_t)d) ^ 0x80000000u);
         }
-    printf("tanhf %llu expm1f %llu expf %llu logf %llu f2bf %llu checked %llu\n", c.tanh_bad, c.expm1_bad, c.exp_bad, c.log_bad, c.bf_bad, c.checked);
-    return (c.tanh_bad | c.expm1_bad | c.exp_bad | c.log_bad | c.bf_bad) ? 1 : 0;
+    printf("tanhf %llu expm1f %llu expf %llu logf %llu sinf %llu cosf %llu f2bf %llu checked %llu\n", c.tanh_bad, c.expm1_bad, c.exp_bad, c.log_bad, c.sin_bad,
+           c.cos_bad, c.bf_bad, c.checked);
+    return (c.tanh_bad | c.expm1_bad | c.exp_bad | c.log_bad | c.sin_bad | c.cos_bad | c.bf_bad) ? 1 : 0;
 }

@@ -122,7 +122,7 @@ def test_binary_broadcast_against_rows_that_are_not_whole_vectors(dev, oracle, d
 
 
 UNARY = ["gelu", "tanh", "exp", "log", "sin", "cos", "abs", "sqrt", "relu", "floor", "ceil", "neg", "silu", "sigmoid"]
-EXACT32 = {"gelu", "tanh", "exp", "log", "abs", "sqrt", "relu", "floor", "ceil", "neg", "silu", "sigmoid"}
+EXACT32 = {"gelu", "tanh", "exp", "log", "sin", "cos", "abs", "sqrt", "relu", "floor", "ceil", "neg", "silu", "sigmoid"}
 
 
 @pytest.mark.parametrize("op", UNARY)
@@ -153,10 +153,8 @@ def test_unary_f16_exhaustive(dev, oracle, op):
     bad, mx = oracle.count_not_close(got, want, 1e-3, 1e-3)
     assert bad == 0, (op, bad, mx)
     mism = mismatch_count(got, want)
-    # sin/cos are evaluated in double and rounded; the host libm float routines can land on the other side of a
-    # float16 rounding boundary for a handful of inputs.  Everything else (log included: the C library's own algorithm) is bit-exact.
-    allowed = 8 if op in ("sin", "cos") else 0
-    assert mism <= allowed, (op, mism)
+    # every op is the C library's own algorithm: bit-exact
+    assert mism == 0, (op, mism)
     assert ulp_diff(got, want).max() <= 1
 
 
