@@ -3,14 +3,16 @@
 //   RT_FN     the function qualifiers (`__device__ inline` in the kernels, `static inline` on the host)
 //   RT_TABLE  the qualifiers of a constant table (`__device__ static const` / `static const`)
 //
-// Two libm routines are restated operation by operation so that their float32 results equal, bit for bit, what the
-// x86-64 glibc 2.35 `tanhf` and `expf` return (checked on the CPU over all 2^32 inputs with this same code compiled
-// by g++).  ratchet's CPU executor calls exactly those through Rust's f32::tanh / f32::exp
-// (crates/ratchet-core/src/cpu/unary.rs:46-65, cpu/softmax.rs:30), and GELU's `1 + tanh(..)` cancellation turns a
+// The libm routines of the unary ops are restated operation by operation so that their float32 results equal, bit for
+// bit, what the x86-64 glibc 2.35 `tanhf`, `expf`, `logf`, `sinf` and `cosf` return (checked on the CPU over all 2^32
+// inputs with this same code compiled by g++).  ratchet's CPU executor calls exactly those through Rust's f32::tanh /
+// f32::exp / f32::ln / f32::sin / f32::cos (crates/ratchet-core/src/cpu/unary.rs:46-65, cpu/softmax.rs:30, cpu/rope.rs), and GELU's `1 + tanh(..)` cancellation turns a
 // 1-ulp tanh difference into hundreds of ulps, so "close" is not good enough there.
 //   tanhf/expm1f: the classic fdlibm float algorithms (float arithmetic only).
 //   expf: the table-driven double-precision algorithm (2^(k/32) table, degree-3 polynomial), with the
 //         reduction r = fma(InvLn2N, x, -kd) that an FMA build of the routine performs.
+//   logf: a 16-entry table of (1/c, log c) and a cubic, in double.  sinf / cosf: the quadrant and the reduced argument in
+//         double (x - n * pi/2 as one fma, as an FMA build performs it), sine and cosine polynomials in double.
 // Everything here must be compiled with -ffp-contract=off: each float operation below is meant to round on its own.
 //
 // Provenance.  The routines below are restatements of published algorithms, with their published constants (a result
@@ -25,6 +27,10 @@
 //     2017-2018 Arm Limited, SPDX-License-Identifier: MIT), which glibc 2.27 and later use for `expf`: the 32-entry
 //     table follows from its defining formula (the comment above it), the three polynomial coefficients and the
 //     reduction constants are the published ones.
+//   rt_logf, rt_sinf, rt_cosf: the single-precision log, sin and cos of the same Arm optimized-routines (`math/logf.c`,
+//     `math/logf_data.c`, `math/sinf.c`, `math/cosf.c`, `math/sincosf.h`, `math/sincosf_data.c`; Copyright (c) 2017-2018 Arm
+//     Limited, SPDX-License-Identifier: MIT), which glibc uses for `logf`, `sinf` and `cosf`: the tables and coefficients are
+//     the published ones.
 #ifndef RT_LIBM_H
 #define RT_LIBM_H
 
